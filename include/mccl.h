@@ -1,0 +1,155 @@
+/*
+ * mccl.h -- C ABI of libmi355ccl.so: the local-reduce and pack/permute kernels of the
+ * collective data path on one MI355X (gfx950).
+ *
+ * The N "peer" buffers of a collective are N device pointers.  In single-GPU mode they
+ * are N allocations in one GPU's HBM; on a multi-GPU node the same entry points take
+ * peer-mapped pointers.  Every entry point
+ *   - takes plain pointers and sizes (no torch types), and an explicit hipStream_t
+ *     (passed as void*; NULL = the HIP null stream),
+ *   - only enqueues work on that stream and returns; it never synchronises,
+ *   - allocates no device memory,
+ *   - returns MCCL_OK (0) or a negative mccl_status_t; mccl_last_error() then holds a
+ *     message for the calling thread.  Nothing throws across this boundary.
+ *
+ * Citations (file:line) are relative to the reference tree (intel/torch-ccl).
+ */
+#ifndef MCCL_H_
+#define MCCL_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types: the entries of cclDatatypes, src/utils.cpp:46-58 (Bool travels as U8). */
+typedef enum {
+  MCCL_U8 = 0,
+  MCCL_I8 = 1,
+  MCCL_I16 = 2,
+  MCCL_I32 = 3,
+  MCCL_I64 = 4,
+  MCCL_F16 = 5,
+  MCCL_F32 = 6,
+  MCCL_F64 = 7,
+  MCCL_BF16 = 8
+} mccl_dtype_t;
+
+/* Reduction ops: the entries of cclOps, src/utils.cpp:38-44, numbered like
+ * c10d::ReduceOp (SUM 0, AVG 1, PRODUCT 2, MIN 3, MAX 4).  AVG is this library's
+ * addition (the reference rejects it on device, src/dispatch_stub.h:320-335): the
+ * SUM chain followed by one division by n in the accumulation type. */
+typedef enum {
+  MCCL_SUM = 0,
+  MCCL_AVG = 1,
+  MCCL_PROD = 2,
+  MCCL_MIN = 3,
+  MCCL_MAX = 4
+} mccl_op_t;
+
+typedef enum {
+  MCCL_OK = 0,
+  MCCL_ERR_INVALID_ARG = -1, /* null pointer, bad enum, n out of range, bad alignment */
+  MCCL_ERR_HIP = -2,         /* a HIP runtime call failed; message names it */
+  MCCL_ERR_UNSUPPORTED = -3
+} mccl_status_t;
+
+/* Kernel variant of the reduction (the reference switches at SMALL_MAX_COUNT between a
+ * single-launch kernel and a persistent one, src/gpu/dpcpp_ccl.cpp:771-775). */
+typedef enum {
+  MCCL_VARIANT_AUTO = 0,      /* pick by message size */
+  MCCL_VARIANT_SMALL = 1,     /* one vector per lane, grid covers the message */
+  MCCL_VARIANT_PERSISTENT = 2 /* fixed grid sized to the CUs, grid-stride loop */
+} mccl_variant_t;
+
+#define MCCL_MAX_RANKS 64
+
+/* One contiguous byte range to copy. */
+typedef struct {
+  const void* src;
+  void* dst;
+  size_t bytes;
+} mccl_segment_t;
+
+int mccl_version(void);
+
+/* Message for the last non-OK status returned on this thread ("" if none). */
+const char* mccl_last_error(void);
+
+size_t mccl_dtype_size(int dtype);
+
+/*
+ * N-buffer reduction: out[i] = in[0][i] (op) in[1][i] (op) ... (op) in[n-1][i], i < count.
+ * Replaces the sum loop of allreducer_small<T>::allreduce (src/gpu/allreduce_small.h:289-361)
+ * and the data kernels of allreducer<T>::allreduce (src/gpu/allreduce.h:306-533), and the
+ * ccl::allreduce call of src/gpu/dpcpp_ccl.cpp:781-788.
+ *   - order: ascending rank; SUM starts from +0 like the reference's "result = 0".
+ *   - f16 / bf16 accumulate in fp32 and round once (nearest even) on store; f32, f64 and
+ *     the integer types accumulate in their own type (integers wrap).
+ *   - out may be exactly one of the inputs (in place); partial overlap is not allowed.
+ *   - any count, any element-aligned pointers; 1 <= n <= MCCL_MAX_RANKS.
+ */
+int mccl_reduce_n(const void* const* in, int n, void* out, size_t count, int dtype, int op,
+                  int variant, void* stream);
+
+/*
+ * Shard reduction of reduce_scatter: for s in [shard_first, shard_first + shard_num):
+ *   out[s - shard_first][j] = reduce_k in[k][s * shard_count + j],  j < shard_count.
+ * One launch covers all requested shards.  Replaces ccl::reduce_scatter at
+ * src/gpu/dpcpp_ccl.cpp:1002-1008 (rank r calls it with shard_first = r, shard_num = 1).
+ */
+int mccl_reduce_scatter_n(const void* const* in, int n, void* const* out, size_t shard_count,
+                          int shard_first, int shard_num, int dtype, int op, void* stream);
+
+/*
+ * Coalesced reductions: nbuf independent N-buffer reductions in one launch
+ * (allreduce_coalesced, src/gpu/dpcpp_ccl.cpp:810-818).  in is laid out [nbuf][n]
+ * (buffer-major), out and counts have nbuf entries.
+ */
+int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size_t* counts,
+                      int nbuf, int dtype, int op, void* stream);
+
+/* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
+ * each other's destinations.  The building block of the copy collectives below. */
+int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream);
+
+/* allgather: out[k*bytes_per_rank : (k+1)*bytes_per_rank] = in[k]
+ * (ccl::allgatherv at src/gpu/dpcpp_ccl.cpp:1176-1182). */
+int mccl_allgather_n(const void* const* in, int n, void* out, size_t bytes_per_rank,
+                     void* stream);
+
+/*
+ * alltoall(v) for all n ranks at once.  split_rows is the n x n row-major matrix
+ * S[r][d] = rows rank r sends to rank d (rank r's inputSplitSizes; rank d's
+ * outputSplitSizes[r] must equal S[r][d]).  Rank d's output segment r, at row offset
+ * sum_{r'<r} S[r'][d], receives rank r's input segment d, at row offset sum_{d'<d} S[r][d']
+ * (count/displacement arithmetic of src/gpu/dpcpp_ccl.cpp:1431-1455).
+ */
+int mccl_alltoallv_n(const void* const* in, void* const* out, int n, const int64_t* split_rows,
+                     size_t row_bytes, void* stream);
+
+/* One rank's share of alltoall(v): rank `rank` pulls its n segments from the peers' input
+ * buffers.  send_displ_bytes[r] = byte offset, inside rank r's input, of the segment
+ * addressed to `rank`; recv_bytes[r] = its length.  Segments land back to back in out. */
+int mccl_alltoallv_pull(const void* const* in, int n, void* out, const size_t* send_displ_bytes,
+                        const size_t* recv_bytes, void* stream);
+
+/* pack: dst = src[0] | src[1] | ... (src/gpu/dpcpp_ccl.cpp:1505-1515);
+ * unpack: the inverse scatter (src/gpu/dpcpp_ccl.cpp:1528-1538). */
+int mccl_pack(const void* const* src, const size_t* bytes, int n, void* dst, void* stream);
+int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, void* stream);
+
+/* Launch geometry the library would use (for reports): returns grid size in workgroups and
+ * writes the workgroup size; count in elements. */
+int mccl_query_launch(size_t count, int n, int dtype, int variant, int* block_size);
+
+/* Tuning knobs (process-wide; <= 0 keeps the default).  Meant for benchmarks. */
+void mccl_set_tuning(int persistent_blocks_per_cu, int block_size, int small_max_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MCCL_H_ */

@@ -1,0 +1,280 @@
+"""GPU parity of the N-buffer reduction (mccl_reduce_n / _reduce_scatter_n / _reduce_multi)
+against the CPU oracle.  Bar: bit-exact for every dtype (the kernel runs the same
+ascending-rank chain and the same single rounding as the oracle; the 1-ulp allowance for
+f16/bf16 is not needed)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (ALL_DTYPES, FLOAT_DTYPES, INT_DTYPES, assert_bits_equal, bits,
+                     oracle_reduce_bits, rank_buffer, to_carrier, TORCH_TO_CODE)
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+OPS = {"sum": O.SUM, "prod": O.PROD, "min": O.MIN, "max": O.MAX}
+
+
+def _run(mccl, cpu_inputs, op, variant=0, out=None):
+    dev_in = [t.to(DEV) for t in cpu_inputs]
+    res = mccl.reduce_n(dev_in, out=out, op=op, variant=variant)
+    torch.cuda.synchronize()
+    return res
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=str)
+@pytest.mark.parametrize("opname", list(OPS))
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+def test_reduce_all_dtypes_ops(mccl, dtype, opname, n):
+    count = 5000  # not a multiple of the vector width: head/tail paths run
+    scale = 1.0 if opname == "prod" else 0.02
+    ins = [rank_buffer(count, dtype, r, scale=scale) for r in range(n)]
+    for variant in (1, 2):
+        got = _run(mccl, ins, OPS[opname], variant)
+        assert_bits_equal(bits(got), oracle_reduce_bits(ins, OPS[opname]),
+                          "%s %s n=%d variant=%d" % (dtype, opname, n, variant))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.int32], ids=str)
+@pytest.mark.parametrize("n", [2, 4, 5, 7, 8, 16, 64])
+@pytest.mark.parametrize("count", [0, 1, 7, 8, 9, 63, 64, 511, 512, 513, 4096 + 3, 131072, 1_000_003])
+def test_reduce_sum_counts_and_ranks(mccl, dtype, n, count):
+    if count > 200000 and n > 8:
+        pytest.skip("large x many ranks adds nothing")
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    got = _run(mccl, ins, O.SUM)
+    if count == 0:
+        assert got.numel() == 0
+        return
+    assert_bits_equal(bits(got), oracle_reduce_bits(ins), "%s n=%d count=%d" % (dtype, n, count))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.uint8, torch.float64], ids=str)
+@pytest.mark.parametrize("shift", [1, 3, 5, 8])
+def test_reduce_shifted_congruent(mccl, dtype, shift):
+    """All buffers start `shift` elements past a 16-byte boundary: the head is peeled."""
+    n, count = 4, 10007
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    dev = []
+    for t in ins:
+        base = torch.zeros(count + 64, dtype=dtype, device=DEV)
+        view = base[shift:shift + count]
+        view.copy_(t)
+        dev.append(view)
+    outbase = torch.zeros(count + 64, dtype=dtype, device=DEV)
+    out = outbase[shift:shift + count]
+    mccl.reduce_n(dev, out=out, op=O.SUM)
+    torch.cuda.synchronize()
+    assert_bits_equal(bits(out), oracle_reduce_bits(ins), "shift=%d" % shift)
+    # canaries: nothing outside the view was written
+    assert int(outbase[:shift].abs().sum()) == 0 and int(outbase[shift + count:].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.int8], ids=str)
+def test_reduce_incongruent_alignment(mccl, dtype):
+    """Each buffer has a different offset mod 16 bytes: the element-wise kernel runs."""
+    n, count = 5, 9001
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    dev = []
+    for r, t in enumerate(ins):
+        base = torch.zeros(count + 64, dtype=dtype, device=DEV)
+        view = base[r + 1:r + 1 + count]
+        view.copy_(t)
+        dev.append(view)
+    out = torch.zeros(count + 64, dtype=dtype, device=DEV)
+    mccl.reduce_n(dev, out=out[:count], op=O.SUM)
+    torch.cuda.synchronize()
+    assert_bits_equal(bits(out[:count]), oracle_reduce_bits(ins), "incongruent")
+    assert int(out[count:].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("which", [0, 3, 7])
+def test_reduce_in_place(mccl, dtype, which):
+    """The allreduce of the reference is in place: out aliases one of the inputs."""
+    n, count = 8, 70001
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    want = oracle_reduce_bits(ins)
+    for variant in (1, 2):
+        dev = [t.to(DEV) for t in ins]
+        mccl.reduce_n(dev, out=dev[which], op=O.SUM, variant=variant)
+        torch.cuda.synchronize()
+        assert_bits_equal(bits(dev[which]), want, "in place on %d variant %d" % (which, variant))
+        for r in range(n):
+            if r != which:
+                assert_bits_equal(bits(dev[r]), bits(ins[r]), "input %d untouched" % r)
+
+
+def _special_values(dtype):
+    """+-0, subnormals, +-inf, max-finite cancellation, rounding ties."""
+    if dtype == torch.bfloat16:
+        pats = [0x0000, 0x8000, 0x0001, 0x8001, 0x007f, 0x0080, 0x7f7f, 0xff7f, 0x7f80, 0xff80,
+                0x3f80, 0xbf80, 0x3f81, 0x3c00, 0x3b80, 0x4000, 0x0100, 0x8100]
+        return torch.tensor(np.array(pats, dtype=np.uint16).view(np.int16)).view(torch.bfloat16)
+    if dtype == torch.float16:
+        pats = [0x0000, 0x8000, 0x0001, 0x8001, 0x03ff, 0x0400, 0x7bff, 0xfbff, 0x7c00, 0xfc00,
+                0x3c00, 0xbc00, 0x3c01, 0x1400, 0x1000, 0x4000, 0x0002, 0x8002]
+        return torch.tensor(np.array(pats, dtype=np.uint16).view(np.int16)).view(torch.float16)
+    pats = [0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x007fffff, 0x00800000, 0x7f7fffff,
+            0xff7fffff, 0x7f800000, 0xff800000, 0x3f800000, 0xbf800000, 0x3f800001, 0x33800000,
+            0x33000000, 0x40000000, 0x00000002, 0x80000002]
+    return torch.tensor(np.array(pats, dtype=np.uint32).view(np.int32)).view(torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+@pytest.mark.parametrize("opname", ["sum", "prod", "min", "max"])
+def test_reduce_special_values(mccl, dtype, opname):
+    """Every ordered triple of special values (signed zeros, subnormals, infinities, ties).
+    NaN results are compared as "is NaN" for fp32 (payloads are not part of the contract);
+    f16/bf16 NaNs are canonical in both implementations and compared bit for bit."""
+    v = _special_values(dtype)
+    k = v.numel()
+    a = v.repeat_interleave(k * k)
+    b = v.repeat_interleave(k).repeat(k)
+    c = v.repeat(k * k)
+    ins = [a.contiguous(), b.contiguous(), c.contiguous()]
+    got = bits(_run(mccl, ins, OPS[opname]))
+    want = oracle_reduce_bits(ins, OPS[opname])
+    if dtype == torch.float32:
+        gf, wf = got.view(np.float32), want.view(np.float32)
+        nan_g, nan_w = np.isnan(gf), np.isnan(wf)
+        assert np.array_equal(nan_g, nan_w)
+        assert_bits_equal(got[~nan_w], want[~nan_w], "%s %s" % (dtype, opname))
+    else:
+        assert_bits_equal(got, want, "%s %s" % (dtype, opname))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+def test_reduce_nan_inputs(mccl, dtype):
+    """NaN in any rank makes the SUM NaN; f16/bf16 produce the canonical quiet NaN."""
+    n, count = 4, 1024
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    ins[2][5] = float("nan")
+    ins[0][100] = float("inf")
+    ins[3][100] = float("-inf")
+    got = _run(mccl, ins, O.SUM)
+    assert torch.isnan(got[5]) and torch.isnan(got[100])
+    want = oracle_reduce_bits(ins)
+    if dtype != torch.float32:
+        assert_bits_equal(bits(got), want, "nan canonical")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64], ids=str)
+def test_reduce_avg(mccl, dtype):
+    """AVG = SUM chain, then one division by n in the accumulation type."""
+    n, count = 8, 4099
+    ins = [rank_buffer(count, dtype, r) for r in range(n)]
+    got = _run(mccl, ins, mccl.AVG)
+    acc_t = torch.float64 if dtype == torch.float64 else torch.float32
+    acc = torch.zeros(count, dtype=acc_t)
+    for t in ins:
+        acc = acc + t.to(acc_t)
+    want = (acc / n).to(dtype)
+    assert_bits_equal(bits(got), bits(want), "avg %s" % dtype)
+
+
+def test_reduce_avg_rejects_integers(mccl):
+    t = [torch.ones(8, dtype=torch.int32, device=DEV) for _ in range(2)]
+    with pytest.raises(RuntimeError, match="AVG"):
+        mccl.reduce_n(t, op=mccl.AVG)
+
+
+# ---- configs of the headline benchmark, at sizes the oracle finishes in seconds ----
+
+def test_config1_fp32_two_ranks_16mib(mccl):
+    """all_reduce SUM fp32, 2 ranks x 4,194,304 elements, uniform[-1,1): bit-exact
+    (a two-operand IEEE add has a single possible value)."""
+    count = 4_194_304
+    ins = [rank_buffer(count, torch.float32, r, dist="uniform") for r in range(2)]
+    got = _run(mccl, ins, O.SUM)
+    assert_bits_equal(bits(got), bits(ins[0] + ins[1]), "C1 vs torch fp32 add")
+    assert_bits_equal(bits(got), oracle_reduce_bits(ins), "C1 vs oracle")
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_config2_bf16_decode_256k(mccl, variant):
+    """bf16 [16 x 8192] per rank, 8 ranks, N(0, 0.02), fp32 accumulation."""
+    ins = [rank_buffer(16 * 8192, torch.bfloat16, r) for r in range(8)]
+    got = _run(mccl, ins, O.SUM, variant)
+    assert_bits_equal(bits(got), oracle_reduce_bits(ins), "C2 variant %d" % variant)
+
+
+def test_config3_bf16_prefill_64mib(mccl):
+    """bf16 [4096 x 8192] per rank, 8 ranks: full size, checked against the oracle (OpenMP)
+    and against an on-device fp32 chain built from torch ops."""
+    count = 4096 * 8192
+    ins = [rank_buffer(count, torch.bfloat16, r) for r in range(8)]
+    dev = [t.to(DEV) for t in ins]
+    got = mccl.reduce_n(dev, op=O.SUM, variant=2)
+    torch.cuda.synchronize()
+    acc = torch.zeros(count, dtype=torch.float32, device=DEV)
+    for t in dev:
+        acc += t.float()
+    assert torch.equal(got.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+    O.set_threads(min(16, O.max_threads()))
+    try:
+        want = oracle_reduce_bits(ins)
+    finally:
+        O.set_threads(1)
+    assert_bits_equal(bits(got), want, "C3")
+
+
+# ---- reduce_scatter ----
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.int64], ids=str)
+@pytest.mark.parametrize("n,m", [(2, 1), (4, 1000), (8, 65536 + 5), (3, 33)])
+def test_reduce_scatter_all_shards(mccl, dtype, n, m):
+    ins = [rank_buffer(n * m, dtype, r) for r in range(n)]
+    dev = [t.to(DEV) for t in ins]
+    outs = [torch.empty(m, dtype=dtype, device=DEV) for _ in range(n)]
+    mccl.reduce_scatter_n(dev, outs, op=O.SUM)
+    torch.cuda.synchronize()
+    code = TORCH_TO_CODE[dtype]
+    want = O.reduce_scatter([to_carrier(t) for t in ins], code, O.SUM)
+    for s in range(n):
+        assert_bits_equal(bits(outs[s]), want[s].view(bits(outs[s]).dtype), "shard %d" % s)
+    # one shard at a time (what a single rank does) gives the same answer
+    for s in range(n):
+        o = torch.empty(m, dtype=dtype, device=DEV)
+        mccl.reduce_scatter_n(dev, [o], op=O.SUM, shard_first=s)
+        torch.cuda.synchronize()
+        assert_bits_equal(bits(o), bits(outs[s]), "single shard %d" % s)
+
+
+def test_reduce_scatter_matches_allreduce_slices(mccl):
+    """Shard s of reduce_scatter == slice s of the allreduce of the same buffers."""
+    n, m = 8, 12345
+    ins = [rank_buffer(n * m, torch.bfloat16, r) for r in range(n)]
+    dev = [t.to(DEV) for t in ins]
+    full = mccl.reduce_n(dev, op=O.SUM)
+    outs = [torch.empty(m, dtype=torch.bfloat16, device=DEV) for _ in range(n)]
+    mccl.reduce_scatter_n(dev, outs, op=O.SUM)
+    torch.cuda.synchronize()
+    for s in range(n):
+        assert_bits_equal(bits(outs[s]), bits(full[s * m:(s + 1) * m]), "shard %d" % s)
+
+
+def test_reduce_multi_coalesced(mccl):
+    """allreduce_coalesced: 5 buckets full((5+i,), rank+1+i) -> W*(i+(W+1)/2)
+    (closed form of the reference's test_allreduce_coalesced_basics), one launch group."""
+    for W in (2, 4, 8):
+        ins = [[torch.full((5 + i,), float(r + 1 + i), device=DEV) for r in range(W)] for i in range(5)]
+        outs = [torch.empty(5 + i, device=DEV) for i in range(5)]
+        mccl.reduce_multi(ins, outs, op=O.SUM)
+        torch.cuda.synchronize()
+        for i, o in enumerate(outs):
+            assert torch.equal(o.cpu(), torch.full((5 + i,), W * (i + (W + 1.0) / 2.0)))
+
+
+def test_reduce_multi_random(mccl):
+    n = 8
+    counts = [1, 17, 4096, 100003, 0, 777]
+    ins_cpu = [[rank_buffer(c, torch.bfloat16, r, seed=77 + b) for r in range(n)] for b, c in enumerate(counts)]
+    ins = [[t.to(DEV) for t in lst] for lst in ins_cpu]
+    outs = [torch.empty(c, dtype=torch.bfloat16, device=DEV) for c in counts]
+    mccl.reduce_multi(ins, outs, op=O.SUM)
+    torch.cuda.synchronize()
+    for b, c in enumerate(counts):
+        if c:
+            assert_bits_equal(bits(outs[b]), oracle_reduce_bits(ins_cpu[b]), "bucket %d" % b)

@@ -1,0 +1,878 @@
+// libmi355ccl: local-reduce and segmented-copy kernels for gfx950 (MI355X) and the C ABI
+// declared in include/mccl.h.
+//
+// Everything here is HBM-bandwidth bound.  Design rules:
+//   * one 16-byte vector per lane per input, so a wavefront reads 1 KiB contiguous from
+//     each of the N inputs; all N (x unroll) loads of a tile are issued before the first
+//     add so the memory system sees N*U independent requests per lane;
+//   * accumulation is a sequential ascending-rank chain held in registers (fp32 for
+//     f16/bf16), one round-to-nearest-even on store;
+//   * outputs are written with non-temporal stores (streamed past the caches);
+//   * a "small" launch gives every lane exactly one vector (grid covers the message, one
+//     wavefront per workgroup so all CUs are used); the "persistent" launch uses a fixed
+//     grid proportional to the CU count and walks tiles grid-stride;
+//   * misaligned heads/tails are peeled element-wise inside the same launch; pointer sets
+//     that are not mutually congruent mod 16 take an element-wise kernel.
+//
+// What each kernel replaces in the reference (intel/torch-ccl):
+//   reduce_vec_kernel / reduce_elem_kernel : the N-peer sum of src/gpu/allreduce_small.h:289-361,
+//       the five data kernels of src/gpu/allreduce.h:306-533, ccl::allreduce /
+//       ccl::reduce_scatter call sites in src/gpu/dpcpp_ccl.cpp:781-788, 1002-1008
+//   copy_segments_kernel : ccl::allgatherv / ccl::alltoall(v) data movement
+//       (src/gpu/dpcpp_ccl.cpp:1176-1182, 1403-1455) and the pack/unpack copy_ loops
+//       (src/gpu/dpcpp_ccl.cpp:1505-1538)
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "mccl.h"
+
+namespace {
+
+// ------------------------------------------------------------------------------------------
+// error plumbing
+// ------------------------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess)                                                               \
+      return fail(MCCL_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),  \
+                  __FILE__, __LINE__);                                                  \
+  } while (0)
+
+// ------------------------------------------------------------------------------------------
+// tuning state and per-device facts
+// ------------------------------------------------------------------------------------------
+constexpr int kBlockPersistent = 256;  // 4 wavefronts
+constexpr int kBlockSmall = 64;        // 1 wavefront: spreads a small message over all CUs
+constexpr int kUnrollPersistent = 2;   // vectors per lane per input per tile
+constexpr int kMaxJobs = 64;           // independent reductions per launch
+constexpr int kMaxSegs = 64;           // copy segments per launch
+constexpr int kCopyBlock = 256;
+constexpr int kCopyUnroll = 4;
+constexpr size_t kCopyChunk = (size_t)kCopyBlock * 16 * kCopyUnroll;  // 16 KiB per chunk
+
+int g_blocks_per_cu = 8;
+size_t g_small_max_bytes = 2u << 20;  // per-rank bytes up to which AUTO picks "small"
+
+struct DeviceFacts {
+  int cus = 0;
+};
+DeviceFacts g_facts[64];
+std::once_flag g_facts_once[64];
+
+int device_cus(int* cus_out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return fail(MCCL_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  hipError_t err = hipSuccess;
+  std::call_once(g_facts_once[dev], [&]() {
+    int cus = 0;
+    err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    g_facts[dev].cus = cus > 0 ? cus : 256;
+  });
+  if (err != hipSuccess) return fail(MCCL_ERR_HIP, "hipDeviceGetAttribute failed: %s", hipGetErrorString(err));
+  *cus_out = g_facts[dev].cus;
+  return MCCL_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// element types
+// ------------------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<MCCL_BF16> {
+  using store_t = uint16_t;
+  using acc_t = float;
+  static constexpr bool kIsFloat = true;
+  static __device__ __forceinline__ acc_t load(store_t h) { return bits_to_f32((uint32_t)h << 16); }
+  // round to nearest even; every NaN becomes 0x7FC0
+  static __device__ __forceinline__ store_t store(acc_t f) {
+    uint32_t u = f32_to_bits(f);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (store_t)(((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : r);
+  }
+};
+
+template <>
+struct Elem<MCCL_F16> {
+  using store_t = uint16_t;
+  using acc_t = float;
+  static constexpr bool kIsFloat = true;
+  static __device__ __forceinline__ acc_t load(store_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+  }
+  // hardware convert is round-to-nearest-even with gradual underflow; NaN -> 0x7E00
+  static __device__ __forceinline__ store_t store(acc_t f) {
+    uint16_t r = __builtin_bit_cast(uint16_t, (_Float16)f);
+    return (f != f) ? (store_t)0x7e00u : r;
+  }
+};
+
+template <typename T, typename UT, int CODE>
+struct IntElem {
+  using store_t = T;
+  using acc_t = T;
+  using uacc_t = UT;
+  static constexpr bool kIsFloat = false;
+  static __device__ __forceinline__ acc_t load(store_t v) { return v; }
+  static __device__ __forceinline__ store_t store(acc_t v) { return v; }
+};
+template <> struct Elem<MCCL_U8> : IntElem<uint8_t, uint8_t, MCCL_U8> {};
+template <> struct Elem<MCCL_I8> : IntElem<int8_t, uint8_t, MCCL_I8> {};
+template <> struct Elem<MCCL_I16> : IntElem<int16_t, uint16_t, MCCL_I16> {};
+template <> struct Elem<MCCL_I32> : IntElem<int32_t, uint32_t, MCCL_I32> {};
+template <> struct Elem<MCCL_I64> : IntElem<int64_t, uint64_t, MCCL_I64> {};
+
+template <typename T>
+struct FloatElem {
+  using store_t = T;
+  using acc_t = T;
+  static constexpr bool kIsFloat = true;
+  static __device__ __forceinline__ acc_t load(store_t v) { return v; }
+  static __device__ __forceinline__ store_t store(acc_t v) { return v; }
+};
+template <> struct Elem<MCCL_F32> : FloatElem<float> {};
+template <> struct Elem<MCCL_F64> : FloatElem<double> {};
+
+// ------------------------------------------------------------------------------------------
+// the reduction chain
+// ------------------------------------------------------------------------------------------
+// First element of the chain.  SUM/AVG start from literal +0 and add rank 0 (so an all -0
+// column yields +0, as "result = 0; result = result + buf[r]" does); the other ops start
+// from rank 0's value.
+template <int DT, int OP>
+__device__ __forceinline__ typename Elem<DT>::acc_t chain_first(typename Elem<DT>::acc_t x) {
+  using A = typename Elem<DT>::acc_t;
+  if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {
+    if constexpr (Elem<DT>::kIsFloat) return (A)0 + x;
+    else return x;
+  } else {
+    return x;
+  }
+}
+
+template <int DT, int OP>
+__device__ __forceinline__ typename Elem<DT>::acc_t chain_next(typename Elem<DT>::acc_t acc,
+                                                                typename Elem<DT>::acc_t x) {
+  using A = typename Elem<DT>::acc_t;
+  if constexpr (Elem<DT>::kIsFloat) {
+    if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) return acc + x;
+    else if constexpr (OP == MCCL_PROD) return acc * x;
+    else if constexpr (OP == MCCL_MIN) return (x < acc) ? x : acc;
+    else return (x > acc) ? x : acc;
+  } else {
+    using U = typename Elem<DT>::uacc_t;
+    if constexpr (OP == MCCL_SUM) return (A)(U)((U)acc + (U)x);
+    else if constexpr (OP == MCCL_PROD) return (A)(U)((U)acc * (U)x);
+    else if constexpr (OP == MCCL_MIN) return (x < acc) ? x : acc;
+    else return (x > acc) ? x : acc;
+  }
+}
+
+template <int DT, int OP>
+__device__ __forceinline__ typename Elem<DT>::acc_t chain_last(typename Elem<DT>::acc_t acc, int n) {
+  using A = typename Elem<DT>::acc_t;
+  if constexpr (OP == MCCL_AVG) return acc / (A)n;
+  else return acc;
+}
+
+// Kernel arguments.  ptr[] holds input base pointers; job j reads ptr[job_ptr0[j] + k] +
+// job_in_off[j] for k < n and writes job_out[j].  reduce_n: one job.  reduce_scatter: one
+// job per shard, same pointers, different byte offsets.  reduce_multi: one job per buffer,
+// each with its own n pointers.
+struct ReduceArgs {
+  const char* ptr[MCCL_MAX_RANKS];
+  char* job_out[kMaxJobs];
+  size_t job_in_off[kMaxJobs];
+  size_t job_count[kMaxJobs];
+  int job_ptr0[kMaxJobs];
+  int n;
+};
+
+template <int DT>
+constexpr int vec_elems() { return 16 / (int)sizeof(typename Elem<DT>::store_t); }
+
+template <int DT>
+union VecU {
+  u32x4 v;
+  typename Elem<DT>::store_t e[vec_elems<DT>()];
+};
+
+// Element-wise reduction of one element (used for peeled heads/tails and the misaligned path).
+template <int DT, int OP>
+__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, size_t in_off, char* out,
+                                           size_t idx) {
+  using S = typename Elem<DT>::store_t;
+  using A = typename Elem<DT>::acc_t;
+  const int n = a.n;
+  A acc = chain_first<DT, OP>(Elem<DT>::load(((const S*)(a.ptr[p0] + in_off))[idx]));
+  for (int k = 1; k < n; ++k)
+    acc = chain_next<DT, OP>(acc, Elem<DT>::load(((const S*)(a.ptr[p0 + k] + in_off))[idx]));
+  acc = chain_last<DT, OP>(acc, n);
+  ((S*)out)[idx] = Elem<DT>::store(acc);
+}
+
+// Loads one 16-byte vector; GUARD adds the bounds check of the last, partial tile.
+template <bool GUARD>
+__device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec) {
+  if constexpr (GUARD) {
+    if (v >= nvec) return (u32x4){0u, 0u, 0u, 0u};
+  }
+#ifdef MCCL_NT_LOAD
+  return __builtin_nontemporal_load(&p[v]);
+#else
+  return p[v];
+#endif
+}
+
+// One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
+// ascending-rank chain in registers and streams the result out.
+// NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
+// NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
+template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD>
+__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t in_byte_off,
+                                            u32x4* ov, size_t v0, size_t nvec, int n) {
+  using A = typename Elem<DT>::acc_t;
+  constexpr int VE = vec_elems<DT>();
+  A acc[U][VE];
+
+  if constexpr (NT > 0) {
+    VecU<DT> x[NT][U];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) {
+      const u32x4* iv = (const u32x4*)(a.ptr[p0 + k] + in_byte_off);
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[k][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x[0][u].e[e]));
+#pragma unroll
+      for (int k = 1; k < NT; ++k)
+#pragma unroll
+        for (int e = 0; e < VE; ++e)
+          acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[k][u].e[e]));
+    }
+  } else {
+    {
+      const u32x4* iv = (const u32x4*)(a.ptr[p0] + in_byte_off);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        VecU<DT> x;
+        x.v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x.e[e]));
+      }
+    }
+    constexpr int G = 4;
+    for (int kb = 1; kb < n; kb += G) {
+      VecU<DT> x[G][U];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        if (kb + g < n) {
+          const u32x4* iv = (const u32x4*)(a.ptr[p0 + kb + g] + in_byte_off);
+#pragma unroll
+          for (int u = 0; u < U; ++u) x[g][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        if (kb + g < n) {
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < VE; ++e)
+              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[g][u].e[e]));
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t v = v0 + (size_t)u * BLOCK;
+    if (!GUARD || v < nvec) {
+      VecU<DT> r;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(chain_last<DT, OP>(acc[u][e], n));
+      __builtin_nontemporal_store(r.v, &ov[v]);
+    }
+  }
+}
+
+// Vector kernel.  Requires, for each job, all input pointers (+offset) and the output
+// pointer congruent mod 16.  The output may be exactly one of the inputs: a lane reads
+// element i of every input before it writes element i, and no other lane touches i.
+template <int DT, int OP, int NT, int U, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
+  using S = typename Elem<DT>::store_t;
+  constexpr int VE = vec_elems<DT>();
+  const int job = blockIdx.y;
+  const int p0 = a.job_ptr0[job];
+  const size_t in_off = a.job_in_off[job];
+  char* out = a.job_out[job];
+  const size_t count = a.job_count[job];
+  const int n = (NT > 0) ? NT : a.n;
+
+  // peel: head elements up to the first 16-byte boundary of out, tail after the last vector
+  size_t head = ((16u - (unsigned)((uintptr_t)out & 15u)) & 15u) / sizeof(S);
+  if (head > count) head = count;
+  const size_t nvec = (count - head) / VE;
+  const size_t tail = count - head - nvec * VE;
+
+  if (blockIdx.x == 0) {
+    const size_t t = threadIdx.x;
+    if (t < head) reduce_one<DT, OP>(a, p0, in_off, out, t);
+    else if (t - head < tail) reduce_one<DT, OP>(a, p0, in_off, out, head + nvec * VE + (t - head));
+  }
+
+  const size_t body_off = head * sizeof(S);  // bytes
+  u32x4* ov = (u32x4*)(out + body_off);
+  constexpr size_t TILE = (size_t)BLOCK * U;
+  const size_t full_tiles = nvec / TILE;
+  const size_t ntiles = (nvec + TILE - 1) / TILE;
+
+  size_t tile = blockIdx.x;
+  for (; tile < full_tiles; tile += gridDim.x)
+    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, tile * TILE + threadIdx.x, nvec, n);
+  if (tile < ntiles)  // at most one partial tile exists and one workgroup reaches it
+    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, tile * TILE + threadIdx.x, nvec, n);
+}
+
+// Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
+// multiple of the element size).  Grid-stride over elements.
+template <int DT, int OP>
+__global__ __launch_bounds__(256) void reduce_elem_kernel(const ReduceArgs a) {
+  const int job = blockIdx.y;
+  const int p0 = a.job_ptr0[job];
+  const size_t in_off = a.job_in_off[job];
+  char* out = a.job_out[job];
+  const size_t count = a.job_count[job];
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
+    reduce_one<DT, OP>(a, p0, in_off, out, i);
+}
+
+// ------------------------------------------------------------------------------------------
+// segmented copy
+// ------------------------------------------------------------------------------------------
+struct CopyArgs {
+  mccl_segment_t seg[kMaxSegs];
+  uint32_t chunk_prefix[kMaxSegs + 1];  // exclusive prefix sum of chunks per segment
+  int nseg;
+};
+
+// Chunk c of a segment covers body bytes [c*kCopyChunk, (c+1)*kCopyChunk) where the body
+// starts after a head that brings dst to a 16-byte (or 4-byte) boundary.  When src and dst
+// are congruent mod 16 the body moves as 16-byte vectors, mod 4 as dwords, else as bytes.
+__global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const CopyArgs a) {
+  const uint32_t total = a.chunk_prefix[a.nseg];
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    // binary search: largest s with chunk_prefix[s] <= chunk
+    int lo = 0, hi = a.nseg;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    const uint32_t c = chunk - a.chunk_prefix[lo];
+    const char* src = (const char*)a.seg[lo].src;
+    char* dst = (char*)a.seg[lo].dst;
+    const size_t bytes = a.seg[lo].bytes;
+    const unsigned diff = (unsigned)(((uintptr_t)src ^ (uintptr_t)dst) & 15u);
+    const unsigned t = threadIdx.x;
+
+    if (diff == 0) {
+      size_t head = (16u - (unsigned)((uintptr_t)dst & 15u)) & 15u;
+      if (head > bytes) head = bytes;
+      if (c == 0 && t < head) dst[t] = src[t];
+      const size_t body = bytes - head;
+      const size_t b0 = (size_t)c * kCopyChunk;
+      if (b0 < body) {
+        const size_t len = (body - b0 < kCopyChunk) ? body - b0 : kCopyChunk;
+        const u32x4* sv = (const u32x4*)(src + head + b0);
+        u32x4* dv = (u32x4*)(dst + head + b0);
+        const size_t nv = len >> 4;
+        if (nv == (size_t)kCopyBlock * kCopyUnroll) {
+          u32x4 x[kCopyUnroll];
+#pragma unroll
+          for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kCopyBlock]);
+#pragma unroll
+          for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kCopyBlock]);
+        } else {
+          for (size_t v = t; v < nv; v += kCopyBlock) dv[v] = sv[v];
+          const size_t rem = len & 15u;
+          if (t < rem) dst[head + b0 + (nv << 4) + t] = src[head + b0 + (nv << 4) + t];
+        }
+      }
+    } else if ((diff & 3u) == 0) {
+      size_t head = (4u - (unsigned)((uintptr_t)dst & 3u)) & 3u;
+      if (head > bytes) head = bytes;
+      if (c == 0 && t < head) dst[t] = src[t];
+      const size_t body = bytes - head;
+      const size_t b0 = (size_t)c * kCopyChunk;
+      if (b0 < body) {
+        const size_t len = (body - b0 < kCopyChunk) ? body - b0 : kCopyChunk;
+        const uint32_t* sw = (const uint32_t*)(src + head + b0);
+        uint32_t* dw = (uint32_t*)(dst + head + b0);
+        const size_t nw = len >> 2;
+        for (size_t v = t; v < nw; v += kCopyBlock) dw[v] = sw[v];
+        const size_t rem = len & 3u;
+        if (t < rem) dst[head + b0 + (nw << 2) + t] = src[head + b0 + (nw << 2) + t];
+      }
+    } else {
+      const size_t b0 = (size_t)c * kCopyChunk;
+      if (b0 < bytes) {
+        const size_t len = (bytes - b0 < kCopyChunk) ? bytes - b0 : kCopyChunk;
+        for (size_t v = t; v < len; v += kCopyBlock) dst[b0 + v] = src[b0 + v];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// host-side launch helpers
+// ------------------------------------------------------------------------------------------
+bool valid_dtype(int dt) { return dt >= MCCL_U8 && dt <= MCCL_BF16; }
+bool valid_op(int op) { return op == MCCL_SUM || op == MCCL_AVG || op == MCCL_PROD || op == MCCL_MIN || op == MCCL_MAX; }
+bool float_dtype(int dt) { return dt == MCCL_F16 || dt == MCCL_F32 || dt == MCCL_F64 || dt == MCCL_BF16; }
+
+size_t dtype_size(int dt) {
+  switch (dt) {
+    case MCCL_U8: case MCCL_I8: return 1;
+    case MCCL_I16: case MCCL_F16: case MCCL_BF16: return 2;
+    case MCCL_I32: case MCCL_F32: return 4;
+    case MCCL_I64: case MCCL_F64: return 8;
+    default: return 0;
+  }
+}
+
+enum Shape { kShapeSmall, kShapePersistent, kShapeElem };
+
+template <int DT, int OP, int NT>
+hipError_t launch_vec(const ReduceArgs& a, Shape shape, dim3 grid, hipStream_t s) {
+  if (shape == kShapeSmall)
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kBlockSmall>), grid, dim3(kBlockSmall), 0, s, a);
+  else
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent>), grid,
+                       dim3(kBlockPersistent), 0, s, a);
+  return hipGetLastError();
+}
+
+template <int DT, int OP>
+hipError_t launch_op(const ReduceArgs& a, Shape shape, dim3 grid, hipStream_t s) {
+  if (shape == kShapeElem) {
+    hipLaunchKernelGGL((reduce_elem_kernel<DT, OP>), grid, dim3(256), 0, s, a);
+    return hipGetLastError();
+  }
+  if constexpr (OP == MCCL_SUM) {
+    switch (a.n) {
+      case 2: return launch_vec<DT, OP, 2>(a, shape, grid, s);
+      case 4: return launch_vec<DT, OP, 4>(a, shape, grid, s);
+      case 8: return launch_vec<DT, OP, 8>(a, shape, grid, s);
+      default: break;
+    }
+  }
+  return launch_vec<DT, OP, 0>(a, shape, grid, s);
+}
+
+template <int DT>
+hipError_t launch_dtype(const ReduceArgs& a, int op, Shape shape, dim3 grid, hipStream_t s) {
+  switch (op) {
+    case MCCL_SUM: return launch_op<DT, MCCL_SUM>(a, shape, grid, s);
+    case MCCL_PROD: return launch_op<DT, MCCL_PROD>(a, shape, grid, s);
+    case MCCL_MIN: return launch_op<DT, MCCL_MIN>(a, shape, grid, s);
+    case MCCL_MAX: return launch_op<DT, MCCL_MAX>(a, shape, grid, s);
+    case MCCL_AVG:
+      if constexpr (Elem<DT>::kIsFloat) return launch_op<DT, MCCL_AVG>(a, shape, grid, s);
+      else return hipErrorInvalidValue;
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_any(const ReduceArgs& a, int dtype, int op, Shape shape, dim3 grid, hipStream_t s) {
+  switch (dtype) {
+    case MCCL_U8: return launch_dtype<MCCL_U8>(a, op, shape, grid, s);
+    case MCCL_I8: return launch_dtype<MCCL_I8>(a, op, shape, grid, s);
+    case MCCL_I16: return launch_dtype<MCCL_I16>(a, op, shape, grid, s);
+    case MCCL_I32: return launch_dtype<MCCL_I32>(a, op, shape, grid, s);
+    case MCCL_I64: return launch_dtype<MCCL_I64>(a, op, shape, grid, s);
+    case MCCL_F16: return launch_dtype<MCCL_F16>(a, op, shape, grid, s);
+    case MCCL_F32: return launch_dtype<MCCL_F32>(a, op, shape, grid, s);
+    case MCCL_F64: return launch_dtype<MCCL_F64>(a, op, shape, grid, s);
+    case MCCL_BF16: return launch_dtype<MCCL_BF16>(a, op, shape, grid, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Geometry of a vector launch over jobs whose largest has max_count elements.
+struct Geometry {
+  Shape shape;
+  unsigned grid_x;
+  int block;
+};
+
+int plan_vec(size_t max_count, int njobs, int dtype, int variant, Geometry* g) {
+  int cus = 0;
+  int rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  const size_t es = dtype_size(dtype);
+  const size_t nvec = max_count / (16 / es) + 1;
+  bool small;
+  if (variant == MCCL_VARIANT_SMALL) small = true;
+  else if (variant == MCCL_VARIANT_PERSISTENT) small = false;
+  else small = max_count * es <= g_small_max_bytes;
+  if (small) {
+    size_t tiles = (nvec + kBlockSmall - 1) / kBlockSmall;
+    if (tiles > 0x7fffffffu) return fail(MCCL_ERR_INVALID_ARG, "message too large for the small variant");
+    g->shape = kShapeSmall;
+    g->grid_x = (unsigned)(tiles ? tiles : 1);
+    g->block = kBlockSmall;
+  } else {
+    const size_t tile = (size_t)kBlockPersistent * kUnrollPersistent;
+    size_t tiles = (nvec + tile - 1) / tile;
+    size_t want = (size_t)cus * g_blocks_per_cu / (size_t)njobs;
+    if (want < 1) want = 1;
+    if (tiles > want) tiles = want;
+    g->shape = kShapePersistent;
+    g->grid_x = (unsigned)(tiles ? tiles : 1);
+    g->block = kBlockPersistent;
+  }
+  return MCCL_OK;
+}
+
+// Launch one batch of jobs (args fully populated).  Jobs whose pointers are congruent mod 16
+// go to the vector kernel; the rest to the element kernel, in at most two launches.
+int launch_jobs(ReduceArgs& a, int njobs, int dtype, int op, int variant, hipStream_t s) {
+  const size_t es = dtype_size(dtype);
+  ReduceArgs vec = a, elem = a;
+  int nv = 0, ne = 0;
+  size_t vmax = 0, emax = 0;
+  for (int j = 0; j < njobs; ++j) {
+    if (a.job_count[j] == 0) continue;
+    const uintptr_t o = (uintptr_t)a.job_out[j];
+    if (o % es) return fail(MCCL_ERR_INVALID_ARG, "output pointer not aligned to the element size");
+    bool congruent = true;
+    for (int k = 0; k < a.n; ++k) {
+      const uintptr_t p = (uintptr_t)(a.ptr[a.job_ptr0[j] + k] + a.job_in_off[j]);
+      if (p % es) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d not aligned to the element size", k);
+      if ((p & 15u) != (o & 15u)) congruent = false;
+    }
+    ReduceArgs& t = congruent ? vec : elem;
+    int& idx = congruent ? nv : ne;
+    t.job_out[idx] = a.job_out[j];
+    t.job_in_off[idx] = a.job_in_off[j];
+    t.job_count[idx] = a.job_count[j];
+    t.job_ptr0[idx] = a.job_ptr0[j];
+    ++idx;
+    size_t& mx = congruent ? vmax : emax;
+    if (a.job_count[j] > mx) mx = a.job_count[j];
+  }
+  if (nv) {
+    Geometry g;
+    int rc = plan_vec(vmax, nv, dtype, variant, &g);
+    if (rc != MCCL_OK) return rc;
+    hipError_t e = launch_any(vec, dtype, op, g.shape, dim3(g.grid_x, nv, 1), s);
+    if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
+  }
+  if (ne) {
+    int cus = 0;
+    int rc = device_cus(&cus);
+    if (rc != MCCL_OK) return rc;
+    size_t blocks = (emax + 255) / 256;
+    size_t cap = (size_t)cus * 8 / ne;
+    if (cap < 1) cap = 1;
+    if (blocks > cap) blocks = cap;
+    hipError_t e = launch_any(elem, dtype, op, kShapeElem, dim3((unsigned)blocks, ne, 1), s);
+    if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
+  }
+  return MCCL_OK;
+}
+
+int check_reduce_args(const void* const* in, int n, int dtype, int op) {
+  if (!in) return fail(MCCL_ERR_INVALID_ARG, "input pointer table is null");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  if (!valid_dtype(dtype)) return fail(MCCL_ERR_INVALID_ARG, "unknown dtype code %d", dtype);
+  if (!valid_op(op)) return fail(MCCL_ERR_INVALID_ARG, "unknown reduce op code %d", op);
+  if (op == MCCL_AVG && !float_dtype(dtype)) return fail(MCCL_ERR_UNSUPPORTED, "AVG is defined for floating-point types only");
+  return MCCL_OK;
+}
+
+int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
+  int cus = 0;
+  int rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  int i = 0;
+  while (i < nseg) {
+    CopyArgs a;
+    int m = 0;
+    uint64_t chunks = 0;
+    a.chunk_prefix[0] = 0;
+    while (i < nseg && m < kMaxSegs) {
+      const mccl_segment_t& sg = segs[i];
+      if (sg.bytes == 0) { ++i; continue; }
+      if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
+      const uint64_t c = (sg.bytes + kCopyChunk - 1) / kCopyChunk;
+      if (chunks + c > 0xffffffffull) {
+        if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "segment %d too large", i);
+        break;
+      }
+      a.seg[m] = sg;
+      chunks += c;
+      a.chunk_prefix[++m] = (uint32_t)chunks;
+      ++i;
+    }
+    if (m == 0) break;
+    a.nseg = m;
+    uint64_t grid = chunks;
+    const uint64_t cap = (uint64_t)cus * 16;
+    if (grid > cap) grid = cap;
+    hipLaunchKernelGGL(copy_segments_kernel, dim3((unsigned)grid), dim3(kCopyBlock), 0, s, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
+  }
+  return MCCL_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------
+extern "C" {
+
+int mccl_version(void) { return 100; }
+
+const char* mccl_last_error(void) { return g_err; }
+
+size_t mccl_dtype_size(int dtype) { return dtype_size(dtype); }
+
+void mccl_set_tuning(int persistent_blocks_per_cu, int block_size, int small_max_bytes) {
+  (void)block_size;
+  if (persistent_blocks_per_cu > 0) g_blocks_per_cu = persistent_blocks_per_cu;
+  if (small_max_bytes > 0) g_small_max_bytes = (size_t)small_max_bytes;
+}
+
+int mccl_query_launch(size_t count, int n, int dtype, int variant, int* block_size) {
+  (void)n;
+  if (!valid_dtype(dtype)) return fail(MCCL_ERR_INVALID_ARG, "unknown dtype code %d", dtype);
+  Geometry g;
+  int rc = plan_vec(count, 1, dtype, variant, &g);
+  if (rc != MCCL_OK) return rc;
+  if (block_size) *block_size = g.block;
+  return (int)g.grid_x;
+}
+
+int mccl_reduce_n(const void* const* in, int n, void* out, size_t count, int dtype, int op,
+                  int variant, void* stream) {
+  int rc = check_reduce_args(in, n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (count == 0) return MCCL_OK;
+  if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer is null");
+  ReduceArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int k = 0; k < n; ++k) {
+    if (!in[k]) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d is null", k);
+    a.ptr[k] = (const char*)in[k];
+  }
+  a.n = n;
+  a.job_out[0] = (char*)out;
+  a.job_count[0] = count;
+  return launch_jobs(a, 1, dtype, op, variant, (hipStream_t)stream);
+}
+
+int mccl_reduce_scatter_n(const void* const* in, int n, void* const* out, size_t shard_count,
+                          int shard_first, int shard_num, int dtype, int op, void* stream) {
+  int rc = check_reduce_args(in, n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (shard_first < 0 || shard_num < 0) return fail(MCCL_ERR_INVALID_ARG, "negative shard range");
+  if (shard_num == 0 || shard_count == 0) return MCCL_OK;
+  if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer table is null");
+  const size_t es = dtype_size(dtype);
+  ReduceArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int k = 0; k < n; ++k) {
+    if (!in[k]) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d is null", k);
+    a.ptr[k] = (const char*)in[k];
+  }
+  a.n = n;
+  for (int s0 = 0; s0 < shard_num; s0 += kMaxJobs) {
+    const int m = (shard_num - s0 < kMaxJobs) ? shard_num - s0 : kMaxJobs;
+    for (int j = 0; j < m; ++j) {
+      if (!out[s0 + j]) return fail(MCCL_ERR_INVALID_ARG, "output pointer %d is null", s0 + j);
+      a.job_out[j] = (char*)out[s0 + j];
+      a.job_in_off[j] = (size_t)(shard_first + s0 + j) * shard_count * es;
+      a.job_count[j] = shard_count;
+      a.job_ptr0[j] = 0;
+    }
+    rc = launch_jobs(a, m, dtype, op, MCCL_VARIANT_AUTO, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size_t* counts,
+                      int nbuf, int dtype, int op, void* stream) {
+  int rc = check_reduce_args(in, n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (nbuf < 0) return fail(MCCL_ERR_INVALID_ARG, "negative buffer count");
+  if (nbuf == 0) return MCCL_OK;
+  if (!out || !counts) return fail(MCCL_ERR_INVALID_ARG, "output or count table is null");
+  int per_launch = MCCL_MAX_RANKS / n;
+  if (per_launch > kMaxJobs) per_launch = kMaxJobs;
+  for (int b0 = 0; b0 < nbuf; b0 += per_launch) {
+    const int m = (nbuf - b0 < per_launch) ? nbuf - b0 : per_launch;
+    ReduceArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n = n;
+    for (int j = 0; j < m; ++j) {
+      for (int k = 0; k < n; ++k) {
+        const void* p = in[(size_t)(b0 + j) * n + k];
+        if (!p && counts[b0 + j]) return fail(MCCL_ERR_INVALID_ARG, "input pointer (%d,%d) is null", b0 + j, k);
+        a.ptr[j * n + k] = (const char*)p;
+      }
+      if (!out[b0 + j] && counts[b0 + j]) return fail(MCCL_ERR_INVALID_ARG, "output pointer %d is null", b0 + j);
+      a.job_out[j] = (char*)out[b0 + j];
+      a.job_count[j] = counts[b0 + j];
+      a.job_ptr0[j] = j * n;
+    }
+    rc = launch_jobs(a, m, dtype, op, MCCL_VARIANT_AUTO, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream) {
+  if (nseg < 0) return fail(MCCL_ERR_INVALID_ARG, "negative segment count");
+  if (nseg == 0) return MCCL_OK;
+  if (!segs) return fail(MCCL_ERR_INVALID_ARG, "segment table is null");
+  return launch_copy(segs, nseg, (hipStream_t)stream);
+}
+
+int mccl_allgather_n(const void* const* in, int n, void* out, size_t bytes_per_rank, void* stream) {
+  if (!in) return fail(MCCL_ERR_INVALID_ARG, "input pointer table is null");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  if (bytes_per_rank == 0) return MCCL_OK;
+  if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer is null");
+  mccl_segment_t segs[MCCL_MAX_RANKS];
+  for (int k = 0; k < n; ++k) {
+    if (!in[k]) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d is null", k);
+    segs[k].src = in[k];
+    segs[k].dst = (char*)out + (size_t)k * bytes_per_rank;
+    segs[k].bytes = bytes_per_rank;
+  }
+  return launch_copy(segs, n, (hipStream_t)stream);
+}
+
+int mccl_alltoallv_n(const void* const* in, void* const* out, int n, const int64_t* split_rows,
+                     size_t row_bytes, void* stream) {
+  if (!in || !out || !split_rows) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  for (int i = 0; i < n * n; ++i)
+    if (split_rows[i] < 0) return fail(MCCL_ERR_INVALID_ARG, "negative split size");
+  // One destination rank per batch of n segments.
+  mccl_segment_t segs[MCCL_MAX_RANKS];
+  for (int d = 0; d < n; ++d) {
+    size_t roff = 0;
+    int m = 0;
+    for (int r = 0; r < n; ++r) {
+      size_t soff = 0;
+      for (int dd = 0; dd < d; ++dd) soff += (size_t)split_rows[r * n + dd];
+      const size_t rows = (size_t)split_rows[r * n + d];
+      if (rows) {
+        if (!in[r] || !out[d]) return fail(MCCL_ERR_INVALID_ARG, "null buffer for a non-empty segment");
+        segs[m].src = (const char*)in[r] + soff * row_bytes;
+        segs[m].dst = (char*)out[d] + roff * row_bytes;
+        segs[m].bytes = rows * row_bytes;
+        ++m;
+      }
+      roff += rows;
+    }
+    int rc = launch_copy(segs, m, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+int mccl_alltoallv_pull(const void* const* in, int n, void* out, const size_t* send_displ_bytes,
+                        const size_t* recv_bytes, void* stream) {
+  if (!in || !send_displ_bytes || !recv_bytes) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  mccl_segment_t segs[MCCL_MAX_RANKS];
+  size_t off = 0;
+  int m = 0;
+  for (int r = 0; r < n; ++r) {
+    if (recv_bytes[r]) {
+      if (!in[r] || !out) return fail(MCCL_ERR_INVALID_ARG, "null buffer for a non-empty segment");
+      segs[m].src = (const char*)in[r] + send_displ_bytes[r];
+      segs[m].dst = (char*)out + off;
+      segs[m].bytes = recv_bytes[r];
+      ++m;
+    }
+    off += recv_bytes[r];
+  }
+  return launch_copy(segs, m, (hipStream_t)stream);
+}
+
+int mccl_pack(const void* const* src, const size_t* bytes, int n, void* dst, void* stream) {
+  if (n < 0) return fail(MCCL_ERR_INVALID_ARG, "negative count");
+  if (n == 0) return MCCL_OK;
+  if (!src || !bytes) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  size_t off = 0;
+  for (int i0 = 0; i0 < n; i0 += kMaxSegs) {
+    mccl_segment_t segs[kMaxSegs];
+    const int m = (n - i0 < kMaxSegs) ? n - i0 : kMaxSegs;
+    for (int i = 0; i < m; ++i) {
+      segs[i].src = src[i0 + i];
+      segs[i].dst = (char*)dst + off;
+      segs[i].bytes = bytes[i0 + i];
+      off += bytes[i0 + i];
+    }
+    int rc = launch_copy(segs, m, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, void* stream) {
+  if (n < 0) return fail(MCCL_ERR_INVALID_ARG, "negative count");
+  if (n == 0) return MCCL_OK;
+  if (!dst || !bytes) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  size_t off = 0;
+  for (int i0 = 0; i0 < n; i0 += kMaxSegs) {
+    mccl_segment_t segs[kMaxSegs];
+    const int m = (n - i0 < kMaxSegs) ? n - i0 : kMaxSegs;
+    for (int i = 0; i < m; ++i) {
+      segs[i].src = (const char*)src + off;
+      segs[i].dst = dst[i0 + i];
+      segs[i].bytes = bytes[i0 + i];
+      off += bytes[i0 + i];
+    }
+    int rc = launch_copy(segs, m, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+}  // extern "C"

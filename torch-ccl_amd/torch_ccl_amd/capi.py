@@ -1,0 +1,84 @@
+"""ctypes binding of libmi355ccl.so (the C ABI declared in include/mccl.h).
+
+torch is imported first on purpose: the library's HIP runtime dependency then resolves to
+the runtime torch already loaded, so both share streams and allocations.  There is no CPU
+fallback anywhere in this module: a missing library is an ImportError, a failed call is a
+RuntimeError carrying mccl_last_error().
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must precede the CDLL below)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmi355ccl.so")
+
+# dtype codes (mccl_dtype_t), mirroring cclDatatypes of the reference (src/utils.cpp:46-58)
+U8, I8, I16, I32, I64, F16, F32, F64, BF16 = range(9)
+# op codes (mccl_op_t), numbered like c10d::ReduceOp
+SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
+VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT = 0, 1, 2
+MAX_RANKS = 64
+
+TORCH_DTYPE = {
+    torch.uint8: U8, torch.int8: I8, torch.int16: I16, torch.int32: I32, torch.int64: I64,
+    torch.float16: F16, torch.float32: F32, torch.float64: F64, torch.bfloat16: BF16,
+    torch.bool: U8,
+}
+
+EXPORTS = (
+    "mccl_version", "mccl_last_error", "mccl_dtype_size", "mccl_reduce_n",
+    "mccl_reduce_scatter_n", "mccl_reduce_multi", "mccl_copy_segments", "mccl_allgather_n",
+    "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
+    "mccl_query_launch", "mccl_set_tuning",
+)
+
+
+class Segment(ctypes.Structure):
+    _fields_ = [("src", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("bytes", ctypes.c_size_t)]
+
+
+_lib = None
+
+
+def lib():
+    """Loads the shared library once; raises ImportError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "libmi355ccl.so is not built (%s); run `python torch-ccl_amd/csrc/build.py`" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    L.mccl_version.restype = i32
+    L.mccl_last_error.restype = ctypes.c_char_p
+    L.mccl_dtype_size.restype = sz
+    L.mccl_dtype_size.argtypes = [i32]
+    L.mccl_reduce_n.argtypes = [vp, i32, vp, sz, i32, i32, i32, vp]
+    L.mccl_reduce_scatter_n.argtypes = [vp, i32, vp, sz, i32, i32, i32, i32, vp]
+    L.mccl_reduce_multi.argtypes = [vp, i32, vp, vp, i32, i32, i32, vp]
+    L.mccl_copy_segments.argtypes = [vp, i32, vp]
+    L.mccl_allgather_n.argtypes = [vp, i32, vp, sz, vp]
+    L.mccl_alltoallv_n.argtypes = [vp, vp, i32, vp, sz, vp]
+    L.mccl_alltoallv_pull.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.mccl_pack.argtypes = [vp, vp, i32, vp, vp]
+    L.mccl_unpack.argtypes = [vp, vp, vp, i32, vp]
+    L.mccl_query_launch.argtypes = [sz, i32, i32, i32, vp]
+    L.mccl_set_tuning.argtypes = [i32, i32, i32]
+    L.mccl_set_tuning.restype = None
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        raise RuntimeError("mccl error %d: %s" % (rc, lib().mccl_last_error().decode()))
+
+
+def ptr_table(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+
+def size_table(sizes):
+    return (ctypes.c_size_t * len(sizes))(*[int(s) for s in sizes])

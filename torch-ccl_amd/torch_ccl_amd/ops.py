@@ -1,0 +1,170 @@
+"""Tensor-level front end of the C ABI: the N "peer" buffers are N torch tensors on one GPU.
+
+These functions only marshal pointers and sizes; the work is done by the HIP kernels in
+libmi355ccl.so on the current torch stream.  Argument checks follow the reference's
+(src/utils.cpp:217-255: contiguous, same dtype) with the device test inverted: tensors must
+live on the GPU.
+"""
+import ctypes
+
+import torch
+
+from . import capi
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check_tensors(tensors, what):
+    first = tensors[0]
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("%s: tensors must be on the GPU (got %s)" % (what, t.device))
+        if not t.is_contiguous():
+            raise RuntimeError("input dense tensor has to be contiguous")
+        if t.dtype != first.dtype:
+            raise RuntimeError("Tensors are not equal in data type")
+        if t.device != first.device:
+            raise RuntimeError("%s: tensors must share one device" % what)
+
+
+def _dtype_code(dtype):
+    try:
+        return capi.TORCH_DTYPE[dtype]
+    except KeyError:
+        raise RuntimeError("unsupported data type %s" % dtype) from None
+
+
+def reduce_n(inputs, out=None, op=capi.SUM, variant=capi.VARIANT_AUTO):
+    """out[i] = inputs[0][i] op ... op inputs[N-1][i] in ascending rank order.
+    out may be one of the inputs (the in-place allreduce of the reference)."""
+    if out is None:
+        out = torch.empty_like(inputs[0])
+    _check_tensors(list(inputs) + [out], "reduce_n")
+    count = out.numel()
+    for t in inputs:
+        if t.numel() != count:
+            raise RuntimeError("reduce_n: all buffers must have the same number of elements")
+    with torch.cuda.device(out.device):
+        rc = capi.lib().mccl_reduce_n(capi.ptr_table([t.data_ptr() for t in inputs]), len(inputs),
+                                      out.data_ptr(), count, _dtype_code(out.dtype), op, variant,
+                                      _stream())
+    capi.check(rc)
+    return out
+
+
+def reduce_scatter_n(inputs, outputs, op=capi.SUM, shard_first=0):
+    """outputs[s] = reduction over ranks of inputs[k][(shard_first+s)*M : (shard_first+s+1)*M]."""
+    _check_tensors(list(inputs) + list(outputs), "reduce_scatter_n")
+    m = outputs[0].numel()
+    for o in outputs:
+        if o.numel() != m:
+            raise RuntimeError("reduce_scatter_n: shard outputs must have equal sizes")
+    for t in inputs:
+        if t.numel() < (shard_first + len(outputs)) * m:
+            raise RuntimeError("input tensor must be the same size as output size times world size")
+    with torch.cuda.device(outputs[0].device):
+        rc = capi.lib().mccl_reduce_scatter_n(
+            capi.ptr_table([t.data_ptr() for t in inputs]), len(inputs),
+            capi.ptr_table([o.data_ptr() for o in outputs]), m, shard_first, len(outputs),
+            _dtype_code(outputs[0].dtype), op, _stream())
+    capi.check(rc)
+    return outputs
+
+
+def reduce_multi(input_lists, outputs, op=capi.SUM):
+    """Coalesced reductions: input_lists[b] is the list of N rank buffers of bucket b."""
+    n = len(input_lists[0])
+    flat = []
+    for b, ins in enumerate(input_lists):
+        if len(ins) != n:
+            raise RuntimeError("reduce_multi: every bucket needs the same rank count")
+        _check_tensors(list(ins) + [outputs[b]], "reduce_multi")
+        for t in ins:
+            if t.numel() != outputs[b].numel():
+                raise RuntimeError("reduce_multi: bucket %d size mismatch" % b)
+            flat.append(t.data_ptr())
+    for o in outputs:
+        if o.dtype != outputs[0].dtype:
+            raise RuntimeError("Tensors are not equal in data type")
+    with torch.cuda.device(outputs[0].device):
+        rc = capi.lib().mccl_reduce_multi(
+            capi.ptr_table(flat), n, capi.ptr_table([o.data_ptr() for o in outputs]),
+            capi.size_table([o.numel() for o in outputs]), len(outputs),
+            _dtype_code(outputs[0].dtype), op, _stream())
+    capi.check(rc)
+    return outputs
+
+
+def allgather_n(inputs, out):
+    """out[k*M:(k+1)*M] = inputs[k]."""
+    _check_tensors(list(inputs) + [out], "allgather_n")
+    m = inputs[0].numel()
+    for t in inputs:
+        if t.numel() != m:
+            raise RuntimeError("allgather_n: inputs must have equal sizes")
+    if out.numel() != m * len(inputs):
+        raise RuntimeError("output tensor size must be equal to world_size times input tensor size")
+    with torch.cuda.device(out.device):
+        rc = capi.lib().mccl_allgather_n(capi.ptr_table([t.data_ptr() for t in inputs]), len(inputs),
+                                         out.data_ptr(), m * out.element_size(), _stream())
+    capi.check(rc)
+    return out
+
+
+def alltoallv_n(inputs, outputs, split_rows):
+    """All ranks' alltoall(v): split_rows[r][d] = dim-0 rows rank r sends to rank d."""
+    _check_tensors(list(inputs) + list(outputs), "alltoallv_n")
+    n = len(inputs)
+    S = torch.as_tensor(split_rows, dtype=torch.int64).reshape(n, n).contiguous()
+    row_bytes = None
+    for t in list(inputs) + list(outputs):
+        if t.numel():
+            rb = t.numel() // t.shape[0] * t.element_size()
+            if row_bytes is None:
+                row_bytes = rb
+            elif rb != row_bytes:
+                raise RuntimeError("alltoallv_n: all tensors need the same row length")
+    if row_bytes is None:
+        return outputs
+    for r in range(n):
+        if inputs[r].shape[0] != int(S[r].sum()):
+            raise RuntimeError("Tensor's dim 0 does not match sum of splits")
+        if outputs[r].shape[0] != int(S[:, r].sum()):
+            raise RuntimeError("Tensor's dim 0 does not match sum of splits")
+    with torch.cuda.device(outputs[0].device):
+        rc = capi.lib().mccl_alltoallv_n(capi.ptr_table([t.data_ptr() for t in inputs]),
+                                         capi.ptr_table([t.data_ptr() for t in outputs]), n,
+                                         ctypes.c_void_p(S.data_ptr()), row_bytes, _stream())
+    capi.check(rc)
+    return outputs
+
+
+def copy_segments(segments):
+    """segments: iterable of (src_ptr, dst_ptr, nbytes)."""
+    segs = list(segments)
+    arr = (capi.Segment * len(segs))(*[capi.Segment(s, d, b) for (s, d, b) in segs])
+    capi.check(capi.lib().mccl_copy_segments(arr, len(segs), _stream()))
+
+
+def pack(srcs, dst):
+    """dst = concatenation of the flattened srcs (byte-exact)."""
+    _check_tensors(list(srcs) + [dst], "pack")
+    sizes = [t.numel() * t.element_size() for t in srcs]
+    if sum(sizes) != dst.numel() * dst.element_size():
+        raise RuntimeError("pack: destination size does not match the sources")
+    capi.check(capi.lib().mccl_pack(capi.ptr_table([t.data_ptr() for t in srcs]),
+                                    capi.size_table(sizes), len(srcs), dst.data_ptr(), _stream()))
+    return dst
+
+
+def unpack(src, dsts):
+    """Inverse of pack: scatter consecutive byte ranges of src into dsts."""
+    _check_tensors([src] + list(dsts), "unpack")
+    sizes = [t.numel() * t.element_size() for t in dsts]
+    if sum(sizes) != src.numel() * src.element_size():
+        raise RuntimeError("unpack: source size does not match the destinations")
+    capi.check(capi.lib().mccl_unpack(src.data_ptr(), capi.ptr_table([t.data_ptr() for t in dsts]),
+                                      capi.size_table(sizes), len(dsts), _stream()))
+    return dsts
