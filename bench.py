@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 8-rank bf16 allreduce local-reduce on one MI355X.
+
+A "step" is one pass of the hot path over one batch: one N-buffer reduction of the
+headline workload (8 rank buffers of bf16 [4096 x 8192], 64 MiB each, already resident
+in HBM, reduced with fp32 accumulation into one bf16 output).  The line printed at the end
+carries the whole-job throughput in algorithmic GB/s ((N+1) * S bytes per step), the HBM
+roofline fraction of the kernel measured with HIP events on the launch stream, the p50/p99
+latency of the 256 KiB decode-sized allreduce, and a CPU baseline (the oracle port, OpenMP)
+timed on this host's cores on the same workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extras all|none|c1,c2,c4,c5,variants]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
+
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published peak
+SEED = 1234
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def rank_generator(torch, seed, rank, device="cpu"):
+    return torch.Generator(device=device).manual_seed(seed * 1_000_003 + rank)
+
+
+def make_rank_buffers(torch, n, count, dtype, std, dev, on_device=False):
+    """One buffer per rank: fp32 N(0, std) from the (seed, rank) generator, rounded to dtype."""
+    bufs = []
+    for r in range(n):
+        if on_device:
+            g = rank_generator(torch, SEED, r, dev)
+            x = torch.empty(count, dtype=dtype, device=dev)
+            step = 1 << 26
+            for lo in range(0, count, step):
+                hi = min(count, lo + step)
+                x[lo:hi] = (torch.randn(hi - lo, generator=g, dtype=torch.float32, device=dev) * std).to(dtype)
+            bufs.append(x)
+        else:
+            g = rank_generator(torch, SEED, r)
+            bufs.append((torch.randn(count, generator=g, dtype=torch.float32) * std).to(dtype).to(dev))
+    return bufs
+
+
+def percentile(sorted_vals, q):
+    i = min(len(sorted_vals) - 1, max(0, int(round(q * (len(sorted_vals) - 1)))))
+    return sorted_vals[i]
+
+
+def cpu_baseline(torch, host_inputs, n, count):
+    """The oracle port (plain C, OpenMP) on this host: same workload, bounded to ~10-20 s."""
+    import numpy as np
+    from oracle import oracle as O
+    threads = min(16, O.max_threads(), len(os.sched_getaffinity(0)))
+    O.set_threads(threads)
+    ins = [t.view(torch.int16).numpy().view(np.uint16) for t in host_inputs]
+    t0 = time.perf_counter()
+    O.reduce(ins, O.BF16, O.SUM)  # warm-up pass, also gives a cost estimate
+    one = time.perf_counter() - t0
+    passes = max(3, min(50, int(12.0 / max(one, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        out = O.reduce(ins, O.BF16, O.SUM)
+    dt = (time.perf_counter() - t0) / passes
+    O.set_threads(1)
+    gbs = (n + 1) * count * 2 / dt / 1e9
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%d full-size passes of the headline workload (8 x 64 MiB bf16 -> 64 MiB) through "
+                      "oracle/mccl_oracle.c with %d OpenMP threads; %.1f ms per pass" % (passes, threads, dt * 1e3),
+            "ms_per_step": round(dt * 1e3, 3)}, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--extras", default="all",
+                    help="comma list of c1,c2,c4,c5,variants,gloo or all/none")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build measures the single-GPU local-reduce path only; "
+            "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
+        sys.exit(2)
+
+    extras = set("c1,c2,c4,c5,variants,gloo".split(",")) if args.extras == "all" else \
+        set() if args.extras == "none" else set(args.extras.split(","))
+
+    import torch
+    import torch_ccl_amd as mccl
+    from torch_ccl_amd import benchlib, capi
+
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the HIP path cannot run here.")
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(0)
+    log("device: %s, %d CUs, %.0f GiB" % (props.name, props.multi_processor_count, props.total_memory / 2**30))
+
+    # ---------------- headline workload: C3 ----------------
+    N, COUNT = 8, 4096 * 8192
+    S = COUNT * 2
+    host_inputs = []
+    for r in range(N):
+        g = rank_generator(torch, SEED, r)
+        host_inputs.append((torch.randn(COUNT, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16))
+    ins = [t.to(dev) for t in host_inputs]
+    out = torch.empty(COUNT, dtype=torch.bfloat16, device=dev)
+    alg_bytes = (N + 1) * S
+
+    # warm-up steps (untimed), then EXACTLY K timed steps between two synchronisations
+    for _ in range(args.warmup):
+        mccl.reduce_n(ins, out=out, op=mccl.SUM)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev_us = benchlib.reduce_throughput([ins], [out], variant=capi.VARIANT_AUTO, warmup=0, iters=args.steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = alg_bytes * args.steps / wall / 1e9
+    achieved = alg_bytes / (ev_us * 1e-6) / 1e9
+    blk, lds = ctypes.c_int(0), ctypes.c_int(0)
+    grid = capi.lib().mccl_query_launch(COUNT, N, capi.BF16, capi.SUM, capi.VARIANT_AUTO,
+                                        ctypes.byref(blk), ctypes.byref(lds))
+    log("C3: %.1f us/launch (events), %.1f GB/s, %.1f%% of peak; wall %.1f us/step" % (
+        ev_us, achieved, achieved / PEAK_HBM_GBS * 100, ms_per_step * 1e3))
+
+    result = {
+        "metric": "8-rank bf16 allreduce local-reduce HBM GB/s (% of peak); p50 us at 256 KB",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, f32 accumulation",
+        "data": "synthetic: N(0,0.02) per (seed=1234, rank), rounded to bf16",
+        "config": {"workload": "C3 allreduce SUM, 8 rank buffers x bf16 [4096 x 8192] (64 MiB each) -> one bf16 "
+                               "output, all resident in one GPU's HBM",
+                   "ranks": N, "elements_per_rank": COUNT, "algorithmic_bytes_per_step": alg_bytes,
+                   "kernel": "reduce_vec_kernel<bf16,SUM,8 ranks> shape=stream grid=%d block=%d lds=%d" % (
+                       grid, blk.value, lds.value)},
+        "pct_of_peak": round(value / PEAK_HBM_GBS * 100, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None,
+                     "kernel_us": round(ev_us, 2),
+                     "note": "achieved = (N+1)*S algorithmic bytes / average launch duration from one HIP "
+                             "event pair around the K timed launches on the launch stream"},
+    }
+
+    # parity spot check of the timed output against an on-device fp32 chain
+    acc = torch.zeros(COUNT, dtype=torch.float32, device=dev)
+    for t in ins:
+        acc += t.float()
+    same = torch.equal(out.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+    result["parity_check"] = "bit-exact vs on-device fp32 chain" if same else "MISMATCH"
+    del acc
+
+    # ---------------- C2: 256 KiB latency ----------------
+    if "c2" in extras:
+        c2 = 16 * 8192
+        sets = 16  # 16 sets x 9 buffers x 256 KiB = 36 MiB rotate through the caches
+        in_sets = [make_rank_buffers(torch, N, c2, torch.bfloat16, 0.02, dev) for _ in range(sets)]
+        outs = [torch.empty(c2, dtype=torch.bfloat16, device=dev) for _ in range(sets)]
+        lat = {}
+        for name, nsets in (("resident", 1), ("rotating", sets)):
+            for vname, v in (("small", capi.VARIANT_SMALL), ("persistent", capi.VARIANT_PERSISTENT)):
+                us = sorted(benchlib.reduce_latency(in_sets[:nsets], outs[:nsets], variant=v, warmup=100, iters=1000))
+                lat["%s_%s" % (vname, name)] = {"p50_us": round(percentile(us, 0.5), 2),
+                                                "p99_us": round(percentile(us, 0.99), 2),
+                                                "min_us": round(us[0], 2)}
+        b2b = benchlib.reduce_throughput(in_sets[:1], outs[:1], variant=capi.VARIANT_SMALL, warmup=100, iters=1000)
+        lat["small_back_to_back_us"] = round(b2b, 2)
+        lat["iters"] = 1000
+        lat["workload"] = "C2 allreduce SUM, 8 x bf16 [16 x 8192] (256 KiB each), one HIP event pair per call"
+        result["latency_256KB"] = lat
+        result["p50_us_256KB"] = lat["small_resident"]["p50_us"]
+        log("C2:", json.dumps(lat))
+        del in_sets, outs
+
+    # ---------------- evidence for the shape choice on C3 and C2 ----------------
+    if "variants" in extras:
+        ev = {}
+        for vname, v in (("small", capi.VARIANT_SMALL), ("persistent", capi.VARIANT_PERSISTENT),
+                         ("stream", capi.VARIANT_STREAM)):
+            us = benchlib.reduce_throughput([ins], [out], variant=v, warmup=5, iters=30)
+            ev[vname] = {"us": round(us, 1), "GBps": round(alg_bytes / us / 1e3, 1)}
+        result["c3_shapes"] = ev
+        log("C3 shapes:", json.dumps(ev))
+
+    # ---------------- C1: fp32, 2 ranks, 16 MiB ----------------
+    if "c1" in extras:
+        c1 = 4_194_304
+        a = []
+        for r in range(2):
+            g = rank_generator(torch, SEED, r)
+            a.append((torch.rand(c1, generator=g, dtype=torch.float32) * 2 - 1).to(dev))
+        o = torch.empty(c1, dtype=torch.float32, device=dev)
+        us = benchlib.reduce_throughput([a], [o], warmup=20, iters=200)
+        ok = torch.equal(o, a[0] + a[1])
+        result["c1_fp32_2ranks_16MiB"] = {"us": round(us, 2), "GBps": round(3 * c1 * 4 / us / 1e3, 1), "bit_exact": ok}
+        log("C1:", json.dumps(result["c1_fp32_2ranks_16MiB"]))
+        del a, o
+
+    # ---------------- C4: reduce_scatter, 8 x 1 GiB ----------------
+    if "c4" in extras:
+        c4 = 536_870_912
+        m = c4 // N
+        big = make_rank_buffers(torch, N, c4, torch.bfloat16, 1e-3, dev, on_device=True)
+        shards = [torch.empty(m, dtype=torch.bfloat16, device=dev) for _ in range(N)]
+        us_all = benchlib.reduce_scatter_throughput(big, shards, 0, warmup=2, iters=5)
+        us_one = benchlib.reduce_scatter_throughput(big, shards[3:4], 3, warmup=2, iters=10)
+        # parity on one shard against an on-device fp32 chain
+        acc = torch.zeros(m, dtype=torch.float32, device=dev)
+        for t in big:
+            acc += t[5 * m:6 * m].float()
+        ok = torch.equal(shards[5].view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+        result["c4_reduce_scatter_8x1GiB"] = {
+            "all_shards_us": round(us_all, 1), "all_shards_GBps": round((N + 1) * c4 * 2 / us_all / 1e3, 1),
+            "one_shard_us": round(us_one, 1), "one_shard_GBps": round((N + 1) * m * 2 / us_one / 1e3, 1),
+            "shard5_bit_exact_vs_fp32_chain": ok}
+        log("C4:", json.dumps(result["c4_reduce_scatter_8x1GiB"]))
+        del big, shards, acc
+
+    # ---------------- C5: MoE dispatch all_to_all_single, uneven splits ----------------
+    if "c5" in extras:
+        tokens, hidden, topk, n_exp = 4096, 7168, 8, 256
+        per_rank = n_exp // N
+        S5 = torch.zeros(N, N, dtype=torch.int64)
+        a2a_in = []
+        for r in range(N):
+            g = rank_generator(torch, SEED, r)
+            logits = torch.randn(tokens, n_exp, generator=g)
+            experts = torch.topk(logits, topk, dim=1).indices
+            dest = (experts.reshape(-1) // per_rank)
+            S5[r] = torch.bincount(dest, minlength=N)
+            gd = rank_generator(torch, SEED, r, dev)
+            a2a_in.append(torch.randn(tokens * topk, hidden, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16))
+        a2a_out = [torch.empty(int(S5[:, d].sum()), hidden, dtype=torch.bfloat16, device=dev) for d in range(N)]
+        us = benchlib.alltoallv_throughput(a2a_in, a2a_out, S5, hidden * 2, warmup=2, iters=5)
+        moved = int(S5.sum()) * hidden * 2
+        # byte-exact spot check of one (source, destination) segment
+        r, d = 2, 6
+        so = int(S5[r, :d].sum()); ro = int(S5[:r, d].sum()); rows = int(S5[r, d])
+        ok = torch.equal(a2a_out[d][ro:ro + rows], a2a_in[r][so:so + rows])
+        result["c5_alltoallv_moe"] = {"us": round(us, 1), "GBps": round(2 * moved / us / 1e3, 1),
+                                      "bytes_moved": moved, "n_experts": n_exp, "experts_per_rank": per_rank,
+                                      "segment_2_to_6_byte_exact": ok,
+                                      "split_rows_rank0": S5[0].tolist()}
+        log("C5:", json.dumps(result["c5_alltoallv_moe"]))
+        del a2a_in, a2a_out
+
+    # ---------------- CPU baseline (the oracle port) ----------------
+    if not args.no_cpu:
+        cb, cpu_out = cpu_baseline(torch, host_inputs, N, COUNT)
+        result["cpu_baseline"] = cb
+        import numpy as np
+        gpu_bits = out.cpu().view(torch.int16).numpy().view(np.uint16)
+        result["cpu_baseline"]["gpu_matches_cpu_bit_exact"] = bool(np.array_equal(gpu_bits, cpu_out))
+        log("CPU:", json.dumps(cb))
+    else:
+        result["cpu_baseline"] = None
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -56,13 +56,26 @@ typedef enum {
   MCCL_ERR_UNSUPPORTED = -3
 } mccl_status_t;
 
-/* Kernel variant of the reduction (the reference switches at SMALL_MAX_COUNT between a
+/* Launch shape of the reduction (the reference switches at SMALL_MAX_COUNT between a
  * single-launch kernel and a persistent one, src/gpu/dpcpp_ccl.cpp:771-775). */
 typedef enum {
-  MCCL_VARIANT_AUTO = 0,      /* pick by message size */
-  MCCL_VARIANT_SMALL = 1,     /* one vector per lane, grid covers the message */
-  MCCL_VARIANT_PERSISTENT = 2 /* fixed grid sized to the CUs, grid-stride loop */
+  MCCL_VARIANT_AUTO = 0,       /* pick by message size: SMALL up to the threshold, else STREAM */
+  MCCL_VARIANT_SMALL = 1,      /* one wavefront per workgroup, one vector per lane, grid covers
+                                  the message, no residency cap: lowest latency */
+  MCCL_VARIANT_PERSISTENT = 2, /* fixed grid sized to the CUs, grid-stride loop */
+  MCCL_VARIANT_STREAM = 3      /* SMALL's geometry with residency capped (through a dynamic-LDS
+                                  reservation) so that ~64 KiB of loads are in flight per CU:
+                                  highest bandwidth on large messages */
 } mccl_variant_t;
+
+/* Tuning knobs for mccl_set_tuning (process-wide; meant for benchmarks and sweeps). */
+typedef enum {
+  MCCL_TUNE_PERSISTENT_BLOCKS_PER_CU = 0, /* grid of the PERSISTENT shape */
+  MCCL_TUNE_STREAM_INFLIGHT_BYTES = 1,    /* load bytes in flight per CU, STREAM shape */
+  MCCL_TUNE_SMALL_MAX_BYTES = 2,          /* per-rank bytes up to which AUTO picks SMALL */
+  MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
+  MCCL_TUNE_COUNT_ = 4
+} mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64
 
@@ -141,12 +154,15 @@ int mccl_alltoallv_pull(const void* const* in, int n, void* out, const size_t* s
 int mccl_pack(const void* const* src, const size_t* bytes, int n, void* dst, void* stream);
 int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, void* stream);
 
-/* Launch geometry the library would use (for reports): returns grid size in workgroups and
- * writes the workgroup size; count in elements. */
-int mccl_query_launch(size_t count, int n, int dtype, int variant, int* block_size);
+/* Launch geometry the library would use for mccl_reduce_n (for reports): returns the grid
+ * size in workgroups (negative = mccl_status_t) and writes the workgroup size and the
+ * dynamic-LDS reservation; count in elements. */
+int mccl_query_launch(size_t count, int n, int dtype, int op, int variant, int* block_size,
+                      int* lds_bytes);
 
-/* Tuning knobs (process-wide; <= 0 keeps the default).  Meant for benchmarks. */
-void mccl_set_tuning(int persistent_blocks_per_cu, int block_size, int small_max_bytes);
+/* Sets a knob of mccl_tune_t; value <= 0 restores the default. */
+int mccl_set_tuning(int knob, long long value);
+long long mccl_get_tuning(int knob);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,55 @@
+/*
+ * mccl_bench.h -- timing loops around the C ABI of include/mccl.h (libmcclbench.so).
+ *
+ * Benchmark support only: these loops call the product entry points unchanged and time
+ * them with HIP events recorded on the launch stream, so that per-call latencies are not
+ * polluted by interpreter overhead.  They have no counterpart in the reference (whose
+ * timing scripts, tests/ddp_allreduce.py:86-117, time from the host).
+ */
+#ifndef MCCL_BENCH_H_
+#define MCCL_BENCH_H_
+
+#include "mccl.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Per-call latency of mccl_reduce_n: `iters` calls, one event pair per call, us_out[i] =
+ * microseconds of call i.  `in` holds nsets*n pointers and `out` nsets pointers; call i
+ * uses set i % nsets (nsets > 1 rotates buffers so the caches do not hold the inputs).
+ */
+int mcclb_reduce_latency(const void* const* in, int n, void* const* out, int nsets, size_t count,
+                         int dtype, int op, int variant, void* stream, int warmup, int iters,
+                         float* us_out);
+
+/* Back-to-back throughput: one event pair around `iters` consecutive calls; *total_us =
+ * elapsed microseconds for all of them. */
+int mcclb_reduce_throughput(const void* const* in, int n, void* const* out, int nsets,
+                            size_t count, int dtype, int op, int variant, void* stream, int warmup,
+                            int iters, float* total_us);
+
+/* The same two loops around mccl_reduce_scatter_n (all shards of one launch). */
+int mcclb_reduce_scatter_throughput(const void* const* in, int n, void* const* out,
+                                    size_t shard_count, int shard_first, int shard_num, int dtype,
+                                    int op, void* stream, int warmup, int iters, float* total_us);
+
+/* ... and around mccl_copy_segments. */
+int mcclb_copy_latency(const mccl_segment_t* segs, int nseg, void* stream, int warmup, int iters,
+                       float* us_out);
+int mcclb_copy_throughput(const mccl_segment_t* segs, int nseg, void* stream, int warmup,
+                          int iters, float* total_us);
+
+/* ... and around mccl_alltoallv_n (all ranks). */
+int mcclb_alltoallv_throughput(const void* const* in, void* const* out, int n,
+                               const int64_t* split_rows, size_t row_bytes, void* stream,
+                               int warmup, int iters, float* total_us);
+
+const char* mcclb_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MCCL_BENCH_H_ */

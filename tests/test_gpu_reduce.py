@@ -30,7 +30,7 @@ def test_reduce_all_dtypes_ops(mccl, dtype, opname, n):
     count = 5000  # not a multiple of the vector width: head/tail paths run
     scale = 1.0 if opname == "prod" else 0.02
     ins = [rank_buffer(count, dtype, r, scale=scale) for r in range(n)]
-    for variant in (1, 2):
+    for variant in (1, 2, 3):
         got = _run(mccl, ins, OPS[opname], variant)
         assert_bits_equal(bits(got), oracle_reduce_bits(ins, OPS[opname]),
                           "%s %s n=%d variant=%d" % (dtype, opname, n, variant))
@@ -96,7 +96,7 @@ def test_reduce_in_place(mccl, dtype, which):
     n, count = 8, 70001
     ins = [rank_buffer(count, dtype, r) for r in range(n)]
     want = oracle_reduce_bits(ins)
-    for variant in (1, 2):
+    for variant in (1, 2, 3):
         dev = [t.to(DEV) for t in ins]
         mccl.reduce_n(dev, out=dev[which], op=O.SUM, variant=variant)
         torch.cuda.synchronize()
@@ -192,7 +192,7 @@ def test_config1_fp32_two_ranks_16mib(mccl):
     assert_bits_equal(bits(got), oracle_reduce_bits(ins), "C1 vs oracle")
 
 
-@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("variant", [1, 2, 3])
 def test_config2_bf16_decode_256k(mccl, variant):
     """bf16 [16 x 8192] per rank, 8 ranks, N(0, 0.02), fp32 accumulation."""
     ins = [rank_buffer(16 * 8192, torch.bfloat16, r) for r in range(8)]
@@ -206,12 +206,14 @@ def test_config3_bf16_prefill_64mib(mccl):
     count = 4096 * 8192
     ins = [rank_buffer(count, torch.bfloat16, r) for r in range(8)]
     dev = [t.to(DEV) for t in ins]
-    got = mccl.reduce_n(dev, op=O.SUM, variant=2)
-    torch.cuda.synchronize()
     acc = torch.zeros(count, dtype=torch.float32, device=DEV)
     for t in dev:
         acc += t.float()
-    assert torch.equal(got.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+    chain = acc.to(torch.bfloat16).view(torch.int16)
+    for variant in (0, 2, 3):
+        got = mccl.reduce_n(dev, op=O.SUM, variant=variant)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), chain), "variant %d" % variant
     O.set_threads(min(16, O.max_threads()))
     try:
         want = oracle_reduce_bits(ins)

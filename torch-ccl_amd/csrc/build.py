@@ -1,6 +1,7 @@
 """Builds the native pieces in-tree for gfx950.
 
   libmi355ccl.so   HIP kernels + C ABI (include/mccl.h); depends on the HIP runtime only.
+  libmcclbench.so  HIP-event timing loops around that ABI (include/mccl_bench.h).
 
 Usage: python torch-ccl_amd/csrc/build.py [--force]
 Outputs land in torch-ccl_amd/torch_ccl_amd/lib/.
@@ -45,8 +46,24 @@ def build_kernels(force=False, extra_flags=(), out=KERNEL_LIB):
     return out
 
 
+BENCH_SRC = os.path.join(HERE, "mccl_bench.cpp")
+BENCH_LIB = os.path.join(LIB_DIR, "libmcclbench.so")
+
+
+def build_bench(force=False):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    srcs = [BENCH_SRC, os.path.join(INCLUDE, "mccl_bench.h"), os.path.join(INCLUDE, "mccl.h")]
+    if force or _stale(BENCH_LIB, srcs):
+        cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-I", INCLUDE, "-o", BENCH_LIB, BENCH_SRC,
+               "-L", LIB_DIR, "-lmi355ccl", "-Wl,-rpath,$ORIGIN"]
+        subprocess.check_call(cmd)
+    return BENCH_LIB
+
+
 def build_all(force=False):
-    return [build_kernels(force)]
+    return [build_kernels(force), build_bench(force)]
 
 
 if __name__ == "__main__":

@@ -1,0 +1,71 @@
+"""Guard against a code-generation hazard seen with hipcc on gfx950: a uniform 64-bit
+compare + select lowered to `v_cmp_*_u64 vcc` ... `s_cselect_b32` where the instruction
+that should turn vcc into SCC has been dropped, so the select consumes the carry bit of an
+unrelated scalar add/sub.  The kernels avoid the source pattern (uniform 64-bit min/max);
+this script compiles the device code to assembly and scans every kernel for a scalar
+select or SCC branch whose nearest SCC writer in the same straight-line region is an
+arithmetic instruction rather than a compare or mask operation.
+
+Usage: python torch-ccl_amd/csrc/check_isa.py   (exit status 1 if anything is flagged)
+"""
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+import build as _build  # noqa: E402
+
+_COMPARE = re.compile(r"^(s_cmp|s_cmpk|s_bitcmp|s_and_b|s_or_b|s_xor_b|s_andn2_b|s_orn2_b|s_lshr_b|s_bfe_|"
+                      r"s_and_saveexec|s_or_saveexec|s_andn2_saveexec|s_not_b)")
+_ARITH = re.compile(r"^(s_add_|s_sub_|s_addc_|s_subb_|s_lshl_b|s_ashr_|s_min_|s_max_|s_abs_|s_absdiff_|"
+                    r"s_lshl[1-4]_add_)")
+_USER = re.compile(r"^(s_cselect_|s_cbranch_scc)")
+
+
+def device_asm(out_path):
+    flags = [f for f in _build.HIP_FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [_build.HIPCC] + flags + ["--cuda-device-only", "-S", "-o", out_path, _build.KERNEL_SRC]
+    subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
+
+
+def scan(asm_path):
+    """Returns a list of (line_no, instruction, scc_source, function)."""
+    flagged = []
+    fn, last = None, None
+    with open(asm_path) as f:
+        for ln, line in enumerate(f, 1):
+            t = line.strip()
+            if not t or t.startswith(";"):
+                continue
+            if t.startswith(".LBB"):
+                last = None  # SCC may arrive from another block: not judged
+                continue
+            if t.startswith("."):
+                continue
+            if re.match(r"^[A-Za-z_][\w.$]*:", t):
+                fn, last = t.split(":")[0], None
+                continue
+            op = t.split()[0]
+            if _USER.match(op) and last is not None and _ARITH.match(last[0]):
+                flagged.append((ln, t, last[1], fn))
+            if _COMPARE.match(op) or _ARITH.match(op):
+                last = (op, t)
+    return flagged
+
+
+def main():
+    with tempfile.TemporaryDirectory() as d:
+        asm = os.path.join(d, "mccl_kernels.s")
+        device_asm(asm)
+        flagged = scan(asm)
+    for ln, ins, src, fn in flagged:
+        print("line %d in %s: `%s` takes SCC from `%s`" % (ln, fn, ins, src))
+    print("flagged: %d" % len(flagged))
+    return 1 if flagged else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

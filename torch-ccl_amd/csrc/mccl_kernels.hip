@@ -8,9 +8,21 @@
 //   * accumulation is a sequential ascending-rank chain held in registers (fp32 for
 //     f16/bf16), one round-to-nearest-even on store;
 //   * outputs are written with non-temporal stores (streamed past the caches);
-//   * a "small" launch gives every lane exactly one vector (grid covers the message, one
-//     wavefront per workgroup so all CUs are used); the "persistent" launch uses a fixed
-//     grid proportional to the CU count and walks tiles grid-stride;
+//   * inputs are read with non-temporal loads: nothing is reused, and on this part the
+//     streaming hint alone is worth about 12 % of bandwidth;
+//   * launch shapes (same kernel code, different geometry):
+//       small      one wavefront per workgroup, one vector per lane, grid covers the
+//                  message: a 256 KiB message lands on all 256 CUs in one launch;
+//       stream     the same geometry plus a dynamic-LDS reservation that caps residency at
+//                  W wavefronts per CU, W chosen so that about 64 KiB of loads are in
+//                  flight per CU.  The hardware dispatcher hands out tiles in address
+//                  order, so the set of live tiles is a compact window that sweeps the
+//                  buffers; with more resident wavefronts the window widens, DRAM pages
+//                  are re-opened more often and bandwidth drops (measured: 87 % of peak
+//                  at W = 8 for eight inputs against 75 % uncapped);
+//       persistent a fixed grid proportional to the CU count walking tiles grid-stride
+//                  (kept selectable; measured slower than "stream" on MI355X because the
+//                  workgroups drift apart and the live window smears);
 //   * misaligned heads/tails are peeled element-wise inside the same launch; pointer sets
 //     that are not mutually congruent mod 16 take an element-wise kernel.
 //
@@ -56,17 +68,35 @@ int fail(int code, const char* fmt, ...) {
 // ------------------------------------------------------------------------------------------
 // tuning state and per-device facts
 // ------------------------------------------------------------------------------------------
-constexpr int kBlockPersistent = 256;  // 4 wavefronts
-constexpr int kBlockSmall = 64;        // 1 wavefront: spreads a small message over all CUs
-constexpr int kUnrollPersistent = 2;   // vectors per lane per input per tile
-constexpr int kMaxJobs = 64;           // independent reductions per launch
-constexpr int kMaxSegs = 64;           // copy segments per launch
-constexpr int kCopyBlock = 256;
-constexpr int kCopyUnroll = 4;
-constexpr size_t kCopyChunk = (size_t)kCopyBlock * 16 * kCopyUnroll;  // 16 KiB per chunk
+constexpr int kWave = 64;               // one wavefront per workgroup (small / stream shapes)
+constexpr int kBlockPersistent = 256;   // 4 wavefronts
+constexpr int kUnrollPersistent = 2;    // vectors per lane per input per tile
+constexpr int kMaxJobs = 64;            // independent reductions per launch
+constexpr int kMaxSegs = 64;            // copy segments per launch
+constexpr int kCopyUnroll = 2;          // vectors per lane per chunk
+constexpr size_t kCopyChunk = (size_t)kWave * 16 * kCopyUnroll;  // 2 KiB per wavefront
+constexpr unsigned kMaxGridX = 1u << 24;  // larger messages wrap through the grid-stride loop
+constexpr size_t kLdsPerCu = 160 * 1024;  // gfx950
+constexpr int kMaxWavesPerCu = 32;
 
-int g_blocks_per_cu = 8;
-size_t g_small_max_bytes = 2u << 20;  // per-rank bytes up to which AUTO picks "small"
+// tunables (mccl_set_tuning); defaults come from sweeps on MI355X
+long long g_tune[MCCL_TUNE_COUNT_] = {
+    /* PERSISTENT_BLOCKS_PER_CU */ 8,
+    /* STREAM_INFLIGHT_BYTES    */ 72 * 1024,
+    /* SMALL_MAX_BYTES          */ 1 << 20,
+    /* COPY_WAVES_PER_CU        */ 28,
+};
+const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 72 * 1024, 1 << 20, 28};
+
+// Dynamic-LDS bytes that limit residency to `waves` single-wavefront workgroups per CU
+// (0 = no reservation needed).
+unsigned lds_for_waves(long long waves) {
+  if (waves >= kMaxWavesPerCu) return 0;
+  if (waves < 1) waves = 1;
+  size_t b = (kLdsPerCu / (size_t)waves) & ~(size_t)511;
+  if (b > 64 * 1024) b = 64 * 1024;
+  return (unsigned)b;
+}
 
 struct DeviceFacts {
   int cus = 0;
@@ -197,15 +227,25 @@ __device__ __forceinline__ typename Elem<DT>::acc_t chain_last(typename Elem<DT>
   else return acc;
 }
 
-// Kernel arguments.  ptr[] holds input base pointers; job j reads ptr[job_ptr0[j] + k] +
-// job_in_off[j] for k < n and writes job_out[j].  reduce_n: one job.  reduce_scatter: one
-// job per shard, same pointers, different byte offsets.  reduce_multi: one job per buffer,
-// each with its own n pointers.
+// One reduction of a launch, fully described by the host so that a wavefront needs one
+// scalar load to start and 32-bit uniform arithmetic only:
+//   elements [0, head)                      peeled, element-wise (out not yet 16-byte aligned)
+//   vectors  [0, nvec) at byte offset head*es   the vector body
+//   elements [head + nvec*VE, +tail)        peeled, element-wise
+struct ReduceJob {
+  char* out;
+  size_t in_off;   // byte offset applied to every input pointer
+  size_t nvec;     // 16-byte vectors in the body
+  uint32_t head;   // elements before the body (< 16)
+  uint32_t tail;   // elements after the body (< 16)
+};
+
+// Kernel arguments.  reduce_n: one job.  reduce_scatter: one job per shard, same pointers,
+// different byte offsets.  reduce_multi (OWN == true kernels): job j reads the n pointers
+// starting at ptr[job_ptr0[j]].
 struct ReduceArgs {
   const char* ptr[MCCL_MAX_RANKS];
-  char* job_out[kMaxJobs];
-  size_t job_in_off[kMaxJobs];
-  size_t job_count[kMaxJobs];
+  ReduceJob job[kMaxJobs];
   int job_ptr0[kMaxJobs];
   int n;
 };
@@ -221,11 +261,10 @@ union VecU {
 
 // Element-wise reduction of one element (used for peeled heads/tails and the misaligned path).
 template <int DT, int OP>
-__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, size_t in_off, char* out,
-                                           size_t idx) {
+__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, int n, size_t in_off,
+                                           char* out, size_t idx) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
-  const int n = a.n;
   A acc = chain_first<DT, OP>(Elem<DT>::load(((const S*)(a.ptr[p0] + in_off))[idx]));
   for (int k = 1; k < n; ++k)
     acc = chain_next<DT, OP>(acc, Elem<DT>::load(((const S*)(a.ptr[p0 + k] + in_off))[idx]));
@@ -239,11 +278,7 @@ __device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec)
   if constexpr (GUARD) {
     if (v >= nvec) return (u32x4){0u, 0u, 0u, 0u};
   }
-#ifdef MCCL_NT_LOAD
-  return __builtin_nontemporal_load(&p[v]);
-#else
-  return p[v];
-#endif
+  return __builtin_nontemporal_load(&p[v]);  // streamed once: keep it out of the caches
 }
 
 // One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
@@ -325,69 +360,80 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t 
 // Vector kernel.  Requires, for each job, all input pointers (+offset) and the output
 // pointer congruent mod 16.  The output may be exactly one of the inputs: a lane reads
 // element i of every input before it writes element i, and no other lane touches i.
-template <int DT, int OP, int NT, int U, int BLOCK>
+// OWN: each job has its own n pointers (coalesced reductions); otherwise all jobs share
+// ptr[0..n) and the pointer loads do not wait for the job record.
+template <int DT, int OP, int NT, int U, int BLOCK, bool OWN>
 __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
   using S = typename Elem<DT>::store_t;
   constexpr int VE = vec_elems<DT>();
-  const int job = blockIdx.y;
-  const int p0 = a.job_ptr0[job];
-  const size_t in_off = a.job_in_off[job];
-  char* out = a.job_out[job];
-  const size_t count = a.job_count[job];
+  const int jid = blockIdx.y;
+  const int p0 = OWN ? a.job_ptr0[jid] : 0;
   const int n = (NT > 0) ? NT : a.n;
-
-  // peel: head elements up to the first 16-byte boundary of out, tail after the last vector
-  size_t head = ((16u - (unsigned)((uintptr_t)out & 15u)) & 15u) / sizeof(S);
-  if (head > count) head = count;
-  const size_t nvec = (count - head) / VE;
-  const size_t tail = count - head - nvec * VE;
+  char* out = a.job[jid].out;
+  const size_t in_off = a.job[jid].in_off;
+  const size_t nvec = a.job[jid].nvec;
+  const uint32_t head = a.job[jid].head;
+  const uint32_t tail = a.job[jid].tail;
 
   if (blockIdx.x == 0) {
-    const size_t t = threadIdx.x;
-    if (t < head) reduce_one<DT, OP>(a, p0, in_off, out, t);
-    else if (t - head < tail) reduce_one<DT, OP>(a, p0, in_off, out, head + nvec * VE + (t - head));
+    const uint32_t t = threadIdx.x;
+    if (t < head) reduce_one<DT, OP>(a, p0, n, in_off, out, t);
+    else if (t - head < tail) reduce_one<DT, OP>(a, p0, n, in_off, out, head + nvec * VE + (t - head));
   }
 
-  const size_t body_off = head * sizeof(S);  // bytes
+  const size_t body_off = (size_t)head * sizeof(S);  // bytes
   u32x4* ov = (u32x4*)(out + body_off);
-  constexpr size_t TILE = (size_t)BLOCK * U;
-  const size_t full_tiles = nvec / TILE;
-  const size_t ntiles = (nvec + TILE - 1) / TILE;
+  constexpr uint32_t TILE = (uint32_t)BLOCK * U;
+  // the host keeps nvec / TILE below 2^32
+  const uint32_t full_tiles = (uint32_t)(nvec / TILE);
+  const uint32_t partial = (uint32_t)(nvec % TILE) ? 1u : 0u;
 
-  size_t tile = blockIdx.x;
+  uint32_t tile = blockIdx.x;
   for (; tile < full_tiles; tile += gridDim.x)
-    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, tile * TILE + threadIdx.x, nvec, n);
-  if (tile < ntiles)  // at most one partial tile exists and one workgroup reaches it
-    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, tile * TILE + threadIdx.x, nvec, n);
+    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
+  if (tile == full_tiles && partial)  // the one partial tile; exactly one workgroup reaches it
+    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
 }
 
 // Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
 // multiple of the element size).  Grid-stride over elements.
-template <int DT, int OP>
+template <int DT, int OP, bool OWN>
 __global__ __launch_bounds__(256) void reduce_elem_kernel(const ReduceArgs a) {
-  const int job = blockIdx.y;
-  const int p0 = a.job_ptr0[job];
-  const size_t in_off = a.job_in_off[job];
-  char* out = a.job_out[job];
-  const size_t count = a.job_count[job];
+  const int jid = blockIdx.y;
+  const int p0 = OWN ? a.job_ptr0[jid] : 0;
+  const size_t in_off = a.job[jid].in_off;
+  char* out = a.job[jid].out;
+  const size_t count = a.job[jid].nvec;  // element count for this kernel
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
-    reduce_one<DT, OP>(a, p0, in_off, out, i);
+    reduce_one<DT, OP>(a, p0, a.n, in_off, out, i);
 }
 
 // ------------------------------------------------------------------------------------------
 // segmented copy
 // ------------------------------------------------------------------------------------------
+// One segment as the kernel sees it.  The host splits it into a head (bytes up to the first
+// 16- or 4-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of
+// `last` bytes, so that the device needs 32-bit uniform arithmetic only.
+struct CopySeg {
+  const char* src;
+  char* dst;
+  uint32_t head;   // bytes before the body
+  uint32_t nfull;  // full chunks in the body
+  uint32_t last;   // bytes of the final partial chunk (0 = none)
+  uint32_t mode;   // 0: 16-byte vectors, 1: dwords, 2: bytes
+};
+
 struct CopyArgs {
-  mccl_segment_t seg[kMaxSegs];
+  CopySeg seg[kMaxSegs];
   uint32_t chunk_prefix[kMaxSegs + 1];  // exclusive prefix sum of chunks per segment
   int nseg;
 };
 
-// Chunk c of a segment covers body bytes [c*kCopyChunk, (c+1)*kCopyChunk) where the body
-// starts after a head that brings dst to a 16-byte (or 4-byte) boundary.  When src and dst
-// are congruent mod 16 the body moves as 16-byte vectors, mod 4 as dwords, else as bytes.
-__global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const CopyArgs a) {
+// Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
+// handed out in order.  When src and dst are congruent mod 16 the body moves as 16-byte
+// vectors (non-temporal both ways for full chunks), mod 4 as dwords, else as bytes.
+__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
     // binary search: largest s with chunk_prefix[s] <= chunk
@@ -397,56 +443,42 @@ __global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const CopyArg
       if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
     }
     const uint32_t c = chunk - a.chunk_prefix[lo];
-    const char* src = (const char*)a.seg[lo].src;
-    char* dst = (char*)a.seg[lo].dst;
-    const size_t bytes = a.seg[lo].bytes;
-    const unsigned diff = (unsigned)(((uintptr_t)src ^ (uintptr_t)dst) & 15u);
-    const unsigned t = threadIdx.x;
+    const uint32_t head = a.seg[lo].head;
+    const uint32_t nfull = a.seg[lo].nfull;
+    const uint32_t mode = a.seg[lo].mode;
+    const uint32_t len = (c < nfull) ? (uint32_t)kCopyChunk : a.seg[lo].last;
+    const uint32_t t = threadIdx.x;
+    const char* src = a.seg[lo].src;
+    char* dst = a.seg[lo].dst;
+    if (c == 0 && t < head) dst[t] = src[t];
+    const size_t off = (size_t)head + (size_t)c * kCopyChunk;  // start of this chunk
+    src += off;
+    dst += off;
 
-    if (diff == 0) {
-      size_t head = (16u - (unsigned)((uintptr_t)dst & 15u)) & 15u;
-      if (head > bytes) head = bytes;
-      if (c == 0 && t < head) dst[t] = src[t];
-      const size_t body = bytes - head;
-      const size_t b0 = (size_t)c * kCopyChunk;
-      if (b0 < body) {
-        const size_t len = (body - b0 < kCopyChunk) ? body - b0 : kCopyChunk;
-        const u32x4* sv = (const u32x4*)(src + head + b0);
-        u32x4* dv = (u32x4*)(dst + head + b0);
-        const size_t nv = len >> 4;
-        if (nv == (size_t)kCopyBlock * kCopyUnroll) {
-          u32x4 x[kCopyUnroll];
+    if (mode == 0) {
+      const u32x4* sv = (const u32x4*)src;
+      u32x4* dv = (u32x4*)dst;
+      if (len == (uint32_t)kCopyChunk) {
+        u32x4 x[kCopyUnroll];
 #pragma unroll
-          for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kCopyBlock]);
+        for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
 #pragma unroll
-          for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kCopyBlock]);
-        } else {
-          for (size_t v = t; v < nv; v += kCopyBlock) dv[v] = sv[v];
-          const size_t rem = len & 15u;
-          if (t < rem) dst[head + b0 + (nv << 4) + t] = src[head + b0 + (nv << 4) + t];
-        }
+        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      } else {
+        const uint32_t nv = len >> 4;
+        for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
+        const uint32_t rem = len & 15u;
+        if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
       }
-    } else if ((diff & 3u) == 0) {
-      size_t head = (4u - (unsigned)((uintptr_t)dst & 3u)) & 3u;
-      if (head > bytes) head = bytes;
-      if (c == 0 && t < head) dst[t] = src[t];
-      const size_t body = bytes - head;
-      const size_t b0 = (size_t)c * kCopyChunk;
-      if (b0 < body) {
-        const size_t len = (body - b0 < kCopyChunk) ? body - b0 : kCopyChunk;
-        const uint32_t* sw = (const uint32_t*)(src + head + b0);
-        uint32_t* dw = (uint32_t*)(dst + head + b0);
-        const size_t nw = len >> 2;
-        for (size_t v = t; v < nw; v += kCopyBlock) dw[v] = sw[v];
-        const size_t rem = len & 3u;
-        if (t < rem) dst[head + b0 + (nw << 2) + t] = src[head + b0 + (nw << 2) + t];
-      }
+    } else if (mode == 1) {
+      const uint32_t* sw = (const uint32_t*)src;
+      uint32_t* dw = (uint32_t*)dst;
+      const uint32_t nw = len >> 2;
+      for (uint32_t v = t; v < nw; v += kWave) dw[v] = sw[v];
+      const uint32_t rem = len & 3u;
+      if (t < rem) dst[(nw << 2) + t] = src[(nw << 2) + t];
     } else {
-      const size_t b0 = (size_t)c * kCopyChunk;
-      if (b0 < bytes) {
-        const size_t len = (bytes - b0 < kCopyChunk) ? bytes - b0 : kCopyChunk;
-        for (size_t v = t; v < len; v += kCopyBlock) dst[b0 + v] = src[b0 + v];
-      }
+      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
     }
   }
 }
@@ -468,132 +500,186 @@ size_t dtype_size(int dt) {
   }
 }
 
-enum Shape { kShapeSmall, kShapePersistent, kShapeElem };
+enum Shape { kShapeSmall, kShapeStream, kShapePersistent, kShapeElem };
 
-template <int DT, int OP, int NT>
-hipError_t launch_vec(const ReduceArgs& a, Shape shape, dim3 grid, hipStream_t s) {
-  if (shape == kShapeSmall)
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kBlockSmall>), grid, dim3(kBlockSmall), 0, s, a);
-  else
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent>), grid,
+// Geometry of a launch.
+struct Geometry {
+  Shape shape;
+  unsigned grid_x;
+  int block;
+  unsigned lds;   // dynamic LDS reservation (occupancy cap), bytes
+  bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
+};
+
+template <int DT, int OP, int NT, bool OWN>
+hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+  const dim3 grid(g.grid_x, njobs, 1);
+  if (g.shape == kShapePersistent)
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent, OWN>), grid,
                        dim3(kBlockPersistent), 0, s, a);
+  else
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kWave, OWN>), grid, dim3(kWave), g.lds, s, a);
   return hipGetLastError();
 }
 
 template <int DT, int OP>
-hipError_t launch_op(const ReduceArgs& a, Shape shape, dim3 grid, hipStream_t s) {
-  if (shape == kShapeElem) {
-    hipLaunchKernelGGL((reduce_elem_kernel<DT, OP>), grid, dim3(256), 0, s, a);
+hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+  if (g.shape == kShapeElem) {
+    if (g.own_ptrs) hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, true>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, false>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
     return hipGetLastError();
   }
+  if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
   if constexpr (OP == MCCL_SUM) {
     switch (a.n) {
-      case 2: return launch_vec<DT, OP, 2>(a, shape, grid, s);
-      case 4: return launch_vec<DT, OP, 4>(a, shape, grid, s);
-      case 8: return launch_vec<DT, OP, 8>(a, shape, grid, s);
+      case 2: return launch_vec<DT, OP, 2, false>(a, g, njobs, s);
+      case 4: return launch_vec<DT, OP, 4, false>(a, g, njobs, s);
+      case 8: return launch_vec<DT, OP, 8, false>(a, g, njobs, s);
       default: break;
     }
   }
-  return launch_vec<DT, OP, 0>(a, shape, grid, s);
+  return launch_vec<DT, OP, 0, false>(a, g, njobs, s);
 }
 
 template <int DT>
-hipError_t launch_dtype(const ReduceArgs& a, int op, Shape shape, dim3 grid, hipStream_t s) {
+hipError_t launch_dtype(const ReduceArgs& a, int op, const Geometry& g, int njobs, hipStream_t s) {
   switch (op) {
-    case MCCL_SUM: return launch_op<DT, MCCL_SUM>(a, shape, grid, s);
-    case MCCL_PROD: return launch_op<DT, MCCL_PROD>(a, shape, grid, s);
-    case MCCL_MIN: return launch_op<DT, MCCL_MIN>(a, shape, grid, s);
-    case MCCL_MAX: return launch_op<DT, MCCL_MAX>(a, shape, grid, s);
+    case MCCL_SUM: return launch_op<DT, MCCL_SUM>(a, g, njobs, s);
+    case MCCL_PROD: return launch_op<DT, MCCL_PROD>(a, g, njobs, s);
+    case MCCL_MIN: return launch_op<DT, MCCL_MIN>(a, g, njobs, s);
+    case MCCL_MAX: return launch_op<DT, MCCL_MAX>(a, g, njobs, s);
     case MCCL_AVG:
-      if constexpr (Elem<DT>::kIsFloat) return launch_op<DT, MCCL_AVG>(a, shape, grid, s);
+      if constexpr (Elem<DT>::kIsFloat) return launch_op<DT, MCCL_AVG>(a, g, njobs, s);
       else return hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
   }
 }
 
-hipError_t launch_any(const ReduceArgs& a, int dtype, int op, Shape shape, dim3 grid, hipStream_t s) {
+hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g, int njobs, hipStream_t s) {
   switch (dtype) {
-    case MCCL_U8: return launch_dtype<MCCL_U8>(a, op, shape, grid, s);
-    case MCCL_I8: return launch_dtype<MCCL_I8>(a, op, shape, grid, s);
-    case MCCL_I16: return launch_dtype<MCCL_I16>(a, op, shape, grid, s);
-    case MCCL_I32: return launch_dtype<MCCL_I32>(a, op, shape, grid, s);
-    case MCCL_I64: return launch_dtype<MCCL_I64>(a, op, shape, grid, s);
-    case MCCL_F16: return launch_dtype<MCCL_F16>(a, op, shape, grid, s);
-    case MCCL_F32: return launch_dtype<MCCL_F32>(a, op, shape, grid, s);
-    case MCCL_F64: return launch_dtype<MCCL_F64>(a, op, shape, grid, s);
-    case MCCL_BF16: return launch_dtype<MCCL_BF16>(a, op, shape, grid, s);
+    case MCCL_U8: return launch_dtype<MCCL_U8>(a, op, g, njobs, s);
+    case MCCL_I8: return launch_dtype<MCCL_I8>(a, op, g, njobs, s);
+    case MCCL_I16: return launch_dtype<MCCL_I16>(a, op, g, njobs, s);
+    case MCCL_I32: return launch_dtype<MCCL_I32>(a, op, g, njobs, s);
+    case MCCL_I64: return launch_dtype<MCCL_I64>(a, op, g, njobs, s);
+    case MCCL_F16: return launch_dtype<MCCL_F16>(a, op, g, njobs, s);
+    case MCCL_F32: return launch_dtype<MCCL_F32>(a, op, g, njobs, s);
+    case MCCL_F64: return launch_dtype<MCCL_F64>(a, op, g, njobs, s);
+    case MCCL_BF16: return launch_dtype<MCCL_BF16>(a, op, g, njobs, s);
     default: return hipErrorInvalidValue;
   }
 }
 
-// Geometry of a vector launch over jobs whose largest has max_count elements.
-struct Geometry {
-  Shape shape;
-  unsigned grid_x;
-  int block;
-};
+// Loads one wavefront keeps in flight per tile: all ranks when the rank count is a
+// compile-time specialisation (SUM with 2, 4 or 8 ranks), else one group of four.
+int loads_in_flight(int n, int op, bool own_ptrs) {
+  if (!own_ptrs && op == MCCL_SUM && (n == 2 || n == 4 || n == 8)) return n;
+  return n < 4 ? n : 4;
+}
 
-int plan_vec(size_t max_count, int njobs, int dtype, int variant, Geometry* g) {
+// Geometry of a vector launch over njobs jobs whose largest has max_count elements.
+int plan_vec(size_t max_count, int njobs, int n, int dtype, int op, int variant, bool own_ptrs,
+             Geometry* g) {
   int cus = 0;
   int rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
   const size_t es = dtype_size(dtype);
   const size_t nvec = max_count / (16 / es) + 1;
-  bool small;
-  if (variant == MCCL_VARIANT_SMALL) small = true;
-  else if (variant == MCCL_VARIANT_PERSISTENT) small = false;
-  else small = max_count * es <= g_small_max_bytes;
-  if (small) {
-    size_t tiles = (nvec + kBlockSmall - 1) / kBlockSmall;
-    if (tiles > 0x7fffffffu) return fail(MCCL_ERR_INVALID_ARG, "message too large for the small variant");
-    g->shape = kShapeSmall;
-    g->grid_x = (unsigned)(tiles ? tiles : 1);
-    g->block = kBlockSmall;
-  } else {
+  Shape shape;
+  switch (variant) {
+    case MCCL_VARIANT_SMALL: shape = kShapeSmall; break;
+    case MCCL_VARIANT_PERSISTENT: shape = kShapePersistent; break;
+    case MCCL_VARIANT_STREAM: shape = kShapeStream; break;
+    case MCCL_VARIANT_AUTO:
+      shape = (max_count * es <= (size_t)g_tune[MCCL_TUNE_SMALL_MAX_BYTES]) ? kShapeSmall : kShapeStream;
+      break;
+    default: return fail(MCCL_ERR_INVALID_ARG, "unknown variant %d", variant);
+  }
+  g->shape = shape;
+  g->lds = 0;
+  g->own_ptrs = own_ptrs;
+  if (shape == kShapePersistent) {
     const size_t tile = (size_t)kBlockPersistent * kUnrollPersistent;
     size_t tiles = (nvec + tile - 1) / tile;
-    size_t want = (size_t)cus * g_blocks_per_cu / (size_t)njobs;
+    size_t want = (size_t)cus * (size_t)g_tune[MCCL_TUNE_PERSISTENT_BLOCKS_PER_CU] / (size_t)njobs;
     if (want < 1) want = 1;
     if (tiles > want) tiles = want;
-    g->shape = kShapePersistent;
     g->grid_x = (unsigned)(tiles ? tiles : 1);
     g->block = kBlockPersistent;
+  } else {
+    size_t tiles = (nvec + kWave - 1) / kWave;
+    if (tiles > kMaxGridX) tiles = kMaxGridX;
+    g->grid_x = (unsigned)(tiles ? tiles : 1);
+    g->block = kWave;
+    if (shape == kShapeStream) {
+      const long long per_wave = (long long)loads_in_flight(n, op, own_ptrs) * kWave * 16;
+      long long waves = g_tune[MCCL_TUNE_STREAM_INFLIGHT_BYTES] / per_wave;
+      if (waves < 2) waves = 2;
+      g->lds = lds_for_waves(waves);
+    }
   }
   return MCCL_OK;
 }
 
-// Launch one batch of jobs (args fully populated).  Jobs whose pointers are congruent mod 16
-// go to the vector kernel; the rest to the element kernel, in at most two launches.
-int launch_jobs(ReduceArgs& a, int njobs, int dtype, int op, int variant, hipStream_t s) {
+// A reduction as the entry points describe it, before the host splits it for the kernels.
+struct JobSpec {
+  char* out;
+  size_t in_off;
+  size_t count;
+  int ptr0;
+};
+
+// Launch one batch of jobs.  a.ptr / a.n are populated; specs describe the jobs.  Jobs whose
+// pointers are congruent mod 16 go to the vector kernel; the rest to the element kernel, in
+// at most two launches.
+int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int op, int variant,
+                bool own_ptrs, hipStream_t s) {
   const size_t es = dtype_size(dtype);
-  ReduceArgs vec = a, elem = a;
+  const size_t ve = 16 / es;
+  ReduceArgs elem = a;  // the vector launch reuses `a`
   int nv = 0, ne = 0;
   size_t vmax = 0, emax = 0;
   for (int j = 0; j < njobs; ++j) {
-    if (a.job_count[j] == 0) continue;
-    const uintptr_t o = (uintptr_t)a.job_out[j];
+    const JobSpec& sp = specs[j];
+    if (sp.count == 0) continue;
+    const uintptr_t o = (uintptr_t)sp.out;
     if (o % es) return fail(MCCL_ERR_INVALID_ARG, "output pointer not aligned to the element size");
     bool congruent = true;
     for (int k = 0; k < a.n; ++k) {
-      const uintptr_t p = (uintptr_t)(a.ptr[a.job_ptr0[j] + k] + a.job_in_off[j]);
+      const uintptr_t p = (uintptr_t)(a.ptr[sp.ptr0 + k] + sp.in_off);
       if (p % es) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d not aligned to the element size", k);
       if ((p & 15u) != (o & 15u)) congruent = false;
     }
-    ReduceArgs& t = congruent ? vec : elem;
-    int& idx = congruent ? nv : ne;
-    t.job_out[idx] = a.job_out[j];
-    t.job_in_off[idx] = a.job_in_off[j];
-    t.job_count[idx] = a.job_count[j];
-    t.job_ptr0[idx] = a.job_ptr0[j];
-    ++idx;
-    size_t& mx = congruent ? vmax : emax;
-    if (a.job_count[j] > mx) mx = a.job_count[j];
+    if (congruent) {
+      size_t head = ((16u - (unsigned)(o & 15u)) & 15u) / es;
+      if (head > sp.count) head = sp.count;
+      const size_t nvec = (sp.count - head) / ve;
+      if (nvec / kWave > 0xfffffff0ull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+      ReduceJob& jb = a.job[nv];
+      jb.out = sp.out;
+      jb.in_off = sp.in_off;
+      jb.nvec = nvec;
+      jb.head = (uint32_t)head;
+      jb.tail = (uint32_t)(sp.count - head - nvec * ve);
+      a.job_ptr0[nv] = sp.ptr0;
+      ++nv;
+      if (sp.count > vmax) vmax = sp.count;
+    } else {
+      ReduceJob& jb = elem.job[ne];
+      jb.out = sp.out;
+      jb.in_off = sp.in_off;
+      jb.nvec = sp.count;  // the element kernel reads this field as the element count
+      jb.head = jb.tail = 0;
+      elem.job_ptr0[ne] = sp.ptr0;
+      ++ne;
+      if (sp.count > emax) emax = sp.count;
+    }
   }
   if (nv) {
     Geometry g;
-    int rc = plan_vec(vmax, nv, dtype, variant, &g);
+    int rc = plan_vec(vmax, nv, a.n, dtype, op, variant, own_ptrs, &g);
     if (rc != MCCL_OK) return rc;
-    hipError_t e = launch_any(vec, dtype, op, g.shape, dim3(g.grid_x, nv, 1), s);
+    hipError_t e = launch_any(a, dtype, op, g, nv, s);
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   }
   if (ne) {
@@ -604,14 +690,21 @@ int launch_jobs(ReduceArgs& a, int njobs, int dtype, int op, int variant, hipStr
     size_t cap = (size_t)cus * 8 / ne;
     if (cap < 1) cap = 1;
     if (blocks > cap) blocks = cap;
-    hipError_t e = launch_any(elem, dtype, op, kShapeElem, dim3((unsigned)blocks, ne, 1), s);
+    Geometry g{kShapeElem, (unsigned)blocks, 256, 0, own_ptrs};
+    hipError_t e = launch_any(elem, dtype, op, g, ne, s);
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   }
   return MCCL_OK;
 }
 
+int check_reduce_args_no_ptr(int n, int dtype, int op);
+
 int check_reduce_args(const void* const* in, int n, int dtype, int op) {
   if (!in) return fail(MCCL_ERR_INVALID_ARG, "input pointer table is null");
+  return check_reduce_args_no_ptr(n, dtype, op);
+}
+
+int check_reduce_args_no_ptr(int n, int dtype, int op) {
   if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
   if (!valid_dtype(dtype)) return fail(MCCL_ERR_INVALID_ARG, "unknown dtype code %d", dtype);
   if (!valid_op(op)) return fail(MCCL_ERR_INVALID_ARG, "unknown reduce op code %d", op);
@@ -633,12 +726,28 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
       const mccl_segment_t& sg = segs[i];
       if (sg.bytes == 0) { ++i; continue; }
       if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
-      const uint64_t c = (sg.bytes + kCopyChunk - 1) / kCopyChunk;
-      if (chunks + c > 0xffffffffull) {
+      const uintptr_t sp = (uintptr_t)sg.src, dp = (uintptr_t)sg.dst;
+      const unsigned diff = (unsigned)((sp ^ dp) & 15u);
+      CopySeg cs;
+      cs.src = (const char*)sg.src;
+      cs.dst = (char*)sg.dst;
+      size_t head;
+      if (diff == 0) { cs.mode = 0; head = (16u - (unsigned)(dp & 15u)) & 15u; }
+      else if ((diff & 3u) == 0) { cs.mode = 1; head = (4u - (unsigned)(dp & 3u)) & 3u; }
+      else { cs.mode = 2; head = 0; }
+      if (head > sg.bytes) head = sg.bytes;
+      const size_t body = sg.bytes - head;
+      const uint64_t nfull = body / kCopyChunk;
+      cs.head = (uint32_t)head;
+      cs.last = (uint32_t)(body % kCopyChunk);
+      uint64_t c = nfull + (cs.last ? 1 : 0);
+      if (c == 0) c = 1;  // head only: chunk 0 still has to run
+      if (nfull > 0xfffffff0ull || chunks + c > 0xffffffffull) {
         if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "segment %d too large", i);
         break;
       }
-      a.seg[m] = sg;
+      cs.nfull = (uint32_t)nfull;
+      a.seg[m] = cs;
       chunks += c;
       a.chunk_prefix[++m] = (uint32_t)chunks;
       ++i;
@@ -646,9 +755,10 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
     if (m == 0) break;
     a.nseg = m;
     uint64_t grid = chunks;
-    const uint64_t cap = (uint64_t)cus * 16;
-    if (grid > cap) grid = cap;
-    hipLaunchKernelGGL(copy_segments_kernel, dim3((unsigned)grid), dim3(kCopyBlock), 0, s, a);
+    if (grid > kMaxGridX) grid = kMaxGridX;
+    // small copies are latency bound: no residency cap below 4 chunks per CU
+    const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_COPY_WAVES_PER_CU]) : 0;
+    hipLaunchKernelGGL(copy_segments_kernel, dim3((unsigned)grid), dim3(kWave), lds, s, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   }
@@ -668,19 +778,26 @@ const char* mccl_last_error(void) { return g_err; }
 
 size_t mccl_dtype_size(int dtype) { return dtype_size(dtype); }
 
-void mccl_set_tuning(int persistent_blocks_per_cu, int block_size, int small_max_bytes) {
-  (void)block_size;
-  if (persistent_blocks_per_cu > 0) g_blocks_per_cu = persistent_blocks_per_cu;
-  if (small_max_bytes > 0) g_small_max_bytes = (size_t)small_max_bytes;
+int mccl_set_tuning(int knob, long long value) {
+  if (knob < 0 || knob >= MCCL_TUNE_COUNT_) return fail(MCCL_ERR_INVALID_ARG, "unknown tuning knob %d", knob);
+  g_tune[knob] = value > 0 ? value : g_tune_default[knob];
+  return MCCL_OK;
 }
 
-int mccl_query_launch(size_t count, int n, int dtype, int variant, int* block_size) {
-  (void)n;
-  if (!valid_dtype(dtype)) return fail(MCCL_ERR_INVALID_ARG, "unknown dtype code %d", dtype);
+long long mccl_get_tuning(int knob) {
+  if (knob < 0 || knob >= MCCL_TUNE_COUNT_) return -1;
+  return g_tune[knob];
+}
+
+int mccl_query_launch(size_t count, int n, int dtype, int op, int variant, int* block_size,
+                      int* lds_bytes) {
+  int rc = check_reduce_args_no_ptr(n, dtype, op);
+  if (rc != MCCL_OK) return rc;
   Geometry g;
-  int rc = plan_vec(count, 1, dtype, variant, &g);
+  rc = plan_vec(count, 1, n, dtype, op, variant, false, &g);
   if (rc != MCCL_OK) return rc;
   if (block_size) *block_size = g.block;
+  if (lds_bytes) *lds_bytes = (int)g.lds;
   return (int)g.grid_x;
 }
 
@@ -697,9 +814,8 @@ int mccl_reduce_n(const void* const* in, int n, void* out, size_t count, int dty
     a.ptr[k] = (const char*)in[k];
   }
   a.n = n;
-  a.job_out[0] = (char*)out;
-  a.job_count[0] = count;
-  return launch_jobs(a, 1, dtype, op, variant, (hipStream_t)stream);
+  const JobSpec spec{(char*)out, 0, count, 0};
+  return launch_jobs(a, &spec, 1, dtype, op, variant, false, (hipStream_t)stream);
 }
 
 int mccl_reduce_scatter_n(const void* const* in, int n, void* const* out, size_t shard_count,
@@ -719,14 +835,12 @@ int mccl_reduce_scatter_n(const void* const* in, int n, void* const* out, size_t
   a.n = n;
   for (int s0 = 0; s0 < shard_num; s0 += kMaxJobs) {
     const int m = (shard_num - s0 < kMaxJobs) ? shard_num - s0 : kMaxJobs;
+    JobSpec specs[kMaxJobs];
     for (int j = 0; j < m; ++j) {
       if (!out[s0 + j]) return fail(MCCL_ERR_INVALID_ARG, "output pointer %d is null", s0 + j);
-      a.job_out[j] = (char*)out[s0 + j];
-      a.job_in_off[j] = (size_t)(shard_first + s0 + j) * shard_count * es;
-      a.job_count[j] = shard_count;
-      a.job_ptr0[j] = 0;
+      specs[j] = JobSpec{(char*)out[s0 + j], (size_t)(shard_first + s0 + j) * shard_count * es, shard_count, 0};
     }
-    rc = launch_jobs(a, m, dtype, op, MCCL_VARIANT_AUTO, (hipStream_t)stream);
+    rc = launch_jobs(a, specs, m, dtype, op, MCCL_VARIANT_AUTO, false, (hipStream_t)stream);
     if (rc != MCCL_OK) return rc;
   }
   return MCCL_OK;
@@ -746,6 +860,7 @@ int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size
     ReduceArgs a;
     memset(&a, 0, sizeof(a));
     a.n = n;
+    JobSpec specs[kMaxJobs];
     for (int j = 0; j < m; ++j) {
       for (int k = 0; k < n; ++k) {
         const void* p = in[(size_t)(b0 + j) * n + k];
@@ -753,11 +868,9 @@ int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size
         a.ptr[j * n + k] = (const char*)p;
       }
       if (!out[b0 + j] && counts[b0 + j]) return fail(MCCL_ERR_INVALID_ARG, "output pointer %d is null", b0 + j);
-      a.job_out[j] = (char*)out[b0 + j];
-      a.job_count[j] = counts[b0 + j];
-      a.job_ptr0[j] = j * n;
+      specs[j] = JobSpec{(char*)out[b0 + j], 0, counts[b0 + j], j * n};
     }
-    rc = launch_jobs(a, m, dtype, op, MCCL_VARIANT_AUTO, (hipStream_t)stream);
+    rc = launch_jobs(a, specs, m, dtype, op, MCCL_VARIANT_AUTO, true, (hipStream_t)stream);
     if (rc != MCCL_OK) return rc;
   }
   return MCCL_OK;

@@ -6,7 +6,7 @@ fails.
 """
 from . import capi
 from .capi import (AVG, MAX, MIN, PROD, SUM, VARIANT_AUTO, VARIANT_PERSISTENT,  # noqa: F401
-                   VARIANT_SMALL)
+                   VARIANT_SMALL, VARIANT_STREAM)
 from .ops import (allgather_n, alltoallv_n, copy_segments, pack, reduce_multi,  # noqa: F401
                   reduce_n, reduce_scatter_n, unpack)
 

@@ -1,0 +1,105 @@
+"""ctypes binding of libmcclbench.so: HIP-event timing loops around the C ABI
+(include/mccl_bench.h).  Benchmark support; not needed to use the library."""
+import ctypes
+import os
+
+import torch
+
+from . import capi
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmcclbench.so")
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        capi.lib()
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libmcclbench.so is not built; run `python torch-ccl_amd/csrc/build.py`")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+        L.mcclb_last_error.restype = ctypes.c_char_p
+        L.mcclb_reduce_latency.argtypes = [vp, i32, vp, i32, sz, i32, i32, i32, vp, i32, i32, vp]
+        L.mcclb_reduce_throughput.argtypes = [vp, i32, vp, i32, sz, i32, i32, i32, vp, i32, i32, vp]
+        L.mcclb_reduce_scatter_throughput.argtypes = [vp, i32, vp, sz, i32, i32, i32, i32, vp, i32, i32, vp]
+        L.mcclb_copy_latency.argtypes = [vp, i32, vp, i32, i32, vp]
+        L.mcclb_copy_throughput.argtypes = [vp, i32, vp, i32, i32, vp]
+        L.mcclb_alltoallv_throughput.argtypes = [vp, vp, i32, vp, sz, vp, i32, i32, vp]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError("mccl bench error %d: %s" % (rc, lib().mcclb_last_error().decode()))
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _sets(input_sets, outputs):
+    n = len(input_sets[0])
+    flat = [t.data_ptr() for s in input_sets for t in s]
+    return n, capi.ptr_table(flat), capi.ptr_table([o.data_ptr() for o in outputs])
+
+
+def reduce_latency(input_sets, outputs, op=capi.SUM, variant=capi.VARIANT_AUTO, warmup=100, iters=1000):
+    """Per-call microseconds (list of floats); call i uses buffer set i % len(input_sets)."""
+    n, ins, outs = _sets(input_sets, outputs)
+    us = (ctypes.c_float * iters)()
+    o = outputs[0]
+    _check(lib().mcclb_reduce_latency(ins, n, outs, len(input_sets), o.numel(),
+                                      capi.TORCH_DTYPE[o.dtype], op, variant, _stream(), warmup, iters, us))
+    return list(us)
+
+
+def reduce_throughput(input_sets, outputs, op=capi.SUM, variant=capi.VARIANT_AUTO, warmup=5, iters=20):
+    """Average microseconds per call over `iters` back-to-back calls."""
+    n, ins, outs = _sets(input_sets, outputs)
+    total = ctypes.c_float(0)
+    o = outputs[0]
+    _check(lib().mcclb_reduce_throughput(ins, n, outs, len(input_sets), o.numel(),
+                                         capi.TORCH_DTYPE[o.dtype], op, variant, _stream(), warmup, iters,
+                                         ctypes.byref(total)))
+    return total.value / iters
+
+
+def reduce_scatter_throughput(inputs, outputs, shard_first=0, op=capi.SUM, warmup=3, iters=10):
+    total = ctypes.c_float(0)
+    o = outputs[0]
+    _check(lib().mcclb_reduce_scatter_throughput(
+        capi.ptr_table([t.data_ptr() for t in inputs]), len(inputs),
+        capi.ptr_table([t.data_ptr() for t in outputs]), o.numel(), shard_first, len(outputs),
+        capi.TORCH_DTYPE[o.dtype], op, _stream(), warmup, iters, ctypes.byref(total)))
+    return total.value / iters
+
+
+def _segs(segments):
+    segs = list(segments)
+    return (capi.Segment * len(segs))(*[capi.Segment(s, d, b) for (s, d, b) in segs]), len(segs)
+
+
+def copy_latency(segments, warmup=100, iters=1000):
+    arr, n = _segs(segments)
+    us = (ctypes.c_float * iters)()
+    _check(lib().mcclb_copy_latency(arr, n, _stream(), warmup, iters, us))
+    return list(us)
+
+
+def copy_throughput(segments, warmup=3, iters=10):
+    arr, n = _segs(segments)
+    total = ctypes.c_float(0)
+    _check(lib().mcclb_copy_throughput(arr, n, _stream(), warmup, iters, ctypes.byref(total)))
+    return total.value / iters
+
+
+def alltoallv_throughput(inputs, outputs, split_rows, row_bytes, warmup=2, iters=5):
+    n = len(inputs)
+    S = torch.as_tensor(split_rows, dtype=torch.int64).reshape(n, n).contiguous()
+    total = ctypes.c_float(0)
+    _check(lib().mcclb_alltoallv_throughput(
+        capi.ptr_table([t.data_ptr() for t in inputs]), capi.ptr_table([t.data_ptr() for t in outputs]), n,
+        ctypes.c_void_p(S.data_ptr()), row_bytes, _stream(), warmup, iters, ctypes.byref(total)))
+    return total.value / iters

@@ -17,7 +17,9 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355ccl.so")
 U8, I8, I16, I32, I64, F16, F32, F64, BF16 = range(9)
 # op codes (mccl_op_t), numbered like c10d::ReduceOp
 SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
-VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT = 0, 1, 2
+VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
+(TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_INFLIGHT_BYTES, TUNE_SMALL_MAX_BYTES,
+ TUNE_COPY_WAVES_PER_CU) = range(4)
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
@@ -30,7 +32,7 @@ EXPORTS = (
     "mccl_version", "mccl_last_error", "mccl_dtype_size", "mccl_reduce_n",
     "mccl_reduce_scatter_n", "mccl_reduce_multi", "mccl_copy_segments", "mccl_allgather_n",
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
-    "mccl_query_launch", "mccl_set_tuning",
+    "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
 )
 
 
@@ -64,9 +66,10 @@ def lib():
     L.mccl_alltoallv_pull.argtypes = [vp, i32, vp, vp, vp, vp]
     L.mccl_pack.argtypes = [vp, vp, i32, vp, vp]
     L.mccl_unpack.argtypes = [vp, vp, vp, i32, vp]
-    L.mccl_query_launch.argtypes = [sz, i32, i32, i32, vp]
-    L.mccl_set_tuning.argtypes = [i32, i32, i32]
-    L.mccl_set_tuning.restype = None
+    L.mccl_query_launch.argtypes = [sz, i32, i32, i32, i32, vp, vp]
+    L.mccl_set_tuning.argtypes = [i32, ctypes.c_longlong]
+    L.mccl_get_tuning.argtypes = [i32]
+    L.mccl_get_tuning.restype = ctypes.c_longlong
     _lib = L
     return L
 
