@@ -24,6 +24,10 @@ sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published peak
 SEED = 1234
+# HBM bytes of one launch of the headline kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of
+# this script, each counter scaled by its reading for a 512 MiB copy of known size
+# (profiles/reduce_bf16_8rank_64MiB_stream.md).  Algorithmic bytes are 603,979,776.
+C3_TRAFFIC_BYTES_ROCPROF = 603_994_814
 
 
 def log(*a):
@@ -86,7 +90,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,variants,gloo or all/none")
+                    help="comma list of c1,c2,c4,c5,variants,copycal or all/none "
+                         "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
+                         "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
 
@@ -95,7 +101,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,variants,gloo".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,variants".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import torch
@@ -151,10 +157,11 @@ def main():
                        grid, blk.value, lds.value)},
         "pct_of_peak": round(value / PEAK_HBM_GBS * 100, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": C3_TRAFFIC_BYTES_ROCPROF,
                      "kernel_us": round(ev_us, 2),
                      "note": "achieved = (N+1)*S algorithmic bytes / average launch duration from one HIP "
-                             "event pair around the K timed launches on the launch stream"},
+                             "event pair around the K timed launches on the launch stream; traffic = "
+                             "calibrated rocprofv3 FETCH_SIZE+WRITE_SIZE bytes per launch (offline run)"},
     }
 
     # parity spot check of the timed output against an on-device fp32 chain
@@ -258,6 +265,18 @@ def main():
                                       "split_rows_rank0": S5[0].tolist()}
         log("C5:", json.dumps(result["c5_alltoallv_moe"]))
         del a2a_in, a2a_out
+
+    # ---------------- counter calibration: a copy of known size ----------------
+    if "copycal" in extras:
+        cal = 512 << 20
+        src = torch.randint(0, 255, (cal,), dtype=torch.uint8, device=dev)
+        dst = torch.empty(cal, dtype=torch.uint8, device=dev)
+        us = benchlib.copy_throughput([(src.data_ptr(), dst.data_ptr(), cal)], warmup=2, iters=10)
+        result["copy_calibration_512MiB"] = {"us": round(us, 1), "GBps": round(2 * cal / us / 1e3, 1),
+                                             "bytes_read": cal, "bytes_written": cal,
+                                             "bit_exact": bool(torch.equal(src, dst))}
+        log("copycal:", json.dumps(result["copy_calibration_512MiB"]))
+        del src, dst
 
     # ---------------- CPU baseline (the oracle port) ----------------
     if not args.no_cpu:

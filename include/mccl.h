@@ -59,7 +59,10 @@ typedef enum {
 /* Launch shape of the reduction (the reference switches at SMALL_MAX_COUNT between a
  * single-launch kernel and a persistent one, src/gpu/dpcpp_ccl.cpp:771-775). */
 typedef enum {
-  MCCL_VARIANT_AUTO = 0,       /* pick by message size: SMALL up to the threshold, else STREAM */
+  MCCL_VARIANT_AUTO = 0,       /* pick by size: SMALL up to MCCL_TUNE_SMALL_MAX_BYTES per rank,
+                                  STREAM once (n+1)*bytes reaches MCCL_TUNE_STREAM_MIN_TOTAL_BYTES
+                                  (the working set no longer fits the 256 MB Infinity Cache),
+                                  PERSISTENT in between */
   MCCL_VARIANT_SMALL = 1,      /* one wavefront per workgroup, one vector per lane, grid covers
                                   the message, no residency cap: lowest latency */
   MCCL_VARIANT_PERSISTENT = 2, /* fixed grid sized to the CUs, grid-stride loop */
@@ -74,7 +77,8 @@ typedef enum {
   MCCL_TUNE_STREAM_INFLIGHT_BYTES = 1,    /* load bytes in flight per CU, STREAM shape */
   MCCL_TUNE_SMALL_MAX_BYTES = 2,          /* per-rank bytes up to which AUTO picks SMALL */
   MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
-  MCCL_TUNE_COUNT_ = 4
+  MCCL_TUNE_STREAM_MIN_TOTAL_BYTES = 4,   /* (n+1)*bytes from which AUTO picks STREAM */
+  MCCL_TUNE_COUNT_ = 5
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64

@@ -1,0 +1,97 @@
+"""No-GPU checks of the native boundary: the shared libraries load, export every symbol the
+headers declare, and the entry points that need no device behave.  Also guards the product
+tree against routing through the CPU oracle."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "torch-ccl_amd")
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mcclb?_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_libmi355ccl_exports_every_declared_symbol(mccl):
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    names = _declared("mccl.h")
+    assert len(names) >= 14
+    for name in names:
+        assert hasattr(L, name), "libmi355ccl.so does not export %s" % name
+    assert sorted(capi.EXPORTS) == names
+
+
+def test_libmcclbench_exports_every_declared_symbol(mccl):
+    from torch_ccl_amd import benchlib
+    L = benchlib.lib()
+    for name in [n for n in _declared("mccl_bench.h") if n.startswith("mcclb_")]:
+        assert hasattr(L, name), "libmcclbench.so does not export %s" % name
+
+
+def test_device_free_entry_points(mccl):
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    assert L.mccl_version() >= 100
+    sizes = {capi.U8: 1, capi.I8: 1, capi.I16: 2, capi.I32: 4, capi.I64: 8,
+             capi.F16: 2, capi.F32: 4, capi.F64: 8, capi.BF16: 2}
+    for code, size in sizes.items():
+        assert L.mccl_dtype_size(code) == size
+    assert L.mccl_dtype_size(99) == 0
+    assert L.mccl_set_tuning(99, 1) == -1
+    assert b"unknown tuning knob" in L.mccl_last_error()
+    default = L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES)
+    assert L.mccl_set_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES, 12345) == 0
+    assert L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES) == 12345
+    assert L.mccl_set_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES, 0) == 0
+    assert L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES) == default
+
+
+def test_argument_errors_need_no_device(mccl):
+    """Validation happens before any HIP call: bad arguments come back as status codes."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    one = capi.ptr_table([0x1000])
+    assert L.mccl_reduce_n(None, 2, None, 8, capi.F32, capi.SUM, 0, None) == -1
+    assert L.mccl_reduce_n(one, 0, None, 8, capi.F32, capi.SUM, 0, None) == -1
+    assert L.mccl_reduce_n(one, 65, None, 8, capi.F32, capi.SUM, 0, None) == -1
+    assert L.mccl_reduce_n(one, 1, None, 8, 42, capi.SUM, 0, None) == -1
+    assert L.mccl_reduce_n(one, 1, None, 8, capi.F32, 7, 0, None) == -1
+    assert L.mccl_reduce_n(one, 1, None, 8, capi.I32, capi.AVG, 0, None) == -3
+    assert b"AVG" in L.mccl_last_error()
+    assert L.mccl_reduce_n(one, 1, None, 0, capi.F32, capi.SUM, 0, None) == 0  # empty message: no-op
+    assert L.mccl_allgather_n(one, 1, None, 0, None) == 0
+    assert L.mccl_copy_segments(None, 0, None) == 0
+    assert L.mccl_copy_segments(None, 3, None) == -1
+
+
+def test_tensor_front_end_rejects_cpu_tensors(mccl):
+    import torch
+    with pytest.raises(RuntimeError, match="must be on the GPU"):
+        mccl.reduce_n([torch.zeros(4), torch.zeros(4)])
+
+
+def test_product_tree_never_touches_the_oracle():
+    """The oracle is the checker; nothing that ships may import, load or call it."""
+    offenders = []
+    for base, _, files in os.walk(PKG):
+        for name in files:
+            if name.endswith((".py", ".hip", ".cpp", ".h", ".hpp")):
+                text = open(os.path.join(base, name), errors="ignore").read()
+                if re.search(r"\boracle\b", text):
+                    offenders.append(os.path.join(base, name))
+    assert not offenders, offenders
+
+
+def test_isa_guard_flags_nothing():
+    """Compiles the device code to assembly and scans for the stale-SCC select pattern."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("check_isa", os.path.join(PKG, "csrc", "check_isa.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert mod.main() == 0

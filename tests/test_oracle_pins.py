@@ -1,0 +1,203 @@
+"""Pins for what the reference's tests leave open in the oracle: conversions against library
+routines (numpy float16, torch bfloat16), rounding-order known answers chosen so that a
+plausible mistake (wrong order, per-step rounding, dropped rank, non-zero start) fails,
+and index maps against brute-force Python loops on tagged tiny inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+
+# ---------------- conversions ----------------
+
+def _float_patterns(rng, n):
+    """fp32 bit patterns: uniform random bits plus every exponent crossed with edge mantissas."""
+    rnd = rng.integers(0, 2 ** 32, size=n, dtype=np.uint64).astype(np.uint32)
+    exps = np.arange(256, dtype=np.uint32) << 23
+    mans = np.array([0, 1, 0xfff, 0x1000, 0x1001, 0x1fff, 0x2000, 0x2001, 0x3000, 0x7fff, 0x8000, 0x8001,
+                     0xffff, 0x10000, 0x18000, 0x3fffff, 0x400000, 0x7fe000, 0x7ff000, 0x7fffff], dtype=np.uint32)
+    edge = (exps[:, None] | mans[None, :]).reshape(-1)
+    edge = np.concatenate([edge, edge | np.uint32(0x80000000)])
+    return np.concatenate([rnd, edge]).view(np.float32)
+
+
+def test_f16_to_f32_exhaustive_vs_numpy():
+    h = np.arange(65536, dtype=np.uint16)
+    got = O.f16_to_f32(h).view(np.uint32)
+    want = h.view(np.float16).astype(np.float32).view(np.uint32)
+    nan = np.isnan(h.view(np.float16))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(got.view(np.float32)[nan]).all()
+
+
+def test_f32_to_f16_vs_numpy():
+    x = _float_patterns(np.random.default_rng(1), 4_000_000)
+    got = O.f32_to_f16(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert (got[nan] == 0x7e00).all()  # canonical quiet NaN
+
+
+def test_f32_to_bf16_vs_torch():
+    x = _float_patterns(np.random.default_rng(2), 4_000_000)
+    got = O.f32_to_bf16(x)
+    want = torch.from_numpy(x.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert (got[nan] == 0x7fc0).all()
+    # and back: widening is exact
+    assert np.array_equal(O.bf16_to_f32(got[~nan]).view(np.uint32), got[~nan].astype(np.uint32) << 16)
+
+
+# ---------------- rounding order and accumulation width ----------------
+
+def test_fp32_sum_is_ascending_rank_order():
+    """(((0 + 1e8) + 1) - 1e8) = 0 in fp32, any other order of the three gives 1 or 8."""
+    a, b, c = np.float32(1e8), np.float32(1.0), np.float32(-1e8)
+    got = O.reduce([np.array([a]), np.array([b]), np.array([c])], O.F32, O.SUM)
+    assert got[0] == np.float32(0.0)
+    got = O.reduce([np.array([a]), np.array([c]), np.array([b])], O.F32, O.SUM)
+    assert got[0] == np.float32(1.0)
+
+
+def test_fp32_sum_starts_from_positive_zero():
+    """result = 0; result += x_r : an all -0 column gives +0 (bit pattern 0), not -0."""
+    neg0 = np.array([-0.0], dtype=np.float32)
+    for n in (1, 2, 5):
+        got = O.reduce([neg0] * n, O.F32, O.SUM)
+        assert got.view(np.uint32)[0] == 0
+    # MIN/MAX/PRODUCT start from rank 0's value instead
+    assert O.reduce([neg0, neg0], O.F32, O.PROD).view(np.uint32)[0] == 0  # (-0)*(-0) = +0
+    assert O.reduce([neg0], O.F32, O.MIN).view(np.uint32)[0] == 0x80000000
+
+
+def test_fp32_two_rank_sum_matches_numpy():
+    rng = np.random.default_rng(3)
+    a = rng.uniform(-1, 1, 100000).astype(np.float32)
+    b = rng.uniform(-1, 1, 100000).astype(np.float32)
+    assert np.array_equal(O.reduce([a, b], O.F32, O.SUM).view(np.uint32), (a + b).view(np.uint32))
+
+
+def test_bf16_accumulates_in_fp32_and_rounds_once():
+    """1 + 3 * 2^-9: fp32 accumulation gives 1 + 0.75 ulp -> rounds up to 0x3F81; rounding to
+    bf16 after every add would stay at 1.0 (0x3F80)."""
+    one = O.f32_to_bf16(np.array([1.0], dtype=np.float32))
+    tiny = O.f32_to_bf16(np.array([2.0 ** -9], dtype=np.float32))
+    assert O.reduce([one, tiny, tiny, tiny], O.BF16, O.SUM)[0] == 0x3F81
+    # tie: 1 + 2 * 2^-9 = 1 + 0.5 ulp -> round to even -> 1.0
+    assert O.reduce([one, tiny, tiny], O.BF16, O.SUM)[0] == 0x3F80
+    # tie above an odd mantissa rounds up: (1 + ulp) + 0.5 ulp -> 1 + 2 ulp
+    odd = np.array([0x3F81], dtype=np.uint16)
+    assert O.reduce([odd, tiny, tiny], O.BF16, O.SUM)[0] == 0x3F82
+
+
+def test_f16_accumulates_in_fp32_and_rounds_once():
+    """Same construction for fp16 (ulp at 1.0 is 2^-10): 1 + 3 * 2^-12 -> 0x3C01."""
+    one = O.f32_to_f16(np.array([1.0], dtype=np.float32))
+    tiny = O.f32_to_f16(np.array([2.0 ** -12], dtype=np.float32))
+    assert O.reduce([one, tiny, tiny, tiny], O.F16, O.SUM)[0] == 0x3C01
+    assert O.reduce([one, tiny, tiny], O.F16, O.SUM)[0] == 0x3C00
+    # overflow to infinity happens only at the final rounding: 60000 + 60000 - 60000 = 60000
+    big = O.f32_to_f16(np.array([60000.0], dtype=np.float32))
+    nbig = O.f32_to_f16(np.array([-60000.0], dtype=np.float32))
+    assert O.reduce([big, big, nbig], O.F16, O.SUM)[0] == big[0]
+    assert O.reduce([big, big], O.F16, O.SUM)[0] == 0x7C00
+
+
+def test_bf16_chain_matches_torch_fp32_chain():
+    """An independent restatement with torch CPU ops: fp32 running sum, one cast at the end."""
+    rng = np.random.default_rng(4)
+    n, count = 8, 50000
+    ins = [O.f32_to_bf16((rng.standard_normal(count) * 0.02).astype(np.float32)) for _ in range(n)]
+    acc = torch.zeros(count, dtype=torch.float32)
+    for x in ins:
+        acc = acc + torch.from_numpy(x.view(np.int16).copy()).view(torch.bfloat16).float()
+    want = acc.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(O.reduce(ins, O.BF16, O.SUM), want)
+
+
+@pytest.mark.parametrize("dtype,np_t", [(O.U8, np.uint8), (O.I8, np.int8), (O.I16, np.int16),
+                                        (O.I32, np.int32), (O.I64, np.int64)])
+def test_integer_sum_and_product_wrap(dtype, np_t):
+    rng = np.random.default_rng(5)
+    info = np.iinfo(np_t)
+    ins = [rng.integers(info.min, info.max, size=1000, dtype=np_t, endpoint=True) for _ in range(7)]
+    with np.errstate(over="ignore"):
+        s = np.zeros(1000, dtype=np_t)
+        p = np.ones(1000, dtype=np_t)
+        for x in ins[::-1]:  # wrap-around arithmetic is associative and commutative: any order
+            s = s + x
+            p = p * x
+    assert np.array_equal(O.reduce(ins, dtype, O.SUM), s)
+    assert np.array_equal(O.reduce(ins, dtype, O.PROD), p)
+    assert np.array_equal(O.reduce(ins, dtype, O.MIN), np.minimum.reduce(ins))
+    assert np.array_equal(O.reduce(ins, dtype, O.MAX), np.maximum.reduce(ins))
+
+
+def test_threads_do_not_change_results():
+    rng = np.random.default_rng(6)
+    ins = [O.f32_to_bf16(rng.standard_normal(300001).astype(np.float32)) for _ in range(8)]
+    one = O.reduce(ins, O.BF16, O.SUM)
+    O.set_threads(4)
+    try:
+        four = O.reduce(ins, O.BF16, O.SUM)
+    finally:
+        O.set_threads(1)
+    assert np.array_equal(one, four)
+
+
+# ---------------- index maps: brute force on tagged inputs ----------------
+
+def test_reduce_scatter_is_sliced_reduce():
+    rng = np.random.default_rng(7)
+    n, m = 5, 37
+    ins = [rng.integers(-1000, 1000, size=n * m).astype(np.int32) for _ in range(n)]
+    full = O.reduce(ins, O.I32, O.SUM)
+    outs = O.reduce_scatter(ins, O.I32, O.SUM)
+    for s in range(n):
+        assert np.array_equal(outs[s], full[s * m:(s + 1) * m])
+    assert np.array_equal(O.reduce_scatter(ins, O.I32, O.SUM, shard_first=3, shard_num=1)[0], full[3 * m:4 * m])
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+def test_alltoallv_brute_force(n):
+    """Every element is tagged (source rank, row, column); the receive side is rebuilt with
+    plain Python loops from the definition: rank d's segment r = rank r's segment d."""
+    rng = np.random.default_rng(n)
+    row = 3
+    S = rng.integers(0, 5, size=(n, n))
+    ins = []
+    for r in range(n):
+        rows = int(S[r].sum())
+        ins.append(np.array([[r * 1_000_000 + i * 10 + c for c in range(row)] for i in range(rows)],
+                            dtype=np.int32).reshape(-1))
+    outs = O.alltoallv(ins, S, row * 4)
+    for d in range(n):
+        want = []
+        for r in range(n):
+            start = sum(int(S[r][dd]) for dd in range(d))
+            for i in range(start, start + int(S[r][d])):
+                want.extend(r * 1_000_000 + i * 10 + c for c in range(row))
+        assert outs[d].view(np.int32).tolist() == want
+
+
+def test_allgather_pack_unpack_brute_force():
+    ins = [np.arange(5, dtype=np.int16) + 100 * r for r in range(4)]
+    assert O.allgather(ins).view(np.int16).tolist() == [100 * r + i for r in range(4) for i in range(5)]
+    parts = [np.arange(k + 1, dtype=np.uint8) + 10 * k for k in range(6)]
+    flat = O.pack(parts)
+    assert flat.tolist() == [10 * k + i for k in range(6) for i in range(k + 1)]
+    back = O.unpack(flat, [k + 1 for k in range(6)])
+    assert all(np.array_equal(a, b) for a, b in zip(back, parts))
+
+
+def test_alltoall_counts_equal_and_empty():
+    counts, displs = O.alltoall_counts(4, 48, 12, None)      # equal split: numel / world
+    assert counts.tolist() == [12] * 4 and displs.tolist() == [0, 12, 24, 36]
+    counts, displs = O.alltoall_counts(3, 60, 10, [1, 0, 9])  # rowLen = 60/10 = 6
+    assert counts.tolist() == [6, 0, 54] and displs.tolist() == [0, 6, 6]
+    counts, displs = O.alltoall_counts(3, 0, 0, [0, 0, 0])    # empty tensor: no division
+    assert counts.tolist() == [0, 0, 0]
