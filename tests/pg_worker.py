@@ -1,0 +1,250 @@
+"""Rank body for the backend tests: N ranks (processes or threads) share cuda:0 and replay the
+reference's functional cases (tests/test_c10d_ccl.py, via tests/golden/c10d_kats.json) plus
+seeded random cases checked bit for bit against the CPU oracle."""
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "torch-ccl_amd"), os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+import torch  # noqa: E402
+import torch.distributed as dist  # noqa: E402
+import torch.distributed.distributed_c10d as c10d  # noqa: E402
+
+DEV = "cuda:0"
+
+
+def _kats(world):
+    with open(os.path.join(ROOT, "tests", "golden", "c10d_kats.json")) as f:
+        return json.load(f)["world_sizes"][str(world)]
+
+
+def _dev(x, dtype=None):
+    return torch.tensor(x, dtype=dtype).to(DEV)
+
+
+def reference_cases(pg, rank, world):
+    """The closed-form cases of the reference's ProcessGroupCCLTest, on GPU tensors."""
+    K = _kats(world)
+    ops = {"SUM": c10d.ReduceOp.SUM, "PRODUCT": c10d.ReduceOp.PRODUCT, "MIN": c10d.ReduceOp.MIN,
+           "MAX": c10d.ReduceOp.MAX}
+    # allreduce basics (:173-187)
+    for name, want in K["allreduce"]["expected"].items():
+        opts = c10d.AllreduceOptions()
+        opts.reduceOp = ops[name]
+        t = _dev(K["allreduce"]["inputs"][rank])
+        pg.allreduce([t], opts).wait()
+        assert t.cpu().tolist() == want, (name, t.cpu().tolist(), want)
+    # allreduce_coalesced (:200-209)
+    ts = [_dev(v, torch.float32) for v in K["allreduce_coalesced"]["inputs"][rank]]
+    opts = c10d.AllreduceCoalescedOptions()
+    opts.reduceOp = c10d.ReduceOp.SUM
+    pg.allreduce_coalesced(ts, opts).wait()
+    for t, want in zip(ts, K["allreduce_coalesced"]["expected"]):
+        assert t.cpu().tolist() == want
+    # _reduce_scatter_base (:550-566)
+    out = torch.empty(1, device=DEV)
+    pg._reduce_scatter_base(out, _dev(K["reduce_scatter_base"]["inputs"][rank], torch.float32)).wait()
+    assert out.cpu().tolist() == K["reduce_scatter_base"]["expected"][rank]
+    # reduce_scatter, list form (:579-610) and variable-length slots (:623-653)
+    for key in ("reduce_scatter_list", "reduce_scatter_list_variable"):
+        want = K[key]["expected"][rank]
+        out = [_dev([0] * len(want))]
+        ins = [[_dev(v) for v in K[key]["inputs"][rank]]]
+        opts = c10d.ReduceScatterOptions()
+        opts.reduceOp = c10d.ReduceOp.SUM
+        pg.reduce_scatter(out, ins, opts).wait()
+        assert out[0].cpu().tolist() == want, (key, out[0].cpu().tolist(), want)
+    # _allgather_base (:377-391) and its error strings (:404-429)
+    out = torch.empty(world, dtype=torch.int64, device=DEV)
+    pg._allgather_base(out, _dev(K["allgather_base"]["inputs"][rank])).wait()
+    assert out.cpu().tolist() == K["allgather_base"]["expected"]
+    try:
+        pg._allgather_base(torch.empty(world + 1, dtype=torch.int64, device=DEV), _dev([rank]))
+        raise AssertionError("size check did not fire")
+    except RuntimeError as e:
+        assert "output tensor size must be equal to world_size times input tensor size" in str(e)
+    try:
+        pg._allgather_base(torch.empty(world + 1, dtype=torch.int64, device=DEV), _dev([rank], torch.float32))
+        raise AssertionError("dtype check did not fire")
+    except RuntimeError as e:
+        assert "Tensors are not equal in data type" in str(e)
+    # allgather, list form (:345-364)
+    for sub in K["allgather_list"]:
+        outs = [[_dev([-1]) for _ in range(world)]]
+        pg.allgather(outs, [_dev(sub["inputs"][rank])]).wait()
+        assert [t.cpu().tolist() for t in outs[0]] == sub["expected"]
+    # alltoall_base, equal (:443-456) and uneven (:458-473) splits
+    out = torch.ones(world, world, device=DEV) * -1
+    pg.alltoall_base(out, _dev(K["alltoall_base_equal"]["inputs"][rank], torch.float32), [], []).wait()
+    assert out.cpu().tolist() == K["alltoall_base_equal"]["expected"][rank]
+    U = K["alltoall_base_unequal"]
+    out = torch.ones((rank + 1) * world, world, device=DEV)
+    pg.alltoall_base(out, _dev(U["inputs"][rank], torch.float32), U["out_splits"][rank], U["in_splits"][rank]).wait()
+    assert out.cpu().tolist() == U["expected"][rank]
+    # alltoall, list form (:498-518)
+    L = K["alltoall_list"]
+    outs = [torch.ones(rank + 1, world, device=DEV) for _ in range(world)]
+    pg.alltoall(outs, [_dev(v, torch.float32) for v in L["inputs"][rank]]).wait()
+    assert [t.cpu().tolist() for t in outs] == L["expected"][rank]
+    # broadcast root check (:109-113)
+    try:
+        opts = c10d.BroadcastOptions()
+        opts.rootRank = -1
+        opts.rootTensor = 0
+        pg.broadcast([torch.zeros(1, device=DEV)], opts)
+        raise AssertionError("rank check did not fire")
+    except ValueError as e:
+        assert "unexpected rank" in str(e)
+    # broadcast data (each root in turn)
+    for root in range(world):
+        opts = c10d.BroadcastOptions()
+        opts.rootRank = root
+        opts.rootTensor = 0
+        t = torch.full((1000,), float(rank), device=DEV)
+        pg.broadcast([t], opts).wait()
+        assert t.cpu().tolist() == [float(root)] * 1000
+    pg.barrier().wait()
+
+
+def oracle_cases(pg, rank, world):
+    """Seeded random buffers: every rank rebuilds all ranks' inputs on the CPU, runs the oracle
+    and compares its own GPU result bit for bit."""
+    from helpers import TORCH_TO_CODE, bits, rank_buffer, to_carrier
+    from oracle import oracle as O
+
+    def bits_np(arr):
+        return arr.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[arr.dtype.itemsize])
+
+    for dtype in (torch.bfloat16, torch.float16, torch.float32, torch.int32):
+        code = TORCH_TO_CODE[dtype]
+        for count in (1, 1000, 131072, (1 << 20) + 3):
+            host = [rank_buffer(count, dtype, r, seed=99) for r in range(world)]
+            t = host[rank].to(DEV)
+            pg.allreduce([t], c10d.AllreduceOptions()).wait()
+            want = bits_np(O.reduce([to_carrier(h) for h in host], code, O.SUM))
+            assert np.array_equal(bits(t), want), ("allreduce", dtype, count)
+        # reduce_scatter_tensor
+        m = 4099
+        host = [rank_buffer(world * m, dtype, r, seed=7) for r in range(world)]
+        out = torch.empty(m, dtype=dtype, device=DEV)
+        pg._reduce_scatter_base(out, host[rank].to(DEV)).wait()
+        want = O.reduce_scatter([to_carrier(h) for h in host], code, O.SUM, shard_first=rank, shard_num=1)[0]
+        assert np.array_equal(bits(out), bits_np(want)), ("reduce_scatter", dtype)
+        # all_gather_into_tensor
+        host = [rank_buffer(m, dtype, r, seed=8) for r in range(world)]
+        out = torch.empty(world * m, dtype=dtype, device=DEV)
+        pg._allgather_base(out, host[rank].to(DEV)).wait()
+        assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather", dtype)
+    # MIN / MAX / PRODUCT / AVG on floats
+    for opname, op, ocode in (("min", c10d.ReduceOp.MIN, O.MIN), ("max", c10d.ReduceOp.MAX, O.MAX),
+                              ("prod", c10d.ReduceOp.PRODUCT, O.PROD)):
+        host = [rank_buffer(5000, torch.float32, r, seed=11, scale=1.0) for r in range(world)]
+        t = host[rank].to(DEV)
+        opts = c10d.AllreduceOptions()
+        opts.reduceOp = op
+        pg.allreduce([t], opts).wait()
+        assert np.array_equal(bits(t), bits_np(O.reduce([to_carrier(h) for h in host], O.F32, ocode))), opname
+    # uneven all_to_all_single: a seeded split matrix every rank agrees on
+    rng = np.random.default_rng(1234)
+    S = rng.integers(0, 300, size=(world, world))
+    S[0, world - 1] = 0
+    hidden = 96
+    host = [rank_buffer(int(S[r].sum()) * hidden, torch.bfloat16, r, seed=5).view(-1, hidden) for r in range(world)]
+    out = torch.zeros(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device=DEV)
+    pg.alltoall_base(out, host[rank].to(DEV), S[:, rank].tolist(), S[rank].tolist()).wait()
+    want = O.alltoallv([to_carrier(h) for h in host], S, hidden * 2)[rank]
+    assert np.array_equal(out.cpu().view(torch.uint8).numpy().reshape(-1), want), "alltoallv"
+    pg.barrier().wait()
+
+
+def dist_api_cases(rank, world):
+    """The public torch.distributed entry points on the default group (backend "ccl")."""
+    t = torch.full((1 << 16,), float(rank + 1), device=DEV)
+    dist.all_reduce(t)
+    assert torch.equal(t.cpu(), torch.full((1 << 16,), world * (world + 1) / 2.0))
+    w = dist.all_reduce(t, async_op=True)
+    w.wait()
+    torch.cuda.synchronize()
+    assert float(t[0]) == world * world * (world + 1) / 2.0
+    fut = dist.all_reduce(t, async_op=True).get_future()
+    fut.wait()
+    assert float(t[123]) == world ** 2 * world * (world + 1) / 2.0
+    # reduce_scatter_tensor / all_gather_into_tensor / all_to_all_single
+    inp = torch.arange(world * 4, dtype=torch.float32, device=DEV)
+    out = torch.empty(4, device=DEV)
+    dist.reduce_scatter_tensor(out, inp)
+    assert out.cpu().tolist() == [world * (rank * 4 + j) for j in range(4)]
+    gathered = torch.empty(world * 3, device=DEV)
+    dist.all_gather_into_tensor(gathered, torch.full((3,), float(rank), device=DEV))
+    assert gathered.cpu().tolist() == [float(r) for r in range(world) for _ in range(3)]
+    a2a = torch.empty(world * 2, device=DEV)
+    dist.all_to_all_single(a2a, torch.full((world * 2,), float(rank), device=DEV))
+    assert a2a.cpu().tolist() == [float(r) for r in range(world) for _ in range(2)]
+    # AVG
+    t = torch.full((100,), float(rank), device=DEV)
+    dist.all_reduce(t, op=dist.ReduceOp.AVG)
+    assert torch.allclose(t.cpu(), torch.full((100,), (world - 1) / 2.0))
+    # coalescing manager (:667-693): two 8-element allreduces equal one 16-element allreduce
+    small = [torch.ones(8, device=DEV) for _ in range(2)]
+    with c10d._coalescing_manager(device=torch.device(DEV)):
+        for s in small:
+            dist.all_reduce(s)
+    torch.cuda.synchronize()
+    big = torch.ones(16, device=DEV)
+    dist.all_reduce(big)
+    for i in range(2):
+        assert torch.equal(small[i].cpu(), big[i * 8:(i + 1) * 8].cpu())
+    # reduce_scatter_tensor of ones (:716-733)
+    o = torch.zeros(2, 2, device=DEV)
+    dist.reduce_scatter_tensor(o, torch.ones(world * 2, 2, device=DEV))
+    assert torch.equal(o.cpu(), torch.full((2, 2), float(world)))
+    # unsupported reduce op and collectives outside the path
+    try:
+        dist.all_reduce(torch.ones(4, dtype=torch.int32, device=DEV), op=dist.ReduceOp.BAND)
+        raise AssertionError("BAND accepted")
+    except RuntimeError as e:
+        assert "Cannot use ReduceOp.BAND" in str(e)
+    dist.barrier()
+
+
+def large_message_case(pg, rank, world):
+    """A message larger than one staging window (1 GiB) is cut into windows."""
+    count = (1 << 28) + 12345  # 1 GiB + a bit of fp32
+    t = torch.arange(count, dtype=torch.float32, device=DEV) * 0 + float(rank + 1)
+    t[-1] = 7.0 * (rank + 1)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    torch.cuda.synchronize()
+    s = world * (world + 1) / 2.0
+    assert float(t[0]) == s and float(t[count // 2]) == s and float(t[-2]) == s and float(t[-1]) == 7.0 * s
+    assert float(t.min()) == s
+
+
+def run_rank(rank, world, store_path, mode):
+    torch.cuda.set_device(0)
+    import torch_ccl_amd  # noqa: F401  registers the backend
+    if mode == "dist":
+        store = dist.FileStore(store_path, world)
+        dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
+        try:
+            dist_api_cases(rank, world)
+        finally:
+            dist.destroy_process_group()
+        return
+    store = dist.FileStore(store_path, world)
+    pg = dist.ProcessGroupCCL(store, rank, world)
+    assert pg.name() == "ccl" and pg.rank() == rank and pg.size() == world
+    if mode == "reference":
+        reference_cases(pg, rank, world)
+    elif mode == "oracle":
+        oracle_cases(pg, rank, world)
+    elif mode == "large":
+        large_message_case(pg, rank, world)
+    else:
+        raise ValueError(mode)
+    torch.cuda.synchronize()
+    del pg

@@ -1,0 +1,62 @@
+"""No-GPU checks of the c10d backend: registration contract, construction, argument errors that
+are raised before any device work."""
+import os
+import tempfile
+
+import pytest
+import torch
+import torch.distributed as dist
+
+
+@pytest.fixture(scope="module")
+def pkg(mccl):
+    return mccl
+
+
+def _pg(world=1, rank=0):
+    d = tempfile.mkdtemp()
+    return dist.ProcessGroupCCL(dist.FileStore(os.path.join(d, "s"), world), rank, world)
+
+
+def test_registration_contract(pkg):
+    """import registers backend "ccl" for ROCm ("cuda") tensors and attaches ProcessGroupCCL to
+    torch.distributed (oneccl_bindings_for_pytorch/csrc/init.cpp:123-154)."""
+    assert "ccl" in dist.Backend.backend_list and "mccl" in dist.Backend.backend_list
+    assert dist.Backend.backend_capability["ccl"] == ["cuda"]
+    assert dist.ProcessGroupCCL is pkg.ProcessGroupCCL
+    assert issubclass(dist.ProcessGroupCCL, torch._C._distributed_c10d.Backend)
+
+
+def test_construct_without_gpu(pkg):
+    pg = _pg(world=4, rank=3)
+    assert pg.name() == "ccl" and pg.rank() == 3 and pg.size() == 4
+    with pytest.raises(ValueError, match="unexpected rank"):
+        _pg(world=2, rank=2)
+
+
+def test_unexpected_root_rank(pkg):
+    """tests/test_c10d_ccl.py:109-113"""
+    pg = _pg()
+    opts = dist.BroadcastOptions()
+    opts.rootRank = -1
+    opts.rootTensor = 0
+    with pytest.raises(ValueError, match="unexpected rank"):
+        pg.broadcast([torch.zeros(1)], opts)
+
+
+def test_cpu_tensors_are_rejected(pkg):
+    pg = _pg()
+    with pytest.raises(RuntimeError, match="Tensors are not in same device type"):
+        pg.allreduce([torch.zeros(4)])
+    with pytest.raises(RuntimeError, match="Tensors are not equal in data type"):
+        pg._allgather_base(torch.zeros(2, dtype=torch.int64), torch.zeros(1))
+    with pytest.raises(RuntimeError, match="does not support tensors count 2"):
+        pg.allreduce([torch.zeros(1), torch.zeros(1)])
+
+
+def test_collectives_outside_the_path_fail_like_the_reference(pkg):
+    pg = _pg()
+    with pytest.raises(RuntimeError, match="isn't implementd on backend"):
+        pg.reduce([torch.zeros(1)])
+    with pytest.raises(RuntimeError, match="does not support allgather_coalesced"):
+        pg.allgather_coalesced([[torch.zeros(1)]], [torch.zeros(1)])

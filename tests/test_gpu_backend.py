@@ -1,0 +1,51 @@
+"""The c10d backend "ccl" end to end on one GPU: N rank processes share cuda:0, rendezvous through
+a FileStore and construct ProcessGroupCCL(store, rank, size) directly, the way the reference's
+MultiProcessTestCase does (tests/test_c10d_ccl.py:97-103)."""
+import os
+import tempfile
+
+import pytest
+import torch
+import torch.multiprocessing as mp
+
+import pg_worker
+
+pytestmark = pytest.mark.gpu
+
+
+def _spawn(world, mode):
+    with tempfile.TemporaryDirectory() as d:
+        mp.spawn(pg_worker.run_rank, args=(world, os.path.join(d, "store"), mode), nprocs=world, join=True)
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_reference_cases(world):
+    _spawn(world, "reference")
+
+
+@pytest.mark.parametrize("world", [2, 8])
+def test_random_cases_against_oracle(world):
+    _spawn(world, "oracle")
+
+
+@pytest.mark.parametrize("world", [2, 4])
+def test_torch_distributed_api(world):
+    _spawn(world, "dist")
+
+
+def test_message_larger_than_one_staging_window():
+    _spawn(2, "large")
+
+
+def test_world_size_one_is_a_no_op():
+    """world == 1: allreduce leaves the tensor alone (src/gpu/dpcpp_ccl.cpp:752-756), -0.0 included."""
+    import torch.distributed as dist
+    import torch_ccl_amd  # noqa: F401
+    with tempfile.TemporaryDirectory() as d:
+        pg = dist.ProcessGroupCCL(dist.FileStore(os.path.join(d, "s"), 1), 0, 1)
+        t = torch.tensor([-0.0, 1.5], device="cuda:0")
+        pg.allreduce([t]).wait()
+        assert t.cpu().view(torch.int32).tolist() == torch.tensor([-0.0, 1.5]).view(torch.int32).tolist()
+        out = torch.empty(2, device="cuda:0")
+        pg._allgather_base(out, t).wait()
+        assert torch.equal(out.cpu(), t.cpu())

@@ -2,6 +2,8 @@
 
   libmi355ccl.so   HIP kernels + C ABI (include/mccl.h); depends on the HIP runtime only.
   libmcclbench.so  HIP-event timing loops around that ABI (include/mccl_bench.h).
+  _C.*.so          the c10d backend (process_group_ccl.cpp) and its Python module; host code
+                   only, links torch's c10d and libmi355ccl.so.
 
 Usage: python torch-ccl_amd/csrc/build.py [--force]
 Outputs land in torch-ccl_amd/torch_ccl_amd/lib/.
@@ -62,8 +64,47 @@ def build_bench(force=False):
     return BENCH_LIB
 
 
+BACKEND_SRCS = [os.path.join(HERE, "process_group_ccl.cpp"), os.path.join(HERE, "python_module.cpp")]
+BACKEND_HDRS = [os.path.join(HERE, "process_group_ccl.hpp"), os.path.join(INCLUDE, "mccl.h")]
+
+
+def backend_lib_path():
+    import sysconfig
+    return os.path.join(os.path.dirname(LIB_DIR), "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_backend(force=False):
+    """The c10d backend is host-only C++ (no device code): g++ against torch's headers."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ext
+    out = backend_lib_path()
+    if not (force or _stale(out, BACKEND_SRCS + BACKEND_HDRS)):
+        return out
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = []
+    for d in ext.include_paths("cuda") + [sysconfig.get_paths()["include"], INCLUDE, HERE]:
+        inc += ["-isystem" if "torch" in d or "rocm" in d or "python" in d else "-I", d]
+    objs = []
+    for src in BACKEND_SRCS:
+        obj = os.path.join(LIB_DIR, os.path.basename(src) + ".o")
+        cmd = ["g++", "-c", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unknown-pragmas",
+               "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
+               "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)] + inc + ["-o", obj, src]
+        subprocess.check_call(cmd)
+        objs.append(obj)
+    cmd = ["g++", "-shared", "-o", out] + objs + [
+        "-L", torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-ltorch_python", "-lc10_hip", "-ltorch_hip",
+        "-lamdhip64", "-L", LIB_DIR, "-lmi355ccl", "-lrt", "-lpthread",
+        "-Wl,-rpath,$ORIGIN/lib", "-Wl,-rpath," + torch_lib]
+    subprocess.check_call(cmd)
+    for obj in objs:
+        os.remove(obj)
+    return out
+
+
 def build_all(force=False):
-    return [build_kernels(force), build_bench(force)]
+    return [build_kernels(force), build_bench(force), build_backend(force)]
 
 
 if __name__ == "__main__":

@@ -1,0 +1,975 @@
+// c10d backend "ccl" for ROCm tensors: see process_group_ccl.hpp for the design.
+#include "process_group_ccl.hpp"
+
+#include <ATen/hip/impl/HIPCachingAllocatorMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <ATen/record_function.h>
+#include <c10/core/DeviceGuard.h>
+#include <fcntl.h>
+#include <sched.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <iostream>
+#include <sstream>
+#include <stdexcept>
+#include <thread>
+
+#include "mccl.h"
+
+namespace mccl_pg {
+
+namespace {
+
+constexpr int kMaxWorld = MCCL_MAX_RANKS;
+constexpr int kTableMax = 2 * kMaxWorld + 8;
+constexpr size_t kStageMin = 2u << 20;   // first staging allocation
+constexpr size_t kStageMax = 1u << 30;   // one staging window; keeps every IPC allocation < 2 GiB
+constexpr uint32_t kMagic = 0x4d43434c;  // "MCCL"
+
+#define HIP_CHECK(expr)                                                                     \
+  do {                                                                                      \
+    hipError_t e_ = (expr);                                                                 \
+    TORCH_CHECK(e_ == hipSuccess, "ccl backend: ", #expr, " failed: ", hipGetErrorString(e_)); \
+  } while (0)
+
+#define MCCL_CHECK(expr)                                                         \
+  do {                                                                           \
+    int rc_ = (expr);                                                            \
+    TORCH_CHECK(rc_ == MCCL_OK, "ccl backend: ", #expr, ": ", mccl_last_error()); \
+  } while (0)
+
+bool envFlag(const char* name, bool dflt) {
+  const char* v = std::getenv(name);
+  if (!v || !*v) return dflt;
+  return std::atoi(v) != 0;
+}
+
+// cclDatatypes of the reference (src/utils.cpp:46-58)
+int dtypeCode(at::ScalarType t) {
+  switch (t) {
+    case at::kByte: return MCCL_U8;
+    case at::kChar: return MCCL_I8;
+    case at::kShort: return MCCL_I16;
+    case at::kInt: return MCCL_I32;
+    case at::kLong: return MCCL_I64;
+    case at::kHalf: return MCCL_F16;
+    case at::kFloat: return MCCL_F32;
+    case at::kDouble: return MCCL_F64;
+    case at::kBFloat16: return MCCL_BF16;
+    case at::kBool: return MCCL_U8;
+    default: TORCH_CHECK(false, "ccl backend: unsupported data type ", c10::toString(t));
+  }
+}
+
+const char* reduceOpName(c10d::ReduceOp::RedOpType op) {
+  switch (op) {
+    case c10d::ReduceOp::SUM: return "SUM";
+    case c10d::ReduceOp::AVG: return "AVG";
+    case c10d::ReduceOp::PRODUCT: return "PRODUCT";
+    case c10d::ReduceOp::MIN: return "MIN";
+    case c10d::ReduceOp::MAX: return "MAX";
+    case c10d::ReduceOp::BAND: return "BAND";
+    case c10d::ReduceOp::BOR: return "BOR";
+    case c10d::ReduceOp::BXOR: return "BXOR";
+    case c10d::ReduceOp::PREMUL_SUM: return "PREMUL_SUM";
+    default: return "UNUSED";
+  }
+}
+
+// cclOps (src/utils.cpp:38-44) and the device allow-list (src/dispatch_stub.h:320-335).  AVG is
+// accepted for floating-point tensors (the reference rejects it on device).
+int opCode(const c10d::ReduceOp& op, at::ScalarType t) {
+  switch (op.op_) {
+    case c10d::ReduceOp::SUM: return MCCL_SUM;
+    case c10d::ReduceOp::PRODUCT: return MCCL_PROD;
+    case c10d::ReduceOp::MIN: return MCCL_MIN;
+    case c10d::ReduceOp::MAX: return MCCL_MAX;
+    case c10d::ReduceOp::AVG:
+      TORCH_CHECK(at::isFloatingType(t), "Cannot use ReduceOp.AVG with integer tensors on CUDA");
+      return MCCL_AVG;
+    default:
+      TORCH_CHECK(false, "Cannot use ReduceOp.", reduceOpName(op.op_), " with CUDA");
+  }
+}
+
+void checkRank(int rank, int size) {
+  if (!(rank >= 0 && rank < size)) throw std::invalid_argument("unexpected rank");
+}
+
+size_t nbytes(const at::Tensor& t) { return (size_t)t.numel() * t.element_size(); }
+
+size_t roundUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// shared-memory control block
+// ---------------------------------------------------------------------------------------------
+struct alignas(128) RankSlot {
+  std::atomic<uint64_t> arrive;  // host barrier: epoch this rank has reached
+  std::atomic<uint64_t> failed;  // non-zero once the rank gave up; peers stop waiting
+  int64_t pid;
+  // per staging slot; written by the owner before it arrives at the barrier of the collective
+  // that uses the slot, read by the peers after that barrier
+  uint64_t gen[2];
+  uint64_t ptr[2];
+  uint64_t capacity[2];
+  hipIpcMemHandle_t handle[2];
+  int64_t table[2][kTableMax];
+};
+
+struct Control {
+  uint32_t magic;
+  uint32_t world;
+  RankSlot slot[1];  // world entries
+};
+
+static_assert(std::atomic<uint64_t>::is_always_lock_free, "barrier counters must be lock-free");
+
+// ---------------------------------------------------------------------------------------------
+// Work
+// ---------------------------------------------------------------------------------------------
+ProcessGroupCCL::WorkCCL::WorkCCL(int rank, c10d::OpType op, const char* title,
+                                  std::vector<at::Tensor> inputs, std::vector<at::Tensor> outputs,
+                                  bool blocking_wait)
+    : c10d::Work(rank, op, title), blocking_wait_(blocking_wait), inputs_(std::move(inputs)),
+      outputs_(std::move(outputs)) {}
+
+ProcessGroupCCL::WorkCCL::~WorkCCL() {
+  if (end_) (void)hipEventDestroy(end_);
+}
+
+bool ProcessGroupCCL::WorkCCL::isCompleted() {
+  if (!end_) return true;
+  return hipEventQuery(end_) == hipSuccess;
+}
+
+bool ProcessGroupCCL::WorkCCL::isSuccess() const { return true; }
+
+void ProcessGroupCCL::WorkCCL::synchronize() {
+  if (!end_) return;
+  if (blocking_wait_) {
+    HIP_CHECK(hipEventSynchronize(end_));
+  } else {
+    // stream-ordered: the caller's current stream waits for the collective (the queue barrier
+    // of src/gpu/dpcpp_ccl.cpp:440-457)
+    hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
+    HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+  }
+}
+
+bool ProcessGroupCCL::WorkCCL::wait(std::chrono::milliseconds /*timeout*/) {
+  synchronize();
+  return true;
+}
+
+std::vector<at::Tensor> ProcessGroupCCL::WorkCCL::result() { return outputs_; }
+
+c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupCCL::WorkCCL::getFuture() {
+  if (!future_) {
+    std::vector<c10::Device> devs;
+    if (end_) devs.emplace_back(at::kCUDA, (c10::DeviceIndex)device_);
+    future_ = c10::make_intrusive<at::ivalue::Future>(c10::ListType::create(c10::TensorType::get()), devs);
+    if (end_) {
+      c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
+      hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
+      HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+      future_->markCompleted(at::IValue(outputs_));  // records the current stream: ordered after end_
+    } else {
+      future_->markCompleted(at::IValue(outputs_));
+    }
+  }
+  return future_;
+}
+
+// ---------------------------------------------------------------------------------------------
+// construction, rendezvous, staging
+// ---------------------------------------------------------------------------------------------
+ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
+                                 std::chrono::milliseconds timeout)
+    : c10d::Backend(rank, size), store_(store), timeout_(timeout) {
+  TORCH_CHECK(size >= 1 && size <= kMaxWorld, "ccl backend: world size ", size, " outside [1, ", kMaxWorld, "]");
+  checkRank(rank, size);
+  // same switches as the reference (src/ProcessGroupCCL.hpp:96-102, src/env.cpp:11-33)
+  same_stream_ = envFlag("CCL_SAME_STREAM", false);
+  blocking_wait_ = envFlag("CCL_BLOCKING_WAIT", false);
+  verbose_ = envFlag("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", false);
+}
+
+c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_ptr<c10d::Store>& store,
+                                                          int rank, int size,
+                                                          std::chrono::milliseconds timeout) {
+  return c10::make_intrusive<ProcessGroupCCL>(store, rank, size, timeout);
+}
+
+ProcessGroupCCL::~ProcessGroupCCL() {
+  if (!initialised_) return;
+  // Peers may still be reading this rank's staging buffers in their last kernel: wait for our own
+  // stream, then give the others a bounded chance to catch up.  A peer that is already gone has
+  // finished its kernels, so a timeout here is harmless.
+  (void)hipSetDevice(device_);
+  if (comm_stream_) (void)hipStreamSynchronize(comm_stream_);
+  try {
+    auto saved = timeout_;
+    timeout_ = std::chrono::milliseconds(2000);
+    hostBarrier();
+    timeout_ = saved;
+  } catch (...) {
+  }
+  (void)hipDeviceSynchronize();
+  for (auto& pm : peers_)
+    for (int s = 0; s < 2; ++s)
+      if (pm.ipc[s] && pm.ptr[s]) (void)hipIpcCloseMemHandle(pm.ptr[s]);
+  for (int s = 0; s < 2; ++s)
+    if (stage_[s].ptr) (void)hipFree(stage_[s].ptr);
+  for (void* p : retired_) (void)hipFree(p);
+  if (fork_event_) (void)hipEventDestroy(fork_event_);
+  if (ctl_) munmap(ctl_, ctl_bytes_);
+}
+
+void ProcessGroupCCL::ensureInit(int device) {
+  if (initialised_) {
+    TORCH_CHECK(device == device_, "ccl backend: a process group is bound to one device (cuda:", device_,
+                "), got a tensor on cuda:", device);
+    return;
+  }
+  device_ = device;
+  HIP_CHECK(hipSetDevice(device_));
+  comm_stream_ = c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, (c10::DeviceIndex)device_).stream();
+  HIP_CHECK(hipEventCreateWithFlags(&fork_event_, hipEventDisableTiming));
+
+  // Groups are created in the same order on every rank, so a per-rank counter in the store
+  // yields the same id everywhere.
+  const int64_t gid = store_->add("mccl/gid/" + std::to_string(rank_), 1);
+  const std::string key = "mccl/shm/" + std::to_string(gid);
+  ctl_bytes_ = roundUp(sizeof(Control) + sizeof(RankSlot) * (size_t)size_, 4096);
+  int fd = -1;
+  if (rank_ == 0) {
+    const auto now = std::chrono::steady_clock::now().time_since_epoch().count();
+    shm_name_ = "/mccl-" + std::to_string((long)getpid()) + "-" + std::to_string(gid) + "-" +
+                std::to_string((long long)now);
+    fd = shm_open(shm_name_.c_str(), O_CREAT | O_EXCL | O_RDWR, 0600);
+    TORCH_CHECK(fd >= 0, "ccl backend: shm_open(", shm_name_, ") failed: ", std::strerror(errno));
+    TORCH_CHECK(ftruncate(fd, (off_t)ctl_bytes_) == 0, "ccl backend: ftruncate failed: ", std::strerror(errno));
+  } else {
+    auto raw = store_->get(key);  // blocks until rank 0 has published the name
+    shm_name_.assign(raw.begin(), raw.end());
+    fd = shm_open(shm_name_.c_str(), O_RDWR, 0600);
+    TORCH_CHECK(fd >= 0, "ccl backend: shm_open(", shm_name_, ") failed: ", std::strerror(errno));
+  }
+  void* m = mmap(nullptr, ctl_bytes_, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  close(fd);
+  TORCH_CHECK(m != MAP_FAILED, "ccl backend: mmap of the control block failed: ", std::strerror(errno));
+  ctl_ = static_cast<Control*>(m);
+  if (rank_ == 0) {
+    ctl_->magic = kMagic;  // fresh shared memory is zero-filled
+    ctl_->world = (uint32_t)size_;
+    store_->set(key, std::vector<uint8_t>(shm_name_.begin(), shm_name_.end()));
+  }
+  ctl_->slot[rank_].pid = (int64_t)getpid();
+  peers_.assign((size_t)size_, PeerMap{});
+  initialised_ = true;
+  for (int s = 0; s < 2; ++s) ensureStage(s, kStageMin);
+
+  auto saved = timeout_;
+  if (timeout_ < std::chrono::milliseconds(120000)) timeout_ = std::chrono::milliseconds(120000);
+  hostBarrier();
+  timeout_ = saved;
+  TORCH_CHECK(ctl_->magic == kMagic && ctl_->world == (uint32_t)size_,
+              "ccl backend: control block mismatch (ranks disagree on the world size)");
+  if (rank_ == 0) shm_unlink(shm_name_.c_str());  // every rank holds a mapping now
+}
+
+void* ProcessGroupCCL::ensureStage(int slot, size_t bytes) {
+  Stage& st = stage_[slot];
+  if (bytes <= st.capacity) return st.ptr;
+  TORCH_CHECK(bytes <= kStageMax, "ccl backend: staging request of ", bytes, " bytes exceeds the window");
+  size_t cap = kStageMin;
+  while (cap < bytes) cap <<= 1;
+  void* p = nullptr;
+  HIP_CHECK(hipMalloc(&p, cap));
+  if (st.ptr) retired_.push_back(st.ptr);  // a peer may still hold a mapping: freed with the group
+  st.ptr = p;
+  st.capacity = cap;
+  RankSlot& me = ctl_->slot[rank_];
+  if (size_ > 1) HIP_CHECK(hipIpcGetMemHandle(&me.handle[slot], p));
+  me.ptr[slot] = (uint64_t)(uintptr_t)p;
+  me.capacity[slot] = cap;
+  me.gen[slot] += 1;
+  return p;
+}
+
+const void* ProcessGroupCCL::peerStage(int peer, int slot) {
+  if (peer == rank_) return stage_[slot].ptr;
+  const RankSlot& rs = ctl_->slot[peer];
+  PeerMap& pm = peers_[(size_t)peer];
+  if (pm.gen[slot] != rs.gen[slot]) {
+    if (pm.ipc[slot] && pm.ptr[slot]) (void)hipIpcCloseMemHandle(pm.ptr[slot]);
+    pm.ptr[slot] = nullptr;
+    pm.ipc[slot] = false;
+    if (rs.pid == (int64_t)getpid()) {
+      pm.ptr[slot] = (void*)(uintptr_t)rs.ptr[slot];  // a thread of this process: same address space
+    } else {
+      void* p = nullptr;
+      HIP_CHECK(hipIpcOpenMemHandle(&p, rs.handle[slot], hipIpcMemLazyEnablePeerAccess));
+      pm.ptr[slot] = p;
+      pm.ipc[slot] = true;
+    }
+    pm.gen[slot] = rs.gen[slot];
+  }
+  return pm.ptr[slot];
+}
+
+void ProcessGroupCCL::hostBarrier() {
+  const uint64_t epoch = ++barrier_epoch_;
+  ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
+  const auto deadline = std::chrono::steady_clock::now() +
+                        std::max(timeout_, std::chrono::milliseconds(30000));
+  for (int r = 0; r < size_; ++r) {
+    unsigned spins = 0;
+    while (ctl_->slot[r].arrive.load(std::memory_order_acquire) < epoch) {
+      if (ctl_->slot[r].failed.load(std::memory_order_acquire))
+        TORCH_CHECK(false, "ccl backend: rank ", r, " reported a failure; aborting the collective");
+      if (++spins < 2000) continue;
+      sched_yield();
+      if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
+        ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+        TORCH_CHECK(false, "ccl backend: timed out waiting for rank ", r, " at collective #", seq_);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// the engine: copy-in, host barrier, data-path kernels
+// ---------------------------------------------------------------------------------------------
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
+  int device = -1;
+  for (const auto& t : plan.inputs) if (t.defined()) { device = t.get_device(); break; }
+  if (device < 0) for (const auto& t : plan.outputs) if (t.defined()) { device = t.get_device(); break; }
+  if (device < 0) device = initialised_ ? device_ : 0;  // barrier without tensors
+  c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device));
+  ensureInit(device);
+  TORCH_CHECK((int)plan.table.size() <= kTableMax, "ccl backend: too many tensors in one collective");
+
+  auto cur_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_);
+  hipStream_t cur = cur_stream.stream();
+  hipStream_t s = same_stream_ ? cur : comm_stream_;
+  if (!same_stream_) {  // sync_streams of the reference (src/gpu/dpcpp_ccl.cpp:186-197)
+    HIP_CHECK(hipEventRecord(fork_event_, cur));
+    HIP_CHECK(hipStreamWaitEvent(comm_stream_, fork_event_, 0));
+  }
+
+  const int slot = (int)(seq_ & 1);
+  ++seq_;
+  if (verbose_) {
+    std::ostringstream os;
+    os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << seq_ << "]";
+    for (const auto& t : plan.inputs) os << " in" << t.sizes();
+    for (const auto& t : plan.outputs) os << " out" << t.sizes();
+    std::cout << os.str() << std::endl;
+  }
+
+  void* stage = ensureStage(slot, plan.stage_bytes);
+  RankSlot& me = ctl_->slot[rank_];
+  for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
+  if (plan.copy_in) plan.copy_in(stage, s);
+  // This rank's staging buffer must be complete before any peer reads it, and (two collectives
+  // later) every peer must be done reading before it is overwritten: one host barrier per
+  // collective plus the two alternating buffers give both.
+  HIP_CHECK(hipStreamSynchronize(s));
+  hostBarrier();
+
+  if (plan.exec) {
+    std::vector<const void*> peer((size_t)size_);
+    std::vector<const int64_t*> tables((size_t)size_);
+    for (int r = 0; r < size_; ++r) {
+      peer[(size_t)r] = peerStage(r, slot);
+      tables[(size_t)r] = ctl_->slot[r].table[slot];
+    }
+    plan.exec(peer, tables, s);
+  }
+
+  auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
+  work->device_ = device_;
+  HIP_CHECK(hipEventCreateWithFlags(&work->end_, hipEventDisableTiming));
+  HIP_CHECK(hipEventRecord(work->end_, s));
+  if (!same_stream_) {  // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
+    auto cs = c10::hip::getStreamFromExternalMasqueradingAsCUDA(comm_stream_, (c10::DeviceIndex)device_);
+    for (const auto* list : {&plan.inputs, &plan.outputs})
+      for (const auto& t : *list)
+        if (t.defined() && t.has_storage() && t.numel() > 0)
+          c10::hip::HIPCachingAllocatorMasqueradingAsCUDA::recordStreamMasqueradingAsCUDA(t.storage().data_ptr(), cs);
+  }
+  last_work_ = work;
+  return work;
+}
+
+void ProcessGroupCCL::checkDeviceTensors(const std::vector<at::Tensor>& tensors) const {
+  // checkSingleTensorHelper / checkSameType of the reference (src/utils.cpp:217-255) with the
+  // device test turned around: this backend takes GPU tensors only.
+  TORCH_CHECK(!tensors.empty(), "ccl backend: empty tensor list");
+  const auto& first = tensors[0];
+  for (const auto& t : tensors)
+    TORCH_CHECK(t.scalar_type() == first.scalar_type(), "Tensors are not equal in data type");
+  for (const auto& t : tensors) {
+    TORCH_CHECK(t.is_cuda(), "Tensors are not in same device type. Expect: cuda But got: ", t.device().type());
+    TORCH_CHECK(t.get_device() == first.get_device(), "ccl backend: tensors of one collective must share a device");
+    TORCH_CHECK(!t.is_sparse(), "ccl backend: sparse tensors are not supported");
+    TORCH_CHECK(t.is_contiguous(t.suggest_memory_format()), "input dense tensor has to be contiguous");
+  }
+}
+
+void ProcessGroupCCL::notImplemented(const char* what) const {
+  TORCH_CHECK(false, "oneccl_bindings_for_pytorch: ", what, " isn't implementd on backend [cuda].");
+}
+
+void ProcessGroupCCL::startCoalescing() { coalescing_ = true; }
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::endCoalescing() {
+  // Collectives issued between start and end have already been enqueued in order on the
+  // communication stream; the last Work covers them all.
+  coalescing_ = false;
+  if (last_work_) return last_work_;
+  return c10::make_intrusive<WorkCCL>(rank_, c10d::OpType::COALESCED, "endCoalescing",
+                                      std::vector<at::Tensor>{}, std::vector<at::Tensor>{}, blocking_wait_);
+}
+
+// ---------------------------------------------------------------------------------------------
+// collectives
+// ---------------------------------------------------------------------------------------------
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor>& tensors,
+                                                          const c10d::BroadcastOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::broadcast", std::vector<c10::IValue>({tensors}));
+  checkRank((int)opts.rootRank, size_);
+  TORCH_CHECK(tensors.size() == 1, "CCL process group does not support tensors count ", tensors.size());
+  checkDeviceTensors(tensors);
+  at::Tensor t = tensors[0];
+  const int root = (int)opts.rootRank;
+  const size_t total = nbytes(t);
+  c10::intrusive_ptr<c10d::Work> work;
+  size_t off = 0;
+  do {
+    const size_t len = std::min(total - off, kStageMax);
+    char* base = total ? (char*)t.data_ptr() + off : nullptr;
+    Plan p;
+    p.op = c10d::OpType::BROADCAST;
+    p.title = "broadcast";
+    p.inputs = {t};
+    p.outputs = {t};
+    p.stage_bytes = (rank_ == root) ? len : 0;
+    if (rank_ == root && len)
+      p.copy_in = [=](void* stage, hipStream_t s) {
+        HIP_CHECK(hipMemcpyAsync(stage, base, len, hipMemcpyDeviceToDevice, s));
+      };
+    if (rank_ != root && len)
+      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+        mccl_segment_t seg{peer[(size_t)root], base, len};
+        MCCL_CHECK(mccl_copy_segments(&seg, 1, s));
+      };
+    work = run(p);
+    off += len;
+  } while (off < total);
+  return work;
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor>& tensors,
+                                                          const c10d::AllreduceOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::allreduce", std::vector<c10::IValue>({tensors}));
+  TORCH_CHECK(tensors.size() == 1, "CCL process group does not support tensors count ", tensors.size());
+  checkDeviceTensors(tensors);
+  at::Tensor t = tensors[0];
+  const int dtype = dtypeCode(t.scalar_type());
+  const int op = opCode(opts.reduceOp, t.scalar_type());
+  const size_t es = t.element_size();
+  const size_t total = (size_t)t.numel();
+  const size_t chunk = kStageMax / es;
+  c10::intrusive_ptr<c10d::Work> work;
+  size_t off = 0;
+  do {
+    const size_t len = std::min(total - off, chunk);
+    char* base = total ? (char*)t.data_ptr() + off * es : nullptr;
+    Plan p;
+    p.op = c10d::OpType::ALLREDUCE;
+    p.title = "allreduce";
+    p.inputs = {t};
+    p.outputs = {t};
+    if (size_ > 1 && len) {  // world == 1: nothing to add (src/gpu/dpcpp_ccl.cpp:752-756)
+      p.stage_bytes = len * es;
+      p.copy_in = [=](void* stage, hipStream_t s) {
+        HIP_CHECK(hipMemcpyAsync(stage, base, len * es, hipMemcpyDeviceToDevice, s));
+      };
+      const int W = size_;
+      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+        MCCL_CHECK(mccl_reduce_n(peer.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
+      };
+    }
+    work = run(p);
+    off += len;
+  } while (off < total);
+  return work;
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce_coalesced(
+    std::vector<at::Tensor>& tensors, const c10d::AllreduceCoalescedOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::allreduce_coalesced", std::vector<c10::IValue>({tensors}));
+  checkDeviceTensors(tensors);
+  const int dtype = dtypeCode(tensors[0].scalar_type());
+  const int op = opCode(opts.reduceOp, tensors[0].scalar_type());
+  // one staging image: the tensors back to back, each on a 16-byte boundary
+  std::vector<size_t> offs(tensors.size());
+  size_t total = 0;
+  for (size_t i = 0; i < tensors.size(); ++i) {
+    offs[i] = total;
+    total += roundUp(nbytes(tensors[i]), 16);
+  }
+  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced allreduce larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::ALLREDUCE_COALESCED;
+  p.title = "allreduce_coalesced";
+  p.inputs = tensors;
+  p.outputs = tensors;
+  if (size_ > 1 && total) {
+    p.stage_bytes = total;
+    std::vector<at::Tensor> ts = tensors;
+    const int W = size_;
+    p.copy_in = [=](void* stage, hipStream_t s) {
+      std::vector<mccl_segment_t> segs;
+      for (size_t i = 0; i < ts.size(); ++i)
+        if (ts[i].numel()) segs.push_back({ts[i].data_ptr(), (char*)stage + offs[i], nbytes(ts[i])});
+      MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+      std::vector<const void*> in;
+      std::vector<void*> out;
+      std::vector<size_t> counts;
+      for (size_t i = 0; i < ts.size(); ++i) {
+        if (!ts[i].numel()) continue;
+        for (int k = 0; k < W; ++k) in.push_back((const char*)peer[(size_t)k] + offs[i]);
+        out.push_back(ts[i].data_ptr());
+        counts.push_back((size_t)ts[i].numel());
+      }
+      MCCL_CHECK(mccl_reduce_multi(in.data(), W, out.data(), counts.data(), (int)out.size(), dtype, op, s));
+    };
+  }
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& output, at::Tensor& input,
+                                                                const c10d::AllgatherOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::_allgather_base", std::vector<c10::IValue>({input}));
+  checkDeviceTensors({output, input});
+  TORCH_CHECK(input.numel() * size_ == output.numel(),
+              "output tensor size must be equal to world_size times input tensor size");
+  const size_t per_rank = nbytes(input);
+  c10::intrusive_ptr<c10d::Work> work;
+  size_t off = 0;
+  do {
+    const size_t len = std::min(per_rank - off, kStageMax);
+    char* in = per_rank ? (char*)input.data_ptr() + off : nullptr;
+    char* out = per_rank ? (char*)output.data_ptr() + off : nullptr;
+    Plan p;
+    p.op = c10d::OpType::_ALLGATHER_BASE;
+    p.title = "_allgather_base";
+    p.inputs = {input};
+    p.outputs = {output};
+    if (len) {
+      p.stage_bytes = len;
+      const int W = size_;
+      p.copy_in = [=](void* stage, hipStream_t s) {
+        HIP_CHECK(hipMemcpyAsync(stage, in, len, hipMemcpyDeviceToDevice, s));
+      };
+      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+        std::vector<mccl_segment_t> segs((size_t)W);
+        for (int r = 0; r < W; ++r) segs[(size_t)r] = {peer[(size_t)r], out + (size_t)r * per_rank, len};
+        MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
+      };
+    }
+    work = run(p);
+    off += len;
+  } while (off < per_rank);
+  return work;
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vector<at::Tensor>>& outputs,
+                                                          std::vector<at::Tensor>& inputs,
+                                                          const c10d::AllgatherOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::allgather", std::vector<c10::IValue>({inputs}));
+  TORCH_CHECK(inputs.size() == 1 && outputs.size() == 1,
+              "CCL process group does not support tensors count ", inputs.size());
+  TORCH_CHECK((int)outputs[0].size() == size_, "allgather: number of output tensors should equal to the world size");
+  std::vector<at::Tensor> all = outputs[0];
+  all.push_back(inputs[0]);
+  checkDeviceTensors(all);
+  at::Tensor input = inputs[0];
+  std::vector<at::Tensor> outs = outputs[0];
+  const size_t mine = nbytes(input);
+  TORCH_CHECK(mine <= kStageMax, "ccl backend: allgather (list) message larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::ALLGATHER;
+  p.title = "allgather";
+  p.inputs = {input};
+  p.outputs = outs;
+  p.stage_bytes = mine;
+  p.table = {(int64_t)mine};
+  const int W = size_;
+  if (mine)
+    p.copy_in = [=](void* stage, hipStream_t s) {
+      HIP_CHECK(hipMemcpyAsync(stage, input.data_ptr(), mine, hipMemcpyDeviceToDevice, s));
+    };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (int r = 0; r < W; ++r) {
+      const size_t b = (size_t)tables[(size_t)r][0];  // allgatherv: every rank announces its byte count
+      TORCH_CHECK(b == nbytes(outs[(size_t)r]), "allgather: output tensor ", r, " does not match the size rank ", r, " sends");
+      if (b) segs.push_back({peer[(size_t)r], outs[(size_t)r].data_ptr(), b});
+    }
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather_coalesced(std::vector<std::vector<at::Tensor>>&,
+                                                                    std::vector<at::Tensor>&,
+                                                                    const c10d::AllgatherOptions&) {
+  TORCH_CHECK(false, "ProcessGroupCCL does not support allgather_coalesced");
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather_into_tensor_coalesced(
+    std::vector<at::Tensor>& outputs, std::vector<at::Tensor>& inputs, const c10d::AllgatherOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::allgather_into_tensor_coalesced", std::vector<c10::IValue>({inputs}));
+  TORCH_CHECK(outputs.size() == inputs.size(), "allgather_into_tensor_coalesced: list sizes differ");
+  checkDeviceTensors(inputs);
+  std::vector<size_t> offs(inputs.size());
+  size_t total = 0;
+  for (size_t i = 0; i < inputs.size(); ++i) {
+    checkDeviceTensors({outputs[i], inputs[i]});
+    TORCH_CHECK(inputs[i].numel() * size_ == outputs[i].numel(),
+                "output tensor size must be equal to world_size times input tensor size");
+    offs[i] = total;
+    total += roundUp(nbytes(inputs[i]), 16);
+  }
+  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced allgather larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::ALLGATHER_COALESCED;
+  p.title = "allgather_into_tensor_coalesced";
+  p.inputs = inputs;
+  p.outputs = outputs;
+  p.stage_bytes = total;
+  std::vector<at::Tensor> ins = inputs, outs = outputs;
+  const int W = size_;
+  p.copy_in = [=](void* stage, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (size_t i = 0; i < ins.size(); ++i)
+      if (ins[i].numel()) segs.push_back({ins[i].data_ptr(), (char*)stage + offs[i], nbytes(ins[i])});
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (size_t i = 0; i < ins.size(); ++i) {
+      const size_t b = nbytes(ins[i]);
+      if (!b) continue;
+      for (int r = 0; r < W; ++r)
+        segs.push_back({(const char*)peer[(size_t)r] + offs[i], (char*)outs[i].data_ptr() + (size_t)r * b, b});
+    }
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor& output, at::Tensor& input,
+                                                                     const c10d::ReduceScatterOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::_reduce_scatter_base", std::vector<c10::IValue>({input}));
+  checkDeviceTensors({output, input});
+  TORCH_CHECK(input.numel() == output.numel() * size_,
+              "input tensor must be the same size as output size times world size");
+  const int dtype = dtypeCode(output.scalar_type());
+  const int op = opCode(opts.reduceOp, output.scalar_type());
+  const size_t es = output.element_size();
+  const size_t M = (size_t)output.numel();
+  const int W = size_;
+  // one window holds the same sub-range [m0, m0+len) of all W shards, back to back
+  const size_t chunk = std::max<size_t>(1, kStageMax / es / (size_t)W);
+  c10::intrusive_ptr<c10d::Work> work;
+  size_t m0 = 0;
+  do {
+    const size_t len = std::min(M - m0, chunk);
+    Plan p;
+    p.op = c10d::OpType::_REDUCE_SCATTER_BASE;
+    p.title = "_reduce_scatter_base";
+    p.inputs = {input};
+    p.outputs = {output};
+    if (len) {
+      p.stage_bytes = len * es * (size_t)W;
+      char* in = (char*)input.data_ptr();
+      char* out = (char*)output.data_ptr() + m0 * es;
+      const int me = rank_;
+      p.copy_in = [=](void* stage, hipStream_t s) {
+        if (len == M) {
+          HIP_CHECK(hipMemcpyAsync(stage, in, M * es * (size_t)W, hipMemcpyDeviceToDevice, s));
+        } else {
+          std::vector<mccl_segment_t> segs((size_t)W);
+          for (int k = 0; k < W; ++k)
+            segs[(size_t)k] = {in + ((size_t)k * M + m0) * es, (char*)stage + (size_t)k * len * es, len * es};
+          MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
+        }
+      };
+      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+        void* o = out;
+        MCCL_CHECK(mccl_reduce_scatter_n(peer.data(), W, &o, len, me, 1, dtype, op, s));
+      };
+    }
+    work = run(p);
+    m0 += len;
+  } while (m0 < M);
+  return work;
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::Tensor>& outputs,
+                                                               std::vector<std::vector<at::Tensor>>& inputs,
+                                                               const c10d::ReduceScatterOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::reduce_scatter", std::vector<c10::IValue>({outputs}));
+  TORCH_CHECK(outputs.size() == 1 && inputs.size() == 1,
+              "CCL process group does not support tensors count ", outputs.size());
+  TORCH_CHECK((int)inputs[0].size() == size_, "reduce_scatter: number of input tensors should equal to the world size");
+  std::vector<at::Tensor> all = inputs[0];
+  all.push_back(outputs[0]);
+  checkDeviceTensors(all);
+  at::Tensor out = outputs[0];
+  std::vector<at::Tensor> ins = inputs[0];
+  const int dtype = dtypeCode(out.scalar_type());
+  const int op = opCode(opts.reduceOp, out.scalar_type());
+  const int W = size_;
+  const int me = rank_;
+  // Slot d of every rank's list is reduced into rank d's output; slots may differ in size
+  // (the reference degrades to W rooted reduces then, src/gpu/dpcpp_ccl.cpp:952-964).  The
+  // staging image is the list packed back to back; the table announces offset and size per slot.
+  Plan p;
+  p.op = c10d::OpType::REDUCE_SCATTER;
+  p.title = "reduce_scatter";
+  p.inputs = ins;
+  p.outputs = {out};
+  p.table.resize((size_t)(2 * W));
+  size_t total = 0;
+  std::vector<size_t> offs((size_t)W);
+  for (int d = 0; d < W; ++d) {
+    offs[(size_t)d] = total;
+    p.table[(size_t)d] = (int64_t)total;
+    p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
+    total += roundUp(nbytes(ins[(size_t)d]), 16);
+  }
+  TORCH_CHECK(total <= kStageMax, "ccl backend: reduce_scatter (list) larger than the staging window");
+  p.stage_bytes = total;
+  p.copy_in = [=](void* stage, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (int d = 0; d < W; ++d)
+      if (ins[(size_t)d].numel())
+        segs.push_back({ins[(size_t)d].data_ptr(), (char*)stage + offs[(size_t)d], nbytes(ins[(size_t)d])});
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    std::vector<const void*> in((size_t)W);
+    for (int k = 0; k < W; ++k) {
+      TORCH_CHECK((size_t)tables[(size_t)k][W + me] == nbytes(out),
+                  "reduce_scatter: rank ", k, "'s input for rank ", me, " does not match the output size");
+      in[(size_t)k] = (const char*)peer[(size_t)k] + tables[(size_t)k][me];
+    }
+    if (out.numel())
+      MCCL_CHECK(mccl_reduce_n(in.data(), W, out.data_ptr(), (size_t)out.numel(), dtype, op, MCCL_VARIANT_AUTO, s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter_tensor_coalesced(
+    std::vector<at::Tensor>& outputs, std::vector<at::Tensor>& inputs, const c10d::ReduceScatterOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::reduce_scatter_tensor_coalesced", std::vector<c10::IValue>({inputs}));
+  TORCH_CHECK(outputs.size() == inputs.size(), "reduce_scatter_tensor_coalesced: list sizes differ");
+  checkDeviceTensors(inputs);
+  checkDeviceTensors(outputs);
+  TORCH_CHECK(inputs[0].scalar_type() == outputs[0].scalar_type(), "Tensors are not equal in data type");
+  const int dtype = dtypeCode(outputs[0].scalar_type());
+  const int op = opCode(opts.reduceOp, outputs[0].scalar_type());
+  std::vector<size_t> offs(inputs.size());
+  size_t total = 0;
+  for (size_t i = 0; i < inputs.size(); ++i) {
+    TORCH_CHECK(inputs[i].numel() == outputs[i].numel() * size_,
+                "input tensor must be the same size as output size times world size");
+    offs[i] = total;
+    total += roundUp(nbytes(inputs[i]), 16);
+  }
+  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced reduce_scatter larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::COALESCED;
+  p.title = "reduce_scatter_tensor_coalesced";
+  p.inputs = inputs;
+  p.outputs = outputs;
+  p.stage_bytes = total;
+  std::vector<at::Tensor> ins = inputs, outs = outputs;
+  const int W = size_;
+  const int me = rank_;
+  p.copy_in = [=](void* stage, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (size_t i = 0; i < ins.size(); ++i)
+      if (ins[i].numel()) segs.push_back({ins[i].data_ptr(), (char*)stage + offs[i], nbytes(ins[i])});
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+    std::vector<const void*> in;
+    std::vector<void*> out;
+    std::vector<size_t> counts;
+    for (size_t i = 0; i < ins.size(); ++i) {
+      if (!outs[i].numel()) continue;
+      const size_t shard = nbytes(outs[i]);
+      for (int k = 0; k < W; ++k) in.push_back((const char*)peer[(size_t)k] + offs[i] + (size_t)me * shard);
+      out.push_back(outs[i].data_ptr());
+      counts.push_back((size_t)outs[i].numel());
+    }
+    MCCL_CHECK(mccl_reduce_multi(in.data(), W, out.data(), counts.data(), (int)out.size(), dtype, op, s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output, at::Tensor& input,
+                                                              std::vector<int64_t>& outputSplitSizes,
+                                                              std::vector<int64_t>& inputSplitSizes,
+                                                              const c10d::AllToAllOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::alltoall_base", std::vector<c10::IValue>({input}));
+  checkDeviceTensors({output, input});
+  const int W = size_;
+  const int me = rank_;
+  const size_t es = input.element_size();
+  std::vector<size_t> send((size_t)W), recv((size_t)W);
+  if (outputSplitSizes.empty() && inputSplitSizes.empty()) {
+    // src/gpu/dpcpp_ccl.cpp:1384-1390
+    TORCH_CHECK(output.numel() == input.numel() && output.scalar_type() == input.scalar_type(),
+                "alltoall_base: tensors are not equal in size or data type");
+    TORCH_CHECK(output.size(0) % W == 0, "alltoall_base: tensor's dim 0 does not divide equally across group size");
+    const size_t c = (size_t)output.numel() / (size_t)W * es;
+    for (int i = 0; i < W; ++i) send[(size_t)i] = recv[(size_t)i] = c;
+  } else {
+    // count arithmetic of src/gpu/dpcpp_ccl.cpp:1431-1445
+    c10d::checkSplitSizes(inputSplitSizes, input, W);
+    c10d::checkSplitSizes(outputSplitSizes, output, W);
+    const bool in_equal = inputSplitSizes.empty(), out_equal = outputSplitSizes.empty();
+    size_t in_len = (size_t)input.numel(), out_len = (size_t)output.numel();
+    if (in_len) in_len /= (in_equal ? (size_t)W : (size_t)input.size(0));
+    if (out_len) out_len /= (out_equal ? (size_t)W : (size_t)output.size(0));
+    for (int i = 0; i < W; ++i) {
+      send[(size_t)i] = (in_equal ? in_len : (size_t)inputSplitSizes[(size_t)i] * in_len) * es;
+      recv[(size_t)i] = (out_equal ? out_len : (size_t)outputSplitSizes[(size_t)i] * out_len) * es;
+    }
+  }
+  const size_t mine = nbytes(input);
+  TORCH_CHECK(mine <= kStageMax, "ccl backend: alltoall message larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::ALLTOALL_BASE;
+  p.title = "alltoall_base";
+  p.inputs = {input};
+  p.outputs = {output};
+  p.stage_bytes = mine;
+  p.table.resize((size_t)(2 * W));
+  size_t displ = 0;
+  for (int d = 0; d < W; ++d) {  // displacements = exclusive prefix sums of the send counts
+    p.table[(size_t)d] = (int64_t)displ;
+    p.table[(size_t)(W + d)] = (int64_t)send[(size_t)d];
+    displ += send[(size_t)d];
+  }
+  if (mine)
+    p.copy_in = [=](void* stage, hipStream_t s) {
+      HIP_CHECK(hipMemcpyAsync(stage, input.data_ptr(), mine, hipMemcpyDeviceToDevice, s));
+    };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    std::vector<size_t> sd((size_t)W);
+    for (int r = 0; r < W; ++r) {
+      TORCH_CHECK((size_t)tables[(size_t)r][W + me] == recv[(size_t)r],
+                  "alltoall_base: rank ", r, " sends ", tables[(size_t)r][W + me], " bytes to rank ", me,
+                  " which expects ", recv[(size_t)r]);
+      sd[(size_t)r] = (size_t)tables[(size_t)r][me];
+    }
+    MCCL_CHECK(mccl_alltoallv_pull(peer.data(), W, output.data_ptr(), sd.data(), recv.data(), s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>& outputs,
+                                                         std::vector<at::Tensor>& inputs,
+                                                         const c10d::AllToAllOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::alltoall", std::vector<c10::IValue>({inputs}));
+  TORCH_CHECK((int)inputs.size() == size_ && (int)outputs.size() == size_,
+              "alltoall: number of input and output tensors should equal to the world size");
+  std::vector<at::Tensor> all = inputs;
+  all.insert(all.end(), outputs.begin(), outputs.end());
+  checkDeviceTensors(all);
+  const int W = size_;
+  const int me = rank_;
+  std::vector<at::Tensor> ins = inputs, outs = outputs;
+  // The pack of the reference (src/gpu/dpcpp_ccl.cpp:1505-1515) is the copy-in itself, and the
+  // pull writes straight into the output tensors, which is its unpack (:1528-1538).
+  Plan p;
+  p.op = c10d::OpType::ALLTOALL;
+  p.title = "alltoall";
+  p.inputs = ins;
+  p.outputs = outs;
+  p.table.resize((size_t)(2 * W));
+  std::vector<size_t> offs((size_t)W);
+  size_t total = 0;
+  for (int d = 0; d < W; ++d) {
+    offs[(size_t)d] = total;
+    p.table[(size_t)d] = (int64_t)total;
+    p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
+    total += roundUp(nbytes(ins[(size_t)d]), 16);
+  }
+  TORCH_CHECK(total <= kStageMax, "ccl backend: alltoall (list) larger than the staging window");
+  p.stage_bytes = total;
+  p.copy_in = [=](void* stage, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (int d = 0; d < W; ++d)
+      if (ins[(size_t)d].numel())
+        segs.push_back({ins[(size_t)d].data_ptr(), (char*)stage + offs[(size_t)d], nbytes(ins[(size_t)d])});
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    std::vector<mccl_segment_t> segs;
+    for (int r = 0; r < W; ++r) {
+      const size_t b = (size_t)tables[(size_t)r][W + me];
+      TORCH_CHECK(b == nbytes(outs[(size_t)r]), "alltoall: output tensor ", r, " does not match what rank ", r, " sends");
+      if (b) segs.push_back({(const char*)peer[(size_t)r] + tables[(size_t)r][me], outs[(size_t)r].data_ptr(), b});
+    }
+    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  return run(p);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::barrier(const c10d::BarrierOptions& /*opts*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::barrier", std::vector<c10::IValue>{});
+  Plan p;
+  p.op = c10d::OpType::BARRIER;
+  p.title = "barrier";
+  auto work = run(p);
+  // a barrier returns once every rank has arrived: nothing is pending on the stream
+  return work;
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce(std::vector<at::Tensor>&, const c10d::ReduceOptions&) {
+  notImplemented("reduce");
+}
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<at::Tensor>>&, std::vector<at::Tensor>&,
+                                                       const c10d::GatherOptions&) {
+  notImplemented("gather");
+}
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&, std::vector<std::vector<at::Tensor>>&,
+                                                        const c10d::ScatterOptions&) {
+  notImplemented("scatter");
+}
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::send(std::vector<at::Tensor>&, int, int) { notImplemented("send"); }
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>&, int, int) { notImplemented("recv"); }
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recvAnysource(std::vector<at::Tensor>&, int) {
+  TORCH_CHECK(false, "ProcessGroupCCL does not support recvAnysource");
+}
+
+}  // namespace mccl_pg

@@ -1,0 +1,184 @@
+// c10d backend "ccl" for ROCm tensors on one MI355X: the host-side mirror of the reference's
+// ProcessGroupCCL (src/ProcessGroupCCL.hpp:111-310) over the C ABI of include/mccl.h.
+//
+// Single-GPU mode: every rank of the group (a process, or a thread of one process) uses
+// device 0.  Each rank owns two staging buffers in HBM.  A collective
+//   1. copies (or packs) the caller's input into the rank's staging buffer   [device copy]
+//   2. waits, on the host, until every rank has finished step 1              [barrier]
+//   3. runs the local-reduce / pull kernel over the N ranks' staging buffers,
+//      writing straight into the caller's output tensor                      [the hot path]
+// which is the structure of the reference's IPC allreduce (copy-in, cross-rank barrier, sum of
+// the N peer buffers: src/gpu/allreduce_small.h:166-361).  Peers' staging buffers are reached
+// through hipIpcOpenMemHandle (other processes) or directly (threads of the same process); the
+// handles, a host barrier and small per-collective tables live in a POSIX shared-memory control
+// block whose name is published through the c10d Store (the role of
+// src/ccl_comm_collector.cpp:10-45 and src/gpu/allreduce.h:1208-1248).
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <torch/csrc/distributed/c10d/Backend.hpp>
+#include <torch/csrc/distributed/c10d/Store.hpp>
+#include <torch/csrc/distributed/c10d/Types.hpp>
+#include <torch/csrc/distributed/c10d/Utils.hpp>
+#include <torch/csrc/distributed/c10d/Work.hpp>
+
+#include <chrono>
+#include <functional>
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace mccl_pg {
+
+struct Control;  // shared-memory control block (process_group_ccl.cpp)
+
+class ProcessGroupCCL : public c10d::Backend {
+ public:
+  // Stream-ordered Work (the contract of XPUWorkCCL, src/gpu/dpcpp_ccl.cpp:382-472): the op is
+  // complete when `end_` has fired on the communication stream; wait() makes the caller's current
+  // stream wait for it, or blocks the host when CCL_BLOCKING_WAIT=1.
+  class WorkCCL : public c10d::Work {
+   public:
+    WorkCCL(int rank, c10d::OpType op, const char* title, std::vector<at::Tensor> inputs,
+            std::vector<at::Tensor> outputs, bool blocking_wait);
+    ~WorkCCL() override;
+    bool isCompleted() override;
+    bool isSuccess() const override;
+    bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
+    void synchronize() override;
+    std::vector<at::Tensor> result() override;
+    c10::intrusive_ptr<c10::ivalue::Future> getFuture() override;
+
+   private:
+    friend class ProcessGroupCCL;
+    hipEvent_t end_ = nullptr;
+    int device_ = 0;
+    bool blocking_wait_ = false;
+    std::vector<at::Tensor> inputs_;   // held until the Work dies (ownership rule of the reference)
+    std::vector<at::Tensor> outputs_;
+    c10::intrusive_ptr<c10::ivalue::Future> future_;
+  };
+
+  static constexpr int64_t OP_TIMEOUT_MILLIS = 10 * 1000;  // src/ProcessGroupCCL.cpp:876
+
+  ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
+                  std::chrono::milliseconds timeout);
+  ~ProcessGroupCCL() override;
+
+  static c10::intrusive_ptr<c10d::Backend> create(const c10::intrusive_ptr<c10d::Store>& store,
+                                                  int rank, int size,
+                                                  std::chrono::milliseconds timeout);
+
+  const std::string getBackendName() const override { return "ccl"; }
+  bool supportsCoalescing() const override { return true; }
+  void startCoalescing() override;
+  c10::intrusive_ptr<c10d::Work> endCoalescing() override;
+  void setTimeout(std::chrono::milliseconds t) override { timeout_ = t; }
+  void setSequenceNumberForGroup() override {}
+  uint64_t getSequenceNumberForGroup() override { return seq_; }
+
+  c10::intrusive_ptr<c10d::Work> broadcast(std::vector<at::Tensor>& tensors,
+                                           const c10d::BroadcastOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> allreduce(std::vector<at::Tensor>& tensors,
+                                           const c10d::AllreduceOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> allreduce_coalesced(
+      std::vector<at::Tensor>& tensors, const c10d::AllreduceCoalescedOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> allgather(std::vector<std::vector<at::Tensor>>& outputs,
+                                           std::vector<at::Tensor>& inputs,
+                                           const c10d::AllgatherOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> _allgather_base(at::Tensor& output, at::Tensor& input,
+                                                 const c10d::AllgatherOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> allgather_coalesced(
+      std::vector<std::vector<at::Tensor>>& outputs, std::vector<at::Tensor>& inputs,
+      const c10d::AllgatherOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> allgather_into_tensor_coalesced(
+      std::vector<at::Tensor>& outputs, std::vector<at::Tensor>& inputs,
+      const c10d::AllgatherOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> reduce_scatter(std::vector<at::Tensor>& outputs,
+                                                std::vector<std::vector<at::Tensor>>& inputs,
+                                                const c10d::ReduceScatterOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> _reduce_scatter_base(at::Tensor& output, at::Tensor& input,
+                                                      const c10d::ReduceScatterOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> reduce_scatter_tensor_coalesced(
+      std::vector<at::Tensor>& outputs, std::vector<at::Tensor>& inputs,
+      const c10d::ReduceScatterOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> alltoall_base(at::Tensor& output, at::Tensor& input,
+                                               std::vector<int64_t>& outputSplitSizes,
+                                               std::vector<int64_t>& inputSplitSizes,
+                                               const c10d::AllToAllOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> alltoall(std::vector<at::Tensor>& outputs,
+                                          std::vector<at::Tensor>& inputs,
+                                          const c10d::AllToAllOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> barrier(const c10d::BarrierOptions& opts) override;
+
+  // Not on the path this backend covers; they fail like DispatchStub::fail does
+  // (src/dispatch_stub.h:288-290).
+  c10::intrusive_ptr<c10d::Work> reduce(std::vector<at::Tensor>&, const c10d::ReduceOptions&) override;
+  c10::intrusive_ptr<c10d::Work> gather(std::vector<std::vector<at::Tensor>>&, std::vector<at::Tensor>&,
+                                        const c10d::GatherOptions&) override;
+  c10::intrusive_ptr<c10d::Work> scatter(std::vector<at::Tensor>&, std::vector<std::vector<at::Tensor>>&,
+                                         const c10d::ScatterOptions&) override;
+  c10::intrusive_ptr<c10d::Work> send(std::vector<at::Tensor>&, int, int) override;
+  c10::intrusive_ptr<c10d::Work> recv(std::vector<at::Tensor>&, int, int) override;
+  c10::intrusive_ptr<c10d::Work> recvAnysource(std::vector<at::Tensor>&, int) override;
+
+ private:
+  // What one collective needs from the engine.
+  struct Plan {
+    c10d::OpType op = c10d::OpType::UNKNOWN;
+    const char* title = "";
+    std::vector<at::Tensor> inputs;
+    std::vector<at::Tensor> outputs;
+    size_t stage_bytes = 0;                 // bytes this rank puts into its staging buffer
+    std::vector<int64_t> table;             // per-collective scalars published to the peers
+    // enqueue the copy-in on `s`; `stage` is this rank's staging buffer
+    std::function<void(void* stage, hipStream_t s)> copy_in;
+    // enqueue the data-path kernels on `s`; peer[r] is rank r's staging buffer,
+    // tables[r] the scalars rank r published
+    std::function<void(const std::vector<const void*>& peer,
+                       const std::vector<const int64_t*>& tables, hipStream_t s)> exec;
+  };
+
+  c10::intrusive_ptr<c10d::Work> run(Plan& plan);
+  void ensureInit(int device);
+  void* ensureStage(int slot, size_t bytes);
+  void hostBarrier();
+  const void* peerStage(int peer, int slot);
+  void checkDeviceTensors(const std::vector<at::Tensor>& tensors) const;
+  [[noreturn]] void notImplemented(const char* what) const;
+
+  c10::intrusive_ptr<c10d::Store> store_;
+  std::chrono::milliseconds timeout_;
+  bool blocking_wait_ = false;  // CCL_BLOCKING_WAIT
+  bool same_stream_ = false;    // CCL_SAME_STREAM
+  bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
+  bool coalescing_ = false;
+  c10::intrusive_ptr<WorkCCL> last_work_;
+
+  bool initialised_ = false;
+  int device_ = 0;
+  hipStream_t comm_stream_ = nullptr;
+  hipEvent_t fork_event_ = nullptr;
+  uint64_t seq_ = 0;
+  uint64_t barrier_epoch_ = 0;
+
+  Control* ctl_ = nullptr;
+  size_t ctl_bytes_ = 0;
+  std::string shm_name_;
+
+  struct Stage {
+    void* ptr = nullptr;
+    size_t capacity = 0;
+  };
+  Stage stage_[2];
+  std::vector<void*> retired_;  // outgrown staging buffers, freed with the group
+
+  struct PeerMap {
+    void* ptr[2] = {nullptr, nullptr};
+    uint64_t gen[2] = {0, 0};
+    bool ipc[2] = {false, false};
+  };
+  std::vector<PeerMap> peers_;
+};
+
+}  // namespace mccl_pg
