@@ -224,6 +224,20 @@ def large_message_case(pg, rank, world):
     assert float(t.min()) == s
 
 
+def missing_rank_case(pg, rank, world):
+    """Rank 1 never joins the second collective: the others must get an error, not hang."""
+    t = torch.ones(16, device=DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    if rank == 1:
+        return
+    try:
+        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        raise AssertionError("collective with a missing rank returned")
+    except RuntimeError as e:
+        assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
+                or "rank 1 left the group" in str(e)), str(e)
+
+
 def run_rank(rank, world, store_path, mode):
     torch.cuda.set_device(0)
     import torch_ccl_amd  # noqa: F401  registers the backend
@@ -244,6 +258,8 @@ def run_rank(rank, world, store_path, mode):
         oracle_cases(pg, rank, world)
     elif mode == "large":
         large_message_case(pg, rank, world)
+    elif mode == "missing":
+        missing_rank_case(pg, rank, world)
     else:
         raise ValueError(mode)
     torch.cuda.synchronize()

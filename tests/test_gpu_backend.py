@@ -49,3 +49,45 @@ def test_world_size_one_is_a_no_op():
         out = torch.empty(2, device="cuda:0")
         pg._allgather_base(out, t).wait()
         assert torch.equal(out.cpu(), t.cpu())
+
+
+def test_missing_rank_raises_instead_of_hanging(monkeypatch):
+    """Failure handling forced from the host: a rank skips a collective; the host barrier of the
+    others gives up after the (shortened) limit and raises.  No kernel waits on the GPU."""
+    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    _spawn(3, "missing")
+
+
+def test_thread_ranks_in_one_process():
+    """Ranks as threads of one process (same address space: staging buffers are shared by raw
+    pointer instead of an IPC handle), rendezvous through a HashStore."""
+    import threading
+    import torch.distributed as dist
+    import torch_ccl_amd  # noqa: F401
+    world = 4
+    store = dist.HashStore()
+    errors = []
+
+    def body(rank):
+        try:
+            pg = dist.ProcessGroupCCL(store, rank, world)
+            t = torch.full((100000,), float(rank + 1), device="cuda:0")
+            pg.allreduce([t]).wait()
+            torch.cuda.synchronize()
+            assert float(t[0]) == world * (world + 1) / 2 and float(t[-1]) == world * (world + 1) / 2
+            out = torch.empty(world * 5, device="cuda:0")
+            pg._allgather_base(out, torch.full((5,), float(rank), device="cuda:0")).wait()
+            torch.cuda.synchronize()
+            assert out.cpu().tolist() == [float(r) for r in range(world) for _ in range(5)]
+            pg.barrier().wait()
+            del pg
+        except Exception as e:  # noqa: BLE001
+            errors.append((rank, repr(e)))
+
+    threads = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+    assert not errors, errors
+    assert not any(th.is_alive() for th in threads)

@@ -280,3 +280,34 @@ def test_reduce_multi_random(mccl):
     for b, c in enumerate(counts):
         if c:
             assert_bits_equal(bits(outs[b]), oracle_reduce_bits(ins_cpu[b]), "bucket %d" % b)
+
+
+# ---- HIP graph capture: the entry points allocate nothing and never synchronise ----
+
+def test_reduce_and_copy_replay_from_a_hip_graph(mccl):
+    """Capture one reduction and one allgather into a graph; replay it several times with eager
+    work and synchronisations in between; every replay must equal the eager result."""
+    n, count = 8, 16 * 8192
+    ins = [rank_buffer(count, torch.bfloat16, r).to(DEV) for r in range(n)]
+    out = torch.zeros(count, dtype=torch.bfloat16, device=DEV)
+    gathered = torch.zeros(n * count, dtype=torch.bfloat16, device=DEV)
+    mccl.reduce_n(ins, out=out)          # warm-up outside the capture (device facts are cached)
+    mccl.allgather_n(ins, gathered)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        mccl.reduce_n(ins, out=out)
+        mccl.allgather_n(ins, gathered)
+    for it in range(4):
+        for r in range(n):               # eager work between replays: new inputs every time
+            ins[r].copy_(rank_buffer(count, torch.bfloat16, r, seed=500 + it))
+        out.zero_()
+        gathered.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = mccl.reduce_n(ins)        # eager result on the same inputs
+        torch.cuda.synchronize()
+        assert_bits_equal(bits(out), bits(want), "graph replay %d" % it)
+        assert_bits_equal(bits(out), oracle_reduce_bits([t.cpu() for t in ins]), "graph replay %d vs oracle" % it)
+        assert_bits_equal(bits(gathered), np.concatenate([bits(t) for t in ins]), "graph allgather %d" % it)

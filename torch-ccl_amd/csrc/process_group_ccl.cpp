@@ -113,6 +113,7 @@ size_t roundUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
 struct alignas(128) RankSlot {
   std::atomic<uint64_t> arrive;  // host barrier: epoch this rank has reached
   std::atomic<uint64_t> failed;  // non-zero once the rank gave up; peers stop waiting
+  std::atomic<uint64_t> departed;  // non-zero once the rank's group object is being destroyed
   int64_t pid;
   // per staging slot; written by the owner before it arrives at the barrier of the collective
   // that uses the slot, read by the peers after that barrier
@@ -214,12 +215,17 @@ ProcessGroupCCL::~ProcessGroupCCL() {
   // finished its kernels, so a timeout here is harmless.
   (void)hipSetDevice(device_);
   if (comm_stream_) (void)hipStreamSynchronize(comm_stream_);
-  try {
-    auto saved = timeout_;
-    timeout_ = std::chrono::milliseconds(2000);
-    hostBarrier();
-    timeout_ = saved;
-  } catch (...) {
+  // Leaving never advances the barrier epoch (a rank that leaves early must not satisfy its
+  // peers' next barrier); it raises a flag instead.  A peer is done with this rank's buffers
+  // once it has left too or has arrived at a later collective.
+  ctl_->slot[rank_].departed.store(1, std::memory_order_release);
+  const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(2000);
+  for (int r = 0; r < size_; ++r) {
+    if (r == rank_) continue;
+    while (!ctl_->slot[r].departed.load(std::memory_order_acquire) &&
+           ctl_->slot[r].arrive.load(std::memory_order_acquire) <= barrier_epoch_ &&
+           std::chrono::steady_clock::now() < deadline)
+      sched_yield();
   }
   (void)hipDeviceSynchronize();
   for (auto& pm : peers_)
@@ -328,13 +334,23 @@ const void* ProcessGroupCCL::peerStage(int peer, int slot) {
 void ProcessGroupCCL::hostBarrier() {
   const uint64_t epoch = ++barrier_epoch_;
   ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
-  const auto deadline = std::chrono::steady_clock::now() +
-                        std::max(timeout_, std::chrono::milliseconds(30000));
+  // Floor of 30 s under short user timeouts (ranks start at different speeds);
+  // MCCL_BARRIER_TIMEOUT_MS overrides it, e.g. to exercise the failure path quickly.
+  std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(30000));
+  if (const char* v = std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
+    const long ms = std::atol(v);
+    if (ms > 0) limit = std::chrono::milliseconds(ms);
+  }
+  const auto deadline = std::chrono::steady_clock::now() + limit;
   for (int r = 0; r < size_; ++r) {
     unsigned spins = 0;
     while (ctl_->slot[r].arrive.load(std::memory_order_acquire) < epoch) {
       if (ctl_->slot[r].failed.load(std::memory_order_acquire))
         TORCH_CHECK(false, "ccl backend: rank ", r, " reported a failure; aborting the collective");
+      if (ctl_->slot[r].departed.load(std::memory_order_acquire)) {
+        ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+        TORCH_CHECK(false, "ccl backend: rank ", r, " left the group before collective #", seq_);
+      }
       if (++spins < 2000) continue;
       sched_yield();
       if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
