@@ -84,13 +84,74 @@ def cpu_baseline(torch, host_inputs, n, count):
             "ms_per_step": round(dt * 1e3, 3)}, out
 
 
+def _gloo_rank(rank, world, store_path, backend, cases, out_path):
+    """One host process of the N-process CPU baseline: same op, same (seed, rank) data, CPU tensors."""
+    os.dup2(2, 1)  # keep the parent's stdout clean for the one JSON line (gloo prints connection notes)
+    import torch
+    import torch.distributed as dist
+    torch.set_num_threads(max(1, len(os.sched_getaffinity(0)) // world))
+    store = dist.FileStore(store_path, world)
+    dist.init_process_group(backend, store=store, rank=rank, world_size=world)
+    res = {}
+    for name, count, dtype_name, std, warm, iters in cases:
+        dtype = getattr(torch, dtype_name)
+        g = rank_generator(torch, SEED, rank)
+        x = (torch.randn(count, generator=g, dtype=torch.float32) * std).to(dtype)
+        t = x.clone()
+        for _ in range(warm):
+            t.copy_(x)
+            dist.all_reduce(t)
+        ts = []
+        for _ in range(iters):
+            t.copy_(x)
+            dist.barrier()
+            t0 = time.perf_counter()
+            dist.all_reduce(t)
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters,
+                     "checksum": float(t.float().sum())}
+    if rank == 0:
+        with open(out_path, "w") as f:
+            json.dump(res, f)
+    dist.destroy_process_group()
+
+
+def gloo_baseline(world=8):
+    """N host processes running the same allreduce through a CPU c10d backend: the reference's
+    "ccl" backend when its wheel is installed, else gloo (the stand-in the reference's own CPU
+    harness uses, tests/DeepSpeed_test/testccl_cpu.py:20).  Reported baseline only."""
+    import importlib.util
+    import tempfile
+    import torch
+    import torch.multiprocessing as mp
+    backend = "ccl" if importlib.util.find_spec("oneccl_bindings_for_pytorch") else "gloo"
+    cases = [("c2_256KiB_bf16", 16 * 8192, "bfloat16", 0.02, 20, 300),
+             ("c3_64MiB_bf16", 4096 * 8192, "bfloat16", 0.02, 3, 12)]
+    with tempfile.TemporaryDirectory() as d:
+        out_path = os.path.join(d, "res.json")
+        mp.spawn(_gloo_rank, args=(world, os.path.join(d, "store"), backend, cases, out_path),
+                 nprocs=world, join=True)
+        with open(out_path) as f:
+            res = json.load(f)
+    out = {"backend": backend, "processes": world, "host_cores": len(os.sched_getaffinity(0)),
+           "os_cpu_count": os.cpu_count(), "torch": torch.__version__,
+           "threads_per_process": max(1, len(os.sched_getaffinity(0)) // world), "pinning": "none"}
+    for name, count, dtype_name, std, warm, iters in cases:
+        r = res[name]
+        nbytes = count * 2
+        out[name] = {"p50_us": round(r["p50_us"], 1), "p99_us": round(r["p99_us"], 1), "iters": r["iters"],
+                     "GBps_effective": round((world + 1) * nbytes / r["p50_us"] / 1e3, 3)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,variants,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,variants,gloo,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -101,7 +162,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,variants".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,variants,gloo".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import torch
@@ -288,6 +349,15 @@ def main():
         log("CPU:", json.dumps(cb))
     else:
         result["cpu_baseline"] = None
+
+    # ---------------- N-process CPU c10d baseline (gloo unless the reference's wheel exists) ----------------
+    if "gloo" in extras and not args.no_cpu:
+        try:
+            result["cpu_c10d_baseline"] = gloo_baseline(N)
+            log("CPU c10d:", json.dumps(result["cpu_c10d_baseline"]))
+        except Exception as e:  # reported baseline only: never fails the benchmark
+            result["cpu_c10d_baseline"] = {"error": repr(e)[:300]}
+            log("CPU c10d baseline failed:", repr(e)[:300])
 
     print(json.dumps(result), flush=True)
 
