@@ -151,7 +151,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,variants,gloo,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,moe,variants,gloo,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -162,7 +162,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,variants,gloo".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,moe,variants,gloo".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import torch
@@ -326,6 +326,56 @@ def main():
                                       "split_rows_rank0": S5[0].tolist()}
         log("C5:", json.dumps(result["c5_alltoallv_moe"]))
         del a2a_in, a2a_out
+
+    # ---------------- the steps either side of C5: token permute fused into the dispatch, weighted combine ----------------
+    if "moe" in extras:
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from moe_helpers import combine_tables, route
+        tokens, hidden, topk, n_exp = 4096, 7168, 8, 256
+        S6, send_tok, _ = route(N, tokens, n_exp, topk, seed=SEED)
+        src_rank, src_row = combine_tables(N, tokens, topk, S6, send_tok)
+        hid = []
+        for r in range(N):
+            gd = rank_generator(torch, SEED, r, dev)
+            hid.append(torch.randn(tokens, hidden, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16))
+        idx = [t.to(dev) for t in send_tok]
+        recv = [torch.empty(int(S6[:, d].sum()), hidden, dtype=torch.bfloat16, device=dev) for d in range(N)]
+        recv2 = [torch.empty_like(t) for t in recv]
+        sends = [torch.empty(tokens * topk, hidden, dtype=torch.bfloat16, device=dev) for _ in range(N)]
+        sr = [t.to(dev) for t in src_rank]
+        so = [t.to(dev) for t in src_row]
+        wts = torch.softmax(torch.randn(tokens, topk, generator=rank_generator(torch, SEED, 99)), dim=1).to(dev)
+        ys = [torch.empty(tokens, hidden, dtype=torch.bfloat16, device=dev) for _ in range(N)]
+
+        def timed(fn, iters=5):
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / iters
+
+        def unfused():
+            for r in range(N):
+                mccl.gather_rows(hid[r], idx[r], out=sends[r])
+            mccl.alltoallv_n(sends, recv2, S6.tolist())
+
+        us_unfused = timed(unfused)
+        us_fused = timed(lambda: mccl.moe_dispatch_n(hid, idx, recv, S6.tolist()))
+        same = all(torch.equal(a, b) for a, b in zip(recv, recv2))
+        us_comb = timed(lambda: [mccl.moe_combine(recv, sr[r], so[r], wts, out=ys[r]) for r in range(N)])
+        moved = N * tokens * topk * hidden * 2
+        comb_bytes = moved + N * tokens * hidden * 2
+        result["moe_dispatch_combine"] = {
+            "unfused_gather_plus_alltoallv_us": round(us_unfused, 1), "fused_dispatch_us": round(us_fused, 1),
+            "fused_dispatch_GBps": round(2 * moved / us_fused / 1e3, 1), "fused_equals_unfused": same,
+            "combine_all_ranks_us": round(us_comb, 1), "combine_GBps": round(comb_bytes / us_comb / 1e3, 1),
+            "rows_routed": N * tokens * topk, "row_bytes": hidden * 2}
+        log("MoE:", json.dumps(result["moe_dispatch_combine"]))
+        del hid, idx, recv, recv2, sends, ys
 
     # ---------------- counter calibration: a copy of known size ----------------
     if "copycal" in extras:

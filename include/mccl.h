@@ -78,7 +78,8 @@ typedef enum {
   MCCL_TUNE_SMALL_MAX_BYTES = 2,          /* per-rank bytes up to which AUTO picks SMALL */
   MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
   MCCL_TUNE_STREAM_MIN_TOTAL_BYTES = 4,   /* (n+1)*bytes from which AUTO picks STREAM */
-  MCCL_TUNE_COUNT_ = 5
+  MCCL_TUNE_COMBINE_PIECES_PER_WAVE = 5,  /* 1 KiB row pieces one wavefront of moe_combine walks */
+  MCCL_TUNE_COUNT_ = 6
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64
@@ -157,6 +158,36 @@ int mccl_alltoallv_pull(const void* const* in, int n, void* out, const size_t* s
  * unpack: the inverse scatter (src/gpu/dpcpp_ccl.cpp:1528-1538). */
 int mccl_pack(const void* const* src, const size_t* bytes, int n, void* dst, void* stream);
 int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, void* stream);
+
+/*
+ * The callers' steps either side of the MoE all_to_all_single (no counterpart in the reference's
+ * sources; its users build the send buffer with a row gather and undo it with a second
+ * all_to_all plus a weighted sum).
+ *
+ * mccl_gather_rows: dst row j = src row row_index[j], j < nrows (the token permute).  row_index
+ * is a DEVICE array of int64; rows whose index is outside [0, src_rows) are left untouched.
+ *
+ * mccl_moe_dispatch_n: the permute fused into the alltoallv copy, for all n ranks at once.
+ * row_index[r] (device, sum_d S[r][d] entries) is rank r's send order: source rows of hidden[r]
+ * grouped by destination, S[r][d] rows for destination d.  Rank d's output segment r receives
+ * them directly; the permuted send buffer is never materialised (one read and one write per
+ * routed row instead of two).
+ *
+ * mccl_moe_combine: y[t][c] = sum_k weights[t*topk+k] * x[src_rank[t*topk+k]][src_row[t*topk+k]][c]
+ * for t < tokens, c < hidden_elems: the return all_to_all fused with the weighted sum over each
+ * token's top-k copies.  src_rank (int32), src_row (int64) and weights (fp32) are DEVICE arrays.
+ * fp32 chain from +0 in ascending k, each product rounded before it is added, one rounding to
+ * the storage type on store; bf16 / f16 / f32; rows must be a multiple of 16 bytes.  Entries
+ * with rank or row out of range contribute nothing.
+ */
+int mccl_gather_rows(const void* src, size_t src_rows, const int64_t* row_index, size_t nrows,
+                     size_t row_bytes, void* dst, void* stream);
+int mccl_moe_dispatch_n(const void* const* hidden, const size_t* hidden_rows,
+                        const int64_t* const* row_index, void* const* out, int n,
+                        const int64_t* split_rows, size_t row_bytes, void* stream);
+int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const int32_t* src_rank,
+                     const int64_t* src_row, const float* weights, size_t tokens, int topk,
+                     size_t hidden_elems, int dtype, void* y, void* stream);
 
 /* Launch geometry the library would use for mccl_reduce_n (for reports): returns the grid
  * size in workgroups (negative = mccl_status_t) and writes the workgroup size and the

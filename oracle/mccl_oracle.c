@@ -21,6 +21,9 @@
  *   oracle_alltoallv        src/gpu/dpcpp_ccl.cpp:1428-1455, src/cpu/cpu_ccl.cpp:924-950
  *                           (rank d's segment r comes from rank r's segment d)
  *   oracle_pack/unpack      src/gpu/dpcpp_ccl.cpp:1505-1515, 1528-1538
+ *   oracle_gather_rows / oracle_moe_dispatch / oracle_moe_combine
+ *                           no reference file: the callers' steps either side of the
+ *                           all_to_all_single of src/gpu/dpcpp_ccl.cpp:1428-1455
  *
  * Parity status
  *   pinned    : indexing of every op (reference tests' closed forms, brute force on
@@ -342,3 +345,72 @@ void oracle_f16_to_f32_array(const uint16_t* in, float* out, size_t n)
 { for (size_t i = 0; i < n; ++i) out[i] = oracle_f16_to_f32(in[i]); }
 void oracle_bf16_to_f32_array(const uint16_t* in, float* out, size_t n)
 { for (size_t i = 0; i < n; ++i) out[i] = oracle_bf16_to_f32(in[i]); }
+
+/* ---------- the steps either side of the MoE all_to_all (BASELINE config 5) ----------
+ * The reference has no MoE code; its callers build the all_to_all_single input by a row
+ * gather ("token permute") and, after the experts, undo it with a second all_to_all and a
+ * weighted sum over each token's top-k copies.  These restate those index maps and the fp32
+ * chain; they are pinned by brute-force loops on tagged inputs and by closed-form weights. */
+
+/* dst row j = src row idx[j]; rows whose index is outside [0, src_rows) are left untouched */
+int oracle_gather_rows(const void* src, size_t src_rows, const int64_t* idx, size_t nrows,
+                       size_t row_bytes, void* dst)
+{
+  for (size_t j = 0; j < nrows; ++j) {
+    if (idx[j] < 0 || (size_t)idx[j] >= src_rows) continue;
+    memcpy((char*)dst + j * row_bytes, (const char*)src + (size_t)idx[j] * row_bytes, row_bytes);
+  }
+  return 0;
+}
+
+/* Fused dispatch for all n ranks: rank r's send order is idx[r] (source rows grouped by
+ * destination, S[r][d] rows for destination d); rank d's output segment r receives them. */
+int oracle_moe_dispatch(const void* const* hidden, const size_t* hidden_rows, const int64_t* const* idx,
+                        void* const* out, int n, const int64_t* split_rows, size_t row_bytes)
+{
+  for (int d = 0; d < n; ++d) {
+    size_t roff = 0;
+    for (int r = 0; r < n; ++r) {
+      size_t soff = 0;
+      for (int dd = 0; dd < d; ++dd) soff += (size_t)split_rows[r * n + dd];
+      size_t rows = (size_t)split_rows[r * n + d];
+      oracle_gather_rows(hidden[r], hidden_rows[r], idx[r] + soff, rows, row_bytes,
+                         (char*)out[d] + roff * row_bytes);
+      roff += rows;
+    }
+  }
+  return 0;
+}
+
+/* y[t][c] = sum_k w[t*topk+k] * x[src_rank[t*topk+k]][src_row[t*topk+k]][c]
+ * fp32 chain from +0 in ascending k; each product is rounded to fp32 before it is added
+ * (no fused multiply-add); one rounding to the storage type at the end. */
+int oracle_moe_combine(const void* const* x, const size_t* x_rows, int n, const int32_t* src_rank,
+                       const int64_t* src_row, const float* w, size_t tokens, int topk,
+                       size_t hidden, int dtype, void* y)
+{
+  if (dtype != DT_BF16 && dtype != DT_F16 && dtype != DT_F32) return -1;
+  for (size_t t = 0; t < tokens; ++t) {
+    for (size_t c = 0; c < hidden; ++c) {
+      float acc = 0.0f;
+      for (int k = 0; k < topk; ++k) {
+        size_t e = t * (size_t)topk + (size_t)k;
+        int r = src_rank[e];
+        int64_t row = src_row[e];
+        if (r < 0 || r >= n || row < 0 || (size_t)row >= x_rows[r]) continue;
+        size_t off = (size_t)row * hidden + c;
+        float xv;
+        if (dtype == DT_BF16) xv = oracle_bf16_to_f32(((const uint16_t*)x[r])[off]);
+        else if (dtype == DT_F16) xv = oracle_f16_to_f32(((const uint16_t*)x[r])[off]);
+        else xv = ((const float*)x[r])[off];
+        volatile float prod = w[e] * xv; /* rounded product, never contracted into an fma */
+        acc = acc + prod;
+      }
+      size_t o = t * hidden + c;
+      if (dtype == DT_BF16) ((uint16_t*)y)[o] = oracle_f32_to_bf16(acc);
+      else if (dtype == DT_F16) ((uint16_t*)y)[o] = oracle_f32_to_f16(acc);
+      else ((float*)y)[o] = acc;
+    }
+  }
+  return 0;
+}

@@ -50,6 +50,9 @@ def lib():
         L.oracle_alltoallv.argtypes = [vp, vp, i32, vp, sz]
         L.oracle_pack.argtypes = [vp, vp, i32, vp]
         L.oracle_unpack.argtypes = [vp, vp, vp, i32]
+        L.oracle_gather_rows.argtypes = [vp, sz, vp, sz, sz, vp]
+        L.oracle_moe_dispatch.argtypes = [vp, vp, vp, vp, i32, vp, sz]
+        L.oracle_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp]
         L.oracle_set_threads.argtypes = [i32]
         for name in ("f32_to_bf16", "f32_to_f16", "f16_to_f32", "bf16_to_f32"):
             getattr(L, "oracle_%s_array" % name).argtypes = [vp, vp, sz]
@@ -183,3 +186,41 @@ def bf16_to_f32(h):
     out = np.empty(h.shape, dtype=np.float32)
     lib().oracle_bf16_to_f32_array(h.ctypes.data, out.ctypes.data, h.size)
     return out
+
+
+def gather_rows(src, idx, row_bytes):
+    """dst row j = src row idx[j] (uint8 arrays); out-of-range indices leave zeros."""
+    src = np.ascontiguousarray(src).view(np.uint8).reshape(-1)
+    idx = np.ascontiguousarray(idx, dtype=np.int64)
+    out = np.zeros(idx.size * row_bytes, dtype=np.uint8)
+    lib().oracle_gather_rows(src.ctypes.data, src.size // row_bytes, idx.ctypes.data, idx.size, row_bytes,
+                             out.ctypes.data)
+    return out
+
+
+def moe_dispatch(hidden, idx, split_rows, row_bytes):
+    """hidden[r]: rank r's rows (uint8); idx[r]: its send order; returns the n receive buffers."""
+    hs = [np.ascontiguousarray(h).view(np.uint8).reshape(-1) for h in hidden]
+    ix = [np.ascontiguousarray(i, dtype=np.int64) for i in idx]
+    n = len(hs)
+    S = np.ascontiguousarray(split_rows, dtype=np.int64).reshape(n, n)
+    outs = [np.zeros(int(S[:, d].sum()) * row_bytes, dtype=np.uint8) for d in range(n)]
+    rows = (ctypes.c_size_t * n)(*[h.size // row_bytes for h in hs])
+    lib().oracle_moe_dispatch(_ptr_array(hs), rows, _ptr_array(ix), _ptr_array(outs), n, S.ctypes.data, row_bytes)
+    return outs
+
+
+def moe_combine(x, src_rank, src_row, w, tokens, topk, hidden, dtype):
+    """x[r]: rank r's expert-output rows in the carrier dtype; returns y [tokens*hidden] carrier."""
+    xs = _check(x, dtype)
+    n = len(xs)
+    sr = np.ascontiguousarray(src_rank, dtype=np.int32)
+    so = np.ascontiguousarray(src_row, dtype=np.int64)
+    ww = np.ascontiguousarray(w, dtype=np.float32)
+    assert sr.size == so.size == ww.size == tokens * topk
+    rows = (ctypes.c_size_t * n)(*[a.size // hidden for a in xs])
+    y = np.empty(tokens * hidden, dtype=CARRIER[dtype])
+    rc = lib().oracle_moe_combine(_ptr_array(xs), rows, n, sr.ctypes.data, so.ctypes.data, ww.ctypes.data,
+                                  tokens, topk, hidden, dtype, y.ctypes.data)
+    assert rc == 0, rc
+    return y

@@ -1,0 +1,108 @@
+"""GPU parity of the steps either side of the MoE all_to_all: row gather, fused dispatch, weighted
+combine.  Copies are byte-exact; the combine is bit-exact against the oracle's fp32 chain."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bits_equal, bits, to_carrier, TORCH_TO_CODE
+from moe_helpers import combine_tables, route
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _u8(t):
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy().reshape(-1)
+
+
+@pytest.mark.parametrize("row_elems,dtype", [(7168, torch.bfloat16), (128, torch.bfloat16), (1025, torch.float32),
+                                             (3, torch.uint8), (1000, torch.int16)])
+def test_gather_rows_matches_oracle(mccl, row_elems, dtype):
+    g = torch.Generator().manual_seed(row_elems)
+    rows = 300
+    src = torch.randint(0, 127, (rows, row_elems), generator=g).to(dtype)
+    idx = torch.randint(0, rows, (1000,), generator=g, dtype=torch.int64)
+    out = mccl.gather_rows(src.to(DEV), idx.to(DEV))
+    torch.cuda.synchronize()
+    want = O.gather_rows(_u8(src), idx.numpy(), row_elems * src.element_size())
+    assert_bits_equal(_u8(out), want, "gather_rows")
+    assert torch.equal(out.cpu(), src[idx])
+
+
+def test_gather_rows_skips_out_of_range_indices(mccl):
+    src = torch.arange(40, dtype=torch.float32).view(10, 4).to(DEV)
+    idx = torch.tensor([3, -1, 10, 0, 99], dtype=torch.int64, device=DEV)
+    out = torch.full((5, 4), -7.0, device=DEV)
+    mccl.gather_rows(src, idx, out=out)
+    torch.cuda.synchronize()
+    assert out.cpu().tolist() == [[12, 13, 14, 15], [-7] * 4, [-7] * 4, [0, 1, 2, 3], [-7] * 4]
+
+
+@pytest.mark.parametrize("n,tokens,hidden,topk,n_exp", [(8, 64, 128, 8, 256), (4, 100, 96, 2, 16), (2, 33, 7168, 4, 8)])
+def test_fused_dispatch_equals_gather_then_alltoallv(mccl, n, tokens, hidden, topk, n_exp):
+    S, send_tok, _ = route(n, tokens, n_exp, topk)
+    hid = []
+    for r in range(n):
+        g = torch.Generator().manual_seed(77 + r)
+        hid.append(torch.randn(tokens, hidden, generator=g).to(torch.bfloat16))
+    dev_h = [h.to(DEV) for h in hid]
+    dev_i = [t.to(DEV) for t in send_tok]
+    fused = [torch.zeros(int(S[:, d].sum()), hidden, dtype=torch.bfloat16, device=DEV) for d in range(n)]
+    mccl.moe_dispatch_n(dev_h, dev_i, fused, S.tolist())
+    # unfused: materialise the permuted send buffers, then the uneven alltoall copy
+    sends = [mccl.gather_rows(dev_h[r], dev_i[r]) for r in range(n)]
+    unfused = [torch.zeros_like(f) for f in fused]
+    mccl.alltoallv_n(sends, unfused, S.tolist())
+    torch.cuda.synchronize()
+    want = O.moe_dispatch([_u8(h) for h in hid], [t.numpy() for t in send_tok], S, hidden * 2)
+    for d in range(n):
+        assert_bits_equal(_u8(fused[d]), want[d], "fused dispatch dest %d" % d)
+        assert_bits_equal(_u8(unfused[d]), want[d], "unfused dispatch dest %d" % d)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+@pytest.mark.parametrize("n,tokens,hidden,topk,n_exp", [(8, 64, 128, 8, 256), (4, 50, 200, 3, 16)])
+def test_combine_matches_oracle(mccl, dtype, n, tokens, hidden, topk, n_exp):
+    """Rank 0's tokens: dispatch, pretend the experts scaled their rows, combine with random
+    weights; compare with the oracle's fp32 chain bit for bit."""
+    S, send_tok, _ = route(n, tokens, n_exp, topk)
+    src_rank, src_row = combine_tables(n, tokens, topk, S, send_tok)
+    x = []
+    for d in range(n):
+        g = torch.Generator().manual_seed(500 + d)
+        x.append(torch.randn(int(S[:, d].sum()), hidden, generator=g).to(dtype))
+    g = torch.Generator().manual_seed(9)
+    w = torch.softmax(torch.randn(tokens, topk, generator=g), dim=1).contiguous()
+    for r in (0, n - 1):
+        y = mccl.moe_combine([t.to(DEV) for t in x], src_rank[r].to(DEV), src_row[r].to(DEV), w.to(DEV))
+        torch.cuda.synchronize()
+        want = O.moe_combine([to_carrier(t) for t in x], src_rank[r].numpy(), src_row[r].numpy(), w.numpy(),
+                             tokens, topk, hidden, TORCH_TO_CODE[dtype])
+        width = {2: np.uint16, 4: np.uint32}[y.element_size()]
+        assert_bits_equal(bits(y), want.view(width), "combine rank %d %s" % (r, dtype))
+
+
+def test_dispatch_then_one_hot_combine_returns_the_tokens(mccl):
+    """Round trip at the real row length: with weight 1 on a token's first copy and 0 elsewhere,
+    combine(dispatch(h)) == h exactly (0 + 1*x + 0*y... adds exact zeros)."""
+    n, tokens, hidden, topk, n_exp = 8, 256, 7168, 8, 256
+    S, send_tok, _ = route(n, tokens, n_exp, topk)
+    src_rank, src_row = combine_tables(n, tokens, topk, S, send_tok)
+    hid = []
+    for r in range(n):
+        g = torch.Generator().manual_seed(31 + r)
+        hid.append((torch.randn(tokens, hidden, generator=g).abs() + 0.5).to(torch.bfloat16).to(DEV))  # no -0, no NaN
+    recv = [torch.zeros(int(S[:, d].sum()), hidden, dtype=torch.bfloat16, device=DEV) for d in range(n)]
+    mccl.moe_dispatch_n(hid, [t.to(DEV) for t in send_tok], recv, S.tolist())
+    w = torch.zeros(tokens, topk)
+    w[:, 0] = 1.0
+    for r in range(n):
+        y = mccl.moe_combine(recv, src_rank[r].to(DEV), src_row[r].to(DEV), w.to(DEV))
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), hid[r].view(torch.int16)), "rank %d" % r
+    # and with uniform weights 1/8 (a power of two: exact products) every copy is the token itself
+    w = torch.full((tokens, topk), 0.125)
+    y = mccl.moe_combine(recv, src_rank[3].to(DEV), src_row[3].to(DEV), w.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), hid[3].view(torch.int16))

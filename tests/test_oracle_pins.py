@@ -201,3 +201,65 @@ def test_alltoall_counts_equal_and_empty():
     assert counts.tolist() == [6, 0, 54] and displs.tolist() == [0, 6, 6]
     counts, displs = O.alltoall_counts(3, 0, 0, [0, 0, 0])    # empty tensor: no division
     assert counts.tolist() == [0, 0, 0]
+
+
+# ---------------- MoE steps: brute force and closed forms ----------------
+
+def test_gather_and_dispatch_brute_force():
+    from moe_helpers import route
+    n, tokens, topk, n_exp, row = 4, 9, 2, 8, 3
+    S, send_tok, send_exp = route(n, tokens, n_exp, topk)
+    hidden = [np.array([[r * 10000 + t * 10 + c for c in range(row)] for t in range(tokens)], dtype=np.int32)
+              for r in range(n)]
+    outs = O.moe_dispatch(hidden, [t.numpy() for t in send_tok], S, row * 4)
+    per_rank = n_exp // n
+    for d in range(n):
+        want = []
+        for r in range(n):  # plain loops from the definition: rows for experts owned by d, by (expert, token)
+            pairs = sorted((int(e), int(t)) for t, e in zip(send_tok[r].tolist(), send_exp[r].tolist())
+                           if e // per_rank == d)
+            for e, t in pairs:
+                want.extend(r * 10000 + t * 10 + c for c in range(row))
+        assert outs[d].view(np.int32).tolist() == want
+    g = O.gather_rows(hidden[1], [5, 0, 5, 8], row * 4).view(np.int32).reshape(4, row)
+    assert g.tolist() == [hidden[1][5].tolist(), hidden[1][0].tolist(), hidden[1][5].tolist(), hidden[1][8].tolist()]
+
+
+def test_combine_closed_forms():
+    """One-hot weights return the selected row; weights 0.5/0.25/0.25 on rows 8, 4, 4 give 6;
+    the chain is fp32 with a rounded product: (2^-9 * 1) three times on top of 1.0 rounds up."""
+    x0 = O.f32_to_bf16(np.array([[8.0, 1.0], [4.0, 2.0 ** -9]], dtype=np.float32)).reshape(-1)
+    x1 = O.f32_to_bf16(np.array([[4.0, 2.0 ** -9]], dtype=np.float32)).reshape(-1)
+    sr = np.array([[0, 0, 1]], dtype=np.int32)
+    so = np.array([[0, 1, 0]], dtype=np.int64)
+    y = O.moe_combine([x0, x1], sr, so, np.array([[1.0, 0.0, 0.0]], dtype=np.float32), 1, 3, 2, O.BF16)
+    assert O.bf16_to_f32(y).tolist() == [8.0, 1.0]
+    y = O.moe_combine([x0, x1], sr, so, np.array([[0.5, 0.25, 0.25]], dtype=np.float32), 1, 3, 2, O.BF16)
+    assert O.bf16_to_f32(y)[0] == 6.0
+    # column 1: 1*1.0 + 1*2^-9 + 1*2^-9 = 1 + 2^-8: a tie in bf16 -> stays 1.0 (even)
+    y = O.moe_combine([x0, x1], sr, so, np.array([[1.0, 1.0, 1.0]], dtype=np.float32), 1, 3, 2, O.BF16)
+    assert y[1] == 0x3F80
+    # with weight 1.5 on the two small terms: 1 + 3*2^-9 -> rounds up (fp32 accumulation, one rounding)
+    y = O.moe_combine([x0, x1], sr, so, np.array([[1.0, 1.5, 1.5]], dtype=np.float32), 1, 3, 2, O.BF16)
+    assert y[1] == 0x3F81
+    # out-of-range entries contribute nothing
+    y = O.moe_combine([x0, x1], np.array([[0, 5, 1]], dtype=np.int32), np.array([[0, 0, 9]], dtype=np.int64),
+                      np.array([[1.0, 1.0, 1.0]], dtype=np.float32), 1, 3, 2, O.BF16)
+    assert O.bf16_to_f32(y).tolist() == [8.0, 1.0]
+
+
+def test_combine_matches_torch_fp32():
+    rng = np.random.default_rng(12)
+    n, rows, hidden, tokens, topk = 3, 20, 16, 11, 4
+    x = [O.f32_to_bf16(rng.standard_normal((rows, hidden)).astype(np.float32)).reshape(-1) for _ in range(n)]
+    sr = rng.integers(0, n, size=(tokens, topk)).astype(np.int32)
+    so = rng.integers(0, rows, size=(tokens, topk)).astype(np.int64)
+    w = rng.random((tokens, topk)).astype(np.float32)
+    y = O.moe_combine(x, sr, so, w, tokens, topk, hidden, O.BF16)
+    xs = [torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).view(rows, hidden).float() for a in x]
+    acc = torch.zeros(tokens, hidden)
+    for k in range(topk):
+        rows_k = torch.stack([xs[sr[t, k]][so[t, k]] for t in range(tokens)])
+        acc = acc + torch.from_numpy(w[:, k:k + 1]) * rows_k
+    want = acc.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16).reshape(-1)
+    assert np.array_equal(y, want)

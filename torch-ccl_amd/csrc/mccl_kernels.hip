@@ -86,8 +86,9 @@ long long g_tune[MCCL_TUNE_COUNT_] = {
     /* SMALL_MAX_BYTES          */ 8 << 20,
     /* COPY_WAVES_PER_CU        */ 28,
     /* STREAM_MIN_TOTAL_BYTES   */ 320ll << 20,
+    /* COMBINE_PIECES_PER_WAVE  */ 2,
 };
-const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 72 * 1024, 8 << 20, 28, 320ll << 20};
+const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 72 * 1024, 8 << 20, 28, 320ll << 20, 2};
 
 // Dynamic-LDS bytes that limit residency to `waves` single-wavefront workgroups per CU
 // (0 = no reservation needed).
@@ -485,6 +486,200 @@ __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) 
 }
 
 // ------------------------------------------------------------------------------------------
+// row gather (token permute) and the fused MoE dispatch / combine
+// ------------------------------------------------------------------------------------------
+// One gather segment: dst row j = src row idx[j], j < nrows.  Rows are row_bytes long.
+struct GatherSeg {
+  const char* src;
+  const int64_t* idx;
+  char* dst;
+  uint32_t nrows;
+  uint32_t src_rows;  // rows with idx outside [0, src_rows) are skipped (left untouched)
+};
+
+struct GatherArgs {
+  GatherSeg seg[kMaxSegs];
+  uint32_t chunk_prefix[kMaxSegs + 1];  // chunks = nrows * pieces_per_row
+  int nseg;
+  uint32_t row_bytes;
+  uint32_t pieces_per_row;  // ceil(row_bytes / kCopyChunk)
+  uint32_t vector_ok;       // all bases 16-byte aligned and row_bytes % 16 == 0
+};
+
+// One wavefront moves one 2 KiB piece of one row.  Chunks are numbered row-major within a
+// segment and handed out in order, so the destination is written as a compact moving window;
+// the sources are whole rows (contiguous row_bytes each).
+__global__ __launch_bounds__(kWave) void gather_rows_kernel(const GatherArgs a) {
+  const uint32_t total = a.chunk_prefix[a.nseg];
+  const uint32_t ppr = a.pieces_per_row;
+  const uint32_t row_bytes = a.row_bytes;
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    int lo = 0, hi = a.nseg;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    const uint32_t lc = chunk - a.chunk_prefix[lo];
+    const uint32_t row = lc / ppr;
+    const uint32_t piece = lc - row * ppr;
+    const int64_t srow = a.seg[lo].idx[row];
+    if (srow < 0 || srow >= (int64_t)a.seg[lo].src_rows) continue;
+    const uint32_t off = piece * (uint32_t)kCopyChunk;
+    const uint32_t left = row_bytes - off;
+    const uint32_t len = left < (uint32_t)kCopyChunk ? left : (uint32_t)kCopyChunk;
+    const char* src = a.seg[lo].src + (size_t)srow * row_bytes + off;
+    char* dst = a.seg[lo].dst + (size_t)row * row_bytes + off;
+    const uint32_t t = threadIdx.x;
+    if (a.vector_ok) {
+      const u32x4* sv = (const u32x4*)src;
+      u32x4* dv = (u32x4*)dst;
+      if (len == (uint32_t)kCopyChunk) {
+        u32x4 x[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) x[u] = sv[t + u * kWave];  // rows are re-read (top-k): cacheable
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      } else {
+        const uint32_t nv = len >> 4;
+        for (uint32_t v = t; v < nv; v += kWave) __builtin_nontemporal_store(sv[v], &dv[v]);
+      }
+    } else {
+      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
+    }
+  }
+}
+
+// Weighted combine: y[t][c] = sum_k w[t][k] * x[rank(t,k)][row(t,k)][c], fp32 chain from +0 in
+// ascending k, every product rounded before it is added, one rounding on store.
+struct CombineArgs {
+  const char* x[MCCL_MAX_RANKS];
+  uint32_t x_rows[MCCL_MAX_RANKS];
+  const int32_t* src_rank;
+  const int64_t* src_row;
+  const float* w;
+  char* y;
+  uint32_t tokens;
+  uint32_t topk;
+  uint32_t row_vecs;        // 16-byte vectors per row
+  uint32_t pieces_per_row;  // ceil(row_vecs / 64)
+  uint32_t pieces_per_wave; // 1 KiB pieces one wavefront walks (routing entries are looked up once)
+  uint32_t waves_per_row;   // ceil(pieces_per_row / pieces_per_wave)
+  int n;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a) {
+  using A = float;
+  constexpr int VE = vec_elems<DT>();
+  constexpr int G = 8;  // row loads in flight per lane (one group covers top-8 routing)
+  const uint32_t total = a.tokens * a.waves_per_row;
+  const size_t row_stride = (size_t)a.row_vecs * 16;
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    const uint32_t tok = chunk / a.waves_per_row;
+    const uint32_t part = chunk - tok * a.waves_per_row;
+    const uint32_t p0 = part * a.pieces_per_wave;
+    const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
+    const size_t e0 = (size_t)tok * a.topk;
+    if (a.topk <= G) {
+      // routing entries looked up once for all pieces this wavefront walks
+      int rk[G];
+      int64_t rw[G];
+      float wk[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool in = (uint32_t)g < a.topk;
+        rk[g] = in ? a.src_rank[e0 + g] : -1;
+        rw[g] = in ? a.src_row[e0 + g] : 0;
+        wk[g] = in ? a.w[e0 + g] : 0.0f;
+      }
+      const u32x4* src[G];
+      bool ok[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool rank_ok = rk[g] >= 0 && rk[g] < a.n;
+        const int r = rank_ok ? rk[g] : 0;
+        ok[g] = rank_ok && rw[g] >= 0 && rw[g] < (int64_t)a.x_rows[r];
+        src[g] = (const u32x4*)(a.x[r] + (ok[g] ? (size_t)rw[g] : 0) * row_stride);
+      }
+      for (uint32_t piece = p0; piece < p1; ++piece) {
+        const uint32_t v = piece * kWave + threadIdx.x;
+        const bool live = v < a.row_vecs;
+        VecU<DT> x[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          x[g].v = (u32x4){0u, 0u, 0u, 0u};
+          if (ok[g] && live) x[g].v = __builtin_nontemporal_load(src[g] + v);
+        }
+        A acc[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if (ok[g]) {
+#pragma unroll
+            for (int e = 0; e < VE; ++e) {
+              const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
+              acc[e] = acc[e] + prod;
+            }
+          }
+        }
+        if (live) {
+          VecU<DT> r;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
+          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
+        }
+      }
+    } else {
+      // general top-k: groups of G entries per piece
+      for (uint32_t piece = p0; piece < p1; ++piece) {
+        const uint32_t v = piece * kWave + threadIdx.x;
+        const bool live = v < a.row_vecs;
+        A acc[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
+        for (uint32_t kb = 0; kb < a.topk; kb += G) {
+          VecU<DT> x[G];
+          float wk[G];
+          bool ok[G];
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            ok[g] = false;
+            wk[g] = 0.0f;
+            x[g].v = (u32x4){0u, 0u, 0u, 0u};
+            if (kb + g < a.topk) {
+              const int r = a.src_rank[e0 + kb + g];
+              const int64_t row = a.src_row[e0 + kb + g];
+              if (r >= 0 && r < a.n && row >= 0 && row < (int64_t)a.x_rows[r]) {
+                ok[g] = true;
+                wk[g] = a.w[e0 + kb + g];
+                if (live) x[g].v = __builtin_nontemporal_load((const u32x4*)(a.x[r] + (size_t)row * row_stride) + v);
+              }
+            }
+          }
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            if (ok[g]) {
+#pragma unroll
+              for (int e = 0; e < VE; ++e) {
+                const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
+                acc[e] = acc[e] + prod;
+              }
+            }
+          }
+        }
+        if (live) {
+          VecU<DT> r;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
+          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // host-side launch helpers
 // ------------------------------------------------------------------------------------------
 bool valid_dtype(int dt) { return dt >= MCCL_U8 && dt <= MCCL_BF16; }
@@ -774,6 +969,62 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
   return MCCL_OK;
 }
 
+// Launches gather segments in batches of kMaxSegs.
+struct GatherSpec {
+  const void* src;
+  size_t src_rows;
+  const int64_t* idx;
+  void* dst;
+  size_t nrows;
+};
+
+int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStream_t s) {
+  if (row_bytes == 0) return MCCL_OK;
+  if (row_bytes > 0x7fffffffull) return fail(MCCL_ERR_INVALID_ARG, "row of %zu bytes is too long", row_bytes);
+  const uint32_t ppr = (uint32_t)((row_bytes + kCopyChunk - 1) / kCopyChunk);
+  int i = 0;
+  while (i < nspec) {
+    GatherArgs a;
+    int m = 0;
+    uint64_t chunks = 0;
+    bool vec = (row_bytes % 16) == 0;
+    a.chunk_prefix[0] = 0;
+    while (i < nspec && m < kMaxSegs) {
+      const GatherSpec& g = specs[i];
+      if (g.nrows == 0) { ++i; continue; }
+      if (!g.src || !g.idx || !g.dst) return fail(MCCL_ERR_INVALID_ARG, "gather segment %d has a null pointer", i);
+      if (g.nrows > 0xffffffffull || g.src_rows > 0xffffffffull)
+        return fail(MCCL_ERR_INVALID_ARG, "gather segment %d has too many rows", i);
+      if ((uintptr_t)g.idx % 8) return fail(MCCL_ERR_INVALID_ARG, "row index table %d is not 8-byte aligned", i);
+      const uint64_t c = (uint64_t)g.nrows * ppr;
+      if (chunks + c > 0xffffffffull) {
+        if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "gather segment %d too large", i);
+        break;
+      }
+      if (((uintptr_t)g.src | (uintptr_t)g.dst) & 15u) vec = false;
+      a.seg[m] = GatherSeg{(const char*)g.src, g.idx, (char*)g.dst, (uint32_t)g.nrows, (uint32_t)g.src_rows};
+      chunks += c;
+      a.chunk_prefix[++m] = (uint32_t)chunks;
+      ++i;
+    }
+    if (m == 0) break;
+    a.nseg = m;
+    a.row_bytes = (uint32_t)row_bytes;
+    a.pieces_per_row = ppr;
+    a.vector_ok = vec ? 1u : 0u;
+    int cus = 0;
+    int rc = device_cus(&cus);
+    if (rc != MCCL_OK) return rc;
+    uint64_t grid = chunks;
+    if (grid > kMaxGridX) grid = kMaxGridX;
+    const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_COPY_WAVES_PER_CU]) : 0;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)grid), dim3(kWave), lds, s, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MCCL_ERR_HIP, "gather kernel launch failed: %s", hipGetErrorString(e));
+  }
+  return MCCL_OK;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------------------------
@@ -994,6 +1245,101 @@ int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, v
     int rc = launch_copy(segs, m, (hipStream_t)stream);
     if (rc != MCCL_OK) return rc;
   }
+  return MCCL_OK;
+}
+
+int mccl_gather_rows(const void* src, size_t src_rows, const int64_t* row_index, size_t nrows,
+                     size_t row_bytes, void* dst, void* stream) {
+  if (nrows == 0 || row_bytes == 0) return MCCL_OK;
+  GatherSpec g{src, src_rows, row_index, dst, nrows};
+  return launch_gather(&g, 1, row_bytes, (hipStream_t)stream);
+}
+
+int mccl_moe_dispatch_n(const void* const* hidden, const size_t* hidden_rows,
+                        const int64_t* const* row_index, void* const* out, int n,
+                        const int64_t* split_rows, size_t row_bytes, void* stream) {
+  if (!hidden || !hidden_rows || !row_index || !out || !split_rows) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  for (int i = 0; i < n * n; ++i)
+    if (split_rows[i] < 0) return fail(MCCL_ERR_INVALID_ARG, "negative split size");
+  GatherSpec specs[MCCL_MAX_RANKS];
+  for (int d = 0; d < n; ++d) {  // one destination rank per batch: its output is written front to back
+    size_t roff = 0;
+    int m = 0;
+    for (int r = 0; r < n; ++r) {
+      size_t soff = 0;
+      for (int dd = 0; dd < d; ++dd) soff += (size_t)split_rows[r * n + dd];
+      const size_t rows = (size_t)split_rows[r * n + d];
+      if (rows) {
+        if (!hidden[r] || !row_index[r] || !out[d]) return fail(MCCL_ERR_INVALID_ARG, "null buffer for a non-empty segment");
+        specs[m++] = GatherSpec{hidden[r], hidden_rows[r], row_index[r] + soff, (char*)out[d] + roff * row_bytes, rows};
+      }
+      roff += rows;
+    }
+    int rc = launch_gather(specs, m, row_bytes, (hipStream_t)stream);
+    if (rc != MCCL_OK) return rc;
+  }
+  return MCCL_OK;
+}
+
+int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const int32_t* src_rank,
+                     const int64_t* src_row, const float* weights, size_t tokens, int topk,
+                     size_t hidden_elems, int dtype, void* y, void* stream) {
+  if (!x || !x_rows) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  if (dtype != MCCL_BF16 && dtype != MCCL_F16 && dtype != MCCL_F32)
+    return fail(MCCL_ERR_UNSUPPORTED, "moe_combine is defined for bf16, f16 and f32");
+  if (topk < 1 || topk > 64) return fail(MCCL_ERR_INVALID_ARG, "topk %d outside [1, 64]", topk);
+  if (tokens == 0 || hidden_elems == 0) return MCCL_OK;
+  if (!src_rank || !src_row || !weights || !y) return fail(MCCL_ERR_INVALID_ARG, "null pointer");
+  const size_t row_bytes = hidden_elems * dtype_size(dtype);
+  if (row_bytes % 16) return fail(MCCL_ERR_UNSUPPORTED, "moe_combine needs rows that are a multiple of 16 bytes");
+  if ((uintptr_t)y & 15u) return fail(MCCL_ERR_INVALID_ARG, "output is not 16-byte aligned");
+  if (((uintptr_t)src_rank & 3u) || ((uintptr_t)src_row & 7u) || ((uintptr_t)weights & 3u))
+    return fail(MCCL_ERR_INVALID_ARG, "index or weight table is misaligned");
+  CombineArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int r = 0; r < n; ++r) {
+    if (x_rows[r] && !x[r]) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d is null", r);
+    if ((uintptr_t)x[r] & 15u) return fail(MCCL_ERR_INVALID_ARG, "input %d is not 16-byte aligned", r);
+    if (x_rows[r] > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "input %d has too many rows", r);
+    a.x[r] = (const char*)x[r];
+    a.x_rows[r] = (uint32_t)x_rows[r];
+  }
+  const size_t row_vecs = row_bytes / 16;
+  const size_t ppr = (row_vecs + kWave - 1) / kWave;
+  if (tokens * ppr > 0xffffffffull || row_vecs > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  a.src_rank = src_rank;
+  a.src_row = src_row;
+  a.w = weights;
+  a.y = (char*)y;
+  a.tokens = (uint32_t)tokens;
+  a.topk = (uint32_t)topk;
+  a.row_vecs = (uint32_t)row_vecs;
+  a.pieces_per_row = (uint32_t)ppr;
+  size_t ppw = (size_t)g_tune[MCCL_TUNE_COMBINE_PIECES_PER_WAVE];
+  if (ppw < 1) ppw = 1;
+  if (ppw > ppr) ppw = ppr;
+  a.pieces_per_wave = (uint32_t)ppw;
+  a.waves_per_row = (uint32_t)((ppr + ppw - 1) / ppw);
+  a.n = n;
+  int cus = 0;
+  int rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  uint64_t grid = (uint64_t)tokens * a.waves_per_row;
+  if (grid > kMaxGridX) grid = kMaxGridX;
+  // Wavefronts here live longer than in the plain reduction (routing-table lookups before the
+  // row loads), and more of them are needed to cover that latency: measured best without a
+  // residency cap.
+  const unsigned lds = 0;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MCCL_BF16: hipLaunchKernelGGL((moe_combine_kernel<MCCL_BF16>), dim3((unsigned)grid), dim3(kWave), lds, s, a); break;
+    case MCCL_F16: hipLaunchKernelGGL((moe_combine_kernel<MCCL_F16>), dim3((unsigned)grid), dim3(kWave), lds, s, a); break;
+    default: hipLaunchKernelGGL((moe_combine_kernel<MCCL_F32>), dim3((unsigned)grid), dim3(kWave), lds, s, a); break;
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "combine kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
 

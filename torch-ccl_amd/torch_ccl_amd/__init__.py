@@ -13,8 +13,8 @@ import torch.distributed as _dist
 from . import capi
 from .capi import (AVG, MAX, MIN, PROD, SUM, VARIANT_AUTO, VARIANT_PERSISTENT,  # noqa: F401
                    VARIANT_SMALL, VARIANT_STREAM)
-from .ops import (allgather_n, alltoallv_n, copy_segments, pack, reduce_multi,  # noqa: F401
-                  reduce_n, reduce_scatter_n, unpack)
+from .ops import (allgather_n, alltoallv_n, copy_segments, gather_rows, moe_combine,  # noqa: F401
+                  moe_dispatch_n, pack, reduce_multi, reduce_n, reduce_scatter_n, unpack)
 
 capi.lib()  # fail loudly at import time when the native library is absent
 

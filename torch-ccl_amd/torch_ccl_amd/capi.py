@@ -19,7 +19,7 @@ U8, I8, I16, I32, I64, F16, F32, F64, BF16 = range(9)
 SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
 VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
 (TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_INFLIGHT_BYTES, TUNE_SMALL_MAX_BYTES,
- TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES) = range(5)
+ TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE) = range(6)
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
@@ -33,6 +33,7 @@ EXPORTS = (
     "mccl_reduce_scatter_n", "mccl_reduce_multi", "mccl_copy_segments", "mccl_allgather_n",
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
+    "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
 )
 
 
@@ -66,6 +67,9 @@ def lib():
     L.mccl_alltoallv_pull.argtypes = [vp, i32, vp, vp, vp, vp]
     L.mccl_pack.argtypes = [vp, vp, i32, vp, vp]
     L.mccl_unpack.argtypes = [vp, vp, vp, i32, vp]
+    L.mccl_gather_rows.argtypes = [vp, sz, vp, sz, sz, vp, vp]
+    L.mccl_moe_dispatch_n.argtypes = [vp, vp, vp, vp, i32, vp, sz, vp]
+    L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_query_launch.argtypes = [sz, i32, i32, i32, i32, vp, vp]
     L.mccl_set_tuning.argtypes = [i32, ctypes.c_longlong]
     L.mccl_get_tuning.argtypes = [i32]

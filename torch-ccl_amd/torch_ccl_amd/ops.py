@@ -168,3 +168,72 @@ def unpack(src, dsts):
     capi.check(capi.lib().mccl_unpack(src.data_ptr(), capi.ptr_table([t.data_ptr() for t in dsts]),
                                       capi.size_table(sizes), len(dsts), _stream()))
     return dsts
+
+
+def _row_bytes(t):
+    return (t.numel() // t.shape[0] if t.shape[0] else 0) * t.element_size()
+
+
+def gather_rows(src, row_index, out=None):
+    """out[j] = src[row_index[j]] (token permute); row_index is an int64 tensor on the GPU."""
+    _check_tensors([src] + ([out] if out is not None else []), "gather_rows")
+    if row_index.dtype != torch.int64 or not row_index.is_cuda or not row_index.is_contiguous():
+        raise RuntimeError("gather_rows: row_index must be a contiguous int64 tensor on the GPU")
+    if out is None:
+        out = torch.empty((row_index.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+    if out.shape[0] != row_index.numel() or tuple(out.shape[1:]) != tuple(src.shape[1:]):
+        raise RuntimeError("gather_rows: output shape does not match the index and the source rows")
+    rb = (src.numel() // src.shape[0] if src.shape[0] else 0) * src.element_size()
+    with torch.cuda.device(src.device):
+        capi.check(capi.lib().mccl_gather_rows(src.data_ptr(), src.shape[0], row_index.data_ptr(),
+                                               row_index.numel(), rb, out.data_ptr(), _stream()))
+    return out
+
+
+def moe_dispatch_n(hidden, row_index, outputs, split_rows):
+    """Fused token permute + alltoallv for all ranks: outputs[d] segment r = hidden[r][row_index[r][...]]."""
+    _check_tensors(list(hidden) + list(outputs), "moe_dispatch_n")
+    n = len(hidden)
+    S = torch.as_tensor(split_rows, dtype=torch.int64).reshape(n, n).contiguous()
+    rb = None
+    for t in list(hidden) + list(outputs):
+        if t.numel():
+            b = _row_bytes(t)
+            if rb is None:
+                rb = b
+            elif b != rb:
+                raise RuntimeError("moe_dispatch_n: all tensors need the same row length")
+    if rb is None:
+        return outputs
+    for r in range(n):
+        ix = row_index[r]
+        if ix.dtype != torch.int64 or not ix.is_cuda or not ix.is_contiguous():
+            raise RuntimeError("moe_dispatch_n: row_index must be contiguous int64 tensors on the GPU")
+        if ix.numel() != int(S[r].sum()):
+            raise RuntimeError("moe_dispatch_n: row_index[%d] does not match the split sizes" % r)
+        if outputs[r].shape[0] != int(S[:, r].sum()):
+            raise RuntimeError("Tensor's dim 0 does not match sum of splits")
+    with torch.cuda.device(outputs[0].device):
+        capi.check(capi.lib().mccl_moe_dispatch_n(
+            capi.ptr_table([t.data_ptr() for t in hidden]), capi.size_table([t.shape[0] for t in hidden]),
+            capi.ptr_table([t.data_ptr() for t in row_index]), capi.ptr_table([t.data_ptr() for t in outputs]),
+            n, ctypes.c_void_p(S.data_ptr()), rb, _stream()))
+    return outputs
+
+
+def moe_combine(x, src_rank, src_row, weights, out=None):
+    """out[t] = sum_k weights[t, k] * x[src_rank[t, k]][src_row[t, k]] with fp32 accumulation."""
+    _check_tensors(list(x) + ([out] if out is not None else []), "moe_combine")
+    tokens, topk = weights.shape
+    for t, dt in ((src_rank, torch.int32), (src_row, torch.int64), (weights, torch.float32)):
+        if t.dtype != dt or not t.is_cuda or not t.is_contiguous() or tuple(t.shape) != (tokens, topk):
+            raise RuntimeError("moe_combine: src_rank int32, src_row int64, weights fp32, all [tokens, topk] on the GPU")
+    hidden = x[0].numel() // x[0].shape[0] if x[0].shape[0] else 0
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=x[0].dtype, device=x[0].device)
+    with torch.cuda.device(out.device):
+        capi.check(capi.lib().mccl_moe_combine(
+            capi.ptr_table([t.data_ptr() for t in x]), capi.size_table([t.shape[0] for t in x]), len(x),
+            src_rank.data_ptr(), src_row.data_ptr(), weights.data_ptr(), tokens, topk, hidden,
+            _dtype_code(out.dtype), out.data_ptr(), _stream()))
+    return out
