@@ -248,6 +248,24 @@ def main():
                                                 "min_us": round(us[0], 2)}
         b2b = benchlib.reduce_throughput(in_sets[:1], outs[:1], variant=capi.VARIANT_SMALL, warmup=100, iters=1000)
         lat["small_back_to_back_us"] = round(b2b, 2)
+        # launch-bound loops belong in a HIP graph: 100 calls captured once, replayed 10 times
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            mccl.reduce_n(in_sets[0], out=outs[0], variant=capi.VARIANT_SMALL)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g):
+            for _ in range(100):
+                mccl.reduce_n(in_sets[0], out=outs[0], variant=capi.VARIANT_SMALL)
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        lat["small_graph_replay_us"] = round(e0.elapsed_time(e1) * 1e3 / 1000, 2)
         lat["iters"] = 1000
         lat["workload"] = "C2 allreduce SUM, 8 x bf16 [16 x 8192] (256 KiB each), one HIP event pair per call"
         result["latency_256KB"] = lat
