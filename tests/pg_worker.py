@@ -238,6 +238,23 @@ def missing_rank_case(pg, rank, world):
                 or "rank 1 left the group" in str(e)), str(e)
 
 
+def env_switch_case(pg, rank, world):
+    """CCL_SAME_STREAM / CCL_BLOCKING_WAIT (src/ProcessGroupCCL.hpp:96-102): results are the same,
+    a blocking wait leaves the Work completed, a same-stream op is ordered on the caller's stream."""
+    t = torch.full((1 << 20,), float(rank + 1), device=DEV)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        t2 = t * 2  # produced on a side stream; the collective must be ordered after it
+        w = pg.allreduce([t2], c10d.AllreduceOptions())
+        w.wait()
+        if os.environ.get("CCL_BLOCKING_WAIT") == "1":
+            assert w.is_completed()
+        r = t2 + 1
+    side.synchronize()
+    assert float(r[0]) == world * (world + 1) + 1 and float(r[-1]) == world * (world + 1) + 1
+    pg.barrier().wait()
+
+
 def run_rank(rank, world, store_path, mode):
     torch.cuda.set_device(0)
     import torch_ccl_amd  # noqa: F401  registers the backend
@@ -258,6 +275,8 @@ def run_rank(rank, world, store_path, mode):
         oracle_cases(pg, rank, world)
     elif mode == "large":
         large_message_case(pg, rank, world)
+    elif mode == "env":
+        env_switch_case(pg, rank, world)
     elif mode == "missing":
         missing_rank_case(pg, rank, world)
     else:

@@ -91,3 +91,10 @@ def test_thread_ranks_in_one_process():
         th.join(timeout=120)
     assert not errors, errors
     assert not any(th.is_alive() for th in threads)
+
+
+@pytest.mark.parametrize("same_stream,blocking", [("1", "0"), ("0", "1"), ("1", "1")])
+def test_env_switches(monkeypatch, same_stream, blocking):
+    monkeypatch.setenv("CCL_SAME_STREAM", same_stream)
+    monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
+    _spawn(2, "env")

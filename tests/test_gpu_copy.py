@@ -180,3 +180,14 @@ def test_moe_dispatch_small(mccl):
     want = O.alltoallv([t.view(torch.int16).numpy() for t in ins], S, hidden * 2)
     for d in range(n):
         assert_bits_equal(_np(dev_out[d]), want[d], "moe dest %d" % d)
+
+
+def test_copy_segment_larger_than_4gib(mccl):
+    """One 4 GiB + 3 byte segment with a misaligned start: 64-bit offsets inside a segment."""
+    nbytes = (1 << 32) + 3
+    src = torch.arange(253, dtype=torch.uint8, device=DEV).repeat(nbytes // 253 + 2)[:nbytes + 16]
+    dst = torch.zeros(nbytes + 32, dtype=torch.uint8, device=DEV)
+    mccl.copy_segments([(src.data_ptr() + 5, dst.data_ptr() + 5, nbytes)])
+    torch.cuda.synchronize()
+    assert torch.equal(dst[5:5 + nbytes], src[5:5 + nbytes])
+    assert int(dst[:5].sum()) == 0 and int(dst[5 + nbytes:].sum()) == 0

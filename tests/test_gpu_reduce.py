@@ -311,3 +311,40 @@ def test_reduce_and_copy_replay_from_a_hip_graph(mccl):
         assert_bits_equal(bits(out), bits(want), "graph replay %d" % it)
         assert_bits_equal(bits(out), oracle_reduce_bits([t.cpu() for t in ins]), "graph replay %d vs oracle" % it)
         assert_bits_equal(bits(gathered), np.concatenate([bits(t) for t in ins]), "graph allgather %d" % it)
+
+
+# ---- 64-bit indexing ----
+
+def test_reduce_more_than_4gib_per_buffer(mccl):
+    """Two u8 buffers of 2^32 + 1000 elements: element indices and byte offsets exceed 32 bits.
+    Inputs are periodic patterns built on the device; the result is checked with torch ops."""
+    count = (1 << 32) + 1000
+    a = torch.arange(251, dtype=torch.uint8, device=DEV).repeat(count // 251 + 1)[:count]
+    b = torch.arange(241, dtype=torch.uint8, device=DEV).repeat(count // 241 + 1)[:count]
+    out = mccl.reduce_n([a, b], op=O.SUM)
+    torch.cuda.synchronize()
+    for lo in (0, (1 << 31) - 5000, (1 << 32) - 5000, count - 9000):
+        sl = slice(lo, lo + 9000)
+        assert torch.equal(out[sl], a[sl] + b[sl]), "slice at %d" % lo
+    # a checksum over everything (uint8 wrap-around sums, reduced in int64)
+    assert int(out.sum(dtype=torch.int64)) == int((a + b).sum(dtype=torch.int64))
+
+
+def test_reduce_scatter_offsets_beyond_4gib(mccl):
+    """Shard offsets larger than 4 GiB: 6 shards of 1 GiB (bf16) per rank, 2 ranks; the last
+    shard starts 5 GiB into each buffer."""
+    n_shards, m = 6, 1 << 29
+    ins = []
+    for r in range(2):
+        g = torch.Generator(device=DEV).manual_seed(1234 * 1_000_003 + r)
+        x = torch.empty(n_shards * m, dtype=torch.bfloat16, device=DEV)
+        for s in range(n_shards):
+            x[s * m:(s + 1) * m] = (torch.randn(m, generator=g, device=DEV) * 1e-3).to(torch.bfloat16)
+        ins.append(x)
+    out = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    for shard in (0, 5):
+        mccl.reduce_scatter_n(ins, [out], op=O.SUM, shard_first=shard)
+        torch.cuda.synchronize()
+        sl = slice(shard * m, (shard + 1) * m)
+        want = (ins[0][sl].float() + ins[1][sl].float()).to(torch.bfloat16)
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16)), "shard %d" % shard
