@@ -117,6 +117,58 @@ def _gloo_rank(rank, world, store_path, backend, cases, out_path):
     dist.destroy_process_group()
 
 
+def _backend_rank(rank, world, store_path, cases, out_path):
+    """One rank process of the drop-in path: dist.all_reduce through backend "ccl" on cuda:0."""
+    os.dup2(2, 1)
+    sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
+    import torch
+    import torch.distributed as dist
+    import torch_ccl_amd  # noqa: F401
+    torch.cuda.set_device(0)
+    dist.init_process_group("ccl", store=dist.FileStore(store_path, world), rank=rank, world_size=world)
+    res = {}
+    for name, count, warm, iters in cases:
+        g = rank_generator(torch, SEED, rank)
+        x = (torch.randn(count, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to("cuda:0")
+        t = x.clone()
+        for _ in range(warm):
+            dist.all_reduce(t)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(iters):
+            t.copy_(x)
+            torch.cuda.synchronize()
+            dist.barrier()
+            t0 = time.perf_counter()
+            dist.all_reduce(t)
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters}
+    if rank == 0:
+        with open(out_path, "w") as f:
+            json.dump(res, f)
+    dist.destroy_process_group()
+
+
+def backend_path(world=8):
+    """The drop-in c10d path end to end: `world` rank processes share cuda:0; every all_reduce is
+    copy-in + host barrier + the local-reduce kernel, timed on the host around the call."""
+    import tempfile
+    import torch.multiprocessing as mp
+    cases = [("c2_256KiB_bf16", 16 * 8192, 20, 200), ("c3_64MiB_bf16", 4096 * 8192, 3, 20)]
+    with tempfile.TemporaryDirectory() as d:
+        out_path = os.path.join(d, "res.json")
+        mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path), nprocs=world, join=True)
+        with open(out_path) as f:
+            res = json.load(f)
+    out = {"processes": world, "note": "host-timed dist.all_reduce incl. copy-in, host barrier, kernel and "
+                                       "synchronize; all ranks run their kernels on the one GPU concurrently"}
+    for name, count, warm, iters in cases:
+        out[name] = {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()}
+    return out
+
+
 def gloo_baseline(world=8):
     """N host processes running the same allreduce through a CPU c10d backend: the reference's
     "ccl" backend when its wheel is installed, else gloo (the stand-in the reference's own CPU
@@ -151,7 +203,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,moe,variants,gloo,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,moe,variants,gloo,backend,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -162,7 +214,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,moe,variants,gloo".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,moe,variants,gloo,backend".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import torch
@@ -426,6 +478,16 @@ def main():
         except Exception as e:  # reported baseline only: never fails the benchmark
             result["cpu_c10d_baseline"] = {"error": repr(e)[:300]}
             log("CPU c10d baseline failed:", repr(e)[:300])
+
+    # ---------------- the drop-in c10d path (8 rank processes on the one GPU) ----------------
+    if "backend" in extras:
+        try:
+            torch.cuda.empty_cache()
+            result["c10d_backend_path"] = backend_path(N)
+            log("c10d backend:", json.dumps(result["c10d_backend_path"]))
+        except Exception as e:  # informational: never fails the benchmark
+            result["c10d_backend_path"] = {"error": repr(e)[:300]}
+            log("c10d backend path failed:", repr(e)[:300])
 
     print(json.dumps(result), flush=True)
 

@@ -105,6 +105,15 @@ size_t nbytes(const at::Tensor& t) { return (size_t)t.numel() * t.element_size()
 
 size_t roundUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Device-to-device copy on the compute queue (the library's own segment copy): no DMA-engine
+// round trip for small messages, full copy bandwidth for large ones.
+void copyAsync(void* dst, const void* src, size_t bytes, hipStream_t s) {
+  if (!bytes) return;
+  mccl_segment_t seg{src, dst, bytes};
+  int rc = mccl_copy_segments(&seg, 1, s);
+  TORCH_CHECK(rc == MCCL_OK, "ccl backend: copy-in failed: ", mccl_last_error());
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------------------------
@@ -365,6 +374,7 @@ void ProcessGroupCCL::hostBarrier() {
 // the engine: copy-in, host barrier, data-path kernels
 // ---------------------------------------------------------------------------------------------
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
+  std::lock_guard<std::mutex> lock(mutex_);
   int device = -1;
   for (const auto& t : plan.inputs) if (t.defined()) { device = t.get_device(); break; }
   if (device < 0) for (const auto& t : plan.outputs) if (t.defined()) { device = t.get_device(); break; }
@@ -391,14 +401,20 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     std::cout << os.str() << std::endl;
   }
 
-  void* stage = ensureStage(slot, plan.stage_bytes);
   RankSlot& me = ctl_->slot[rank_];
-  for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
-  if (plan.copy_in) plan.copy_in(stage, s);
-  // This rank's staging buffer must be complete before any peer reads it, and (two collectives
-  // later) every peer must be done reading before it is overwritten: one host barrier per
-  // collective plus the two alternating buffers give both.
-  HIP_CHECK(hipStreamSynchronize(s));
+  try {
+    void* stage = ensureStage(slot, plan.stage_bytes);
+    for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
+    if (plan.copy_in) plan.copy_in(stage, s);
+    // This rank's staging buffer must be complete before any peer reads it, and (two
+    // collectives later) every peer must be done reading before it is overwritten: one host
+    // barrier per collective plus the two alternating buffers give both.
+    HIP_CHECK(hipStreamSynchronize(s));
+  } catch (...) {
+    // this rank will not arrive: tell the peers now instead of letting them run into the timeout
+    me.failed.store(1, std::memory_order_release);
+    throw;
+  }
   hostBarrier();
 
   if (plan.exec) {
@@ -422,7 +438,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
         if (t.defined() && t.has_storage() && t.numel() > 0)
           c10::hip::HIPCachingAllocatorMasqueradingAsCUDA::recordStreamMasqueradingAsCUDA(t.storage().data_ptr(), cs);
   }
-  last_work_ = work;
+  if (coalescing_) last_work_ = work;
   return work;
 }
 
@@ -451,7 +467,11 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::endCoalescing() {
   // Collectives issued between start and end have already been enqueued in order on the
   // communication stream; the last Work covers them all.
   coalescing_ = false;
-  if (last_work_) return last_work_;
+  if (last_work_) {
+    auto w = last_work_;
+    last_work_.reset();
+    return w;
+  }
   return c10::make_intrusive<WorkCCL>(rank_, c10d::OpType::COALESCED, "endCoalescing",
                                       std::vector<at::Tensor>{}, std::vector<at::Tensor>{}, blocking_wait_);
 }
@@ -481,7 +501,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
     p.stage_bytes = (rank_ == root) ? len : 0;
     if (rank_ == root && len)
       p.copy_in = [=](void* stage, hipStream_t s) {
-        HIP_CHECK(hipMemcpyAsync(stage, base, len, hipMemcpyDeviceToDevice, s));
+        copyAsync(stage, base, len, s);
       };
     if (rank_ != root && len)
       p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
@@ -518,7 +538,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
     if (size_ > 1 && len) {  // world == 1: nothing to add (src/gpu/dpcpp_ccl.cpp:752-756)
       p.stage_bytes = len * es;
       p.copy_in = [=](void* stage, hipStream_t s) {
-        HIP_CHECK(hipMemcpyAsync(stage, base, len * es, hipMemcpyDeviceToDevice, s));
+        copyAsync(stage, base, len * es, s);
       };
       const int W = size_;
       p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
@@ -598,7 +618,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
       p.stage_bytes = len;
       const int W = size_;
       p.copy_in = [=](void* stage, hipStream_t s) {
-        HIP_CHECK(hipMemcpyAsync(stage, in, len, hipMemcpyDeviceToDevice, s));
+        copyAsync(stage, in, len, s);
       };
       p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
         std::vector<mccl_segment_t> segs((size_t)W);
@@ -636,7 +656,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   const int W = size_;
   if (mine)
     p.copy_in = [=](void* stage, hipStream_t s) {
-      HIP_CHECK(hipMemcpyAsync(stage, input.data_ptr(), mine, hipMemcpyDeviceToDevice, s));
+      copyAsync(stage, input.data_ptr(), mine, s);
     };
   p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
@@ -727,7 +747,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
       const int me = rank_;
       p.copy_in = [=](void* stage, hipStream_t s) {
         if (len == M) {
-          HIP_CHECK(hipMemcpyAsync(stage, in, M * es * (size_t)W, hipMemcpyDeviceToDevice, s));
+          copyAsync(stage, in, M * es * (size_t)W, s);
         } else {
           std::vector<mccl_segment_t> segs((size_t)W);
           for (int k = 0; k < W; ++k)
@@ -897,7 +917,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
   }
   if (mine)
     p.copy_in = [=](void* stage, hipStream_t s) {
-      HIP_CHECK(hipMemcpyAsync(stage, input.data_ptr(), mine, hipMemcpyDeviceToDevice, s));
+      copyAsync(stage, input.data_ptr(), mine, s);
     };
   p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
     std::vector<size_t> sd((size_t)W);

@@ -25,6 +25,7 @@
 #include <chrono>
 #include <functional>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -153,7 +154,8 @@ class ProcessGroupCCL : public c10d::Backend {
   bool same_stream_ = false;    // CCL_SAME_STREAM
   bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
   bool coalescing_ = false;
-  c10::intrusive_ptr<WorkCCL> last_work_;
+  c10::intrusive_ptr<WorkCCL> last_work_;  // only kept between startCoalescing and endCoalescing
+  std::mutex mutex_;  // one collective of a group at a time (the reference serialises on a global mutex)
 
   bool initialised_ = false;
   int device_ = 0;
