@@ -255,6 +255,45 @@ def env_switch_case(pg, rank, world):
     pg.barrier().wait()
 
 
+def ddp_case(rank, world):
+    """A real caller: DistributedDataParallel over backend "ccl" (the reference's demo/demo.py trains
+    nn.Linear under DDP).  Gradients after backward must equal the average of the per-rank
+    gradients computed without DDP."""
+    import torch.nn as nn
+    from torch.nn.parallel import DistributedDataParallel as DDP
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(64, 128), nn.ReLU(), nn.Linear(128, 10)).to(DEV)
+    ref = nn.Sequential(nn.Linear(64, 128), nn.ReLU(), nn.Linear(128, 10)).to(DEV)
+    ref.load_state_dict(model.state_dict())
+    ddp = DDP(model, device_ids=[0])
+    xs = [torch.randn(32, 64, generator=torch.Generator().manual_seed(100 + r)) for r in range(world)]
+    ys = [torch.randn(32, 10, generator=torch.Generator().manual_seed(200 + r)) for r in range(world)]
+    loss = ((ddp(xs[rank].to(DEV)) - ys[rank].to(DEV)) ** 2).mean()
+    loss.backward()
+    torch.cuda.synchronize()
+    # reference: every rank's gradient on the same weights, averaged in fp32 in rank order
+    grads = None
+    for r in range(world):
+        ref.zero_grad()
+        ((ref(xs[r].to(DEV)) - ys[r].to(DEV)) ** 2).mean().backward()
+        g = [p.grad.detach().clone() for p in ref.parameters()]
+        grads = g if grads is None else [a + b for a, b in zip(grads, g)]
+    for p, g in zip(ddp.module.parameters(), grads):
+        assert torch.allclose(p.grad, g / world, rtol=1e-5, atol=1e-6), float((p.grad - g / world).abs().max())
+    # FSDP-style step: all_gather_into_tensor of parameter shards, reduce_scatter_tensor of gradients
+    flat = torch.cat([p.detach().reshape(-1) for p in ref.parameters()])
+    pad = (-flat.numel()) % world
+    flat = torch.cat([flat, flat.new_zeros(pad)])
+    shard = flat.view(world, -1)[rank].contiguous()
+    full = torch.empty_like(flat)
+    dist.all_gather_into_tensor(full, shard)
+    assert torch.equal(full, flat)
+    gshard = torch.empty_like(shard)
+    dist.reduce_scatter_tensor(gshard, flat * (rank + 1))
+    want = flat.view(world, -1)[rank] * (world * (world + 1) / 2)
+    assert torch.allclose(gshard, want, rtol=1e-6)
+
+
 def run_rank(rank, world, store_path, mode):
     torch.cuda.set_device(0)
     import torch_ccl_amd  # noqa: F401  registers the backend
@@ -263,6 +302,14 @@ def run_rank(rank, world, store_path, mode):
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
             dist_api_cases(rank, world)
+        finally:
+            dist.destroy_process_group()
+        return
+    if mode == "ddp":
+        store = dist.FileStore(store_path, world)
+        dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
+        try:
+            ddp_case(rank, world)
         finally:
             dist.destroy_process_group()
         return

@@ -98,3 +98,8 @@ def test_env_switches(monkeypatch, same_stream, blocking):
     monkeypatch.setenv("CCL_SAME_STREAM", same_stream)
     monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
     _spawn(2, "env")
+
+
+@pytest.mark.parametrize("world", [2, 4])
+def test_ddp_and_fsdp_style_callers(world):
+    _spawn(world, "ddp")
