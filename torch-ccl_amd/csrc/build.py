@@ -41,7 +41,9 @@ def _stale(out, srcs):
 
 def build_kernels(force=False, extra_flags=(), out=KERNEL_LIB):
     os.makedirs(os.path.dirname(out), exist_ok=True)
-    srcs = [KERNEL_SRC, os.path.join(INCLUDE, "mccl.h")]
+    srcs = [KERNEL_SRC, os.path.join(INCLUDE, "mccl.h")] + [
+        os.path.join(HERE, h) for h in ("kernels_common.hpp", "kernels_reduce.hpp", "kernels_copy.hpp",
+                                        "kernels_moe.hpp")]
     if force or _stale(out, srcs):
         cmd = [HIPCC] + HIP_FLAGS + list(extra_flags) + ["-o", out, KERNEL_SRC]
         subprocess.check_call(cmd)

@@ -1,0 +1,81 @@
+// Segmented copy kernel: the data movement of allgather / alltoall(v) (ccl::allgatherv,
+// ccl::alltoall(v): src/gpu/dpcpp_ccl.cpp:1176-1182, 1403-1455) and of the pack / unpack loops
+// (src/gpu/dpcpp_ccl.cpp:1505-1538).
+#pragma once
+
+#include "kernels_common.hpp"
+
+namespace {
+
+// One segment as the kernel sees it.  The host splits it into a head (bytes up to the first
+// 16- or 4-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of
+// `last` bytes, so that the device needs 32-bit uniform arithmetic only.
+struct CopySeg {
+  const char* src;
+  char* dst;
+  uint32_t head;   // bytes before the body
+  uint32_t nfull;  // full chunks in the body
+  uint32_t last;   // bytes of the final partial chunk (0 = none)
+  uint32_t mode;   // 0: 16-byte vectors, 1: dwords, 2: bytes
+};
+
+struct CopyArgs {
+  CopySeg seg[kMaxSegs];
+  uint32_t chunk_prefix[kMaxSegs + 1];  // exclusive prefix sum of chunks per segment
+  int nseg;
+};
+
+// Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
+// handed out in order.  When src and dst are congruent mod 16 the body moves as 16-byte
+// vectors (non-temporal both ways for full chunks), mod 4 as dwords, else as bytes.
+__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
+  const uint32_t total = a.chunk_prefix[a.nseg];
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    // binary search: largest s with chunk_prefix[s] <= chunk
+    int lo = 0, hi = a.nseg;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    const uint32_t c = chunk - a.chunk_prefix[lo];
+    const uint32_t head = a.seg[lo].head;
+    const uint32_t nfull = a.seg[lo].nfull;
+    const uint32_t mode = a.seg[lo].mode;
+    const uint32_t len = (c < nfull) ? (uint32_t)kCopyChunk : a.seg[lo].last;
+    const uint32_t t = threadIdx.x;
+    const char* src = a.seg[lo].src;
+    char* dst = a.seg[lo].dst;
+    if (c == 0 && t < head) dst[t] = src[t];
+    const size_t off = (size_t)head + (size_t)c * kCopyChunk;  // start of this chunk
+    src += off;
+    dst += off;
+
+    if (mode == 0) {
+      const u32x4* sv = (const u32x4*)src;
+      u32x4* dv = (u32x4*)dst;
+      if (len == (uint32_t)kCopyChunk) {
+        u32x4 x[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      } else {
+        const uint32_t nv = len >> 4;
+        for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
+        const uint32_t rem = len & 15u;
+        if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
+      }
+    } else if (mode == 1) {
+      const uint32_t* sw = (const uint32_t*)src;
+      uint32_t* dw = (uint32_t*)dst;
+      const uint32_t nw = len >> 2;
+      for (uint32_t v = t; v < nw; v += kWave) dw[v] = sw[v];
+      const uint32_t rem = len & 3u;
+      if (t < rem) dst[(nw << 2) + t] = src[(nw << 2) + t];
+    } else {
+      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
+    }
+  }
+}
+
+}  // namespace

@@ -1,0 +1,200 @@
+// Row gather (token permute), fused MoE dispatch and weighted combine: the callers' steps either
+// side of the all_to_all_single of src/gpu/dpcpp_ccl.cpp:1428-1455 (no kernel of the reference).
+#pragma once
+
+#include "kernels_common.hpp"
+
+namespace {
+
+// One gather segment: dst row j = src row idx[j], j < nrows.  Rows are row_bytes long.
+struct GatherSeg {
+  const char* src;
+  const int64_t* idx;
+  char* dst;
+  uint32_t nrows;
+  uint32_t src_rows;  // rows with idx outside [0, src_rows) are skipped (left untouched)
+};
+
+struct GatherArgs {
+  GatherSeg seg[kMaxSegs];
+  uint32_t chunk_prefix[kMaxSegs + 1];  // chunks = nrows * pieces_per_row
+  int nseg;
+  uint32_t row_bytes;
+  uint32_t pieces_per_row;  // ceil(row_bytes / kCopyChunk)
+  uint32_t vector_ok;       // all bases 16-byte aligned and row_bytes % 16 == 0
+};
+
+// One wavefront moves one 2 KiB piece of one row.  Chunks are numbered row-major within a
+// segment and handed out in order, so the destination is written as a compact moving window;
+// the sources are whole rows (contiguous row_bytes each).
+__global__ __launch_bounds__(kWave) void gather_rows_kernel(const GatherArgs a) {
+  const uint32_t total = a.chunk_prefix[a.nseg];
+  const uint32_t ppr = a.pieces_per_row;
+  const uint32_t row_bytes = a.row_bytes;
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    int lo = 0, hi = a.nseg;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    const uint32_t lc = chunk - a.chunk_prefix[lo];
+    const uint32_t row = lc / ppr;
+    const uint32_t piece = lc - row * ppr;
+    const int64_t srow = a.seg[lo].idx[row];
+    if (srow < 0 || srow >= (int64_t)a.seg[lo].src_rows) continue;
+    const uint32_t off = piece * (uint32_t)kCopyChunk;
+    const uint32_t left = row_bytes - off;
+    const uint32_t len = left < (uint32_t)kCopyChunk ? left : (uint32_t)kCopyChunk;
+    const char* src = a.seg[lo].src + (size_t)srow * row_bytes + off;
+    char* dst = a.seg[lo].dst + (size_t)row * row_bytes + off;
+    const uint32_t t = threadIdx.x;
+    if (a.vector_ok) {
+      const u32x4* sv = (const u32x4*)src;
+      u32x4* dv = (u32x4*)dst;
+      if (len == (uint32_t)kCopyChunk) {
+        u32x4 x[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) x[u] = sv[t + u * kWave];  // rows are re-read (top-k): cacheable
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      } else {
+        const uint32_t nv = len >> 4;
+        for (uint32_t v = t; v < nv; v += kWave) __builtin_nontemporal_store(sv[v], &dv[v]);
+      }
+    } else {
+      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
+    }
+  }
+}
+
+// Weighted combine: y[t][c] = sum_k w[t][k] * x[rank(t,k)][row(t,k)][c], fp32 chain from +0 in
+// ascending k, every product rounded before it is added, one rounding on store.
+struct CombineArgs {
+  const char* x[MCCL_MAX_RANKS];
+  uint32_t x_rows[MCCL_MAX_RANKS];
+  const int32_t* src_rank;
+  const int64_t* src_row;
+  const float* w;
+  char* y;
+  uint32_t tokens;
+  uint32_t topk;
+  uint32_t row_vecs;        // 16-byte vectors per row
+  uint32_t pieces_per_row;  // ceil(row_vecs / 64)
+  uint32_t pieces_per_wave; // 1 KiB pieces one wavefront walks (routing entries are looked up once)
+  uint32_t waves_per_row;   // ceil(pieces_per_row / pieces_per_wave)
+  int n;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a) {
+  using A = float;
+  constexpr int VE = vec_elems<DT>();
+  constexpr int G = 8;  // row loads in flight per lane (one group covers top-8 routing)
+  const uint32_t total = a.tokens * a.waves_per_row;
+  const size_t row_stride = (size_t)a.row_vecs * 16;
+  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+    const uint32_t tok = chunk / a.waves_per_row;
+    const uint32_t part = chunk - tok * a.waves_per_row;
+    const uint32_t p0 = part * a.pieces_per_wave;
+    const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
+    const size_t e0 = (size_t)tok * a.topk;
+    if (a.topk <= G) {
+      // routing entries looked up once for all pieces this wavefront walks
+      int rk[G];
+      int64_t rw[G];
+      float wk[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool in = (uint32_t)g < a.topk;
+        rk[g] = in ? a.src_rank[e0 + g] : -1;
+        rw[g] = in ? a.src_row[e0 + g] : 0;
+        wk[g] = in ? a.w[e0 + g] : 0.0f;
+      }
+      const u32x4* src[G];
+      bool ok[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const bool rank_ok = rk[g] >= 0 && rk[g] < a.n;
+        const int r = rank_ok ? rk[g] : 0;
+        ok[g] = rank_ok && rw[g] >= 0 && rw[g] < (int64_t)a.x_rows[r];
+        src[g] = (const u32x4*)(a.x[r] + (ok[g] ? (size_t)rw[g] : 0) * row_stride);
+      }
+      for (uint32_t piece = p0; piece < p1; ++piece) {
+        const uint32_t v = piece * kWave + threadIdx.x;
+        const bool live = v < a.row_vecs;
+        VecU<DT> x[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          x[g].v = (u32x4){0u, 0u, 0u, 0u};
+          if (ok[g] && live) x[g].v = __builtin_nontemporal_load(src[g] + v);
+        }
+        A acc[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if (ok[g]) {
+#pragma unroll
+            for (int e = 0; e < VE; ++e) {
+              const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
+              acc[e] = acc[e] + prod;
+            }
+          }
+        }
+        if (live) {
+          VecU<DT> r;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
+          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
+        }
+      }
+    } else {
+      // general top-k: groups of G entries per piece
+      for (uint32_t piece = p0; piece < p1; ++piece) {
+        const uint32_t v = piece * kWave + threadIdx.x;
+        const bool live = v < a.row_vecs;
+        A acc[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
+        for (uint32_t kb = 0; kb < a.topk; kb += G) {
+          VecU<DT> x[G];
+          float wk[G];
+          bool ok[G];
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            ok[g] = false;
+            wk[g] = 0.0f;
+            x[g].v = (u32x4){0u, 0u, 0u, 0u};
+            if (kb + g < a.topk) {
+              const int r = a.src_rank[e0 + kb + g];
+              const int64_t row = a.src_row[e0 + kb + g];
+              if (r >= 0 && r < a.n && row >= 0 && row < (int64_t)a.x_rows[r]) {
+                ok[g] = true;
+                wk[g] = a.w[e0 + kb + g];
+                if (live) x[g].v = __builtin_nontemporal_load((const u32x4*)(a.x[r] + (size_t)row * row_stride) + v);
+              }
+            }
+          }
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            if (ok[g]) {
+#pragma unroll
+              for (int e = 0; e < VE; ++e) {
+                const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
+                acc[e] = acc[e] + prod;
+              }
+            }
+          }
+        }
+        if (live) {
+          VecU<DT> r;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
+          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
+        }
+      }
+    }
+  }
+}
+
+}  // namespace

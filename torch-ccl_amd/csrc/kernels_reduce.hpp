@@ -1,0 +1,184 @@
+// N-buffer reduction kernels (allreduce local-reduce, reduce_scatter shard reduction, coalesced
+// reductions).  What they replace in the reference: the N-peer sum of
+// src/gpu/allreduce_small.h:289-361, the five data kernels of src/gpu/allreduce.h:306-533 and the
+// ccl::allreduce / ccl::reduce_scatter call sites of src/gpu/dpcpp_ccl.cpp:781-788, 1002-1008.
+#pragma once
+
+#include "kernels_common.hpp"
+
+namespace {
+
+// One reduction of a launch, fully described by the host so that a wavefront needs one
+// scalar load to start and 32-bit uniform arithmetic only:
+//   elements [0, head)                      peeled, element-wise (out not yet 16-byte aligned)
+//   vectors  [0, nvec) at byte offset head*es   the vector body
+//   elements [head + nvec*VE, +tail)        peeled, element-wise
+struct ReduceJob {
+  char* out;
+  size_t in_off;   // byte offset applied to every input pointer
+  size_t nvec;     // 16-byte vectors in the body
+  uint32_t head;   // elements before the body (< 16)
+  uint32_t tail;   // elements after the body (< 16)
+};
+
+// Kernel arguments.  reduce_n: one job.  reduce_scatter: one job per shard, same pointers,
+// different byte offsets.  reduce_multi (OWN == true kernels): job j reads the n pointers
+// starting at ptr[job_ptr0[j]].
+struct ReduceArgs {
+  const char* ptr[MCCL_MAX_RANKS];
+  ReduceJob job[kMaxJobs];
+  int job_ptr0[kMaxJobs];
+  int n;
+};
+
+// Element-wise reduction of one element (used for peeled heads/tails and the misaligned path).
+template <int DT, int OP>
+__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, int n, size_t in_off,
+                                           char* out, size_t idx) {
+  using S = typename Elem<DT>::store_t;
+  using A = typename Elem<DT>::acc_t;
+  A acc = chain_first<DT, OP>(Elem<DT>::load(((const S*)(a.ptr[p0] + in_off))[idx]));
+  for (int k = 1; k < n; ++k)
+    acc = chain_next<DT, OP>(acc, Elem<DT>::load(((const S*)(a.ptr[p0 + k] + in_off))[idx]));
+  acc = chain_last<DT, OP>(acc, n);
+  ((S*)out)[idx] = Elem<DT>::store(acc);
+}
+
+// Loads one 16-byte vector; GUARD adds the bounds check of the last, partial tile.
+template <bool GUARD>
+__device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec) {
+  if constexpr (GUARD) {
+    if (v >= nvec) return (u32x4){0u, 0u, 0u, 0u};
+  }
+  return __builtin_nontemporal_load(&p[v]);  // streamed once: keep it out of the caches
+}
+
+// One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
+// ascending-rank chain in registers and streams the result out.
+// NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
+// NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
+template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD>
+__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t in_byte_off,
+                                            u32x4* ov, size_t v0, size_t nvec, int n) {
+  using A = typename Elem<DT>::acc_t;
+  constexpr int VE = vec_elems<DT>();
+  A acc[U][VE];
+
+  if constexpr (NT > 0) {
+    VecU<DT> x[NT][U];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) {
+      const u32x4* iv = (const u32x4*)(a.ptr[p0 + k] + in_byte_off);
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[k][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x[0][u].e[e]));
+#pragma unroll
+      for (int k = 1; k < NT; ++k)
+#pragma unroll
+        for (int e = 0; e < VE; ++e)
+          acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[k][u].e[e]));
+    }
+  } else {
+    {
+      const u32x4* iv = (const u32x4*)(a.ptr[p0] + in_byte_off);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        VecU<DT> x;
+        x.v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x.e[e]));
+      }
+    }
+    constexpr int G = 4;
+    for (int kb = 1; kb < n; kb += G) {
+      VecU<DT> x[G][U];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        if (kb + g < n) {
+          const u32x4* iv = (const u32x4*)(a.ptr[p0 + kb + g] + in_byte_off);
+#pragma unroll
+          for (int u = 0; u < U; ++u) x[g][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        if (kb + g < n) {
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < VE; ++e)
+              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[g][u].e[e]));
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const size_t v = v0 + (size_t)u * BLOCK;
+    if (!GUARD || v < nvec) {
+      VecU<DT> r;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(chain_last<DT, OP>(acc[u][e], n));
+      __builtin_nontemporal_store(r.v, &ov[v]);
+    }
+  }
+}
+
+// Vector kernel.  Requires, for each job, all input pointers (+offset) and the output
+// pointer congruent mod 16.  The output may be exactly one of the inputs: a lane reads
+// element i of every input before it writes element i, and no other lane touches i.
+// OWN: each job has its own n pointers (coalesced reductions); otherwise all jobs share
+// ptr[0..n) and the pointer loads do not wait for the job record.
+template <int DT, int OP, int NT, int U, int BLOCK, bool OWN>
+__global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
+  using S = typename Elem<DT>::store_t;
+  constexpr int VE = vec_elems<DT>();
+  const int jid = blockIdx.y;
+  const int p0 = OWN ? a.job_ptr0[jid] : 0;
+  const int n = (NT > 0) ? NT : a.n;
+  char* out = a.job[jid].out;
+  const size_t in_off = a.job[jid].in_off;
+  const size_t nvec = a.job[jid].nvec;
+  const uint32_t head = a.job[jid].head;
+  const uint32_t tail = a.job[jid].tail;
+
+  if (blockIdx.x == 0) {
+    const uint32_t t = threadIdx.x;
+    if (t < head) reduce_one<DT, OP>(a, p0, n, in_off, out, t);
+    else if (t - head < tail) reduce_one<DT, OP>(a, p0, n, in_off, out, head + nvec * VE + (t - head));
+  }
+
+  const size_t body_off = (size_t)head * sizeof(S);  // bytes
+  u32x4* ov = (u32x4*)(out + body_off);
+  constexpr uint32_t TILE = (uint32_t)BLOCK * U;
+  // the host keeps nvec / TILE below 2^32
+  const uint32_t full_tiles = (uint32_t)(nvec / TILE);
+  const uint32_t partial = (uint32_t)(nvec % TILE) ? 1u : 0u;
+
+  uint32_t tile = blockIdx.x;
+  for (; tile < full_tiles; tile += gridDim.x)
+    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
+  if (tile == full_tiles && partial)  // the one partial tile; exactly one workgroup reaches it
+    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
+}
+
+// Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
+// multiple of the element size).  Grid-stride over elements.
+template <int DT, int OP, bool OWN>
+__global__ __launch_bounds__(256) void reduce_elem_kernel(const ReduceArgs a) {
+  const int jid = blockIdx.y;
+  const int p0 = OWN ? a.job_ptr0[jid] : 0;
+  const size_t in_off = a.job[jid].in_off;
+  char* out = a.job[jid].out;
+  const size_t count = a.job[jid].nvec;  // element count for this kernel
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
+    reduce_one<DT, OP>(a, p0, a.n, in_off, out, i);
+}
+
+}  // namespace

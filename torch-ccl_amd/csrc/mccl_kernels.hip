@@ -1,5 +1,6 @@
-// libmi355ccl: local-reduce and segmented-copy kernels for gfx950 (MI355X) and the C ABI
-// declared in include/mccl.h.
+// libmi355ccl: launch planning and the C ABI declared in include/mccl.h.  The device code is in
+// kernels_common.hpp (element types, the reduction chain), kernels_reduce.hpp, kernels_copy.hpp
+// and kernels_moe.hpp.
 //
 // Everything here is HBM-bandwidth bound.  Design rules:
 //   * one 16-byte vector per lane per input, so a wavefront reads 1 KiB contiguous from
@@ -42,6 +43,11 @@
 
 #include "mccl.h"
 
+#include "kernels_common.hpp"
+#include "kernels_copy.hpp"
+#include "kernels_moe.hpp"
+#include "kernels_reduce.hpp"
+
 namespace {
 
 // ------------------------------------------------------------------------------------------
@@ -68,13 +74,6 @@ int fail(int code, const char* fmt, ...) {
 // ------------------------------------------------------------------------------------------
 // tuning state and per-device facts
 // ------------------------------------------------------------------------------------------
-constexpr int kWave = 64;               // one wavefront per workgroup (small / stream shapes)
-constexpr int kBlockPersistent = 256;   // 4 wavefronts
-constexpr int kUnrollPersistent = 2;    // vectors per lane per input per tile
-constexpr int kMaxJobs = 64;            // independent reductions per launch
-constexpr int kMaxSegs = 64;            // copy segments per launch
-constexpr int kCopyUnroll = 2;          // vectors per lane per chunk
-constexpr size_t kCopyChunk = (size_t)kWave * 16 * kCopyUnroll;  // 2 KiB per wavefront
 constexpr unsigned kMaxGridX = 1u << 24;  // larger messages wrap through the grid-stride loop
 constexpr size_t kLdsPerCu = 160 * 1024;  // gfx950
 constexpr int kMaxWavesPerCu = 32;
@@ -119,564 +118,6 @@ int device_cus(int* cus_out) {
   if (err != hipSuccess) return fail(MCCL_ERR_HIP, "hipDeviceGetAttribute failed: %s", hipGetErrorString(err));
   *cus_out = g_facts[dev].cus;
   return MCCL_OK;
-}
-
-// ------------------------------------------------------------------------------------------
-// element types
-// ------------------------------------------------------------------------------------------
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
-__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
-
-template <int DT>
-struct Elem;
-
-template <>
-struct Elem<MCCL_BF16> {
-  using store_t = uint16_t;
-  using acc_t = float;
-  static constexpr bool kIsFloat = true;
-  static __device__ __forceinline__ acc_t load(store_t h) { return bits_to_f32((uint32_t)h << 16); }
-  // round to nearest even; every NaN becomes 0x7FC0
-  static __device__ __forceinline__ store_t store(acc_t f) {
-    uint32_t u = f32_to_bits(f);
-    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    return (store_t)(((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : r);
-  }
-};
-
-template <>
-struct Elem<MCCL_F16> {
-  using store_t = uint16_t;
-  using acc_t = float;
-  static constexpr bool kIsFloat = true;
-  static __device__ __forceinline__ acc_t load(store_t h) {
-    return (float)__builtin_bit_cast(_Float16, h);
-  }
-  // hardware convert is round-to-nearest-even with gradual underflow; NaN -> 0x7E00
-  static __device__ __forceinline__ store_t store(acc_t f) {
-    uint16_t r = __builtin_bit_cast(uint16_t, (_Float16)f);
-    return (f != f) ? (store_t)0x7e00u : r;
-  }
-};
-
-template <typename T, typename UT, int CODE>
-struct IntElem {
-  using store_t = T;
-  using acc_t = T;
-  using uacc_t = UT;
-  static constexpr bool kIsFloat = false;
-  static __device__ __forceinline__ acc_t load(store_t v) { return v; }
-  static __device__ __forceinline__ store_t store(acc_t v) { return v; }
-};
-template <> struct Elem<MCCL_U8> : IntElem<uint8_t, uint8_t, MCCL_U8> {};
-template <> struct Elem<MCCL_I8> : IntElem<int8_t, uint8_t, MCCL_I8> {};
-template <> struct Elem<MCCL_I16> : IntElem<int16_t, uint16_t, MCCL_I16> {};
-template <> struct Elem<MCCL_I32> : IntElem<int32_t, uint32_t, MCCL_I32> {};
-template <> struct Elem<MCCL_I64> : IntElem<int64_t, uint64_t, MCCL_I64> {};
-
-template <typename T>
-struct FloatElem {
-  using store_t = T;
-  using acc_t = T;
-  static constexpr bool kIsFloat = true;
-  static __device__ __forceinline__ acc_t load(store_t v) { return v; }
-  static __device__ __forceinline__ store_t store(acc_t v) { return v; }
-};
-template <> struct Elem<MCCL_F32> : FloatElem<float> {};
-template <> struct Elem<MCCL_F64> : FloatElem<double> {};
-
-// ------------------------------------------------------------------------------------------
-// the reduction chain
-// ------------------------------------------------------------------------------------------
-// First element of the chain.  SUM/AVG start from literal +0 and add rank 0 (so an all -0
-// column yields +0, as "result = 0; result = result + buf[r]" does); the other ops start
-// from rank 0's value.
-template <int DT, int OP>
-__device__ __forceinline__ typename Elem<DT>::acc_t chain_first(typename Elem<DT>::acc_t x) {
-  using A = typename Elem<DT>::acc_t;
-  if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {
-    if constexpr (Elem<DT>::kIsFloat) return (A)0 + x;
-    else return x;
-  } else {
-    return x;
-  }
-}
-
-template <int DT, int OP>
-__device__ __forceinline__ typename Elem<DT>::acc_t chain_next(typename Elem<DT>::acc_t acc,
-                                                                typename Elem<DT>::acc_t x) {
-  using A = typename Elem<DT>::acc_t;
-  if constexpr (Elem<DT>::kIsFloat) {
-    if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) return acc + x;
-    else if constexpr (OP == MCCL_PROD) return acc * x;
-    else if constexpr (OP == MCCL_MIN) return (x < acc) ? x : acc;
-    else return (x > acc) ? x : acc;
-  } else {
-    using U = typename Elem<DT>::uacc_t;
-    if constexpr (OP == MCCL_SUM) return (A)(U)((U)acc + (U)x);
-    else if constexpr (OP == MCCL_PROD) return (A)(U)((U)acc * (U)x);
-    else if constexpr (OP == MCCL_MIN) return (x < acc) ? x : acc;
-    else return (x > acc) ? x : acc;
-  }
-}
-
-template <int DT, int OP>
-__device__ __forceinline__ typename Elem<DT>::acc_t chain_last(typename Elem<DT>::acc_t acc, int n) {
-  using A = typename Elem<DT>::acc_t;
-  if constexpr (OP == MCCL_AVG) return acc / (A)n;
-  else return acc;
-}
-
-// One reduction of a launch, fully described by the host so that a wavefront needs one
-// scalar load to start and 32-bit uniform arithmetic only:
-//   elements [0, head)                      peeled, element-wise (out not yet 16-byte aligned)
-//   vectors  [0, nvec) at byte offset head*es   the vector body
-//   elements [head + nvec*VE, +tail)        peeled, element-wise
-struct ReduceJob {
-  char* out;
-  size_t in_off;   // byte offset applied to every input pointer
-  size_t nvec;     // 16-byte vectors in the body
-  uint32_t head;   // elements before the body (< 16)
-  uint32_t tail;   // elements after the body (< 16)
-};
-
-// Kernel arguments.  reduce_n: one job.  reduce_scatter: one job per shard, same pointers,
-// different byte offsets.  reduce_multi (OWN == true kernels): job j reads the n pointers
-// starting at ptr[job_ptr0[j]].
-struct ReduceArgs {
-  const char* ptr[MCCL_MAX_RANKS];
-  ReduceJob job[kMaxJobs];
-  int job_ptr0[kMaxJobs];
-  int n;
-};
-
-template <int DT>
-constexpr int vec_elems() { return 16 / (int)sizeof(typename Elem<DT>::store_t); }
-
-template <int DT>
-union VecU {
-  u32x4 v;
-  typename Elem<DT>::store_t e[vec_elems<DT>()];
-};
-
-// Element-wise reduction of one element (used for peeled heads/tails and the misaligned path).
-template <int DT, int OP>
-__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, int n, size_t in_off,
-                                           char* out, size_t idx) {
-  using S = typename Elem<DT>::store_t;
-  using A = typename Elem<DT>::acc_t;
-  A acc = chain_first<DT, OP>(Elem<DT>::load(((const S*)(a.ptr[p0] + in_off))[idx]));
-  for (int k = 1; k < n; ++k)
-    acc = chain_next<DT, OP>(acc, Elem<DT>::load(((const S*)(a.ptr[p0 + k] + in_off))[idx]));
-  acc = chain_last<DT, OP>(acc, n);
-  ((S*)out)[idx] = Elem<DT>::store(acc);
-}
-
-// Loads one 16-byte vector; GUARD adds the bounds check of the last, partial tile.
-template <bool GUARD>
-__device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec) {
-  if constexpr (GUARD) {
-    if (v >= nvec) return (u32x4){0u, 0u, 0u, 0u};
-  }
-  return __builtin_nontemporal_load(&p[v]);  // streamed once: keep it out of the caches
-}
-
-// One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
-// ascending-rank chain in registers and streams the result out.
-// NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
-// NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
-template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD>
-__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t in_byte_off,
-                                            u32x4* ov, size_t v0, size_t nvec, int n) {
-  using A = typename Elem<DT>::acc_t;
-  constexpr int VE = vec_elems<DT>();
-  A acc[U][VE];
-
-  if constexpr (NT > 0) {
-    VecU<DT> x[NT][U];
-#pragma unroll
-    for (int k = 0; k < NT; ++k) {
-      const u32x4* iv = (const u32x4*)(a.ptr[p0 + k] + in_byte_off);
-#pragma unroll
-      for (int u = 0; u < U; ++u) x[k][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x[0][u].e[e]));
-#pragma unroll
-      for (int k = 1; k < NT; ++k)
-#pragma unroll
-        for (int e = 0; e < VE; ++e)
-          acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[k][u].e[e]));
-    }
-  } else {
-    {
-      const u32x4* iv = (const u32x4*)(a.ptr[p0] + in_byte_off);
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        VecU<DT> x;
-        x.v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x.e[e]));
-      }
-    }
-    constexpr int G = 4;
-    for (int kb = 1; kb < n; kb += G) {
-      VecU<DT> x[G][U];
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        if (kb + g < n) {
-          const u32x4* iv = (const u32x4*)(a.ptr[p0 + kb + g] + in_byte_off);
-#pragma unroll
-          for (int u = 0; u < U; ++u) x[g][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        if (kb + g < n) {
-#pragma unroll
-          for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int e = 0; e < VE; ++e)
-              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[g][u].e[e]));
-        }
-      }
-    }
-  }
-
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const size_t v = v0 + (size_t)u * BLOCK;
-    if (!GUARD || v < nvec) {
-      VecU<DT> r;
-#pragma unroll
-      for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(chain_last<DT, OP>(acc[u][e], n));
-      __builtin_nontemporal_store(r.v, &ov[v]);
-    }
-  }
-}
-
-// Vector kernel.  Requires, for each job, all input pointers (+offset) and the output
-// pointer congruent mod 16.  The output may be exactly one of the inputs: a lane reads
-// element i of every input before it writes element i, and no other lane touches i.
-// OWN: each job has its own n pointers (coalesced reductions); otherwise all jobs share
-// ptr[0..n) and the pointer loads do not wait for the job record.
-template <int DT, int OP, int NT, int U, int BLOCK, bool OWN>
-__global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
-  using S = typename Elem<DT>::store_t;
-  constexpr int VE = vec_elems<DT>();
-  const int jid = blockIdx.y;
-  const int p0 = OWN ? a.job_ptr0[jid] : 0;
-  const int n = (NT > 0) ? NT : a.n;
-  char* out = a.job[jid].out;
-  const size_t in_off = a.job[jid].in_off;
-  const size_t nvec = a.job[jid].nvec;
-  const uint32_t head = a.job[jid].head;
-  const uint32_t tail = a.job[jid].tail;
-
-  if (blockIdx.x == 0) {
-    const uint32_t t = threadIdx.x;
-    if (t < head) reduce_one<DT, OP>(a, p0, n, in_off, out, t);
-    else if (t - head < tail) reduce_one<DT, OP>(a, p0, n, in_off, out, head + nvec * VE + (t - head));
-  }
-
-  const size_t body_off = (size_t)head * sizeof(S);  // bytes
-  u32x4* ov = (u32x4*)(out + body_off);
-  constexpr uint32_t TILE = (uint32_t)BLOCK * U;
-  // the host keeps nvec / TILE below 2^32
-  const uint32_t full_tiles = (uint32_t)(nvec / TILE);
-  const uint32_t partial = (uint32_t)(nvec % TILE) ? 1u : 0u;
-
-  uint32_t tile = blockIdx.x;
-  for (; tile < full_tiles; tile += gridDim.x)
-    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
-  if (tile == full_tiles && partial)  // the one partial tile; exactly one workgroup reaches it
-    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
-}
-
-// Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
-// multiple of the element size).  Grid-stride over elements.
-template <int DT, int OP, bool OWN>
-__global__ __launch_bounds__(256) void reduce_elem_kernel(const ReduceArgs a) {
-  const int jid = blockIdx.y;
-  const int p0 = OWN ? a.job_ptr0[jid] : 0;
-  const size_t in_off = a.job[jid].in_off;
-  char* out = a.job[jid].out;
-  const size_t count = a.job[jid].nvec;  // element count for this kernel
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
-    reduce_one<DT, OP>(a, p0, a.n, in_off, out, i);
-}
-
-// ------------------------------------------------------------------------------------------
-// segmented copy
-// ------------------------------------------------------------------------------------------
-// One segment as the kernel sees it.  The host splits it into a head (bytes up to the first
-// 16- or 4-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of
-// `last` bytes, so that the device needs 32-bit uniform arithmetic only.
-struct CopySeg {
-  const char* src;
-  char* dst;
-  uint32_t head;   // bytes before the body
-  uint32_t nfull;  // full chunks in the body
-  uint32_t last;   // bytes of the final partial chunk (0 = none)
-  uint32_t mode;   // 0: 16-byte vectors, 1: dwords, 2: bytes
-};
-
-struct CopyArgs {
-  CopySeg seg[kMaxSegs];
-  uint32_t chunk_prefix[kMaxSegs + 1];  // exclusive prefix sum of chunks per segment
-  int nseg;
-};
-
-// Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
-// handed out in order.  When src and dst are congruent mod 16 the body moves as 16-byte
-// vectors (non-temporal both ways for full chunks), mod 4 as dwords, else as bytes.
-__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
-  const uint32_t total = a.chunk_prefix[a.nseg];
-  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
-    // binary search: largest s with chunk_prefix[s] <= chunk
-    int lo = 0, hi = a.nseg;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
-    }
-    const uint32_t c = chunk - a.chunk_prefix[lo];
-    const uint32_t head = a.seg[lo].head;
-    const uint32_t nfull = a.seg[lo].nfull;
-    const uint32_t mode = a.seg[lo].mode;
-    const uint32_t len = (c < nfull) ? (uint32_t)kCopyChunk : a.seg[lo].last;
-    const uint32_t t = threadIdx.x;
-    const char* src = a.seg[lo].src;
-    char* dst = a.seg[lo].dst;
-    if (c == 0 && t < head) dst[t] = src[t];
-    const size_t off = (size_t)head + (size_t)c * kCopyChunk;  // start of this chunk
-    src += off;
-    dst += off;
-
-    if (mode == 0) {
-      const u32x4* sv = (const u32x4*)src;
-      u32x4* dv = (u32x4*)dst;
-      if (len == (uint32_t)kCopyChunk) {
-        u32x4 x[kCopyUnroll];
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
-      } else {
-        const uint32_t nv = len >> 4;
-        for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
-        const uint32_t rem = len & 15u;
-        if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
-      }
-    } else if (mode == 1) {
-      const uint32_t* sw = (const uint32_t*)src;
-      uint32_t* dw = (uint32_t*)dst;
-      const uint32_t nw = len >> 2;
-      for (uint32_t v = t; v < nw; v += kWave) dw[v] = sw[v];
-      const uint32_t rem = len & 3u;
-      if (t < rem) dst[(nw << 2) + t] = src[(nw << 2) + t];
-    } else {
-      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------
-// row gather (token permute) and the fused MoE dispatch / combine
-// ------------------------------------------------------------------------------------------
-// One gather segment: dst row j = src row idx[j], j < nrows.  Rows are row_bytes long.
-struct GatherSeg {
-  const char* src;
-  const int64_t* idx;
-  char* dst;
-  uint32_t nrows;
-  uint32_t src_rows;  // rows with idx outside [0, src_rows) are skipped (left untouched)
-};
-
-struct GatherArgs {
-  GatherSeg seg[kMaxSegs];
-  uint32_t chunk_prefix[kMaxSegs + 1];  // chunks = nrows * pieces_per_row
-  int nseg;
-  uint32_t row_bytes;
-  uint32_t pieces_per_row;  // ceil(row_bytes / kCopyChunk)
-  uint32_t vector_ok;       // all bases 16-byte aligned and row_bytes % 16 == 0
-};
-
-// One wavefront moves one 2 KiB piece of one row.  Chunks are numbered row-major within a
-// segment and handed out in order, so the destination is written as a compact moving window;
-// the sources are whole rows (contiguous row_bytes each).
-__global__ __launch_bounds__(kWave) void gather_rows_kernel(const GatherArgs a) {
-  const uint32_t total = a.chunk_prefix[a.nseg];
-  const uint32_t ppr = a.pieces_per_row;
-  const uint32_t row_bytes = a.row_bytes;
-  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
-    int lo = 0, hi = a.nseg;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
-    }
-    const uint32_t lc = chunk - a.chunk_prefix[lo];
-    const uint32_t row = lc / ppr;
-    const uint32_t piece = lc - row * ppr;
-    const int64_t srow = a.seg[lo].idx[row];
-    if (srow < 0 || srow >= (int64_t)a.seg[lo].src_rows) continue;
-    const uint32_t off = piece * (uint32_t)kCopyChunk;
-    const uint32_t left = row_bytes - off;
-    const uint32_t len = left < (uint32_t)kCopyChunk ? left : (uint32_t)kCopyChunk;
-    const char* src = a.seg[lo].src + (size_t)srow * row_bytes + off;
-    char* dst = a.seg[lo].dst + (size_t)row * row_bytes + off;
-    const uint32_t t = threadIdx.x;
-    if (a.vector_ok) {
-      const u32x4* sv = (const u32x4*)src;
-      u32x4* dv = (u32x4*)dst;
-      if (len == (uint32_t)kCopyChunk) {
-        u32x4 x[kCopyUnroll];
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) x[u] = sv[t + u * kWave];  // rows are re-read (top-k): cacheable
-#pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
-      } else {
-        const uint32_t nv = len >> 4;
-        for (uint32_t v = t; v < nv; v += kWave) __builtin_nontemporal_store(sv[v], &dv[v]);
-      }
-    } else {
-      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
-    }
-  }
-}
-
-// Weighted combine: y[t][c] = sum_k w[t][k] * x[rank(t,k)][row(t,k)][c], fp32 chain from +0 in
-// ascending k, every product rounded before it is added, one rounding on store.
-struct CombineArgs {
-  const char* x[MCCL_MAX_RANKS];
-  uint32_t x_rows[MCCL_MAX_RANKS];
-  const int32_t* src_rank;
-  const int64_t* src_row;
-  const float* w;
-  char* y;
-  uint32_t tokens;
-  uint32_t topk;
-  uint32_t row_vecs;        // 16-byte vectors per row
-  uint32_t pieces_per_row;  // ceil(row_vecs / 64)
-  uint32_t pieces_per_wave; // 1 KiB pieces one wavefront walks (routing entries are looked up once)
-  uint32_t waves_per_row;   // ceil(pieces_per_row / pieces_per_wave)
-  int n;
-};
-
-template <int DT>
-__global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a) {
-  using A = float;
-  constexpr int VE = vec_elems<DT>();
-  constexpr int G = 8;  // row loads in flight per lane (one group covers top-8 routing)
-  const uint32_t total = a.tokens * a.waves_per_row;
-  const size_t row_stride = (size_t)a.row_vecs * 16;
-  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
-    const uint32_t tok = chunk / a.waves_per_row;
-    const uint32_t part = chunk - tok * a.waves_per_row;
-    const uint32_t p0 = part * a.pieces_per_wave;
-    const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
-    const size_t e0 = (size_t)tok * a.topk;
-    if (a.topk <= G) {
-      // routing entries looked up once for all pieces this wavefront walks
-      int rk[G];
-      int64_t rw[G];
-      float wk[G];
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const bool in = (uint32_t)g < a.topk;
-        rk[g] = in ? a.src_rank[e0 + g] : -1;
-        rw[g] = in ? a.src_row[e0 + g] : 0;
-        wk[g] = in ? a.w[e0 + g] : 0.0f;
-      }
-      const u32x4* src[G];
-      bool ok[G];
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const bool rank_ok = rk[g] >= 0 && rk[g] < a.n;
-        const int r = rank_ok ? rk[g] : 0;
-        ok[g] = rank_ok && rw[g] >= 0 && rw[g] < (int64_t)a.x_rows[r];
-        src[g] = (const u32x4*)(a.x[r] + (ok[g] ? (size_t)rw[g] : 0) * row_stride);
-      }
-      for (uint32_t piece = p0; piece < p1; ++piece) {
-        const uint32_t v = piece * kWave + threadIdx.x;
-        const bool live = v < a.row_vecs;
-        VecU<DT> x[G];
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          x[g].v = (u32x4){0u, 0u, 0u, 0u};
-          if (ok[g] && live) x[g].v = __builtin_nontemporal_load(src[g] + v);
-        }
-        A acc[VE];
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          if (ok[g]) {
-#pragma unroll
-            for (int e = 0; e < VE; ++e) {
-              const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
-              acc[e] = acc[e] + prod;
-            }
-          }
-        }
-        if (live) {
-          VecU<DT> r;
-#pragma unroll
-          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
-          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
-        }
-      }
-    } else {
-      // general top-k: groups of G entries per piece
-      for (uint32_t piece = p0; piece < p1; ++piece) {
-        const uint32_t v = piece * kWave + threadIdx.x;
-        const bool live = v < a.row_vecs;
-        A acc[VE];
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
-        for (uint32_t kb = 0; kb < a.topk; kb += G) {
-          VecU<DT> x[G];
-          float wk[G];
-          bool ok[G];
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            ok[g] = false;
-            wk[g] = 0.0f;
-            x[g].v = (u32x4){0u, 0u, 0u, 0u};
-            if (kb + g < a.topk) {
-              const int r = a.src_rank[e0 + kb + g];
-              const int64_t row = a.src_row[e0 + kb + g];
-              if (r >= 0 && r < a.n && row >= 0 && row < (int64_t)a.x_rows[r]) {
-                ok[g] = true;
-                wk[g] = a.w[e0 + kb + g];
-                if (live) x[g].v = __builtin_nontemporal_load((const u32x4*)(a.x[r] + (size_t)row * row_stride) + v);
-              }
-            }
-          }
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            if (ok[g]) {
-#pragma unroll
-              for (int e = 0; e < VE; ++e) {
-                const float prod = wk[g] * Elem<DT>::load(x[g].e[e]);
-                acc[e] = acc[e] + prod;
-              }
-            }
-          }
-        }
-        if (live) {
-          VecU<DT> r;
-#pragma unroll
-          for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
-          __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
-        }
-      }
-    }
-  }
 }
 
 // ------------------------------------------------------------------------------------------
