@@ -217,6 +217,12 @@ def main():
     extras = set("c1,c2,c4,c5,moe,variants,gloo,backend".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("mccl_build", os.path.join(ROOT, "torch-ccl_amd", "csrc", "build.py"))
+    build_mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build_mod)
+    build_mod.ensure_built()  # uses what is built; compiles only if nothing is
+
     import torch
     import torch_ccl_amd as mccl
     from torch_ccl_amd import benchlib, capi

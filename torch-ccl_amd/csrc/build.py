@@ -109,6 +109,19 @@ def build_all(force=False):
     return [build_kernels(force), build_bench(force), build_backend(force)]
 
 
+def ensure_built():
+    """Builds only what does not exist yet (no staleness check): for tests, smoke() and bench.py,
+    which use the libraries that are there and compile only when nothing is."""
+    built = []
+    if not os.path.exists(KERNEL_LIB):
+        built.append(build_kernels(force=True))
+    if not os.path.exists(BENCH_LIB):
+        built.append(build_bench(force=True))
+    if not os.path.exists(backend_lib_path()):
+        built.append(build_backend(force=True))
+    return built
+
+
 if __name__ == "__main__":
     for path in build_all(force="--force" in sys.argv):
         print(path)
