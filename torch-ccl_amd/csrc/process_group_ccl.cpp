@@ -30,6 +30,10 @@ constexpr int kTableMax = 2 * kMaxWorld + 8;
 constexpr size_t kStageMin = 2u << 20;   // first staging allocation
 constexpr size_t kStageMax = 1u << 30;   // one staging window; keeps every IPC allocation < 2 GiB
 constexpr uint32_t kMagic = 0x4d43434c;  // "MCCL"
+// Collectives staging at most this many bytes run on the caller's stream: the host waits for the
+// copy-in in any case, there is no kernel long enough to be worth overlapping, and the
+// cross-stream event dependency alone costs more than the kernel.
+constexpr size_t kInlineStreamMax = 1u << 20;
 
 #define HIP_CHECK(expr)                                                                     \
   do {                                                                                      \
@@ -209,6 +213,7 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   same_stream_ = envFlag("CCL_SAME_STREAM", false);
   blocking_wait_ = envFlag("CCL_BLOCKING_WAIT", false);
   verbose_ = envFlag("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", false);
+  profile_ = envFlag("MCCL_PG_PROFILE", false);
 }
 
 c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_ptr<c10d::Store>& store,
@@ -218,6 +223,13 @@ c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_p
 }
 
 ProcessGroupCCL::~ProcessGroupCCL() {
+  if (profile_ && phase_calls_) {
+    std::ostringstream os;
+    os << "ccl backend rank " << rank_ << ": " << phase_calls_ << " collectives, mean us per phase: copy-in enqueue "
+       << phase_us_[0] / phase_calls_ << ", stream synchronise " << phase_us_[1] / phase_calls_ << ", host barrier "
+       << phase_us_[2] / phase_calls_ << ", kernel enqueue " << phase_us_[3] / phase_calls_;
+    std::cerr << os.str() << std::endl;
+  }
   if (!initialised_) return;
   // Peers may still be reading this rank's staging buffers in their last kernel: wait for our own
   // stream, then give the others a bounded chance to catch up.  A peer that is already gone has
@@ -385,8 +397,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
 
   auto cur_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_);
   hipStream_t cur = cur_stream.stream();
-  hipStream_t s = same_stream_ ? cur : comm_stream_;
-  if (!same_stream_) {  // sync_streams of the reference (src/gpu/dpcpp_ccl.cpp:186-197)
+  const bool same_stream = same_stream_ || plan.stage_bytes <= kInlineStreamMax;
+  hipStream_t s = same_stream ? cur : comm_stream_;
+  if (!same_stream) {  // sync_streams of the reference (src/gpu/dpcpp_ccl.cpp:186-197)
     HIP_CHECK(hipEventRecord(fork_event_, cur));
     HIP_CHECK(hipStreamWaitEvent(comm_stream_, fork_event_, 0));
   }
@@ -402,10 +415,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   }
 
   RankSlot& me = ctl_->slot[rank_];
+  using clk = std::chrono::steady_clock;
+  auto us_since = [](clk::time_point t) { return std::chrono::duration<double, std::micro>(clk::now() - t).count(); };
+  auto t0 = clk::now();
   try {
     void* stage = ensureStage(slot, plan.stage_bytes);
     for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
     if (plan.copy_in) plan.copy_in(stage, s);
+    if (profile_) { phase_us_[0] += us_since(t0); t0 = clk::now(); }
     // This rank's staging buffer must be complete before any peer reads it, and (two
     // collectives later) every peer must be done reading before it is overwritten: one host
     // barrier per collective plus the two alternating buffers give both.
@@ -415,7 +432,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     me.failed.store(1, std::memory_order_release);
     throw;
   }
+  if (profile_) { phase_us_[1] += us_since(t0); t0 = clk::now(); }
   hostBarrier();
+  if (profile_) { phase_us_[2] += us_since(t0); t0 = clk::now(); }
 
   if (plan.exec) {
     std::vector<const void*> peer((size_t)size_);
@@ -426,12 +445,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     }
     plan.exec(peer, tables, s);
   }
+  if (profile_) { phase_us_[3] += us_since(t0); ++phase_calls_; }
 
   auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
   work->device_ = device_;
   HIP_CHECK(hipEventCreateWithFlags(&work->end_, hipEventDisableTiming));
   HIP_CHECK(hipEventRecord(work->end_, s));
-  if (!same_stream_) {  // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
+  if (!same_stream) {  // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
     auto cs = c10::hip::getStreamFromExternalMasqueradingAsCUDA(comm_stream_, (c10::DeviceIndex)device_);
     for (const auto* list : {&plan.inputs, &plan.outputs})
       for (const auto& t : *list)
