@@ -6,6 +6,12 @@ this script compiles the device code to assembly and scans every kernel for a sc
 select or SCC branch whose nearest SCC writer in the same straight-line region is an
 arithmetic instruction rather than a compare or mask operation.
 
+The same scan enforces two numeric rules of the kernels: no packed-fp32 arithmetic
+(v_pk_add/mul/fma_f32) anywhere, and no fused multiply-add outside the AVG kernels (whose
+division by the rank count expands to a correctly rounded sequence that uses v_fma_f32): every
+add and every product of the reduction chains must round on its own.  Scratch (register spill)
+instructions are flagged as well.
+
 Usage: python torch-ccl_amd/csrc/check_isa.py   (exit status 1 if anything is flagged)
 """
 import os
@@ -23,10 +29,14 @@ _COMPARE = re.compile(r"^(s_cmp|s_cmpk|s_bitcmp|s_and_b|s_or_b|s_xor_b|s_andn2_b
 _ARITH = re.compile(r"^(s_add_|s_sub_|s_addc_|s_subb_|s_lshl_b|s_ashr_|s_min_|s_max_|s_abs_|s_absdiff_|"
                     r"s_lshl[1-4]_add_)")
 _USER = re.compile(r"^(s_cselect_|s_cbranch_scc)")
+_PACKED = re.compile(r"^v_pk_(add|mul|fma)_f32")
+_FMA = re.compile(r"^(v_fma_f32|v_fmac_f32|v_mad_f32|v_fma_f64|v_fmac_f64)")
+_AVG_KERNEL = re.compile(r"reduce_(vec|elem)_kernelILi\d+ELi1E")  # second template argument = MCCL_AVG
+_SCRATCH = re.compile(r"^scratch_")
 
 
 def device_asm(out_path):
-    flags = [f for f in _build.HIP_FLAGS if f not in ("-shared", "-fPIC")]
+    flags = [f for f in _build.HIP_FLAGS if f not in ("-shared", "-fPIC")] + ["-I", HERE]
     cmd = [_build.HIPCC] + flags + ["--cuda-device-only", "-S", "-o", out_path, _build.KERNEL_SRC]
     subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
 
@@ -49,6 +59,12 @@ def scan(asm_path):
                 fn, last = t.split(":")[0], None
                 continue
             op = t.split()[0]
+            if _PACKED.match(op):
+                flagged.append((ln, t, "packed fp32 arithmetic", fn))
+            if _FMA.match(op) and not _AVG_KERNEL.search(fn or ""):
+                flagged.append((ln, t, "fused multiply-add outside the AVG kernels", fn))
+            if _SCRATCH.match(op):
+                flagged.append((ln, t, "scratch access (register spill)", fn))
             if _USER.match(op) and last is not None and _ARITH.match(last[0]):
                 flagged.append((ln, t, last[1], fn))
             if _COMPARE.match(op) or _ARITH.match(op):
@@ -62,7 +78,7 @@ def main():
         device_asm(asm)
         flagged = scan(asm)
     for ln, ins, src, fn in flagged:
-        print("line %d in %s: `%s` takes SCC from `%s`" % (ln, fn, ins, src))
+        print("line %d in %s: `%s` <- %s" % (ln, fn, ins, src))
     print("flagged: %d" % len(flagged))
     return 1 if flagged else 0
 
