@@ -140,6 +140,15 @@ def oracle_cases(pg, rank, world):
         out = torch.empty(world * m, dtype=dtype, device=DEV)
         pg._allgather_base(out, host[rank].to(DEV)).wait()
         assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather", dtype)
+    # two-shot path (>= 4 MiB, >= 4 ranks): ragged counts, every dtype width, same bits as the oracle
+    for dtype, count in ((torch.bfloat16, (4 << 20) + 777), (torch.float32, (2 << 20) + 5), (torch.int8, (8 << 20) + 3),
+                         (torch.float64, (1 << 20) + 1)):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(count, dtype, r, seed=21) for r in range(world)]
+        t = host[rank].to(DEV)
+        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        want = bits_np(O.reduce([to_carrier(h) for h in host], code, O.SUM))
+        assert np.array_equal(bits(t), want), ("two-shot allreduce", dtype, count)
     # MIN / MAX / PRODUCT / AVG on floats
     for opname, op, ocode in (("min", c10d.ReduceOp.MIN, O.MIN), ("max", c10d.ReduceOp.MAX, O.MAX),
                               ("prod", c10d.ReduceOp.PRODUCT, O.PROD)):

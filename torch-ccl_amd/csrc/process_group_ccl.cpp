@@ -34,6 +34,13 @@ constexpr uint32_t kMagic = 0x4d43434c;  // "MCCL"
 // copy-in in any case, there is no kernel long enough to be worth overlapping, and the
 // cross-stream event dependency alone costs more than the kernel.
 constexpr size_t kInlineStreamMax = 1u << 20;
+// Allreduce messages of at least this many bytes, in groups of at least kTwoShotMinRanks, use
+// the two-shot algorithm: every rank reduces only its 1/W shard of the staged inputs, then all
+// ranks gather the W finished shards.  Per rank that moves about (4 + 1/W) S bytes instead of
+// (W + 3) S; results are identical (same ascending-rank chain per element).  It is also the
+// algorithm for W GPUs on xGMI, where each shard is reduced by the GPU that owns it.
+constexpr size_t kTwoShotMinBytes = 4u << 20;
+constexpr int kTwoShotMinRanks = 4;
 
 #define HIP_CHECK(expr)                                                                     \
   do {                                                                                      \
@@ -444,6 +451,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
       tables[(size_t)r] = ctl_->slot[r].table[slot];
     }
     plan.exec(peer, tables, s);
+    if (plan.exec2) {
+      try {
+        HIP_CHECK(hipStreamSynchronize(s));
+      } catch (...) {
+        me.failed.store(1, std::memory_order_release);
+        throw;
+      }
+      hostBarrier();
+      plan.exec2(peer, tables, s);
+    }
   }
   if (profile_) { phase_us_[3] += us_since(t0); ++phase_calls_; }
 
@@ -544,7 +561,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
   const int op = opCode(opts.reduceOp, t.scalar_type());
   const size_t es = t.element_size();
   const size_t total = (size_t)t.numel();
-  const size_t chunk = kStageMax / es;
+  // one staging window holds the input, plus (two-shot) the shard this rank reduces
+  size_t chunk = kStageMax / es;
+  if (size_ >= kTwoShotMinRanks) chunk = (chunk / (size_t)(size_ + 1) * (size_t)size_) & ~(size_t)4095;
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
@@ -556,14 +575,44 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
     p.inputs = {t};
     p.outputs = {t};
     if (size_ > 1 && len) {  // world == 1: nothing to add (src/gpu/dpcpp_ccl.cpp:752-756)
-      p.stage_bytes = len * es;
-      p.copy_in = [=](void* stage, hipStream_t s) {
-        copyAsync(stage, base, len * es, s);
-      };
       const int W = size_;
-      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
-        MCCL_CHECK(mccl_reduce_n(peer.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
-      };
+      const int me = rank_;
+      const size_t in_bytes = roundUp(len * es, 256);
+      // elements per shard: a whole number of 64-element groups, so that every shard starts on a
+      // 16-byte boundary of the staging buffers whatever the element size; the last may be shorter
+      const size_t shard = roundUp((len + (size_t)W - 1) / (size_t)W, 64);
+      const bool two_shot = W >= kTwoShotMinRanks && len * es >= kTwoShotMinBytes &&
+                            in_bytes + roundUp(shard * es, 256) <= kStageMax;
+      p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, base, len * es, s); };
+      if (!two_shot) {
+        p.stage_bytes = len * es;
+        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+          MCCL_CHECK(mccl_reduce_n(peer.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
+        };
+      } else {
+        // staging image: [the rank's input, in_bytes][the shard this rank reduces]
+        p.stage_bytes = in_bytes + roundUp(shard * es, 256);
+        auto shard_len = [=](int r) {
+          const size_t lo = std::min(len, (size_t)r * shard);
+          return std::min(len, lo + shard) - lo;
+        };
+        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+          const size_t n_me = shard_len(me);
+          if (!n_me) return;
+          std::vector<const void*> in((size_t)W);
+          for (int k = 0; k < W; ++k) in[(size_t)k] = (const char*)peer[(size_t)k] + (size_t)me * shard * es;
+          void* red = (char*)peer[(size_t)me] + in_bytes;  // peer[me] is this rank's own staging buffer
+          MCCL_CHECK(mccl_reduce_n(in.data(), W, red, n_me, dtype, op, MCCL_VARIANT_AUTO, s));
+        };
+        p.exec2 = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+          std::vector<mccl_segment_t> segs;
+          for (int r = 0; r < W; ++r) {
+            const size_t n_r = shard_len(r);
+            if (n_r) segs.push_back({(const char*)peer[(size_t)r] + in_bytes, base + (size_t)r * shard * es, n_r * es});
+          }
+          MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+        };
+      }
     }
     work = run(p);
     off += len;

@@ -138,6 +138,10 @@ class ProcessGroupCCL : public c10d::Backend {
     // tables[r] the scalars rank r published
     std::function<void(const std::vector<const void*>& peer,
                        const std::vector<const int64_t*>& tables, hipStream_t s)> exec;
+    // optional second phase: runs after every rank has finished `exec` (one more stream
+    // synchronisation and host barrier); used by the two-shot allreduce
+    std::function<void(const std::vector<const void*>& peer,
+                       const std::vector<const int64_t*>& tables, hipStream_t s)> exec2;
   };
 
   c10::intrusive_ptr<c10d::Work> run(Plan& plan);
