@@ -31,9 +31,21 @@ struct ReduceArgs {
   int n;
 };
 
+// The same for the common call: one job, at most kLeanRanks inputs.  104 bytes instead of 2.8 KB:
+// the launch path of the runtime gets measurably slower above ~104 bytes of kernel arguments
+// (2.6 -> 3.6 us per back-to-back launch), which is most of the cost of a small message.
+constexpr int kLeanRanks = 8;
+struct LeanReduceArgs {
+  const char* ptr[kLeanRanks];
+  ReduceJob job[1];
+  int n;
+  int job_ptr0[1];  // never read (OWN kernels take ReduceArgs); keeps the two types interchangeable
+};
+static_assert(sizeof(LeanReduceArgs) <= 104, "lean kernel arguments must stay below the launch-cost step");
+
 // Element-wise reduction of one element (used for peeled heads/tails and the misaligned path).
-template <int DT, int OP>
-__device__ __forceinline__ void reduce_one(const ReduceArgs& a, int p0, int n, size_t in_off,
+template <int DT, int OP, typename ARGS>
+__device__ __forceinline__ void reduce_one(const ARGS& a, int p0, int n, size_t in_off,
                                            char* out, size_t idx) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
@@ -57,8 +69,8 @@ __device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec)
 // ascending-rank chain in registers and streams the result out.
 // NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
 // NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
-template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD>
-__device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t in_byte_off,
+template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD, typename ARGS>
+__device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byte_off,
                                             u32x4* ov, size_t v0, size_t nvec, int n) {
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
@@ -134,8 +146,8 @@ __device__ __forceinline__ void reduce_tile(const ReduceArgs& a, int p0, size_t 
 // element i of every input before it writes element i, and no other lane touches i.
 // OWN: each job has its own n pointers (coalesced reductions); otherwise all jobs share
 // ptr[0..n) and the pointer loads do not wait for the job record.
-template <int DT, int OP, int NT, int U, int BLOCK, bool OWN>
-__global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
+template <int DT, int OP, int NT, int U, int BLOCK, bool OWN, typename ARGS>
+__global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
   using S = typename Elem<DT>::store_t;
   constexpr int VE = vec_elems<DT>();
   const int jid = blockIdx.y;
@@ -169,8 +181,8 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ReduceArgs a) {
 
 // Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
 // multiple of the element size).  Grid-stride over elements.
-template <int DT, int OP, bool OWN>
-__global__ __launch_bounds__(256) void reduce_elem_kernel(const ReduceArgs a) {
+template <int DT, int OP, bool OWN, typename ARGS>
+__global__ __launch_bounds__(256) void reduce_elem_kernel(const ARGS a) {
   const int jid = blockIdx.y;
   const int p0 = OWN ? a.job_ptr0[jid] : 0;
   const size_t in_off = a.job[jid].in_off;

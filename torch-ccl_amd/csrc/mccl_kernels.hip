@@ -148,22 +148,38 @@ struct Geometry {
   bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
 };
 
-template <int DT, int OP, int NT, bool OWN>
-hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+template <int DT, int OP, int NT, bool OWN, typename ARGS>
+hipError_t launch_vec_args(const ARGS& a, const Geometry& g, int njobs, hipStream_t s) {
   const dim3 grid(g.grid_x, njobs, 1);
   if (g.shape == kShapePersistent)
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent, OWN>), grid,
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent, OWN, ARGS>), grid,
                        dim3(kBlockPersistent), 0, s, a);
   else
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kWave, OWN>), grid, dim3(kWave), g.lds, s, a);
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kWave, OWN, ARGS>), grid, dim3(kWave), g.lds, s, a);
   return hipGetLastError();
+}
+
+// One job over at most kLeanRanks shared pointers travels in the 104-byte argument block.
+template <int DT, int OP, int NT, bool OWN>
+hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+  if constexpr (!OWN) {
+    if (njobs == 1 && a.n <= kLeanRanks) {
+      LeanReduceArgs lean;
+      for (int k = 0; k < kLeanRanks; ++k) lean.ptr[k] = k < a.n ? a.ptr[k] : nullptr;
+      lean.job[0] = a.job[0];
+      lean.n = a.n;
+      lean.job_ptr0[0] = 0;
+      return launch_vec_args<DT, OP, NT, false, LeanReduceArgs>(lean, g, 1, s);
+    }
+  }
+  return launch_vec_args<DT, OP, NT, OWN, ReduceArgs>(a, g, njobs, s);
 }
 
 template <int DT, int OP>
 hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
   if (g.shape == kShapeElem) {
-    if (g.own_ptrs) hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, true>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, false>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
+    if (g.own_ptrs) hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, true, ReduceArgs>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, false, ReduceArgs>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
     return hipGetLastError();
   }
   if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
