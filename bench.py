@@ -203,7 +203,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,moe,variants,gloo,backend,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,moe,variants,ceilings,gloo,backend,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -214,7 +214,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,moe,variants,gloo,backend".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,moe,variants,ceilings,gloo,backend".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import importlib.util
@@ -303,6 +303,25 @@ def main():
     result["parity_check"] = "bit-exact vs on-device fp32 chain" if same else "MISMATCH"
     del acc
 
+    # ---------------- what the part sustains: a bare streaming kernel on the same buffers ----------------
+    if "ceilings" in extras:
+        sink = torch.empty_like(out)
+        wide = torch.empty(512 << 20, dtype=torch.uint8, device=dev)  # pure-write target beyond the caches
+        cases = (("read_8_streams", ins, sink, 0, 64, 9), ("write_1_stream_512MiB", [], wide, 1, 256, 0),
+                 ("copy_1_to_1", ins[:1], sink, 1, 64, 0), ("read_8_write_1", ins, sink, 1, 64, 8))
+        ceil = {}
+        for name, rd, wr, do_write, block, per_cu in cases:
+            us = benchlib.probe_stream(rd, wr, do_write, block=block, workgroups_per_cu=per_cu)
+            nbytes = len(rd) * S + (wr.numel() * wr.element_size() if do_write else 0)
+            ceil[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                          "pct_of_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS * 100, 1)}
+        ceil["note"] = ("bare xor kernel of the bench library (no conversions, no product code), one 16-byte vector "
+                        "per lane per stream; read_8_write_1 is the traffic mix of C3")
+        result["machine_ceilings"] = ceil
+        result["roofline"]["frac_of_bare_kernel_same_mix"] = round(ceil["read_8_write_1"]["us"] / ev_us, 4)
+        log("ceilings:", json.dumps(ceil))
+        del sink, wide
+
     # ---------------- C2: 256 KiB latency ----------------
     if "c2" in extras:
         c2 = 16 * 8192
@@ -375,6 +394,8 @@ def main():
         shards = [torch.empty(m, dtype=torch.bfloat16, device=dev) for _ in range(N)]
         us_all = benchlib.reduce_scatter_throughput(big, shards, 0, warmup=2, iters=5)
         us_one = benchlib.reduce_scatter_throughput(big, shards[3:4], 3, warmup=2, iters=10)
+        # each shard reduced by a launch of its own (what each rank of a group runs)
+        us_each = [benchlib.reduce_scatter_throughput(big, shards[r:r + 1], r, warmup=1, iters=5) for r in range(N)]
         # parity on one shard against an on-device fp32 chain
         acc = torch.zeros(m, dtype=torch.float32, device=dev)
         for t in big:
@@ -383,37 +404,45 @@ def main():
         result["c4_reduce_scatter_8x1GiB"] = {
             "all_shards_us": round(us_all, 1), "all_shards_GBps": round((N + 1) * c4 * 2 / us_all / 1e3, 1),
             "one_shard_us": round(us_one, 1), "one_shard_GBps": round((N + 1) * m * 2 / us_one / 1e3, 1),
+            "each_shard_own_launch_us": [round(u, 1) for u in us_each],
+            "each_shard_own_launch_GBps": round((N + 1) * c4 * 2 / sum(us_each) / 1e3, 1),
             "shard5_bit_exact_vs_fp32_chain": ok}
         log("C4:", json.dumps(result["c4_reduce_scatter_8x1GiB"]))
         del big, shards, acc
 
     # ---------------- C5: MoE dispatch all_to_all_single, uneven splits ----------------
     if "c5" in extras:
-        tokens, hidden, topk, n_exp = 4096, 7168, 8, 256
-        per_rank = n_exp // N
-        S5 = torch.zeros(N, N, dtype=torch.int64)
+        # The config names 256 experts and 8 experts per rank, which disagree for 8 ranks: the default is
+        # 256 experts (32 per rank); the 64-expert reading (8 per rank) runs as well.  Only the split
+        # matrix differs; the bytes moved are the same.
+        tokens, hidden, topk = 4096, 7168, 8
         a2a_in = []
         for r in range(N):
-            g = rank_generator(torch, SEED, r)
-            logits = torch.randn(tokens, n_exp, generator=g)
-            experts = torch.topk(logits, topk, dim=1).indices
-            dest = (experts.reshape(-1) // per_rank)
-            S5[r] = torch.bincount(dest, minlength=N)
             gd = rank_generator(torch, SEED, r, dev)
             a2a_in.append(torch.randn(tokens * topk, hidden, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16))
-        a2a_out = [torch.empty(int(S5[:, d].sum()), hidden, dtype=torch.bfloat16, device=dev) for d in range(N)]
-        us = benchlib.alltoallv_throughput(a2a_in, a2a_out, S5, hidden * 2, warmup=2, iters=5)
-        moved = int(S5.sum()) * hidden * 2
-        # byte-exact spot check of one (source, destination) segment
-        r, d = 2, 6
-        so = int(S5[r, :d].sum()); ro = int(S5[:r, d].sum()); rows = int(S5[r, d])
-        ok = torch.equal(a2a_out[d][ro:ro + rows], a2a_in[r][so:so + rows])
-        result["c5_alltoallv_moe"] = {"us": round(us, 1), "GBps": round(2 * moved / us / 1e3, 1),
-                                      "bytes_moved": moved, "n_experts": n_exp, "experts_per_rank": per_rank,
-                                      "segment_2_to_6_byte_exact": ok,
-                                      "split_rows_rank0": S5[0].tolist()}
-        log("C5:", json.dumps(result["c5_alltoallv_moe"]))
-        del a2a_in, a2a_out
+        for n_exp, key in ((256, "c5_alltoallv_moe"), (64, "c5_alltoallv_moe_64_experts")):
+            per_rank = n_exp // N
+            S5 = torch.zeros(N, N, dtype=torch.int64)
+            for r in range(N):
+                g = rank_generator(torch, SEED, r)
+                logits = torch.randn(tokens, n_exp, generator=g)
+                experts = torch.topk(logits, topk, dim=1).indices
+                dest = (experts.reshape(-1) // per_rank)
+                S5[r] = torch.bincount(dest, minlength=N)
+            a2a_out = [torch.empty(int(S5[:, d].sum()), hidden, dtype=torch.bfloat16, device=dev) for d in range(N)]
+            us = benchlib.alltoallv_throughput(a2a_in, a2a_out, S5, hidden * 2, warmup=2, iters=5)
+            moved = int(S5.sum()) * hidden * 2
+            # byte-exact spot check of one (source, destination) segment
+            r, d = 2, 6
+            so = int(S5[r, :d].sum()); ro = int(S5[:r, d].sum()); rows = int(S5[r, d])
+            ok = torch.equal(a2a_out[d][ro:ro + rows], a2a_in[r][so:so + rows])
+            result[key] = {"us": round(us, 1), "GBps": round(2 * moved / us / 1e3, 1),
+                           "bytes_moved": moved, "n_experts": n_exp, "experts_per_rank": per_rank,
+                           "segment_2_to_6_byte_exact": ok,
+                           "split_rows_rank0": S5[0].tolist()}
+            log("C5:", json.dumps(result[key]))
+            del a2a_out
+        del a2a_in
 
     # ---------------- the steps either side of C5: token permute fused into the dispatch, weighted combine ----------------
     if "moe" in extras:

@@ -46,6 +46,18 @@ int mcclb_alltoallv_throughput(const void* const* in, void* const* out, int n,
                                const int64_t* split_rows, size_t row_bytes, void* stream,
                                int warmup, int iters, float* total_us);
 
+/*
+ * Machine probe (no product code): a bare streaming kernel in the launch shape of the large-message
+ * reduction.  Each lane reads one 16-byte vector from each of `n_read` (0, 1, 2, 4 or 8) buffers of
+ * `bytes` bytes, xors them and, if `write` is non-zero, writes the result to `out` (`bytes` bytes;
+ * must be a valid buffer even when `write` is 0).  `block` is 64 or 256 lanes per workgroup;
+ * `workgroups_per_cu` > 0 caps residency.  Tells what the part sustains for pure reads, pure
+ * writes and a read:write mix: the practical ceiling the product kernels are compared with.
+ */
+int mcclb_probe_stream(const void* const* in, int n_read, void* out, int write, size_t bytes,
+                       int block, int workgroups_per_cu, void* stream, int warmup, int iters,
+                       float* total_us);
+
 const char* mcclb_last_error(void);
 
 #ifdef __cplusplus

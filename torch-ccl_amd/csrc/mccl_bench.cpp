@@ -1,6 +1,7 @@
 // libmcclbench: HIP-event timing loops around the C ABI (see include/mccl_bench.h).
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <cstdio>
 #include <functional>
 #include <vector>
@@ -91,6 +92,52 @@ int throughput_loop(const std::function<int(int)>& call, hipStream_t s, int warm
   return rc == MCCL_OK ? MCCL_OK : fail_mccl(rc);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Machine probe: a bare streaming kernel (no product code) in the launch shape of the library's
+// large-message reduction: workgroups of `BLOCK` lanes, one 16-byte vector per lane per stream,
+// residency capped by a dynamic-LDS reservation.  Reads NR streams, xors them, and writes the
+// result (WR = 1) or keeps the store behind a compare that random data never satisfies (WR = 0).
+// It tells what this part sustains for pure reads, pure writes and a given read:write mix, which
+// is the ceiling the product kernels are compared with.
+// ---------------------------------------------------------------------------------------------
+typedef uint32_t probe_vec __attribute__((ext_vector_type(4)));
+struct ProbeArgs {
+  const probe_vec* in[8];
+  probe_vec* out;
+};
+
+template <int NR, int WR, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void probe_stream_kernel(const ProbeArgs p) {
+  const size_t v = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+  probe_vec acc = (probe_vec){1u, 2u, 3u, 4u};
+  probe_vec x[NR > 0 ? NR : 1];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) x[r] = __builtin_nontemporal_load(&p.in[r][v]);
+#pragma unroll
+  for (int r = 0; r < NR; ++r) acc ^= x[r];
+  if (WR) __builtin_nontemporal_store(acc, &p.out[v]);
+  else if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u && acc.z == 77u && acc.w == 0xfeedbeefu) p.out[v] = acc;
+}
+
+template <int NR, int WR>
+void probe_launch(const ProbeArgs& p, unsigned nvec, int block, unsigned lds, hipStream_t s) {
+  if (block == 256) hipLaunchKernelGGL((probe_stream_kernel<NR, WR, 256>), dim3(nvec / 256), dim3(256), lds, s, p);
+  else hipLaunchKernelGGL((probe_stream_kernel<NR, WR, 64>), dim3(nvec / 64), dim3(64), lds, s, p);
+}
+
+template <int WR>
+bool probe_dispatch(int n_read, const ProbeArgs& p, unsigned nvec, int block, unsigned lds, hipStream_t s) {
+  switch (n_read) {
+    case 0: if (!WR) return false; probe_launch<0, WR>(p, nvec, block, lds, s); return true;
+    case 1: probe_launch<1, WR>(p, nvec, block, lds, s); return true;
+    case 2: probe_launch<2, WR>(p, nvec, block, lds, s); return true;
+    case 4: probe_launch<4, WR>(p, nvec, block, lds, s); return true;
+    case 8: probe_launch<8, WR>(p, nvec, block, lds, s); return true;
+    default: return false;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -145,6 +192,36 @@ int mcclb_alltoallv_throughput(const void* const* in, void* const* out, int n,
                                int warmup, int iters, float* total_us) {
   auto call = [&](int) { return mccl_alltoallv_n(in, out, n, split_rows, row_bytes, stream); };
   return throughput_loop(call, (hipStream_t)stream, warmup, iters, total_us);
+}
+
+
+int mcclb_probe_stream(const void* const* in, int n_read, void* out, int write, size_t bytes,
+                       int block, int workgroups_per_cu, void* stream, int warmup, int iters,
+                       float* total_us) {
+  if (!out || (n_read > 0 && !in) || (block != 64 && block != 256) || bytes == 0 || bytes % 4096 ||
+      bytes / 16 > 0xffffffffull) {
+    snprintf(g_err, sizeof(g_err), "probe: needs an output buffer, a block of 64 or 256 and a size that is a multiple of 4 KiB");
+    return MCCL_ERR_INVALID_ARG;
+  }
+  ProbeArgs p{};
+  for (int r = 0; r < n_read && r < 8; ++r) {
+    if (!in[r]) { snprintf(g_err, sizeof(g_err), "probe: input %d is null", r); return MCCL_ERR_INVALID_ARG; }
+    p.in[r] = (const probe_vec*)in[r];
+  }
+  p.out = (probe_vec*)out;
+  unsigned lds = 0;
+  if (workgroups_per_cu > 0 && workgroups_per_cu * (block / 64) < 32) {
+    lds = (unsigned)((160 * 1024 / workgroups_per_cu) & ~511);
+    if (lds > 64 * 1024) lds = 64 * 1024;
+  }
+  const unsigned nvec = (unsigned)(bytes / 16);
+  hipStream_t s = (hipStream_t)stream;
+  auto call = [&](int) {
+    const bool ok = write ? probe_dispatch<1>(n_read, p, nvec, block, lds, s) : probe_dispatch<0>(n_read, p, nvec, block, lds, s);
+    if (!ok) return (int)MCCL_ERR_INVALID_ARG;
+    return hipGetLastError() == hipSuccess ? (int)MCCL_OK : (int)MCCL_ERR_HIP;
+  };
+  return throughput_loop(call, s, warmup, iters, total_us);
 }
 
 }  // extern "C"

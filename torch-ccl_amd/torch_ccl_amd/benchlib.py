@@ -26,6 +26,7 @@ def lib():
         L.mcclb_copy_latency.argtypes = [vp, i32, vp, i32, i32, vp]
         L.mcclb_copy_throughput.argtypes = [vp, i32, vp, i32, i32, vp]
         L.mcclb_alltoallv_throughput.argtypes = [vp, vp, i32, vp, sz, vp, i32, i32, vp]
+        L.mcclb_probe_stream.argtypes = [vp, i32, vp, i32, sz, i32, i32, vp, i32, i32, vp]
         _lib = L
     return _lib
 
@@ -102,4 +103,15 @@ def alltoallv_throughput(inputs, outputs, split_rows, row_bytes, warmup=2, iters
     _check(lib().mcclb_alltoallv_throughput(
         capi.ptr_table([t.data_ptr() for t in inputs]), capi.ptr_table([t.data_ptr() for t in outputs]), n,
         ctypes.c_void_p(S.data_ptr()), row_bytes, _stream(), warmup, iters, ctypes.byref(total)))
+    return total.value / iters
+
+
+def probe_stream(inputs, output, write, block=64, workgroups_per_cu=0, warmup=3, iters=20):
+    """Bare streaming kernel of the bench library (no product code): reads len(inputs) buffers, writes
+    `output` when `write`; returns microseconds per launch."""
+    nbytes = output.numel() * output.element_size()
+    total = ctypes.c_float(0)
+    ins = capi.ptr_table([t.data_ptr() for t in inputs]) if inputs else None
+    _check(lib().mcclb_probe_stream(ins, len(inputs), ctypes.c_void_p(output.data_ptr()), int(bool(write)), nbytes,
+                                    block, workgroups_per_cu, _stream(), warmup, iters, ctypes.byref(total)))
     return total.value / iters
