@@ -348,3 +348,42 @@ def test_reduce_scatter_offsets_beyond_4gib(mccl):
         sl = slice(shard * m, (shard + 1) * m)
         want = (ins[0][sl].float() + ins[1][sl].float()).to(torch.bfloat16)
         assert torch.equal(out.view(torch.int16), want.view(torch.int16)), "shard %d" % shard
+
+
+# ---- re-entrancy ----
+
+def test_concurrent_callers_on_their_own_streams(mccl):
+    """The entry points are re-entrant: four host threads, each on a stream of its own, run
+    reductions and copies of different shapes at the same time; every result matches the oracle."""
+    import threading
+
+    shapes = [(8, 131072, torch.bfloat16), (3, 1_000_003, torch.float32), (2, 4_194_304, torch.float16), (5, 77_777, torch.int32)]
+    errors = []
+
+    def worker(idx):
+        try:
+            n, count, dtype = shapes[idx]
+            cpu = [rank_buffer(count, dtype, 10 * idx + r) for r in range(n)]
+            want = oracle_reduce_bits(cpu)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                dev = [t.to(DEV) for t in cpu]
+                out = torch.empty(count, dtype=dtype, device=DEV)
+                gathered = torch.empty(n * count, dtype=dtype, device=DEV)
+                for it in range(25):
+                    out.zero_()
+                    mccl.reduce_n(dev, out=out, op=O.SUM, variant=it % 4)
+                    mccl.allgather_n(dev, gathered)
+                    stream.synchronize()
+                    assert_bits_equal(bits(out), want, "thread %d iteration %d" % (idx, it))
+                assert_bits_equal(bits(gathered), np.concatenate([bits(t) for t in cpu]), "thread %d allgather" % idx)
+        except BaseException as e:  # surfaced in the main thread
+            errors.append((idx, e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(shapes))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors

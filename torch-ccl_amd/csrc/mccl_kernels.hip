@@ -19,11 +19,12 @@
 //                  flight per CU.  The hardware dispatcher hands out tiles in address
 //                  order, so the set of live tiles is a compact window that sweeps the
 //                  buffers; with more resident wavefronts the window widens, DRAM pages
-//                  are re-opened more often and bandwidth drops (measured: 87 % of peak
-//                  at W = 8 for eight inputs against 75 % uncapped);
-//       persistent a fixed grid proportional to the CU count walking tiles grid-stride
-//                  (kept selectable; measured slower than "stream" on MI355X because the
-//                  workgroups drift apart and the live window smears);
+//                  are re-opened more often and bandwidth drops (measured: 83-87 % of peak
+//                  at W = 8-9 for eight inputs against 75 % uncapped);
+//       persistent a fixed grid proportional to the CU count walking tiles grid-stride.
+//                  Slower than "stream" on large messages (the workgroups drift apart and
+//                  the live window smears) but a few percent ahead while the whole working
+//                  set fits the 256 MB Infinity Cache, which is where AUTO uses it;
 //   * misaligned heads/tails are peeled element-wise inside the same launch; pointer sets
 //     that are not mutually congruent mod 16 take an element-wise kernel.
 //
