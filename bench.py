@@ -382,7 +382,18 @@ def main():
         o = torch.empty(c1, dtype=torch.float32, device=dev)
         us = benchlib.reduce_throughput([a], [o], warmup=20, iters=200)
         ok = torch.equal(o, a[0] + a[1])
-        result["c1_fp32_2ranks_16MiB"] = {"us": round(us, 2), "GBps": round(3 * c1 * 4 / us / 1e3, 1), "bit_exact": ok}
+        shapes = {name: round(benchlib.reduce_throughput([a], [o], variant=v, warmup=20, iters=200), 2)
+                  for name, v in (("small", capi.VARIANT_SMALL), ("persistent", capi.VARIANT_PERSISTENT),
+                                  ("stream", capi.VARIANT_STREAM))}
+        # the same with the three buffers 4 KiB off their power-of-two spacing
+        st = mccl.staggered_copies(a + [o])
+        us_st = benchlib.reduce_throughput([st[:2]], [st[2]], warmup=20, iters=200)
+        result["c1_fp32_2ranks_16MiB"] = {"us": round(us, 2), "GBps": round(3 * c1 * 4 / us / 1e3, 1), "bit_exact": ok,
+                                          "us_by_shape": shapes,
+                                          "buffer_offsets_MiB": [round((t.data_ptr() - a[0].data_ptr()) / 2**20, 3) for t in a + [o]],
+                                          "staggered_4KiB_us": round(us_st, 2),
+                                          "staggered_4KiB_GBps": round(3 * c1 * 4 / us_st / 1e3, 1)}
+        del st
         log("C1:", json.dumps(result["c1_fp32_2ranks_16MiB"]))
         del a, o
 
@@ -401,7 +412,16 @@ def main():
         for t in big:
             acc += t[5 * m:6 * m].float()
         ok = torch.equal(shards[5].view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+        # the same with the rank buffers 4 KiB off their power-of-two spacing (what a caller who
+        # places the buffers itself would do)
+        offs4 = [round((t.data_ptr() - big[0].data_ptr()) / 2**20, 3) for t in big]
+        big_st = mccl.staggered_copies(big)
+        us_all_st = benchlib.reduce_scatter_throughput(big_st, shards, 0, warmup=2, iters=5)
+        del big_st
         result["c4_reduce_scatter_8x1GiB"] = {
+            "rank_buffer_offsets_MiB": offs4,
+            "all_shards_staggered_4KiB_us": round(us_all_st, 1),
+            "all_shards_staggered_4KiB_GBps": round((N + 1) * c4 * 2 / us_all_st / 1e3, 1),
             "all_shards_us": round(us_all, 1), "all_shards_GBps": round((N + 1) * c4 * 2 / us_all / 1e3, 1),
             "one_shard_us": round(us_one, 1), "one_shard_GBps": round((N + 1) * m * 2 / us_one / 1e3, 1),
             "each_shard_own_launch_us": [round(u, 1) for u in us_each],

@@ -74,7 +74,9 @@ typedef enum {
 /* Tuning knobs for mccl_set_tuning (process-wide; meant for benchmarks and sweeps). */
 typedef enum {
   MCCL_TUNE_PERSISTENT_BLOCKS_PER_CU = 0, /* grid of the PERSISTENT shape */
-  MCCL_TUNE_STREAM_INFLIGHT_BYTES = 1,    /* load bytes in flight per CU, STREAM shape */
+  MCCL_TUNE_STREAM_WAVES_PER_CU = 1,      /* resident wavefronts per CU of the STREAM shape; default 0 =
+                                             chosen by the number of loads a wavefront keeps in flight
+                                             (8 ranks: 8, 4 ranks: 12, 2 ranks: no cap) */
   MCCL_TUNE_SMALL_MAX_BYTES = 2,          /* per-rank bytes up to which AUTO picks SMALL */
   MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
   MCCL_TUNE_STREAM_MIN_TOTAL_BYTES = 4,   /* (n+1)*bytes from which AUTO picks STREAM */

@@ -45,11 +45,11 @@ def test_device_free_entry_points(mccl):
     assert L.mccl_dtype_size(99) == 0
     assert L.mccl_set_tuning(99, 1) == -1
     assert b"unknown tuning knob" in L.mccl_last_error()
-    default = L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES)
-    assert L.mccl_set_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES, 12345) == 0
-    assert L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES) == 12345
-    assert L.mccl_set_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES, 0) == 0
-    assert L.mccl_get_tuning(capi.TUNE_STREAM_INFLIGHT_BYTES) == default
+    default = L.mccl_get_tuning(capi.TUNE_COPY_WAVES_PER_CU)
+    assert L.mccl_set_tuning(capi.TUNE_COPY_WAVES_PER_CU, 12) == 0
+    assert L.mccl_get_tuning(capi.TUNE_COPY_WAVES_PER_CU) == 12
+    assert L.mccl_set_tuning(capi.TUNE_COPY_WAVES_PER_CU, 0) == 0
+    assert L.mccl_get_tuning(capi.TUNE_COPY_WAVES_PER_CU) == default
 
 
 def test_argument_errors_need_no_device(mccl):

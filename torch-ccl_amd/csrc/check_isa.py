@@ -12,6 +12,14 @@ division by the rank count expands to a correctly rounded sequence that uses v_f
 add and every product of the reduction chains must round on its own.  Scratch (register spill)
 instructions are flagged as well.
 
+A third scan audits the cache hints of the 16-byte vector accesses, which decide several percent
+of bandwidth and which the compiler has dropped silently before (the `nt` of a non-temporal
+store vanished on one path of the tile loop, and byte-typed kernels lost it on some loads): in the
+reduction kernels every vector load must be non-temporal, each tile path must hold the non-temporal
+store (a hand-written instruction) beside the cacheable one, and the hand-written store must be
+followed by the wait state the compiler cannot know it needs; the full-chunk
+path of the copy kernel, the combine kernel and the stores of the row gather must be non-temporal.
+
 Usage: python torch-ccl_amd/csrc/check_isa.py   (exit status 1 if anything is flagged)
 """
 import os
@@ -72,11 +80,67 @@ def scan(asm_path):
     return flagged
 
 
+_REDUCE_VEC = re.compile(r"reduce_vec_kernelILi\d+ELi\d+ELi\d+ELi\d+ELi\d+ELb[01]E")
+
+
+def scan_hints(asm_path):
+    """Returns a list of (function, problem) for vector accesses whose cache hint is not the intended one."""
+    counts, fn, pending, unguarded = {}, None, None, []
+    with open(asm_path) as f:
+        for line in f:
+            t = line.strip()
+            m = re.match(r"^(_Z[\w.$]*):", t)
+            if m:
+                fn = m.group(1)
+                continue
+            if pending and t and not t.startswith((";", ".")):
+                # the hand-written store carries its own wait state (the compiler cannot know it needs one)
+                if not t.startswith("s_nop"):
+                    unguarded.append((pending, "vector store of the reduction is not followed by s_nop"))
+                pending = None
+            if fn and _REDUCE_VEC.search(fn) and t.startswith("global_store_dwordx4") and t.split(";")[0].strip().endswith(" nt"):
+                pending = fn
+            if fn and (t.startswith("global_load_dwordx4") or t.startswith("global_store_dwordx4")):
+                t = t.split(";")[0].strip()
+                key = ("load" if t.startswith("global_load") else "store", "nt" if t.endswith(" nt") else "plain")
+                c = counts.setdefault(fn, {})
+                c[key] = c.get(key, 0) + 1
+    bad, seen_reduce = list(unguarded), 0
+    for fn, c in counts.items():
+        get = lambda kind, hint: c.get((kind, hint), 0)
+        if _REDUCE_VEC.search(fn):
+            seen_reduce += 1
+            if get("store", "plain") != get("store", "nt"):
+                bad.append((fn, "streamed and cacheable vector stores do not pair up: %r" % c))
+            if get("load", "plain"):
+                bad.append((fn, "%d vector load(s) without nt" % get("load", "plain")))
+            if not get("store", "nt") or not get("load", "nt"):
+                bad.append((fn, "no non-temporal vector accesses found: %r" % c))
+        elif "moe_combine_kernel" in fn:
+            if get("load", "plain") or get("store", "plain"):
+                bad.append((fn, "combine kernel has vector accesses without nt: %r" % c))
+        elif "gather_rows_kernel" in fn:
+            if get("store", "plain"):
+                bad.append((fn, "row gather has vector stores without nt: %r" % c))
+        elif "copy_segments_kernel" in fn:
+            if get("load", "nt") < 2 or get("store", "nt") < 2:
+                bad.append((fn, "copy kernel lost its nt hints: %r" % c))
+    if not seen_reduce:
+        bad.append(("reduce_vec_kernel", "no reduction kernel recognised (name mangling changed?)"))
+    return bad
+
+
 def main():
     with tempfile.TemporaryDirectory() as d:
         asm = os.path.join(d, "mccl_kernels.s")
         device_asm(asm)
         flagged = scan(asm)
+        hints = scan_hints(asm)
+    for fn, problem in hints:
+        print("cache hint in %s: %s" % (fn, problem))
+    print("cache hints flagged: %d" % len(hints))
+    if hints:
+        return 1
     for ln, ins, src, fn in flagged:
         print("line %d in %s: `%s` <- %s" % (ln, fn, ins, src))
     print("flagged: %d" % len(flagged))

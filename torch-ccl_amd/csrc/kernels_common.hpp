@@ -95,6 +95,25 @@ union VecU {
   typename Elem<DT>::store_t e[vec_elems<DT>()];
 };
 
+// Element e of a vector.  One-byte types go through shifts on the 32-bit lanes: read through the
+// union, the compiler re-types the 16-byte load as a byte vector and loses its cache hint on the way.
+template <int DT>
+__device__ __forceinline__ typename Elem<DT>::store_t vec_get(const VecU<DT>& x, int e) {
+  using S = typename Elem<DT>::store_t;
+  if constexpr (sizeof(S) == 1) return (S)(uint8_t)(x.v[e >> 2] >> ((e & 3) * 8));
+  else return x.e[e];
+}
+
+template <int DT>
+__device__ __forceinline__ void vec_set(VecU<DT>& x, int e, typename Elem<DT>::store_t val) {
+  using S = typename Elem<DT>::store_t;
+  if constexpr (sizeof(S) == 1) {  // x starts as zero: or the byte in
+    x.v[e >> 2] |= (uint32_t)(uint8_t)val << ((uint32_t)(e & 3) * 8);
+  } else {
+    x.e[e] = val;
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // the reduction chain
 // ------------------------------------------------------------------------------------------

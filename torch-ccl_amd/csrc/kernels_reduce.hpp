@@ -24,11 +24,14 @@ struct ReduceJob {
 // Kernel arguments.  reduce_n: one job.  reduce_scatter: one job per shard, same pointers,
 // different byte offsets.  reduce_multi (OWN == true kernels): job j reads the n pointers
 // starting at ptr[job_ptr0[j]].
+constexpr uint32_t kFlagStreamOut = 1u;  // write the output with non-temporal stores
+
 struct ReduceArgs {
   const char* ptr[MCCL_MAX_RANKS];
   ReduceJob job[kMaxJobs];
   int job_ptr0[kMaxJobs];
   int n;
+  uint32_t flags;
 };
 
 // The same for the common call: one job, at most kLeanRanks inputs.  104 bytes instead of 2.8 KB:
@@ -39,7 +42,7 @@ struct LeanReduceArgs {
   const char* ptr[kLeanRanks];
   ReduceJob job[1];
   int n;
-  int job_ptr0[1];  // never read (OWN kernels take ReduceArgs); keeps the two types interchangeable
+  uint32_t flags;
 };
 static_assert(sizeof(LeanReduceArgs) <= 104, "lean kernel arguments must stay below the launch-cost step");
 
@@ -65,14 +68,28 @@ __device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec)
   return __builtin_nontemporal_load(&p[v]);  // streamed once: keep it out of the caches
 }
 
+// Non-temporal 16-byte store.  Written as an instruction because the compiler drops the
+// non-temporal hint of __builtin_nontemporal_store on the unguarded path of the tile loop
+// (the store came out as a plain global_store_dwordx4 there, which costs 2-3 % of bandwidth).
+// The compiler does not know that this is a store of more than 8 bytes, after which the data
+// registers must not be overwritten in the next cycle (it would schedule the hazard's wait state
+// itself for a store it knows), so the wait states are part of the instruction sequence.  The
+// operands are vector registers only: no scalar-to-vector-memory hazard can arise.  Stores the
+// compiler cannot see in its vmcnt bookkeeping only ever make its waits stricter (loads return in
+// order among themselves).
+__device__ __forceinline__ void store_vec_nt(u32x4* p, u32x4 x) {
+  asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(p), "v"(x) : "memory");
+}
+
 // One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
 // ascending-rank chain in registers and streams the result out.
 // NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
 // NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
 template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD, typename ARGS>
 __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byte_off,
-                                            u32x4* ov, size_t v0, size_t nvec, int n) {
+                                            u32x4* ov, size_t v0, size_t nvec, int n, bool stream_out) {
   using A = typename Elem<DT>::acc_t;
+  using S = typename Elem<DT>::store_t;
   constexpr int VE = vec_elems<DT>();
   A acc[U][VE];
 
@@ -87,12 +104,12 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x[0][u].e[e]));
+      for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x[0][u], e)));
 #pragma unroll
       for (int k = 1; k < NT; ++k)
 #pragma unroll
         for (int e = 0; e < VE; ++e)
-          acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[k][u].e[e]));
+          acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(vec_get<DT>(x[k][u], e)));
     }
   } else {
     {
@@ -102,7 +119,7 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
         VecU<DT> x;
         x.v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
 #pragma unroll
-        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(x.e[e]));
+        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x, e)));
       }
     }
     constexpr int G = 4;
@@ -123,7 +140,7 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
           for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int e = 0; e < VE; ++e)
-              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(x[g][u].e[e]));
+              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(vec_get<DT>(x[g][u], e)));
         }
       }
     }
@@ -134,9 +151,12 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
     const size_t v = v0 + (size_t)u * BLOCK;
     if (!GUARD || v < nvec) {
       VecU<DT> r;
+      if constexpr (sizeof(S) == 1) r.v = (u32x4){0u, 0u, 0u, 0u};  // vec_set ors the bytes in
 #pragma unroll
-      for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(chain_last<DT, OP>(acc[u][e], n));
-      __builtin_nontemporal_store(r.v, &ov[v]);
+      for (int e = 0; e < VE; ++e) vec_set<DT>(r, e, Elem<DT>::store(chain_last<DT, OP>(acc[u][e], n)));
+      // large outputs are streamed past the caches; small ones stay cacheable for their consumer
+      if (stream_out) store_vec_nt(&ov[v], r.v);
+      else ov[v] = r.v;
     }
   }
 }
@@ -151,8 +171,10 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
   using S = typename Elem<DT>::store_t;
   constexpr int VE = vec_elems<DT>();
   const int jid = blockIdx.y;
-  const int p0 = OWN ? a.job_ptr0[jid] : 0;
+  int p0 = 0;
+  if constexpr (OWN) p0 = a.job_ptr0[jid];
   const int n = (NT > 0) ? NT : a.n;
+  const bool stream_out = (a.flags & kFlagStreamOut) != 0;
   char* out = a.job[jid].out;
   const size_t in_off = a.job[jid].in_off;
   const size_t nvec = a.job[jid].nvec;
@@ -174,9 +196,9 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
 
   uint32_t tile = blockIdx.x;
   for (; tile < full_tiles; tile += gridDim.x)
-    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
+    reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n, stream_out);
   if (tile == full_tiles && partial)  // the one partial tile; exactly one workgroup reaches it
-    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n);
+    reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n, stream_out);
 }
 
 // Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
@@ -184,7 +206,8 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
 template <int DT, int OP, bool OWN, typename ARGS>
 __global__ __launch_bounds__(256) void reduce_elem_kernel(const ARGS a) {
   const int jid = blockIdx.y;
-  const int p0 = OWN ? a.job_ptr0[jid] : 0;
+  int p0 = 0;
+  if constexpr (OWN) p0 = a.job_ptr0[jid];
   const size_t in_off = a.job[jid].in_off;
   char* out = a.job[jid].out;
   const size_t count = a.job[jid].nvec;  // element count for this kernel

@@ -8,7 +8,8 @@
 //     add so the memory system sees N*U independent requests per lane;
 //   * accumulation is a sequential ascending-rank chain held in registers (fp32 for
 //     f16/bf16), one round-to-nearest-even on store;
-//   * outputs are written with non-temporal stores (streamed past the caches);
+//   * outputs are written with non-temporal stores (streamed past the caches): worth 2-5 %
+//     against plain stores, most on multi-GiB footprints;
 //   * inputs are read with non-temporal loads: nothing is reused, and on this part the
 //     streaming hint alone is worth about 12 % of bandwidth;
 //   * launch shapes (same kernel code, different geometry):
@@ -19,8 +20,8 @@
 //                  flight per CU.  The hardware dispatcher hands out tiles in address
 //                  order, so the set of live tiles is a compact window that sweeps the
 //                  buffers; with more resident wavefronts the window widens, DRAM pages
-//                  are re-opened more often and bandwidth drops (measured: 83-87 % of peak
-//                  at W = 8-9 for eight inputs against 75 % uncapped);
+//                  are re-opened more often and bandwidth drops (measured: 84-87 % of peak
+//                  at W = 7-8 for eight inputs against 75 % uncapped);
 //       persistent a fixed grid proportional to the CU count walking tiles grid-stride.
 //                  Slower than "stream" on large messages (the workgroups drift apart and
 //                  the live window smears) but a few percent ahead while the whole working
@@ -82,13 +83,13 @@ constexpr int kMaxWavesPerCu = 32;
 // tunables (mccl_set_tuning); defaults come from sweeps on MI355X
 long long g_tune[MCCL_TUNE_COUNT_] = {
     /* PERSISTENT_BLOCKS_PER_CU */ 8,
-    /* STREAM_INFLIGHT_BYTES    */ 72 * 1024,
-    /* SMALL_MAX_BYTES          */ 8 << 20,
+    /* STREAM_WAVES_PER_CU      */ 0,
+    /* SMALL_MAX_BYTES          */ 4 << 20,
     /* COPY_WAVES_PER_CU        */ 28,
-    /* STREAM_MIN_TOTAL_BYTES   */ 320ll << 20,
+    /* STREAM_MIN_TOTAL_BYTES   */ 112ll << 20,
     /* COMBINE_PIECES_PER_WAVE  */ 2,
 };
-const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 72 * 1024, 8 << 20, 28, 320ll << 20, 2};
+const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 0, 4 << 20, 28, 112ll << 20, 2};
 
 // Dynamic-LDS bytes that limit residency to `waves` single-wavefront workgroups per CU
 // (0 = no reservation needed).
@@ -147,6 +148,7 @@ struct Geometry {
   int block;
   unsigned lds;   // dynamic LDS reservation (occupancy cap), bytes
   bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
+  bool stream_out;  // write the output with non-temporal stores
 };
 
 template <int DT, int OP, int NT, bool OWN, typename ARGS>
@@ -169,7 +171,7 @@ hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStre
       for (int k = 0; k < kLeanRanks; ++k) lean.ptr[k] = k < a.n ? a.ptr[k] : nullptr;
       lean.job[0] = a.job[0];
       lean.n = a.n;
-      lean.job_ptr0[0] = 0;
+      lean.flags = a.flags;
       return launch_vec_args<DT, OP, NT, false, LeanReduceArgs>(lean, g, 1, s);
     }
   }
@@ -231,6 +233,21 @@ int loads_in_flight(int n, int op, bool own_ptrs) {
   return n < 4 ? n : 4;
 }
 
+// Resident wavefronts per CU of the stream shape.  Enough loads in flight to cover the memory
+// latency at full bandwidth (about 14 MB over the chip), and no more: every further wavefront
+// widens the window of live tiles and costs DRAM page locality.  Measured optima on MI355X
+// (bf16, 64 MiB per rank, warm and rotating through 9 GiB): with all loads of a tile in flight
+// 7-8 wavefronts for 8 ranks (6 falls off a cliff: 75 % of peak against 87 %), 12 for 4 ranks, no
+// cap for 2; with loads in groups of four 14, with three 24.
+long long stream_waves(int n, int op, bool own_ptrs) {
+  if (g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU] > 0) return g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU];
+  const int in_flight = loads_in_flight(n, op, own_ptrs);
+  if (in_flight == 8) return 8;
+  if (in_flight == 4) return in_flight == n ? 12 : 14;
+  if (in_flight == 3) return 24;
+  return kMaxWavesPerCu;
+}
+
 // Geometry of a vector launch over njobs jobs whose largest has max_count elements.
 int plan_vec(size_t max_count, int njobs, int n, int dtype, int op, int variant, bool own_ptrs,
              Geometry* g) {
@@ -239,24 +256,29 @@ int plan_vec(size_t max_count, int njobs, int n, int dtype, int op, int variant,
   if (rc != MCCL_OK) return rc;
   const size_t es = dtype_size(dtype);
   const size_t nvec = max_count / (16 / es) + 1;
+  // Measured crossovers on MI355X.  Up to a few MiB per rank a launch is latency-bound: one
+  // wavefront per tile, cacheable output.  From about 112 MiB of traffic per launch the capped
+  // in-order stream with a streamed (non-temporal) output wins by 3-15 %.  In between, four or
+  // more ranks do best with the persistent grid and a cacheable output (the working set sits in
+  // the Infinity Cache, where a streamed output costs up to 20 %); with fewer ranks the output is
+  // a third or more of the traffic and streaming it pays from 8 MiB per rank on.
+  const size_t per_rank = max_count * es;
+  const size_t total = per_rank * (size_t)(n + 1) * (size_t)njobs;
+  const bool small_msg = per_rank <= (size_t)g_tune[MCCL_TUNE_SMALL_MAX_BYTES];
+  const bool large_msg = total >= (size_t)g_tune[MCCL_TUNE_STREAM_MIN_TOTAL_BYTES];
   Shape shape;
   switch (variant) {
     case MCCL_VARIANT_SMALL: shape = kShapeSmall; break;
     case MCCL_VARIANT_PERSISTENT: shape = kShapePersistent; break;
     case MCCL_VARIANT_STREAM: shape = kShapeStream; break;
-    case MCCL_VARIANT_AUTO: {
-      // measured crossovers on MI355X: launch-bound up to a few MiB per rank; while the whole
-      // working set fits the Infinity Cache the persistent grid is a few percent ahead;
-      // beyond it the capped in-order stream wins by 5-12 %.
-      const size_t per_rank = max_count * es;
-      const size_t total = per_rank * (size_t)(n + 1) * (size_t)njobs;
-      if (per_rank <= (size_t)g_tune[MCCL_TUNE_SMALL_MAX_BYTES]) shape = kShapeSmall;
-      else if (total >= (size_t)g_tune[MCCL_TUNE_STREAM_MIN_TOTAL_BYTES]) shape = kShapeStream;
-      else shape = kShapePersistent;
+    case MCCL_VARIANT_AUTO:
+      if (small_msg) shape = kShapeSmall;
+      else if (large_msg) shape = kShapeStream;
+      else shape = n >= 4 ? kShapePersistent : kShapeSmall;
       break;
-    }
     default: return fail(MCCL_ERR_INVALID_ARG, "unknown variant %d", variant);
   }
+  g->stream_out = !small_msg && (large_msg || n < 4);
   g->shape = shape;
   g->lds = 0;
   g->own_ptrs = own_ptrs;
@@ -273,12 +295,7 @@ int plan_vec(size_t max_count, int njobs, int n, int dtype, int op, int variant,
     if (tiles > kMaxGridX) tiles = kMaxGridX;
     g->grid_x = (unsigned)(tiles ? tiles : 1);
     g->block = kWave;
-    if (shape == kShapeStream) {
-      const long long per_wave = (long long)loads_in_flight(n, op, own_ptrs) * kWave * 16;
-      long long waves = g_tune[MCCL_TUNE_STREAM_INFLIGHT_BYTES] / per_wave;
-      if (waves < 2) waves = 2;
-      g->lds = lds_for_waves(waves);
-    }
+    if (shape == kShapeStream) g->lds = lds_for_waves(stream_waves(n, op, own_ptrs));
   }
   return MCCL_OK;
 }
@@ -341,6 +358,9 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
     Geometry g;
     int rc = plan_vec(vmax, nv, a.n, dtype, op, variant, own_ptrs, &g);
     if (rc != MCCL_OK) return rc;
+    // outputs of launches that move more than the Infinity Cache holds are streamed past the
+    // caches (2-5 % of bandwidth); smaller ones stay cacheable for whoever reads them next
+    a.flags = g.stream_out ? kFlagStreamOut : 0u;
     hipError_t e = launch_any(a, dtype, op, g, nv, s);
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   }
@@ -352,7 +372,7 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
     size_t cap = (size_t)cus * 8 / ne;
     if (cap < 1) cap = 1;
     if (blocks > cap) blocks = cap;
-    Geometry g{kShapeElem, (unsigned)blocks, 256, 0, own_ptrs};
+    Geometry g{kShapeElem, (unsigned)blocks, 256, 0, own_ptrs, false};
     hipError_t e = launch_any(elem, dtype, op, g, ne, s);
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   }

@@ -176,14 +176,16 @@ class ProcessGroupCCL : public c10d::Backend {
   std::string shm_name_;
 
   struct Stage {
-    void* ptr = nullptr;
+    void* base = nullptr;  // the allocation
+    void* ptr = nullptr;   // where this rank's data starts (staggered by rank inside the allocation)
     size_t capacity = 0;
   };
   Stage stage_[2];
   std::vector<void*> retired_;  // outgrown staging buffers, freed with the group
 
   struct PeerMap {
-    void* ptr[2] = {nullptr, nullptr};
+    void* base[2] = {nullptr, nullptr};  // mapping of the peer's allocation (what gets closed)
+    void* ptr[2] = {nullptr, nullptr};   // the peer's data inside it
     uint64_t gen[2] = {0, 0};
     bool ipc[2] = {false, false};
   };
