@@ -15,8 +15,8 @@ instructions are flagged as well.
 A third scan audits the cache hints of the 16-byte vector accesses, which decide several percent
 of bandwidth and which the compiler has dropped silently before (the `nt` of a non-temporal
 store vanished on one path of the tile loop, and byte-typed kernels lost it on some loads): in the
-reduction kernels every vector load must be non-temporal, each tile path must hold the non-temporal
-store (a hand-written instruction) beside the cacheable one, and the hand-written store must be
+reduction kernels every vector load must be non-temporal, each tile path must hold the
+streaming store (a hand-written `sc1` instruction) beside the cacheable one, and that store must be
 followed by the wait state the compiler cannot know it needs; the full-chunk
 path of the copy kernel, the combine kernel and the stores of the row gather must be non-temporal.
 
@@ -83,6 +83,13 @@ def scan(asm_path):
 _REDUCE_VEC = re.compile(r"reduce_vec_kernelILi\d+ELi\d+ELi\d+ELi\d+ELi\d+ELb[01]E")
 
 
+def _hint(instruction):
+    """Cache-policy flags of a global load/store ('plain' if none)."""
+    words = instruction.split(";")[0].replace(",", " ").split()
+    flags = [w for w in words if w in ("sc0", "sc1", "nt")]
+    return " ".join(flags) if flags else "plain"
+
+
 def scan_hints(asm_path):
     """Returns a list of (function, problem) for vector accesses whose cache hint is not the intended one."""
     counts, fn, pending, unguarded = {}, None, None, []
@@ -98,11 +105,11 @@ def scan_hints(asm_path):
                 if not t.startswith("s_nop"):
                     unguarded.append((pending, "vector store of the reduction is not followed by s_nop"))
                 pending = None
-            if fn and _REDUCE_VEC.search(fn) and t.startswith("global_store_dwordx4") and t.split(";")[0].strip().endswith(" nt"):
+            if fn and _REDUCE_VEC.search(fn) and t.startswith("global_store_dwordx4") and _hint(t) == "sc1":
                 pending = fn
             if fn and (t.startswith("global_load_dwordx4") or t.startswith("global_store_dwordx4")):
                 t = t.split(";")[0].strip()
-                key = ("load" if t.startswith("global_load") else "store", "nt" if t.endswith(" nt") else "plain")
+                key = ("load" if t.startswith("global_load") else "store", _hint(t))
                 c = counts.setdefault(fn, {})
                 c[key] = c.get(key, 0) + 1
     bad, seen_reduce = list(unguarded), 0
@@ -110,12 +117,12 @@ def scan_hints(asm_path):
         get = lambda kind, hint: c.get((kind, hint), 0)
         if _REDUCE_VEC.search(fn):
             seen_reduce += 1
-            if get("store", "plain") != get("store", "nt"):
-                bad.append((fn, "streamed and cacheable vector stores do not pair up: %r" % c))
-            if get("load", "plain"):
-                bad.append((fn, "%d vector load(s) without nt" % get("load", "plain")))
-            if not get("store", "nt") or not get("load", "nt"):
-                bad.append((fn, "no non-temporal vector accesses found: %r" % c))
+            if get("store", "plain") != get("store", "sc1") or not get("store", "sc1"):
+                bad.append((fn, "streamed (sc1) and cacheable vector stores do not pair up: %r" % c))
+            if set(k for k in c if k[0] == "load") != {("load", "nt")}:
+                bad.append((fn, "vector loads must all be nt: %r" % c))
+            if set(k for k in c if k[0] == "store") != {("store", "plain"), ("store", "sc1")}:
+                bad.append((fn, "unexpected vector store flavour: %r" % c))
         elif "moe_combine_kernel" in fn:
             if get("load", "plain") or get("store", "plain"):
                 bad.append((fn, "combine kernel has vector accesses without nt: %r" % c))

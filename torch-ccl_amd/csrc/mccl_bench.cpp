@@ -116,7 +116,10 @@ __global__ __launch_bounds__(BLOCK) void probe_stream_kernel(const ProbeArgs p) 
   for (int r = 0; r < NR; ++r) x[r] = __builtin_nontemporal_load(&p.in[r][v]);
 #pragma unroll
   for (int r = 0; r < NR; ++r) acc ^= x[r];
-  if (WR) __builtin_nontemporal_store(acc, &p.out[v]);
+  // the streaming store of the product kernels (write-through at agent scope), spelled as an
+  // instruction so that the hint survives; the wait state after it covers the hazard the compiler
+  // cannot see
+  if (WR) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&p.out[v]), "v"(acc) : "memory");
   else if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u && acc.z == 77u && acc.w == 0xfeedbeefu) p.out[v] = acc;
 }
 
