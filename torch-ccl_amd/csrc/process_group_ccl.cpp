@@ -11,6 +11,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -236,11 +237,16 @@ c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_p
 }
 
 ProcessGroupCCL::~ProcessGroupCCL() {
-  if (profile_ && phase_calls_) {
+  if (profile_ && !phase_us_[0].empty()) {
+    // medians: the first calls of a group pay for allocations and peer mappings
     std::ostringstream os;
-    os << "ccl backend rank " << rank_ << ": " << phase_calls_ << " collectives, mean us per phase: copy-in enqueue "
-       << phase_us_[0] / phase_calls_ << ", stream synchronise " << phase_us_[1] / phase_calls_ << ", host barrier "
-       << phase_us_[2] / phase_calls_ << ", kernel enqueue " << phase_us_[3] / phase_calls_;
+    os << "ccl backend rank " << rank_ << ": " << phase_us_[0].size() << " collectives with a payload, median us per phase:";
+    const char* names[4] = {" copy-in enqueue ", ", stream synchronise ", ", host barrier ", ", kernel enqueue "};
+    for (int i = 0; i < 4; ++i) {
+      auto& v = phase_us_[i];
+      std::nth_element(v.begin(), v.begin() + (long)(v.size() / 2), v.end());
+      os << names[i] << v[v.size() / 2];
+    }
     std::cerr << os.str() << std::endl;
   }
   if (!initialised_) return;
@@ -433,12 +439,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   RankSlot& me = ctl_->slot[rank_];
   using clk = std::chrono::steady_clock;
   auto us_since = [](clk::time_point t) { return std::chrono::duration<double, std::micro>(clk::now() - t).count(); };
+  const bool timed = profile_ && plan.stage_bytes > 0 && phase_us_[0].size() < (1u << 20);
   auto t0 = clk::now();
   try {
     void* stage = ensureStage(slot, plan.stage_bytes);
     for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
     if (plan.copy_in) plan.copy_in(stage, s);
-    if (profile_) { phase_us_[0] += us_since(t0); t0 = clk::now(); }
+    if (timed) { phase_us_[0].push_back((float)us_since(t0)); t0 = clk::now(); }
     // This rank's staging buffer must be complete before any peer reads it, and (two
     // collectives later) every peer must be done reading before it is overwritten: one host
     // barrier per collective plus the two alternating buffers give both.
@@ -448,9 +455,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     me.failed.store(1, std::memory_order_release);
     throw;
   }
-  if (profile_) { phase_us_[1] += us_since(t0); t0 = clk::now(); }
+  if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
   hostBarrier();
-  if (profile_) { phase_us_[2] += us_since(t0); t0 = clk::now(); }
+  if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
 
   if (plan.exec) {
     std::vector<const void*> peer((size_t)size_);
@@ -471,7 +478,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
       plan.exec2(peer, tables, s);
     }
   }
-  if (profile_) { phase_us_[3] += us_since(t0); ++phase_calls_; }
+  if (timed) phase_us_[3].push_back((float)us_since(t0));
 
   auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
   work->device_ = device_;

@@ -158,8 +158,8 @@ class ProcessGroupCCL : public c10d::Backend {
   bool same_stream_ = false;    // CCL_SAME_STREAM
   bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
   bool profile_ = false;        // MCCL_PG_PROFILE: host-side phase timers, printed when the group dies
-  double phase_us_[4] = {0, 0, 0, 0};  // copy-in enqueue, stream synchronise, host barrier, kernel enqueue
-  uint64_t phase_calls_ = 0;
+  // per collective with a payload: copy-in enqueue, stream synchronise, host barrier, kernel enqueue
+  std::vector<float> phase_us_[4];
   bool coalescing_ = false;
   c10::intrusive_ptr<WorkCCL> last_work_;  // only kept between startCoalescing and endCoalescing
   std::mutex mutex_;  // one collective of a group at a time (the reference serialises on a global mutex)
