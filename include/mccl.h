@@ -81,7 +81,8 @@ typedef enum {
   MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
   MCCL_TUNE_STREAM_MIN_TOTAL_BYTES = 4,   /* (n+1)*bytes from which AUTO picks STREAM */
   MCCL_TUNE_COMBINE_PIECES_PER_WAVE = 5,  /* 1 KiB row pieces one wavefront of moe_combine walks */
-  MCCL_TUNE_COUNT_ = 6
+  MCCL_TUNE_COMBINE_WAVES_PER_CU = 6,     /* residency cap of moe_combine; default 0 = none */
+  MCCL_TUNE_COUNT_ = 7
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64

@@ -85,7 +85,9 @@ struct CombineArgs {
   int n;
 };
 
-template <int DT>
+// FAST: top-k of at most 8 (one group of row loads covers a token); the general path is a kernel
+// of its own so that each gets its own register budget.
+template <int DT, bool FAST>
 __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a) {
   using A = float;
   constexpr int VE = vec_elems<DT>();
@@ -98,36 +100,48 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
     const uint32_t p0 = part * a.pieces_per_wave;
     const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
     const size_t e0 = (size_t)tok * a.topk;
-    if (a.topk <= G) {
-      // routing entries looked up once for all pieces this wavefront walks
-      int rk[G];
-      int64_t rw[G];
-      float wk[G];
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const bool in = (uint32_t)g < a.topk;
-        rk[g] = in ? a.src_rank[e0 + g] : -1;
-        rw[g] = in ? a.src_row[e0 + g] : 0;
-        wk[g] = in ? a.w[e0 + g] : 0.0f;
+    if constexpr (FAST) {
+      // The token's routing entries are looked up once for all pieces this wavefront walks: lane g
+      // loads entry g (three loads in flight at once), and the values are broadcast into scalar
+      // registers, so that everything derived from them (the peer pointer picked from the argument
+      // block, the bounds checks, the row address) is scalar work and the row loads start after
+      // one memory round trip instead of two.
+      int my_rank = -1;
+      int64_t my_row = 0;
+      float my_w = 0.0f;
+      if (threadIdx.x < a.topk) {
+        my_rank = a.src_rank[e0 + threadIdx.x];
+        my_row = a.src_row[e0 + threadIdx.x];
+        my_w = a.w[e0 + threadIdx.x];
       }
       const u32x4* src[G];
       bool ok[G];
+      float wk[G];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const bool rank_ok = rk[g] >= 0 && rk[g] < a.n;
-        const int r = rank_ok ? rk[g] : 0;
-        ok[g] = rank_ok && rw[g] >= 0 && rw[g] < (int64_t)a.x_rows[r];
-        src[g] = (const u32x4*)(a.x[r] + (ok[g] ? (size_t)rw[g] : 0) * row_stride);
+        const int rk = __builtin_amdgcn_readlane(my_rank, g);
+        const uint32_t row_lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)my_row, g);
+        const uint32_t row_hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)my_row >> 32), g);
+        const int64_t rw = (int64_t)(((uint64_t)row_hi << 32) | row_lo);
+        wk[g] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_w), g));
+        const bool rank_ok = rk >= 0 && rk < a.n;
+        const int r = rank_ok ? rk : 0;
+        ok[g] = rank_ok && rw >= 0 && rw < (int64_t)a.x_rows[r];
+        src[g] = (const u32x4*)(a.x[r] + (ok[g] ? (size_t)rw : 0) * row_stride);
       }
-      for (uint32_t piece = p0; piece < p1; ++piece) {
+      // Double-buffered walk over the pieces: the row loads of piece i+1 are in flight while piece i
+      // is weighted, summed and stored, so a wavefront never sits without memory requests.
+      auto load_piece = [&](uint32_t piece, VecU<DT>(&x)[G]) {
         const uint32_t v = piece * kWave + threadIdx.x;
         const bool live = v < a.row_vecs;
-        VecU<DT> x[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
           x[g].v = (u32x4){0u, 0u, 0u, 0u};
           if (ok[g] && live) x[g].v = __builtin_nontemporal_load(src[g] + v);
         }
+      };
+      auto finish_piece = [&](uint32_t piece, const VecU<DT>(&x)[G]) {
+        const uint32_t v = piece * kWave + threadIdx.x;
         A acc[VE];
 #pragma unroll
         for (int e = 0; e < VE; ++e) acc[e] = 0.0f;
@@ -141,11 +155,21 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
             }
           }
         }
-        if (live) {
+        if (v < a.row_vecs) {
           VecU<DT> r;
 #pragma unroll
           for (int e = 0; e < VE; ++e) r.e[e] = Elem<DT>::store(acc[e]);
           __builtin_nontemporal_store(r.v, (u32x4*)(a.y + (size_t)tok * row_stride) + v);
+        }
+      };
+      VecU<DT> xa[G], xb[G];
+      load_piece(p0, xa);
+      for (uint32_t piece = p0; piece < p1; piece += 2) {
+        if (piece + 1 < p1) load_piece(piece + 1, xb);
+        finish_piece(piece, xa);
+        if (piece + 1 < p1) {
+          if (piece + 2 < p1) load_piece(piece + 2, xa);
+          finish_piece(piece + 1, xb);
         }
       }
     } else {

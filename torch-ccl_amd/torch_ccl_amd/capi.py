@@ -19,7 +19,8 @@ U8, I8, I16, I32, I64, F16, F32, F64, BF16 = range(9)
 SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
 VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
 (TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_WAVES_PER_CU, TUNE_SMALL_MAX_BYTES,
- TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE) = range(6)
+ TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
+ TUNE_COMBINE_WAVES_PER_CU) = range(7)
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
