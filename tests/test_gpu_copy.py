@@ -191,3 +191,16 @@ def test_copy_segment_larger_than_4gib(mccl):
     torch.cuda.synchronize()
     assert torch.equal(dst[5:5 + nbytes], src[5:5 + nbytes])
     assert int(dst[:5].sum()) == 0 and int(dst[5 + nbytes:].sum()) == 0
+
+
+def test_staggered_copies_keep_the_data_and_leave_the_power_of_two_spacing(mccl):
+    ts = [torch.full((1 << 20,), float(k), dtype=torch.float32, device=DEV) for k in range(5)]
+    st = mccl.staggered_copies(ts)
+    torch.cuda.synchronize()
+    for k, (a, b) in enumerate(zip(ts, st)):
+        assert torch.equal(a, b) and b.data_ptr() % 256 == 0
+        if k:
+            assert (b.data_ptr() - st[k - 1].data_ptr()) == (4 << 20) + 4096
+    out = mccl.reduce_n(st[:4], op=O.SUM)
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.full_like(out, 6.0))

@@ -106,3 +106,29 @@ def test_dispatch_then_one_hot_combine_returns_the_tokens(mccl):
     y = mccl.moe_combine(recv, src_rank[3].to(DEV), src_row[3].to(DEV), w.to(DEV))
     torch.cuda.synchronize()
     assert torch.equal(y.view(torch.int16), hid[3].view(torch.int16))
+
+
+@pytest.mark.parametrize("topk", [1, 5, 8, 9, 12, 17])
+@pytest.mark.parametrize("hidden", [8, 520, 7168])
+def test_combine_any_topk_with_skipped_entries(mccl, topk, hidden):
+    """Random routing tables (any rank, any row) for top-k below, at and above the 8 entries one
+    group of row loads covers; a tenth of the entries point outside their buffer (negative rank,
+    rank >= n, negative row, row past the end) and must be skipped, as the oracle skips them."""
+    n, tokens, dtype = 4, 77, torch.bfloat16
+    g = torch.Generator().manual_seed(1000 * topk + hidden)
+    rows = [60 + 11 * r for r in range(n)]
+    x = [torch.randn(rows[r], hidden, generator=g).to(dtype) for r in range(n)]
+    src_rank = torch.randint(0, n, (tokens, topk), generator=g, dtype=torch.int32)
+    src_row = torch.stack([torch.randint(0, rows[int(r)], (1,), generator=g)[0] for r in src_rank.reshape(-1)]).reshape(tokens, topk).to(torch.int64)
+    bad = torch.rand(tokens, topk, generator=g) < 0.1
+    kind = torch.randint(0, 4, (tokens, topk), generator=g)
+    src_rank = torch.where(bad & (kind == 0), torch.full_like(src_rank, -1), src_rank)
+    src_rank = torch.where(bad & (kind == 1), torch.full_like(src_rank, n), src_rank)
+    src_row = torch.where(bad & (kind == 2), torch.full_like(src_row, -3), src_row)
+    src_row = torch.where(bad & (kind == 3), torch.full_like(src_row, 10_000), src_row)
+    w = torch.randn(tokens, topk, generator=g).contiguous()
+    y = mccl.moe_combine([t.to(DEV) for t in x], src_rank.to(DEV), src_row.to(DEV), w.to(DEV))
+    torch.cuda.synchronize()
+    want = O.moe_combine([to_carrier(t) for t in x], src_rank.numpy(), src_row.numpy(), w.numpy(),
+                         tokens, topk, hidden, TORCH_TO_CODE[dtype])
+    assert_bits_equal(bits(y), want.view(np.uint16), "combine topk %d hidden %d" % (topk, hidden))
