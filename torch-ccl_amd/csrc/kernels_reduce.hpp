@@ -86,7 +86,7 @@ __device__ __forceinline__ void store_vec_stream(u32x4* p, u32x4 x) {
 // One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
 // ascending-rank chain in registers and streams the result out.
 // NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
-// NT == 0: runtime rank count; rank 0 first, then groups of 4 ranks.
+// NT == 0: runtime rank count, groups of 4 ranks.
 template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD, typename ARGS>
 __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byte_off,
                                             u32x4* ov, size_t v0, size_t nvec, int n, bool stream_out) {
@@ -114,18 +114,12 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
           acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(vec_get<DT>(x[k][u], e)));
     }
   } else {
-    {
-      const u32x4* iv = (const u32x4*)(a.ptr[p0] + in_byte_off);
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        VecU<DT> x;
-        x.v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
-#pragma unroll
-        for (int e = 0; e < VE; ++e) acc[u][e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x, e)));
-      }
-    }
     constexpr int G = 4;
-    for (int kb = 1; kb < n; kb += G) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int e = 0; e < VE; ++e) acc[u][e] = (A)0;  // overwritten by rank 0's element
+    for (int kb = 0; kb < n; kb += G) {
       VecU<DT> x[G][U];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -141,8 +135,11 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
 #pragma unroll
           for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int e = 0; e < VE; ++e)
-              acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(vec_get<DT>(x[g][u], e)));
+            for (int e = 0; e < VE; ++e) {
+              const A xv = Elem<DT>::load(vec_get<DT>(x[g][u], e));
+              if (g == 0 && kb == 0) acc[u][e] = chain_first<DT, OP>(xv);
+              else acc[u][e] = chain_next<DT, OP>(acc[u][e], xv);
+            }
         }
       }
     }

@@ -187,7 +187,7 @@ hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStrea
     return hipGetLastError();
   }
   if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
-  if constexpr (OP == MCCL_SUM) {
+  if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {  // the ops of gradient reductions
     switch (a.n) {
       case 2: return launch_vec<DT, OP, 2, false>(a, g, njobs, s);
       case 4: return launch_vec<DT, OP, 4, false>(a, g, njobs, s);
@@ -228,25 +228,26 @@ hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g,
 }
 
 // Loads one wavefront keeps in flight per tile: all ranks when the rank count is a
-// compile-time specialisation (SUM with 2, 4 or 8 ranks), else one group of four.
+// compile-time specialisation (SUM and AVG with 2, 4 or 8 ranks), else one group of four.
 int loads_in_flight(int n, int op, bool own_ptrs) {
-  if (!own_ptrs && op == MCCL_SUM && (n == 2 || n == 4 || n == 8)) return n;
+  if (!own_ptrs && (op == MCCL_SUM || op == MCCL_AVG) && (n == 2 || n == 4 || n == 8)) return n;
   return n < 4 ? n : 4;
 }
 
 // Resident wavefronts per CU of the stream shape.  Enough loads in flight to cover the memory
 // latency at full bandwidth (about 14 MB over the chip), and no more: every further wavefront
 // widens the window of live tiles and costs DRAM page locality.  Measured optima on MI355X
-// (bf16, 64 MiB per rank, warm and rotating through 9 GiB): with all loads of a tile in flight
-// 7-8 wavefronts for 8 ranks (6 falls off a cliff: 75 % of peak against 87 %), 12 for 4 ranks, no
-// cap for 2; with loads in groups of four 14, with three 24.
+// (bf16, 64 MiB per rank, one buffer set and rotating through several GiB): 7-8 wavefronts when
+// a wavefront keeps 8 loads in flight (6 falls off a cliff: 75 % of peak against 87 %), 12 with 4
+// (also the generic path, which loads in groups of four), 14 with 3, no cap with 2 or 1.
 long long stream_waves(int n, int op, bool own_ptrs) {
   if (g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU] > 0) return g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU];
-  const int in_flight = loads_in_flight(n, op, own_ptrs);
-  if (in_flight == 8) return 8;
-  if (in_flight == 4) return in_flight == n ? 12 : 14;
-  if (in_flight == 3) return 24;
-  return kMaxWavesPerCu;
+  switch (loads_in_flight(n, op, own_ptrs)) {
+    case 8: return 8;
+    case 4: return 12;
+    case 3: return 14;
+    default: return kMaxWavesPerCu;
+  }
 }
 
 // Geometry of a vector launch over njobs jobs whose largest has max_count elements.
