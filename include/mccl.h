@@ -59,16 +59,18 @@ typedef enum {
 /* Launch shape of the reduction (the reference switches at SMALL_MAX_COUNT between a
  * single-launch kernel and a persistent one, src/gpu/dpcpp_ccl.cpp:771-775). */
 typedef enum {
-  MCCL_VARIANT_AUTO = 0,       /* pick by size: SMALL up to MCCL_TUNE_SMALL_MAX_BYTES per rank,
-                                  STREAM once (n+1)*bytes reaches MCCL_TUNE_STREAM_MIN_TOTAL_BYTES
-                                  (the working set no longer fits the 256 MB Infinity Cache),
-                                  PERSISTENT in between */
+  MCCL_VARIANT_AUTO = 0,       /* pick by size: SMALL up to MCCL_TUNE_SMALL_MAX_BYTES per rank
+                                  (4 MiB), STREAM once (n+1)*bytes reaches
+                                  MCCL_TUNE_STREAM_MIN_TOTAL_BYTES (112 MiB); in between
+                                  PERSISTENT for 4 ranks or more, SMALL for fewer.  Whatever the
+                                  shape, outputs of launches beyond those sizes are written with
+                                  streaming stores, smaller ones stay cacheable */
   MCCL_VARIANT_SMALL = 1,      /* one wavefront per workgroup, one vector per lane, grid covers
                                   the message, no residency cap: lowest latency */
   MCCL_VARIANT_PERSISTENT = 2, /* fixed grid sized to the CUs, grid-stride loop */
   MCCL_VARIANT_STREAM = 3      /* SMALL's geometry with residency capped (through a dynamic-LDS
-                                  reservation) so that ~64 KiB of loads are in flight per CU:
-                                  highest bandwidth on large messages */
+                                  reservation) so that about 14 MB of loads are in flight over the
+                                  chip and no more: highest bandwidth on large messages */
 } mccl_variant_t;
 
 /* Tuning knobs for mccl_set_tuning (process-wide; meant for benchmarks and sweeps). */
