@@ -83,7 +83,9 @@ typedef enum {
   MCCL_TUNE_COPY_WAVES_PER_CU = 3,        /* residency cap of the segmented copy */
   MCCL_TUNE_STREAM_MIN_TOTAL_BYTES = 4,   /* (n+1)*bytes from which AUTO picks STREAM */
   MCCL_TUNE_COMBINE_PIECES_PER_WAVE = 5,  /* 1 KiB row pieces one wavefront of moe_combine walks */
-  MCCL_TUNE_COMBINE_WAVES_PER_CU = 6,     /* residency cap of moe_combine; default 0 = none */
+  MCCL_TUNE_COMBINE_WAVES_PER_CU = 6,     /* moe_combine with top-k <= 8: default 0 = one wavefront per
+                                             row chunk; > 0 = persistent grid of that many wavefronts
+                                             per CU, each walking several chunks (measured slower) */
   MCCL_TUNE_COUNT_ = 7
 } mccl_tune_t;
 

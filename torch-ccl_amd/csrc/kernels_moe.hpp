@@ -94,26 +94,34 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
   constexpr int G = 8;  // row loads in flight per lane (one group covers top-8 routing)
   const uint32_t total = a.tokens * a.waves_per_row;
   const size_t row_stride = (size_t)a.row_vecs * 16;
-  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
-    const uint32_t tok = chunk / a.waves_per_row;
-    const uint32_t part = chunk - tok * a.waves_per_row;
-    const uint32_t p0 = part * a.pieces_per_wave;
-    const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
-    const size_t e0 = (size_t)tok * a.topk;
-    if constexpr (FAST) {
-      // The token's routing entries are looked up once for all pieces this wavefront walks: lane g
-      // loads entry g (three loads in flight at once), and the values are broadcast into scalar
-      // registers, so that everything derived from them (the peer pointer picked from the argument
-      // block, the bounds checks, the row address) is scalar work and the row loads start after
-      // one memory round trip instead of two.
-      int my_rank = -1;
-      int64_t my_row = 0;
-      float my_w = 0.0f;
-      if (threadIdx.x < a.topk) {
-        my_rank = a.src_rank[e0 + threadIdx.x];
-        my_row = a.src_row[e0 + threadIdx.x];
-        my_w = a.w[e0 + threadIdx.x];
+  if constexpr (FAST) {
+    // The token's routing entries are looked up once for all pieces a wavefront walks: lane g
+    // loads entry g (three loads in flight at once), and the values are broadcast into scalar
+    // registers, so that everything derived from them (the peer pointer picked from the argument
+    // block, the bounds checks, the row address) is scalar work and the row loads start after
+    // one memory round trip instead of two.  With a grid smaller than the number of chunks a
+    // wavefront walks several chunks and looks up the next chunk's entries while it streams the
+    // rows of the current one.
+    auto issue_routing = [&](uint32_t c, int& rk, int64_t& rw, float& wt) {
+      rk = -1;
+      rw = 0;
+      wt = 0.0f;
+      if (c < total && threadIdx.x < a.topk) {
+        const size_t e = (size_t)(c / a.waves_per_row) * a.topk + threadIdx.x;
+        rk = a.src_rank[e];
+        rw = a.src_row[e];
+        wt = a.w[e];
       }
+    };
+    int my_rank;
+    int64_t my_row;
+    float my_w;
+    issue_routing(blockIdx.x, my_rank, my_row, my_w);
+    for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+      const uint32_t tok = chunk / a.waves_per_row;
+      const uint32_t part = chunk - tok * a.waves_per_row;
+      const uint32_t p0 = part * a.pieces_per_wave;
+      const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
       const u32x4* src[G];
       bool ok[G];
       float wk[G];
@@ -164,6 +172,10 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
       };
       VecU<DT> xa[G], xb[G];
       load_piece(p0, xa);
+      int next_rank;
+      int64_t next_row;
+      float next_w;
+      issue_routing(chunk + gridDim.x, next_rank, next_row, next_w);  // behind this chunk's first rows
       for (uint32_t piece = p0; piece < p1; piece += 2) {
         if (piece + 1 < p1) load_piece(piece + 1, xb);
         finish_piece(piece, xa);
@@ -172,7 +184,17 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
           finish_piece(piece + 1, xb);
         }
       }
-    } else {
+      my_rank = next_rank;
+      my_row = next_row;
+      my_w = next_w;
+    }
+  } else {
+    for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+      const uint32_t tok = chunk / a.waves_per_row;
+      const uint32_t part = chunk - tok * a.waves_per_row;
+      const uint32_t p0 = part * a.pieces_per_wave;
+      const uint32_t p1 = (p0 + a.pieces_per_wave < a.pieces_per_row) ? p0 + a.pieces_per_wave : a.pieces_per_row;
+      const size_t e0 = (size_t)tok * a.topk;
       // general top-k: groups of G entries per piece
       for (uint32_t piece = p0; piece < p1; ++piece) {
         const uint32_t v = piece * kWave + threadIdx.x;

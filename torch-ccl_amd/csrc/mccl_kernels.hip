@@ -77,6 +77,9 @@ int fail(int code, const char* fmt, ...) {
 // tuning state and per-device facts
 // ------------------------------------------------------------------------------------------
 constexpr unsigned kMaxGridX = 1u << 24;  // larger messages wrap through the grid-stride loop
+// Chunk counters are 32 bits wide and advance by the grid size: the limit leaves room for the
+// last step past the end.
+constexpr uint64_t kMaxChunks = 0xf0000000ull;
 constexpr size_t kLdsPerCu = 160 * 1024;  // gfx950
 constexpr int kMaxWavesPerCu = 32;
 
@@ -426,7 +429,7 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
       cs.last = (uint32_t)(body % kCopyChunk);
       uint64_t c = nfull + (cs.last ? 1 : 0);
       if (c == 0) c = 1;  // head only: chunk 0 still has to run
-      if (nfull > 0xfffffff0ull || chunks + c > 0xffffffffull) {
+      if (nfull > 0xf0000000ull || chunks + c > kMaxChunks) {
         if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "segment %d too large", i);
         break;
       }
@@ -477,7 +480,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
         return fail(MCCL_ERR_INVALID_ARG, "gather segment %d has too many rows", i);
       if ((uintptr_t)g.idx % 8) return fail(MCCL_ERR_INVALID_ARG, "row index table %d is not 8-byte aligned", i);
       const uint64_t c = (uint64_t)g.nrows * ppr;
-      if (chunks + c > 0xffffffffull) {
+      if (chunks + c > kMaxChunks) {
         if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "gather segment %d too large", i);
         break;
       }
@@ -788,7 +791,7 @@ int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const in
   }
   const size_t row_vecs = row_bytes / 16;
   const size_t ppr = (row_vecs + kWave - 1) / kWave;
-  if (tokens * ppr > 0xffffffffull || row_vecs > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  if (tokens * ppr > kMaxChunks || row_vecs > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
   a.src_rank = src_rank;
   a.src_row = src_row;
   a.w = weights;
@@ -806,13 +809,18 @@ int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const in
   int cus = 0;
   int rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
+  // One wavefront per chunk of a row, no residency cap (5.7 TB/s uncapped, 5.1 at 8 wavefronts
+  // per CU).  Measured and not adopted: a persistent grid whose wavefronts look up the next
+  // chunk's routing entries while they stream the current rows (the knob below; 3-8 % slower at
+  // every grid size, so the lookup is not what bounds the kernel), and one contiguous range of
+  // tokens per XCD so that the wavefronts sharing routing entries meet in one L2 (9 % slower).
   uint64_t grid = (uint64_t)tokens * a.waves_per_row;
   if (grid > kMaxGridX) grid = kMaxGridX;
-  // Wavefronts here live longer than in the plain reduction (routing-table lookups before the
-  // row loads), and more of them are needed to cover that latency: measured best without a
-  // residency cap (5.7 TB/s uncapped, 5.1 at 8 wavefronts per CU).  Giving each XCD one contiguous
-  // range of tokens, so that the wavefronts sharing routing entries meet in one L2, is 9 % slower.
-  const unsigned lds = g_tune[MCCL_TUNE_COMBINE_WAVES_PER_CU] > 0 ? lds_for_waves(g_tune[MCCL_TUNE_COMBINE_WAVES_PER_CU]) : 0;
+  if (topk <= 8 && g_tune[MCCL_TUNE_COMBINE_WAVES_PER_CU] > 0) {
+    const uint64_t persistent = (uint64_t)cus * (uint64_t)g_tune[MCCL_TUNE_COMBINE_WAVES_PER_CU];
+    if (grid > persistent) grid = persistent;
+  }
+  const unsigned lds = 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 g3((unsigned)grid), b3(kWave);
   const bool fast = topk <= 8;
