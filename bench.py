@@ -203,7 +203,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,moe,variants,ceilings,gloo,backend,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,moe,variants,ceilings,lists,gloo,backend,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -214,7 +214,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,moe,variants,ceilings,gloo,backend".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,moe,variants,ceilings,lists,gloo,backend".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import importlib.util
@@ -371,6 +371,50 @@ def main():
             ev[vname] = {"us": round(us, 1), "GBps": round(alg_bytes / us / 1e3, 1)}
         result["c3_shapes"] = ev
         log("C3 shapes:", json.dumps(ev))
+
+    # ---------------- coalesced and list forms: one fused launch against one launch per tensor ----------------
+    if "lists" in extras:
+        def timed_us(fn, reps=20):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / reps
+        nb, cnt = 32, 256 * 1024  # 32 gradient tensors of 512 KiB (bf16) on each of 8 ranks
+        buckets = [make_rank_buffers(torch, N, cnt, torch.bfloat16, 0.02, dev, on_device=True) for _ in range(nb)]
+        bouts = [torch.empty(cnt, dtype=torch.bfloat16, device=dev) for _ in range(nb)]
+        # argument tables built once: the timed loops are the C ABI calls alone
+        L = capi.lib()
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        all_in = capi.ptr_table([t.data_ptr() for b in buckets for t in b])
+        all_out = capi.ptr_table([o.data_ptr() for o in bouts])
+        counts = capi.size_table([cnt] * nb)
+        per_in = [capi.ptr_table([t.data_ptr() for t in b]) for b in buckets]
+        per_out = [ctypes.c_void_p(o.data_ptr()) for o in bouts]
+        us_fused = timed_us(lambda: L.mccl_reduce_multi(all_in, N, all_out, counts, nb, capi.BF16, capi.SUM, st))
+        fused_copy = [t.clone() for t in bouts]
+        us_each = timed_us(lambda: [L.mccl_reduce_n(per_in[b], N, per_out[b], cnt, capi.BF16, capi.SUM,
+                                                    capi.VARIANT_AUTO, st) for b in range(nb)])
+        same = all(torch.equal(x.view(torch.int16), y.view(torch.int16)) for x, y in zip(fused_copy, bouts))
+        pieces = [torch.randn(cnt * (1 + k % 3), device=dev).to(torch.bfloat16) for k in range(16)]
+        flat = torch.empty(sum(t.numel() for t in pieces), dtype=torch.bfloat16, device=dev)
+        us_pack = timed_us(lambda: mccl.pack(pieces, flat))
+        us_copy_ = timed_us(lambda: [flat[o:o + t.numel()].copy_(t) for o, t in
+                                     zip([sum(p.numel() for p in pieces[:i]) for i in range(len(pieces))], pieces)])
+        result["coalesced_and_list_forms"] = {
+            "note": "HIP events around 20 repetitions; reduce calls go straight to the C ABI with prebuilt argument tables, pack/copy through the Python front ends",
+            "allreduce_coalesced_32x512KiB_8ranks": {"fused_launches_us": round(us_fused, 1),
+                                                      "one_launch_per_tensor_us": round(us_each, 1),
+                                                      "bit_identical": same},
+            "pack_16_tensors_%dMiB" % (flat.numel() * 2 >> 20): {"fused_pack_us": round(us_pack, 1),
+                                                                  "torch_copy_per_tensor_us": round(us_copy_, 1)}}
+        log("lists:", json.dumps(result["coalesced_and_list_forms"]))
+        del buckets, bouts, fused_copy, pieces, flat
 
     # ---------------- C1: fp32, 2 ranks, 16 MiB ----------------
     if "c1" in extras:
