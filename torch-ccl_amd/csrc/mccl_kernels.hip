@@ -38,6 +38,7 @@
 //       (src/gpu/dpcpp_ccl.cpp:1505-1538)
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -83,8 +84,9 @@ constexpr uint64_t kMaxChunks = 0xf0000000ull;
 constexpr size_t kLdsPerCu = 160 * 1024;  // gfx950
 constexpr int kMaxWavesPerCu = 32;
 
-// tunables (mccl_set_tuning); defaults come from sweeps on MI355X
-long long g_tune[MCCL_TUNE_COUNT_] = {
+// tunables (mccl_set_tuning); defaults come from sweeps on MI355X.  Read by every launch and
+// written by whoever sweeps them, possibly from another thread: relaxed atomics.
+constexpr long long kTuneDefault[MCCL_TUNE_COUNT_] = {
     /* PERSISTENT_BLOCKS_PER_CU */ 8,
     /* STREAM_WAVES_PER_CU      */ 0,
     /* SMALL_MAX_BYTES          */ 4 << 20,
@@ -93,7 +95,15 @@ long long g_tune[MCCL_TUNE_COUNT_] = {
     /* COMBINE_PIECES_PER_WAVE  */ 2,
     /* COMBINE_WAVES_PER_CU     */ 0,
 };
-const long long g_tune_default[MCCL_TUNE_COUNT_] = {8, 0, 4 << 20, 28, 112ll << 20, 2, 0};
+struct TuneTable {
+  std::atomic<long long> v[MCCL_TUNE_COUNT_];
+  TuneTable() {
+    for (int i = 0; i < MCCL_TUNE_COUNT_; ++i) v[i].store(kTuneDefault[i], std::memory_order_relaxed);
+  }
+  long long operator[](int knob) const { return v[knob].load(std::memory_order_relaxed); }
+  void set(int knob, long long value) { v[knob].store(value, std::memory_order_relaxed); }
+};
+TuneTable g_tune;
 
 // Dynamic-LDS bytes that limit residency to `waves` single-wavefront workgroups per CU
 // (0 = no reservation needed).
@@ -523,7 +533,7 @@ size_t mccl_dtype_size(int dtype) { return dtype_size(dtype); }
 
 int mccl_set_tuning(int knob, long long value) {
   if (knob < 0 || knob >= MCCL_TUNE_COUNT_) return fail(MCCL_ERR_INVALID_ARG, "unknown tuning knob %d", knob);
-  g_tune[knob] = value > 0 ? value : g_tune_default[knob];
+  g_tune.set(knob, value > 0 ? value : kTuneDefault[knob]);
   return MCCL_OK;
 }
 
