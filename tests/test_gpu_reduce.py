@@ -387,3 +387,35 @@ def test_concurrent_callers_on_their_own_streams(mccl):
         t.join()
     torch.cuda.synchronize()
     assert not errors, errors
+
+
+# ---- large launches write their output with streaming stores: every dtype through that path ----
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES, ids=str)
+def test_reduce_streamed_output_all_dtypes(mccl, dtype):
+    """Two ranks, a little over 5 MiB per rank (beyond the size up to which outputs stay cacheable),
+    odd element count so that the peeled tail runs as well; all three launch shapes."""
+    es = torch.empty(0, dtype=dtype).element_size()
+    count = (5 << 20) // es + 3
+    ins = [rank_buffer(count, dtype, r) for r in range(2)]
+    want = oracle_reduce_bits(ins)
+    for variant in (0, 1, 2, 3):
+        got = _run(mccl, ins, O.SUM, variant)
+        assert_bits_equal(bits(got), want, "%s variant %d" % (dtype, variant))
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float64], ids=str)
+@pytest.mark.parametrize("opname", ["sum", "max"])
+def test_reduce_eight_ranks_beyond_the_stream_threshold(mccl, dtype, opname):
+    """8 ranks x 16 MiB (144 MiB per launch: the stream shape with its streaming stores), for the
+    compile-time rank count (sum) and the generic path (max)."""
+    es = torch.empty(0, dtype=dtype).element_size()
+    count = (16 << 20) // es
+    ins = [rank_buffer(count, dtype, r) for r in range(8)]
+    O.set_threads(min(16, O.max_threads()))
+    try:
+        want = oracle_reduce_bits(ins, OPS[opname])
+    finally:
+        O.set_threads(1)
+    got = _run(mccl, ins, OPS[opname])
+    assert_bits_equal(bits(got), want, "%s %s" % (dtype, opname))
