@@ -59,9 +59,14 @@ __device__ __forceinline__ void reduce_one(const ARGS& a, int p0, int n, size_t 
   ((S*)out)[idx] = Elem<DT>::store(acc);
 }
 
-// Loads one 16-byte vector; GUARD adds the bounds check of the last, partial tile.
+// Loads one 16-byte vector; GUARD adds the bounds check of the last, partial tile.  The vector body
+// is aligned on the output; an input that is not congruent with it mod 16 is read at whatever
+// alignment its elements have (global loads may be unaligned on this target: the hardware splits
+// them), hence the under-aligned pointer type.  Aligned inputs get the same instruction.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+
 template <bool GUARD>
-__device__ __forceinline__ u32x4 load_vec(const u32x4* p, size_t v, size_t nvec) {
+__device__ __forceinline__ u32x4 load_vec(const u32x4_unaligned* p, size_t v, size_t nvec) {
   if constexpr (GUARD) {
     if (v >= nvec) return (u32x4){0u, 0u, 0u, 0u};
   }
@@ -99,7 +104,7 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
     VecU<DT> x[NT][U];
 #pragma unroll
     for (int k = 0; k < NT; ++k) {
-      const u32x4* iv = (const u32x4*)(a.ptr[p0 + k] + in_byte_off);
+      const u32x4_unaligned* iv = (const u32x4_unaligned*)(a.ptr[p0 + k] + in_byte_off);
 #pragma unroll
       for (int u = 0; u < U; ++u) x[k][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
     }
@@ -124,7 +129,7 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         if (kb + g < n) {
-          const u32x4* iv = (const u32x4*)(a.ptr[p0 + kb + g] + in_byte_off);
+          const u32x4_unaligned* iv = (const u32x4_unaligned*)(a.ptr[p0 + kb + g] + in_byte_off);
 #pragma unroll
           for (int u = 0; u < U; ++u) x[g][u].v = load_vec<GUARD>(iv, v0 + (size_t)u * BLOCK, nvec);
         }
@@ -160,8 +165,8 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
   }
 }
 
-// Vector kernel.  Requires, for each job, all input pointers (+offset) and the output
-// pointer congruent mod 16.  The output may be exactly one of the inputs: a lane reads
+// Vector kernel.  The host aligns the vector body on the output; inputs need element alignment
+// only.  The output may be exactly one of the inputs: a lane reads
 // element i of every input before it writes element i, and no other lane touches i.
 // OWN: each job has its own n pointers (coalesced reductions); otherwise all jobs share
 // ptr[0..n) and the pointer loads do not wait for the job record.
@@ -198,21 +203,6 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
     reduce_tile<DT, OP, NT, U, BLOCK, false>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n, stream_out);
   if (tile == full_tiles && partial)  // the one partial tile; exactly one workgroup reaches it
     reduce_tile<DT, OP, NT, U, BLOCK, true>(a, p0, in_off + body_off, ov, (size_t)tile * TILE + threadIdx.x, nvec, n, stream_out);
-}
-
-// Element-wise kernel for pointer sets that are not congruent mod 16 (any alignment that is a
-// multiple of the element size).  Grid-stride over elements.
-template <int DT, int OP, bool OWN, typename ARGS>
-__global__ __launch_bounds__(256) void reduce_elem_kernel(const ARGS a) {
-  const int jid = blockIdx.y;
-  int p0 = 0;
-  if constexpr (OWN) p0 = a.job_ptr0[jid];
-  const size_t in_off = a.job[jid].in_off;
-  char* out = a.job[jid].out;
-  const size_t count = a.job[jid].nvec;  // element count for this kernel
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
-    reduce_one<DT, OP>(a, p0, a.n, in_off, out, i);
 }
 
 }  // namespace

@@ -26,11 +26,12 @@
 //                  Slower than "stream" on large messages (the workgroups drift apart and
 //                  the live window smears) but a few percent ahead while the whole working
 //                  set fits the 256 MB Infinity Cache, which is where AUTO uses it;
-//   * misaligned heads/tails are peeled element-wise inside the same launch; pointer sets
-//     that are not mutually congruent mod 16 take an element-wise kernel.
+//   * misaligned heads/tails are peeled element-wise inside the same launch up to the first
+//     16-byte boundary of the output; inputs that are not congruent with the output mod 16
+//     are read with unaligned vector loads (the hardware splits them).
 //
 // What each kernel replaces in the reference (intel/torch-ccl):
-//   reduce_vec_kernel / reduce_elem_kernel : the N-peer sum of src/gpu/allreduce_small.h:289-361,
+//   reduce_vec_kernel : the N-peer sum of src/gpu/allreduce_small.h:289-361,
 //       the five data kernels of src/gpu/allreduce.h:306-533, ccl::allreduce /
 //       ccl::reduce_scatter call sites in src/gpu/dpcpp_ccl.cpp:781-788, 1002-1008
 //   copy_segments_kernel : ccl::allgatherv / ccl::alltoall(v) data movement
@@ -153,7 +154,7 @@ size_t dtype_size(int dt) {
   }
 }
 
-enum Shape { kShapeSmall, kShapeStream, kShapePersistent, kShapeElem };
+enum Shape { kShapeSmall, kShapeStream, kShapePersistent };
 
 // Geometry of a launch.
 struct Geometry {
@@ -194,11 +195,6 @@ hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStre
 
 template <int DT, int OP>
 hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
-  if (g.shape == kShapeElem) {
-    if (g.own_ptrs) hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, true, ReduceArgs>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((reduce_elem_kernel<DT, OP, false, ReduceArgs>), dim3(g.grid_x, njobs, 1), dim3(256), 0, s, a);
-    return hipGetLastError();
-  }
   if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
   if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {  // the ops of gradient reductions
     switch (a.n) {
@@ -323,51 +319,37 @@ struct JobSpec {
   int ptr0;
 };
 
-// Launch one batch of jobs.  a.ptr / a.n are populated; specs describe the jobs.  Jobs whose
-// pointers are congruent mod 16 go to the vector kernel; the rest to the element kernel, in
-// at most two launches.
+// Launch one batch of jobs.  a.ptr / a.n are populated; specs describe the jobs.  The vector
+// body of a job starts at the first 16-byte boundary of its output; inputs need element alignment
+// only.
 int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int op, int variant,
                 bool own_ptrs, hipStream_t s) {
   const size_t es = dtype_size(dtype);
   const size_t ve = 16 / es;
-  ReduceArgs elem = a;  // the vector launch reuses `a`
-  int nv = 0, ne = 0;
-  size_t vmax = 0, emax = 0;
+  int nv = 0;
+  size_t vmax = 0;
   for (int j = 0; j < njobs; ++j) {
     const JobSpec& sp = specs[j];
     if (sp.count == 0) continue;
     const uintptr_t o = (uintptr_t)sp.out;
     if (o % es) return fail(MCCL_ERR_INVALID_ARG, "output pointer not aligned to the element size");
-    bool congruent = true;
     for (int k = 0; k < a.n; ++k) {
       const uintptr_t p = (uintptr_t)(a.ptr[sp.ptr0 + k] + sp.in_off);
       if (p % es) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d not aligned to the element size", k);
-      if ((p & 15u) != (o & 15u)) congruent = false;
     }
-    if (congruent) {
-      size_t head = ((16u - (unsigned)(o & 15u)) & 15u) / es;
-      if (head > sp.count) head = sp.count;
-      const size_t nvec = (sp.count - head) / ve;
-      if (nvec / kWave > 0xfffffff0ull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
-      ReduceJob& jb = a.job[nv];
-      jb.out = sp.out;
-      jb.in_off = sp.in_off;
-      jb.nvec = nvec;
-      jb.head = (uint32_t)head;
-      jb.tail = (uint32_t)(sp.count - head - nvec * ve);
-      a.job_ptr0[nv] = sp.ptr0;
-      ++nv;
-      if (sp.count > vmax) vmax = sp.count;
-    } else {
-      ReduceJob& jb = elem.job[ne];
-      jb.out = sp.out;
-      jb.in_off = sp.in_off;
-      jb.nvec = sp.count;  // the element kernel reads this field as the element count
-      jb.head = jb.tail = 0;
-      elem.job_ptr0[ne] = sp.ptr0;
-      ++ne;
-      if (sp.count > emax) emax = sp.count;
-    }
+    size_t head = ((16u - (unsigned)(o & 15u)) & 15u) / es;
+    if (head > sp.count) head = sp.count;
+    const size_t nvec = (sp.count - head) / ve;
+    if (nvec / kWave > 0xf0000000ull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+    ReduceJob& jb = a.job[nv];
+    jb.out = sp.out;
+    jb.in_off = sp.in_off;
+    jb.nvec = nvec;
+    jb.head = (uint32_t)head;
+    jb.tail = (uint32_t)(sp.count - head - nvec * ve);
+    a.job_ptr0[nv] = sp.ptr0;
+    ++nv;
+    if (sp.count > vmax) vmax = sp.count;
   }
   if (nv) {
     Geometry g;
@@ -377,18 +359,6 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
     // caches (2-5 % of bandwidth); smaller ones stay cacheable for whoever reads them next
     a.flags = g.stream_out ? kFlagStreamOut : 0u;
     hipError_t e = launch_any(a, dtype, op, g, nv, s);
-    if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
-  }
-  if (ne) {
-    int cus = 0;
-    int rc = device_cus(&cus);
-    if (rc != MCCL_OK) return rc;
-    size_t blocks = (emax + 255) / 256;
-    size_t cap = (size_t)cus * 8 / ne;
-    if (cap < 1) cap = 1;
-    if (blocks > cap) blocks = cap;
-    Geometry g{kShapeElem, (unsigned)blocks, 256, 0, own_ptrs, false};
-    hipError_t e = launch_any(elem, dtype, op, g, ne, s);
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   }
   return MCCL_OK;
