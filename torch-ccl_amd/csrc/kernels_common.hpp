@@ -23,6 +23,9 @@ constexpr size_t kCopyChunk = (size_t)kWave * 16 * kCopyUnroll;  // 2 KiB per wa
 // element types
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// The same vector behind a pointer that promises no alignment: global loads may be unaligned on
+// this target (the hardware splits them), and an aligned address gets the same instruction.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
 
 __device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }

@@ -8,15 +8,15 @@
 namespace {
 
 // One segment as the kernel sees it.  The host splits it into a head (bytes up to the first
-// 16- or 4-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of
-// `last` bytes, so that the device needs 32-bit uniform arithmetic only.
+// 16-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of `last`
+// bytes, so that the device needs 32-bit uniform arithmetic only.
 struct CopySeg {
   const char* src;
   char* dst;
   uint32_t head;   // bytes before the body
   uint32_t nfull;  // full chunks in the body
   uint32_t last;   // bytes of the final partial chunk (0 = none)
-  uint32_t mode;   // 0: 16-byte vectors, 1: dwords, 2: bytes
+  uint32_t pad_;
 };
 
 struct CopyArgs {
@@ -26,8 +26,9 @@ struct CopyArgs {
 };
 
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
-// handed out in order.  When src and dst are congruent mod 16 the body moves as 16-byte
-// vectors (non-temporal both ways for full chunks), mod 4 as dwords, else as bytes.
+// handed out in order.  The body moves as 16-byte vectors aligned on dst (non-temporal both
+// ways for full chunks); a source that is not congruent with dst mod 16 is read with unaligned
+// vector loads.
 __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
@@ -40,7 +41,6 @@ __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) 
     const uint32_t c = chunk - a.chunk_prefix[lo];
     const uint32_t head = a.seg[lo].head;
     const uint32_t nfull = a.seg[lo].nfull;
-    const uint32_t mode = a.seg[lo].mode;
     const uint32_t len = (c < nfull) ? (uint32_t)kCopyChunk : a.seg[lo].last;
     const uint32_t t = threadIdx.x;
     const char* src = a.seg[lo].src;
@@ -50,30 +50,19 @@ __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) 
     src += off;
     dst += off;
 
-    if (mode == 0) {
-      const u32x4* sv = (const u32x4*)src;
-      u32x4* dv = (u32x4*)dst;
-      if (len == (uint32_t)kCopyChunk) {
-        u32x4 x[kCopyUnroll];
+    const u32x4_unaligned* sv = (const u32x4_unaligned*)src;
+    u32x4* dv = (u32x4*)dst;
+    if (len == (uint32_t)kCopyChunk) {
+      u32x4 x[kCopyUnroll];
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
+      for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
-      } else {
-        const uint32_t nv = len >> 4;
-        for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
-        const uint32_t rem = len & 15u;
-        if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
-      }
-    } else if (mode == 1) {
-      const uint32_t* sw = (const uint32_t*)src;
-      uint32_t* dw = (uint32_t*)dst;
-      const uint32_t nw = len >> 2;
-      for (uint32_t v = t; v < nw; v += kWave) dw[v] = sw[v];
-      const uint32_t rem = len & 3u;
-      if (t < rem) dst[(nw << 2) + t] = src[(nw << 2) + t];
+      for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
     } else {
-      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
+      const uint32_t nv = len >> 4;
+      for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
+      const uint32_t rem = len & 15u;
+      if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
     }
   }
 }

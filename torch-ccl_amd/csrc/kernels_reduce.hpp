@@ -63,7 +63,6 @@ __device__ __forceinline__ void reduce_one(const ARGS& a, int p0, int n, size_t 
 // is aligned on the output; an input that is not congruent with it mod 16 is read at whatever
 // alignment its elements have (global loads may be unaligned on this target: the hardware splits
 // them), hence the under-aligned pointer type.  Aligned inputs get the same instruction.
-typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
 
 template <bool GUARD>
 __device__ __forceinline__ u32x4 load_vec(const u32x4_unaligned* p, size_t v, size_t nvec) {

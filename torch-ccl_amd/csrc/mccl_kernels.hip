@@ -393,15 +393,12 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
       const mccl_segment_t& sg = segs[i];
       if (sg.bytes == 0) { ++i; continue; }
       if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
-      const uintptr_t sp = (uintptr_t)sg.src, dp = (uintptr_t)sg.dst;
-      const unsigned diff = (unsigned)((sp ^ dp) & 15u);
+      const uintptr_t dp = (uintptr_t)sg.dst;
       CopySeg cs;
       cs.src = (const char*)sg.src;
       cs.dst = (char*)sg.dst;
-      size_t head;
-      if (diff == 0) { cs.mode = 0; head = (16u - (unsigned)(dp & 15u)) & 15u; }
-      else if ((diff & 3u) == 0) { cs.mode = 1; head = (4u - (unsigned)(dp & 3u)) & 3u; }
-      else { cs.mode = 2; head = 0; }
+      cs.pad_ = 0;
+      size_t head = (16u - (unsigned)(dp & 15u)) & 15u;  // the body is aligned on dst
       if (head > sg.bytes) head = sg.bytes;
       const size_t body = sg.bytes - head;
       const uint64_t nfull = body / kCopyChunk;
