@@ -8,7 +8,7 @@
 namespace {
 
 // One segment as the kernel sees it.  The host splits it into a head (bytes up to the first
-// 16-byte boundary of dst), `nfull` chunks of kCopyChunk bytes and one last chunk of `last`
+// 128-byte boundary of dst: the body starts on a cache line), `nfull` chunks of kCopyChunk bytes and one last chunk of `last`
 // bytes, so that the device needs 32-bit uniform arithmetic only.
 struct CopySeg {
   const char* src;
@@ -45,7 +45,8 @@ __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) 
     const uint32_t t = threadIdx.x;
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
-    if (c == 0 && t < head) dst[t] = src[t];
+    if (c == 0)
+      for (uint32_t i = t; i < head; i += kWave) dst[i] = src[i];  // head < 128
     const size_t off = (size_t)head + (size_t)c * kCopyChunk;  // start of this chunk
     src += off;
     dst += off;

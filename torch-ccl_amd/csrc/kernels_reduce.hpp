@@ -10,14 +10,14 @@ namespace {
 
 // One reduction of a launch, fully described by the host so that a wavefront needs one
 // scalar load to start and 32-bit uniform arithmetic only:
-//   elements [0, head)                      peeled, element-wise (out not yet 16-byte aligned)
+//   elements [0, head)                      peeled, element-wise (out not yet 128-byte aligned)
 //   vectors  [0, nvec) at byte offset head*es   the vector body
 //   elements [head + nvec*VE, +tail)        peeled, element-wise
 struct ReduceJob {
   char* out;
   size_t in_off;   // byte offset applied to every input pointer
   size_t nvec;     // 16-byte vectors in the body
-  uint32_t head;   // elements before the body (< 16)
+  uint32_t head;   // elements before the body (< 128): the body starts on a cache line of out
   uint32_t tail;   // elements after the body (< 16)
 };
 
@@ -186,8 +186,9 @@ __global__ __launch_bounds__(BLOCK) void reduce_vec_kernel(const ARGS a) {
 
   if (blockIdx.x == 0) {
     const uint32_t t = threadIdx.x;
-    if (t < head) reduce_one<DT, OP>(a, p0, n, in_off, out, t);
-    else if (t - head < tail) reduce_one<DT, OP>(a, p0, n, in_off, out, head + nvec * VE + (t - head));
+    // head < 128 and tail < 16 elements: a couple of strides of the workgroup at most
+    for (uint32_t i = t; i < head + tail; i += BLOCK)
+      reduce_one<DT, OP>(a, p0, n, in_off, out, i < head ? (size_t)i : (size_t)head + nvec * VE + (i - head));
   }
 
   const size_t body_off = (size_t)head * sizeof(S);  // bytes

@@ -320,7 +320,7 @@ struct JobSpec {
 };
 
 // Launch one batch of jobs.  a.ptr / a.n are populated; specs describe the jobs.  The vector
-// body of a job starts at the first 16-byte boundary of its output; inputs need element alignment
+// body of a job starts at the first 128-byte boundary of its output (full cache lines per tile); inputs need element alignment
 // only.
 int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int op, int variant,
                 bool own_ptrs, hipStream_t s) {
@@ -337,7 +337,7 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
       const uintptr_t p = (uintptr_t)(a.ptr[sp.ptr0 + k] + sp.in_off);
       if (p % es) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d not aligned to the element size", k);
     }
-    size_t head = ((16u - (unsigned)(o & 15u)) & 15u) / es;
+    size_t head = ((128u - (unsigned)(o & 127u)) & 127u) / es;  // the body starts on a cache line of out
     if (head > sp.count) head = sp.count;
     const size_t nvec = (sp.count - head) / ve;
     if (nvec / kWave > 0xf0000000ull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
@@ -398,7 +398,7 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
       cs.src = (const char*)sg.src;
       cs.dst = (char*)sg.dst;
       cs.pad_ = 0;
-      size_t head = (16u - (unsigned)(dp & 15u)) & 15u;  // the body is aligned on dst
+      size_t head = (128u - (unsigned)(dp & 127u)) & 127u;  // the body starts on a cache line of dst
       if (head > sg.bytes) head = sg.bytes;
       const size_t body = sg.bytes - head;
       const uint64_t nfull = body / kCopyChunk;
