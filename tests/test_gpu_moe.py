@@ -132,3 +132,23 @@ def test_combine_any_topk_with_skipped_entries(mccl, topk, hidden):
     want = O.moe_combine([to_carrier(t) for t in x], src_rank.numpy(), src_row.numpy(), w.numpy(),
                          tokens, topk, hidden, TORCH_TO_CODE[dtype])
     assert_bits_equal(bits(y), want.view(np.uint16), "combine topk %d hidden %d" % (topk, hidden))
+
+
+@pytest.mark.parametrize("row_bytes", [1, 15, 16, 17, 2047, 2048, 2049, 4099, 14338])
+@pytest.mark.parametrize("src_off,dst_off", [(0, 0), (1, 0), (0, 3), (5, 9)])
+def test_gather_rows_any_row_size_and_alignment(mccl, row_bytes, src_off, dst_off):
+    """Byte rows of every size class (below a vector, around one 2 KiB piece, several pieces with a
+    ragged end) gathered between buffers that start off any boundary; the bytes around the
+    destination must stay untouched."""
+    g = torch.Generator().manual_seed(row_bytes * 31 + src_off * 7 + dst_off)
+    rows, picks = 37, 90
+    src_buf = torch.randint(0, 255, (src_off + rows * row_bytes + 8,), generator=g, dtype=torch.uint8).to(DEV)
+    dst_buf = torch.full((dst_off + picks * row_bytes + 64,), 0xAB, dtype=torch.uint8, device=DEV)
+    src = src_buf[src_off:src_off + rows * row_bytes].view(rows, row_bytes)
+    dst = dst_buf[dst_off:dst_off + picks * row_bytes].view(picks, row_bytes)
+    idx = torch.randint(0, rows, (picks,), generator=g, dtype=torch.int64)
+    mccl.gather_rows(src, idx.to(DEV), out=dst)
+    torch.cuda.synchronize()
+    want = O.gather_rows(_u8(src), idx.numpy(), row_bytes)
+    assert_bits_equal(_u8(dst), want, "gather_rows %d bytes" % row_bytes)
+    assert int((dst_buf[:dst_off] != 0xAB).sum()) == 0 and int((dst_buf[dst_off + picks * row_bytes:] != 0xAB).sum()) == 0

@@ -21,7 +21,6 @@ struct GatherArgs {
   int nseg;
   uint32_t row_bytes;
   uint32_t pieces_per_row;  // ceil(row_bytes / kCopyChunk)
-  uint32_t vector_ok;       // all bases 16-byte aligned and row_bytes % 16 == 0
 };
 
 // One wavefront moves one 2 KiB piece of one row.  Chunks are numbered row-major within a
@@ -48,22 +47,26 @@ __global__ __launch_bounds__(kWave) void gather_rows_kernel(const GatherArgs a) 
     const char* src = a.seg[lo].src + (size_t)srow * row_bytes + off;
     char* dst = a.seg[lo].dst + (size_t)row * row_bytes + off;
     const uint32_t t = threadIdx.x;
-    if (a.vector_ok) {
-      const u32x4* sv = (const u32x4*)src;
-      u32x4* dv = (u32x4*)dst;
-      if (len == (uint32_t)kCopyChunk) {
-        u32x4 x[kCopyUnroll];
+    // 16-byte vectors aligned on the destination; bytes up to the first boundary and after the
+    // last whole vector; the source is read at whatever alignment it has
+    uint32_t head = (16u - (uint32_t)((uintptr_t)dst & 15u)) & 15u;
+    if (head > len) head = len;
+    if (t < head) dst[t] = src[t];
+    const uint32_t body = len - head;
+    const uint32_t nv = body >> 4;
+    const u32x4_unaligned* sv = (const u32x4_unaligned*)(src + head);
+    u32x4* dv = (u32x4*)(dst + head);
+    if (nv == (uint32_t)(kCopyChunk / 16)) {
+      u32x4 x[kCopyUnroll];
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) x[u] = sv[t + u * kWave];  // rows are re-read (top-k): cacheable
+      for (int u = 0; u < kCopyUnroll; ++u) x[u] = sv[t + u * kWave];  // rows are re-read (top-k): cacheable
 #pragma unroll
-        for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
-      } else {
-        const uint32_t nv = len >> 4;
-        for (uint32_t v = t; v < nv; v += kWave) __builtin_nontemporal_store(sv[v], &dv[v]);
-      }
+      for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
     } else {
-      for (uint32_t v = t; v < len; v += kWave) dst[v] = src[v];
+      for (uint32_t v = t; v < nv; v += kWave) __builtin_nontemporal_store((u32x4)sv[v], &dv[v]);
     }
+    const uint32_t rem = body & 15u;
+    if (t < rem) dst[head + (nv << 4) + t] = src[head + (nv << 4) + t];
   }
 }
 

@@ -447,7 +447,6 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
     GatherArgs a;
     int m = 0;
     uint64_t chunks = 0;
-    bool vec = (row_bytes % 16) == 0;
     a.chunk_prefix[0] = 0;
     while (i < nspec && m < kMaxSegs) {
       const GatherSpec& g = specs[i];
@@ -461,7 +460,6 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
         if (m == 0) return fail(MCCL_ERR_INVALID_ARG, "gather segment %d too large", i);
         break;
       }
-      if (((uintptr_t)g.src | (uintptr_t)g.dst) & 15u) vec = false;
       a.seg[m] = GatherSeg{(const char*)g.src, g.idx, (char*)g.dst, (uint32_t)g.nrows, (uint32_t)g.src_rows};
       chunks += c;
       a.chunk_prefix[++m] = (uint32_t)chunks;
@@ -471,7 +469,6 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
     a.nseg = m;
     a.row_bytes = (uint32_t)row_bytes;
     a.pieces_per_row = ppr;
-    a.vector_ok = vec ? 1u : 0u;
     int cus = 0;
     int rc = device_cus(&cus);
     if (rc != MCCL_OK) return rc;
