@@ -141,10 +141,10 @@ def test_pack_unpack_roundtrip(mccl, sizes):
 
 @pytest.mark.parametrize("src_off", [0, 1, 4, 7])
 @pytest.mark.parametrize("dst_off", [0, 2, 4, 9])
-@pytest.mark.parametrize("nbytes", [1, 5, 31, 16384 * 3 + 11])
+@pytest.mark.parametrize("nbytes", [1, 5, 31, 127, 129, 2048 + 130, 16384 * 3 + 11])
 def test_copy_segments_alignments(mccl, src_off, dst_off, nbytes):
-    """Every src/dst alignment class: congruent mod 16 (vector path), mod 4 (dword path),
-    neither (byte path); canaries around the destination stay untouched."""
+    """Every src/dst alignment class (congruent mod 16, mod 4, neither), sizes below one vector,
+    below one cache line and several chunks; canaries around the destination stay untouched."""
     rng = np.random.default_rng(src_off * 100 + dst_off * 10 + nbytes % 7)
     src = _bytes(rng, nbytes + 64).to(DEV)
     dst = torch.full((nbytes + 64,), 0xAB, dtype=torch.uint8, device=DEV)
@@ -204,3 +204,27 @@ def test_staggered_copies_keep_the_data_and_leave_the_power_of_two_spacing(mccl)
     out = mccl.reduce_n(st[:4], op=O.SUM)
     torch.cuda.synchronize()
     assert torch.equal(out, torch.full_like(out, 6.0))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_copy_many_random_segments_in_one_call(mccl, seed):
+    """300 segments of random size (0 .. 10 KiB) at random byte offsets in one call: more than one
+    kernel-argument table's worth, every alignment, empty segments in between.  The destination
+    ranges are disjoint; everything outside them keeps its canary."""
+    rng = np.random.default_rng(seed)
+    sizes = rng.integers(0, 10240, size=300)
+    sizes[rng.integers(0, 300, size=20)] = 0
+    gaps = rng.integers(1, 40, size=300)
+    src = _bytes(rng, int(sizes.sum()) + 4096).to(DEV)
+    dst = torch.full((int((sizes + gaps).sum()) + 64,), 0xCD, dtype=torch.uint8, device=DEV)
+    want = np.full(dst.numel(), 0xCD, dtype=np.uint8)
+    src_np = src.cpu().numpy()
+    segs, so, do = [], int(rng.integers(0, 16)), int(rng.integers(0, 16))
+    for sz, gap in zip(sizes.tolist(), gaps.tolist()):
+        segs.append((src.data_ptr() + so, dst.data_ptr() + do, sz))
+        want[do:do + sz] = src_np[so:so + sz]
+        so += sz
+        do += sz + gap
+    mccl.copy_segments(segs)
+    torch.cuda.synchronize()
+    assert_bits_equal(dst.cpu().numpy(), want, "random segments")
