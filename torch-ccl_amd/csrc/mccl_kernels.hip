@@ -8,8 +8,9 @@
 //     add so the memory system sees N*U independent requests per lane;
 //   * accumulation is a sequential ascending-rank chain held in registers (fp32 for
 //     f16/bf16), one round-to-nearest-even on store;
-//   * outputs are written with non-temporal stores (streamed past the caches): worth 2-5 %
-//     against plain stores, most on multi-GiB footprints;
+//   * large outputs are written with streaming stores (written through past the caches at
+//     agent scope): worth 2-5 % against plain stores, most on multi-GiB footprints; small
+//     outputs stay cacheable for their consumer;
 //   * inputs are read with non-temporal loads: nothing is reused, and on this part the
 //     streaming hint alone is worth about 12 % of bandwidth;
 //   * launch shapes (same kernel code, different geometry):
@@ -163,7 +164,7 @@ struct Geometry {
   int block;
   unsigned lds;   // dynamic LDS reservation (occupancy cap), bytes
   bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
-  bool stream_out;  // write the output with non-temporal stores
+  bool stream_out;  // write the output with streaming (write-through) stores
 };
 
 template <int DT, int OP, int NT, bool OWN, typename ARGS>
@@ -269,7 +270,7 @@ int plan_vec(size_t max_count, int njobs, int n, int dtype, int op, int variant,
   const size_t nvec = max_count / (16 / es) + 1;
   // Measured crossovers on MI355X.  Up to a few MiB per rank a launch is latency-bound: one
   // wavefront per tile, cacheable output.  From about 112 MiB of traffic per launch the capped
-  // in-order stream with a streamed (non-temporal) output wins by 3-15 %.  In between, four or
+  // in-order stream with a streamed (written-through) output wins by 3-15 %.  In between, four or
   // more ranks do best with the persistent grid and a cacheable output (the working set sits in
   // the Infinity Cache, where a streamed output costs up to 20 %); with fewer ranks the output is
   // a third or more of the traffic and streaming it pays from 8 MiB per rank on.
@@ -320,8 +321,8 @@ struct JobSpec {
 };
 
 // Launch one batch of jobs.  a.ptr / a.n are populated; specs describe the jobs.  The vector
-// body of a job starts at the first 128-byte boundary of its output (full cache lines per tile); inputs need element alignment
-// only.
+// body of a job starts at the first 128-byte boundary of its output (full cache lines per
+// tile); inputs need element alignment only.
 int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int op, int variant,
                 bool own_ptrs, hipStream_t s) {
   const size_t es = dtype_size(dtype);
