@@ -200,8 +200,8 @@ def gloo_baseline(world=8):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--extras", default="all",
                     help="comma list of c1,c2,c4,c5,moe,variants,ceilings,placement,lists,gloo,backend,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
