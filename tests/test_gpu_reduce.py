@@ -419,3 +419,37 @@ def test_reduce_eight_ranks_beyond_the_stream_threshold(mccl, dtype, opname):
         O.set_threads(1)
     got = _run(mccl, ins, OPS[opname])
     assert_bits_equal(bits(got), want, "%s %s" % (dtype, opname))
+
+
+# ---- seeded fuzz over every parameter at once ----
+
+@pytest.mark.parametrize("seed", range(6))
+def test_reduce_random_combinations(mccl, seed):
+    """25 random combinations per seed of dtype, op, rank count (1..20), element count, launch shape
+    and independent element offsets of every input and of the output inside padded buffers (so
+    that heads, tails, unaligned inputs and canaries all come into play together)."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(25):
+        dtype = ALL_DTYPES[int(rng.integers(0, len(ALL_DTYPES)))]
+        opname = ["sum", "prod", "min", "max"][int(rng.integers(0, 4))]
+        n = int(rng.integers(1, 21))
+        count = int(rng.choice([1, 7, 63, 64, 65, 1000, 4097, 70_001, 300_003]))
+        variant = int(rng.integers(0, 4))
+        pad = 80
+        offs = [int(rng.integers(0, pad)) for _ in range(n + 1)]
+        scale = 1.0 if opname == "prod" else 0.02
+        cpu = [rank_buffer(count, dtype, 100 * case + r, scale=scale) for r in range(n)]
+        dev = []
+        for r in range(n):
+            buf = torch.zeros(count + pad, dtype=dtype, device=DEV)
+            buf[offs[r]:offs[r] + count] = cpu[r].to(DEV)
+            dev.append(buf[offs[r]:offs[r] + count])
+        canary = rank_buffer(count + pad, dtype, 999, scale=scale).to(DEV)
+        out_buf = canary.clone()
+        out = out_buf[offs[n]:offs[n] + count]
+        mccl.reduce_n(dev, out=out, op=OPS[opname], variant=variant)
+        torch.cuda.synchronize()
+        what = "seed %d case %d: %s %s n=%d count=%d variant=%d offsets=%s" % (seed, case, dtype, opname, n, count, variant, offs)
+        assert_bits_equal(bits(out), oracle_reduce_bits(cpu, OPS[opname]), what)
+        assert_bits_equal(bits(out_buf[:offs[n]]), bits(canary[:offs[n]]), what + " (bytes before the output)")
+        assert_bits_equal(bits(out_buf[offs[n] + count:]), bits(canary[offs[n] + count:]), what + " (bytes after the output)")
