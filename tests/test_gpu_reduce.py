@@ -160,10 +160,11 @@ def test_reduce_nan_inputs(mccl, dtype):
         assert_bits_equal(bits(got), want, "nan canonical")
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64], ids=str)
-def test_reduce_avg(mccl, dtype):
-    """AVG = SUM chain, then one division by n in the accumulation type."""
-    n, count = 8, 4099
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES, ids=str)
+@pytest.mark.parametrize("n,count", [(2, 4099), (3, 4099), (4, 70_001), (8, 4099), (16, 1000), (8, 9 * (1 << 20) + 5)])
+def test_reduce_avg(mccl, dtype, n, count):
+    """AVG = SUM chain, then one division by n in the accumulation type; compile-time rank counts
+    (2, 4, 8), the generic path, and a size whose output is written with streaming stores."""
     ins = [rank_buffer(count, dtype, r) for r in range(n)]
     got = _run(mccl, ins, mccl.AVG)
     acc_t = torch.float64 if dtype == torch.float64 else torch.float32
@@ -171,7 +172,7 @@ def test_reduce_avg(mccl, dtype):
     for t in ins:
         acc = acc + t.to(acc_t)
     want = (acc / n).to(dtype)
-    assert_bits_equal(bits(got), bits(want), "avg %s" % dtype)
+    assert_bits_equal(bits(got), bits(want), "avg %s n=%d" % (dtype, n))
 
 
 def test_reduce_avg_rejects_integers(mccl):
