@@ -18,13 +18,18 @@ INCLUDE = os.path.join(ROOT, "include")
 LIB_DIR = os.path.join(os.path.dirname(HERE), "torch_ccl_amd", "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-KERNEL_SRC = os.path.join(HERE, "mccl_kernels.hip")
+KERNEL_SRC = os.path.join(HERE, "mccl_kernels.hip")          # planning, C ABI, copy and MoE kernels
+REDUCE_SRC = os.path.join(HERE, "mccl_reduce_dtype.hip")     # reduction kernels, one object per dtype
+REDUCE_DTYPES = range(9)                                      # mccl_dtype_t codes
 KERNEL_LIB = os.path.join(LIB_DIR, "libmi355ccl.so")
+KERNEL_HDRS = [os.path.join(INCLUDE, "mccl.h")] + [
+    os.path.join(HERE, h) for h in ("kernels_common.hpp", "kernels_reduce.hpp", "kernels_copy.hpp",
+                                    "kernels_moe.hpp", "reduce_launch.hpp")]
 
 # -ffp-contract=off / no fast-math: the reduction chain must round add by add.
 # packed-fp32 ops are switched off for all device code.
 HIP_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
@@ -39,14 +44,43 @@ def _stale(out, srcs):
     return any(os.path.getmtime(s) > t for s in srcs)
 
 
+def kernel_units():
+    """(source, extra flags, tag) of every translation unit of libmi355ccl.so."""
+    units = [(KERNEL_SRC, [], "main")]
+    units += [(REDUCE_SRC, ["-DMCCL_REDUCE_DT=%d" % dt], "dt%d" % dt) for dt in REDUCE_DTYPES]
+    return units
+
+
+def _run_parallel(cmds, jobs=8):
+    """Runs the command lines concurrently; raises with the first failure."""
+    from concurrent.futures import ThreadPoolExecutor
+    def run(cmd):
+        p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        return cmd, p.returncode, p.stdout
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(run, cmds))
+    for cmd, rc, out in results:
+        if rc != 0:
+            sys.stderr.write(out)
+            raise subprocess.CalledProcessError(rc, cmd)
+
+
 def build_kernels(force=False, extra_flags=(), out=KERNEL_LIB):
     os.makedirs(os.path.dirname(out), exist_ok=True)
-    srcs = [KERNEL_SRC, os.path.join(INCLUDE, "mccl.h")] + [
-        os.path.join(HERE, h) for h in ("kernels_common.hpp", "kernels_reduce.hpp", "kernels_copy.hpp",
-                                        "kernels_moe.hpp")]
-    if force or _stale(out, srcs):
-        cmd = [HIPCC] + HIP_FLAGS + list(extra_flags) + ["-o", out, KERNEL_SRC]
-        subprocess.check_call(cmd)
+    if not (force or _stale(out, [KERNEL_SRC, REDUCE_SRC] + KERNEL_HDRS)):
+        return out
+    obj_dir = out + ".objs"
+    os.makedirs(obj_dir, exist_ok=True)
+    objs, cmds = [], []
+    for src, flags, tag in kernel_units():
+        obj = os.path.join(obj_dir, tag + ".o")
+        objs.append(obj)
+        cmds.append([HIPCC] + HIP_FLAGS + list(flags) + list(extra_flags) + ["-c", "-o", obj, src])
+    _run_parallel(cmds)
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
+    for obj in objs:
+        os.remove(obj)
+    os.rmdir(obj_dir)
     return out
 
 
@@ -87,14 +121,14 @@ def build_backend(force=False):
     inc = []
     for d in ext.include_paths("cuda") + [sysconfig.get_paths()["include"], INCLUDE, HERE]:
         inc += ["-isystem" if "torch" in d or "rocm" in d or "python" in d else "-I", d]
-    objs = []
+    objs, cmds = [], []
     for src in BACKEND_SRCS:
         obj = os.path.join(LIB_DIR, os.path.basename(src) + ".o")
-        cmd = ["g++", "-c", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unknown-pragmas",
-               "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
-               "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)] + inc + ["-o", obj, src]
-        subprocess.check_call(cmd)
+        cmds.append(["g++", "-c", "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unknown-pragmas",
+                     "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
+                     "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)] + inc + ["-o", obj, src])
         objs.append(obj)
+    _run_parallel(cmds)
     cmd = ["g++", "-shared", "-o", out] + objs + [
         "-L", torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-ltorch_python", "-lc10_hip", "-ltorch_hip",
         "-lamdhip64", "-L", LIB_DIR, "-lmi355ccl", "-lrt", "-lpthread",

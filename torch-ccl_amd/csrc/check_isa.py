@@ -44,9 +44,19 @@ _SCRATCH = re.compile(r"^scratch_")
 
 
 def device_asm(out_path):
-    flags = [f for f in _build.HIP_FLAGS if f not in ("-shared", "-fPIC")] + ["-I", HERE]
-    cmd = [_build.HIPCC] + flags + ["--cuda-device-only", "-S", "-o", out_path, _build.KERNEL_SRC]
-    subprocess.check_call(cmd, stderr=subprocess.DEVNULL)
+    """Device assembly of every translation unit of the kernel library, concatenated into out_path."""
+    flags = [f for f in _build.HIP_FLAGS if f != "-fPIC"] + ["-I", HERE]
+    parts, cmds = [], []
+    for src, extra, tag in _build.kernel_units():
+        part = "%s.%s.s" % (out_path, tag)
+        parts.append(part)
+        cmds.append([_build.HIPCC] + flags + list(extra) + ["--cuda-device-only", "-S", "-o", part, src])
+    _build._run_parallel(cmds)
+    with open(out_path, "w") as out:
+        for part in parts:
+            with open(part) as f:
+                out.write(f.read())
+            os.remove(part)
 
 
 def scan(asm_path):

@@ -51,7 +51,7 @@
 #include "kernels_common.hpp"
 #include "kernels_copy.hpp"
 #include "kernels_moe.hpp"
-#include "kernels_reduce.hpp"
+#include "reduce_launch.hpp"
 
 namespace {
 
@@ -155,84 +155,18 @@ size_t dtype_size(int dt) {
   }
 }
 
-enum Shape { kShapeSmall, kShapeStream, kShapePersistent };
-
-// Geometry of a launch.
-struct Geometry {
-  Shape shape;
-  unsigned grid_x;
-  int block;
-  unsigned lds;   // dynamic LDS reservation (occupancy cap), bytes
-  bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
-  bool stream_out;  // write the output with streaming (write-through) stores
-};
-
-template <int DT, int OP, int NT, bool OWN, typename ARGS>
-hipError_t launch_vec_args(const ARGS& a, const Geometry& g, int njobs, hipStream_t s) {
-  const dim3 grid(g.grid_x, njobs, 1);
-  if (g.shape == kShapePersistent)
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent, OWN, ARGS>), grid,
-                       dim3(kBlockPersistent), 0, s, a);
-  else
-    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kWave, OWN, ARGS>), grid, dim3(kWave), g.lds, s, a);
-  return hipGetLastError();
-}
-
-// One job over at most kLeanRanks shared pointers travels in the 104-byte argument block.
-template <int DT, int OP, int NT, bool OWN>
-hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
-  if constexpr (!OWN) {
-    if (njobs == 1 && a.n <= kLeanRanks) {
-      LeanReduceArgs lean;
-      for (int k = 0; k < kLeanRanks; ++k) lean.ptr[k] = k < a.n ? a.ptr[k] : nullptr;
-      lean.job[0] = a.job[0];
-      lean.n = a.n;
-      lean.flags = a.flags;
-      return launch_vec_args<DT, OP, NT, false, LeanReduceArgs>(lean, g, 1, s);
-    }
-  }
-  return launch_vec_args<DT, OP, NT, OWN, ReduceArgs>(a, g, njobs, s);
-}
-
-template <int DT, int OP>
-hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
-  if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
-  if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {  // the ops of gradient reductions
-    switch (a.n) {
-      case 2: return launch_vec<DT, OP, 2, false>(a, g, njobs, s);
-      case 4: return launch_vec<DT, OP, 4, false>(a, g, njobs, s);
-      case 8: return launch_vec<DT, OP, 8, false>(a, g, njobs, s);
-      default: break;
-    }
-  }
-  return launch_vec<DT, OP, 0, false>(a, g, njobs, s);
-}
-
-template <int DT>
-hipError_t launch_dtype(const ReduceArgs& a, int op, const Geometry& g, int njobs, hipStream_t s) {
-  switch (op) {
-    case MCCL_SUM: return launch_op<DT, MCCL_SUM>(a, g, njobs, s);
-    case MCCL_PROD: return launch_op<DT, MCCL_PROD>(a, g, njobs, s);
-    case MCCL_MIN: return launch_op<DT, MCCL_MIN>(a, g, njobs, s);
-    case MCCL_MAX: return launch_op<DT, MCCL_MAX>(a, g, njobs, s);
-    case MCCL_AVG:
-      if constexpr (Elem<DT>::kIsFloat) return launch_op<DT, MCCL_AVG>(a, g, njobs, s);
-      else return hipErrorInvalidValue;
-    default: return hipErrorInvalidValue;
-  }
-}
-
 hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g, int njobs, hipStream_t s) {
+  const int own = g.own_ptrs ? 1 : 0;
   switch (dtype) {
-    case MCCL_U8: return launch_dtype<MCCL_U8>(a, op, g, njobs, s);
-    case MCCL_I8: return launch_dtype<MCCL_I8>(a, op, g, njobs, s);
-    case MCCL_I16: return launch_dtype<MCCL_I16>(a, op, g, njobs, s);
-    case MCCL_I32: return launch_dtype<MCCL_I32>(a, op, g, njobs, s);
-    case MCCL_I64: return launch_dtype<MCCL_I64>(a, op, g, njobs, s);
-    case MCCL_F16: return launch_dtype<MCCL_F16>(a, op, g, njobs, s);
-    case MCCL_F32: return launch_dtype<MCCL_F32>(a, op, g, njobs, s);
-    case MCCL_F64: return launch_dtype<MCCL_F64>(a, op, g, njobs, s);
-    case MCCL_BF16: return launch_dtype<MCCL_BF16>(a, op, g, njobs, s);
+    case MCCL_U8: return mccl_launch_reduce_dt0(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_I8: return mccl_launch_reduce_dt1(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_I16: return mccl_launch_reduce_dt2(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_I32: return mccl_launch_reduce_dt3(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_I64: return mccl_launch_reduce_dt4(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_F16: return mccl_launch_reduce_dt5(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_F32: return mccl_launch_reduce_dt6(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_F64: return mccl_launch_reduce_dt7(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
+    case MCCL_BF16: return mccl_launch_reduce_dt8(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
     default: return hipErrorInvalidValue;
   }
 }

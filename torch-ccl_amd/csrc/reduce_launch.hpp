@@ -1,0 +1,95 @@
+// Launch dispatch of the reduction kernels: shape x argument block x rank-count specialisation x
+// op for one element type.  Each element type is compiled as a translation unit of its own
+// (mccl_reduce_dtype.hip, built once per type), which is what keeps the build parallel.
+#pragma once
+
+#include "kernels_reduce.hpp"
+
+namespace {
+
+enum Shape { kShapeSmall, kShapeStream, kShapePersistent };
+
+// Geometry of a launch.
+struct Geometry {
+  Shape shape;
+  unsigned grid_x;
+  int block;
+  unsigned lds;   // dynamic LDS reservation (occupancy cap), bytes
+  bool own_ptrs;  // jobs carry their own pointer sets (coalesced reductions)
+  bool stream_out;  // write the output with streaming (write-through) stores
+};
+
+template <int DT, int OP, int NT, bool OWN, typename ARGS>
+hipError_t launch_vec_args(const ARGS& a, const Geometry& g, int njobs, hipStream_t s) {
+  const dim3 grid(g.grid_x, njobs, 1);
+  if (g.shape == kShapePersistent)
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, kUnrollPersistent, kBlockPersistent, OWN, ARGS>), grid,
+                       dim3(kBlockPersistent), 0, s, a);
+  else
+    hipLaunchKernelGGL((reduce_vec_kernel<DT, OP, NT, 1, kWave, OWN, ARGS>), grid, dim3(kWave), g.lds, s, a);
+  return hipGetLastError();
+}
+
+// One job over at most kLeanRanks shared pointers travels in the 104-byte argument block.
+template <int DT, int OP, int NT, bool OWN>
+hipError_t launch_vec(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+  if constexpr (!OWN) {
+    if (njobs == 1 && a.n <= kLeanRanks) {
+      LeanReduceArgs lean;
+      for (int k = 0; k < kLeanRanks; ++k) lean.ptr[k] = k < a.n ? a.ptr[k] : nullptr;
+      lean.job[0] = a.job[0];
+      lean.n = a.n;
+      lean.flags = a.flags;
+      return launch_vec_args<DT, OP, NT, false, LeanReduceArgs>(lean, g, 1, s);
+    }
+  }
+  return launch_vec_args<DT, OP, NT, OWN, ReduceArgs>(a, g, njobs, s);
+}
+
+template <int DT, int OP>
+hipError_t launch_op(const ReduceArgs& a, const Geometry& g, int njobs, hipStream_t s) {
+  if (g.own_ptrs) return launch_vec<DT, OP, 0, true>(a, g, njobs, s);
+  if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) {  // the ops of gradient reductions
+    switch (a.n) {
+      case 2: return launch_vec<DT, OP, 2, false>(a, g, njobs, s);
+      case 4: return launch_vec<DT, OP, 4, false>(a, g, njobs, s);
+      case 8: return launch_vec<DT, OP, 8, false>(a, g, njobs, s);
+      default: break;
+    }
+  }
+  return launch_vec<DT, OP, 0, false>(a, g, njobs, s);
+}
+
+template <int DT>
+hipError_t launch_dtype(const ReduceArgs& a, int op, const Geometry& g, int njobs, hipStream_t s) {
+  switch (op) {
+    case MCCL_SUM: return launch_op<DT, MCCL_SUM>(a, g, njobs, s);
+    case MCCL_PROD: return launch_op<DT, MCCL_PROD>(a, g, njobs, s);
+    case MCCL_MIN: return launch_op<DT, MCCL_MIN>(a, g, njobs, s);
+    case MCCL_MAX: return launch_op<DT, MCCL_MAX>(a, g, njobs, s);
+    case MCCL_AVG:
+      if constexpr (Elem<DT>::kIsFloat) return launch_op<DT, MCCL_AVG>(a, g, njobs, s);
+      else return hipErrorInvalidValue;
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+// Entry points of the per-type translation units.  Plain types only: the argument block and the
+// geometry live in unnamed namespaces and are therefore distinct types in every translation unit
+// (with one layout).  `reduce_args` points at a ReduceArgs.
+#define MCCL_REDUCE_ENTRY_ARGS                                                                 \
+  const void *reduce_args, int op, int shape, unsigned grid_x, unsigned lds, int own_ptrs, int njobs, \
+      hipStream_t stream
+extern "C" {
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt0(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt1(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt2(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt3(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt4(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt5(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt6(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt7(MCCL_REDUCE_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt8(MCCL_REDUCE_ENTRY_ARGS);
+}
