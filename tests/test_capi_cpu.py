@@ -70,6 +70,42 @@ def test_argument_errors_need_no_device(mccl):
     assert L.mccl_copy_segments(None, 3, None) == -1
 
 
+def test_overlapping_buffers_are_rejected_before_any_launch(mccl):
+    """In place means: the output is exactly the range the reduction reads from one rank.  Any other
+    overlap between an output and something the same launch reads or writes is refused."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    base, nbytes = 0x10000000, 4096 * 4
+    ins = capi.ptr_table([base, base + 0x100000])
+    out = ctypes.c_void_p
+    # partial overlap with input 1
+    assert L.mccl_reduce_n(ins, 2, out(base + 0x100000 + 64), 4096, capi.F32, capi.SUM, 0, None) == -1
+    assert b"partially overlaps input 1" in L.mccl_last_error()
+    assert L.mccl_reduce_n(ins, 2, out(base - nbytes + 4), 4096, capi.F32, capi.SUM, 0, None) == -1
+    assert b"partially overlaps input 0" in L.mccl_last_error()
+    # reduce_scatter: shard 0's output inside the range shard 1 reads from rank 0
+    outs = capi.ptr_table([base + 0x200000, base + 1024 * 4 + 16])
+    assert L.mccl_reduce_scatter_n(ins, 2, outs, 1024, 0, 2, capi.F32, capi.SUM, None) == -1
+    assert b"overlaps input 0 of reduction 1" in L.mccl_last_error()
+    # two outputs of one coalesced launch overlapping each other
+    tab = capi.ptr_table([base, base + 0x100000, base + 0x200000, base + 0x300000])
+    outs = capi.ptr_table([base + 0x400000, base + 0x400000 + 512])
+    counts = (ctypes.c_size_t * 2)(1024, 1024)
+    assert L.mccl_reduce_multi(tab, 2, outs, counts, 2, capi.F32, capi.SUM, None) == -1
+    assert b"outputs" in L.mccl_last_error() and b"overlap" in L.mccl_last_error()
+
+
+def test_pack_and_unpack_reject_a_null_flat_buffer(mccl):
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    tab = capi.ptr_table([0x1000, 0x2000])
+    sizes = (ctypes.c_size_t * 2)(16, 16)
+    assert L.mccl_pack(tab, sizes, 2, None, None) == -1
+    assert L.mccl_unpack(None, tab, sizes, 2, None) == -1
+    zero = (ctypes.c_size_t * 2)(0, 0)
+    assert L.mccl_pack(tab, zero, 2, None, None) == 0
+
+
 def test_tensor_front_end_rejects_cpu_tensors(mccl):
     import torch
     with pytest.raises(RuntimeError, match="must be on the GPU"):

@@ -28,8 +28,9 @@
 //                  the live window smears) but a few percent ahead while the whole working
 //                  set fits the 256 MB Infinity Cache, which is where AUTO uses it;
 //   * misaligned heads/tails are peeled element-wise inside the same launch up to the first
-//     16-byte boundary of the output; inputs that are not congruent with the output mod 16
-//     are read with unaligned vector loads (the hardware splits them).
+//     128-byte boundary of the output (whole cache lines per tile); inputs that are not
+//     congruent with the output mod 16 are read with unaligned vector loads (the hardware
+//     splits them).
 //
 // What each kernel replaces in the reference (intel/torch-ccl):
 //   reduce_vec_kernel : the N-peer sum of src/gpu/allreduce_small.h:289-361,
@@ -275,7 +276,7 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
     size_t head = ((128u - (unsigned)(o & 127u)) & 127u) / es;  // the body starts on a cache line of out
     if (head > sp.count) head = sp.count;
     const size_t nvec = (sp.count - head) / ve;
-    if (nvec / kWave > 0xf0000000ull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+    if (nvec / kWave > kMaxChunks) return fail(MCCL_ERR_INVALID_ARG, "message too large");
     ReduceJob& jb = a.job[nv];
     jb.out = sp.out;
     jb.in_off = sp.in_off;
@@ -285,6 +286,24 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
     a.job_ptr0[nv] = sp.ptr0;
     ++nv;
     if (sp.count > vmax) vmax = sp.count;
+  }
+  // An output may be exactly the input range its own job reads from one rank (in place); any
+  // other overlap with something this launch reads or writes would race between wavefronts.
+  for (int j = 0; j < nv; ++j) {
+    const uintptr_t o0 = (uintptr_t)a.job[j].out;
+    const uintptr_t o1 = o0 + (a.job[j].head + a.job[j].nvec * ve + a.job[j].tail) * es;
+    for (int i = 0; i < nv; ++i) {
+      const size_t ibytes = (a.job[i].head + a.job[i].nvec * ve + a.job[i].tail) * es;
+      if (i != j) {
+        const uintptr_t q0 = (uintptr_t)a.job[i].out;
+        if (o0 < q0 + ibytes && q0 < o1) return fail(MCCL_ERR_INVALID_ARG, "outputs %d and %d overlap", j, i);
+      }
+      for (int k = 0; k < a.n; ++k) {
+        const uintptr_t p0 = (uintptr_t)(a.ptr[a.job_ptr0[i] + k] + a.job[i].in_off);
+        if (o0 < p0 + ibytes && p0 < o1 && !(i == j && p0 == o0))
+          return fail(MCCL_ERR_INVALID_ARG, "output %d partially overlaps input %d of reduction %d", j, k, i);
+      }
+    }
   }
   if (nv) {
     Geometry g;
@@ -604,6 +623,10 @@ int mccl_pack(const void* const* src, const size_t* bytes, int n, void* dst, voi
   if (n < 0) return fail(MCCL_ERR_INVALID_ARG, "negative count");
   if (n == 0) return MCCL_OK;
   if (!src || !bytes) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  size_t total = 0;
+  for (int i = 0; i < n; ++i) total += bytes[i];
+  if (!total) return MCCL_OK;
+  if (!dst) return fail(MCCL_ERR_INVALID_ARG, "destination pointer is null");
   size_t off = 0;
   for (int i0 = 0; i0 < n; i0 += kMaxSegs) {
     mccl_segment_t segs[kMaxSegs];
@@ -624,6 +647,10 @@ int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, v
   if (n < 0) return fail(MCCL_ERR_INVALID_ARG, "negative count");
   if (n == 0) return MCCL_OK;
   if (!dst || !bytes) return fail(MCCL_ERR_INVALID_ARG, "null table");
+  size_t total = 0;
+  for (int i = 0; i < n; ++i) total += bytes[i];
+  if (!total) return MCCL_OK;
+  if (!src) return fail(MCCL_ERR_INVALID_ARG, "source pointer is null");
   size_t off = 0;
   for (int i0 = 0; i0 < n; i0 += kMaxSegs) {
     mccl_segment_t segs[kMaxSegs];
