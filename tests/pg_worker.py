@@ -91,6 +91,49 @@ def reference_cases(pg, rank, world):
     outs = [torch.ones(rank + 1, world, device=DEV) for _ in range(world)]
     pg.alltoall(outs, [_dev(v, torch.float32) for v in L["inputs"][rank]]).wait()
     assert [t.cpu().tolist() for t in outs] == L["expected"][rank]
+    # reduce to each root in turn (:221-237): the allreduce closed forms, on the root only
+    for name, want in K["allreduce"]["expected"].items():
+        for root in range(world):
+            opts = c10d.ReduceOptions()
+            opts.reduceOp = ops[name]
+            opts.rootRank = root
+            t = _dev(K["allreduce"]["inputs"][rank])
+            pg.reduce([t], opts).wait()
+            if rank == root:
+                assert t.cpu().tolist() == want, (name, root, t.cpu().tolist(), want)
+            else:
+                assert t.cpu().tolist() == K["allreduce"]["inputs"][rank]  # untouched off the root
+    # gather, every rank root in turn, work items collected first (:254-277)
+    outputs = [_dev([-1]) for _ in range(world)]
+    work = []
+    for root in range(world):
+        opts = c10d.GatherOptions()
+        opts.rootRank = root
+        work.append(pg.gather([outputs] if root == rank else [], [_dev([rank])], opts))
+    for w in work:
+        w.wait()
+    assert [t.cpu().tolist() for t in outputs] == [[r] for r in range(world)]
+    try:
+        opts = c10d.GatherOptions()
+        opts.rootRank = (rank + 1) % world
+        pg.gather([outputs], [_dev([rank])], opts)
+        raise AssertionError("non-root output check did not fire")
+    except RuntimeError as e:
+        assert "gather: number of output tensors should be 0 for non-root" in str(e)
+    # scatter from each root in turn (:290-308)
+    for root in range(world):
+        opts = c10d.ScatterOptions()
+        opts.rootRank = root
+        output = [_dev([-1])]
+        pg.scatter(output, [[_dev([r]) for r in range(world)]] if root == rank else [], opts).wait()
+        assert output[0].cpu().tolist() == [rank]
+    try:
+        opts = c10d.ScatterOptions()
+        opts.rootRank = rank
+        pg.scatter([_dev([-1])], [[_dev([0])] * (world + 1)], opts)
+        raise AssertionError("input list check did not fire")
+    except ValueError as e:
+        assert "Incorrect input list size" in str(e)
     # broadcast root check (:109-113)
     try:
         opts = c10d.BroadcastOptions()
@@ -158,6 +201,34 @@ def oracle_cases(pg, rank, world):
         opts.reduceOp = op
         pg.allreduce([t], opts).wait()
         assert np.array_equal(bits(t), bits_np(O.reduce([to_carrier(h) for h in host], O.F32, ocode))), opname
+    # rooted reduce: only the root's tensor changes, to the oracle's bits
+    for dtype, count, op, ocode in ((torch.bfloat16, 300001, c10d.ReduceOp.SUM, O.SUM), (torch.float32, 77, c10d.ReduceOp.MAX, O.MAX),
+                                    (torch.int64, 4097, c10d.ReduceOp.PRODUCT, O.PROD)):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(count, dtype, r, seed=31) for r in range(world)]
+        root = count % world
+        t = host[rank].to(DEV)
+        opts = c10d.ReduceOptions()
+        opts.reduceOp = op
+        opts.rootRank = root
+        pg.reduce([t], opts).wait()
+        want = bits_np(O.reduce([to_carrier(h) for h in host], code, ocode)) if rank == root else bits(host[rank])
+        assert np.array_equal(bits(t), want), ("reduce", dtype, count)
+    # gather and scatter of odd-sized byte tensors, byte for byte
+    root = world - 1
+    host = [rank_buffer(10007, torch.int8, r, seed=41) for r in range(world)]
+    outs = [torch.zeros(10007, dtype=torch.int8, device=DEV) for _ in range(world)]
+    opts = c10d.GatherOptions()
+    opts.rootRank = root
+    pg.gather([outs] if rank == root else [], [host[rank].to(DEV)], opts).wait()
+    if rank == root:
+        for r in range(world):
+            assert np.array_equal(bits(outs[r]), bits(host[r])), ("gather", r)
+    out = torch.zeros(10007, dtype=torch.int8, device=DEV)
+    opts = c10d.ScatterOptions()
+    opts.rootRank = root
+    pg.scatter([out], [[h.to(DEV) for h in host]] if rank == root else [], opts).wait()
+    assert np.array_equal(bits(out), bits(host[rank])), "scatter"
     # uneven all_to_all_single: a seeded split matrix every rank agrees on
     rng = np.random.default_rng(1234)
     S = rng.integers(0, 300, size=(world, world))
@@ -212,6 +283,18 @@ def dist_api_cases(rank, world):
     o = torch.zeros(2, 2, device=DEV)
     dist.reduce_scatter_tensor(o, torch.ones(world * 2, 2, device=DEV))
     assert torch.equal(o.cpu(), torch.full((2, 2), float(world)))
+    # rooted collectives through the public API
+    t = torch.full((10,), float(rank + 1), device=DEV)
+    dist.reduce(t, dst=world - 1)
+    if rank == world - 1:
+        assert t.cpu().tolist() == [world * (world + 1) / 2.0] * 10
+    got = [torch.zeros(3, device=DEV) for _ in range(world)] if rank == 0 else None
+    dist.gather(torch.full((3,), float(rank), device=DEV), got, dst=0)
+    if rank == 0:
+        assert [g.cpu().tolist() for g in got] == [[float(r)] * 3 for r in range(world)]
+    piece = torch.zeros(2, device=DEV)
+    dist.scatter(piece, [torch.full((2,), float(10 + r), device=DEV) for r in range(world)] if rank == 1 else None, src=1)
+    assert piece.cpu().tolist() == [float(10 + rank)] * 2
     # unsupported reduce op and collectives outside the path
     try:
         dist.all_reduce(torch.ones(4, dtype=torch.int32, device=DEV), op=dist.ReduceOp.BAND)

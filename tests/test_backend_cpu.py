@@ -57,6 +57,6 @@ def test_cpu_tensors_are_rejected(pkg):
 def test_collectives_outside_the_path_fail_like_the_reference(pkg):
     pg = _pg()
     with pytest.raises(RuntimeError, match="isn't implementd on backend"):
-        pg.reduce([torch.zeros(1)])
+        pg.send([torch.zeros(1)], 0, 0)
     with pytest.raises(RuntimeError, match="does not support allgather_coalesced"):
         pg.allgather_coalesced([[torch.zeros(1)]], [torch.zeros(1)])

@@ -275,6 +275,7 @@ ProcessGroupCCL::~ProcessGroupCCL() {
     if (stage_[s].base) (void)hipFree(stage_[s].base);
   for (void* p : retired_) (void)hipFree(p);
   if (fork_event_) (void)hipEventDestroy(fork_event_);
+  if (tail_event_) (void)hipEventDestroy(tail_event_);
   if (ctl_) munmap(ctl_, ctl_bytes_);
 }
 
@@ -288,6 +289,7 @@ void ProcessGroupCCL::ensureInit(int device) {
   HIP_CHECK(hipSetDevice(device_));
   comm_stream_ = c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, (c10::DeviceIndex)device_).stream();
   HIP_CHECK(hipEventCreateWithFlags(&fork_event_, hipEventDisableTiming));
+  HIP_CHECK(hipEventCreateWithFlags(&tail_event_, hipEventDisableTiming));
 
   // Groups are created in the same order on every rank, so a per-rank counter in the store
   // yields the same id everywhere.
@@ -448,7 +450,10 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     if (timed) { phase_us_[0].push_back((float)us_since(t0)); t0 = clk::now(); }
     // This rank's staging buffer must be complete before any peer reads it, and (two
     // collectives later) every peer must be done reading before it is overwritten: one host
-    // barrier per collective plus the two alternating buffers give both.
+    // barrier per collective plus the two alternating buffers give both, provided the
+    // synchronisation below covers this rank's earlier kernels.  On one stream it does; a
+    // previous collective that ran on another stream is waited for through its tail event.
+    if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipEventSynchronize(tail_event_));
     HIP_CHECK(hipStreamSynchronize(s));
   } catch (...) {
     // this rank will not arrive: tell the peers now instead of letting them run into the timeout
@@ -479,6 +484,11 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     }
   }
   if (timed) phase_us_[3].push_back((float)us_since(t0));
+  if (plan.exec) {
+    HIP_CHECK(hipEventRecord(tail_event_, s));
+    tail_stream_ = s;
+    tail_pending_ = true;
+  }
 
   auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
   work->device_ = device_;
@@ -1076,16 +1086,162 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::barrier(const c10d::BarrierOptio
   return work;
 }
 
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce(std::vector<at::Tensor>&, const c10d::ReduceOptions&) {
-  notImplemented("reduce");
+// Rooted reduction (XPUCCLStubs::reduce_, src/gpu/dpcpp_ccl.cpp:820-857): every rank stages its
+// tensor, the root runs the N-buffer reduction into its own; the other ranks' tensors keep their
+// values.
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce(std::vector<at::Tensor>& tensors,
+                                                       const c10d::ReduceOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::reduce", std::vector<c10::IValue>({tensors}));
+  checkRank((int)opts.rootRank, size_);
+  TORCH_CHECK(tensors.size() == 1, "CCL process group does not support tensors count ", tensors.size());
+  checkDeviceTensors(tensors);
+  at::Tensor t = tensors[0];
+  const int dtype = dtypeCode(t.scalar_type());
+  const int op = opCode(opts.reduceOp, t.scalar_type());
+  const int root = (int)opts.rootRank;
+  const size_t es = t.element_size();
+  const size_t total = (size_t)t.numel();
+  const size_t chunk = kStageMax / es;
+  c10::intrusive_ptr<c10d::Work> work;
+  size_t off = 0;
+  do {
+    const size_t len = std::min(total - off, chunk);
+    char* base = total ? (char*)t.data_ptr() + off * es : nullptr;
+    Plan p;
+    p.op = c10d::OpType::REDUCE;
+    p.title = "reduce";
+    p.inputs = {t};
+    p.outputs = {t};
+    if (size_ > 1 && len) {
+      const int W = size_;
+      p.stage_bytes = len * es;
+      p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, base, len * es, s); };
+      if (rank_ == root)
+        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+          MCCL_CHECK(mccl_reduce_n(peer.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
+        };
+    }
+    work = run(p);
+    off += len;
+  } while (off < total);
+  return work;
 }
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<at::Tensor>>&, std::vector<at::Tensor>&,
-                                                       const c10d::GatherOptions&) {
-  notImplemented("gather");
+
+// gather (XPUCCLStubs::gather_, src/gpu/dpcpp_ccl.cpp:1237-1299): every rank stages its tensor and
+// announces its size; the root copies all of them into its output list in one launch.
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<at::Tensor>>& outputs,
+                                                       std::vector<at::Tensor>& inputs,
+                                                       const c10d::GatherOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::gather", std::vector<c10::IValue>({inputs}));
+  checkRank((int)opts.rootRank, size_);
+  TORCH_CHECK(inputs.size() == 1, "CCL process group does not support tensors count ", inputs.size());
+  const int root = (int)opts.rootRank;
+  std::vector<at::Tensor> outs;
+  if (rank_ != root) {
+    TORCH_CHECK(outputs.size() == 0, "gather: number of output tensors should be 0 for non-root");
+    checkDeviceTensors(inputs);
+  } else {
+    TORCH_CHECK(outputs.size() == 1, "gather: multi-GPU collective is not supported");
+    TORCH_CHECK((int)outputs[0].size() == size_, "gather: number of output tensors should equal to the world size");
+    outs = outputs[0];
+    std::vector<at::Tensor> all = outs;
+    all.push_back(inputs[0]);
+    checkDeviceTensors(all);
+  }
+  at::Tensor input = inputs[0];
+  const size_t mine = nbytes(input);
+  TORCH_CHECK(mine <= kStageMax, "ccl backend: gather message larger than the staging window");
+  Plan p;
+  p.op = c10d::OpType::GATHER;
+  p.title = "gather";
+  p.inputs = {input};
+  p.outputs = outs;
+  p.stage_bytes = mine;
+  p.table = {(int64_t)mine};
+  const int W = size_;
+  if (mine) p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, input.data_ptr(), mine, s); };
+  if (rank_ == root)
+    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+      std::vector<mccl_segment_t> segs;
+      for (int r = 0; r < W; ++r) {
+        const size_t b = (size_t)tables[(size_t)r][0];
+        TORCH_CHECK(b == nbytes(outs[(size_t)r]), "gather: output tensor ", r, " does not match the size rank ", r, " sends");
+        if (b) segs.push_back({peer[(size_t)r], outs[(size_t)r].data_ptr(), b});
+      }
+      MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+  return run(p);
 }
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&, std::vector<std::vector<at::Tensor>>&,
-                                                        const c10d::ScatterOptions&) {
-  notImplemented("scatter");
+
+// scatter (XPUCCLStubs::scatter_, src/gpu/dpcpp_ccl.cpp:1301-1369): the root stages its input list
+// back to back and announces where each piece lies; every rank pulls its own piece.
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>& outputs,
+                                                        std::vector<std::vector<at::Tensor>>& inputs,
+                                                        const c10d::ScatterOptions& opts) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::scatter", std::vector<c10::IValue>({outputs}));
+  checkRank((int)opts.rootRank, size_);
+  const int root = (int)opts.rootRank;
+  const int W = size_;
+  std::vector<at::Tensor> ins;
+  if (rank_ == root) {
+    if (inputs.size() != 1) {
+      std::ostringstream ss;
+      ss << "ProcessGroupCCL::scatter: requires a single-element input list containing a list with " << W << " tensors.";
+      C10_THROW_ERROR(ValueError, ss.str());
+    }
+    if ((int)inputs[0].size() != W) {
+      std::ostringstream ss;
+      ss << "ProcessGroupCCL::scatter: Incorrect input list size " << inputs[0].size()
+         << ". Input list size should be " << W << ", same as size of the process group.";
+      C10_THROW_ERROR(ValueError, ss.str());
+    }
+    ins = inputs[0];
+  } else {
+    TORCH_CHECK(inputs.size() == 0, "scatter: number of input tensors should be 0 for non-root");
+  }
+  TORCH_CHECK(outputs.size() == 1, "CCL process group does not support tensors count ", outputs.size());
+  std::vector<at::Tensor> all = ins;
+  all.push_back(outputs[0]);
+  checkDeviceTensors(all);
+  at::Tensor out = outputs[0];
+  Plan p;
+  p.op = c10d::OpType::SCATTER;
+  p.title = "scatter";
+  p.inputs = ins;
+  p.outputs = {out};
+  const int me = rank_;
+  if (rank_ == root) {
+    // staging image: the W pieces back to back, each on a 16-byte boundary; table = W offsets, W sizes
+    std::vector<size_t> offs((size_t)W);
+    size_t total = 0;
+    p.table.assign((size_t)(2 * W), 0);
+    for (int r = 0; r < W; ++r) {
+      offs[(size_t)r] = total;
+      p.table[(size_t)r] = (int64_t)total;
+      p.table[(size_t)(W + r)] = (int64_t)nbytes(ins[(size_t)r]);
+      if (r != root) total += roundUp(nbytes(ins[(size_t)r]), 16);  // the root's own piece is not staged
+    }
+    TORCH_CHECK(total <= kStageMax, "ccl backend: scatter larger than the staging window");
+    TORCH_CHECK(nbytes(ins[(size_t)root]) == nbytes(out), "scatter: output tensor does not match the size the root sends");
+    p.stage_bytes = total;
+    p.copy_in = [=](void* stage, hipStream_t s) {
+      std::vector<mccl_segment_t> segs;
+      for (int r = 0; r < W; ++r)
+        if (r != root && ins[(size_t)r].numel())
+          segs.push_back({ins[(size_t)r].data_ptr(), (char*)stage + offs[(size_t)r], nbytes(ins[(size_t)r])});
+      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    p.exec = [=](const std::vector<const void*>&, const std::vector<const int64_t*>&, hipStream_t s) {
+      copyAsync(out.data_ptr(), ins[(size_t)root].data_ptr(), nbytes(out), s);
+    };
+  } else {
+    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+      const size_t b = (size_t)tables[(size_t)root][W + me];
+      TORCH_CHECK(b == nbytes(out), "scatter: output tensor does not match the size the root sends");
+      copyAsync(out.data_ptr(), (const char*)peer[(size_t)root] + tables[(size_t)root][me], b, s);
+    };
+  }
+  return run(p);
 }
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::send(std::vector<at::Tensor>&, int, int) { notImplemented("send"); }
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>&, int, int) { notImplemented("recv"); }

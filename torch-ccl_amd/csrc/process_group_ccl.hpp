@@ -112,13 +112,14 @@ class ProcessGroupCCL : public c10d::Backend {
                                           const c10d::AllToAllOptions& opts) override;
   c10::intrusive_ptr<c10d::Work> barrier(const c10d::BarrierOptions& opts) override;
 
+  // Rooted forms over the same kernels: the root reduces / pulls, the others only stage.
+  c10::intrusive_ptr<c10d::Work> reduce(std::vector<at::Tensor>& tensors, const c10d::ReduceOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> gather(std::vector<std::vector<at::Tensor>>& outputs, std::vector<at::Tensor>& inputs,
+                                        const c10d::GatherOptions& opts) override;
+  c10::intrusive_ptr<c10d::Work> scatter(std::vector<at::Tensor>& outputs, std::vector<std::vector<at::Tensor>>& inputs,
+                                         const c10d::ScatterOptions& opts) override;
   // Not on the path this backend covers; they fail like DispatchStub::fail does
   // (src/dispatch_stub.h:288-290).
-  c10::intrusive_ptr<c10d::Work> reduce(std::vector<at::Tensor>&, const c10d::ReduceOptions&) override;
-  c10::intrusive_ptr<c10d::Work> gather(std::vector<std::vector<at::Tensor>>&, std::vector<at::Tensor>&,
-                                        const c10d::GatherOptions&) override;
-  c10::intrusive_ptr<c10d::Work> scatter(std::vector<at::Tensor>&, std::vector<std::vector<at::Tensor>>&,
-                                         const c10d::ScatterOptions&) override;
   c10::intrusive_ptr<c10d::Work> send(std::vector<at::Tensor>&, int, int) override;
   c10::intrusive_ptr<c10d::Work> recv(std::vector<at::Tensor>&, int, int) override;
   c10::intrusive_ptr<c10d::Work> recvAnysource(std::vector<at::Tensor>&, int) override;
@@ -168,6 +169,12 @@ class ProcessGroupCCL : public c10d::Backend {
   int device_ = 0;
   hipStream_t comm_stream_ = nullptr;
   hipEvent_t fork_event_ = nullptr;
+  // End of the previous collective's device work and the stream it ran on.  A collective that runs
+  // on another stream waits for it on the host before its barrier, so that "every earlier kernel of
+  // this rank has finished reading the peers' staging buffers" holds whichever streams were used.
+  hipEvent_t tail_event_ = nullptr;
+  hipStream_t tail_stream_ = nullptr;
+  bool tail_pending_ = false;
   uint64_t seq_ = 0;
   uint64_t barrier_epoch_ = 0;
 
