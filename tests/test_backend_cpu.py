@@ -60,3 +60,14 @@ def test_collectives_outside_the_path_fail_like_the_reference(pkg):
         pg.send([torch.zeros(1)], 0, 0)
     with pytest.raises(RuntimeError, match="does not support allgather_coalesced"):
         pg.allgather_coalesced([[torch.zeros(1)]], [torch.zeros(1)])
+
+
+def test_reference_import_name_registers_the_backend(pkg):
+    """`import oneccl_bindings_for_pytorch` is what users of the reference write (README.md:176-190)."""
+    import oneccl_bindings_for_pytorch as torch_ccl
+    import torch.distributed as dist
+    assert torch_ccl.ProcessGroupCCL is dist.ProcessGroupCCL
+    assert "ccl" in dist.Backend.backend_list
+    assert os.path.isdir(torch_ccl.cwd)
+    a, b = torch.zeros(4), torch.zeros(4, 4).t()
+    assert torch_ccl.is_available([a]) and not torch_ccl.is_available([b]) and not torch_ccl.is_available([a, a])
