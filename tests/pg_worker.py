@@ -295,6 +295,18 @@ def dist_api_cases(rank, world):
     piece = torch.zeros(2, device=DEV)
     dist.scatter(piece, [torch.full((2,), float(10 + r), device=DEV) for r in range(world)] if rank == 1 else None, src=1)
     assert piece.cpu().tolist() == [float(10 + rank)] * 2
+    # point to point through the public API: blocking pair, then isend / irecv round the ring
+    if rank == 0:
+        dist.send(torch.arange(6, dtype=torch.float32, device=DEV), dst=1)
+    elif rank == 1:
+        r = torch.zeros(6, device=DEV)
+        dist.recv(r, src=0)
+        assert r.cpu().tolist() == [0.0, 1.0, 2.0, 3.0, 4.0, 5.0]
+    r = torch.zeros(4, device=DEV)
+    reqs = [dist.irecv(r, src=(rank - 1) % world), dist.isend(torch.full((4,), float(rank), device=DEV), dst=(rank + 1) % world)]
+    for q in reqs:
+        q.wait()
+    assert r.cpu().tolist() == [float((rank - 1) % world)] * 4
     # unsupported reduce op and collectives outside the path
     try:
         dist.all_reduce(torch.ones(4, dtype=torch.int32, device=DEV), op=dist.ReduceOp.BAND)
@@ -302,6 +314,61 @@ def dist_api_cases(rank, world):
     except RuntimeError as e:
         assert "Cannot use ReduceOp.BAND" in str(e)
     dist.barrier()
+
+
+def p2p_cases(pg, rank, world):
+    """send / recv: ring exchange, several messages in flight each way, waits out of posting order,
+    more messages than the sender has buffers, empty and odd sizes; byte for byte."""
+    from helpers import bits, rank_buffer
+    nxt, prv = (rank + 1) % world, (rank - 1) % world
+
+    def payload(src, dst, i, count, dtype=torch.uint8):
+        return rank_buffer(count, dtype, src * 64 + dst, seed=1000 + i)
+
+    # ring: everybody sends to the next rank and receives from the previous one
+    for i, count in enumerate((1, 0, 4097, (1 << 20) + 3)):
+        got = torch.full((count,), 7, dtype=torch.uint8, device=DEV)
+        w = pg.recv([got], prv, 0)
+        pg.send([payload(rank, nxt, i, count).to(DEV)], nxt, 0).wait()
+        w.wait()
+        assert np.array_equal(bits(got), bits(payload(prv, rank, i, count))), ("ring", count)
+    # two receives and two sends posted each way, then waited receive-first (neither side may block)
+    sizes = (300001, 12)
+    gots = [torch.zeros(c, dtype=torch.bfloat16, device=DEV) for c in sizes]
+    works = [pg.recv([g], prv, 0) for g in gots]
+    works += [pg.send([payload(rank, nxt, 10 + j, c, torch.bfloat16).to(DEV)], nxt, 0) for j, c in enumerate(sizes)]
+    assert works[2].is_completed() and works[3].is_completed()  # the data has left the tensors
+    works[1].wait()  # second receive first: the first one is completed on the way
+    assert works[0].is_completed()
+    for w in works:
+        w.wait()
+    for j, c in enumerate(sizes):
+        assert np.array_equal(bits(gots[j]), bits(payload(prv, rank, 10 + j, c, torch.bfloat16))), ("batch", j)
+    # ten messages to one destination: more than the sender has buffers, so it has to wait for the receiver
+    if rank == 0:
+        for i in range(10):
+            pg.send([payload(0, 1, 20 + i, 1000 + i).to(DEV)], 1, 0).wait()
+    elif rank == 1:
+        for i in range(10):
+            got = torch.zeros(1000 + i, dtype=torch.uint8, device=DEV)
+            pg.recv([got], 0, 0).wait()
+            assert np.array_equal(bits(got), bits(payload(0, 1, 20 + i, 1000 + i))), ("burst", i)
+    # a growing message reuses and then replaces the buffers (the receiver must re-map them)
+    for i, count in enumerate((100, 70000, 100, 300000)):
+        got = torch.zeros(count, dtype=torch.uint8, device=DEV)
+        w = pg.recv([got], nxt, 0)
+        pg.send([payload(rank, prv, 40 + i, count).to(DEV)], prv, 0).wait()
+        w.wait()
+        assert np.array_equal(bits(got), bits(payload(nxt, rank, 40 + i, count))), ("grow", count)
+    # polling: is_completed turns true once the sender has published, without a wait
+    got = torch.zeros(5, dtype=torch.uint8, device=DEV)
+    w = pg.recv([got], prv, 0)
+    pg.send([payload(rank, nxt, 50, 5).to(DEV)], nxt, 0).wait()
+    for _ in range(200000):
+        if w.is_completed():
+            break
+    assert w.is_completed() and np.array_equal(bits(got), bits(payload(prv, rank, 50, 5)))
+    pg.barrier().wait()
 
 
 def large_message_case(pg, rank, world):
@@ -314,6 +381,18 @@ def large_message_case(pg, rank, world):
     s = world * (world + 1) / 2.0
     assert float(t[0]) == s and float(t[count // 2]) == s and float(t[-2]) == s and float(t[-1]) == 7.0 * s
     assert float(t.min()) == s
+    del t
+    # point to point across the 1 GiB window: two chunks travel as two messages
+    count = (1 << 30) + 5
+    if rank == 0:
+        big = torch.arange(count, dtype=torch.int64, device=DEV).to(torch.uint8)
+        pg.send([big], 1, 0).wait()
+    elif rank == 1:
+        got = torch.zeros(count, dtype=torch.uint8, device=DEV)
+        pg.recv([got], 0, 0).wait()
+        want = torch.arange(count, dtype=torch.int64, device=DEV).to(torch.uint8)
+        assert torch.equal(got, want)
+    pg.barrier().wait()
 
 
 def missing_rank_case(pg, rank, world):
@@ -328,6 +407,30 @@ def missing_rank_case(pg, rank, world):
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
                 or "rank 1 left the group" in str(e)), str(e)
+
+
+def missing_sender_case(pg, rank, world):
+    """Rank 0 posts a receive for a message rank 1 never sends: the wait must raise, not hang; a
+    mismatched size raises on the receiver as well."""
+    t = torch.ones(16, device=DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    if rank == 1:
+        pg.send([torch.ones(8, device=DEV)], 0, 0).wait()
+        return
+    got = torch.zeros(4, device=DEV)
+    try:
+        pg.recv([got], 1, 0).wait()  # 16 bytes expected, 32 sent
+        raise AssertionError("size mismatch accepted")
+    except RuntimeError as e:
+        assert "recv expects 16 bytes from rank 1 but the message holds 32" in str(e), str(e)
+    w = pg.recv([torch.zeros(4, device=DEV)], 1, 0)
+    assert not w.is_completed()
+    try:
+        w.wait()
+        raise AssertionError("receive without a sender returned")
+    except RuntimeError as e:
+        assert ("timed out waiting for a message" in str(e) or "reported a failure" in str(e)
+                or "left the group" in str(e)), str(e)
 
 
 def env_switch_case(pg, rank, world):
@@ -412,12 +515,16 @@ def run_rank(rank, world, store_path, mode):
         reference_cases(pg, rank, world)
     elif mode == "oracle":
         oracle_cases(pg, rank, world)
+    elif mode == "p2p":
+        p2p_cases(pg, rank, world)
     elif mode == "large":
         large_message_case(pg, rank, world)
     elif mode == "env":
         env_switch_case(pg, rank, world)
     elif mode == "missing":
         missing_rank_case(pg, rank, world)
+    elif mode == "missing_sender":
+        missing_sender_case(pg, rank, world)
     else:
         raise ValueError(mode)
     torch.cuda.synchronize()

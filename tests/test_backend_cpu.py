@@ -56,8 +56,12 @@ def test_cpu_tensors_are_rejected(pkg):
 
 def test_collectives_outside_the_path_fail_like_the_reference(pkg):
     pg = _pg()
-    with pytest.raises(RuntimeError, match="isn't implementd on backend"):
+    with pytest.raises(RuntimeError, match="does not support recvAnysource"):
+        pg.recv_anysource([torch.zeros(1)], 0)
+    with pytest.raises(RuntimeError, match="Tensors are not in same device type"):
         pg.send([torch.zeros(1)], 0, 0)
+    with pytest.raises(ValueError, match="unexpected rank"):
+        pg.recv([torch.zeros(1)], 5, 0)
     with pytest.raises(RuntimeError, match="does not support allgather_coalesced"):
         pg.allgather_coalesced([[torch.zeros(1)]], [torch.zeros(1)])
 

@@ -33,6 +33,11 @@ def test_torch_distributed_api(world):
     _spawn(world, "dist")
 
 
+@pytest.mark.parametrize("world", [2, 3, 8])
+def test_send_recv(world):
+    _spawn(world, "p2p")
+
+
 def test_message_larger_than_one_staging_window():
     _spawn(2, "large")
 
@@ -58,6 +63,11 @@ def test_missing_rank_raises_instead_of_hanging(monkeypatch):
     _spawn(3, "missing")
 
 
+def test_receive_without_a_sender_raises_instead_of_hanging(monkeypatch):
+    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    _spawn(2, "missing_sender")
+
+
 def test_thread_ranks_in_one_process():
     """Ranks as threads of one process (same address space: staging buffers are shared by raw
     pointer instead of an IPC handle), rendezvous through a HashStore."""
@@ -79,8 +89,13 @@ def test_thread_ranks_in_one_process():
             pg._allgather_base(out, torch.full((5,), float(rank), device="cuda:0")).wait()
             torch.cuda.synchronize()
             assert out.cpu().tolist() == [float(r) for r in range(world) for _ in range(5)]
+            got = torch.zeros(1000, device="cuda:0")
+            w = pg.recv([got], (rank - 1) % world, 0)
+            pg.send([torch.full((1000,), float(rank), device="cuda:0")], (rank + 1) % world, 0).wait()
+            w.wait()
+            assert got.cpu().tolist() == [float((rank - 1) % world)] * 1000
             pg.barrier().wait()
-            del pg
+            del w, pg
         except Exception as e:  # noqa: BLE001
             errors.append((rank, repr(e)))
 

@@ -137,6 +137,28 @@ void copyAsync(void* dst, const void* src, size_t bytes, hipStream_t s) {
 // ---------------------------------------------------------------------------------------------
 // shared-memory control block
 // ---------------------------------------------------------------------------------------------
+constexpr int kRing = 4;  // ProcessGroupCCL::kP2PRing
+constexpr size_t kP2PMinBytes = 64u << 10;
+
+// One staging buffer of the sender and the message it currently holds.
+struct P2PEntry {
+  uint64_t gen;       // bumped whenever the sender replaces the buffer
+  uint64_t ptr;       // the sender's address (threads of the same process use it directly)
+  uint64_t capacity;
+  uint64_t bytes;     // payload of the message
+  hipIpcMemHandle_t handle;
+};
+
+// Mailbox of one ordered pair; lives in the sender's slot, indexed by destination.  Message k
+// (from 1) travels in ring[(k - 1) % kRing]; the sender writes the entry and then `posted`, the
+// receiver reads the entry after it has seen `posted` and writes `consumed` once its copy out of
+// the buffer has finished.
+struct alignas(64) P2PBox {
+  std::atomic<uint64_t> posted;
+  std::atomic<uint64_t> consumed;
+  P2PEntry ring[kRing];
+};
+
 struct alignas(128) RankSlot {
   std::atomic<uint64_t> arrive;  // host barrier: epoch this rank has reached
   std::atomic<uint64_t> failed;  // non-zero once the rank gave up; peers stop waiting
@@ -149,6 +171,7 @@ struct alignas(128) RankSlot {
   uint64_t capacity[2];
   hipIpcMemHandle_t handle[2];
   int64_t table[2][kTableMax];
+  P2PBox p2p[kMaxWorld];
 };
 
 struct Control {
@@ -267,7 +290,30 @@ ProcessGroupCCL::~ProcessGroupCCL() {
            std::chrono::steady_clock::now() < deadline)
       sched_yield();
   }
+  // Messages this rank has sent and nobody has copied out yet live in its staging buffers: give
+  // the receivers a bounded time, then flag the failure so that a late receiver raises instead of
+  // reading freed memory.
+  {
+    const auto p2p_deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(10000);
+    for (int d = 0; d < size_; ++d) {
+      P2PBox& box = ctl_->slot[rank_].p2p[d];
+      while (box.consumed.load(std::memory_order_acquire) < box.posted.load(std::memory_order_relaxed)) {
+        if (ctl_->slot[d].departed.load(std::memory_order_acquire) || ctl_->slot[d].failed.load(std::memory_order_acquire) ||
+            std::chrono::steady_clock::now() > p2p_deadline) {
+          ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+          break;
+        }
+        sched_yield();
+      }
+    }
+  }
   (void)hipDeviceSynchronize();
+  for (auto& pr : p2p_recv_)
+    for (int i = 0; i < kP2PRing; ++i)
+      if (pr.ipc[i] && pr.base[i]) (void)hipIpcCloseMemHandle(pr.base[i]);
+  for (auto& ps : p2p_send_)
+    for (int i = 0; i < kP2PRing; ++i)
+      if (ps.base[i]) (void)hipFree(ps.base[i]);
   for (auto& pm : peers_)
     for (int s = 0; s < 2; ++s)
       if (pm.ipc[s] && pm.base[s]) (void)hipIpcCloseMemHandle(pm.base[s]);
@@ -321,6 +367,8 @@ void ProcessGroupCCL::ensureInit(int device) {
   }
   ctl_->slot[rank_].pid = (int64_t)getpid();
   peers_.assign((size_t)size_, PeerMap{});
+  p2p_send_.assign((size_t)size_, P2PSend{});
+  p2p_recv_.assign((size_t)size_, P2PRecv{});
   initialised_ = true;
   for (int s = 0; s < 2; ++s) ensureStage(s, kStageMin);
 
@@ -518,10 +566,6 @@ void ProcessGroupCCL::checkDeviceTensors(const std::vector<at::Tensor>& tensors)
     TORCH_CHECK(!t.is_sparse(), "ccl backend: sparse tensors are not supported");
     TORCH_CHECK(t.is_contiguous(t.suggest_memory_format()), "input dense tensor has to be contiguous");
   }
-}
-
-void ProcessGroupCCL::notImplemented(const char* what) const {
-  TORCH_CHECK(false, "oneccl_bindings_for_pytorch: ", what, " isn't implementd on backend [cuda].");
 }
 
 void ProcessGroupCCL::startCoalescing() { coalescing_ = true; }
@@ -1243,8 +1287,192 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
   }
   return run(p);
 }
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::send(std::vector<at::Tensor>&, int, int) { notImplemented("send"); }
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>&, int, int) { notImplemented("recv"); }
+// ---------------------------------------------------------------------------------------------
+// point to point
+// ---------------------------------------------------------------------------------------------
+void ProcessGroupCCL::spinUntil(const std::function<bool()>& ready, int peer, const char* what,
+                                const std::function<bool()>& abandoned) {
+  std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(30000));
+  if (const char* v = std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
+    const long ms = std::atol(v);
+    if (ms > 0) limit = std::chrono::milliseconds(ms);
+  }
+  const auto deadline = std::chrono::steady_clock::now() + limit;
+  unsigned spins = 0;
+  while (!ready()) {
+    if (ctl_->slot[peer].failed.load(std::memory_order_acquire))
+      TORCH_CHECK(false, "ccl backend: rank ", peer, " reported a failure while this rank was waiting for ", what);
+    if (ctl_->slot[peer].departed.load(std::memory_order_acquire) && abandoned() && !ready()) {
+      ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+      TORCH_CHECK(false, "ccl backend: rank ", peer, " left the group while this rank was waiting for ", what);
+    }
+    if (++spins < 2000) continue;
+    sched_yield();
+    if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
+      ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+      TORCH_CHECK(false, "ccl backend: timed out waiting for ", what, " (rank ", peer, ")");
+    }
+  }
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::send(std::vector<at::Tensor>& tensors, int dstRank, int /*tag*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::send", std::vector<c10::IValue>({tensors}));
+  checkRank(dstRank, size_);
+  TORCH_CHECK(tensors.size() == 1, "CCL process group does not support tensors count ", tensors.size());
+  checkDeviceTensors(tensors);
+  at::Tensor t = tensors[0];
+  std::lock_guard<std::mutex> lock(mutex_);
+  c10::DeviceGuard dev_guard(t.device());
+  ensureInit(t.get_device());
+  hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_).stream();
+  P2PBox& box = ctl_->slot[rank_].p2p[dstRank];
+  P2PSend& mine = p2p_send_[(size_t)dstRank];
+  const size_t total = nbytes(t);
+  size_t off = 0;
+  do {  // an empty tensor still travels as one (empty) message, so that sends and receives pair up
+    const size_t len = std::min(total - off, kStageMax);
+    const uint64_t k = box.posted.load(std::memory_order_relaxed) + 1;
+    spinUntil([&] { return k - box.consumed.load(std::memory_order_acquire) <= (uint64_t)kRing; }, dstRank,
+              "a free send buffer", [] { return true; });
+    const int slot = (int)((k - 1) % kRing);
+    P2PEntry& e = box.ring[slot];
+    if (len > mine.capacity[slot]) {
+      size_t cap = kP2PMinBytes;
+      while (cap < len) cap <<= 1;
+      void* base = nullptr;
+      HIP_CHECK(hipMalloc(&base, cap));
+      if (mine.base[slot]) retired_.push_back(mine.base[slot]);  // the receiver may still hold a mapping
+      mine.base[slot] = base;
+      mine.capacity[slot] = cap;
+      if (size_ > 1) HIP_CHECK(hipIpcGetMemHandle(&e.handle, base));
+      e.ptr = (uint64_t)(uintptr_t)base;
+      e.capacity = cap;
+      e.gen += 1;
+    }
+    if (len) {
+      copyAsync(mine.base[slot], (const char*)t.data_ptr() + off, len, cur);
+      HIP_CHECK(hipStreamSynchronize(cur));  // the message is published only once it is complete
+    }
+    e.bytes = len;
+    box.posted.store(k, std::memory_order_release);
+    off += len;
+  } while (off < total);
+  // the data has left the tensor: nothing is pending
+  return c10::make_intrusive<WorkCCL>(rank_, c10d::OpType::SEND, "send", std::vector<at::Tensor>{t},
+                                      std::vector<at::Tensor>{}, blocking_wait_);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>& tensors, int srcRank, int /*tag*/) {
+  RECORD_FUNCTION("oneccl_bindings_for_pytorch::recv", std::vector<c10::IValue>({tensors}));
+  checkRank(srcRank, size_);
+  TORCH_CHECK(tensors.size() == 1, "CCL process group does not support tensors count ", tensors.size());
+  checkDeviceTensors(tensors);
+  auto state = std::make_shared<RecvState>();
+  state->tensor = tensors[0];
+  state->src = srcRank;
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    c10::DeviceGuard dev_guard(state->tensor.device());
+    ensureInit(state->tensor.get_device());
+    P2PRecv& pr = p2p_recv_[(size_t)srcRank];
+    const size_t total = nbytes(state->tensor);
+    const uint64_t nmsg = total ? (total + kStageMax - 1) / kStageMax : 1;
+    state->first_seq = pr.assigned + 1;
+    pr.assigned += nmsg;
+    pr.pending.push_back(state);
+  }
+  auto self = c10::intrusive_ptr<ProcessGroupCCL>::unsafe_reclaim_from_nonowning(this);
+  return c10::make_intrusive<RecvWorkCCL>(std::move(self), std::move(state), rank_);
+}
+
+void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocking) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  if (target->done) return;
+  c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
+  hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_).stream();
+  P2PBox& box = ctl_->slot[src].p2p[rank_];
+  P2PRecv& pr = p2p_recv_[(size_t)src];
+  while (!pr.pending.empty()) {
+    std::shared_ptr<RecvState> st = pr.pending.front();
+    const size_t total = nbytes(st->tensor);
+    size_t off = 0;
+    uint64_t k = st->first_seq;
+    if (!blocking && box.posted.load(std::memory_order_acquire) < k + (total ? (total - 1) / kStageMax : 0)) return;
+    do {
+      const size_t len = std::min(total - off, kStageMax);
+      spinUntil([&] { return box.posted.load(std::memory_order_acquire) >= k; }, src, "a message",
+                [&] { return box.posted.load(std::memory_order_acquire) < k; });
+      const int slot = (int)((k - 1) % kRing);
+      const P2PEntry& e = box.ring[slot];
+      if (e.bytes != len) {
+        // The two sides disagree about the message stream: drop the message and the receive, and
+        // flag the group as failed (what follows on this pair can no longer be matched reliably).
+        const uint64_t have = e.bytes;
+        box.consumed.store(k, std::memory_order_release);
+        st->done = true;
+        pr.pending.pop_front();
+        ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+        TORCH_CHECK(false, "ccl backend: recv expects ", len, " bytes from rank ", src, " but the message holds ", have);
+      }
+      if (len) {
+        const void* from = nullptr;
+        if (ctl_->slot[src].pid == (int64_t)getpid()) {
+          from = (const void*)(uintptr_t)e.ptr;
+        } else {
+          if (pr.gen[slot] != e.gen) {
+            if (pr.ipc[slot] && pr.base[slot]) (void)hipIpcCloseMemHandle(pr.base[slot]);
+            pr.base[slot] = nullptr;
+            pr.ipc[slot] = false;
+            void* m = nullptr;
+            HIP_CHECK(hipIpcOpenMemHandle(&m, e.handle, hipIpcMemLazyEnablePeerAccess));
+            pr.base[slot] = m;
+            pr.ipc[slot] = true;
+            pr.gen[slot] = e.gen;
+          }
+          from = pr.base[slot];
+        }
+        TORCH_CHECK(!ctl_->slot[src].failed.load(std::memory_order_acquire),
+                    "ccl backend: rank ", src, " gave up on a message before it was received");
+        copyAsync((char*)st->tensor.data_ptr() + off, from, len, cur);
+        HIP_CHECK(hipStreamSynchronize(cur));  // the sender may reuse the buffer once `consumed` moves
+      }
+      box.consumed.store(k, std::memory_order_release);
+      ++k;
+      off += len;
+    } while (off < total);
+    st->done = true;
+    pr.pending.pop_front();
+    if (st.get() == target) return;
+  }
+}
+
+ProcessGroupCCL::RecvWorkCCL::RecvWorkCCL(c10::intrusive_ptr<ProcessGroupCCL> pg, std::shared_ptr<RecvState> state,
+                                          int rank)
+    : c10d::Work(rank, c10d::OpType::RECV, "recv"), pg_(std::move(pg)), state_(std::move(state)) {}
+
+bool ProcessGroupCCL::RecvWorkCCL::isCompleted() {
+  pg_->progressRecv(state_->src, state_.get(), /*blocking=*/false);
+  return state_->done;
+}
+
+void ProcessGroupCCL::RecvWorkCCL::synchronize() { pg_->progressRecv(state_->src, state_.get(), /*blocking=*/true); }
+
+bool ProcessGroupCCL::RecvWorkCCL::wait(std::chrono::milliseconds /*timeout*/) {
+  synchronize();
+  return true;
+}
+
+std::vector<at::Tensor> ProcessGroupCCL::RecvWorkCCL::result() { return {state_->tensor}; }
+
+c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupCCL::RecvWorkCCL::getFuture() {
+  if (!future_) {
+    synchronize();  // the host has waited for the copy: the tensor is ready for any stream
+    future_ = c10::make_intrusive<at::ivalue::Future>(c10::ListType::create(c10::TensorType::get()));
+    future_->markCompleted(at::IValue(std::vector<at::Tensor>{state_->tensor}));
+  }
+  return future_;
+}
+
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recvAnysource(std::vector<at::Tensor>&, int) {
   TORCH_CHECK(false, "ProcessGroupCCL does not support recvAnysource");
 }

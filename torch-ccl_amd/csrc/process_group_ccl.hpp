@@ -23,6 +23,7 @@
 #include <torch/csrc/distributed/c10d/Work.hpp>
 
 #include <chrono>
+#include <deque>
 #include <functional>
 #include <memory>
 #include <mutex>
@@ -57,6 +58,33 @@ class ProcessGroupCCL : public c10d::Backend {
     bool blocking_wait_ = false;
     std::vector<at::Tensor> inputs_;   // held until the Work dies (ownership rule of the reference)
     std::vector<at::Tensor> outputs_;
+    c10::intrusive_ptr<c10::ivalue::Future> future_;
+  };
+
+  // What a posted receive still has to do; the group keeps these per source in posting order.
+  struct RecvState {
+    at::Tensor tensor;
+    int src = 0;
+    uint64_t first_seq = 0;  // sequence number (from 1) of the first message of this receive
+    bool done = false;
+  };
+
+  // Work of a receive (XPUP2PAsyncWork of the reference, src/gpu/dpcpp_ccl.cpp:1590-1627).  The
+  // message is matched and copied out when somebody waits for it (or polls isCompleted once the
+  // sender has published it): no progress thread runs behind the caller's back.
+  class RecvWorkCCL : public c10d::Work {
+   public:
+    RecvWorkCCL(c10::intrusive_ptr<ProcessGroupCCL> pg, std::shared_ptr<RecvState> state, int rank);
+    bool isCompleted() override;
+    bool isSuccess() const override { return true; }
+    bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
+    void synchronize() override;
+    std::vector<at::Tensor> result() override;
+    c10::intrusive_ptr<c10::ivalue::Future> getFuture() override;
+
+   private:
+    c10::intrusive_ptr<ProcessGroupCCL> pg_;  // a pending receive keeps its group alive
+    std::shared_ptr<RecvState> state_;
     c10::intrusive_ptr<c10::ivalue::Future> future_;
   };
 
@@ -118,10 +146,13 @@ class ProcessGroupCCL : public c10d::Backend {
                                         const c10d::GatherOptions& opts) override;
   c10::intrusive_ptr<c10d::Work> scatter(std::vector<at::Tensor>& outputs, std::vector<std::vector<at::Tensor>>& inputs,
                                          const c10d::ScatterOptions& opts) override;
-  // Not on the path this backend covers; they fail like DispatchStub::fail does
-  // (src/dispatch_stub.h:288-290).
-  c10::intrusive_ptr<c10d::Work> send(std::vector<at::Tensor>&, int, int) override;
-  c10::intrusive_ptr<c10d::Work> recv(std::vector<at::Tensor>&, int, int) override;
+  // Point to point: a send copies the tensor into one of a few staging buffers kept per
+  // destination and publishes it; it returns as soon as the data has left the tensor and blocks
+  // only while all of those buffers hold unconsumed messages.  A receive is matched in posting
+  // order per source when it is waited for.  The tag is ignored, as in the reference.
+  c10::intrusive_ptr<c10d::Work> send(std::vector<at::Tensor>& tensors, int dstRank, int tag) override;
+  c10::intrusive_ptr<c10d::Work> recv(std::vector<at::Tensor>& tensors, int srcRank, int tag) override;
+  // Not supported by the reference either (src/ProcessGroupCCL.cpp:1217-1222).
   c10::intrusive_ptr<c10d::Work> recvAnysource(std::vector<at::Tensor>&, int) override;
 
  private:
@@ -151,7 +182,13 @@ class ProcessGroupCCL : public c10d::Backend {
   void hostBarrier();
   const void* peerStage(int peer, int slot);
   void checkDeviceTensors(const std::vector<at::Tensor>& tensors) const;
-  [[noreturn]] void notImplemented(const char* what) const;
+  // Spins (then yields) until ready() holds; raises when `peer` reports a failure, when it has
+  // left and abandoned() says that what is awaited can no longer come, or at the time limit.
+  void spinUntil(const std::function<bool()>& ready, int peer, const char* what,
+                 const std::function<bool()>& abandoned);
+  // Completes the receives posted for `src` in order, up to and including `target`.  With
+  // blocking == false it stops at the first message the sender has not published yet.
+  void progressRecv(int src, const RecvState* target, bool blocking);
 
   c10::intrusive_ptr<c10d::Store> store_;
   std::chrono::milliseconds timeout_;
@@ -197,6 +234,22 @@ class ProcessGroupCCL : public c10d::Backend {
     bool ipc[2] = {false, false};
   };
   std::vector<PeerMap> peers_;
+
+  // point to point
+  static constexpr int kP2PRing = 4;
+  struct P2PSend {  // per destination: this rank's staging buffers
+    void* base[kP2PRing] = {nullptr, nullptr, nullptr, nullptr};
+    size_t capacity[kP2PRing] = {0, 0, 0, 0};
+  };
+  struct P2PRecv {  // per source
+    uint64_t assigned = 0;  // messages handed to posted receives so far
+    std::deque<std::shared_ptr<RecvState>> pending;
+    void* base[kP2PRing] = {nullptr, nullptr, nullptr, nullptr};  // mappings of the sender's buffers
+    uint64_t gen[kP2PRing] = {0, 0, 0, 0};
+    bool ipc[kP2PRing] = {false, false, false, false};
+  };
+  std::vector<P2PSend> p2p_send_;
+  std::vector<P2PRecv> p2p_recv_;
 };
 
 }  // namespace mccl_pg
