@@ -489,6 +489,37 @@ def ddp_case(rank, world):
     assert torch.allclose(gshard, want, rtol=1e-6)
 
 
+def subgroup_case(rank, world):
+    """Subgroups as the reference's tests/ds_subgroup_allreduce.py builds them: a one-rank group, then
+    strided groups of `sub` ranks; plus a rooted op and a send / recv addressed by global rank inside
+    a subgroup."""
+    sub = 2
+    warm = torch.ones(1, dtype=torch.bfloat16, device=DEV)
+    dist.all_reduce(warm)
+    assert float(warm[0]) == world
+    x = torch.ones(2048, dtype=torch.bfloat16, device=DEV)
+    g1 = dist.new_group([0])
+    if rank == 0:
+        dist.all_reduce(x, group=g1)
+        assert torch.equal(x.cpu(), torch.ones(2048, dtype=torch.bfloat16))
+    members = [[i + (world // sub) * j for j in range(sub)] for i in range(world // sub)]
+    groups = [dist.new_group(m) for m in members]
+    for m, g in zip(members, groups):
+        if rank in m:
+            dist.all_reduce(x, group=g)
+            assert torch.equal(x.cpu(), torch.full((2048,), float(sub), dtype=torch.bfloat16))
+            t = torch.full((5,), float(rank), device=DEV)
+            dist.broadcast(t, src=m[-1], group=g)
+            assert t.cpu().tolist() == [float(m[-1])] * 5
+            got = torch.zeros(3, device=DEV)
+            peer = m[1 - m.index(rank)]
+            reqs = [dist.irecv(got, src=peer, group=g), dist.isend(torch.full((3,), float(rank), device=DEV), dst=peer, group=g)]
+            for q in reqs:
+                q.wait()
+            assert got.cpu().tolist() == [float(peer)] * 3
+    dist.barrier()
+
+
 def run_rank(rank, world, store_path, mode):
     torch.cuda.set_device(0)
     import torch_ccl_amd  # noqa: F401  registers the backend
@@ -497,6 +528,14 @@ def run_rank(rank, world, store_path, mode):
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
             dist_api_cases(rank, world)
+        finally:
+            dist.destroy_process_group()
+        return
+    if mode == "subgroup":
+        store = dist.FileStore(store_path, world)
+        dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
+        try:
+            subgroup_case(rank, world)
         finally:
             dist.destroy_process_group()
         return

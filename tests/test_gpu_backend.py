@@ -38,6 +38,10 @@ def test_send_recv(world):
     _spawn(world, "p2p")
 
 
+def test_subgroups():
+    _spawn(4, "subgroup")
+
+
 def test_message_larger_than_one_staging_window():
     _spawn(2, "large")
 
