@@ -489,6 +489,35 @@ def ddp_case(rank, world):
     assert torch.allclose(gshard, want, rtol=1e-6)
 
 
+def identity_replay_case(rank, world):
+    """The reference's tests/test_allreduce.py in small: fp16 data of 0.1 is allreduced and divided
+    by the (power-of-two) world size round after round, interleaved with elementwise kernels that
+    consume it on the caller's stream.  x*W/W == x exactly, so data must keep its bits and the
+    accumulator must equal a replay without any collective; a collective that ran before its
+    input was ready, or let its consumer start early, breaks that.  Two sizes: one staged on the
+    caller's stream (28 KiB), one on the communication stream (2 MiB)."""
+    assert world & (world - 1) == 0
+    for count, rounds in ((14336, 150), (1 << 20, 40)):
+        data = (torch.ones(count, dtype=torch.float16) * 0.1).to(DEV)
+        keep = data.clone()
+        a = torch.zeros(8, count, dtype=torch.float16, device=DEV)
+        want = torch.zeros(8, count, dtype=torch.float16, device=DEV)
+        for _ in range(rounds):
+            a[0] += data * 0.1
+            for _ in range(4):
+                a += 0.01
+            dist.all_reduce(data)
+            data /= world
+        for _ in range(rounds):
+            want[0] += keep * 0.1
+            for _ in range(4):
+                want += 0.01
+        torch.cuda.synchronize()
+        assert torch.equal(data.view(torch.int16), keep.view(torch.int16)), count
+        assert torch.equal(a.view(torch.int16), want.view(torch.int16)), count
+    dist.barrier()
+
+
 def subgroup_case(rank, world):
     """Subgroups as the reference's tests/ds_subgroup_allreduce.py builds them: a one-rank group, then
     strided groups of `sub` ranks; plus a rooted op and a send / recv addressed by global rank inside
@@ -531,11 +560,11 @@ def run_rank(rank, world, store_path, mode):
         finally:
             dist.destroy_process_group()
         return
-    if mode == "subgroup":
+    if mode in ("subgroup", "replay"):
         store = dist.FileStore(store_path, world)
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
-            subgroup_case(rank, world)
+            (subgroup_case if mode == "subgroup" else identity_replay_case)(rank, world)
         finally:
             dist.destroy_process_group()
         return

@@ -38,6 +38,11 @@ def test_send_recv(world):
     _spawn(world, "p2p")
 
 
+@pytest.mark.parametrize("world", [2, 8])
+def test_identity_replay_interleaved_with_compute(world):
+    _spawn(world, "replay")
+
+
 def test_subgroups():
     _spawn(4, "subgroup")
 
