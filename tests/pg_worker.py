@@ -489,6 +489,54 @@ def ddp_case(rank, world):
     assert torch.allclose(gshard, want, rtol=1e-6)
 
 
+def reference_p2p_cases(rank, world):
+    """The four cases of the reference's tests/test_c10d_p2p.py (world size 6, cubes of rank+1
+    elements per side filled with rank+1): a pair (:38-68), a relay 1 -> 3 -> 5 (:73-109), every
+    rank sending to all others in turn (:114-147), and the same with tags (:152-183)."""
+    def cube(n, value=None):
+        return torch.full((n, n, n), float(n if value is None else value))
+
+    dist.all_reduce(torch.zeros(1, device=DEV))  # the reference's tests start with one, too
+    mine = cube(rank + 1).to(DEV)
+    if rank == 0:
+        dist.send(mine, 1)
+    elif rank == 1:
+        out = cube(1, -1).to(DEV)
+        dist.recv(out, 0)
+        assert torch.equal(out.cpu(), cube(1))
+    if rank == 1:
+        dist.send(mine, 3)
+    if rank == 3:
+        out = cube(2, -1).to(DEV)
+        dist.recv(out, 1)
+        assert torch.equal(out.cpu(), cube(2))
+        dist.send(mine, 5)
+    if rank == 5:
+        out = cube(4, -1).to(DEV)
+        dist.recv(out, 3)
+        assert torch.equal(out.cpu(), cube(4))
+    for src in range(world):
+        if src == rank:
+            for dst in range(world):
+                if dst != rank:
+                    dist.send(mine, dst)
+        else:
+            out = cube(src + 1, -1).to(DEV)
+            dist.recv(out, src)
+            assert torch.equal(out.cpu(), cube(src + 1))
+    tagged = cube(10, rank).to(DEV)
+    for dst in range(world):
+        if dst == rank:
+            for src in range(world):
+                if src != rank:
+                    out = cube(10, -1).to(DEV)
+                    dist.recv(out, src, tag=src)
+                    assert bool(out.eq(src).all())
+        else:
+            dist.send(tagged, dst, tag=rank)
+    dist.barrier()
+
+
 def identity_replay_case(rank, world):
     """The reference's tests/test_allreduce.py in small: fp16 data of 0.1 is allreduced and divided
     by the (power-of-two) world size round after round, interleaved with elementwise kernels that
@@ -560,11 +608,11 @@ def run_rank(rank, world, store_path, mode):
         finally:
             dist.destroy_process_group()
         return
-    if mode in ("subgroup", "replay"):
+    if mode in ("subgroup", "replay", "reference_p2p"):
         store = dist.FileStore(store_path, world)
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
-            (subgroup_case if mode == "subgroup" else identity_replay_case)(rank, world)
+            {"subgroup": subgroup_case, "replay": identity_replay_case, "reference_p2p": reference_p2p_cases}[mode](rank, world)
         finally:
             dist.destroy_process_group()
         return

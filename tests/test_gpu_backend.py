@@ -47,6 +47,10 @@ def test_subgroups():
     _spawn(4, "subgroup")
 
 
+def test_reference_send_recv_cases():
+    _spawn(6, "reference_p2p")
+
+
 def test_message_larger_than_one_staging_window():
     _spawn(2, "large")
 
