@@ -364,9 +364,10 @@ def p2p_cases(pg, rank, world):
     got = torch.zeros(5, dtype=torch.uint8, device=DEV)
     w = pg.recv([got], prv, 0)
     pg.send([payload(rank, nxt, 50, 5).to(DEV)], nxt, 0).wait()
-    for _ in range(200000):
-        if w.is_completed():
-            break
+    import time
+    deadline = time.time() + 60.0
+    while not w.is_completed() and time.time() < deadline:
+        pass
     assert w.is_completed() and np.array_equal(bits(got), bits(payload(prv, rank, 50, 5)))
     pg.barrier().wait()
 
