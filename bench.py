@@ -521,7 +521,20 @@ def main():
                            "split_rows_rank0": S5[0].tolist()}
             log("C5:", json.dumps(result[key]))
             del a2a_out
-        del a2a_in
+        # the same exchange at decode size: 16 tokens per rank (128 routed rows, 1.75 MiB per rank),
+        # all 64 segments in one launch
+        S5s = torch.zeros(N, N, dtype=torch.int64)
+        for r in range(N):
+            g = rank_generator(torch, SEED, r)
+            experts = torch.topk(torch.randn(tokens, 256, generator=g)[:16], topk, dim=1).indices
+            S5s[r] = torch.bincount(experts.reshape(-1) // 32, minlength=N)
+        small_in = [t[:16 * topk] for t in a2a_in]
+        small_out = [torch.empty(int(S5s[:, d].sum()), hidden, dtype=torch.bfloat16, device=dev) for d in range(N)]
+        us = benchlib.alltoallv_throughput(small_in, small_out, S5s, hidden * 2, warmup=20, iters=200)
+        result["c5_alltoallv_decode_16_tokens"] = {"us": round(us, 2), "bytes_moved": int(S5s.sum()) * hidden * 2,
+                                                   "launches": 1}
+        log("C5 decode size:", json.dumps(result["c5_alltoallv_decode_16_tokens"]))
+        del a2a_in, small_in, small_out
 
     # ---------------- the steps either side of C5: token permute fused into the dispatch, weighted combine ----------------
     if "moe" in extras:
