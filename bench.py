@@ -177,7 +177,10 @@ def gloo_baseline(world=8):
     import tempfile
     import torch
     import torch.multiprocessing as mp
-    backend = "ccl" if importlib.util.find_spec("oneccl_bindings_for_pytorch") else "gloo"
+    # the reference's wheel, not the import-name shim this repository carries beside its own package
+    spec = importlib.util.find_spec("oneccl_bindings_for_pytorch")
+    reference_wheel = spec is not None and spec.origin and not os.path.abspath(spec.origin).startswith(ROOT + os.sep)
+    backend = "ccl" if reference_wheel else "gloo"
     cases = [("c2_256KiB_bf16", 16 * 8192, "bfloat16", 0.02, 20, 300),
              ("c3_64MiB_bf16", 4096 * 8192, "bfloat16", 0.02, 3, 12)]
     with tempfile.TemporaryDirectory() as d:
