@@ -39,7 +39,8 @@ def test_gather_rows_skips_out_of_range_indices(mccl):
     assert out.cpu().tolist() == [[12, 13, 14, 15], [-7] * 4, [-7] * 4, [0, 1, 2, 3], [-7] * 4]
 
 
-@pytest.mark.parametrize("n,tokens,hidden,topk,n_exp", [(8, 64, 128, 8, 256), (4, 100, 96, 2, 16), (2, 33, 7168, 4, 8)])
+@pytest.mark.parametrize("n,tokens,hidden,topk,n_exp", [(8, 64, 128, 8, 256), (4, 100, 96, 2, 16), (2, 33, 7168, 4, 8),
+                                                        (17, 30, 64, 3, 34)])
 def test_fused_dispatch_equals_gather_then_alltoallv(mccl, n, tokens, hidden, topk, n_exp):
     S, send_tok, _ = route(n, tokens, n_exp, topk)
     hid = []
