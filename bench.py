@@ -389,6 +389,14 @@ def main():
             ev[vname] = {"us": round(us, 1), "GBps": round(alg_bytes / us / 1e3, 1)}
         result["c3_shapes"] = ev
         log("C3 shapes:", json.dumps(ev))
+        # the reference's allreduce is in place on each rank's own buffer: the same launch writing
+        # into rank 0's input (same bytes moved; the written DRAM pages were read a moment before)
+        fresh = [t.clone() for t in ins]
+        us = benchlib.reduce_throughput([fresh], [fresh[0]], warmup=5, iters=30)
+        result["c3_in_place_on_rank0"] = {"us": round(us, 1), "GBps": round(alg_bytes / us / 1e3, 1),
+                                          "pct_of_peak": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS * 100, 1)}
+        log("C3 in place:", json.dumps(result["c3_in_place_on_rank0"]))
+        del fresh
 
     # ---------------- coalesced and list forms: one fused launch against one launch per tensor ----------------
     if "lists" in extras:
