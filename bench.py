@@ -433,7 +433,7 @@ def main():
         us_copy_ = timed_us(lambda: [flat[o:o + t.numel()].copy_(t) for o, t in
                                      zip([sum(p.numel() for p in pieces[:i]) for i in range(len(pieces))], pieces)])
         result["coalesced_and_list_forms"] = {
-            "note": "HIP events around 20 repetitions; reduce calls go straight to the C ABI with prebuilt argument tables, pack/copy through the Python front ends",
+            "note": "HIP events bracketing 20 repetitions; reduce calls go straight to the C ABI with prebuilt argument tables, pack/copy through the Python front ends",
             "allreduce_coalesced_32x512KiB_8ranks": {"fused_launches_us": round(us_fused, 1),
                                                       "one_launch_per_tensor_us": round(us_each, 1),
                                                       "bit_identical": same},
