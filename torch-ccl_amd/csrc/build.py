@@ -139,8 +139,24 @@ def build_backend(force=False):
     return out
 
 
+C_CALLER_SRC = os.path.join(ROOT, "tests", "c_abi", "caller.c")
+C_CALLER_BIN = os.path.join(ROOT, "tests", "c_abi", "caller")
+
+
+def build_c_caller(force=False):
+    """The plain-C host of tests/c_abi: gcc in C mode against include/mccl.h and the HIP runtime's
+    C API; proves that the boundary needs no C++ and no torch."""
+    if force or _stale(C_CALLER_BIN, [C_CALLER_SRC, os.path.join(INCLUDE, "mccl.h"), KERNEL_LIB]):
+        subprocess.check_call(["gcc", "-std=c11", "-O1", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__=1",
+                               "-I", INCLUDE, "-isystem", "/opt/rocm/include", "-o", C_CALLER_BIN, C_CALLER_SRC,
+                               "-L", LIB_DIR, "-lmi355ccl", "-L", "/opt/rocm/lib", "-lamdhip64",
+                               "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,$ORIGIN/../../torch-ccl_amd/torch_ccl_amd/lib",
+                               "-Wl,-rpath,/opt/rocm/lib"])
+    return C_CALLER_BIN
+
+
 def build_all(force=False):
-    return [build_kernels(force), build_bench(force), build_backend(force)]
+    return [build_kernels(force), build_bench(force), build_backend(force), build_c_caller(force)]
 
 
 def ensure_built():
@@ -153,6 +169,8 @@ def ensure_built():
         built.append(build_bench(force=True))
     if not os.path.exists(backend_lib_path()):
         built.append(build_backend(force=True))
+    if not os.path.exists(C_CALLER_BIN):
+        built.append(build_c_caller(force=True))
     return built
 
 
