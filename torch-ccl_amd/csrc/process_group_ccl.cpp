@@ -372,10 +372,7 @@ void ProcessGroupCCL::ensureInit(int device) {
   initialised_ = true;
   for (int s = 0; s < 2; ++s) ensureStage(s, kStageMin);
 
-  auto saved = timeout_;
-  if (timeout_ < std::chrono::milliseconds(120000)) timeout_ = std::chrono::milliseconds(120000);
-  hostBarrier();
-  timeout_ = saved;
+  hostBarrier(/*start_up=*/true);
   TORCH_CHECK(ctl_->magic == kMagic && ctl_->world == (uint32_t)size_,
               "ccl backend: control block mismatch (ranks disagree on the world size)");
   if (rank_ == 0) shm_unlink(shm_name_.c_str());  // every rank holds a mapping now
@@ -424,13 +421,14 @@ const void* ProcessGroupCCL::peerStage(int peer, int slot) {
   return pm.ptr[slot];
 }
 
-void ProcessGroupCCL::hostBarrier() {
+void ProcessGroupCCL::hostBarrier(bool start_up) {
   const uint64_t epoch = ++barrier_epoch_;
   ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
-  // Floor of 30 s under short user timeouts (ranks start at different speeds);
-  // MCCL_BARRIER_TIMEOUT_MS overrides it, e.g. to exercise the failure path quickly.
-  std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(30000));
-  if (const char* v = std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
+  // Floor of 30 s under short user timeouts; MCCL_BARRIER_TIMEOUT_MS overrides it, e.g. to
+  // exercise the failure path quickly.  The first barrier of a group waits for ranks that may
+  // still be starting (a first import on a cold machine takes a minute): two minutes at least.
+  std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(start_up ? 120000 : 30000));
+  if (const char* v = start_up ? nullptr : std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
     const long ms = std::atol(v);
     if (ms > 0) limit = std::chrono::milliseconds(ms);
   }

@@ -179,7 +179,9 @@ class ProcessGroupCCL : public c10d::Backend {
   c10::intrusive_ptr<c10d::Work> run(Plan& plan);
   void ensureInit(int device);
   void* ensureStage(int slot, size_t bytes);
-  void hostBarrier();
+  // start_up: the first barrier of a group, which also absorbs the ranks' different start-up
+  // times: at least two minutes, and not shortened by MCCL_BARRIER_TIMEOUT_MS
+  void hostBarrier(bool start_up = false);
   const void* peerStage(int peer, int slot);
   void checkDeviceTensors(const std::vector<at::Tensor>& tensors) const;
   // Spins (then yields) until ready() holds; raises when `peer` reports a failure, when it has
