@@ -288,7 +288,8 @@ def main():
                                "output, all resident in one GPU's HBM",
                    "ranks": N, "elements_per_rank": COUNT, "algorithmic_bytes_per_step": alg_bytes,
                    "kernel": "reduce_vec_kernel<bf16,SUM,8 ranks> shape=stream grid=%d block=%d lds=%d" % (
-                       grid, blk.value, lds.value)},
+                       grid, blk.value, lds.value),
+                   "buffer_offsets_MiB": [round((t.data_ptr() - ins[0].data_ptr()) / 2**20, 3) for t in ins + [out]]},
         "pct_of_peak": round(value / PEAK_HBM_GBS * 100, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": C3_TRAFFIC_BYTES_ROCPROF,
