@@ -111,3 +111,22 @@ def test_config5_moe_alltoallv_full_size(mccl, n_experts):
     cpu_in = [t.cpu().view(torch.int16).numpy().view(np.uint16) for t in ins]
     want = O.alltoallv(cpu_in, S.numpy(), hidden * 2)[d]
     assert_bits_equal(bits(outs[d]).view(np.uint8), want, "oracle, destination %d" % d)
+
+
+def test_more_than_four_gi_elements(mccl):
+    """Element and byte offsets beyond 2^32: two u8 buffers of 4 GiB + 1000 bytes summed (u8 wraps),
+    and the same span moved as one copy segment; checked against torch's own elementwise add and
+    compare on the device."""
+    count = (1 << 32) + 1000
+    g = torch.Generator(device=DEV).manual_seed(5)
+    a = torch.randint(0, 256, (count,), dtype=torch.uint8, device=DEV, generator=g)
+    b = torch.randint(0, 256, (count,), dtype=torch.uint8, device=DEV, generator=g)
+    out = mccl.reduce_n([a, b])
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + b)
+    assert int(out[-1]) == (int(a[-1]) + int(b[-1])) % 256
+    dst = torch.zeros(count + 3, dtype=torch.uint8, device=DEV)
+    mccl.copy_segments([(a.data_ptr() + 1, dst.data_ptr() + 3, count - 1)])  # both ends off any boundary
+    torch.cuda.synchronize()
+    assert torch.equal(dst[3:3 + count - 1], a[1:])
+    assert int(dst[:3].sum()) == 0 and int(dst[-1]) == 0
