@@ -130,3 +130,21 @@ def test_more_than_four_gi_elements(mccl):
     torch.cuda.synchronize()
     assert torch.equal(dst[3:3 + count - 1], a[1:])
     assert int(dst[:3].sum()) == 0 and int(dst[-1]) == 0
+
+
+def test_grids_that_wrap(mccl):
+    """33 GiB in one buffer: more tiles (reduction) and more chunks (copy) than the largest grid the
+    launches use, so every workgroup walks several of them."""
+    count = 33 * (1 << 30) + 5
+    a = torch.empty(count, dtype=torch.uint8, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(9)
+    step = 1 << 32
+    for lo in range(0, count, step):
+        a[lo:lo + step].random_(0, 256, generator=g)
+    out = mccl.reduce_n([a])  # one rank: the chain from +0 returns the input
+    torch.cuda.synchronize()
+    assert torch.equal(out, a)
+    out.zero_()
+    mccl.copy_segments([(a.data_ptr(), out.data_ptr(), count)])
+    torch.cuda.synchronize()
+    assert torch.equal(out, a)
