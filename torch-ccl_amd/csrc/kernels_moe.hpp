@@ -88,13 +88,16 @@ struct CombineArgs {
   int n;
 };
 
-// FAST: top-k of at most 8 (one group of row loads covers a token); the general path is a kernel
-// of its own so that each gets its own register budget.
-template <int DT, bool FAST>
+// GROUP > 0: top-k of at most GROUP (2, 4 or 8: one group of row loads covers a token), each a
+// kernel of its own with its own register budget - a top-2 combine holds a quarter of the rows of
+// a top-8 one and fits half as many registers, so that more wavefronts (and loads) are in flight.
+// GROUP == 0: any top-k, entries in groups of 8.
+template <int DT, int GROUP>
 __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a) {
   using A = float;
   constexpr int VE = vec_elems<DT>();
-  constexpr int G = 8;  // row loads in flight per lane (one group covers top-8 routing)
+  constexpr bool FAST = GROUP > 0;
+  constexpr int G = FAST ? GROUP : 8;  // row loads in flight per lane and piece
   const uint32_t total = a.tokens * a.waves_per_row;
   const size_t row_stride = (size_t)a.row_vecs * 16;
   if constexpr (FAST) {

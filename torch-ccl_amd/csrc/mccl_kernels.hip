@@ -759,7 +759,10 @@ int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const in
   int rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
   // One wavefront per chunk of a row, no residency cap (5.7 TB/s uncapped, 5.1 at 8 wavefronts
-  // per CU).  Measured and not adopted: a persistent grid whose wavefronts look up the next
+  // per CU).  Top-k up to 2, 4 and 8 are kernels of their own: with fewer row buffers a
+  // wavefront needs fewer registers and more of them are resident (top-2 at 4096-wide rows 63 ->
+  // 67 % of the HBM peak, top-4 at 5120 68 -> 74 %, top-1 47 -> 63 %); four row buffers deep
+  // instead of two for top-2 changed nothing and cost top-1 seven points.  Measured and not adopted: a persistent grid whose wavefronts look up the next
   // chunk's routing entries while they stream the current rows (the knob below; 3-8 % slower at
   // every grid size, so the lookup is not what bounds the kernel), and one contiguous range of
   // tokens per XCD so that the wavefronts sharing routing entries meet in one L2 (9 % slower).
@@ -772,21 +775,20 @@ int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const in
   const unsigned lds = 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 g3((unsigned)grid), b3(kWave);
-  const bool fast = topk <= 8;
-  switch (dtype) {
-    case MCCL_BF16:
-      if (fast) hipLaunchKernelGGL((moe_combine_kernel<MCCL_BF16, true>), g3, b3, lds, s, a);
-      else hipLaunchKernelGGL((moe_combine_kernel<MCCL_BF16, false>), g3, b3, lds, s, a);
-      break;
-    case MCCL_F16:
-      if (fast) hipLaunchKernelGGL((moe_combine_kernel<MCCL_F16, true>), g3, b3, lds, s, a);
-      else hipLaunchKernelGGL((moe_combine_kernel<MCCL_F16, false>), g3, b3, lds, s, a);
-      break;
-    default:
-      if (fast) hipLaunchKernelGGL((moe_combine_kernel<MCCL_F32, true>), g3, b3, lds, s, a);
-      else hipLaunchKernelGGL((moe_combine_kernel<MCCL_F32, false>), g3, b3, lds, s, a);
-      break;
+  const int group = topk <= 2 ? 2 : topk <= 4 ? 4 : topk <= 8 ? 8 : 0;
+#define MCCL_LAUNCH_COMBINE(DT)                                                                     \
+  switch (group) {                                                                                  \
+    case 2: hipLaunchKernelGGL((moe_combine_kernel<DT, 2>), g3, b3, lds, s, a); break;              \
+    case 4: hipLaunchKernelGGL((moe_combine_kernel<DT, 4>), g3, b3, lds, s, a); break;              \
+    case 8: hipLaunchKernelGGL((moe_combine_kernel<DT, 8>), g3, b3, lds, s, a); break;              \
+    default: hipLaunchKernelGGL((moe_combine_kernel<DT, 0>), g3, b3, lds, s, a); break;             \
   }
+  switch (dtype) {
+    case MCCL_BF16: MCCL_LAUNCH_COMBINE(MCCL_BF16); break;
+    case MCCL_F16: MCCL_LAUNCH_COMBINE(MCCL_F16); break;
+    default: MCCL_LAUNCH_COMBINE(MCCL_F32); break;
+  }
+#undef MCCL_LAUNCH_COMBINE
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "combine kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
