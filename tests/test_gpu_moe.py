@@ -109,7 +109,7 @@ def test_dispatch_then_one_hot_combine_returns_the_tokens(mccl):
     assert torch.equal(y.view(torch.int16), hid[3].view(torch.int16))
 
 
-@pytest.mark.parametrize("topk", [1, 5, 8, 9, 12, 17])
+@pytest.mark.parametrize("topk", [1, 2, 3, 4, 5, 8, 9, 12, 17])
 @pytest.mark.parametrize("hidden", [8, 520, 7168])
 def test_combine_any_topk_with_skipped_entries(mccl, topk, hidden):
     """Random routing tables (any rank, any row) for top-k below, at and above the 8 entries one
