@@ -135,7 +135,7 @@ def test_combine_any_topk_with_skipped_entries(mccl, topk, hidden):
     assert_bits_equal(bits(y), want.view(np.uint16), "combine topk %d hidden %d" % (topk, hidden))
 
 
-@pytest.mark.parametrize("row_bytes", [1, 15, 16, 17, 2047, 2048, 2049, 4099, 14338])
+@pytest.mark.parametrize("row_bytes", [1, 15, 16, 17, 32, 48, 256, 1008, 1024, 1040, 2047, 2048, 2049, 2560, 4099, 6160, 14338])
 @pytest.mark.parametrize("src_off,dst_off", [(0, 0), (1, 0), (0, 3), (5, 9)])
 def test_gather_rows_any_row_size_and_alignment(mccl, row_bytes, src_off, dst_off):
     """Byte rows of every size class (below a vector, around one 2 KiB piece, several pieces with a
@@ -153,3 +153,35 @@ def test_gather_rows_any_row_size_and_alignment(mccl, row_bytes, src_off, dst_of
     want = O.gather_rows(_u8(src), idx.numpy(), row_bytes)
     assert_bits_equal(_u8(dst), want, "gather_rows %d bytes" % row_bytes)
     assert int((dst_buf[:dst_off] != 0xAB).sum()) == 0 and int((dst_buf[dst_off + picks * row_bytes:] != 0xAB).sum()) == 0
+
+
+@pytest.mark.parametrize("row_bytes", [16, 80, 512, 1024, 1536, 2560, 10256])
+def test_gather_small_rows_skip_out_of_range_and_ragged_ends(mccl, row_bytes):
+    """Rows that are not a whole number of 2 KiB pieces travel as 2 KiB windows of the destination
+    (several rows, or parts of two, per wavefront): a byte count that does not fill the last window,
+    indices outside the source (skipped: the destination row keeps its bytes) and the fused dispatch
+    over several segments."""
+    g = torch.Generator().manual_seed(row_bytes)
+    rows, picks = 53, 1001
+    src = torch.randint(0, 255, (rows, row_bytes), generator=g, dtype=torch.uint8)
+    idx = torch.randint(0, rows, (picks,), generator=g, dtype=torch.int64)
+    bad = torch.rand(picks, generator=g) < 0.15
+    idx = torch.where(bad, torch.where(torch.rand(picks, generator=g) < 0.5, torch.full_like(idx, -2), torch.full_like(idx, rows + 7)), idx)
+    out = torch.full((picks, row_bytes), 0xCD, dtype=torch.uint8, device=DEV)
+    mccl.gather_rows(src.to(DEV), idx.to(DEV), out=out)
+    torch.cuda.synchronize()
+    want = torch.full((picks, row_bytes), 0xCD, dtype=torch.uint8)
+    good = ~bad
+    want[good] = src[idx[good]]
+    assert torch.equal(out.cpu(), want)
+    # fused dispatch with small rows: 3 ranks, uneven splits, against gather + alltoallv
+    n = 3
+    S = np.array([[5, 0, 300], [17, 40, 1], [0, 129, 64]])
+    hid = [torch.randint(0, 255, (200, row_bytes), generator=g, dtype=torch.uint8).to(DEV) for _ in range(n)]
+    ix = [torch.randint(0, 200, (int(S[r].sum()),), generator=g, dtype=torch.int64).to(DEV) for r in range(n)]
+    fused = [torch.zeros(int(S[:, d].sum()), row_bytes, dtype=torch.uint8, device=DEV) for d in range(n)]
+    mccl.moe_dispatch_n(hid, ix, fused, S.tolist())
+    torch.cuda.synchronize()
+    want = O.moe_dispatch([_u8(h) for h in hid], [t.cpu().numpy() for t in ix], S, row_bytes)
+    for d in range(n):
+        assert_bits_equal(_u8(fused[d]), want[d], "small-row dispatch dest %d" % d)

@@ -21,6 +21,10 @@ struct GatherArgs {
   int nseg;
   uint32_t row_bytes;
   uint32_t pieces_per_row;  // ceil(row_bytes / kCopyChunk)
+  // 1: rows that are not a whole number of 2 KiB pieces (and are multiples of 16 bytes in 16-byte
+  // aligned buffers): a chunk is a 2 KiB window of the segment's destination, whichever rows it
+  // covers, instead of a piece of one row.  chunks = ceil(nrows * row_bytes / 2 KiB) then.
+  uint32_t flat;
 };
 
 // One wavefront moves one 2 KiB piece of one row.  Chunks are numbered row-major within a
@@ -37,6 +41,36 @@ __global__ __launch_bounds__(kWave) void gather_rows_kernel(const GatherArgs a) 
       if (a.chunk_prefix[mid] <= chunk) lo = mid; else hi = mid;
     }
     const uint32_t lc = chunk - a.chunk_prefix[lo];
+    if (a.flat) {
+      // The destination rows of a segment are one contiguous range, so the wavefront writes 2 KiB
+      // front to back whatever the row length (a 1 KiB row per wavefront would leave half the
+      // lanes idle, a 2.5 KiB row three quarters of every second wavefront); every lane looks up
+      // the source row of its own vectors (a chunk's lanes share a handful of index entries).
+      const uint32_t vpr = row_bytes >> 4;               // vectors per row
+      const uint32_t seg_vecs = a.seg[lo].nrows * vpr;   // the host keeps this below 2^32
+      const u32x4* sbase = (const u32x4*)a.seg[lo].src;
+      u32x4* dvec = (u32x4*)a.seg[lo].dst;
+      u32x4 x[kCopyUnroll];
+      bool ok[kCopyUnroll];
+#pragma unroll
+      for (int u = 0; u < kCopyUnroll; ++u) {
+        const uint32_t v = lc * (uint32_t)(kCopyChunk / 16) + threadIdx.x + (uint32_t)u * kWave;
+        ok[u] = false;
+        if (v < seg_vecs) {
+          const uint32_t r = v / vpr;
+          const int64_t sr = a.seg[lo].idx[r];
+          if (sr >= 0 && sr < (int64_t)a.seg[lo].src_rows) {
+            ok[u] = true;
+            x[u] = sbase[(size_t)sr * vpr + (v - r * vpr)];
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kCopyUnroll; ++u)
+        if (ok[u])
+          __builtin_nontemporal_store(x[u], &dvec[lc * (uint32_t)(kCopyChunk / 16) + threadIdx.x + (uint32_t)u * kWave]);
+      continue;
+    }
     const uint32_t row = lc / ppr;
     const uint32_t piece = lc - row * ppr;
     const int64_t srow = a.seg[lo].idx[row];
