@@ -69,7 +69,7 @@ def scan(asm_path):
             if not t or t.startswith(";"):
                 continue
             if t.startswith(".LBB"):
-                last = None  # SCC may arrive from another block: not judged
+                last = None  # SCC may arrive from another block: left alone
                 continue
             if t.startswith("."):
                 continue
