@@ -106,6 +106,51 @@ def test_pack_and_unpack_reject_a_null_flat_buffer(mccl):
     assert L.mccl_pack(tab, zero, 2, None, None) == 0
 
 
+def test_alignment_and_range_errors_need_no_device(mccl):
+    """Every refusal that depends on addresses, sizes or enum values only."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    err = lambda: L.mccl_last_error().decode()
+    vp = ctypes.c_void_p
+    two = capi.ptr_table([0x10000, 0x20000])
+    # element alignment of inputs and output
+    assert L.mccl_reduce_n(capi.ptr_table([0x10000, 0x20002]), 2, vp(0x30000), 64, capi.F32, capi.SUM, 0, None) == -1
+    assert "input pointer 1 not aligned" in err()
+    assert L.mccl_reduce_n(two, 2, vp(0x30001), 64, capi.BF16, capi.SUM, 0, None) == -1
+    assert "output pointer not aligned" in err()
+    assert L.mccl_reduce_n(two, 2, vp(0x30000), 64, capi.F32, capi.SUM, 9, None) == -1 and "variant" in err()
+    assert L.mccl_reduce_n(capi.ptr_table([0x10000, 0]), 2, vp(0x30000), 64, capi.F32, capi.SUM, 0, None) == -1
+    assert "input pointer 1 is null" in err()
+    # shard and bucket ranges
+    outs = capi.ptr_table([0x30000])
+    assert L.mccl_reduce_scatter_n(two, 2, outs, 16, -1, 1, capi.F32, capi.SUM, None) == -1 and "negative shard" in err()
+    assert L.mccl_reduce_scatter_n(two, 2, outs, 16, 0, 0, capi.F32, capi.SUM, None) == 0  # nothing to do
+    assert L.mccl_reduce_multi(two, 2, outs, (ctypes.c_size_t * 1)(4), -3, capi.F32, capi.SUM, None) == -1
+    # alltoallv: negative splits, rank count
+    splits = (ctypes.c_int64 * 4)(1, -1, 0, 2)
+    assert L.mccl_alltoallv_n(two, two, 2, splits, 16, None) == -1 and "negative split" in err()
+    assert L.mccl_alltoallv_n(two, two, 0, splits, 16, None) == -1 and "rank count" in err()
+    assert L.mccl_allgather_n(two, 65, vp(0x30000), 16, None) == -1
+    # gather: index table alignment, row length, row counts
+    assert L.mccl_gather_rows(vp(0x10000), 10, vp(0x20004), 5, 64, vp(0x30000), None) == -1 and "8-byte aligned" in err()
+    assert L.mccl_gather_rows(vp(0x10000), 10, vp(0x20000), 5, 1 << 31, vp(0x30000), None) == -1 and "too long" in err()
+    assert L.mccl_gather_rows(vp(0x10000), 1 << 32, vp(0x20000), 5, 64, vp(0x30000), None) == -1 and "too many rows" in err()
+    assert L.mccl_gather_rows(None, 10, vp(0x20000), 5, 64, vp(0x30000), None) == -1 and "null pointer" in err()
+    assert L.mccl_gather_rows(None, 10, None, 0, 64, None, None) == 0
+    # combine: dtype, top-k range, row length, alignment of every operand
+    x = capi.ptr_table([0x10000, 0x20000])
+    rows = (ctypes.c_size_t * 2)(8, 8)
+    args = lambda **kw: [kw.get("x", x), rows, 2, vp(kw.get("rank", 0x40000)), vp(kw.get("row", 0x50000)), vp(kw.get("w", 0x60000)),
+                         4, kw.get("topk", 2), kw.get("hidden", 64), kw.get("dtype", capi.BF16), vp(kw.get("y", 0x70000)), None]
+    assert L.mccl_moe_combine(*args(dtype=capi.I32)) == -3 and "bf16, f16 and f32" in err()
+    assert L.mccl_moe_combine(*args(topk=0)) == -1 and L.mccl_moe_combine(*args(topk=65)) == -1 and "topk" in err()
+    assert L.mccl_moe_combine(*args(hidden=63)) == -3 and "multiple of 16 bytes" in err()
+    assert L.mccl_moe_combine(*args(y=0x70008)) == -1 and "output is not 16-byte aligned" in err()
+    assert L.mccl_moe_combine(*args(x=capi.ptr_table([0x10000, 0x20008]))) == -1 and "input 1 is not 16-byte aligned" in err()
+    assert L.mccl_moe_combine(*args(row=0x50004)) == -1 and "misaligned" in err()
+    assert L.mccl_moe_combine(*args(w=0x60002)) == -1 and "misaligned" in err()
+
+
 def test_tensor_front_end_rejects_cpu_tensors(mccl):
     import torch
     with pytest.raises(RuntimeError, match="must be on the GPU"):

@@ -488,6 +488,7 @@ int mccl_reduce_n(const void* const* in, int n, void* out, size_t count, int dty
                   int variant, void* stream) {
   int rc = check_reduce_args(in, n, dtype, op);
   if (rc != MCCL_OK) return rc;
+  if (variant < MCCL_VARIANT_AUTO || variant > MCCL_VARIANT_STREAM) return fail(MCCL_ERR_INVALID_ARG, "unknown variant %d", variant);
   if (count == 0) return MCCL_OK;
   if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer is null");
   ReduceArgs a;
