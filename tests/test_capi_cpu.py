@@ -131,6 +131,9 @@ def test_alignment_and_range_errors_need_no_device(mccl):
     assert L.mccl_alltoallv_n(two, two, 2, splits, 16, None) == -1 and "negative split" in err()
     assert L.mccl_alltoallv_n(two, two, 0, splits, 16, None) == -1 and "rank count" in err()
     assert L.mccl_allgather_n(two, 65, vp(0x30000), 16, None) == -1
+    # copies: a null end of a non-empty segment
+    seg = (capi.Segment * 2)(capi.Segment(0x10000, 0x20000, 16), capi.Segment(0x10000, None, 16))
+    assert L.mccl_copy_segments(seg, 2, None) == -1 and "segment 1 has a null pointer" in err()
     # gather: index table alignment, row length, row counts
     assert L.mccl_gather_rows(vp(0x10000), 10, vp(0x20004), 5, 64, vp(0x30000), None) == -1 and "8-byte aligned" in err()
     assert L.mccl_gather_rows(vp(0x10000), 10, vp(0x20000), 5, 1 << 31, vp(0x30000), None) == -1 and "too long" in err()

@@ -335,6 +335,8 @@ int check_reduce_args_no_ptr(int n, int dtype, int op) {
 }
 
 int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
+  for (int k = 0; k < nseg; ++k)  // refusals first, before anything is enqueued
+    if (segs[k].bytes && (!segs[k].src || !segs[k].dst)) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", k);
   int cus = 0;
   int rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
@@ -347,7 +349,6 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
     while (i < nseg && m < kMaxSegs) {
       const mccl_segment_t& sg = segs[i];
       if (sg.bytes == 0) { ++i; continue; }
-      if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
       const uintptr_t dp = (uintptr_t)sg.dst;
       CopySeg cs;
       cs.src = (const char*)sg.src;
