@@ -142,7 +142,8 @@ def alltoallv_n(inputs, outputs, split_rows):
 
 
 def copy_segments(segments):
-    """segments: iterable of (src_ptr, dst_ptr, nbytes)."""
+    """segments: iterable of (src_ptr, dst_ptr, nbytes); raw device addresses, so the copy runs on the
+    current stream of the current device (the other front ends switch to their tensors' device)."""
     segs = list(segments)
     arr = (capi.Segment * len(segs))(*[capi.Segment(s, d, b) for (s, d, b) in segs])
     capi.check(capi.lib().mccl_copy_segments(arr, len(segs), _stream()))
@@ -154,8 +155,9 @@ def pack(srcs, dst):
     sizes = [t.numel() * t.element_size() for t in srcs]
     if sum(sizes) != dst.numel() * dst.element_size():
         raise RuntimeError("pack: destination size does not match the sources")
-    capi.check(capi.lib().mccl_pack(capi.ptr_table([t.data_ptr() for t in srcs]),
-                                    capi.size_table(sizes), len(srcs), dst.data_ptr(), _stream()))
+    with torch.cuda.device(dst.device):
+        capi.check(capi.lib().mccl_pack(capi.ptr_table([t.data_ptr() for t in srcs]),
+                                        capi.size_table(sizes), len(srcs), dst.data_ptr(), _stream()))
     return dst
 
 
@@ -165,8 +167,9 @@ def unpack(src, dsts):
     sizes = [t.numel() * t.element_size() for t in dsts]
     if sum(sizes) != src.numel() * src.element_size():
         raise RuntimeError("unpack: source size does not match the destinations")
-    capi.check(capi.lib().mccl_unpack(src.data_ptr(), capi.ptr_table([t.data_ptr() for t in dsts]),
-                                      capi.size_table(sizes), len(dsts), _stream()))
+    with torch.cuda.device(src.device):
+        capi.check(capi.lib().mccl_unpack(src.data_ptr(), capi.ptr_table([t.data_ptr() for t in dsts]),
+                                          capi.size_table(sizes), len(dsts), _stream()))
     return dsts
 
 
