@@ -383,6 +383,25 @@ def large_message_case(pg, rank, world):
     assert float(t[0]) == s and float(t[count // 2]) == s and float(t[-2]) == s and float(t[-1]) == 7.0 * s
     assert float(t.min()) == s
     del t
+    # uneven all_to_all_single with inputs beyond one staging window (1200 and 1300 MiB): rows of
+    # 1 MiB tagged with (source rank, row), so every output row names where it came from
+    S = [[300, 900], [1100, 200]]
+    row = 1 << 20
+    def tagged(r, nrows):
+        tag = (torch.arange(nrows, device=DEV) * 7 + r * 97) % 251
+        return tag.to(torch.uint8).view(-1, 1).expand(nrows, row).contiguous()
+    inp = tagged(rank, sum(S[rank]))
+    out = torch.zeros(S[0][rank] + S[1][rank], row, dtype=torch.uint8, device=DEV)
+    pg.alltoall_base(out, inp, [S[0][rank], S[1][rank]], S[rank]).wait()
+    torch.cuda.synchronize()
+    pos = 0
+    for r in range(2):
+        first = sum(S[r][:rank])
+        want = ((torch.arange(first, first + S[r][rank], device=DEV) * 7 + r * 97) % 251).to(torch.uint8)
+        got = out[pos:pos + S[r][rank]]
+        assert torch.equal(got[:, 0], want) and torch.equal(got[:, -1], want) and torch.equal(got[:, row // 2], want), r
+        pos += S[r][rank]
+    del inp, out
     # point to point across the 1 GiB window: two chunks travel as two messages
     count = (1 << 30) + 5
     if rank == 0:

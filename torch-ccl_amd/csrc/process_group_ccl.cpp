@@ -1043,35 +1043,61 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
     }
   }
   const size_t mine = nbytes(input);
-  TORCH_CHECK(mine <= kStageMax, "ccl backend: alltoall message larger than the staging window");
-  Plan p;
-  p.op = c10d::OpType::ALLTOALL_BASE;
-  p.title = "alltoall_base";
-  p.inputs = {input};
-  p.outputs = {output};
-  p.stage_bytes = mine;
-  p.table.resize((size_t)(2 * W));
-  size_t displ = 0;
-  for (int d = 0; d < W; ++d) {  // displacements = exclusive prefix sums of the send counts
-    p.table[(size_t)d] = (int64_t)displ;
-    p.table[(size_t)(W + d)] = (int64_t)send[(size_t)d];
+  std::vector<size_t> send_displ((size_t)W), recv_off((size_t)W);
+  size_t displ = 0, roff = 0;
+  for (int d = 0; d < W; ++d) {  // displacements = exclusive prefix sums of the counts
+    send_displ[(size_t)d] = displ;
+    recv_off[(size_t)d] = roff;
     displ += send[(size_t)d];
+    roff += recv[(size_t)d];
   }
-  if (mine)
-    p.copy_in = [=](void* stage, hipStream_t s) {
-      copyAsync(stage, input.data_ptr(), mine, s);
-    };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
-    std::vector<size_t> sd((size_t)W);
-    for (int r = 0; r < W; ++r) {
-      TORCH_CHECK((size_t)tables[(size_t)r][W + me] == recv[(size_t)r],
-                  "alltoall_base: rank ", r, " sends ", tables[(size_t)r][W + me], " bytes to rank ", me,
-                  " which expects ", recv[(size_t)r]);
-      sd[(size_t)r] = (size_t)tables[(size_t)r][me];
+  // Inputs larger than one staging window travel in windows: window w holds bytes
+  // [w * kStageMax, (w + 1) * kStageMax) of every rank's input, and a rank pulls the part of each
+  // of its segments that lies inside.  How many windows there are depends on the largest input
+  // of the group, which every rank learns from the tables of the first window.
+  auto nwin = std::make_shared<size_t>(1);
+  c10::intrusive_ptr<c10d::Work> work;
+  for (size_t w = 0; w < *nwin; ++w) {
+    const size_t w0 = w * kStageMax;
+    const size_t wlen = w0 < mine ? std::min(mine - w0, kStageMax) : 0;
+    Plan p;
+    p.op = c10d::OpType::ALLTOALL_BASE;
+    p.title = "alltoall_base";
+    p.inputs = {input};
+    p.outputs = {output};
+    p.stage_bytes = wlen;
+    p.table.resize((size_t)(2 * W + 1));
+    for (int d = 0; d < W; ++d) {
+      p.table[(size_t)d] = (int64_t)send_displ[(size_t)d];
+      p.table[(size_t)(W + d)] = (int64_t)send[(size_t)d];
     }
-    MCCL_CHECK(mccl_alltoallv_pull(peer.data(), W, output.data_ptr(), sd.data(), recv.data(), s));
-  };
-  return run(p);
+    p.table[(size_t)(2 * W)] = (int64_t)mine;
+    if (wlen)
+      p.copy_in = [=](void* stage, hipStream_t s) {
+        copyAsync(stage, (const char*)input.data_ptr() + w0, wlen, s);
+      };
+    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+      size_t largest = 0;
+      std::vector<mccl_segment_t> segs;
+      for (int r = 0; r < W; ++r) {
+        const int64_t* tr = tables[(size_t)r];
+        TORCH_CHECK((size_t)tr[W + me] == recv[(size_t)r],
+                    "alltoall_base: rank ", r, " sends ", tr[W + me], " bytes to rank ", me,
+                    " which expects ", recv[(size_t)r]);
+        largest = std::max(largest, (size_t)tr[2 * W]);
+        // the segment addressed to this rank inside rank r's input, cut to the window
+        const size_t seg0 = (size_t)tr[me], seg1 = seg0 + recv[(size_t)r];
+        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w0 + kStageMax);
+        if (lo < hi)
+          segs.push_back({(const char*)peer[(size_t)r] + (lo - w0),
+                          (char*)output.data_ptr() + recv_off[(size_t)r] + (lo - seg0), hi - lo});
+      }
+      *nwin = std::max<size_t>(1, (largest + kStageMax - 1) / kStageMax);
+      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    work = run(p);
+  }
+  return work;
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>& outputs,
