@@ -13,6 +13,9 @@
 // handles, a host barrier and small per-collective tables live in a POSIX shared-memory control
 // block whose name is published through the c10d Store (the role of
 // src/ccl_comm_collector.cpp:10-45 and src/gpu/allreduce.h:1208-1248).
+// A staging buffer is at most 1 GiB (shared allocations stay well below 2 GiB); longer messages
+// travel in windows.  Point-to-point messages use a mailbox per ordered pair of ranks in the same
+// control block (see send / recv below).
 #pragma once
 
 #include <hip/hip_runtime_api.h>
