@@ -206,6 +206,19 @@ def test_staggered_copies_keep_the_data_and_leave_the_power_of_two_spacing(mccl)
     assert torch.equal(out, torch.full_like(out, 6.0))
 
 
+def test_empty_staggered_places_rank_buffers_off_the_regular_spacing(mccl):
+    bufs = mccl.empty_staggered(8, (3, 1 << 18), torch.bfloat16, device=DEV)
+    nbytes = 3 * (1 << 18) * 2
+    assert all(b.shape == (3, 1 << 18) and b.dtype == torch.bfloat16 and b.data_ptr() % 256 == 0 for b in bufs)
+    assert all(bufs[k].data_ptr() - bufs[k - 1].data_ptr() == nbytes + 4096 for k in range(1, 8))
+    for k, b in enumerate(bufs):
+        b.fill_(float(k))
+    out = mccl.reduce_n([b.view(-1) for b in bufs])
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.full_like(out, 28.0))
+    assert all(torch.equal(b, torch.full_like(b, float(k))) for k, b in enumerate(bufs))  # neighbours untouched
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_copy_many_random_segments_in_one_call(mccl, seed):
     """300 segments of random size (0 .. 10 KiB) at random byte offsets in one call: more than one

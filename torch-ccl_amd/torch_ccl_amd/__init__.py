@@ -13,7 +13,7 @@ import torch.distributed as _dist
 from . import capi
 from .capi import (AVG, MAX, MIN, PROD, SUM, VARIANT_AUTO, VARIANT_PERSISTENT,  # noqa: F401
                    VARIANT_SMALL, VARIANT_STREAM)
-from .ops import (allgather_n, alltoallv_n, copy_segments, gather_rows, moe_combine,  # noqa: F401
+from .ops import (allgather_n, alltoallv_n, copy_segments, empty_staggered, gather_rows, moe_combine,  # noqa: F401
                   moe_dispatch_n, pack, reduce_multi, reduce_n, reduce_scatter_n, staggered_copies,
                   unpack)
 

@@ -242,6 +242,24 @@ def moe_combine(x, src_rank, src_row, weights, out=None):
     return out
 
 
+def empty_staggered(n, shape, dtype, device="cuda", stagger_bytes=4096):
+    """n uninitialised tensors of one shape carved from a single allocation, buffer k starting
+    stagger_bytes past the end of buffer k-1 (rounded up to 256 bytes): rank buffers allocated this
+    way never sit at one of the spacings that map element i of every rank to the same DRAM bank
+    (which is where a caching allocator puts equal tensors of 1 GiB and more)."""
+    numel = 1
+    for d in (shape if isinstance(shape, (tuple, list, torch.Size)) else (shape,)):
+        numel *= int(d)
+    nbytes = numel * torch.empty(0, dtype=dtype).element_size()
+    offs, pos = [], 0
+    for k in range(n):
+        pos = (pos + (stagger_bytes if k else 0) + 255) // 256 * 256
+        offs.append(pos)
+        pos += nbytes
+    slab = torch.empty(max(pos, 1), dtype=torch.uint8, device=device)
+    return [slab[off:off + nbytes].view(dtype).view(shape) for off in offs]
+
+
 def staggered_copies(tensors, stagger_bytes=4096):
     """Copies of `tensors` carved from one allocation so that buffer k starts k * stagger_bytes past
     the end of buffer k-1 (rounded up to 256 bytes).  Rank buffers that sit an exact power of two
