@@ -402,6 +402,16 @@ def large_message_case(pg, rank, world):
         assert torch.equal(got[:, 0], want) and torch.equal(got[:, -1], want) and torch.equal(got[:, row // 2], want), r
         pos += S[r][rank]
     del inp, out
+    # coalesced forms whose staging image would exceed one window fall back to one collective per tensor
+    ts = [torch.full((160 << 20,), float(rank + 1 + i), device=DEV) for i in range(2)]  # 2 x 640 MiB
+    o = c10d.AllreduceCoalescedOptions()
+    o.reduceOp = c10d.ReduceOp.SUM
+    pg.allreduce_coalesced(ts, o).wait()
+    torch.cuda.synchronize()
+    for i, t in enumerate(ts):
+        want = sum(r + 1 + i for r in range(world))
+        assert float(t[0]) == want and float(t[-1]) == want and float(t.min()) == want == float(t.max())
+    del ts
     # point to point across the 1 GiB window: two chunks travel as two messages
     count = (1 << 30) + 5
     if rank == 0:
@@ -586,6 +596,36 @@ def identity_replay_case(rank, world):
     dist.barrier()
 
 
+def coalesced_window_cases(rank, world):
+    """Coalesced forms on the default group whose staging image exceeds the (shrunk) window: they
+    fall back to one windowed collective per tensor and must give the same results."""
+    pg = c10d._get_default_group()
+    n = 50_000  # 200 KB of fp32 per tensor: several 64 KiB windows each
+    ts = [torch.full((n + i,), float(rank + 1 + i), device=DEV) for i in range(3)]
+    o = c10d.AllreduceCoalescedOptions()
+    o.reduceOp = c10d.ReduceOp.SUM
+    pg.allreduce_coalesced(ts, o).wait()
+    torch.cuda.synchronize()
+    for i, t in enumerate(ts):
+        want = float(sum(r + 1 + i for r in range(world)))
+        assert float(t.min()) == want == float(t.max()), ("allreduce_coalesced", i)
+    ins = [torch.full((world * (n + i),), float(rank + 1), device=DEV) for i in range(2)]
+    outs = [torch.empty(n + i, device=DEV) for i in range(2)]
+    pg.reduce_scatter_tensor_coalesced(outs, ins, c10d.ReduceScatterOptions()).wait()
+    torch.cuda.synchronize()
+    for t in outs:
+        assert float(t.min()) == world * (world + 1) / 2.0 == float(t.max())
+    gin = [torch.full((n + i,), float(rank * 10 + i), device=DEV) for i in range(2)]
+    gout = [torch.empty(world * (n + i), device=DEV) for i in range(2)]
+    pg.allgather_into_tensor_coalesced(gout, gin).wait()
+    torch.cuda.synchronize()
+    for i, t in enumerate(gout):
+        got = t.view(world, n + i)
+        for r in range(world):
+            assert float(got[r].min()) == float(r * 10 + i) == float(got[r].max())
+    dist.barrier()
+
+
 def subgroup_case(rank, world):
     """Subgroups as the reference's tests/ds_subgroup_allreduce.py builds them: a one-rank group, then
     strided groups of `sub` ranks; plus a rooted op and a send / recv addressed by global rank inside
@@ -628,11 +668,12 @@ def run_rank(rank, world, store_path, mode):
         finally:
             dist.destroy_process_group()
         return
-    if mode in ("subgroup", "replay", "reference_p2p"):
+    if mode in ("subgroup", "replay", "reference_p2p", "coalesced_windows"):
         store = dist.FileStore(store_path, world)
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
-            {"subgroup": subgroup_case, "replay": identity_replay_case, "reference_p2p": reference_p2p_cases}[mode](rank, world)
+            {"subgroup": subgroup_case, "replay": identity_replay_case, "reference_p2p": reference_p2p_cases,
+             "coalesced_windows": coalesced_window_cases}[mode](rank, world)
         finally:
             dist.destroy_process_group()
         return

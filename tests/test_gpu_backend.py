@@ -51,6 +51,17 @@ def test_reference_send_recv_cases():
     _spawn(6, "reference_p2p")
 
 
+@pytest.mark.parametrize("window,world,mode", [("65536", 2, "oracle"), ("65536", 4, "oracle"), ("4096", 3, "p2p"),
+                                               ("65536", 2, "reference"), ("65536", 4, "dist"),
+                                               ("65536", 4, "coalesced_windows"), ("6291456", 8, "oracle")])
+def test_every_windowed_path_with_a_shrunk_window(monkeypatch, window, world, mode):
+    """MCCL_STAGE_WINDOW_BYTES shrinks the staging window, so that messages of a few hundred KiB travel
+    in many windows: the same case sets as above must give the same bits.  The 6 MiB window with 8
+    ranks puts the two-shot allreduce and a second, shorter window into one message."""
+    monkeypatch.setenv("MCCL_STAGE_WINDOW_BYTES", window)
+    _spawn(world, mode)
+
+
 def test_message_larger_than_one_staging_window():
     _spawn(2, "large")
 

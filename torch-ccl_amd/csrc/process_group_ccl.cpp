@@ -29,7 +29,7 @@ namespace {
 constexpr int kMaxWorld = MCCL_MAX_RANKS;
 constexpr int kTableMax = 2 * kMaxWorld + 8;
 constexpr size_t kStageMin = 2u << 20;   // first staging allocation
-constexpr size_t kStageMax = 1u << 30;   // one staging window; keeps every IPC allocation < 2 GiB
+constexpr size_t kStageMaxDefault = 1u << 30;  // one staging window; keeps every IPC allocation < 2 GiB
 // Rank r's staging buffer starts (r mod 16) x 4 KiB into its allocation.  Equal-sized allocations
 // tend to sit a power of two apart, and rank buffers at such a spacing make every wavefront of the
 // reduction hit the same DRAM banks with all its loads (6-20 % of bandwidth on large messages).
@@ -251,6 +251,13 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   blocking_wait_ = envFlag("CCL_BLOCKING_WAIT", false);
   verbose_ = envFlag("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", false);
   profile_ = envFlag("MCCL_PG_PROFILE", false);
+  // The staging window can be shrunk (never enlarged) so that tests reach every windowed path
+  // with small tensors.
+  stage_max_ = kStageMaxDefault;
+  if (const char* v = std::getenv("MCCL_STAGE_WINDOW_BYTES")) {
+    const long long b = std::atoll(v);
+    if (b >= 4096 && (size_t)b < kStageMaxDefault) stage_max_ = (size_t)b & ~(size_t)4095;
+  }
 }
 
 c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_ptr<c10d::Store>& store,
@@ -370,7 +377,7 @@ void ProcessGroupCCL::ensureInit(int device) {
   p2p_send_.assign((size_t)size_, P2PSend{});
   p2p_recv_.assign((size_t)size_, P2PRecv{});
   initialised_ = true;
-  for (int s = 0; s < 2; ++s) ensureStage(s, kStageMin);
+  for (int s = 0; s < 2; ++s) ensureStage(s, std::min(kStageMin, stage_max_));
 
   hostBarrier(/*start_up=*/true);
   TORCH_CHECK(ctl_->magic == kMagic && ctl_->world == (uint32_t)size_,
@@ -381,7 +388,7 @@ void ProcessGroupCCL::ensureInit(int device) {
 void* ProcessGroupCCL::ensureStage(int slot, size_t bytes) {
   Stage& st = stage_[slot];
   if (bytes <= st.capacity) return st.ptr;
-  TORCH_CHECK(bytes <= kStageMax, "ccl backend: staging request of ", bytes, " bytes exceeds the window");
+  TORCH_CHECK(bytes <= stage_max_, "ccl backend: staging request of ", bytes, " bytes exceeds the window");
   size_t cap = kStageMin;
   while (cap < bytes) cap <<= 1;
   void* base = nullptr;
@@ -596,7 +603,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
-    const size_t len = std::min(total - off, kStageMax);
+    const size_t len = std::min(total - off, stage_max_);
     char* base = total ? (char*)t.data_ptr() + off : nullptr;
     Plan p;
     p.op = c10d::OpType::BROADCAST;
@@ -630,7 +637,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
   const size_t es = t.element_size();
   const size_t total = (size_t)t.numel();
   // one staging window holds the input; the two-shot form reduces each shard in place there
-  const size_t chunk = kStageMax / es;
+  const size_t chunk = stage_max_ / es;
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
@@ -706,7 +713,18 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce_coalesced(
     offs[i] = total;
     total += roundUp(nbytes(tensors[i]), 16);
   }
-  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced allreduce larger than the staging window");
+  if (total > stage_max_) {
+    // more than one staging window: one (windowed) allreduce per tensor; same results, same order
+    // on every rank (the shapes of a coalesced call agree across ranks)
+    c10::intrusive_ptr<c10d::Work> last;
+    c10d::AllreduceOptions one;
+    one.reduceOp = opts.reduceOp;
+    for (auto& t : tensors) {
+      std::vector<at::Tensor> v{t};
+      last = allreduce(v, one);
+    }
+    return last;
+  }
   Plan p;
   p.op = c10d::OpType::ALLREDUCE_COALESCED;
   p.title = "allreduce_coalesced";
@@ -748,7 +766,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
-    const size_t len = std::min(per_rank - off, kStageMax);
+    const size_t len = std::min(per_rank - off, stage_max_);
     char* in = per_rank ? (char*)input.data_ptr() + off : nullptr;
     char* out = per_rank ? (char*)output.data_ptr() + off : nullptr;
     Plan p;
@@ -787,7 +805,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   at::Tensor input = inputs[0];
   std::vector<at::Tensor> outs = outputs[0];
   const size_t mine = nbytes(input);
-  TORCH_CHECK(mine <= kStageMax, "ccl backend: allgather (list) message larger than the staging window");
+  TORCH_CHECK(mine <= stage_max_, "ccl backend: allgather (list) message larger than the staging window");
   Plan p;
   p.op = c10d::OpType::ALLGATHER;
   p.title = "allgather";
@@ -832,7 +850,11 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather_into_tensor_coalesced(
     offs[i] = total;
     total += roundUp(nbytes(inputs[i]), 16);
   }
-  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced allgather larger than the staging window");
+  if (total > stage_max_) {  // more than one staging window: one (windowed) all-gather per tensor
+    c10::intrusive_ptr<c10d::Work> last;
+    for (size_t i = 0; i < inputs.size(); ++i) last = _allgather_base(outputs[i], inputs[i], c10d::AllgatherOptions());
+    return last;
+  }
   Plan p;
   p.op = c10d::OpType::ALLGATHER_COALESCED;
   p.title = "allgather_into_tensor_coalesced";
@@ -872,7 +894,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
   const size_t M = (size_t)output.numel();
   const int W = size_;
   // one window holds the same sub-range [m0, m0+len) of all W shards, back to back
-  const size_t chunk = std::max<size_t>(1, kStageMax / es / (size_t)W);
+  const size_t chunk = std::max<size_t>(1, stage_max_ / es / (size_t)W);
   c10::intrusive_ptr<c10d::Work> work;
   size_t m0 = 0;
   do {
@@ -941,7 +963,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
     p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
     total += roundUp(nbytes(ins[(size_t)d]), 16);
   }
-  TORCH_CHECK(total <= kStageMax, "ccl backend: reduce_scatter (list) larger than the staging window");
+  TORCH_CHECK(total <= stage_max_, "ccl backend: reduce_scatter (list) larger than the staging window");
   p.stage_bytes = total;
   p.copy_in = [=](void* stage, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
@@ -980,7 +1002,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter_tensor_coalesced(
     offs[i] = total;
     total += roundUp(nbytes(inputs[i]), 16);
   }
-  TORCH_CHECK(total <= kStageMax, "ccl backend: coalesced reduce_scatter larger than the staging window");
+  if (total > stage_max_) {  // more than one staging window: one (windowed) reduce-scatter per tensor
+    c10::intrusive_ptr<c10d::Work> last;
+    c10d::ReduceScatterOptions one;
+    one.reduceOp = opts.reduceOp;
+    for (size_t i = 0; i < inputs.size(); ++i) last = _reduce_scatter_base(outputs[i], inputs[i], one);
+    return last;
+  }
   Plan p;
   p.op = c10d::OpType::COALESCED;
   p.title = "reduce_scatter_tensor_coalesced";
@@ -1052,14 +1080,15 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
     roff += recv[(size_t)d];
   }
   // Inputs larger than one staging window travel in windows: window w holds bytes
-  // [w * kStageMax, (w + 1) * kStageMax) of every rank's input, and a rank pulls the part of each
+  // [w * window, (w + 1) * window) of every rank's input, and a rank pulls the part of each
   // of its segments that lies inside.  How many windows there are depends on the largest input
   // of the group, which every rank learns from the tables of the first window.
   auto nwin = std::make_shared<size_t>(1);
+  const size_t window = stage_max_;
   c10::intrusive_ptr<c10d::Work> work;
   for (size_t w = 0; w < *nwin; ++w) {
-    const size_t w0 = w * kStageMax;
-    const size_t wlen = w0 < mine ? std::min(mine - w0, kStageMax) : 0;
+    const size_t w0 = w * window;
+    const size_t wlen = w0 < mine ? std::min(mine - w0, window) : 0;
     Plan p;
     p.op = c10d::OpType::ALLTOALL_BASE;
     p.title = "alltoall_base";
@@ -1087,12 +1116,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
         largest = std::max(largest, (size_t)tr[2 * W]);
         // the segment addressed to this rank inside rank r's input, cut to the window
         const size_t seg0 = (size_t)tr[me], seg1 = seg0 + recv[(size_t)r];
-        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w0 + kStageMax);
+        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w0 + window);
         if (lo < hi)
           segs.push_back({(const char*)peer[(size_t)r] + (lo - w0),
                           (char*)output.data_ptr() + recv_off[(size_t)r] + (lo - seg0), hi - lo});
       }
-      *nwin = std::max<size_t>(1, (largest + kStageMax - 1) / kStageMax);
+      *nwin = std::max<size_t>(1, (largest + window - 1) / window);
       if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
     };
     work = run(p);
@@ -1128,7 +1157,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>
     p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
     total += roundUp(nbytes(ins[(size_t)d]), 16);
   }
-  TORCH_CHECK(total <= kStageMax, "ccl backend: alltoall (list) larger than the staging window");
+  TORCH_CHECK(total <= stage_max_, "ccl backend: alltoall (list) larger than the staging window");
   p.stage_bytes = total;
   p.copy_in = [=](void* stage, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
@@ -1174,7 +1203,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce(std::vector<at::Tensor>& 
   const int root = (int)opts.rootRank;
   const size_t es = t.element_size();
   const size_t total = (size_t)t.numel();
-  const size_t chunk = kStageMax / es;
+  const size_t chunk = stage_max_ / es;
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
@@ -1225,7 +1254,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<a
   }
   at::Tensor input = inputs[0];
   const size_t mine = nbytes(input);
-  TORCH_CHECK(mine <= kStageMax, "ccl backend: gather message larger than the staging window");
+  TORCH_CHECK(mine <= stage_max_, "ccl backend: gather message larger than the staging window");
   Plan p;
   p.op = c10d::OpType::GATHER;
   p.title = "gather";
@@ -1296,7 +1325,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
       p.table[(size_t)(W + r)] = (int64_t)nbytes(ins[(size_t)r]);
       if (r != root) total += roundUp(nbytes(ins[(size_t)r]), 16);  // the root's own piece is not staged
     }
-    TORCH_CHECK(total <= kStageMax, "ccl backend: scatter larger than the staging window");
+    TORCH_CHECK(total <= stage_max_, "ccl backend: scatter larger than the staging window");
     TORCH_CHECK(nbytes(ins[(size_t)root]) == nbytes(out), "scatter: output tensor does not match the size the root sends");
     p.stage_bytes = total;
     p.copy_in = [=](void* stage, hipStream_t s) {
@@ -1322,7 +1351,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
 // point to point
 // ---------------------------------------------------------------------------------------------
 void ProcessGroupCCL::spinUntil(const std::function<bool()>& ready, int peer, const char* what,
-                                const std::function<bool()>& abandoned) {
+                                const std::function<bool()>& abandoned, const std::function<void()>& idle) {
   std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(30000));
   if (const char* v = std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
     const long ms = std::atol(v);
@@ -1337,6 +1366,7 @@ void ProcessGroupCCL::spinUntil(const std::function<bool()>& ready, int peer, co
       ctl_->slot[rank_].failed.store(1, std::memory_order_release);
       TORCH_CHECK(false, "ccl backend: rank ", peer, " left the group while this rank was waiting for ", what);
     }
+    if (idle) idle();
     if (++spins < 2000) continue;
     sched_yield();
     if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
@@ -1361,10 +1391,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::send(std::vector<at::Tensor>& te
   const size_t total = nbytes(t);
   size_t off = 0;
   do {  // an empty tensor still travels as one (empty) message, so that sends and receives pair up
-    const size_t len = std::min(total - off, kStageMax);
+    const size_t len = std::min(total - off, stage_max_);
     const uint64_t k = box.posted.load(std::memory_order_relaxed) + 1;
     spinUntil([&] { return k - box.consumed.load(std::memory_order_acquire) <= (uint64_t)kRing; }, dstRank,
-              "a free send buffer", [] { return true; });
+              "a free send buffer", [] { return true; },
+              [&] {  // while waiting, take in what others have sent to this rank's posted receives
+                for (int src = 0; src < size_; ++src)
+                  if (!p2p_recv_[(size_t)src].pending.empty()) progressRecvLocked(src, nullptr, /*blocking=*/false);
+              });
     const int slot = (int)((k - 1) % kRing);
     P2PEntry& e = box.ring[slot];
     if (len > mine.capacity[slot]) {
@@ -1407,8 +1441,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>& te
     ensureInit(state->tensor.get_device());
     P2PRecv& pr = p2p_recv_[(size_t)srcRank];
     const size_t total = nbytes(state->tensor);
-    const uint64_t nmsg = total ? (total + kStageMax - 1) / kStageMax : 1;
-    state->first_seq = pr.assigned + 1;
+    const uint64_t nmsg = total ? (total + stage_max_ - 1) / stage_max_ : 1;
+    state->next_seq = pr.assigned + 1;
     pr.assigned += nmsg;
     pr.pending.push_back(state);
   }
@@ -1418,7 +1452,11 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>& te
 
 void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocking) {
   std::lock_guard<std::mutex> lock(mutex_);
-  if (target->done) return;
+  progressRecvLocked(src, target, blocking);
+}
+
+void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool blocking) {
+  if (target && target->done) return;
   c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
   hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_).stream();
   P2PBox& box = ctl_->slot[src].p2p[rank_];
@@ -1426,13 +1464,15 @@ void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocki
   while (!pr.pending.empty()) {
     std::shared_ptr<RecvState> st = pr.pending.front();
     const size_t total = nbytes(st->tensor);
-    size_t off = 0;
-    uint64_t k = st->first_seq;
-    if (!blocking && box.posted.load(std::memory_order_acquire) < k + (total ? (total - 1) / kStageMax : 0)) return;
-    do {
-      const size_t len = std::min(total - off, kStageMax);
-      spinUntil([&] { return box.posted.load(std::memory_order_acquire) >= k; }, src, "a message",
-                [&] { return box.posted.load(std::memory_order_acquire) < k; });
+    // message by message; what has arrived is kept when a non-blocking call has to stop half way
+    for (bool finished = false; !finished;) {
+      const uint64_t k = st->next_seq;
+      if (box.posted.load(std::memory_order_acquire) < k) {
+        if (!blocking) return;
+        spinUntil([&] { return box.posted.load(std::memory_order_acquire) >= k; }, src, "a message",
+                  [&] { return box.posted.load(std::memory_order_acquire) < k; });
+      }
+      const size_t len = std::min(total - st->off, stage_max_);
       const int slot = (int)((k - 1) % kRing);
       const P2PEntry& e = box.ring[slot];
       if (e.bytes != len) {
@@ -1464,13 +1504,14 @@ void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocki
         }
         TORCH_CHECK(!ctl_->slot[src].failed.load(std::memory_order_acquire),
                     "ccl backend: rank ", src, " gave up on a message before it was received");
-        copyAsync((char*)st->tensor.data_ptr() + off, from, len, cur);
+        copyAsync((char*)st->tensor.data_ptr() + st->off, from, len, cur);
         HIP_CHECK(hipStreamSynchronize(cur));  // the sender may reuse the buffer once `consumed` moves
       }
       box.consumed.store(k, std::memory_order_release);
-      ++k;
-      off += len;
-    } while (off < total);
+      st->next_seq = k + 1;
+      st->off += len;
+      finished = st->off >= total;
+    }
     st->done = true;
     pr.pending.pop_front();
     if (st.get() == target) return;

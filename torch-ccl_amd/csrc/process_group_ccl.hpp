@@ -68,7 +68,8 @@ class ProcessGroupCCL : public c10d::Backend {
   struct RecvState {
     at::Tensor tensor;
     int src = 0;
-    uint64_t first_seq = 0;  // sequence number (from 1) of the first message of this receive
+    uint64_t next_seq = 0;  // sequence number (from 1) of the next message of this receive
+    size_t off = 0;         // bytes of the tensor already filled (a long tensor travels as several messages)
     bool done = false;
   };
 
@@ -189,11 +190,16 @@ class ProcessGroupCCL : public c10d::Backend {
   void checkDeviceTensors(const std::vector<at::Tensor>& tensors) const;
   // Spins (then yields) until ready() holds; raises when `peer` reports a failure, when it has
   // left and abandoned() says that what is awaited can no longer come, or at the time limit.
+  // `idle`, when given, runs between polls (a send that waits for a free buffer uses it to
+  // complete this rank's own posted receives, so that ranks sending round a ring cannot block
+  // each other for good).
   void spinUntil(const std::function<bool()>& ready, int peer, const char* what,
-                 const std::function<bool()>& abandoned);
-  // Completes the receives posted for `src` in order, up to and including `target`.  With
-  // blocking == false it stops at the first message the sender has not published yet.
+                 const std::function<bool()>& abandoned, const std::function<void()>& idle = nullptr);
+  // Completes the receives posted for `src` in order, up to and including `target` (all of them
+  // when target is null).  With blocking == false it stops at the first message the sender has
+  // not published yet.  progressRecv takes the group's mutex, the Locked form expects it held.
   void progressRecv(int src, const RecvState* target, bool blocking);
+  void progressRecvLocked(int src, const RecvState* target, bool blocking);
 
   c10::intrusive_ptr<c10d::Store> store_;
   std::chrono::milliseconds timeout_;
@@ -201,6 +207,7 @@ class ProcessGroupCCL : public c10d::Backend {
   bool same_stream_ = false;    // CCL_SAME_STREAM
   bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
   bool profile_ = false;        // MCCL_PG_PROFILE: host-side phase timers, printed when the group dies
+  size_t stage_max_ = 0;        // bytes of one staging window (1 GiB; MCCL_STAGE_WINDOW_BYTES shrinks it for tests)
   // per collective with a payload: copy-in enqueue, stream synchronise, host barrier, kernel enqueue
   std::vector<float> phase_us_[4];
   bool coalescing_ = false;
