@@ -360,6 +360,21 @@ def p2p_cases(pg, rank, world):
         pg.send([payload(rank, prv, 40 + i, count).to(DEV)], prv, 0).wait()
         w.wait()
         assert np.array_equal(bits(got), bits(payload(nxt, rank, 40 + i, count))), ("grow", count)
+    # a receive posted before a collective, waited for after it: the sender may need more buffers
+    # than it has before it can join the collective, so the receiver has to take messages in
+    # while it waits in the collective's barrier
+    count = 300000
+    if rank == 0:
+        got = torch.zeros(count, dtype=torch.uint8, device=DEV)
+        w = pg.recv([got], 1, 0)
+    elif rank == 1:
+        pg.send([payload(1, 0, 60, count).to(DEV)], 0, 0).wait()
+    t = torch.ones(8, device=DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    assert t.cpu().tolist() == [float(world)] * 8
+    if rank == 0:
+        w.wait()
+        assert np.array_equal(bits(got), bits(payload(1, 0, 60, count))), "receive across a collective"
     # polling: is_completed turns true once the sender has published, without a wait
     got = torch.zeros(5, dtype=torch.uint8, device=DEV)
     w = pg.recv([got], prv, 0)

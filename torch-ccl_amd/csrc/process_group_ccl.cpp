@@ -450,6 +450,11 @@ void ProcessGroupCCL::hostBarrier(bool start_up) {
         TORCH_CHECK(false, "ccl backend: rank ", r, " left the group before collective #", seq_);
       }
       if (++spins < 2000) continue;
+      // A peer may be late because it is still sending to this rank and has run out of send
+      // buffers: take in what has arrived for the receives this rank has posted.
+      if (!start_up)
+        for (int src = 0; src < size_; ++src)
+          if (!p2p_recv_[(size_t)src].pending.empty()) progressRecvLocked(src, nullptr, /*blocking=*/false);
       sched_yield();
       if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
         ctl_->slot[rank_].failed.store(1, std::memory_order_release);
