@@ -375,6 +375,25 @@ def p2p_cases(pg, rank, world):
     if rank == 0:
         w.wait()
         assert np.array_equal(bits(got), bits(payload(1, 0, 60, count))), "receive across a collective"
+    # three ranks: 0 posts a receive from 2 and then blocks on one from 1; 2 sends 0 a long tensor
+    # before it sends 1 what 1 needs to send 0 its message - 0 must take 2's messages in while it
+    # waits for 1
+    if world >= 3:
+        count = 200000
+        if rank == 0:
+            a = torch.zeros(count, dtype=torch.uint8, device=DEV)
+            b = torch.zeros(16, dtype=torch.uint8, device=DEV)
+            wa = pg.recv([a], 2, 0)
+            pg.recv([b], 1, 0).wait()
+            wa.wait()
+            assert np.array_equal(bits(a), bits(payload(2, 0, 70, count))) and np.array_equal(bits(b), bits(payload(2, 1, 71, 16)))
+        elif rank == 1:
+            b = torch.zeros(16, dtype=torch.uint8, device=DEV)
+            pg.recv([b], 2, 0).wait()
+            pg.send([b], 0, 0).wait()
+        elif rank == 2:
+            pg.send([payload(2, 0, 70, count).to(DEV)], 0, 0).wait()
+            pg.send([payload(2, 1, 71, 16).to(DEV)], 1, 0).wait()
     # polling: is_completed turns true once the sender has published, without a wait
     got = torch.zeros(5, dtype=torch.uint8, device=DEV)
     w = pg.recv([got], prv, 0)

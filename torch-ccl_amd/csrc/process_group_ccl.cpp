@@ -1475,7 +1475,12 @@ void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool 
       if (box.posted.load(std::memory_order_acquire) < k) {
         if (!blocking) return;
         spinUntil([&] { return box.posted.load(std::memory_order_acquire) >= k; }, src, "a message",
-                  [&] { return box.posted.load(std::memory_order_acquire) < k; });
+                  [&] { return box.posted.load(std::memory_order_acquire) < k; },
+                  [&] {  // meanwhile, whatever other ranks have sent to receives posted here
+                    for (int other = 0; other < size_; ++other)
+                      if (other != src && !p2p_recv_[(size_t)other].pending.empty())
+                        progressRecvLocked(other, nullptr, /*blocking=*/false);
+                  });
       }
       const size_t len = std::min(total - st->off, stage_max_);
       const int slot = (int)((k - 1) % kRing);
