@@ -406,6 +406,48 @@ def p2p_cases(pg, rank, world):
     pg.barrier().wait()
 
 
+def list_window_cases(pg, rank, world):
+    """List and rooted forms whose staging image exceeds the (shrunk) window: they fall back to
+    windowed broadcasts, rooted reduces or point-to-point messages and must give the same results."""
+    n = 3001  # 12 KB of fp32: three windows of 4 KiB
+    val = lambda r, i=0: float(r * 3 + i + 1)
+    # allgather (list)
+    outs = [torch.zeros(n, device=DEV) for _ in range(world)]
+    pg.allgather([outs], [torch.full((n,), val(rank), device=DEV)]).wait()
+    torch.cuda.synchronize()
+    for r in range(world):
+        assert float(outs[r].min()) == val(r) == float(outs[r].max()), ("allgather", r)
+    # reduce_scatter (list): slot d of every rank's list is summed into rank d's output
+    ins = [torch.full((n,), val(rank, d), device=DEV) for d in range(world)]
+    keep = [t.clone() for t in ins]
+    out = torch.zeros(n, device=DEV)
+    o = c10d.ReduceScatterOptions()
+    o.reduceOp = c10d.ReduceOp.SUM
+    pg.reduce_scatter([out], [ins], o).wait()
+    torch.cuda.synchronize()
+    want = sum(val(r, rank) for r in range(world))
+    assert float(out.min()) == want == float(out.max()), "reduce_scatter"
+    assert all(torch.equal(a, b) for a, b in zip(ins, keep)), "reduce_scatter must not touch its inputs"
+    # gather and scatter, every rank root in turn
+    for root in range(world):
+        go = c10d.GatherOptions()
+        go.rootRank = root
+        got = [torch.zeros(n, device=DEV) for _ in range(world)]
+        pg.gather([got] if rank == root else [], [torch.full((n,), val(rank, root), device=DEV)], go).wait()
+        torch.cuda.synchronize()
+        if rank == root:
+            for r in range(world):
+                assert float(got[r].min()) == val(r, root) == float(got[r].max()), ("gather", root, r)
+        so = c10d.ScatterOptions()
+        so.rootRank = root
+        piece = torch.zeros(n, device=DEV)
+        src = [[torch.full((n,), val(r, root) + 0.5, device=DEV) for r in range(world)]] if rank == root else []
+        pg.scatter([piece], src, so).wait()
+        torch.cuda.synchronize()
+        assert float(piece.min()) == val(rank, root) + 0.5 == float(piece.max()), ("scatter", root)
+    pg.barrier().wait()
+
+
 def large_message_case(pg, rank, world):
     """A message larger than one staging window (1 GiB) is cut into windows."""
     count = (1 << 28) + 12345  # 1 GiB + a bit of fp32
@@ -728,6 +770,8 @@ def run_rank(rank, world, store_path, mode):
         oracle_cases(pg, rank, world)
     elif mode == "p2p":
         p2p_cases(pg, rank, world)
+    elif mode == "list_windows":
+        list_window_cases(pg, rank, world)
     elif mode == "large":
         large_message_case(pg, rank, world)
     elif mode == "env":

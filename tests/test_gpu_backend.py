@@ -55,7 +55,9 @@ def test_reference_send_recv_cases():
                                                ("65536", 2, "reference"), ("65536", 4, "dist"),
                                                ("65536", 4, "coalesced_windows"), ("6291456", 8, "oracle"),
                                                ("8192", 2, "ddp"), ("4096", 6, "reference_p2p"), ("65536", 4, "subgroup"),
-                                               ("65536", 2, "replay"), ("4096", 8, "p2p")])
+                                               ("65536", 2, "replay"), ("4096", 8, "p2p"),
+                                               ("4096", 3, "list_windows"), ("4096", 8, "list_windows"),
+                                               ("1073741824", 4, "list_windows")])
 def test_every_windowed_path_with_a_shrunk_window(monkeypatch, window, world, mode):
     """MCCL_STAGE_WINDOW_BYTES shrinks the staging window, so that messages of a few hundred KiB travel
     in many windows: the same case sets as above must give the same bits.  The 6 MiB window with 8

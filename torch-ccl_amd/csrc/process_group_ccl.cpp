@@ -810,7 +810,28 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   at::Tensor input = inputs[0];
   std::vector<at::Tensor> outs = outputs[0];
   const size_t mine = nbytes(input);
-  TORCH_CHECK(mine <= stage_max_, "ccl backend: allgather (list) message larger than the staging window");
+  size_t largest = mine;
+  for (const auto& o : outs) largest = std::max(largest, nbytes(o));  // what each rank sends: known everywhere
+  if (largest > stage_max_) {
+    // more than one staging window: one (windowed) broadcast per rank, straight into outs[r]
+    c10::intrusive_ptr<c10d::Work> last;
+    for (int r = 0; r < size_; ++r) {
+      c10d::BroadcastOptions bo;
+      bo.rootRank = r;
+      bo.rootTensor = 0;
+      if (r == rank_) {
+        TORCH_CHECK(mine == nbytes(outs[(size_t)r]), "allgather: output tensor ", r, " does not match the size rank ", r, " sends");
+        std::vector<at::Tensor> v{input};
+        last = broadcast(v, bo);
+        hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(input.get_device()).stream();
+        copyAsync(outs[(size_t)r].data_ptr(), input.data_ptr(), mine, cur);
+      } else {
+        std::vector<at::Tensor> v{outs[(size_t)r]};
+        last = broadcast(v, bo);
+      }
+    }
+    return last;
+  }
   Plan p;
   p.op = c10d::OpType::ALLGATHER;
   p.title = "allgather";
@@ -968,7 +989,28 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
     p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
     total += roundUp(nbytes(ins[(size_t)d]), 16);
   }
-  TORCH_CHECK(total <= stage_max_, "ccl backend: reduce_scatter (list) larger than the staging window");
+  if (total > stage_max_) {
+    // more than one staging window: W (windowed) rooted reduces, as the reference does for slots of
+    // unequal size.  The root reduces in place in its output, which first takes its own slot.
+    c10::intrusive_ptr<c10d::Work> last;
+    for (int d = 0; d < W; ++d) {
+      c10d::ReduceOptions ro;
+      ro.reduceOp = opts.reduceOp;
+      ro.rootRank = d;
+      ro.rootTensor = 0;
+      if (d == me) {
+        TORCH_CHECK(nbytes(out) == nbytes(ins[(size_t)d]), "reduce_scatter: output tensor does not match slot ", d);
+        hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(out.get_device()).stream();
+        copyAsync(out.data_ptr(), ins[(size_t)d].data_ptr(), nbytes(out), cur);
+        std::vector<at::Tensor> v{out};
+        last = reduce(v, ro);
+      } else {
+        std::vector<at::Tensor> v{ins[(size_t)d]};  // only staged: a non-root tensor keeps its values
+        last = reduce(v, ro);
+      }
+    }
+    return last;
+  }
   p.stage_bytes = total;
   p.copy_in = [=](void* stage, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
@@ -1259,7 +1301,22 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<a
   }
   at::Tensor input = inputs[0];
   const size_t mine = nbytes(input);
-  TORCH_CHECK(mine <= stage_max_, "ccl backend: gather message larger than the staging window");
+  if (mine > stage_max_) {
+    // more than one staging window: point to point (every rank sends the same number of bytes,
+    // src/gpu/dpcpp_ccl.cpp:1270-1289)
+    if (rank_ != root) return send(inputs, root, 0);
+    std::vector<c10::intrusive_ptr<c10d::Work>> pending;
+    for (int r = 0; r < size_; ++r) {
+      TORCH_CHECK(nbytes(outs[(size_t)r]) == mine, "gather: output tensor ", r, " does not match the size rank ", r, " sends");
+      if (r == root) continue;
+      std::vector<at::Tensor> v{outs[(size_t)r]};
+      pending.push_back(recv(v, r, 0));
+    }
+    hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(input.get_device()).stream();
+    copyAsync(outs[(size_t)root].data_ptr(), input.data_ptr(), mine, cur);
+    for (auto& w : pending) w->wait();
+    return c10::make_intrusive<WorkCCL>(rank_, c10d::OpType::GATHER, "gather", std::vector<at::Tensor>{input}, outs, blocking_wait_);
+  }
   Plan p;
   p.op = c10d::OpType::GATHER;
   p.title = "gather";
@@ -1313,6 +1370,21 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
   all.push_back(outputs[0]);
   checkDeviceTensors(all);
   at::Tensor out = outputs[0];
+  // Every rank receives the same number of bytes (src/gpu/dpcpp_ccl.cpp:1341-1359), so all ranks
+  // know the size of the root's staging image from their own output.  More than one staging
+  // window: point to point.
+  if ((size_t)(W - 1) * roundUp(nbytes(out), 16) > stage_max_) {
+    if (rank_ != root) return recv(outputs, root, 0);
+    for (int r = 0; r < W; ++r) {
+      TORCH_CHECK(nbytes(ins[(size_t)r]) == nbytes(out), "scatter: input tensor ", r, " does not match the size rank ", r, " receives");
+      if (r == root) continue;
+      std::vector<at::Tensor> v{ins[(size_t)r]};
+      send(v, r, 0);
+    }
+    hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(out.get_device()).stream();
+    copyAsync(out.data_ptr(), ins[(size_t)root].data_ptr(), nbytes(out), cur);
+    return c10::make_intrusive<WorkCCL>(rank_, c10d::OpType::SCATTER, "scatter", ins, std::vector<at::Tensor>{out}, blocking_wait_);
+  }
   Plan p;
   p.op = c10d::OpType::SCATTER;
   p.title = "scatter";
