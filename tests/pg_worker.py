@@ -428,6 +428,14 @@ def list_window_cases(pg, rank, world):
     want = sum(val(r, rank) for r in range(world))
     assert float(out.min()) == want == float(out.max()), "reduce_scatter"
     assert all(torch.equal(a, b) for a, b in zip(ins, keep)), "reduce_scatter must not touch its inputs"
+    # all_to_all (list), uneven sizes: rank r sends rank d a tensor of 1000 + 97 r + 13 d floats
+    size = lambda r, d: 1000 + 97 * r + 13 * d
+    a_in = [torch.full((size(rank, d),), val(rank, d), device=DEV) for d in range(world)]
+    a_out = [torch.zeros(size(r, rank), device=DEV) for r in range(world)]
+    pg.alltoall(a_out, a_in).wait()
+    torch.cuda.synchronize()
+    for r in range(world):
+        assert float(a_out[r].min()) == val(r, rank) == float(a_out[r].max()), ("alltoall", r)
     # gather and scatter, every rank root in turn
     for root in range(world):
         go = c10d.GatherOptions()

@@ -1189,40 +1189,60 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>
   const int me = rank_;
   std::vector<at::Tensor> ins = inputs, outs = outputs;
   // The pack of the reference (src/gpu/dpcpp_ccl.cpp:1505-1515) is the copy-in itself, and the
-  // pull writes straight into the output tensors, which is its unpack (:1528-1538).
-  Plan p;
-  p.op = c10d::OpType::ALLTOALL;
-  p.title = "alltoall";
-  p.inputs = ins;
-  p.outputs = outs;
-  p.table.resize((size_t)(2 * W));
+  // pull writes straight into the output tensors, which is its unpack (:1528-1538).  The packed
+  // image (the inputs back to back, each on a 16-byte boundary) travels in windows like the input
+  // of alltoall_base: window w holds image bytes [w * window, (w + 1) * window) of every rank.
   std::vector<size_t> offs((size_t)W);
   size_t total = 0;
   for (int d = 0; d < W; ++d) {
     offs[(size_t)d] = total;
-    p.table[(size_t)d] = (int64_t)total;
-    p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
     total += roundUp(nbytes(ins[(size_t)d]), 16);
   }
-  TORCH_CHECK(total <= stage_max_, "ccl backend: alltoall (list) larger than the staging window");
-  p.stage_bytes = total;
-  p.copy_in = [=](void* stage, hipStream_t s) {
-    std::vector<mccl_segment_t> segs;
-    for (int d = 0; d < W; ++d)
-      if (ins[(size_t)d].numel())
-        segs.push_back({ins[(size_t)d].data_ptr(), (char*)stage + offs[(size_t)d], nbytes(ins[(size_t)d])});
-    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
-  };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
-    std::vector<mccl_segment_t> segs;
-    for (int r = 0; r < W; ++r) {
-      const size_t b = (size_t)tables[(size_t)r][W + me];
-      TORCH_CHECK(b == nbytes(outs[(size_t)r]), "alltoall: output tensor ", r, " does not match what rank ", r, " sends");
-      if (b) segs.push_back({(const char*)peer[(size_t)r] + tables[(size_t)r][me], outs[(size_t)r].data_ptr(), b});
+  auto nwin = std::make_shared<size_t>(1);
+  const size_t window = stage_max_;
+  c10::intrusive_ptr<c10d::Work> work;
+  for (size_t w = 0; w < *nwin; ++w) {
+    const size_t w0 = w * window, w1 = w0 + window;
+    Plan p;
+    p.op = c10d::OpType::ALLTOALL;
+    p.title = "alltoall";
+    p.inputs = ins;
+    p.outputs = outs;
+    p.table.resize((size_t)(2 * W + 1));
+    for (int d = 0; d < W; ++d) {
+      p.table[(size_t)d] = (int64_t)offs[(size_t)d];
+      p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
     }
-    MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
-  };
-  return run(p);
+    p.table[(size_t)(2 * W)] = (int64_t)total;
+    p.stage_bytes = w0 < total ? std::min(total - w0, window) : 0;
+    p.copy_in = [=](void* stage, hipStream_t s) {
+      std::vector<mccl_segment_t> segs;
+      for (int d = 0; d < W; ++d) {  // the part of input d that lies inside the window
+        const size_t lo = std::max(offs[(size_t)d], w0), hi = std::min(offs[(size_t)d] + nbytes(ins[(size_t)d]), w1);
+        if (lo < hi)
+          segs.push_back({(const char*)ins[(size_t)d].data_ptr() + (lo - offs[(size_t)d]), (char*)stage + (lo - w0), hi - lo});
+      }
+      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+      size_t largest = 0;
+      std::vector<mccl_segment_t> segs;
+      for (int r = 0; r < W; ++r) {
+        const int64_t* tr = tables[(size_t)r];
+        const size_t b = (size_t)tr[W + me];
+        TORCH_CHECK(b == nbytes(outs[(size_t)r]), "alltoall: output tensor ", r, " does not match what rank ", r, " sends");
+        largest = std::max(largest, (size_t)tr[2 * W]);
+        const size_t seg0 = (size_t)tr[me], seg1 = seg0 + b;
+        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w1);
+        if (lo < hi)
+          segs.push_back({(const char*)peer[(size_t)r] + (lo - w0), (char*)outs[(size_t)r].data_ptr() + (lo - seg0), hi - lo});
+      }
+      *nwin = std::max<size_t>(1, (largest + window - 1) / window);
+      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    work = run(p);
+  }
+  return work;
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::barrier(const c10d::BarrierOptions& /*opts*/) {
