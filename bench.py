@@ -145,6 +145,39 @@ def _backend_rank(rank, world, store_path, cases, out_path):
             ts.append(time.perf_counter() - t0)
         ts.sort()
         res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters}
+        del x, t
+
+    def timed(fn, iters=8, warm=2):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(iters):
+            dist.barrier()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return {"p50_us": ts[len(ts) // 2] * 1e6, "iters": iters}
+
+    # C4 through the backend: reduce_scatter_tensor of a 1 GiB bf16 gradient per rank (one staging window)
+    grad = torch.empty(536_870_912, dtype=torch.bfloat16, device="cuda:0").normal_(0, 1e-3)
+    shard = torch.empty(536_870_912 // world, dtype=torch.bfloat16, device="cuda:0")
+    res["c4_reduce_scatter_tensor_1GiB_bf16"] = timed(lambda: dist.reduce_scatter_tensor(shard, grad), iters=5, warm=1)
+    del grad, shard
+    # C5 through the backend: all_to_all_single with the routing counts of the 256-expert reading
+    tokens, hidden, topk = 4096, 7168, 8
+    S = torch.zeros(world, world, dtype=torch.int64)
+    for r in range(world):
+        g = rank_generator(torch, SEED, r)
+        experts = torch.topk(torch.randn(tokens, 256, generator=g), topk, dim=1).indices
+        S[r] = torch.bincount(experts.reshape(-1) // (256 // world), minlength=world)
+    a_in = torch.empty(tokens * topk, hidden, dtype=torch.bfloat16, device="cuda:0").normal_()
+    a_out = torch.empty(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device="cuda:0")
+    res["c5_all_to_all_single_448MiB_bf16"] = timed(
+        lambda: dist.all_to_all_single(a_out, a_in, S[:, rank].tolist(), S[rank].tolist()), iters=5, warm=1)
+    del a_in, a_out
     if rank == 0:
         with open(out_path, "w") as f:
             json.dump(res, f)
@@ -162,9 +195,9 @@ def backend_path(world=8):
         mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path), nprocs=world, join=True)
         with open(out_path) as f:
             res = json.load(f)
-    out = {"processes": world, "note": "host-timed dist.all_reduce incl. copy-in, host barrier, kernel and "
+    out = {"processes": world, "note": "host-timed dist.* calls incl. copy-in, host barrier, kernel and "
                                        "synchronize; all ranks run their kernels on the one GPU concurrently"}
-    for name, count, warm, iters in cases:
+    for name in res:
         out[name] = {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()}
     return out
 
