@@ -65,6 +65,12 @@ def cases_for(W):
         "inputs": [[[[float(r)] * W for _ in range(i + 1)] for i in range(W)] for r in range(W)],
         "expected": [[[[float(i)] * W for _ in range(r + 1)] for i in range(W)] for r in range(W)],
     }
+    # reduce to every root in turn, :221-237: the allreduce cases, checked on the root only
+    c["reduce"] = {"inputs": inputs, "expected": c["allreduce"]["expected"], "roots": list(range(W))}
+    # gather, :254-277: rank r contributes [r]; every rank is root once and then holds [[0], [1], ...]
+    c["gather"] = {"inputs": [[r] for r in range(W)], "expected": [[r] for r in range(W)], "roots": list(range(W))}
+    # scatter, :290-308: every root in turn scatters [[0], [1], ...]; rank r receives [r]
+    c["scatter"] = {"inputs": [[r] for r in range(W)], "expected": [[r] for r in range(W)], "roots": list(range(W))}
     # coalescing manager, :667-693: two 8-element allreduces of ones == one 16-element allreduce
     c["coalesced_allreduce_ones"] = {"num_colls": 2, "size_per_coll": 8, "expected_value": float(W)}
     # reduce_scatter_tensor of ones, :716-733: -> W
@@ -72,9 +78,27 @@ def cases_for(W):
     return c
 
 
+def p2p_cases():
+    """tests/test_c10d_p2p.py (world size 6): rank r owns a cube of side r+1 filled with r+1
+    (:29-36).  A pair 0 -> 1 (:38-68), a relay 1 -> 3 -> 5 (:73-109), every rank to every other in
+    turn (:114-147), and cubes of side 10 filled with the sender's rank, tagged (:152-183)."""
+    W = 6
+    return {
+        "world_size": W,
+        "cube": [{"side": r + 1, "value": float(r + 1)} for r in range(W)],
+        "pair": {"src": 0, "dst": 1},
+        "relay": [{"src": 1, "dst": 3}, {"src": 3, "dst": 5}],
+        "all_pairs": [{"src": s, "dst": d} for s in range(W) for d in range(W) if s != d],
+        "tagged": {"side": 10, "messages": [{"src": s, "dst": d, "tag": s, "value": float(s)}
+                                            for d in range(W) for s in range(W) if s != d]},
+    }
+
+
 def main():
-    data = {"source": "closed forms of intel/torch-ccl tests/test_c10d_ccl.py (lines cited in make_kat_fixture.py)",
-            "world_sizes": {str(W): cases_for(W) for W in range(2, 9)}}
+    data = {"source": "closed forms of intel/torch-ccl tests/test_c10d_ccl.py and tests/test_c10d_p2p.py "
+                      "(lines cited in make_kat_fixture.py)",
+            "world_sizes": {str(W): cases_for(W) for W in range(2, 9)},
+            "p2p": p2p_cases()}
     with open(os.path.join(HERE, "c10d_kats.json"), "w") as f:
         json.dump(data, f, separators=(",", ":"))
     print("wrote c10d_kats.json")

@@ -92,27 +92,27 @@ def reference_cases(pg, rank, world):
     pg.alltoall(outs, [_dev(v, torch.float32) for v in L["inputs"][rank]]).wait()
     assert [t.cpu().tolist() for t in outs] == L["expected"][rank]
     # reduce to each root in turn (:221-237): the allreduce closed forms, on the root only
-    for name, want in K["allreduce"]["expected"].items():
-        for root in range(world):
+    for name, want in K["reduce"]["expected"].items():
+        for root in K["reduce"]["roots"]:
             opts = c10d.ReduceOptions()
             opts.reduceOp = ops[name]
             opts.rootRank = root
-            t = _dev(K["allreduce"]["inputs"][rank])
+            t = _dev(K["reduce"]["inputs"][rank])
             pg.reduce([t], opts).wait()
             if rank == root:
                 assert t.cpu().tolist() == want, (name, root, t.cpu().tolist(), want)
             else:
-                assert t.cpu().tolist() == K["allreduce"]["inputs"][rank]  # untouched off the root
+                assert t.cpu().tolist() == K["reduce"]["inputs"][rank]  # untouched off the root
     # gather, every rank root in turn, work items collected first (:254-277)
     outputs = [_dev([-1]) for _ in range(world)]
     work = []
-    for root in range(world):
+    for root in K["gather"]["roots"]:
         opts = c10d.GatherOptions()
         opts.rootRank = root
-        work.append(pg.gather([outputs] if root == rank else [], [_dev([rank])], opts))
+        work.append(pg.gather([outputs] if root == rank else [], [_dev(K["gather"]["inputs"][rank])], opts))
     for w in work:
         w.wait()
-    assert [t.cpu().tolist() for t in outputs] == [[r] for r in range(world)]
+    assert [t.cpu().tolist() for t in outputs] == K["gather"]["expected"]
     try:
         opts = c10d.GatherOptions()
         opts.rootRank = (rank + 1) % world
@@ -121,12 +121,12 @@ def reference_cases(pg, rank, world):
     except RuntimeError as e:
         assert "gather: number of output tensors should be 0 for non-root" in str(e)
     # scatter from each root in turn (:290-308)
-    for root in range(world):
+    for root in K["scatter"]["roots"]:
         opts = c10d.ScatterOptions()
         opts.rootRank = root
         output = [_dev([-1])]
-        pg.scatter(output, [[_dev([r]) for r in range(world)]] if root == rank else [], opts).wait()
-        assert output[0].cpu().tolist() == [rank]
+        pg.scatter(output, [[_dev(v) for v in K["scatter"]["inputs"]]] if root == rank else [], opts).wait()
+        assert output[0].cpu().tolist() == K["scatter"]["expected"][rank]
     try:
         opts = c10d.ScatterOptions()
         opts.rootRank = rank
@@ -604,50 +604,35 @@ def ddp_case(rank, world):
 
 
 def reference_p2p_cases(rank, world):
-    """The four cases of the reference's tests/test_c10d_p2p.py (world size 6, cubes of rank+1
-    elements per side filled with rank+1): a pair (:38-68), a relay 1 -> 3 -> 5 (:73-109), every
-    rank sending to all others in turn (:114-147), and the same with tags (:152-183)."""
-    def cube(n, value=None):
-        return torch.full((n, n, n), float(n if value is None else value))
+    """The four cases of the reference's tests/test_c10d_p2p.py (world size 6), from the fixture:
+    cubes of rank+1 elements per side filled with rank+1; a pair, a relay 1 -> 3 -> 5, every rank
+    sending to all others in turn, and the same with tags."""
+    with open(os.path.join(ROOT, "tests", "golden", "c10d_kats.json")) as f:
+        P = json.load(f)["p2p"]
+    assert world == P["world_size"]
+
+    def cube(r, fill=None):
+        side = P["cube"][r]["side"]
+        return torch.full((side, side, side), P["cube"][r]["value"] if fill is None else fill)
 
     dist.all_reduce(torch.zeros(1, device=DEV))  # the reference's tests start with one, too
-    mine = cube(rank + 1).to(DEV)
-    if rank == 0:
-        dist.send(mine, 1)
-    elif rank == 1:
-        out = cube(1, -1).to(DEV)
-        dist.recv(out, 0)
-        assert torch.equal(out.cpu(), cube(1))
-    if rank == 1:
-        dist.send(mine, 3)
-    if rank == 3:
-        out = cube(2, -1).to(DEV)
-        dist.recv(out, 1)
-        assert torch.equal(out.cpu(), cube(2))
-        dist.send(mine, 5)
-    if rank == 5:
-        out = cube(4, -1).to(DEV)
-        dist.recv(out, 3)
-        assert torch.equal(out.cpu(), cube(4))
-    for src in range(world):
-        if src == rank:
-            for dst in range(world):
-                if dst != rank:
-                    dist.send(mine, dst)
-        else:
-            out = cube(src + 1, -1).to(DEV)
-            dist.recv(out, src)
-            assert torch.equal(out.cpu(), cube(src + 1))
-    tagged = cube(10, rank).to(DEV)
-    for dst in range(world):
-        if dst == rank:
-            for src in range(world):
-                if src != rank:
-                    out = cube(10, -1).to(DEV)
-                    dist.recv(out, src, tag=src)
-                    assert bool(out.eq(src).all())
-        else:
-            dist.send(tagged, dst, tag=rank)
+    mine = cube(rank).to(DEV)
+    for hop in [P["pair"]] + P["relay"] + P["all_pairs"]:
+        if rank == hop["src"]:
+            dist.send(mine, hop["dst"])
+        elif rank == hop["dst"]:
+            out = cube(hop["src"], -1.0).to(DEV)
+            dist.recv(out, hop["src"])
+            assert torch.equal(out.cpu(), cube(hop["src"])), hop
+    side = P["tagged"]["side"]
+    tagged = torch.full((side, side, side), float(rank), device=DEV)
+    for m in P["tagged"]["messages"]:
+        if rank == m["src"]:
+            dist.send(tagged, m["dst"], tag=m["tag"])
+        elif rank == m["dst"]:
+            out = torch.full((side, side, side), -1.0, device=DEV)
+            dist.recv(out, m["src"], tag=m["tag"])
+            assert bool(out.eq(m["value"]).all()), m
     dist.barrier()
 
 
