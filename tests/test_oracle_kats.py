@@ -139,3 +139,16 @@ def _decode(x, dtype):
     if dtype == O.F16:
         return O.f16_to_f32(x).astype(np.float64)
     return x.astype(np.float64)
+
+
+def test_fixture_matches_its_generator():
+    """tests/golden/c10d_kats.json is exactly what tests/golden/make_kat_fixture.py writes."""
+    import importlib.util
+    here = os.path.dirname(__file__)
+    spec = importlib.util.spec_from_file_location("make_kat_fixture", os.path.join(here, "golden", "make_kat_fixture.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    with open(os.path.join(here, "golden", "c10d_kats.json")) as f:
+        committed = json.load(f)
+    assert committed["world_sizes"] == json.loads(json.dumps({str(W): mod.cases_for(W) for W in range(2, 9)}))
+    assert committed["p2p"] == json.loads(json.dumps(mod.p2p_cases()))
