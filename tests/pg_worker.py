@@ -283,6 +283,19 @@ def dist_api_cases(rank, world):
     o = torch.zeros(2, 2, device=DEV)
     dist.reduce_scatter_tensor(o, torch.ones(world * 2, 2, device=DEV))
     assert torch.equal(o.cpu(), torch.full((2, 2), float(world)))
+    # many asynchronous all_reduces of mixed sizes in flight before the first wait: small ones run on
+    # the caller's stream, large ones on the communication stream, the two staging slots alternate
+    rng = np.random.default_rng(77)
+    sizes = [int(x) for x in rng.choice([1, 300, 70_000, 300_000, 1_100_000, 2_500_000], size=40)]
+    ts = [torch.full((n,), float(rank + 1 + i % 3), device=DEV) for i, n in enumerate(sizes)]
+    works = [dist.all_reduce(t, async_op=True) for t in ts]
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    for i, t in enumerate(ts):
+        want = float(sum(r + 1 + i % 3 for r in range(world)))
+        assert float(t.min()) == want == float(t.max()), ("async all_reduce", i, sizes[i])
+    del ts, works
     # rooted collectives through the public API
     t = torch.full((10,), float(rank + 1), device=DEV)
     dist.reduce(t, dst=world - 1)
