@@ -21,13 +21,29 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
+sys.path.insert(0, os.path.join(ROOT, "bench"))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published peak
 SEED = 1234
-# HBM bytes of one launch of the headline kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of
-# this script, each counter scaled by its reading for a 512 MiB copy of known size
-# (profiles/reduce_bf16_8rank_64MiB_stream.md).  Algorithmic bytes are 603,979,776.
-C3_TRAFFIC_BYTES_ROCPROF = 604_011_594
+# HBM bytes of one launch of the headline kernel come from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of
+# this script, each counter scaled by its reading for a 512 MiB copy of known size; the summary of
+# those runs is this file, and the figure is read from its "Calibrated traffic" line.
+C3_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "reduce_bf16_8rank_64MiB_stream.md")
+
+
+def profiled_traffic_bytes(path=C3_TRAFFIC_PROFILE):
+    """Bytes per launch from the committed counter summary (None when the file or the line is
+    missing, so that a stale or absent profile shows as null instead of a made-up number)."""
+    import re
+    try:
+        with open(path) as f:
+            for line in f:
+                m = re.search(r"Calibrated traffic of one reduce launch:.*?=\s*([0-9][0-9 ,_]*)\s*B\b", line)
+                if m:
+                    return int(re.sub(r"[ ,_]", "", m.group(1)))
+    except OSError:
+        pass
+    return None
 
 
 def log(*a):
@@ -121,6 +137,7 @@ def _backend_rank(rank, world, store_path, cases, out_path):
     """One rank process of the drop-in path: dist.all_reduce through backend "ccl" on cuda:0."""
     os.dup2(2, 1)
     sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
+sys.path.insert(0, os.path.join(ROOT, "bench"))
     import torch
     import torch.distributed as dist
     import torch_ccl_amd  # noqa: F401
@@ -273,7 +290,8 @@ def main():
 
     import torch
     import torch_ccl_amd as mccl
-    from torch_ccl_amd import benchlib, capi
+    from torch_ccl_amd import capi
+    import benchlib
 
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible; the HIP path cannot run here.")
@@ -297,11 +315,16 @@ def main():
     # warm-up steps (untimed), then EXACTLY K timed steps between two synchronisations
     for _ in range(args.warmup):
         mccl.reduce_n(ins, out=out, op=mccl.SUM)
+    # everything that is not a launch happens before the clock starts: library handle, pointer
+    # tables, the event pair
+    loop = benchlib.ReduceLoop([ins], [out], variant=capi.VARIANT_AUTO)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    ev_us = benchlib.reduce_throughput([ins], [out], variant=capi.VARIANT_AUTO, warmup=0, iters=args.steps)
+    loop.run(args.steps)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    ev_us = loop.elapsed_us() / args.steps
+    loop.close()
     ms_per_step = wall / args.steps * 1e3
     value = alg_bytes * args.steps / wall / 1e9
     achieved = alg_bytes / (ev_us * 1e-6) / 1e9
@@ -325,11 +348,12 @@ def main():
                    "buffer_offsets_MiB": [round((t.data_ptr() - ins[0].data_ptr()) / 2**20, 3) for t in ins + [out]]},
         "pct_of_peak": round(value / PEAK_HBM_GBS * 100, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": C3_TRAFFIC_BYTES_ROCPROF,
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": profiled_traffic_bytes(),
                      "kernel_us": round(ev_us, 2),
                      "note": "achieved = (N+1)*S algorithmic bytes / average launch duration from one HIP "
                              "event pair around the K timed launches on the launch stream; traffic = "
-                             "calibrated rocprofv3 FETCH_SIZE+WRITE_SIZE bytes per launch (offline run)"},
+                             "calibrated rocprofv3 FETCH_SIZE+WRITE_SIZE bytes per launch, read from "
+                             "profiles/reduce_bf16_8rank_64MiB_stream.md (offline run of this script)"},
     }
 
     # parity spot check of the timed output against an on-device fp32 chain
@@ -667,6 +691,13 @@ def main():
         result["c10d_backend_path"] = backend_result
 
     print(json.dumps(result), flush=True)
+    # a throughput figure for wrong results is no figure: the line above says what mismatched
+    bad = [k for k in ("parity_check",) if result.get(k) == "MISMATCH"]
+    if result.get("cpu_baseline") and result["cpu_baseline"].get("gpu_matches_cpu_bit_exact") is False:
+        bad.append("cpu_baseline.gpu_matches_cpu_bit_exact")
+    if bad:
+        log("bench.py: PARITY MISMATCH in", ", ".join(bad))
+        sys.exit(4)
 
 
 if __name__ == "__main__":

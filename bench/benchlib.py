@@ -1,13 +1,13 @@
 """ctypes binding of libmcclbench.so: HIP-event timing loops around the C ABI
-(include/mccl_bench.h).  Benchmark support; not needed to use the library."""
+(mccl_bench.h beside this file).  Benchmark support; not needed to use the library."""
 import ctypes
 import os
 
 import torch
 
-from . import capi
+from torch_ccl_amd import capi
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmcclbench.so")
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmcclbench.so")
 _lib = None
 
 
@@ -22,6 +22,11 @@ def lib():
         L.mcclb_last_error.restype = ctypes.c_char_p
         L.mcclb_reduce_latency.argtypes = [vp, i32, vp, i32, sz, i32, i32, i32, vp, i32, i32, vp]
         L.mcclb_reduce_throughput.argtypes = [vp, i32, vp, i32, sz, i32, i32, i32, vp, i32, i32, vp]
+        L.mcclb_loop_create.argtypes = [ctypes.POINTER(vp)]
+        L.mcclb_loop_reduce.argtypes = [vp, vp, i32, vp, i32, sz, i32, i32, i32, vp, i32]
+        L.mcclb_loop_elapsed_us.argtypes = [vp, vp]
+        L.mcclb_loop_destroy.argtypes = [vp]
+        L.mcclb_loop_destroy.restype = None
         L.mcclb_reduce_scatter_throughput.argtypes = [vp, i32, vp, sz, i32, i32, i32, i32, vp, i32, i32, vp]
         L.mcclb_copy_latency.argtypes = [vp, i32, vp, i32, i32, vp]
         L.mcclb_copy_throughput.argtypes = [vp, i32, vp, i32, i32, vp]
@@ -65,6 +70,40 @@ def reduce_throughput(input_sets, outputs, op=capi.SUM, variant=capi.VARIANT_AUT
                                          capi.TORCH_DTYPE[o.dtype], op, variant, _stream(), warmup, iters,
                                          ctypes.byref(total)))
     return total.value / iters
+
+
+class ReduceLoop:
+    """`iters` back-to-back calls of mccl_reduce_n with everything that is not a launch done up front:
+    the library handle, the pointer tables and the event pair exist before the caller starts its
+    clock.  run() only records, enqueues and records; elapsed_us() (after the caller's own
+    synchronisation) is the time between the two events."""
+
+    def __init__(self, input_sets, outputs, op=capi.SUM, variant=capi.VARIANT_AUTO):
+        self._lib = lib()
+        self._keep = (input_sets, outputs)
+        self._n, self._ins, self._outs = _sets(input_sets, outputs)
+        o = outputs[0]
+        self._args = (len(input_sets), o.numel(), capi.TORCH_DTYPE[o.dtype], op, variant)
+        self._h = ctypes.c_void_p()
+        _check(self._lib.mcclb_loop_create(ctypes.byref(self._h)))
+        self._stream = _stream()
+
+    def run(self, iters):
+        nsets, count, dtype, op, variant = self._args
+        rc = self._lib.mcclb_loop_reduce(self._h, self._ins, self._n, self._outs, nsets, count, dtype, op, variant,
+                                         self._stream, iters)
+        if rc != 0:
+            _check(rc)
+
+    def elapsed_us(self):
+        total = ctypes.c_float(0)
+        _check(self._lib.mcclb_loop_elapsed_us(self._h, ctypes.byref(total)))
+        return total.value
+
+    def close(self):
+        if self._h:
+            self._lib.mcclb_loop_destroy(self._h)
+            self._h = ctypes.c_void_p()
 
 
 def reduce_scatter_throughput(inputs, outputs, shard_first=0, op=capi.SUM, warmup=3, iters=10):

@@ -1,4 +1,4 @@
-// libmcclbench: HIP-event timing loops around the C ABI (see include/mccl_bench.h).
+// libmcclbench: HIP-event timing loops around the C ABI (see mccl_bench.h beside this file).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -167,6 +167,59 @@ int mcclb_reduce_throughput(const void* const* in, int n, void* const* out, int 
     return mccl_reduce_n(in + (size_t)set * n, n, out[set], count, dtype, op, variant, stream);
   };
   return throughput_loop(call, (hipStream_t)stream, warmup, iters, total_us);
+}
+
+// A timed loop whose set-up (the two events) happens before the caller starts its own clock.
+struct TimedLoop {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+};
+
+int mcclb_loop_create(void** loop) {
+  if (!loop) { snprintf(g_err, sizeof(g_err), "loop must be non-null"); return MCCL_ERR_INVALID_ARG; }
+  TimedLoop* t = new TimedLoop();
+  hipError_t e = hipEventCreate(&t->e0);
+  if (e == hipSuccess) e = hipEventCreate(&t->e1);
+  if (e != hipSuccess) {
+    if (t->e0) (void)hipEventDestroy(t->e0);
+    delete t;
+    return fail_hip("hipEventCreate", e);
+  }
+  *loop = t;
+  return MCCL_OK;
+}
+
+int mcclb_loop_reduce(void* loop, const void* const* in, int n, void* const* out, int nsets,
+                      size_t count, int dtype, int op, int variant, void* stream, int iters) {
+  TimedLoop* t = static_cast<TimedLoop*>(loop);
+  if (!t || iters <= 0) { snprintf(g_err, sizeof(g_err), "needs a loop and iters > 0"); return MCCL_ERR_INVALID_ARG; }
+  if (nsets < 1) nsets = 1;
+  hipStream_t s = (hipStream_t)stream;
+  HIP_OK(hipEventRecord(t->e0, s));
+  int rc = MCCL_OK;
+  for (int i = 0; i < iters && rc == MCCL_OK; ++i) {
+    const int set = i % nsets;
+    rc = mccl_reduce_n(in + (size_t)set * n, n, out[set], count, dtype, op, variant, stream);
+  }
+  HIP_OK(hipEventRecord(t->e1, s));
+  return rc == MCCL_OK ? MCCL_OK : fail_mccl(rc);
+}
+
+int mcclb_loop_elapsed_us(void* loop, float* total_us) {
+  TimedLoop* t = static_cast<TimedLoop*>(loop);
+  if (!t || !total_us) { snprintf(g_err, sizeof(g_err), "needs a loop and an output"); return MCCL_ERR_INVALID_ARG; }
+  HIP_OK(hipEventSynchronize(t->e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, t->e0, t->e1));
+  *total_us = ms * 1000.f;
+  return MCCL_OK;
+}
+
+void mcclb_loop_destroy(void* loop) {
+  TimedLoop* t = static_cast<TimedLoop*>(loop);
+  if (!t) return;
+  (void)hipEventDestroy(t->e0);
+  (void)hipEventDestroy(t->e1);
+  delete t;
 }
 
 int mcclb_reduce_scatter_throughput(const void* const* in, int n, void* const* out,

@@ -1,5 +1,6 @@
 /*
  * mccl_bench.h -- timing loops around the C ABI of include/mccl.h (libmcclbench.so).
+ * Lives beside bench.py: it is benchmark support, not part of the library's boundary.
  *
  * Benchmark support only: these loops call the product entry points unchanged and time
  * them with HIP events recorded on the launch stream, so that per-call latencies are not
@@ -29,6 +30,18 @@ int mcclb_reduce_latency(const void* const* in, int n, void* const* out, int nse
 int mcclb_reduce_throughput(const void* const* in, int n, void* const* out, int nsets,
                             size_t count, int dtype, int op, int variant, void* stream, int warmup,
                             int iters, float* total_us);
+
+/*
+ * The same back-to-back loop with its set-up taken out, for a caller that times the loop with a
+ * clock of its own: mcclb_loop_create makes the two events; mcclb_loop_reduce records the first,
+ * enqueues `iters` calls of mccl_reduce_n and records the second, without synchronising;
+ * mcclb_loop_elapsed_us waits for the second event and returns the time between the two.
+ */
+int mcclb_loop_create(void** loop);
+int mcclb_loop_reduce(void* loop, const void* const* in, int n, void* const* out, int nsets,
+                      size_t count, int dtype, int op, int variant, void* stream, int iters);
+int mcclb_loop_elapsed_us(void* loop, float* total_us);
+void mcclb_loop_destroy(void* loop);
 
 /* The same two loops around mccl_reduce_scatter_n (all shards of one launch). */
 int mcclb_reduce_scatter_throughput(const void* const* in, int n, void* const* out,

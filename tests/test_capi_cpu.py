@@ -11,8 +11,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PKG = os.path.join(ROOT, "torch-ccl_amd")
 
 
-def _declared(header):
-    text = open(os.path.join(ROOT, "include", header)).read()
+def _declared(header, folder="include"):
+    text = open(os.path.join(ROOT, folder, header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mcclb?_[a-z0-9_]+)\s*\(", text)))
 
@@ -28,9 +28,13 @@ def test_libmi355ccl_exports_every_declared_symbol(mccl):
 
 
 def test_libmcclbench_exports_every_declared_symbol(mccl):
-    from torch_ccl_amd import benchlib
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "bench"))
+    import benchlib
     L = benchlib.lib()
-    for name in [n for n in _declared("mccl_bench.h") if n.startswith("mcclb_")]:
+    names = [n for n in _declared("mccl_bench.h", "bench") if n.startswith("mcclb_")]
+    assert len(names) >= 12
+    for name in names:
         assert hasattr(L, name), "libmcclbench.so does not export %s" % name
 
 

@@ -1,7 +1,7 @@
 """Builds the native pieces in-tree for gfx950.
 
   libmi355ccl.so   HIP kernels + C ABI (include/mccl.h); depends on the HIP runtime only.
-  libmcclbench.so  HIP-event timing loops around that ABI (include/mccl_bench.h).
+  libmcclbench.so  HIP-event timing loops around that ABI (bench/mccl_bench.h; lands in bench/).
   _C.*.so          the c10d backend (process_group_ccl.cpp) and its Python module; host code
                    only, links torch's c10d and libmi355ccl.so.
 
@@ -84,18 +84,18 @@ def build_kernels(force=False, extra_flags=(), out=KERNEL_LIB):
     return out
 
 
-BENCH_SRC = os.path.join(HERE, "mccl_bench.cpp")
-BENCH_LIB = os.path.join(LIB_DIR, "libmcclbench.so")
+BENCH_DIR = os.path.join(ROOT, "bench")
+BENCH_SRC = os.path.join(BENCH_DIR, "mccl_bench.cpp")
+BENCH_LIB = os.path.join(BENCH_DIR, "libmcclbench.so")
 
 
 def build_bench(force=False):
-    os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [BENCH_SRC, os.path.join(INCLUDE, "mccl_bench.h"), os.path.join(INCLUDE, "mccl.h")]
+    srcs = [BENCH_SRC, os.path.join(BENCH_DIR, "mccl_bench.h"), os.path.join(INCLUDE, "mccl.h"), KERNEL_LIB]
     if force or _stale(BENCH_LIB, srcs):
         cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-               "-I", INCLUDE, "-o", BENCH_LIB, BENCH_SRC,
-               "-L", LIB_DIR, "-lmi355ccl", "-Wl,-rpath,$ORIGIN"]
+               "-I", INCLUDE, "-I", BENCH_DIR, "-o", BENCH_LIB, BENCH_SRC,
+               "-L", LIB_DIR, "-lmi355ccl", "-Wl,-rpath,$ORIGIN/../torch-ccl_amd/torch_ccl_amd/lib"]
         subprocess.check_call(cmd)
     return BENCH_LIB
 
@@ -159,9 +159,20 @@ def build_all(force=False):
     return [build_kernels(force), build_bench(force), build_backend(force), build_c_caller(force)]
 
 
+def stale_outputs():
+    """Built libraries that are older than one of their sources."""
+    checks = [(KERNEL_LIB, [KERNEL_SRC, REDUCE_SRC] + KERNEL_HDRS),
+              (BENCH_LIB, [BENCH_SRC, os.path.join(BENCH_DIR, "mccl_bench.h")]),
+              (backend_lib_path(), BACKEND_SRCS + BACKEND_HDRS)]
+    return [out for out, srcs in checks if os.path.exists(out) and _stale(out, srcs)]
+
+
 def ensure_built():
-    """Builds only what does not exist yet (no staleness check): for tests, smoke() and bench.py,
-    which use the libraries that are there and compile only when nothing is."""
+    """Builds only what does not exist yet: for tests, smoke() and bench.py, which use the libraries
+    that are there and compile only when nothing is.  A library older than its sources is used as
+    it is, with a warning on stderr, so that an edit without a rebuild does not pass unnoticed."""
+    for out in stale_outputs():
+        sys.stderr.write("warning: %s is older than its sources; run `python torch-ccl_amd/csrc/build.py`\n" % out)
     built = []
     if not os.path.exists(KERNEL_LIB):
         built.append(build_kernels(force=True))
