@@ -137,7 +137,6 @@ def _backend_rank(rank, world, store_path, cases, out_path):
     """One rank process of the drop-in path: dist.all_reduce through backend "ccl" on cuda:0."""
     os.dup2(2, 1)
     sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
-sys.path.insert(0, os.path.join(ROOT, "bench"))
     import torch
     import torch.distributed as dist
     import torch_ccl_amd  # noqa: F401
