@@ -139,6 +139,46 @@ int mccl_reduce_scatter_n(const void* const* in, int n, void* const* out, size_t
 int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size_t* counts,
                       int nbuf, int dtype, int op, void* stream);
 
+/*
+ * Cross-rank barrier on device flags, for ranks that are processes (or GPUs) of their own: the
+ * one-thread sync kernels between the data kernels of the reference's large allreduce
+ * (src/gpu/allreduce.h:731-769, 835-877).  flags[r] is the address, in the caller's own mapping,
+ * of rank r's 64-bit flag word (device memory the peers can reach, e.g. opened from an IPC handle;
+ * zero before the first use).  One wavefront stores `epoch` into flags[rank] and then waits until
+ * every flags[r] has reached `epoch`.  Epochs must grow from call to call (the words are never
+ * cleared) and all ranks must pass the same epoch for the same barrier.  Stream-ordered: what the
+ * stream enqueued before the barrier is complete and visible to a peer's kernels enqueued after
+ * its own barrier of the same epoch.  No host thread takes part.
+ *   The wait is bounded: after timeout_us microseconds (0 = 10 s) the kernel stores 1 + the rank it
+ * was waiting for into status[0] and the low half of the epoch into status[1], and returns; status
+ * may be null, or two 32-bit words the GPU can write (device memory or mapped pinned host memory)
+ * that the caller zeroes and reads.
+ *   Callers whose ranks share one process must give every rank a stream that maps to a hardware
+ * queue of its own: a waiting wavefront blocks the kernels queued behind it.
+ */
+int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us,
+                      void* status, void* stream);
+
+/*
+ * One-launch small allreduce across rank processes: copy-in, rank synchronisation and the
+ * N-peer reduction in a single kernel, the structure of allreducer_small<T>::allreduce
+ * (src/gpu/allreduce_small.h:166-361).  Rank `rank` contributes in[0..count) and receives the
+ * reduction of all n contributions in out (out may be in).  stage[r] is rank r's staging buffer
+ * (at least count elements rounded up to 16 bytes, 16-byte aligned) and tile_flags[r] its array of
+ * 32-bit flags, one per MCCL_FUSED_TILE_BYTES of message (zero before the first use), both in the
+ * caller's own mapping.  Every rank calls with the same count, dtype, op and epoch; epochs must
+ * grow from call to call on the same staging buffers, and a staging buffer may be reused only
+ * after every peer has started a later collective (two alternating sets do).  Same arithmetic and
+ * bits as mccl_reduce_n over the n contributions.  At most MCCL_FUSED_MAX_RANKS ranks.  The wait
+ * is bounded and reported like mccl_rank_barrier's; a tile whose peers did not arrive in time is
+ * left unwritten.
+ */
+#define MCCL_FUSED_MAX_RANKS 8
+#define MCCL_FUSED_TILE_BYTES 1024
+int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
+                         void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
+                         uint64_t timeout_us, void* status, void* stream);
+
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream);

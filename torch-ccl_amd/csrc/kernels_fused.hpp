@@ -1,0 +1,113 @@
+// One-launch small allreduce across rank processes: copy-in, cross-rank flags and the N-peer
+// reduction in a single kernel, the structure of the reference's small allreduce
+// (src/gpu/allreduce_small.h:166-361: copy into the IPC-visible buffer, rank barrier, sum of the N
+// peer buffers).  Where the reference synchronises the whole grid and then all ranks, this kernel
+// synchronises tile by tile: the wavefront that owns tile t of rank r
+//   1. copies its 1 KiB of the caller's tensor into rank r's staging buffer,
+//   2. publishes flag[r][t] = epoch (release),
+//   3. waits until flag[q][t] has reached the epoch for every peer q (acquire, bounded),
+//   4. reads tile t of every peer's staging buffer, runs the ascending-rank chain (its own
+//      contribution comes from the registers of step 1) and writes the caller's output.
+// A wavefront depends on the wavefronts of the same tile in the peers' launches only, so no grid
+// has to be resident as a whole, and a launch needs no second kernel and no host round trip.
+// Visibility inside the kernel rests on the fences: the release fence writes the tile back before
+// the flag is stored, the acquire fence after the wait invalidates what this wavefront's caches
+// hold of the peers' buffers.
+#pragma once
+
+#include "kernels_common.hpp"
+#include "kernels_sync.hpp"
+
+namespace {
+
+constexpr int kFusedRanks = 8;
+
+struct FusedArgs {
+  const char* in;             // this rank's contribution (element-aligned)
+  char* out;                  // result; may be `in`
+  char* stage[kFusedRanks];   // staging buffer of every rank (16-byte aligned), this process's mappings
+  uint32_t* flag[kFusedRanks];  // per-tile flags of every rank
+  uint64_t nvec;              // whole 16-byte vectors of the message
+  uint64_t limit_ticks;
+  uint32_t* status;
+  uint32_t tail;              // elements after the last whole vector (< elements per vector)
+  uint32_t epoch;
+  int n;
+  int rank;
+};
+
+// 32-bit epochs wrap: compare as a signed distance.
+__device__ __forceinline__ bool wait_flag32(const uint32_t* word, uint32_t epoch, uint64_t limit_ticks) {
+  const uint64_t t0 = wall_clock64();
+  while ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) < 0) {
+    if (wall_clock64() - t0 > limit_ticks) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  return true;
+}
+
+template <int DT, int OP>
+__global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs a) {
+  using S = typename Elem<DT>::store_t;
+  using A = typename Elem<DT>::acc_t;
+  constexpr int VE = vec_elems<DT>();
+  const uint32_t tile = blockIdx.x;
+  const int lane = threadIdx.x;
+  const uint64_t v = (uint64_t)tile * kWave + lane;
+  const bool whole = v < a.nvec;
+  const bool part = v == a.nvec && a.tail != 0;  // the one vector that is not whole
+
+  // 1. copy-in
+  VecU<DT> mine;
+  mine.v = (u32x4){0u, 0u, 0u, 0u};
+  if (whole) {
+    mine.v = __builtin_nontemporal_load(&((const u32x4_unaligned*)a.in)[v]);
+  } else if (part) {
+    for (uint32_t e = 0; e < a.tail; ++e) vec_set<DT>(mine, (int)e, ((const S*)a.in)[v * VE + e]);
+  }
+  if (whole || part) ((u32x4*)a.stage[a.rank])[v] = mine.v;
+  // 2. publish: the tile is written back before the flag can be seen
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  if (lane == 0) __hip_atomic_store(a.flag[a.rank] + tile, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  // 3. wait for the same tile of every peer
+  bool ok = true;
+  if (lane < a.n && lane != a.rank) {
+    ok = wait_flag32(a.flag[lane] + tile, a.epoch, a.limit_ticks);
+    if (!ok) report_late(a.status, lane, a.epoch);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  // a tile whose peers did not arrive is left alone (the failure is reported through `status`)
+  if (__builtin_amdgcn_ballot_w64(!ok) != 0) return;
+  if (!(whole || part)) return;
+
+  // 4. the N-peer reduction, ascending rank order; all peer loads are issued before the first add
+  VecU<DT> x[kFusedRanks];
+#pragma unroll
+  for (int k = 0; k < kFusedRanks; ++k) {
+    if (k < a.n) {
+      if (k == a.rank) x[k].v = mine.v;
+      else x[k].v = __builtin_nontemporal_load(&((const u32x4*)a.stage[k])[v]);
+    }
+  }
+  A acc[VE];
+#pragma unroll
+  for (int e = 0; e < VE; ++e) acc[e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x[0], e)));
+#pragma unroll
+  for (int k = 1; k < kFusedRanks; ++k) {
+    if (k < a.n) {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) acc[e] = chain_next<DT, OP>(acc[e], Elem<DT>::load(vec_get<DT>(x[k], e)));
+    }
+  }
+  VecU<DT> r;
+  r.v = (u32x4){0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < VE; ++e) vec_set<DT>(r, e, Elem<DT>::store(chain_last<DT, OP>(acc[e], a.n)));
+  if (whole) {
+    ((u32x4_unaligned*)a.out)[v] = r.v;
+  } else {
+    for (uint32_t e = 0; e < a.tail; ++e) ((S*)a.out)[v * VE + e] = vec_get<DT>(r, (int)e);
+  }
+}
+
+}  // namespace

@@ -36,6 +36,10 @@
 //   reduce_vec_kernel : the N-peer sum of src/gpu/allreduce_small.h:289-361,
 //       the five data kernels of src/gpu/allreduce.h:306-533, ccl::allreduce /
 //       ccl::reduce_scatter call sites in src/gpu/dpcpp_ccl.cpp:781-788, 1002-1008
+//   rank_barrier_kernel : the one-thread sync kernels between the data kernels of
+//       src/gpu/allreduce.h:731-769, 835-877
+//   allreduce_fused_kernel : the whole small allreduce of src/gpu/allreduce_small.h:166-361
+//       (copy-in, rank barrier, N-peer sum in one launch)
 //   copy_segments_kernel : ccl::allgatherv / ccl::alltoall(v) data movement
 //       (src/gpu/dpcpp_ccl.cpp:1176-1182, 1403-1455) and the pack/unpack copy_ loops
 //       (src/gpu/dpcpp_ccl.cpp:1505-1538)
@@ -52,6 +56,7 @@
 #include "kernels_common.hpp"
 #include "kernels_copy.hpp"
 #include "kernels_moe.hpp"
+#include "kernels_sync.hpp"
 #include "reduce_launch.hpp"
 
 namespace {
@@ -171,6 +176,29 @@ hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g,
     case MCCL_BF16: return mccl_launch_reduce_dt8(&a, op, g.shape, g.grid_x, g.lds, own, njobs, s);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned grid_x, hipStream_t s) {
+  switch (dtype) {
+    case MCCL_U8: return mccl_launch_fused_dt0(&a, op, grid_x, s);
+    case MCCL_I8: return mccl_launch_fused_dt1(&a, op, grid_x, s);
+    case MCCL_I16: return mccl_launch_fused_dt2(&a, op, grid_x, s);
+    case MCCL_I32: return mccl_launch_fused_dt3(&a, op, grid_x, s);
+    case MCCL_I64: return mccl_launch_fused_dt4(&a, op, grid_x, s);
+    case MCCL_F16: return mccl_launch_fused_dt5(&a, op, grid_x, s);
+    case MCCL_F32: return mccl_launch_fused_dt6(&a, op, grid_x, s);
+    case MCCL_F64: return mccl_launch_fused_dt7(&a, op, grid_x, s);
+    case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, grid_x, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Ticks of the 100 MHz wall clock a device-side wait may last; 0 asks for the default of 10 s.
+constexpr uint64_t kTicksPerUs = 100;
+uint64_t wait_limit_ticks(uint64_t timeout_us) {
+  if (timeout_us == 0) timeout_us = 10ull * 1000 * 1000;
+  if (timeout_us > 3600ull * 1000 * 1000) timeout_us = 3600ull * 1000 * 1000;
+  return timeout_us * kTicksPerUs;
 }
 
 // Loads one wavefront keeps in flight per tile: all ranks when the rank count is a
@@ -456,7 +484,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 100; }
+int mccl_version(void) { return 110; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -558,6 +586,89 @@ int mccl_reduce_multi(const void* const* in, int n, void* const* out, const size
     rc = launch_jobs(a, specs, m, dtype, op, MCCL_VARIANT_AUTO, true, (hipStream_t)stream);
     if (rc != MCCL_OK) return rc;
   }
+  return MCCL_OK;
+}
+
+int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us,
+                      void* status, void* stream) {
+  if (!flags) return fail(MCCL_ERR_INVALID_ARG, "flag pointer table is null");
+  if (n < 1 || n > MCCL_MAX_RANKS) return fail(MCCL_ERR_INVALID_ARG, "rank count %d outside [1, %d]", n, MCCL_MAX_RANKS);
+  if (rank < 0 || rank >= n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", rank, n);
+  if ((uintptr_t)status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
+  for (int r = 0; r < n; ++r) {
+    if (!flags[r]) return fail(MCCL_ERR_INVALID_ARG, "flag pointer %d is null", r);
+    if ((uintptr_t)flags[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "flag pointer %d is not 8-byte aligned", r);
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (n <= kLeanSyncRanks) {
+    LeanBarrierArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int r = 0; r < n; ++r) a.flag[r] = (uint64_t*)flags[r];
+    a.epoch = epoch;
+    a.limit_ticks = wait_limit_ticks(timeout_us);
+    a.status = (uint32_t*)status;
+    a.n = n;
+    a.rank = rank;
+    hipLaunchKernelGGL(rank_barrier_kernel<LeanBarrierArgs>, dim3(1), dim3(kWave), 0, s, a);
+  } else {
+    BarrierArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int r = 0; r < n; ++r) a.flag[r] = (uint64_t*)flags[r];
+    a.epoch = epoch;
+    a.limit_ticks = wait_limit_ticks(timeout_us);
+    a.status = (uint32_t*)status;
+    a.n = n;
+    a.rank = rank;
+    hipLaunchKernelGGL(rank_barrier_kernel<BarrierArgs>, dim3(1), dim3(kWave), 0, s, a);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "barrier kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
+                         void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
+                         uint64_t timeout_us, void* status, void* stream) {
+  int rc = check_reduce_args_no_ptr(n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (n > MCCL_FUSED_MAX_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "the one-launch allreduce takes at most %d ranks, got %d", MCCL_FUSED_MAX_RANKS, n);
+  if (rank < 0 || rank >= n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", rank, n);
+  if (!stage || !tile_flags) return fail(MCCL_ERR_INVALID_ARG, "staging or flag pointer table is null");
+  if ((uintptr_t)status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
+  const size_t es = dtype_size(dtype);
+  for (int r = 0; r < n; ++r) {
+    if (!stage[r] || !tile_flags[r]) return fail(MCCL_ERR_INVALID_ARG, "staging or flag pointer %d is null", r);
+    if ((uintptr_t)stage[r] % 16) return fail(MCCL_ERR_INVALID_ARG, "staging buffer %d is not 16-byte aligned", r);
+    if ((uintptr_t)tile_flags[r] % 4) return fail(MCCL_ERR_INVALID_ARG, "flag array %d is not 4-byte aligned", r);
+  }
+  if (count == 0) return MCCL_OK;
+  if (!in || !out) return fail(MCCL_ERR_INVALID_ARG, "input or output pointer is null");
+  if ((uintptr_t)in % es || (uintptr_t)out % es) return fail(MCCL_ERR_INVALID_ARG, "input or output pointer not aligned to the element size");
+  if (in != out) {
+    const uintptr_t i0 = (uintptr_t)in, o0 = (uintptr_t)out;
+    if (i0 < o0 + count * es && o0 < i0 + count * es) return fail(MCCL_ERR_INVALID_ARG, "output partially overlaps the input");
+  }
+  const size_t ve = 16 / es;
+  const size_t nvec = count / ve;
+  const size_t tiles = (nvec + (count % ve ? 1 : 0) + kWave - 1) / kWave;
+  if (tiles > kMaxGridX) return fail(MCCL_ERR_INVALID_ARG, "message too large for the one-launch allreduce");
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  a.in = (const char*)in;
+  a.out = (char*)out;
+  for (int r = 0; r < n; ++r) {
+    a.stage[r] = (char*)stage[r];
+    a.flag[r] = (uint32_t*)tile_flags[r];
+  }
+  a.nvec = nvec;
+  a.limit_ticks = wait_limit_ticks(timeout_us);
+  a.status = (uint32_t*)status;
+  a.tail = (uint32_t)(count % ve);
+  a.epoch = epoch;
+  a.n = n;
+  a.rank = rank;
+  hipError_t e = launch_fused_any(a, dtype, op, (unsigned)tiles, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "fused allreduce launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
 

@@ -23,3 +23,7 @@ extern "C" hipError_t MCCL_PASTE(mccl_launch_reduce_dt, MCCL_REDUCE_DT)(MCCL_RED
   g.stream_out = false;  // travels in the argument block's flags
   return launch_dtype<MCCL_REDUCE_DT>(*static_cast<const ReduceArgs*>(reduce_args), op, g, njobs, stream);
 }
+
+extern "C" hipError_t MCCL_PASTE(mccl_launch_fused_dt, MCCL_REDUCE_DT)(MCCL_FUSED_ENTRY_ARGS) {
+  return launch_fused_dtype<MCCL_REDUCE_DT>(*static_cast<const FusedArgs*>(fused_args), op, grid_x, stream);
+}

@@ -3,6 +3,7 @@
 // (mccl_reduce_dtype.hip, built once per type), which is what keeps the build parallel.
 #pragma once
 
+#include "kernels_fused.hpp"
 #include "kernels_reduce.hpp"
 
 namespace {
@@ -74,6 +75,27 @@ hipError_t launch_dtype(const ReduceArgs& a, int op, const Geometry& g, int njob
   }
 }
 
+// The one-launch small allreduce: one wavefront per 1 KiB tile.
+template <int DT>
+hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned grid_x, hipStream_t s) {
+  const dim3 grid(grid_x, 1, 1), block(kWave);
+  switch (op) {
+    case MCCL_SUM: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_SUM>), grid, block, 0, s, a); break;
+    case MCCL_PROD: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_PROD>), grid, block, 0, s, a); break;
+    case MCCL_MIN: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_MIN>), grid, block, 0, s, a); break;
+    case MCCL_MAX: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_MAX>), grid, block, 0, s, a); break;
+    case MCCL_AVG:
+      if constexpr (Elem<DT>::kIsFloat) {
+        hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_AVG>), grid, block, 0, s, a);
+        break;
+      } else {
+        return hipErrorInvalidValue;
+      }
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace
 
 // Entry points of the per-type translation units.  Plain types only: the argument block and the
@@ -92,4 +114,17 @@ __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt5(MCCL_RED
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt6(MCCL_REDUCE_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt7(MCCL_REDUCE_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt8(MCCL_REDUCE_ENTRY_ARGS);
+}
+// `fused_args` points at a FusedArgs.
+#define MCCL_FUSED_ENTRY_ARGS const void *fused_args, int op, unsigned grid_x, hipStream_t stream
+extern "C" {
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt0(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt1(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt2(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt3(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt4(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt5(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt6(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt7(MCCL_FUSED_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt8(MCCL_FUSED_ENTRY_ARGS);
 }

@@ -35,6 +35,7 @@ EXPORTS = (
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
+    "mccl_rank_barrier", "mccl_allreduce_fused",
 )
 
 
@@ -71,6 +72,8 @@ def lib():
     L.mccl_gather_rows.argtypes = [vp, sz, vp, sz, sz, vp, vp]
     L.mccl_moe_dispatch_n.argtypes = [vp, vp, vp, vp, i32, vp, sz, vp]
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
+    L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
+    L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, vp]
     L.mccl_query_launch.argtypes = [sz, i32, i32, i32, i32, vp, vp]
     L.mccl_set_tuning.argtypes = [i32, ctypes.c_longlong]
     L.mccl_get_tuning.argtypes = [i32]
