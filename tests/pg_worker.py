@@ -536,6 +536,161 @@ def missing_rank_case(pg, rank, world):
                 or "rank 1 left the group" in str(e)), str(e)
 
 
+def zero_copy_cases(pg, rank, world):
+    """Large single-tensor collectives between rank processes read the peers' tensors in place.
+    Same bits as the oracle: tensors that are views at odd offsets of larger allocations, a tensor
+    reused call after call (cached mappings), an allocation that is freed and handed out again at
+    the same address with other contents (a stale mapping would read the old bytes), and a rank
+    whose tensor cannot be shared (everybody stages instead)."""
+    from helpers import TORCH_TO_CODE, bits, rank_buffer, to_carrier
+    from oracle import oracle as O
+
+    def bits_np(arr):
+        return arr.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[arr.dtype.itemsize])
+
+    def view_of(host, pad):
+        """The tensor as a view `pad` elements into a larger device allocation."""
+        big = torch.empty(host.numel() + 2 * pad + 64, dtype=host.dtype, device=DEV)
+        v = big[pad:pad + host.numel()]
+        v.copy_(host)
+        return v
+
+    def allreduce_check(dtype, count, seed, pad=0, keep=None):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(count, dtype, r, seed=seed) for r in range(world)]
+        t = keep if keep is not None else view_of(host[rank], pad)
+        if keep is not None:
+            t.copy_(host[rank])
+        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        want = bits_np(O.reduce([to_carrier(h) for h in host], code, O.SUM))
+        assert np.array_equal(bits(t), want), ("allreduce", dtype, count, seed, pad)
+        return t
+
+    # allreduce: odd counts and offsets, every element width
+    for dtype, count, pad in ((torch.bfloat16, (3 << 20) + 7, 3), (torch.float32, (1 << 20) + 1, 1), (torch.int8, (5 << 20) + 13, 5),
+                              (torch.float64, (1 << 19) + 3, 0), (torch.bfloat16, 1 << 19, 0)):
+        allreduce_check(dtype, count, seed=61, pad=pad)
+    # the same tensor again and again: the peers' mappings are cached
+    t = None
+    for i in range(6):
+        t = allreduce_check(torch.bfloat16, 2 << 20, seed=70 + i, keep=t)
+    # freed and allocated again: torch returns the segment to the runtime, the next allocation of
+    # the same size usually lands on the same address, with new contents
+    for i in range(3):
+        x = allreduce_check(torch.float32, (3 << 20) + 11, seed=80 + i)
+        del x
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+    # reduce_scatter_tensor, all_gather_into_tensor, broadcast, uneven all_to_all_single
+    for dtype, m, pad in ((torch.bfloat16, 300007, 1), (torch.float32, 262144, 0)):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(world * m, dtype, r, seed=91) for r in range(world)]
+        out = torch.empty(m, dtype=dtype, device=DEV)
+        pg._reduce_scatter_base(out, view_of(host[rank], pad)).wait()
+        want = O.reduce_scatter([to_carrier(h) for h in host], code, O.SUM, shard_first=rank, shard_num=1)[0]
+        assert np.array_equal(bits(out), bits_np(want)), ("reduce_scatter", dtype, m)
+        host = [rank_buffer(m * 4, dtype, r, seed=92) for r in range(world)]
+        out = torch.empty(world * m * 4, dtype=dtype, device=DEV)
+        pg._allgather_base(out, view_of(host[rank], pad)).wait()
+        assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather", dtype, m)
+        root = m % world
+        src = rank_buffer(m * 4 + 3, dtype, root, seed=93)
+        t = view_of(src if rank == root else torch.zeros_like(src), pad)
+        opts = c10d.BroadcastOptions()
+        opts.rootRank = root
+        pg.broadcast([t], opts).wait()
+        assert np.array_equal(bits(t), bits(src)), ("broadcast", dtype, m)
+    rng = np.random.default_rng(4321)
+    S = rng.integers(0, 3000, size=(world, world))
+    S[world - 1, 0] = 0
+    hidden = 256
+    host = [rank_buffer(int(S[r].sum()) * hidden, torch.bfloat16, r, seed=6).view(-1, hidden) for r in range(world)]
+    out = torch.zeros(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device=DEV)
+    pg.alltoall_base(out, host[rank].to(DEV), S[:, rank].tolist(), S[rank].tolist()).wait()
+    want = O.alltoallv([to_carrier(h) for h in host], S, hidden * 2)[rank]
+    assert np.array_equal(out.cpu().view(torch.uint8).numpy().reshape(-1), want), "alltoallv"
+    # rank 1's tensor lives in an allocation too large to be shared between processes: every rank
+    # stages, results are the same
+    count = (2 << 20) + 5
+    host = [rank_buffer(count, torch.bfloat16, r, seed=99) for r in range(world)]
+    if rank == 1:
+        big = torch.empty((2 << 30) // 2 + 4096, dtype=torch.bfloat16, device=DEV)
+        t = big[4096:4096 + count]
+        t.copy_(host[rank])
+    else:
+        t = host[rank].to(DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    want = bits_np(O.reduce([to_carrier(h) for h in host], O.BF16, O.SUM))
+    assert np.array_equal(bits(t), want), "allreduce with an unshareable tensor on rank 1"
+    pg.barrier().wait()
+
+
+def missing_rank_device_case(pg, rank, world):
+    """Device-side waits: rank 1 never joins the second collective.  The survivors' kernel gives up
+    by itself at the (shortened) limit and names the late rank; their Work reports the failure
+    instead of success, the tensor is left alone, and the group refuses further collectives."""
+    t = torch.ones(16, device=DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    torch.cuda.synchronize()
+    assert t.cpu().tolist() == [float(world)] * 16
+    if rank == 1:
+        return
+    blocking = os.environ.get("CCL_BLOCKING_WAIT") == "1"
+    before = t.clone()
+    w = pg.allreduce([t], c10d.AllreduceOptions())
+    if blocking:
+        try:
+            w.wait()
+            raise AssertionError("blocking wait on a collective with a missing rank returned")
+        except RuntimeError as e:
+            assert "timed out waiting for rank 1 on the device" in str(e), str(e)
+    else:
+        w.wait()  # stream-ordered: returns at once, the failure shows when the device gets there
+        torch.cuda.synchronize()
+    assert w.is_completed()
+    assert not w.is_success()
+    assert torch.equal(t, before)
+    try:
+        pg.allreduce([t], c10d.AllreduceOptions())
+        raise AssertionError("a failed group accepted another collective")
+    except RuntimeError as e:
+        assert "timed out waiting for rank 1" in str(e), str(e)
+
+
+def late_peer_case(pg, rank, world):
+    """wait(timeout) in blocking mode: rank 1 joins 1.5 s late, the others wait with a 200 ms limit
+    and get the reference's "Caught collective operation timeout"; the collective itself still
+    completes once the late rank arrives, with the right result."""
+    import datetime
+    import time
+    t = torch.ones(1 << 18, device=DEV)
+    pg.allreduce([t], c10d.AllreduceOptions()).wait()
+    if rank == 1:
+        time.sleep(1.5)
+    w = pg.allreduce([t], c10d.AllreduceOptions())
+    if rank != 1:
+        try:
+            w.wait(datetime.timedelta(milliseconds=200))
+            raise AssertionError("wait(timeout) did not time out")
+        except RuntimeError as e:
+            assert "Caught collective operation timeout" in str(e), str(e)
+    w.wait(datetime.timedelta(seconds=20))
+    assert w.is_completed() and w.is_success()
+    assert float(t[0]) == float(world * world) and float(t[-1]) == float(world * world)
+    # a receive honours its timeout too
+    if rank == 0:
+        r = pg.recv([torch.zeros(4, device=DEV)], 1, 0)
+        t0 = time.time()
+        try:
+            r.wait(datetime.timedelta(milliseconds=300))
+            raise AssertionError("recv wait(timeout) did not time out")
+        except RuntimeError as e:
+            assert "timed out waiting for a message" in str(e), str(e)
+        assert time.time() - t0 < 5.0
+    else:
+        time.sleep(1.0)  # stay in the group while rank 0 waits: it must run into its own limit
+
+
 def missing_sender_case(pg, rank, world):
     """Rank 0 posts a receive for a message rank 1 never sends: the wait must raise, not hang; a
     mismatched size raises on the receiver as well."""
@@ -786,6 +941,12 @@ def run_rank(rank, world, store_path, mode):
         missing_rank_case(pg, rank, world)
     elif mode == "missing_sender":
         missing_sender_case(pg, rank, world)
+    elif mode == "zero_copy":
+        zero_copy_cases(pg, rank, world)
+    elif mode == "missing_device":
+        missing_rank_device_case(pg, rank, world)
+    elif mode == "late_peer":
+        late_peer_case(pg, rank, world)
     else:
         raise ValueError(mode)
     torch.cuda.synchronize()

@@ -88,7 +88,40 @@ def test_missing_rank_raises_instead_of_hanging(monkeypatch):
     """Failure handling forced from the host: a rank skips a collective; the host barrier of the
     others gives up after the (shortened) limit and raises.  No kernel waits on the GPU."""
     monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    monkeypatch.setenv("MCCL_PG_SYNC", "host")
     _spawn(3, "missing")
+
+
+@pytest.mark.parametrize("blocking", ["0", "1"])
+def test_missing_rank_with_device_side_waits(monkeypatch, blocking):
+    """The same failure with the cross-rank wait on the device: the kernel's own bounded wait ends
+    it (a 1.5 s limit forced from the host), the Work reports failure, the group refuses to go on."""
+    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
+    _spawn(3, "missing_device")
+
+
+def test_wait_honours_its_timeout(monkeypatch):
+    monkeypatch.setenv("CCL_BLOCKING_WAIT", "1")
+    _spawn(3, "late_peer")
+
+
+@pytest.mark.parametrize("world", [2, 8])
+def test_zero_copy_collectives(world):
+    _spawn(world, "zero_copy")
+
+
+@pytest.mark.parametrize("world,mode", [(2, "reference"), (4, "oracle"), (3, "p2p"), (4, "dist"), (2, "zero_copy")])
+def test_host_synchronised_fallback(monkeypatch, world, mode):
+    """MCCL_PG_SYNC=host: the same cases with hipStreamSynchronize + the host barrier instead of
+    device-side waits (what ranks that share a process always use)."""
+    monkeypatch.setenv("MCCL_PG_SYNC", "host")
+    _spawn(world, mode)
+
+
+def test_staged_when_zero_copy_is_switched_off(monkeypatch):
+    monkeypatch.setenv("MCCL_PG_ZERO_COPY", "0")
+    _spawn(4, "oracle")
 
 
 def test_receive_without_a_sender_raises_instead_of_hanging(monkeypatch):

@@ -48,6 +48,24 @@ constexpr size_t kInlineStreamMax = 1u << 20;
 // algorithm for W GPUs on xGMI, where each shard is reduced by the GPU that owns it.
 constexpr size_t kTwoShotMinBytes = 4u << 20;
 constexpr int kTwoShotMinRanks = 4;
+// Device-synchronised groups: allreduces of at most this many bytes (and at most
+// MCCL_FUSED_MAX_RANKS ranks) are one launch of mccl_allreduce_fused on the caller's stream.
+constexpr size_t kFusedMaxBytes = 1u << 20;
+// Tensors of at least this many bytes are offered to the peers in place (zero-copy) instead of
+// being staged; an allocation must stay below 2 GiB to be shared between processes.
+constexpr size_t kZeroCopyMinBytes = 1u << 20;
+constexpr uint64_t kShareMaxAllocation = (2ull << 30) - (64u << 20);
+constexpr int kMaxExports = 32;
+constexpr int kEmptyShare = kMaxExports;  // "this rank's range is empty": nothing to map
+// Layout of a rank's arena (device memory mapped by every peer at start-up).
+constexpr size_t kArenaBarOff = 0;        // 64-bit barrier word
+constexpr size_t kArenaFinalOff = 128;    // 64-bit departure word
+constexpr size_t kArenaFusedFlagsOff = 4096;                 // two sets of tile flags, 8 KiB each
+constexpr size_t kArenaFusedFlagsStride = 8192;
+constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buffers of 1 MiB, each
+constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
+constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
+static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
 
 #define HIP_CHECK(expr)                                                                     \
   do {                                                                                      \
@@ -161,16 +179,35 @@ struct alignas(64) P2PBox {
 
 struct alignas(128) RankSlot {
   std::atomic<uint64_t> arrive;  // host barrier: epoch this rank has reached
+  std::atomic<uint64_t> entered;  // collectives this rank's host thread has entered (device-synchronised groups)
   std::atomic<uint64_t> failed;  // non-zero once the rank gave up; peers stop waiting
   std::atomic<uint64_t> departed;  // non-zero once the rank's group object is being destroyed
   int64_t pid;
-  // per staging slot; written by the owner before it arrives at the barrier of the collective
-  // that uses the slot, read by the peers after that barrier
-  uint64_t gen[2];
-  uint64_t ptr[2];
-  uint64_t capacity[2];
-  hipIpcMemHandle_t handle[2];
-  int64_t table[2][kTableMax];
+  // What the rank tells its peers for one collective: written before it arrives at the host
+  // rendezvous of that collective, read by the peers after it.  Two records alternate, counted in
+  // collectives that rendezvous: a rank can only be one rendezvous ahead of the slowest reader
+  // (it cannot pass the next rendezvous before everybody has arrived there, i.e. is done reading).
+  struct Published {
+    uint64_t stage_gen;            // the staging buffer of the device slot this collective uses
+    uint64_t stage_ptr;
+    hipIpcMemHandle_t stage_handle;
+    // zero-copy offer: entry of `exports` (< 0: cannot share; kEmptyShare: empty range), its
+    // generation, and where the offered range starts inside the allocation
+    int64_t share_entry;
+    uint64_t share_gen;
+    uint64_t share_off;
+    int64_t table[kTableMax];      // per-collective scalars (split sizes, displacements)
+  } pub[2];
+  // device-side synchronisation: the rank's arena (flag words, fused-allreduce staging)
+  uint64_t arena_ptr;
+  hipIpcMemHandle_t arena_handle;
+  // zero-copy: allocations of this rank the peers may map
+  struct ExportEntry {
+    std::atomic<uint64_t> gen;  // bumped whenever the entry changes or its allocation is freed
+    uint64_t base;
+    uint64_t size;
+    hipIpcMemHandle_t handle;
+  } exports[kMaxExports];
   P2PBox p2p[kMaxWorld];
 };
 
@@ -183,16 +220,63 @@ struct Control {
 static_assert(std::atomic<uint64_t>::is_always_lock_free, "barrier counters must be lock-free");
 
 // ---------------------------------------------------------------------------------------------
+// what a group shares with its Works
+// ---------------------------------------------------------------------------------------------
+hipEvent_t GroupShared::getEvent() {
+  {
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!free_events.empty()) {
+      hipEvent_t e = free_events.back();
+      free_events.pop_back();
+      return e;
+    }
+  }
+  hipEvent_t e = nullptr;
+  HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  return e;
+}
+
+void GroupShared::putEvent(hipEvent_t e) {
+  std::lock_guard<std::mutex> lock(mutex);
+  free_events.push_back(e);
+}
+
+std::string GroupShared::failureMessage() {
+  if (status && status[0] != 0 && !failed.load(std::memory_order_acquire)) {
+    std::ostringstream os;
+    os << "ccl backend: timed out waiting for rank " << (status[0] - 1)
+       << " on the device (cross-rank wait of a collective); the group cannot be used any more";
+    fail(os.str());
+  }
+  if (!failed.load(std::memory_order_acquire)) return std::string();
+  std::lock_guard<std::mutex> lock(mutex);
+  return failure;
+}
+
+void GroupShared::fail(const std::string& why) {
+  std::lock_guard<std::mutex> lock(mutex);
+  if (failure.empty()) failure = why;
+  failed.store(true, std::memory_order_release);
+}
+
+GroupShared::~GroupShared() {
+  for (hipEvent_t e : free_events) (void)hipEventDestroy(e);
+  if (status) (void)hipHostFree((void*)status);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Work
 // ---------------------------------------------------------------------------------------------
 ProcessGroupCCL::WorkCCL::WorkCCL(int rank, c10d::OpType op, const char* title,
                                   std::vector<at::Tensor> inputs, std::vector<at::Tensor> outputs,
                                   bool blocking_wait)
-    : c10d::Work(rank, op, title), blocking_wait_(blocking_wait), inputs_(std::move(inputs)),
-      outputs_(std::move(outputs)) {}
+    : c10d::Work(rank, op, title), start_(std::chrono::steady_clock::now()), blocking_wait_(blocking_wait),
+      inputs_(std::move(inputs)), outputs_(std::move(outputs)) {}
 
 ProcessGroupCCL::WorkCCL::~WorkCCL() {
-  if (end_) (void)hipEventDestroy(end_);
+  if (!end_) return;
+  if (shared_) shared_->putEvent(end_);  // a recycled event is only ever re-recorded: safe while pending
+  else (void)hipEventDestroy(end_);
 }
 
 bool ProcessGroupCCL::WorkCCL::isCompleted() {
@@ -200,22 +284,48 @@ bool ProcessGroupCCL::WorkCCL::isCompleted() {
   return hipEventQuery(end_) == hipSuccess;
 }
 
-bool ProcessGroupCCL::WorkCCL::isSuccess() const { return true; }
+bool ProcessGroupCCL::WorkCCL::isSuccess() const {
+  return !shared_ || shared_->failureMessage().empty();
+}
 
-void ProcessGroupCCL::WorkCCL::synchronize() {
-  if (!end_) return;
-  if (blocking_wait_) {
-    HIP_CHECK(hipEventSynchronize(end_));
-  } else {
-    // stream-ordered: the caller's current stream waits for the collective (the queue barrier
-    // of src/gpu/dpcpp_ccl.cpp:440-457)
-    hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
-    HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+std::exception_ptr ProcessGroupCCL::WorkCCL::exception() const {
+  if (!shared_) return nullptr;
+  const std::string why = shared_->failureMessage();
+  if (why.empty()) return nullptr;
+  return std::make_exception_ptr(std::runtime_error(why));
+}
+
+void ProcessGroupCCL::WorkCCL::waitInternal(std::chrono::milliseconds timeout) {
+  if (end_) {
+    if (blocking_wait_) {
+      // synchronizeInternal of the reference (src/utils.h:295-319): poll until done or timed out
+      const std::chrono::milliseconds limit = timeout == kNoTimeout ? op_timeout_ : timeout;
+      unsigned spins = 0;
+      while (hipEventQuery(end_) != hipSuccess) {
+        if (limit.count() > 0) {
+          const auto ran = std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now() - start_);
+          TORCH_CHECK(ran < limit, "[Rank ", rank_, "] Caught collective operation timeout:  ran for ", ran.count(),
+                      " milliseconds before timing out.");
+        }
+        if (++spins > 200) std::this_thread::sleep_for(std::chrono::microseconds(50));
+      }
+    } else {
+      // stream-ordered: the caller's current stream waits for the collective (the queue barrier
+      // of src/gpu/dpcpp_ccl.cpp:440-457)
+      hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
+      HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+    }
+  }
+  if (shared_) {
+    const std::string why = shared_->failureMessage();
+    TORCH_CHECK(why.empty(), why);
   }
 }
 
-bool ProcessGroupCCL::WorkCCL::wait(std::chrono::milliseconds /*timeout*/) {
-  synchronize();
+void ProcessGroupCCL::WorkCCL::synchronize() { waitInternal(kNoTimeout); }
+
+bool ProcessGroupCCL::WorkCCL::wait(std::chrono::milliseconds timeout) {
+  waitInternal(timeout);
   return true;
 }
 
@@ -226,6 +336,10 @@ c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupCCL::WorkCCL::getFuture() {
     std::vector<c10::Device> devs;
     if (end_) devs.emplace_back(at::kCUDA, (c10::DeviceIndex)device_);
     future_ = c10::make_intrusive<at::ivalue::Future>(c10::ListType::create(c10::TensorType::get()), devs);
+    if (auto err = exception()) {  // finishAsyncWorkCCLError of the reference: the future carries the error
+      future_->setError(err);
+      return future_;
+    }
     if (end_) {
       c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
       hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
@@ -241,6 +355,30 @@ c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupCCL::WorkCCL::getFuture() {
 // ---------------------------------------------------------------------------------------------
 // construction, rendezvous, staging
 // ---------------------------------------------------------------------------------------------
+namespace {
+
+// Groups that have exported allocations to their peers, for the allocator's segment-free
+// notification.  The tracker is attached once per process and never detached (torch offers no way
+// to), so it only touches groups that are still registered here.
+std::mutex g_registry_mutex;
+std::vector<ProcessGroupCCL*> g_registry;
+std::once_flag g_tracker_once;
+
+void attachSegmentTracker() {
+  std::call_once(g_tracker_once, [] {
+    c10::hip::HIPCachingAllocator::attachAllocatorTraceTracker([](const c10::hip::HIPCachingAllocator::TraceEntry& te) {
+      if (te.action_ != c10::hip::HIPCachingAllocator::TraceEntry::SEGMENT_FREE &&
+          te.action_ != c10::hip::HIPCachingAllocator::TraceEntry::SEGMENT_UNMAP)
+        return;
+      // called under the allocator's lock: flags only, no HIP and no torch calls
+      std::lock_guard<std::mutex> lock(g_registry_mutex);
+      for (ProcessGroupCCL* pg : g_registry) pg->segmentFreed((uint64_t)te.addr_);
+    });
+  });
+}
+
+}  // namespace
+
 ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
                                  std::chrono::milliseconds timeout)
     : c10d::Backend(rank, size), store_(store), timeout_(timeout) {
@@ -251,6 +389,8 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   blocking_wait_ = envFlag("CCL_BLOCKING_WAIT", false);
   verbose_ = envFlag("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", false);
   profile_ = envFlag("MCCL_PG_PROFILE", false);
+  if (const char* v = std::getenv("MCCL_PG_SYNC")) want_device_sync_ = std::string(v) != "host";
+  zero_copy_ = envFlag("MCCL_PG_ZERO_COPY", true);
   // The staging window can be shrunk (never enlarged) so that tests reach every windowed path
   // with small tensors.
   stage_max_ = kStageMaxDefault;
@@ -258,6 +398,7 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
     const long long b = std::atoll(v);
     if (b >= 4096 && (size_t)b < kStageMaxDefault) stage_max_ = (size_t)b & ~(size_t)4095;
   }
+  shared_ = std::make_shared<GroupShared>();
 }
 
 c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_ptr<c10d::Store>& store,
@@ -267,35 +408,51 @@ c10::intrusive_ptr<c10d::Backend> ProcessGroupCCL::create(const c10::intrusive_p
 }
 
 ProcessGroupCCL::~ProcessGroupCCL() {
+  {
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    g_registry.erase(std::remove(g_registry.begin(), g_registry.end(), this), g_registry.end());
+  }
   if (profile_ && !phase_us_[0].empty()) {
     // medians: the first calls of a group pay for allocations and peer mappings
     std::ostringstream os;
     os << "ccl backend rank " << rank_ << ": " << phase_us_[0].size() << " collectives with a payload, median us per phase:";
-    const char* names[4] = {" copy-in enqueue ", ", stream synchronise ", ", host barrier ", ", kernel enqueue "};
+    const char* names[4] = {" copy-in enqueue ", device_sync_ ? ", host rendezvous " : ", stream synchronise ",
+                            device_sync_ ? ", barrier enqueue " : ", host barrier ", ", kernel enqueue "};
     for (int i = 0; i < 4; ++i) {
       auto& v = phase_us_[i];
+      if (v.empty()) continue;
       std::nth_element(v.begin(), v.begin() + (long)(v.size() / 2), v.end());
       os << names[i] << v[v.size() / 2];
     }
     std::cerr << os.str() << std::endl;
   }
   if (!initialised_) return;
-  // Peers may still be reading this rank's staging buffers in their last kernel: wait for our own
-  // stream, then give the others a bounded chance to catch up.  A peer that is already gone has
+  // Peers may still be reading this rank's buffers in their last kernels: wait for our own
+  // streams, then give the others a bounded chance to catch up.  A peer that is already gone has
   // finished its kernels, so a timeout here is harmless.
   (void)hipSetDevice(device_);
   if (comm_stream_) (void)hipStreamSynchronize(comm_stream_);
+  if (tail_pending_) (void)hipEventSynchronize(tail_event_);
   // Leaving never advances the barrier epoch (a rank that leaves early must not satisfy its
-  // peers' next barrier); it raises a flag instead.  A peer is done with this rank's buffers
-  // once it has left too or has arrived at a later collective.
+  // peers' next barrier); it raises a flag instead.
   ctl_->slot[rank_].departed.store(1, std::memory_order_release);
-  const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(2000);
-  for (int r = 0; r < size_; ++r) {
-    if (r == rank_) continue;
-    while (!ctl_->slot[r].departed.load(std::memory_order_acquire) &&
-           ctl_->slot[r].arrive.load(std::memory_order_acquire) <= barrier_epoch_ &&
-           std::chrono::steady_clock::now() < deadline)
-      sched_yield();
+  if (device_sync_ && size_ > 1) {
+    // The departure barrier: its own flag word, so that it can never be mistaken for a collective.
+    // Once it has passed (or its 2 s are over) every peer that leaves too has drained its stream.
+    if (shared_->failureMessage().empty()) {
+      (void)mccl_rank_barrier(final_flags_.data(), size_, rank_, 1, 2000000, nullptr, comm_stream_);
+      (void)hipStreamSynchronize(comm_stream_);
+    }
+  } else {
+    // A peer is done with this rank's buffers once it has left too or has arrived at a later collective.
+    const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(2000);
+    for (int r = 0; r < size_; ++r) {
+      if (r == rank_) continue;
+      while (!ctl_->slot[r].departed.load(std::memory_order_acquire) &&
+             ctl_->slot[r].arrive.load(std::memory_order_acquire) <= barrier_epoch_ &&
+             std::chrono::steady_clock::now() < deadline)
+        sched_yield();
+    }
   }
   // Messages this rank has sent and nobody has copied out yet live in its staging buffers: give
   // the receivers a bounded time, then flag the failure so that a late receiver raises instead of
@@ -315,6 +472,7 @@ ProcessGroupCCL::~ProcessGroupCCL() {
     }
   }
   (void)hipDeviceSynchronize();
+  closeImports();
   for (auto& pr : p2p_recv_)
     for (int i = 0; i < kP2PRing; ++i)
       if (pr.ipc[i] && pr.base[i]) (void)hipIpcCloseMemHandle(pr.base[i]);
@@ -324,9 +482,12 @@ ProcessGroupCCL::~ProcessGroupCCL() {
   for (auto& pm : peers_)
     for (int s = 0; s < 2; ++s)
       if (pm.ipc[s] && pm.base[s]) (void)hipIpcCloseMemHandle(pm.base[s]);
+  for (int r = 0; r < (int)peer_arena_.size(); ++r)
+    if (r != rank_ && peer_arena_[(size_t)r]) (void)hipIpcCloseMemHandle(peer_arena_[(size_t)r]);
   for (int s = 0; s < 2; ++s)
     if (stage_[s].base) (void)hipFree(stage_[s].base);
   for (void* p : retired_) (void)hipFree(p);
+  if (arena_) (void)hipFree(arena_);
   if (fork_event_) (void)hipEventDestroy(fork_event_);
   if (tail_event_) (void)hipEventDestroy(tail_event_);
   if (ctl_) munmap(ctl_, ctl_bytes_);
@@ -339,6 +500,7 @@ void ProcessGroupCCL::ensureInit(int device) {
     return;
   }
   device_ = device;
+  shared_->device = device;
   HIP_CHECK(hipSetDevice(device_));
   comm_stream_ = c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, (c10::DeviceIndex)device_).stream();
   HIP_CHECK(hipEventCreateWithFlags(&fork_event_, hipEventDisableTiming));
@@ -372,17 +534,80 @@ void ProcessGroupCCL::ensureInit(int device) {
     ctl_->world = (uint32_t)size_;
     store_->set(key, std::vector<uint8_t>(shm_name_.begin(), shm_name_.end()));
   }
-  ctl_->slot[rank_].pid = (int64_t)getpid();
+  RankSlot& me = ctl_->slot[rank_];
+  me.pid = (int64_t)getpid();
   peers_.assign((size_t)size_, PeerMap{});
   p2p_send_.assign((size_t)size_, P2PSend{});
   p2p_recv_.assign((size_t)size_, P2PRecv{});
+  exports_.assign((size_t)kMaxExports, Export{});
+  imports_.assign((size_t)size_, std::vector<Import>((size_t)kMaxExports));
   initialised_ = true;
   for (int s = 0; s < 2; ++s) ensureStage(s, std::min(kStageMin, stage_max_));
+
+  // The arena: flag words and the buffers of the one-launch allreduce, zeroed, published before the
+  // start-up barrier and mapped by everybody right after it.
+  if (size_ > 1) {
+    HIP_CHECK(hipMalloc(&arena_, kArenaBytes));
+    HIP_CHECK(hipMemset(arena_, 0, kArenaBytes));
+    HIP_CHECK(hipDeviceSynchronize());
+    HIP_CHECK(hipIpcGetMemHandle(&me.arena_handle, arena_));
+    me.arena_ptr = (uint64_t)(uintptr_t)arena_;
+    void* host_status = nullptr;
+    HIP_CHECK(hipHostMalloc(&host_status, 64, hipHostMallocMapped));
+    std::memset(host_status, 0, 64);
+    shared_->status = static_cast<volatile uint32_t*>(host_status);
+    HIP_CHECK(hipHostGetDevicePointer(&status_dev_, host_status, 0));
+  }
 
   hostBarrier(/*start_up=*/true);
   TORCH_CHECK(ctl_->magic == kMagic && ctl_->world == (uint32_t)size_,
               "ccl backend: control block mismatch (ranks disagree on the world size)");
   if (rank_ == 0) shm_unlink(shm_name_.c_str());  // every rank holds a mapping now
+
+  // Device-side waits need ranks whose kernels can never queue up behind each other: processes of
+  // their own.  Every rank sees the same pid table, so the decision is the same everywhere (the
+  // environment switch has to agree across ranks like any other setting of the group).
+  bool distinct = true;
+  for (int a = 0; a < size_; ++a)
+    for (int b = a + 1; b < size_; ++b)
+      if (ctl_->slot[a].pid == ctl_->slot[b].pid) distinct = false;
+  device_sync_ = size_ > 1 && distinct && want_device_sync_;
+  if (size_ > 1) {
+    peer_arena_.assign((size_t)size_, nullptr);
+    bar_flags_.assign((size_t)size_, nullptr);
+    final_flags_.assign((size_t)size_, nullptr);
+    for (int sl = 0; sl < 2; ++sl) {
+      fused_stage_[sl].assign((size_t)size_, nullptr);
+      fused_flags_[sl].assign((size_t)size_, nullptr);
+    }
+    for (int r = 0; r < size_; ++r) {
+      char* base = nullptr;
+      if (r == rank_) {
+        base = static_cast<char*>(arena_);
+      } else if (ctl_->slot[r].pid == (int64_t)getpid()) {
+        base = (char*)(uintptr_t)ctl_->slot[r].arena_ptr;
+      } else {
+        void* p = nullptr;
+        HIP_CHECK(hipIpcOpenMemHandle(&p, ctl_->slot[r].arena_handle, hipIpcMemLazyEnablePeerAccess));
+        base = static_cast<char*>(p);
+      }
+      peer_arena_[(size_t)r] = (ctl_->slot[r].pid == (int64_t)getpid()) ? nullptr : base;  // what gets closed
+      bar_flags_[(size_t)r] = base + kArenaBarOff;
+      final_flags_[(size_t)r] = base + kArenaFinalOff;
+      for (int sl = 0; sl < 2; ++sl) {
+        fused_flags_[sl][(size_t)r] = base + kArenaFusedFlagsOff + (size_t)sl * kArenaFusedFlagsStride;
+        fused_stage_[sl][(size_t)r] = base + kArenaFusedStageOff + (size_t)sl * kArenaFusedStageStride + stageOffset(r);
+      }
+    }
+    peer_arena_[(size_t)rank_] = nullptr;
+    // nobody starts a collective before everybody has mapped everything
+    hostBarrier(/*start_up=*/true);
+  }
+  if (device_sync_ && zero_copy_) {
+    attachSegmentTracker();
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    g_registry.push_back(this);
+  }
 }
 
 void* ProcessGroupCCL::ensureStage(int slot, size_t bytes) {
@@ -397,40 +622,151 @@ void* ProcessGroupCCL::ensureStage(int slot, size_t bytes) {
   st.base = base;
   st.ptr = static_cast<char*>(base) + stageOffset(rank_);
   st.capacity = cap;
-  RankSlot& me = ctl_->slot[rank_];
-  if (size_ > 1) HIP_CHECK(hipIpcGetMemHandle(&me.handle[slot], base));
-  me.ptr[slot] = (uint64_t)(uintptr_t)st.ptr;
-  me.capacity[slot] = cap;
-  me.gen[slot] += 1;
+  if (size_ > 1) HIP_CHECK(hipIpcGetMemHandle(&st.handle, base));
+  st.gen += 1;
   return st.ptr;
 }
 
-const void* ProcessGroupCCL::peerStage(int peer, int slot) {
+// Copies what the peers need to know of this rank's staging buffer `slot` into the record of the
+// current collective.
+void ProcessGroupCCL::publishStage(int slot, int pub) {
+  RankSlot::Published& rec = ctl_->slot[rank_].pub[pub];
+  rec.stage_gen = stage_[slot].gen;
+  rec.stage_ptr = (uint64_t)(uintptr_t)stage_[slot].ptr;
+  rec.stage_handle = stage_[slot].handle;
+}
+
+void ProcessGroupCCL::quiesce() {
+  if (tail_pending_) HIP_CHECK(hipEventSynchronize(tail_event_));
+}
+
+const void* ProcessGroupCCL::peerStage(int peer, int slot, int pub) {
   if (peer == rank_) return stage_[slot].ptr;
+  const RankSlot::Published& rec = ctl_->slot[peer].pub[pub];
   const RankSlot& rs = ctl_->slot[peer];
   PeerMap& pm = peers_[(size_t)peer];
-  if (pm.gen[slot] != rs.gen[slot]) {
-    if (pm.ipc[slot] && pm.base[slot]) (void)hipIpcCloseMemHandle(pm.base[slot]);
+  if (pm.gen[slot] != rec.stage_gen) {
+    if (pm.ipc[slot] && pm.base[slot]) {
+      quiesce();  // earlier kernels of this rank may still read through the old mapping
+      (void)hipIpcCloseMemHandle(pm.base[slot]);
+    }
     pm.ptr[slot] = nullptr;
     pm.base[slot] = nullptr;
     pm.ipc[slot] = false;
     if (rs.pid == (int64_t)getpid()) {
-      pm.ptr[slot] = (void*)(uintptr_t)rs.ptr[slot];  // a thread of this process: same address space
+      pm.ptr[slot] = (void*)(uintptr_t)rec.stage_ptr;  // a thread of this process: same address space
     } else {
       void* p = nullptr;
-      HIP_CHECK(hipIpcOpenMemHandle(&p, rs.handle[slot], hipIpcMemLazyEnablePeerAccess));
+      HIP_CHECK(hipIpcOpenMemHandle(&p, rec.stage_handle, hipIpcMemLazyEnablePeerAccess));
       pm.base[slot] = p;
       pm.ptr[slot] = static_cast<char*>(p) + stageOffset(peer);
       pm.ipc[slot] = true;
     }
-    pm.gen[slot] = rs.gen[slot];
+    pm.gen[slot] = rec.stage_gen;
   }
   return pm.ptr[slot];
 }
 
-void ProcessGroupCCL::hostBarrier(bool start_up) {
-  const uint64_t epoch = ++barrier_epoch_;
-  ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
+// ---------------------------------------------------------------------------------------------
+// zero-copy: exporting the caller's allocation, importing the peers'
+// ---------------------------------------------------------------------------------------------
+void ProcessGroupCCL::segmentFreed(uint64_t base) {
+  // g_registry_mutex is held; the allocator's lock too.  The entry stays in the table (its handle
+  // is dead) until it is evicted; the generation tells the peers to drop their mapping.
+  if (!ctl_) return;
+  for (int i = 0; i < kMaxExports; ++i) {
+    if (exports_[(size_t)i].valid && exports_[(size_t)i].base == base) {
+      exports_[(size_t)i].valid = false;
+      ctl_->slot[rank_].exports[i].gen.fetch_add(1, std::memory_order_release);
+    }
+  }
+}
+
+// Publishes the allocation that holds [ptr, ptr + bytes) and returns its entry in this rank's
+// export table (or -1 when it cannot be shared: not an allocation of torch's caching allocator,
+// 2 GiB or more, or refused by the runtime).  *offset = where ptr lies inside it.
+int ProcessGroupCCL::exportRange(const void* ptr, size_t bytes, uint64_t* offset) {
+  if (!bytes) return kEmptyShare;  // nothing to read: trivially shareable
+  if (!zero_copy_ || !ptr) return -1;
+  // Only allocations whose release this group gets to hear of (the allocator's segment-free
+  // notification) are shared: a cached mapping of anything else could go stale unnoticed.
+  void* base = nullptr;
+  size_t size = 0;
+  try {
+    base = c10::hip::HIPCachingAllocator::getBaseAllocation(const_cast<void*>(ptr), &size);
+  } catch (const c10::Error&) {
+    return -1;
+  }
+  if (!base || size >= kShareMaxAllocation) return -1;
+  const uint64_t off = (uint64_t)((const char*)ptr - (const char*)base);
+  if (off + bytes > size) return -1;
+  RankSlot& me = ctl_->slot[rank_];
+  std::lock_guard<std::mutex> lock(g_registry_mutex);
+  int idx = -1;
+  for (int i = 0; i < kMaxExports; ++i)
+    if (exports_[(size_t)i].valid && exports_[(size_t)i].base == (uint64_t)(uintptr_t)base &&
+        exports_[(size_t)i].size == size) { idx = i; break; }
+  if (idx < 0) {
+    hipIpcMemHandle_t h;
+    if (hipIpcGetMemHandle(&h, base) != hipSuccess) {
+      (void)hipGetLastError();  // e.g. memory of an expandable segment: not shareable
+      return -1;
+    }
+    for (int i = 0; i < kMaxExports && idx < 0; ++i)
+      if (!exports_[(size_t)i].valid) idx = i;  // a never-used entry, or one whose allocation is gone
+    while (idx < 0) {
+      // evict round robin, but never an entry of the last two offers: a slow peer may still be
+      // opening it
+      const int victim = export_clock_;
+      export_clock_ = (export_clock_ + 1) % kMaxExports;
+      if (victim != recent_export_[0] && victim != recent_export_[1]) idx = victim;
+    }
+    me.exports[idx].gen.fetch_add(1, std::memory_order_release);
+    me.exports[idx].base = (uint64_t)(uintptr_t)base;
+    me.exports[idx].size = size;
+    me.exports[idx].handle = h;
+    exports_[(size_t)idx] = Export{(uint64_t)(uintptr_t)base, size, true};
+  }
+  *offset = off;
+  recent_export_[1] = recent_export_[0];
+  recent_export_[0] = idx;
+  return idx;
+}
+
+// The range rank `peer` offered in record `pub`, in this process's address space.  Call after the
+// rendezvous.
+const void* ProcessGroupCCL::importRange(int peer, int pub) {
+  const RankSlot& rs = ctl_->slot[peer];
+  const RankSlot::Published& rec = rs.pub[pub];
+  const int idx = (int)rec.share_entry;
+  if (idx == kEmptyShare) return nullptr;
+  TORCH_CHECK(idx >= 0 && idx < kMaxExports, "ccl backend: rank ", peer, " published no shareable range");
+  Import& im = imports_[(size_t)peer][(size_t)idx];
+  const uint64_t gen = rec.share_gen;
+  if (im.gen != gen || !im.base) {
+    if (im.base) {
+      quiesce();  // earlier kernels of this rank may still read through the old mapping
+      (void)hipIpcCloseMemHandle(im.base);
+      im.base = nullptr;
+    }
+    void* p = nullptr;
+    HIP_CHECK(hipIpcOpenMemHandle(&p, rs.exports[idx].handle, hipIpcMemLazyEnablePeerAccess));
+    im.base = p;
+    im.gen = gen;
+  }
+  return static_cast<const char*>(im.base) + rec.share_off;
+}
+
+void ProcessGroupCCL::closeImports() {
+  for (auto& per_peer : imports_)
+    for (auto& im : per_peer)
+      if (im.base) {
+        (void)hipIpcCloseMemHandle(im.base);
+        im.base = nullptr;
+      }
+}
+
+std::chrono::milliseconds ProcessGroupCCL::waitLimit(bool start_up) const {
   // Floor of 30 s under short user timeouts; MCCL_BARRIER_TIMEOUT_MS overrides it, e.g. to
   // exercise the failure path quickly.  The first barrier of a group waits for ranks that may
   // still be starting (a first import on a cold machine takes a minute): two minutes at least.
@@ -439,14 +775,23 @@ void ProcessGroupCCL::hostBarrier(bool start_up) {
     const long ms = std::atol(v);
     if (ms > 0) limit = std::chrono::milliseconds(ms);
   }
-  const auto deadline = std::chrono::steady_clock::now() + limit;
+  return limit;
+}
+
+void ProcessGroupCCL::hostBarrier(bool start_up) {
+  const uint64_t epoch = ++barrier_epoch_;
+  ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
+  const auto deadline = std::chrono::steady_clock::now() + waitLimit(start_up);
   for (int r = 0; r < size_; ++r) {
     unsigned spins = 0;
     while (ctl_->slot[r].arrive.load(std::memory_order_acquire) < epoch) {
-      if (ctl_->slot[r].failed.load(std::memory_order_acquire))
+      if (ctl_->slot[r].failed.load(std::memory_order_acquire)) {
+        shared_->fail(c10::str("ccl backend: rank ", r, " reported a failure; aborting the collective"));
         TORCH_CHECK(false, "ccl backend: rank ", r, " reported a failure; aborting the collective");
+      }
       if (ctl_->slot[r].departed.load(std::memory_order_acquire)) {
         ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+        shared_->fail(c10::str("ccl backend: rank ", r, " left the group before collective #", seq_));
         TORCH_CHECK(false, "ccl backend: rank ", r, " left the group before collective #", seq_);
       }
       if (++spins < 2000) continue;
@@ -458,14 +803,53 @@ void ProcessGroupCCL::hostBarrier(bool start_up) {
       sched_yield();
       if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) {
         ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+        shared_->fail(c10::str("ccl backend: timed out waiting for rank ", r, " at collective #", seq_));
         TORCH_CHECK(false, "ccl backend: timed out waiting for rank ", r, " at collective #", seq_);
       }
     }
   }
 }
 
+// A rank with posted receives must not park a waiting kernel on its stream while a peer is still
+// blocked in a send to it (the peer would never reach the collective, and the copy out of the
+// peer's buffers would queue up behind the waiting kernel).  So it first takes messages in until
+// every peer's host thread has entered this collective.  Ranks without posted receives only
+// announce themselves.
+void ProcessGroupCCL::awaitPeersEntered(uint64_t seq) {
+  ctl_->slot[rank_].entered.store(seq + 1, std::memory_order_release);
+  bool pending = false;
+  for (const auto& pr : p2p_recv_) pending = pending || !pr.pending.empty();
+  if (!pending) return;
+  const auto deadline = std::chrono::steady_clock::now() + waitLimit(false);
+  for (int r = 0; r < size_; ++r) {
+    unsigned spins = 0;
+    while (ctl_->slot[r].entered.load(std::memory_order_acquire) < seq + 1) {
+      if (ctl_->slot[r].failed.load(std::memory_order_acquire) || ctl_->slot[r].departed.load(std::memory_order_acquire))
+        return;  // the collective itself reports it
+      for (int src = 0; src < size_; ++src)
+        if (!p2p_recv_[(size_t)src].pending.empty()) progressRecvLocked(src, nullptr, /*blocking=*/false);
+      if (++spins < 64) continue;
+      sched_yield();
+      if ((spins & 0x3ff) == 0 && std::chrono::steady_clock::now() > deadline) return;
+    }
+  }
+}
+
+void ProcessGroupCCL::throwIfFailed() {
+  const std::string why = shared_->failureMessage();
+  if (why.empty()) return;
+  if (ctl_) ctl_->slot[rank_].failed.store(1, std::memory_order_release);
+  TORCH_CHECK(false, why);
+}
+
+// The device-side cross-rank barrier on `s` (the sync kernels of src/gpu/allreduce.h:731-769).
+void ProcessGroupCCL::deviceBarrier(uint64_t epoch, hipStream_t s) {
+  const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+  MCCL_CHECK(mccl_rank_barrier(bar_flags_.data(), size_, rank_, epoch, limit_us, status_dev_, s));
+}
+
 // ---------------------------------------------------------------------------------------------
-// the engine: copy-in, host barrier, data-path kernels
+// the engine: make the input visible to the peers, cross-rank barrier, data-path kernels
 // ---------------------------------------------------------------------------------------------
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   std::lock_guard<std::mutex> lock(mutex_);
@@ -476,16 +860,19 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device));
   ensureInit(device);
   TORCH_CHECK((int)plan.table.size() <= kTableMax, "ccl backend: too many tensors in one collective");
+  throwIfFailed();
 
   auto cur_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_);
   hipStream_t cur = cur_stream.stream();
-  const bool same_stream = same_stream_ || plan.stage_bytes <= kInlineStreamMax;
+  const size_t payload = std::max(plan.stage_bytes, plan.share ? plan.share_bytes : (size_t)0);
+  const bool same_stream = same_stream_ || payload <= kInlineStreamMax;
   hipStream_t s = same_stream ? cur : comm_stream_;
   if (!same_stream) {  // sync_streams of the reference (src/gpu/dpcpp_ccl.cpp:186-197)
     HIP_CHECK(hipEventRecord(fork_event_, cur));
     HIP_CHECK(hipStreamWaitEvent(comm_stream_, fork_event_, 0));
   }
 
+  const uint64_t seq = seq_;
   const int slot = (int)(seq_ & 1);
   ++seq_;
   if (verbose_) {
@@ -495,15 +882,27 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
     for (const auto& t : plan.outputs) os << " out" << t.sizes();
     std::cout << os.str() << std::endl;
   }
+  if (device_sync_) {
+    runDeviceSynced(plan, s, slot, seq);
+  } else {
+    runHostSynced(plan, s, slot);
+  }
+  return finishRun(plan, s, same_stream, /*device_work=*/true);
+}
 
+// Ranks that share a process (or MCCL_PG_SYNC=host): copy-in, hipStreamSynchronize, host barrier,
+// kernels.  No kernel ever waits for another rank.
+void ProcessGroupCCL::runHostSynced(Plan& plan, hipStream_t s, int slot) {
   RankSlot& me = ctl_->slot[rank_];
+  const int pub = slot;  // every collective meets at the host barrier: the records alternate with the slots
   using clk = std::chrono::steady_clock;
   auto us_since = [](clk::time_point t) { return std::chrono::duration<double, std::micro>(clk::now() - t).count(); };
   const bool timed = profile_ && plan.stage_bytes > 0 && phase_us_[0].size() < (1u << 20);
   auto t0 = clk::now();
   try {
     void* stage = ensureStage(slot, plan.stage_bytes);
-    for (size_t i = 0; i < plan.table.size(); ++i) me.table[slot][i] = plan.table[i];
+    publishStage(slot, pub);
+    for (size_t i = 0; i < plan.table.size(); ++i) me.pub[pub].table[i] = plan.table[i];
     if (plan.copy_in) plan.copy_in(stage, s);
     if (timed) { phase_us_[0].push_back((float)us_since(t0)); t0 = clk::now(); }
     // This rank's staging buffer must be complete before any peer reads it, and (two
@@ -523,34 +922,136 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
 
   if (plan.exec) {
-    std::vector<const void*> peer((size_t)size_);
-    std::vector<const int64_t*> tables((size_t)size_);
-    for (int r = 0; r < size_; ++r) {
-      peer[(size_t)r] = peerStage(r, slot);
-      tables[(size_t)r] = ctl_->slot[r].table[slot];
+    PeerView pv;
+    pv.stage.resize((size_t)size_);
+    pv.tables.resize((size_t)size_);
+    try {
+      for (int r = 0; r < size_; ++r) {
+        pv.stage[(size_t)r] = peerStage(r, slot, pub);
+        pv.tables[(size_t)r] = ctl_->slot[r].pub[pub].table;
+      }
+      plan.exec(pv, s);
+      if (plan.exec2 && (!plan.two_phase || plan.two_phase(pv))) HIP_CHECK(hipStreamSynchronize(s));
+    } catch (...) {
+      me.failed.store(1, std::memory_order_release);  // the peers must not wait for this rank at the next barrier
+      throw;
     }
-    plan.exec(peer, tables, s);
-    if (plan.exec2) {
+    if (plan.exec2 && (!plan.two_phase || plan.two_phase(pv))) {
+      hostBarrier();
       try {
-        HIP_CHECK(hipStreamSynchronize(s));
+        plan.exec2(pv, s);
       } catch (...) {
         me.failed.store(1, std::memory_order_release);
         throw;
       }
-      hostBarrier();
-      plan.exec2(peer, tables, s);
     }
   }
   if (timed) phase_us_[3].push_back((float)us_since(t0));
-  if (plan.exec) {
+}
+
+// Ranks that are processes of their own: everything a collective needs from its peers on the
+// device arrives through flag kernels on the collective's stream; the host only enqueues.  What
+// the host still exchanges -- tables of the v-collectives, new staging handles, the ranges offered
+// for zero-copy -- goes through the control block in a rendezvous of the host threads (no GPU
+// synchronisation); the one-launch allreduce needs none of it.
+//
+// Why one barrier per collective is enough to reuse the two alternating staging slots: the device
+// work of collective k contains a wait for every peer's START of its collective k (barrier flag
+// or tile flags), and a rank's collectives execute in order on the device.  So when this rank's
+// collective k + 1 has completed, every peer has started k + 1 and therefore finished k: slot
+// (k & 1) is free when this rank's collective k + 2 writes it.
+void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
+  RankSlot& me = ctl_->slot[rank_];
+  using clk = std::chrono::steady_clock;
+  auto us_since = [](clk::time_point t) { return std::chrono::duration<double, std::micro>(clk::now() - t).count(); };
+  const bool timed = profile_ && plan.stage_bytes > 0 && phase_us_[0].size() < (1u << 20);
+  auto t0 = clk::now();
+  const uint64_t epoch = 4 * seq;  // up to three barriers per collective: epoch + 1, + 2, + 3
+  try {
+    awaitPeersEntered(seq);
+    // a rank's collectives are totally ordered on the device, whichever streams they use
+    if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipStreamWaitEvent(s, tail_event_, 0));
+    if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS) {
+      const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+      MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
+                                      fused_stage_[slot].data(), fused_flags_[slot].data(), size_, rank_,
+                                      (uint32_t)(seq + 1), limit_us, status_dev_, s));
+      if (timed) phase_us_[3].push_back((float)us_since(t0));
+      return;
+    }
+    const bool candidate = zero_copy_ && plan.share;
+    // the record this collective publishes in: they alternate per collective that rendezvous
+    const int pub = (int)(rendezvous_count_++ & 1);
+    RankSlot::Published& rec = me.pub[pub];
+    for (size_t i = 0; i < plan.table.size(); ++i) rec.table[i] = plan.table[i];
+    void* stage = nullptr;
+    if (candidate) {
+      uint64_t off = 0;
+      const int entry = exportRange(plan.share_ptr, plan.share_bytes, &off);
+      rec.share_entry = entry;
+      rec.share_off = off;
+      rec.share_gen = (entry >= 0 && entry < kMaxExports) ? me.exports[entry].gen.load(std::memory_order_acquire) : 0;
+      stage = ensureStage(slot, plan.zero_copy_stage_bytes);
+    } else {
+      rec.share_entry = -1;
+      stage = ensureStage(slot, plan.stage_bytes);
+    }
+    publishStage(slot, pub);
+    if (timed) { phase_us_[0].push_back((float)us_since(t0)); t0 = clk::now(); }
+    hostBarrier();  // of the host threads only: tables, handles and offers are published
+    bool zero_copy = candidate;
+    if (candidate) {
+      for (int r = 0; r < size_; ++r)
+        if (ctl_->slot[r].pub[pub].share_entry < 0) zero_copy = false;
+      if (!zero_copy) {  // somebody cannot share: everybody stages (every rank sees the same offers)
+        stage = ensureStage(slot, plan.stage_bytes);
+        publishStage(slot, pub);  // nobody reads the staging part of a record before the second rendezvous
+        hostBarrier();
+      }
+    }
+    PeerView pv;
+    pv.stage.resize((size_t)size_);
+    pv.tables.resize((size_t)size_);
+    pv.zero_copy = zero_copy;
+    for (int r = 0; r < size_; ++r) {
+      pv.stage[(size_t)r] = peerStage(r, slot, pub);
+      pv.tables[(size_t)r] = ctl_->slot[r].pub[pub].table;
+    }
+    if (zero_copy) {
+      pv.user.resize((size_t)size_);
+      for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
+    }
+    if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
+    if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
+    deviceBarrier(epoch + 1, s);  // every rank's input is complete (staged, or ready in place)
+    if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
+    if (plan.exec) plan.exec(pv, s);
+    if (plan.exec2 && (!plan.two_phase || plan.two_phase(pv))) {
+      deviceBarrier(epoch + 2, s);
+      plan.exec2(pv, s);
+    }
+    // in place: nobody may touch its tensor again before every peer has read it
+    if (zero_copy) deviceBarrier(epoch + 3, s);
+    if (timed) phase_us_[3].push_back((float)us_since(t0));
+  } catch (...) {
+    // this rank may not have enqueued what its peers wait for: tell them now
+    me.failed.store(1, std::memory_order_release);
+    shared_->fail("ccl backend: a collective of this rank failed on the host; the group cannot be used any more");
+    throw;
+  }
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work) {
+  if (device_work) {
     HIP_CHECK(hipEventRecord(tail_event_, s));
     tail_stream_ = s;
     tail_pending_ = true;
   }
-
   auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
   work->device_ = device_;
-  HIP_CHECK(hipEventCreateWithFlags(&work->end_, hipEventDisableTiming));
+  work->shared_ = shared_;
+  work->op_timeout_ = timeout_;
+  work->end_ = shared_->getEvent();
   HIP_CHECK(hipEventRecord(work->end_, s));
   if (!same_stream) {  // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
     auto cs = c10::hip::getStreamFromExternalMasqueradingAsCUDA(comm_stream_, (c10::DeviceIndex)device_);
@@ -558,6 +1059,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
       for (const auto& t : *list)
         if (t.defined() && t.has_storage() && t.numel() > 0)
           c10::hip::HIPCachingAllocatorMasqueradingAsCUDA::recordStreamMasqueradingAsCUDA(t.storage().data_ptr(), cs);
+  }
+  if (plan.host_complete) {
+    // a barrier returns once every rank has arrived: the host waits for the flag kernel
+    work->blocking_wait_ = true;
+    work->waitInternal(kNoTimeout);
+    work->blocking_wait_ = blocking_wait_;
   }
   if (coalescing_) last_work_ = work;
   return work;
@@ -616,13 +1123,18 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
     p.inputs = {t};
     p.outputs = {t};
     p.stage_bytes = (rank_ == root) ? len : 0;
+    // large messages: the peers read the root's tensor in place (every rank offers its own tensor:
+    // the offer has to look the same on all ranks)
+    p.share = len >= kZeroCopyMinBytes;
+    p.share_ptr = base;
+    p.share_bytes = len;
     if (rank_ == root && len)
       p.copy_in = [=](void* stage, hipStream_t s) {
         copyAsync(stage, base, len, s);
       };
     if (rank_ != root && len)
-      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
-        mccl_segment_t seg{peer[(size_t)root], base, len};
+      p.exec = [=](const PeerView& pv, hipStream_t s) {
+        mccl_segment_t seg{pv.zero_copy ? pv.user[(size_t)root] : pv.stage[(size_t)root], base, len};
         MCCL_CHECK(mccl_copy_segments(&seg, 1, s));
       };
     work = run(p);
@@ -660,44 +1172,65 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // 16-byte boundary of the staging buffers whatever the element size; the last may be shorter
       const size_t shard = roundUp((len + (size_t)W - 1) / (size_t)W, 64);
       const bool two_shot = W >= kTwoShotMinRanks && len * es >= kTwoShotMinBytes;
+      auto shard_len = [=](int r) {
+        const size_t lo = std::min(len, (size_t)r * shard);
+        return std::min(len, lo + shard) - lo;
+      };
+      // Small messages between rank processes: one launch does copy-in, rank synchronisation and
+      // the N-peer sum (the reference's small allreduce, src/gpu/allreduce_small.h:166-361).
+      p.fused_ok = len * es <= kFusedMaxBytes;
+      p.fused_ptr = base;
+      p.fused_count = len;
+      p.fused_dtype = dtype;
+      p.fused_op = op;
+      // Large messages between rank processes: the peers read this tensor in place.  Rank r
+      // reduces shard r of all tensors into its staging buffer (nobody writes a tensor while
+      // anybody reads one), then all ranks gather the W finished shards into their tensors:
+      // about 3 S bytes per rank and no copy-in, against (4 + 1/W) S for the staged two-shot.
+      p.share = !p.fused_ok && len * es >= kZeroCopyMinBytes;
+      p.share_ptr = base;
+      p.share_bytes = len * es;
+      p.zero_copy_stage_bytes = shard * es;
+      p.stage_bytes = len * es;
       p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, base, len * es, s); };
-      if (!two_shot) {
-        p.stage_bytes = len * es;
-        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
-          // This rank's contribution is read from the tensor itself (its staging copy holds the
-          // same bytes), which makes the reduction in place: the output lands on DRAM pages the
-          // kernel has just read (5 % faster than a separate output on large messages).
-          std::vector<const void*> in = peer;
-          in[(size_t)me] = base;
-          MCCL_CHECK(mccl_reduce_n(in.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
-        };
-      } else {
-        // Rank r reduces shard r of all staged inputs in place in its own staging buffer: nobody
-        // else reads that range in this phase (rank k reads shard k of every buffer), the output
-        // lands on DRAM pages the kernel has just read, and after the second barrier shard r of
-        // staging buffer r is the finished shard.
-        p.stage_bytes = len * es;
-        auto shard_len = [=](int r) {
-          const size_t lo = std::min(len, (size_t)r * shard);
-          return std::min(len, lo + shard) - lo;
-        };
-        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+      p.two_phase = [=](const PeerView& pv) { return pv.zero_copy || two_shot; };
+      p.exec = [=](const PeerView& pv, hipStream_t s) {
+        if (pv.zero_copy) {
           const size_t n_me = shard_len(me);
           if (!n_me) return;
           std::vector<const void*> in((size_t)W);
-          for (int k = 0; k < W; ++k) in[(size_t)k] = (const char*)peer[(size_t)k] + (size_t)me * shard * es;
-          void* red = (char*)peer[(size_t)me] + (size_t)me * shard * es;  // peer[me] is this rank's own staging buffer
+          for (int k = 0; k < W; ++k) in[(size_t)k] = (const char*)pv.user[(size_t)k] + (size_t)me * shard * es;
+          MCCL_CHECK(mccl_reduce_n(in.data(), W, (void*)pv.stage[(size_t)me], n_me, dtype, op, MCCL_VARIANT_AUTO, s));
+        } else if (!two_shot) {
+          // This rank's contribution is read from the tensor itself (its staging copy holds the
+          // same bytes), which makes the reduction in place: the output lands on DRAM pages the
+          // kernel has just read (5 % faster than a separate output on large messages).
+          std::vector<const void*> in = pv.stage;
+          in[(size_t)me] = base;
+          MCCL_CHECK(mccl_reduce_n(in.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
+        } else {
+          // Rank r reduces shard r of all staged inputs in place in its own staging buffer: nobody
+          // else reads that range in this phase (rank k reads shard k of every buffer), the output
+          // lands on DRAM pages the kernel has just read, and after the second barrier shard r of
+          // staging buffer r is the finished shard.
+          const size_t n_me = shard_len(me);
+          if (!n_me) return;
+          std::vector<const void*> in((size_t)W);
+          for (int k = 0; k < W; ++k) in[(size_t)k] = (const char*)pv.stage[(size_t)k] + (size_t)me * shard * es;
+          void* red = (char*)pv.stage[(size_t)me] + (size_t)me * shard * es;  // pv.stage[me] is this rank's own staging buffer
           MCCL_CHECK(mccl_reduce_n(in.data(), W, red, n_me, dtype, op, MCCL_VARIANT_AUTO, s));
-        };
-        p.exec2 = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
-          std::vector<mccl_segment_t> segs;
-          for (int r = 0; r < W; ++r) {
-            const size_t n_r = shard_len(r);
-            if (n_r) segs.push_back({(const char*)peer[(size_t)r] + (size_t)r * shard * es, base + (size_t)r * shard * es, n_r * es});
-          }
-          MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
-        };
-      }
+        }
+      };
+      p.exec2 = [=](const PeerView& pv, hipStream_t s) {
+        // the finished shard of rank r: the start of its staging buffer (zero-copy) or shard r of it
+        std::vector<mccl_segment_t> segs;
+        for (int r = 0; r < W; ++r) {
+          const size_t n_r = shard_len(r);
+          const size_t at = pv.zero_copy ? 0 : (size_t)r * shard * es;
+          if (n_r) segs.push_back({(const char*)pv.stage[(size_t)r] + at, base + (size_t)r * shard * es, n_r * es});
+        }
+        MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+      };
     }
     work = run(p);
     off += len;
@@ -745,13 +1278,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce_coalesced(
         if (ts[i].numel()) segs.push_back({ts[i].data_ptr(), (char*)stage + offs[i], nbytes(ts[i])});
       MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
     };
-    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
       std::vector<const void*> in;
       std::vector<void*> out;
       std::vector<size_t> counts;
       for (size_t i = 0; i < ts.size(); ++i) {
         if (!ts[i].numel()) continue;
-        for (int k = 0; k < W; ++k) in.push_back((const char*)peer[(size_t)k] + offs[i]);
+        for (int k = 0; k < W; ++k) in.push_back((const char*)pv.stage[(size_t)k] + offs[i]);
         out.push_back(ts[i].data_ptr());
         counts.push_back((size_t)ts[i].numel());
       }
@@ -781,13 +1314,17 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
     p.outputs = {output};
     if (len) {
       p.stage_bytes = len;
+      p.share = len >= kZeroCopyMinBytes;  // large inputs are read in place by the peers
+      p.share_ptr = in;
+      p.share_bytes = len;
       const int W = size_;
       p.copy_in = [=](void* stage, hipStream_t s) {
         copyAsync(stage, in, len, s);
       };
-      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+      p.exec = [=](const PeerView& pv, hipStream_t s) {
         std::vector<mccl_segment_t> segs((size_t)W);
-        for (int r = 0; r < W; ++r) segs[(size_t)r] = {peer[(size_t)r], out + (size_t)r * per_rank, len};
+        for (int r = 0; r < W; ++r)
+          segs[(size_t)r] = {pv.zero_copy ? pv.user[(size_t)r] : pv.stage[(size_t)r], out + (size_t)r * per_rank, len};
         MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
       };
     }
@@ -844,12 +1381,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
     p.copy_in = [=](void* stage, hipStream_t s) {
       copyAsync(stage, input.data_ptr(), mine, s);
     };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
     for (int r = 0; r < W; ++r) {
-      const size_t b = (size_t)tables[(size_t)r][0];  // allgatherv: every rank announces its byte count
+      const size_t b = (size_t)pv.tables[(size_t)r][0];  // allgatherv: every rank announces its byte count
       TORCH_CHECK(b == nbytes(outs[(size_t)r]), "allgather: output tensor ", r, " does not match the size rank ", r, " sends");
-      if (b) segs.push_back({peer[(size_t)r], outs[(size_t)r].data_ptr(), b});
+      if (b) segs.push_back({pv.stage[(size_t)r], outs[(size_t)r].data_ptr(), b});
     }
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
@@ -895,13 +1432,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather_into_tensor_coalesced(
       if (ins[i].numel()) segs.push_back({ins[i].data_ptr(), (char*)stage + offs[i], nbytes(ins[i])});
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
     std::vector<mccl_segment_t> segs;
     for (size_t i = 0; i < ins.size(); ++i) {
       const size_t b = nbytes(ins[i]);
       if (!b) continue;
       for (int r = 0; r < W; ++r)
-        segs.push_back({(const char*)peer[(size_t)r] + offs[i], (char*)outs[i].data_ptr() + (size_t)r * b, b});
+        segs.push_back({(const char*)pv.stage[(size_t)r] + offs[i], (char*)outs[i].data_ptr() + (size_t)r * b, b});
     }
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
@@ -945,9 +1482,19 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
           MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
         }
       };
-      p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+      // large inputs are read in place by the peers: rank r reduces slice r of every rank's tensor
+      p.share = len * es * (size_t)W >= kZeroCopyMinBytes;
+      p.share_ptr = in;
+      p.share_bytes = M * es * (size_t)W;
+      p.exec = [=](const PeerView& pv, hipStream_t s) {
         void* o = out;
-        MCCL_CHECK(mccl_reduce_scatter_n(peer.data(), W, &o, len, me, 1, dtype, op, s));
+        if (pv.zero_copy) {
+          std::vector<const void*> src((size_t)W);
+          for (int k = 0; k < W; ++k) src[(size_t)k] = (const char*)pv.user[(size_t)k] + ((size_t)me * M + m0) * es;
+          MCCL_CHECK(mccl_reduce_n(src.data(), W, o, len, dtype, op, MCCL_VARIANT_AUTO, s));
+        } else {
+          MCCL_CHECK(mccl_reduce_scatter_n(pv.stage.data(), W, &o, len, me, 1, dtype, op, s));
+        }
       };
     }
     work = run(p);
@@ -1019,12 +1566,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
         segs.push_back({ins[(size_t)d].data_ptr(), (char*)stage + offs[(size_t)d], nbytes(ins[(size_t)d])});
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
     std::vector<const void*> in((size_t)W);
     for (int k = 0; k < W; ++k) {
-      TORCH_CHECK((size_t)tables[(size_t)k][W + me] == nbytes(out),
+      TORCH_CHECK((size_t)pv.tables[(size_t)k][W + me] == nbytes(out),
                   "reduce_scatter: rank ", k, "'s input for rank ", me, " does not match the output size");
-      in[(size_t)k] = (const char*)peer[(size_t)k] + tables[(size_t)k][me];
+      in[(size_t)k] = (const char*)pv.stage[(size_t)k] + pv.tables[(size_t)k][me];
     }
     if (out.numel())
       MCCL_CHECK(mccl_reduce_n(in.data(), W, out.data_ptr(), (size_t)out.numel(), dtype, op, MCCL_VARIANT_AUTO, s));
@@ -1071,14 +1618,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter_tensor_coalesced(
       if (ins[i].numel()) segs.push_back({ins[i].data_ptr(), (char*)stage + offs[i], nbytes(ins[i])});
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
-  p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
     std::vector<const void*> in;
     std::vector<void*> out;
     std::vector<size_t> counts;
     for (size_t i = 0; i < ins.size(); ++i) {
       if (!outs[i].numel()) continue;
       const size_t shard = nbytes(outs[i]);
-      for (int k = 0; k < W; ++k) in.push_back((const char*)peer[(size_t)k] + offs[i] + (size_t)me * shard);
+      for (int k = 0; k < W; ++k) in.push_back((const char*)pv.stage[(size_t)k] + offs[i] + (size_t)me * shard);
       out.push_back(outs[i].data_ptr());
       counts.push_back((size_t)outs[i].numel());
     }
@@ -1148,15 +1695,20 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
       p.table[(size_t)(W + d)] = (int64_t)send[(size_t)d];
     }
     p.table[(size_t)(2 * W)] = (int64_t)mine;
+    // The inputs differ in size from rank to rank, so the offer cannot depend on a size: every
+    // all-to-all offers its input, and the peers pull their segments out of it in place.
+    p.share = true;
+    p.share_ptr = mine ? input.data_ptr() : nullptr;
+    p.share_bytes = mine;
     if (wlen)
       p.copy_in = [=](void* stage, hipStream_t s) {
         copyAsync(stage, (const char*)input.data_ptr() + w0, wlen, s);
       };
-    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
       size_t largest = 0;
       std::vector<mccl_segment_t> segs;
       for (int r = 0; r < W; ++r) {
-        const int64_t* tr = tables[(size_t)r];
+        const int64_t* tr = pv.tables[(size_t)r];
         TORCH_CHECK((size_t)tr[W + me] == recv[(size_t)r],
                     "alltoall_base: rank ", r, " sends ", tr[W + me], " bytes to rank ", me,
                     " which expects ", recv[(size_t)r]);
@@ -1165,7 +1717,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
         const size_t seg0 = (size_t)tr[me], seg1 = seg0 + recv[(size_t)r];
         const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w0 + window);
         if (lo < hi)
-          segs.push_back({(const char*)peer[(size_t)r] + (lo - w0),
+          segs.push_back({pv.zero_copy ? (const char*)pv.user[(size_t)r] + lo : (const char*)pv.stage[(size_t)r] + (lo - w0),
                           (char*)output.data_ptr() + recv_off[(size_t)r] + (lo - seg0), hi - lo});
       }
       *nwin = std::max<size_t>(1, (largest + window - 1) / window);
@@ -1224,18 +1776,18 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>
       }
       if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
     };
-    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
       size_t largest = 0;
       std::vector<mccl_segment_t> segs;
       for (int r = 0; r < W; ++r) {
-        const int64_t* tr = tables[(size_t)r];
+        const int64_t* tr = pv.tables[(size_t)r];
         const size_t b = (size_t)tr[W + me];
         TORCH_CHECK(b == nbytes(outs[(size_t)r]), "alltoall: output tensor ", r, " does not match what rank ", r, " sends");
         largest = std::max(largest, (size_t)tr[2 * W]);
         const size_t seg0 = (size_t)tr[me], seg1 = seg0 + b;
         const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w1);
         if (lo < hi)
-          segs.push_back({(const char*)peer[(size_t)r] + (lo - w0), (char*)outs[(size_t)r].data_ptr() + (lo - seg0), hi - lo});
+          segs.push_back({(const char*)pv.stage[(size_t)r] + (lo - w0), (char*)outs[(size_t)r].data_ptr() + (lo - seg0), hi - lo});
       }
       *nwin = std::max<size_t>(1, (largest + window - 1) / window);
       if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
@@ -1250,6 +1802,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::barrier(const c10d::BarrierOptio
   Plan p;
   p.op = c10d::OpType::BARRIER;
   p.title = "barrier";
+  p.host_complete = true;
   auto work = run(p);
   // a barrier returns once every rank has arrived: nothing is pending on the stream
   return work;
@@ -1286,8 +1839,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce(std::vector<at::Tensor>& 
       p.stage_bytes = len * es;
       p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, base, len * es, s); };
       if (rank_ == root)
-        p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>&, hipStream_t s) {
-          std::vector<const void*> in = peer;
+        p.exec = [=](const PeerView& pv, hipStream_t s) {
+          std::vector<const void*> in = pv.stage;
           in[(size_t)root] = base;  // in place on the root's tensor, as in allreduce
           MCCL_CHECK(mccl_reduce_n(in.data(), W, base, len, dtype, op, MCCL_VARIANT_AUTO, s));
         };
@@ -1347,12 +1900,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::gather(std::vector<std::vector<a
   const int W = size_;
   if (mine) p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, input.data_ptr(), mine, s); };
   if (rank_ == root)
-    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
       std::vector<mccl_segment_t> segs;
       for (int r = 0; r < W; ++r) {
-        const size_t b = (size_t)tables[(size_t)r][0];
+        const size_t b = (size_t)pv.tables[(size_t)r][0];
         TORCH_CHECK(b == nbytes(outs[(size_t)r]), "gather: output tensor ", r, " does not match the size rank ", r, " sends");
-        if (b) segs.push_back({peer[(size_t)r], outs[(size_t)r].data_ptr(), b});
+        if (b) segs.push_back({pv.stage[(size_t)r], outs[(size_t)r].data_ptr(), b});
       }
       MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
     };
@@ -1432,14 +1985,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
           segs.push_back({ins[(size_t)r].data_ptr(), (char*)stage + offs[(size_t)r], nbytes(ins[(size_t)r])});
       if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
     };
-    p.exec = [=](const std::vector<const void*>&, const std::vector<const int64_t*>&, hipStream_t s) {
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
       copyAsync(out.data_ptr(), ins[(size_t)root].data_ptr(), nbytes(out), s);
     };
   } else {
-    p.exec = [=](const std::vector<const void*>& peer, const std::vector<const int64_t*>& tables, hipStream_t s) {
-      const size_t b = (size_t)tables[(size_t)root][W + me];
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
+      const size_t b = (size_t)pv.tables[(size_t)root][W + me];
       TORCH_CHECK(b == nbytes(out), "scatter: output tensor does not match the size the root sends");
-      copyAsync(out.data_ptr(), (const char*)peer[(size_t)root] + tables[(size_t)root][me], b, s);
+      copyAsync(out.data_ptr(), (const char*)pv.stage[(size_t)root] + pv.tables[(size_t)root][me], b, s);
     };
   }
   return run(p);
@@ -1448,12 +2001,10 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::scatter(std::vector<at::Tensor>&
 // point to point
 // ---------------------------------------------------------------------------------------------
 void ProcessGroupCCL::spinUntil(const std::function<bool()>& ready, int peer, const char* what,
-                                const std::function<bool()>& abandoned, const std::function<void()>& idle) {
-  std::chrono::milliseconds limit = std::max(timeout_, std::chrono::milliseconds(30000));
-  if (const char* v = std::getenv("MCCL_BARRIER_TIMEOUT_MS")) {
-    const long ms = std::atol(v);
-    if (ms > 0) limit = std::chrono::milliseconds(ms);
-  }
+                                const std::function<bool()>& abandoned, const std::function<void()>& idle,
+                                std::chrono::milliseconds limit_override) {
+  // a wait(timeout) of the caller's wins over the group's limit
+  const std::chrono::milliseconds limit = limit_override.count() > 0 ? limit_override : waitLimit(false);
   const auto deadline = std::chrono::steady_clock::now() + limit;
   unsigned spins = 0;
   while (!ready()) {
@@ -1547,12 +2098,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::recv(std::vector<at::Tensor>& te
   return c10::make_intrusive<RecvWorkCCL>(std::move(self), std::move(state), rank_);
 }
 
-void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocking) {
+void ProcessGroupCCL::progressRecv(int src, const RecvState* target, bool blocking, std::chrono::milliseconds limit) {
   std::lock_guard<std::mutex> lock(mutex_);
-  progressRecvLocked(src, target, blocking);
+  progressRecvLocked(src, target, blocking, limit);
 }
 
-void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool blocking) {
+void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool blocking, std::chrono::milliseconds limit) {
   if (target && target->done) return;
   c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
   hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_).stream();
@@ -1572,7 +2123,7 @@ void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool 
                     for (int other = 0; other < size_; ++other)
                       if (other != src && !p2p_recv_[(size_t)other].pending.empty())
                         progressRecvLocked(other, nullptr, /*blocking=*/false);
-                  });
+                  }, limit);
       }
       const size_t len = std::min(total - st->off, stage_max_);
       const int slot = (int)((k - 1) % kRing);
@@ -1580,12 +2131,18 @@ void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool 
       if (e.bytes != len) {
         // The two sides disagree about the message stream: drop the message and the receive, and
         // flag the group as failed (what follows on this pair can no longer be matched reliably).
+        // The error belongs to this receive: its own wait() raises it, whichever call got here.
         const uint64_t have = e.bytes;
         box.consumed.store(k, std::memory_order_release);
+        const std::string why = c10::str("ccl backend: recv expects ", len, " bytes from rank ", src,
+                                         " but the message holds ", have);
+        st->error = std::make_exception_ptr(std::runtime_error(why));
         st->done = true;
         pr.pending.pop_front();
         ctl_->slot[rank_].failed.store(1, std::memory_order_release);
-        TORCH_CHECK(false, "ccl backend: recv expects ", len, " bytes from rank ", src, " but the message holds ", have);
+        shared_->fail(why);
+        if (st.get() == target) std::rethrow_exception(st->error);
+        break;  // go on with the next posted receive of this source
       }
       if (len) {
         const void* from = nullptr;
@@ -1614,6 +2171,7 @@ void ProcessGroupCCL::progressRecvLocked(int src, const RecvState* target, bool 
       st->off += len;
       finished = st->off >= total;
     }
+    if (st->error) continue;  // dropped above
     st->done = true;
     pr.pending.pop_front();
     if (st.get() == target) return;
@@ -1625,14 +2183,25 @@ ProcessGroupCCL::RecvWorkCCL::RecvWorkCCL(c10::intrusive_ptr<ProcessGroupCCL> pg
     : c10d::Work(rank, c10d::OpType::RECV, "recv"), pg_(std::move(pg)), state_(std::move(state)) {}
 
 bool ProcessGroupCCL::RecvWorkCCL::isCompleted() {
-  pg_->progressRecv(state_->src, state_.get(), /*blocking=*/false);
+  if (!state_->done) {
+    try {
+      pg_->progressRecv(state_->src, state_.get(), /*blocking=*/false);
+    } catch (...) {
+      if (!state_->error) throw;  // this receive's own failure is reported by wait() / exception()
+    }
+  }
   return state_->done;
 }
 
-void ProcessGroupCCL::RecvWorkCCL::synchronize() { pg_->progressRecv(state_->src, state_.get(), /*blocking=*/true); }
+bool ProcessGroupCCL::RecvWorkCCL::isSuccess() const { return !state_->error; }
 
-bool ProcessGroupCCL::RecvWorkCCL::wait(std::chrono::milliseconds /*timeout*/) {
-  synchronize();
+std::exception_ptr ProcessGroupCCL::RecvWorkCCL::exception() const { return state_->error; }
+
+void ProcessGroupCCL::RecvWorkCCL::synchronize() { wait(kNoTimeout); }
+
+bool ProcessGroupCCL::RecvWorkCCL::wait(std::chrono::milliseconds timeout) {
+  if (!state_->done) pg_->progressRecv(state_->src, state_.get(), /*blocking=*/true, timeout);
+  if (state_->error) std::rethrow_exception(state_->error);
   return true;
 }
 

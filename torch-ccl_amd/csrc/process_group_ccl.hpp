@@ -2,16 +2,24 @@
 // ProcessGroupCCL (src/ProcessGroupCCL.hpp:111-310) over the C ABI of include/mccl.h.
 //
 // Single-GPU mode: every rank of the group (a process, or a thread of one process) uses
-// device 0.  Each rank owns two staging buffers in HBM.  A collective
-//   1. copies (or packs) the caller's input into the rank's staging buffer   [device copy]
-//   2. waits, on the host, until every rank has finished step 1              [barrier]
-//   3. runs the local-reduce / pull kernel over the N ranks' staging buffers,
-//      writing straight into the caller's output tensor                      [the hot path]
-// which is the structure of the reference's IPC allreduce (copy-in, cross-rank barrier, sum of
-// the N peer buffers: src/gpu/allreduce_small.h:166-361).  Peers' staging buffers are reached
-// through hipIpcOpenMemHandle (other processes) or directly (threads of the same process); the
-// handles, a host barrier and small per-collective tables live in a POSIX shared-memory control
-// block whose name is published through the c10d Store (the role of
+// device 0.  A collective is the structure of the reference's IPC allreduce (copy-in, cross-rank
+// barrier, sum of the N peer buffers: src/gpu/allreduce_small.h:166-361):
+//   1. the peers get to see this rank's input: a copy (or pack) into the rank's staging buffer
+//      in HBM, or -- for large single-tensor collectives whose tensors the peers can map -- the
+//      caller's tensor itself (the reference hands the user buffer to the IPC exchange the same
+//      way, src/gpu/allreduce.h:1214-1224);
+//   2. a cross-rank barrier;
+//   3. the local-reduce / pull kernel over the N ranks' buffers, writing straight into the
+//      caller's output tensor                                                [the hot path]
+// When the ranks are processes of their own, step 2 is a flag kernel on the collective's stream
+// (mccl_rank_barrier): no host thread waits for the GPU and no stream is synchronised, so a
+// collective only enqueues work.  Allreduces of up to 1 MiB are one kernel that does all three
+// steps (mccl_allreduce_fused).  Ranks that are threads of one process share streams and hardware
+// queues, where a waiting kernel could block the kernel it waits for: they keep the host barrier
+// (hipStreamSynchronize + a spin on the control block), which MCCL_PG_SYNC=host also selects.
+// Peers' buffers are reached through hipIpcOpenMemHandle (other processes) or directly (threads of
+// the same process); the handles, the host rendezvous and small per-collective tables live in a
+// POSIX shared-memory control block whose name is published through the c10d Store (the role of
 // src/ccl_comm_collector.cpp:10-45 and src/gpu/allreduce.h:1208-1248).
 // A staging buffer is at most 1 GiB (shared allocations stay well below 2 GiB); longer messages
 // travel in windows.  Point-to-point messages use a mailbox per ordered pair of ranks in the same
@@ -25,17 +33,38 @@
 #include <torch/csrc/distributed/c10d/Utils.hpp>
 #include <torch/csrc/distributed/c10d/Work.hpp>
 
+#include <atomic>
 #include <chrono>
 #include <deque>
 #include <functional>
 #include <memory>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 namespace mccl_pg {
 
 struct Control;  // shared-memory control block (process_group_ccl.cpp)
+
+// What the Works of a group share with it and may outlive it with: recycled events and the
+// group's health.  `status` is two words of pinned host memory the device-side waits write when
+// they give up (1 + the late rank, the epoch); `failed` is raised by the host side.
+struct GroupShared {
+  std::mutex mutex;
+  std::vector<hipEvent_t> free_events;
+  volatile uint32_t* status = nullptr;
+  std::atomic<bool> failed{false};
+  std::string failure;  // guarded by mutex
+  int device = 0;
+
+  hipEvent_t getEvent();
+  void putEvent(hipEvent_t e);
+  // Non-empty once a device-side wait has timed out or the host side has given up.
+  std::string failureMessage();
+  void fail(const std::string& why);
+  ~GroupShared();
+};
 
 class ProcessGroupCCL : public c10d::Backend {
  public:
@@ -48,7 +77,14 @@ class ProcessGroupCCL : public c10d::Backend {
             std::vector<at::Tensor> outputs, bool blocking_wait);
     ~WorkCCL() override;
     bool isCompleted() override;
+    // false once the group has failed (a peer did not arrive in time, a rank reported a failure);
+    // exception() then carries the reason (src/ProcessGroupCCL.cpp:866-869)
     bool isSuccess() const override;
+    std::exception_ptr exception() const override;
+    // Non-blocking mode: the caller's stream waits for the collective.  CCL_BLOCKING_WAIT=1: the
+    // host waits, at most `timeout` (the group's timeout when kNoTimeout is passed), and raises
+    // "Caught collective operation timeout" like the reference (src/utils.h:295-319).  Both raise
+    // when the group has failed.
     bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
     void synchronize() override;
     std::vector<at::Tensor> result() override;
@@ -56,7 +92,11 @@ class ProcessGroupCCL : public c10d::Backend {
 
    private:
     friend class ProcessGroupCCL;
+    void waitInternal(std::chrono::milliseconds timeout);
     hipEvent_t end_ = nullptr;
+    std::shared_ptr<GroupShared> shared_;
+    std::chrono::milliseconds op_timeout_{0};
+    std::chrono::steady_clock::time_point start_;
     int device_ = 0;
     bool blocking_wait_ = false;
     std::vector<at::Tensor> inputs_;   // held until the Work dies (ownership rule of the reference)
@@ -71,6 +111,7 @@ class ProcessGroupCCL : public c10d::Backend {
     uint64_t next_seq = 0;  // sequence number (from 1) of the next message of this receive
     size_t off = 0;         // bytes of the tensor already filled (a long tensor travels as several messages)
     bool done = false;
+    std::exception_ptr error;  // why the receive failed; raised by its own wait(), whoever progressed it
   };
 
   // Work of a receive (XPUP2PAsyncWork of the reference, src/gpu/dpcpp_ccl.cpp:1590-1627).  The
@@ -80,7 +121,8 @@ class ProcessGroupCCL : public c10d::Backend {
    public:
     RecvWorkCCL(c10::intrusive_ptr<ProcessGroupCCL> pg, std::shared_ptr<RecvState> state, int rank);
     bool isCompleted() override;
-    bool isSuccess() const override { return true; }
+    bool isSuccess() const override;
+    std::exception_ptr exception() const override;
     bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
     void synchronize() override;
     std::vector<at::Tensor> result() override;
@@ -160,6 +202,15 @@ class ProcessGroupCCL : public c10d::Backend {
   c10::intrusive_ptr<c10d::Work> recvAnysource(std::vector<at::Tensor>&, int) override;
 
  private:
+  // What the data-path kernels of one collective get to see of the peers.
+  struct PeerView {
+    std::vector<const void*> stage;         // rank r's staging buffer (this process's mapping)
+    std::vector<const int64_t*> tables;     // the scalars rank r published
+    bool zero_copy = false;                 // the peers' tensors are read in place: nothing was staged
+    std::vector<const void*> user;          // zero_copy: rank r's published tensor range
+  };
+  using ExecFn = std::function<void(const PeerView& pv, hipStream_t s)>;
+
   // What one collective needs from the engine.
   struct Plan {
     c10d::OpType op = c10d::OpType::UNKNOWN;
@@ -170,23 +221,52 @@ class ProcessGroupCCL : public c10d::Backend {
     std::vector<int64_t> table;             // per-collective scalars published to the peers
     // enqueue the copy-in on `s`; `stage` is this rank's staging buffer
     std::function<void(void* stage, hipStream_t s)> copy_in;
-    // enqueue the data-path kernels on `s`; peer[r] is rank r's staging buffer,
-    // tables[r] the scalars rank r published
-    std::function<void(const std::vector<const void*>& peer,
-                       const std::vector<const int64_t*>& tables, hipStream_t s)> exec;
-    // optional second phase: runs after every rank has finished `exec` (one more stream
-    // synchronisation and host barrier); used by the two-shot allreduce
-    std::function<void(const std::vector<const void*>& peer,
-                       const std::vector<const int64_t*>& tables, hipStream_t s)> exec2;
+    // enqueue the data-path kernels on `s`
+    ExecFn exec;
+    // optional second phase: runs after every rank has finished `exec` (one more barrier);
+    // used by the two-shot allreduce.  two_phase, when set, says whether this run needs it.
+    ExecFn exec2;
+    std::function<bool(const PeerView& pv)> two_phase;
+    // Zero-copy offer (device-synchronised groups only): the byte range of the caller's tensor
+    // that the peers may read in place of a staged copy.  `share` must come out the same on every
+    // rank (it may depend on sizes all ranks agree on, never on this rank's own).  The offer is
+    // taken when every rank of the group can share its range (an allocation of torch's caching
+    // allocator below 2 GiB); copy_in is then skipped, exec / exec2 run with pv.zero_copy set, and
+    // a closing barrier keeps every rank from touching its tensor before all peers have read it.
+    bool share = false;
+    const void* share_ptr = nullptr;
+    size_t share_bytes = 0;
+    size_t zero_copy_stage_bytes = 0;       // staging this rank still needs in zero-copy mode
+    // Eligible for the one-launch small allreduce (device-synchronised groups of at most 8 ranks):
+    // no staging slot, no table, no rendezvous.  The staged plan above stays as the fallback.
+    bool fused_ok = false;
+    void* fused_ptr = nullptr;
+    size_t fused_count = 0;
+    int fused_dtype = 0;
+    int fused_op = 0;
+    bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
   c10::intrusive_ptr<c10d::Work> run(Plan& plan);
+  c10::intrusive_ptr<c10d::Work> finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work);
+  void runHostSynced(Plan& plan, hipStream_t s, int slot);
+  void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
+  void deviceBarrier(uint64_t epoch, hipStream_t s);
+  void throwIfFailed();
+  void awaitPeersEntered(uint64_t seq);
+  // zero-copy: publish / map caller-owned allocations
+  int exportRange(const void* ptr, size_t bytes, uint64_t* offset);
+  const void* importRange(int peer, int pub);
+  void closeImports();
+  void quiesce();  // host waits for this rank's outstanding collective work (before a mapping is closed)
   void ensureInit(int device);
   void* ensureStage(int slot, size_t bytes);
   // start_up: the first barrier of a group, which also absorbs the ranks' different start-up
   // times: at least two minutes, and not shortened by MCCL_BARRIER_TIMEOUT_MS
   void hostBarrier(bool start_up = false);
-  const void* peerStage(int peer, int slot);
+  std::chrono::milliseconds waitLimit(bool start_up) const;
+  const void* peerStage(int peer, int slot, int pub);
+  void publishStage(int slot, int pub);
   void checkDeviceTensors(const std::vector<at::Tensor>& tensors) const;
   // Spins (then yields) until ready() holds; raises when `peer` reports a failure, when it has
   // left and abandoned() says that what is awaited can no longer come, or at the time limit.
@@ -194,12 +274,16 @@ class ProcessGroupCCL : public c10d::Backend {
   // complete this rank's own posted receives, so that ranks sending round a ring cannot block
   // each other for good).
   void spinUntil(const std::function<bool()>& ready, int peer, const char* what,
-                 const std::function<bool()>& abandoned, const std::function<void()>& idle = nullptr);
+                 const std::function<bool()>& abandoned, const std::function<void()>& idle = nullptr,
+                 std::chrono::milliseconds limit_override = std::chrono::milliseconds(0));
   // Completes the receives posted for `src` in order, up to and including `target` (all of them
   // when target is null).  With blocking == false it stops at the first message the sender has
   // not published yet.  progressRecv takes the group's mutex, the Locked form expects it held.
-  void progressRecv(int src, const RecvState* target, bool blocking);
-  void progressRecvLocked(int src, const RecvState* target, bool blocking);
+  // `limit` > 0 replaces the group's time limit for the blocking wait (a wait(timeout) of the caller's).
+  void progressRecv(int src, const RecvState* target, bool blocking,
+                    std::chrono::milliseconds limit = std::chrono::milliseconds(0));
+  void progressRecvLocked(int src, const RecvState* target, bool blocking,
+                          std::chrono::milliseconds limit = std::chrono::milliseconds(0));
 
   c10::intrusive_ptr<c10d::Store> store_;
   std::chrono::milliseconds timeout_;
@@ -207,6 +291,11 @@ class ProcessGroupCCL : public c10d::Backend {
   bool same_stream_ = false;    // CCL_SAME_STREAM
   bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
   bool profile_ = false;        // MCCL_PG_PROFILE: host-side phase timers, printed when the group dies
+  bool want_device_sync_ = true;  // MCCL_PG_SYNC != "host"
+  bool zero_copy_ = true;         // MCCL_PG_ZERO_COPY != 0
+  // Decided at start-up, the same on every rank: all ranks are processes of their own (and the
+  // environment does not ask for the host barrier), so cross-rank waits can live on the device.
+  bool device_sync_ = false;
   size_t stage_max_ = 0;        // bytes of one staging window (1 GiB; MCCL_STAGE_WINDOW_BYTES shrinks it for tests)
   // per collective with a payload: copy-in enqueue, stream synchronise, host barrier, kernel enqueue
   std::vector<float> phase_us_[4];
@@ -235,6 +324,8 @@ class ProcessGroupCCL : public c10d::Backend {
     void* base = nullptr;  // the allocation
     void* ptr = nullptr;   // where this rank's data starts (staggered by rank inside the allocation)
     size_t capacity = 0;
+    uint64_t gen = 0;      // bumped whenever the buffer is replaced
+    hipIpcMemHandle_t handle{};
   };
   Stage stage_[2];
   std::vector<void*> retired_;  // outgrown staging buffers, freed with the group
@@ -246,6 +337,38 @@ class ProcessGroupCCL : public c10d::Backend {
     bool ipc[2] = {false, false};
   };
   std::vector<PeerMap> peers_;
+
+  // device-side synchronisation: one small arena per rank (flag words, and the staging buffers and
+  // tile flags of the one-launch allreduce), mapped by every peer at start-up
+  void* arena_ = nullptr;
+  std::vector<void*> peer_arena_;           // this process's mapping of rank r's arena
+  std::vector<void*> bar_flags_;            // rank r's barrier word
+  std::vector<void*> final_flags_;          // rank r's departure word
+  std::vector<void*> fused_stage_[2];       // rank r's staging buffer of the one-launch allreduce, per slot
+  std::vector<void*> fused_flags_[2];
+  void* status_dev_ = nullptr;              // device address of shared_->status
+  std::shared_ptr<GroupShared> shared_;
+
+  // zero-copy exports (this rank's allocations the peers may map) and imports
+  struct Export {
+    uint64_t base = 0;
+    uint64_t size = 0;
+    bool valid = false;
+  };
+  std::vector<Export> exports_;             // mirrors the export table of this rank's control slot
+  int export_clock_ = 0;                    // next table entry to evict
+  int recent_export_[2] = {-1, -1};         // entries of the last two offers: not evicted
+  uint64_t rendezvous_count_ = 0;           // device-synchronised collectives that met at the host rendezvous
+  struct Import {
+    void* base = nullptr;
+    uint64_t gen = 0;
+  };
+  std::vector<std::vector<Import>> imports_;  // [peer][export entry]
+ public:
+  // Called (under the allocator's lock) when torch's caching allocator returns a segment to the
+  // runtime: an export of that segment must not be handed to the peers again.
+  void segmentFreed(uint64_t base);
+ private:
 
   // point to point
   static constexpr int kP2PRing = 4;
