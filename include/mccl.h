@@ -86,7 +86,13 @@ typedef enum {
   MCCL_TUNE_COMBINE_WAVES_PER_CU = 6,     /* moe_combine with top-k <= 8: default 0 = one wavefront per
                                              row chunk; > 0 = persistent grid of that many wavefronts
                                              per CU, each walking several chunks (measured slower) */
-  MCCL_TUNE_COUNT_ = 7
+  MCCL_TUNE_XRANK_WAVES_ALL_RANKS = 7,    /* wavefronts the launches of ALL ranks of a one-launch
+                                             collective (mccl_*_sync) may hold together; each
+                                             rank's grid is this divided by the rank count.  Must
+                                             stay below what the GPU keeps resident at once
+                                             (256 CUs x 32), or ranks could wait for launches
+                                             that find no room */
+  MCCL_TUNE_COUNT_ = 8
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64
@@ -178,6 +184,59 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
 int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
                          void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
                          uint64_t timeout_us, void* status, void* stream);
+
+/*
+ * One-launch collectives between rank processes that read the peers' buffers in place.  With
+ * several processes on one GPU every launch of a process waits for its turn at the dispatcher, so
+ * the cross-rank waits are folded into the data kernel: the launch itself publishes "this rank's
+ * stream has reached the collective" (ready_epoch, in words[rank]), every workgroup waits until all
+ * ranks' words have reached ready_epoch before it touches a peer's buffer, and -- when done_epoch
+ * is non-zero -- the kernel does not complete before every rank has published done_epoch, i.e. has
+ * finished reading (the caller's buffers may then be reused in stream order).  This replaces the
+ * separate sync kernels of src/gpu/allreduce.h:731-769, 835-877 around the data kernels.
+ *   words[r]: rank r's 64-bit word as for mccl_rank_barrier (the same word may serve both; epochs
+ * grow: ready_epoch of a call > any epoch used before, done_epoch > ready_epoch).  done_counter:
+ * one 32-bit word of this rank's device memory, zero before the first call (the kernel leaves it
+ * zero).  Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
+ * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
+ */
+typedef struct {
+  void* const* words;
+  int n;
+  int rank;
+  uint64_t ready_epoch;
+  uint64_t done_epoch;
+  void* done_counter;
+  uint64_t timeout_us; /* 0 = 10 s */
+  void* status;
+} mccl_xsync_t;
+
+/* mccl_copy_segments whose sources are peers' buffers: allgather / alltoall(v) / broadcast pulls
+ * (ccl::allgatherv, ccl::alltoallv, src/gpu/dpcpp_ccl.cpp:1176-1182, 1428-1455) in one launch.
+ * At most 64 segments; zero segments still take part in the waits. */
+int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsync_t* sync, void* stream);
+
+/* mccl_reduce_n whose inputs are peers' buffers (in[r]: rank r's contribution at this rank's
+ * slice): the shard reduction of reduce_scatter (ccl::reduce_scatter, src/gpu/dpcpp_ccl.cpp:1002-1008)
+ * in one launch.  Same arithmetic and bits as mccl_reduce_n; out must not overlap an input. */
+int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, int op,
+                     const mccl_xsync_t* sync, void* stream);
+
+/*
+ * In-place allreduce of tensors[rank] over all ranks' tensors in one launch: the two-shot
+ * algorithm of the reference's large path (reduce-scatter through scratch, all-gather:
+ * src/gpu/allreduce.h:306-533).  Rank r reduces shard r (mccl_allreduce_sync_shard(count, n)
+ * elements, the last shards may be shorter or empty) of all tensors into stage[r] and publishes
+ * tile_flags[r][t] = tile_epoch per MCCL_FUSED_TILE_BYTES; all ranks copy the finished shards
+ * into their tensors tile by tile.  stage[r]: at least one shard, 16-byte aligned; tile_flags[r]:
+ * one 32-bit word per tile of a shard, zero before the first use; tile epochs grow from call to
+ * call; a set may be reused once every peer has started a later collective.  done_epoch of the
+ * descriptor is ignored (a rank's kernel ends only after it has seen every owner's every flag,
+ * and only shard owners read a tensor).  Same bits as mccl_reduce_n over the n tensors.
+ */
+size_t mccl_allreduce_sync_shard(size_t count, int n);
+int mccl_allreduce_sync(void* const* tensors, void* const* stage, void* const* tile_flags, size_t count,
+                        int dtype, int op, uint32_t tile_epoch, const mccl_xsync_t* sync, void* stream);
 
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */

@@ -147,6 +147,100 @@ def fused_case(rank, world, queues, barrier):
     barrier.wait(timeout=120)
 
 
+def xrank_case(rank, world, queues, barrier):
+    """The one-launch collectives that read the peers' buffers in place -- mccl_reduce_sync
+    (reduce_scatter shard), mccl_allreduce_sync (two-shot allreduce) and mccl_copy_segments_sync
+    (alltoallv pull) -- against the oracle, bit for bit, call after call on the same shared buffers
+    with nothing but the kernels' own waits between them."""
+    from helpers import TORCH_TO_CODE, assert_bits_equal, bits, oracle_reduce_bits, rank_buffer, to_carrier
+    from oracle import oracle as O
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    BUF = 24 << 20
+    shared_in = torch.zeros(BUF, dtype=torch.uint8, device=DEV)      # what the peers read in place
+    word = torch.zeros(8, dtype=torch.int64, device=DEV)             # [0]: the sync word
+    counter = torch.zeros(8, dtype=torch.int32, device=DEV)
+    stage = [torch.zeros((4 << 20) + 64, dtype=torch.uint8, device=DEV) for _ in range(2)]
+    tflag = [torch.zeros(4096 + 8, dtype=torch.int32, device=DEV) for _ in range(2)]
+    torch.cuda.synchronize()
+    shared = _exchange(rank, world, queues, barrier, [shared_in, word] + stage + tflag)
+    words = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])
+    st = _status()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    call = [0]
+
+    def sync(done=True):
+        call[0] += 1
+        return capi.XSync(ctypes.cast(words, ctypes.c_void_p), world, rank, 4 * call[0] + 1, 4 * call[0] + 3 if done else 0,
+                          counter.data_ptr(), 5_000_000, st.data_ptr())
+
+    def mine(dtype, count, off):
+        return shared_in[off:off + count * torch.empty(0, dtype=dtype).element_size()].view(dtype)
+
+    ops = {"SUM": (capi.SUM, O.SUM), "PROD": (capi.PROD, O.PROD), "MIN": (capi.MIN, O.MIN), "MAX": (capi.MAX, O.MAX)}
+    checks = []
+    # reduce_scatter shard: rank r reduces slice r of every rank's buffer
+    for i, (dtype, m, name, off) in enumerate([(torch.bfloat16, 70001, "SUM", 0), (torch.float32, 4099, "MAX", 4), (torch.int8, 300007, "SUM", 1),
+                                              (torch.float64, 1, "PROD", 8), (torch.float16, 1 << 19, "SUM", 16), (torch.int64, 33, "MIN", 0),
+                                              (torch.bfloat16, 1 << 20, "SUM", 2)]):
+        es = torch.empty(0, dtype=dtype).element_size()
+        off = off // es * es
+        host = [rank_buffer(world * m, dtype, r, seed=300 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
+        mine(dtype, world * m, off).copy_(host[rank])
+        out = torch.empty(m, dtype=dtype, device=DEV)
+        ins = capi.ptr_table([shared[r][0].data_ptr() + off + rank * m * es for r in range(world)])
+        sy = sync()
+        capi.check(L.mccl_reduce_sync(ins, out.data_ptr(), m, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
+        want = oracle_reduce_bits([h[rank * m:(rank + 1) * m] for h in host], ops[name][1])
+        checks.append((out, want, ("reduce_sync", str(dtype), m, name)))
+    # allreduce in place on the shared buffer
+    for i, (dtype, count, name, off) in enumerate([(torch.bfloat16, (2 << 20) + 77, "SUM", 0), (torch.float32, 1025, "SUM", 4), (torch.int8, (3 << 20) + 5, "MAX", 3),
+                                                  (torch.float64, 7, "SUM", 8), (torch.bfloat16, 3, "MIN", 2), (torch.float16, 1 << 21, "SUM", 0),
+                                                  (torch.int32, 100003, "PROD", 4), (torch.bfloat16, 4096 * 1024, "SUM", 0)]):
+        es = torch.empty(0, dtype=dtype).element_size()
+        off = off // es * es
+        host = [rank_buffer(count, dtype, r, seed=400 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
+        t = mine(dtype, count, off)
+        t.copy_(host[rank])
+        shard = L.mccl_allreduce_sync_shard(count, world)
+        assert shard * es <= 4 << 20 and shard * es // 1024 <= 4096
+        slot = call[0] & 1
+        sy = sync(done=False)
+        capi.check(L.mccl_allreduce_sync(
+            capi.ptr_table([shared[r][0].data_ptr() + off for r in range(world)]),
+            capi.ptr_table([shared[r][2 + slot].data_ptr() for r in range(world)]),
+            capi.ptr_table([shared[r][4 + slot].data_ptr() for r in range(world)]),
+            count, TORCH_TO_CODE[dtype], ops[name][0], call[0], ctypes.byref(sy), stream))
+        want = oracle_reduce_bits(host, ops[name][1])
+        checks.append((t.clone(), want, ("allreduce_sync", str(dtype), count, name)))
+    # alltoallv pull: rank d copies its segment out of every rank's buffer
+    rng = np.random.default_rng(99)
+    for i in range(4):
+        S = rng.integers(0, 4000, size=(world, world))
+        S[rng.integers(0, world), rng.integers(0, world)] = 0
+        row = (16, 96, 2, 1024)[i]
+        host = [rank_buffer(int(S[r].sum()) * row, torch.uint8, r, seed=500 + i) for r in range(world)]
+        mine(torch.uint8, host[rank].numel(), 0).copy_(host[rank])
+        out = torch.zeros(int(S[:, rank].sum()) * row, dtype=torch.uint8, device=DEV)
+        segs, roff = [], 0
+        for r in range(world):
+            b = int(S[r, rank]) * row
+            if b:
+                segs.append(capi.Segment(shared[r][0].data_ptr() + int(S[r, :rank].sum()) * row, out.data_ptr() + roff, b))
+            roff += b
+        arr = (capi.Segment * max(1, len(segs)))(*segs)
+        sy = sync()
+        capi.check(L.mccl_copy_segments_sync(arr, len(segs), ctypes.byref(sy), stream))
+        want = O.alltoallv([to_carrier(h) for h in host], S, row)[rank]
+        checks.append((out, want, ("copy_segments_sync", row, i)))
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    assert counter.cpu().tolist()[0] == 0
+    for o, w, what in checks:
+        assert_bits_equal(bits(o), np.asarray(w).view(bits(o).dtype) if np.asarray(w).dtype != bits(o).dtype else w, what)
+    barrier.wait(timeout=120)
+
+
 def timeout_case(rank, world, queues, barrier):
     """A peer that never signals: the waiting kernels end by themselves at their (tiny) limit, name
     the late rank, and leave the output alone.  Rank 1 simply does not call."""
@@ -180,5 +274,5 @@ def timeout_case(rank, world, queues, barrier):
 
 def run_rank(rank, world, queues, barrier, mode):
     torch.cuda.set_device(0)
-    {"barrier": barrier_case, "fused": fused_case, "timeout": timeout_case}[mode](rank, world, queues, barrier)
+    {"barrier": barrier_case, "fused": fused_case, "timeout": timeout_case, "xrank": xrank_case}[mode](rank, world, queues, barrier)
     torch.cuda.synchronize()

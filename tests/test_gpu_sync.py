@@ -28,6 +28,11 @@ def test_allreduce_fused_matches_the_oracle(world):
     _spawn(world, "fused")
 
 
+@pytest.mark.parametrize("world", [2, 5, 8])
+def test_one_launch_collectives_match_the_oracle(world):
+    _spawn(world, "xrank")
+
+
 def test_waits_are_bounded_and_name_the_late_rank():
     """Failure forced from the host (a rank that never calls, a 0.2 s limit): every kernel exits by
     itself."""

@@ -24,7 +24,7 @@ REDUCE_DTYPES = range(9)                                      # mccl_dtype_t cod
 KERNEL_LIB = os.path.join(LIB_DIR, "libmi355ccl.so")
 KERNEL_HDRS = [os.path.join(INCLUDE, "mccl.h")] + [
     os.path.join(HERE, h) for h in ("kernels_common.hpp", "kernels_reduce.hpp", "kernels_copy.hpp",
-                                    "kernels_moe.hpp", "kernels_sync.hpp", "kernels_fused.hpp", "reduce_launch.hpp")]
+                                    "kernels_moe.hpp", "kernels_sync.hpp", "kernels_fused.hpp", "kernels_xrank.hpp", "reduce_launch.hpp")]
 
 # -ffp-contract=off / no fast-math: the reduction chain must round add by add.
 # packed-fp32 ops are switched off for all device code.

@@ -39,7 +39,7 @@ _ARITH = re.compile(r"^(s_add_|s_sub_|s_addc_|s_subb_|s_lshl_b|s_ashr_|s_min_|s_
 _USER = re.compile(r"^(s_cselect_|s_cbranch_scc)")
 _PACKED = re.compile(r"^v_pk_(add|mul|fma)_f32")
 _FMA = re.compile(r"^(v_fma_f32|v_fmac_f32|v_mad_f32|v_fma_f64|v_fmac_f64)")
-_AVG_KERNEL = re.compile(r"(reduce_(vec|elem)_kernel|allreduce_fused_kernel)ILi\d+ELi1E")  # second template argument = MCCL_AVG
+_AVG_KERNEL = re.compile(r"(reduce_(vec|elem)_kernel|allreduce_fused_kernel|xrank_reduce_kernel)ILi\d+ELi1E")  # second template argument = MCCL_AVG
 _SCRATCH = re.compile(r"^scratch_")
 
 

@@ -4,6 +4,7 @@
 #pragma once
 
 #include "kernels_common.hpp"
+#include "kernels_sync.hpp"
 
 namespace {
 
@@ -25,11 +26,18 @@ struct CopyArgs {
   int nseg;
 };
 
+// The same plus the cross-rank waits of a one-launch collective between rank processes: the
+// sources are the peers' buffers, complete once every rank has reached the collective.
+struct SyncCopyArgs {
+  CopyArgs copy;
+  XSync sync;
+};
+
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
 // handed out in order.  The body moves as 16-byte vectors aligned on dst (non-temporal both
 // ways for full chunks); a source that is not congruent with dst mod 16 is read with unaligned
 // vector loads.
-__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
+__device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
     // binary search: largest s with chunk_prefix[s] <= chunk
@@ -66,6 +74,13 @@ __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) 
       if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
     }
   }
+}
+
+__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) { copy_segments_body(a); }
+
+__global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCopyArgs a) {
+  if (xsync_begin(a.sync)) copy_segments_body(a.copy);
+  xsync_end(a.sync, gridDim.x);
 }
 
 }  // namespace

@@ -64,6 +64,67 @@ __device__ __forceinline__ void report_late(uint32_t* status, int late_rank, uin
   __hip_atomic_store(status, (uint32_t)(late_rank + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// The same two waits folded into a data kernel, so that a collective is ONE launch per rank: with
+// several processes on one GPU every launch of a process waits for its turn at the dispatcher
+// (on the order of 15-20 us per process), which makes the number of launches per collective the
+// cost that matters.
+//   begin: workgroup 0 publishes `ready_epoch` in this rank's word ("this rank's stream has reached
+//          the collective: its input is complete"); every workgroup waits until all words have
+//          reached it.  Workgroups dispatched later find the words set and pass with one load each.
+//   end:   every workgroup counts itself out; the last one publishes `done_epoch` ("this rank has
+//          finished reading the peers' buffers") and waits until every rank has done the same, so the
+//          kernel -- and with it the stream -- does not complete before the peers are done with
+//          this rank's buffers.  done_epoch == 0: no closing wait.
+// A launch that uses these must fit on the GPU together with the launches of all its peers
+// (waiting workgroups occupy their slots): the host caps its grid accordingly.
+struct XSync {
+  uint64_t* word[kLeanSyncRanks];  // rank r's 64-bit word
+  uint64_t ready_epoch;
+  uint64_t done_epoch;
+  uint32_t* done_count;            // this rank's counter: zero between launches
+  uint64_t limit_ticks;
+  uint32_t* status;
+  int n;
+  int rank;
+};
+
+// Returns false (for the whole wavefront) when a peer did not arrive in time.
+__device__ __forceinline__ bool xsync_begin(const XSync& x) {
+  const int lane = threadIdx.x & (kWave - 1);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
+    __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  bool ok = true;
+  if (lane < x.n && lane != x.rank) {
+    ok = wait_flag64(x.word[lane], x.ready_epoch, x.limit_ticks);
+    if (!ok) report_late(x.status, lane, (uint32_t)x.ready_epoch);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  return __builtin_amdgcn_ballot_w64(!ok) == 0;
+}
+
+// Call once per workgroup, by all its lanes, after the workgroup's last access to a peer's buffer.
+__device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
+  if (x.done_epoch == 0) return;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  __syncthreads();
+  if (threadIdx.x >= kWave) return;  // the first wavefront of the workgroup does the rest
+  const int lane = threadIdx.x;
+  uint32_t last = 0;
+  if (lane == 0) {
+    const uint32_t before = __hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    last = before + 1 == workgroups ? 1u : 0u;
+    if (last) {
+      __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+  last = __builtin_amdgcn_readfirstlane(last);
+  if (!last) return;
+  if (lane < x.n && lane != x.rank) {
+    if (!wait_flag64(x.word[lane], x.done_epoch, x.limit_ticks)) report_late(x.status, lane, (uint32_t)x.done_epoch);
+  }
+}
+
 template <typename ARGS>
 __global__ __launch_bounds__(kWave) void rank_barrier_kernel(const ARGS a) {
   const int lane = threadIdx.x;

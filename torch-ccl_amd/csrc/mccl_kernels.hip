@@ -103,6 +103,7 @@ constexpr long long kTuneDefault[MCCL_TUNE_COUNT_] = {
     /* STREAM_MIN_TOTAL_BYTES   */ 112ll << 20,
     /* COMBINE_PIECES_PER_WAVE  */ 2,
     /* COMBINE_WAVES_PER_CU     */ 0,
+    /* XRANK_WAVES_ALL_RANKS    */ 4096,
 };
 struct TuneTable {
   std::atomic<long long> v[MCCL_TUNE_COUNT_];
@@ -189,6 +190,21 @@ hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned grid
     case MCCL_F32: return mccl_launch_fused_dt6(&a, op, grid_x, s);
     case MCCL_F64: return mccl_launch_fused_dt7(&a, op, grid_x, s);
     case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, grid_x, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned grid_x, hipStream_t s) {
+  switch (dtype) {
+    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, grid_x, s);
+    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, grid_x, s);
+    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, grid_x, s);
+    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, grid_x, s);
+    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, grid_x, s);
+    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, grid_x, s);
+    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, grid_x, s);
+    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, grid_x, s);
+    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, grid_x, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -484,7 +500,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 110; }
+int mccl_version(void) { return 120; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -669,6 +685,175 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
   a.rank = rank;
   hipError_t e = launch_fused_any(a, dtype, op, (unsigned)tiles, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "fused allreduce launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+// Workgroups (single wavefronts) of a launch that waits for its peers inside the kernel: all
+// ranks' launches must be resident at once, so each gets its share of a fixed budget.
+unsigned xrank_grid(uint64_t tiles, int n) {
+  uint64_t cap = (uint64_t)g_tune[MCCL_TUNE_XRANK_WAVES_ALL_RANKS] / (uint64_t)n;
+  if (cap < 1) cap = 1;
+  if (tiles < 1) tiles = 1;
+  return (unsigned)(tiles < cap ? tiles : cap);
+}
+
+int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
+  if (!sy) return fail(MCCL_ERR_INVALID_ARG, "sync descriptor is null");
+  if (!sy->words) return fail(MCCL_ERR_INVALID_ARG, "sync word table is null");
+  if (sy->n < 1 || sy->n > kXRanks) return fail(MCCL_ERR_UNSUPPORTED, "one-launch collectives take 1 to %d ranks, got %d", kXRanks, sy->n);
+  if (sy->rank < 0 || sy->rank >= sy->n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", sy->rank, sy->n);
+  if (sy->ready_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "ready_epoch must be positive");
+  if (sy->done_epoch != 0 && sy->done_epoch <= sy->ready_epoch) return fail(MCCL_ERR_INVALID_ARG, "done_epoch must be 0 or above ready_epoch");
+  if (sy->done_epoch != 0 && !sy->done_counter) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs a done counter");
+  if ((uintptr_t)sy->done_counter % 4 || (uintptr_t)sy->status % 4) return fail(MCCL_ERR_INVALID_ARG, "counter or status word is not 4-byte aligned");
+  memset(x, 0, sizeof(*x));
+  for (int r = 0; r < sy->n; ++r) {
+    if (!sy->words[r]) return fail(MCCL_ERR_INVALID_ARG, "sync word %d is null", r);
+    if ((uintptr_t)sy->words[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "sync word %d is not 8-byte aligned", r);
+    x->word[r] = (uint64_t*)sy->words[r];
+  }
+  x->ready_epoch = sy->ready_epoch;
+  x->done_epoch = sy->done_epoch;
+  x->done_count = (uint32_t*)sy->done_counter;
+  x->limit_ticks = wait_limit_ticks(sy->timeout_us);
+  x->status = (uint32_t*)sy->status;
+  x->n = sy->n;
+  x->rank = sy->rank;
+  return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsync_t* sync, void* stream) {
+  SyncCopyArgs a;
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  if (nseg < 0 || nseg > kMaxSegs) return fail(MCCL_ERR_INVALID_ARG, "a one-launch copy takes 0 to %d segments, got %d", kMaxSegs, nseg);
+  if (nseg && !segs) return fail(MCCL_ERR_INVALID_ARG, "segment table is null");
+  int m = 0;
+  uint64_t chunks = 0;
+  a.copy.chunk_prefix[0] = 0;
+  for (int i = 0; i < nseg; ++i) {
+    const mccl_segment_t& sg = segs[i];
+    if (sg.bytes == 0) continue;
+    if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
+    const uintptr_t dp = (uintptr_t)sg.dst;
+    CopySeg cs;
+    cs.src = (const char*)sg.src;
+    cs.dst = (char*)sg.dst;
+    cs.pad_ = 0;
+    size_t head = (128u - (unsigned)(dp & 127u)) & 127u;
+    if (head > sg.bytes) head = sg.bytes;
+    const size_t body = sg.bytes - head;
+    const uint64_t nfull = body / kCopyChunk;
+    cs.head = (uint32_t)head;
+    cs.last = (uint32_t)(body % kCopyChunk);
+    uint64_t c = nfull + (cs.last ? 1 : 0);
+    if (c == 0) c = 1;
+    if (nfull > 0xf0000000ull || chunks + c > kMaxChunks) return fail(MCCL_ERR_INVALID_ARG, "segment %d too large for a one-launch copy", i);
+    cs.nfull = (uint32_t)nfull;
+    a.copy.seg[m] = cs;
+    chunks += c;
+    a.copy.chunk_prefix[++m] = (uint32_t)chunks;
+  }
+  a.copy.nseg = m;  // may be 0: the launch still takes part in the waits
+  const unsigned grid = xrank_grid(chunks, a.sync.n);
+  hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, int op,
+                     const mccl_xsync_t* sync, void* stream) {
+  XRankArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_reduce_args(in, a.sync.n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  const size_t es = dtype_size(dtype);
+  if (count) {
+    if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer is null");
+    if ((uintptr_t)out % es) return fail(MCCL_ERR_INVALID_ARG, "output pointer not aligned to the element size");
+    for (int k = 0; k < a.sync.n; ++k) {
+      if (!in[k]) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d is null", k);
+      if ((uintptr_t)in[k] % es) return fail(MCCL_ERR_INVALID_ARG, "input pointer %d not aligned to the element size", k);
+      a.in[k] = (const char*)in[k];
+    }
+  }
+  const size_t ve = 16 / es;
+  const uint64_t vecs = count / ve + (count % ve ? 1 : 0);
+  if (vecs + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  a.out1 = (char*)out;
+  a.nvec1 = (uint32_t)(count / ve);
+  a.tail1 = (uint32_t)(count % ve);
+  a.tiles1 = (uint32_t)((vecs + kWave - 1) / kWave);
+  a.stream_out = count * es >= (32u << 20) ? 1u : 0u;
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n), (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+size_t mccl_allreduce_sync_shard(size_t count, int n) {
+  if (n < 1) return 0;
+  const size_t per = (count + (size_t)n - 1) / (size_t)n;
+  return (per + 63) / 64 * 64;
+}
+
+int mccl_allreduce_sync(void* const* tensors, void* const* stage, void* const* tile_flags, size_t count,
+                        int dtype, int op, uint32_t tile_epoch, const mccl_xsync_t* sync, void* stream) {
+  XRankArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (!tensors || !stage || !tile_flags) return fail(MCCL_ERR_INVALID_ARG, "tensor, staging or flag table is null");
+  const int n = a.sync.n, me = a.sync.rank;
+  const size_t es = dtype_size(dtype);
+  const size_t shard = mccl_allreduce_sync_shard(count, n);
+  for (int r = 0; r < n; ++r) {
+    if (!stage[r] || !tile_flags[r] || (count && !tensors[r])) return fail(MCCL_ERR_INVALID_ARG, "tensor, staging or flag pointer %d is null", r);
+    if ((uintptr_t)stage[r] % 16) return fail(MCCL_ERR_INVALID_ARG, "staging buffer %d is not 16-byte aligned", r);
+    if ((uintptr_t)tile_flags[r] % 4) return fail(MCCL_ERR_INVALID_ARG, "flag array %d is not 4-byte aligned", r);
+    if ((uintptr_t)tensors[r] % es) return fail(MCCL_ERR_INVALID_ARG, "tensor %d not aligned to the element size", r);
+  }
+  auto shard_len = [&](int r) {
+    const size_t lo = (size_t)r * shard < count ? (size_t)r * shard : count;
+    const size_t hi = lo + shard < count ? lo + shard : count;
+    return hi - lo;
+  };
+  const size_t n_me = shard_len(me);
+  const size_t ve = 16 / es;
+  if ((uint64_t)shard * es / 16 + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  for (int k = 0; k < n; ++k) a.in[k] = (const char*)tensors[k] + (size_t)me * shard * es;
+  a.out1 = (char*)stage[me];
+  a.my_flags = (uint32_t*)tile_flags[me];
+  a.nvec1 = (uint32_t)(n_me / ve);
+  a.tail1 = (uint32_t)(n_me % ve);
+  a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
+  a.tile_epoch = tile_epoch;
+  uint32_t tiles2 = 0;
+  for (int q = 0; q < n; ++q) {
+    const uint64_t bytes = (uint64_t)shard_len(q) * es;
+    a.shard_src[q] = (const char*)stage[q];
+    a.shard_flags[q] = (const uint32_t*)tile_flags[q];
+    a.shard_dst[q] = (char*)tensors[me] + (size_t)q * shard * es;
+    a.full2[q] = (uint32_t)(bytes / kXTileBytes);
+    a.last2[q] = (uint32_t)(bytes % kXTileBytes);
+    const uint32_t tq = a.full2[q] + (a.last2[q] ? 1u : 0u);
+    if (tq > tiles2) tiles2 = tq;
+  }
+  a.tiles2 = tiles2;
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(tiles2, n), (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
 

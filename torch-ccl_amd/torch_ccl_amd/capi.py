@@ -20,7 +20,7 @@ SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
 VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
 (TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_WAVES_PER_CU, TUNE_SMALL_MAX_BYTES,
  TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
- TUNE_COMBINE_WAVES_PER_CU) = range(7)
+ TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS) = range(8)
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
@@ -36,7 +36,15 @@ EXPORTS = (
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
     "mccl_rank_barrier", "mccl_allreduce_fused",
+    "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync", "mccl_allreduce_sync_shard",
 )
+
+
+class XSync(ctypes.Structure):
+    """mccl_xsync_t"""
+    _fields_ = [("words", ctypes.c_void_p), ("n", ctypes.c_int), ("rank", ctypes.c_int),
+                ("ready_epoch", ctypes.c_uint64), ("done_epoch", ctypes.c_uint64), ("done_counter", ctypes.c_void_p),
+                ("timeout_us", ctypes.c_uint64), ("status", ctypes.c_void_p)]
 
 
 class Segment(ctypes.Structure):
@@ -74,6 +82,11 @@ def lib():
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
     L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, vp]
+    L.mccl_copy_segments_sync.argtypes = [vp, i32, vp, vp]
+    L.mccl_reduce_sync.argtypes = [vp, vp, sz, i32, i32, vp, vp]
+    L.mccl_allreduce_sync.argtypes = [vp, vp, vp, sz, i32, i32, ctypes.c_uint32, vp, vp]
+    L.mccl_allreduce_sync_shard.argtypes = [sz, i32]
+    L.mccl_allreduce_sync_shard.restype = sz
     L.mccl_query_launch.argtypes = [sz, i32, i32, i32, i32, vp, vp]
     L.mccl_set_tuning.argtypes = [i32, ctypes.c_longlong]
     L.mccl_get_tuning.argtypes = [i32]
