@@ -161,7 +161,28 @@ def _backend_rank(rank, world, store_path, cases, out_path):
             ts.append(time.perf_counter() - t0)
         ts.sort()
         res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters}
+        # the same call back to back (20 calls, one synchronize): what a loop of collectives pays per call
+        torch.cuda.synchronize()
+        dist.barrier()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            dist.all_reduce(t)
+        torch.cuda.synchronize()
+        res[name]["back_to_back_us"] = (time.perf_counter() - t0) / 20 * 1e6
         del x, t
+    # the floor of this way of timing: one trivial kernel of this process + synchronize, with all rank
+    # processes doing the same at the same moment (every launch waits for its process's turn)
+    one = torch.zeros(64, device="cuda:0")
+    ts = []
+    for _ in range(200):
+        torch.cuda.synchronize()
+        dist.barrier()
+        t0 = time.perf_counter()
+        one.add_(1.0)
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    res["one_trivial_kernel_plus_synchronize"] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": 200}
 
     def timed(fn, iters=8, warm=2):
         for _ in range(warm):
@@ -201,8 +222,8 @@ def _backend_rank(rank, world, store_path, cases, out_path):
 
 
 def backend_path(world=8):
-    """The drop-in c10d path end to end: `world` rank processes share cuda:0; every all_reduce is
-    copy-in + host barrier + the local-reduce kernel, timed on the host around the call."""
+    """The drop-in c10d path end to end: `world` rank processes share cuda:0 and call dist.* on GPU
+    tensors, timed on the host around the call plus a synchronize."""
     import tempfile
     import torch.multiprocessing as mp
     cases = [("c2_256KiB_bf16", 16 * 8192, 20, 200), ("c3_64MiB_bf16", 4096 * 8192, 3, 20)]
@@ -211,8 +232,11 @@ def backend_path(world=8):
         mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path), nprocs=world, join=True)
         with open(out_path) as f:
             res = json.load(f)
-    out = {"processes": world, "note": "host-timed dist.* calls incl. copy-in, host barrier, kernel and "
-                                       "synchronize; all ranks run their kernels on the one GPU concurrently"}
+    out = {"processes": world, "note": "host-timed dist.* call + synchronize per rank process; all ranks share the one "
+                                       "GPU.  Cross-rank waits run on the device (flag kernels, or inside the data "
+                                       "kernel), large tensors are read by the peers in place; every launch of a "
+                                       "process waits for its turn at the dispatcher, which is what "
+                                       "one_trivial_kernel_plus_synchronize measures"}
     for name in res:
         out[name] = {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()}
     return out

@@ -181,6 +181,7 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
  */
 #define MCCL_FUSED_MAX_RANKS 8
 #define MCCL_FUSED_TILE_BYTES 1024
+#define MCCL_SYNC_FLAG_BYTES 4096 /* bytes of a shard per flag of mccl_allreduce_sync */
 int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
                          void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
                          uint64_t timeout_us, void* status, void* stream);
@@ -227,9 +228,9 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
  * algorithm of the reference's large path (reduce-scatter through scratch, all-gather:
  * src/gpu/allreduce.h:306-533).  Rank r reduces shard r (mccl_allreduce_sync_shard(count, n)
  * elements, the last shards may be shorter or empty) of all tensors into stage[r] and publishes
- * tile_flags[r][t] = tile_epoch per MCCL_FUSED_TILE_BYTES; all ranks copy the finished shards
- * into their tensors tile by tile.  stage[r]: at least one shard, 16-byte aligned; tile_flags[r]:
- * one 32-bit word per tile of a shard, zero before the first use; tile epochs grow from call to
+ * tile_flags[r][c] = tile_epoch per MCCL_SYNC_FLAG_BYTES of it; all ranks copy the finished shards
+ * into their tensors chunk by chunk.  stage[r]: at least one shard, 16-byte aligned; tile_flags[r]:
+ * one 32-bit word per MCCL_SYNC_FLAG_BYTES of a shard, zero before the first use; tile epochs grow from call to
  * call; a set may be reused once every peer has started a later collective.  done_epoch of the
  * descriptor is ignored (a rank's kernel ends only after it has seen every owner's every flag,
  * and only shard owners read a tensor).  Same bits as mccl_reduce_n over the n tensors.

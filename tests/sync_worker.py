@@ -203,7 +203,7 @@ def xrank_case(rank, world, queues, barrier):
         t = mine(dtype, count, off)
         t.copy_(host[rank])
         shard = L.mccl_allreduce_sync_shard(count, world)
-        assert shard * es <= 4 << 20 and shard * es // 1024 <= 4096
+        assert shard * es <= 4 << 20
         slot = call[0] & 1
         sy = sync(done=False)
         capi.check(L.mccl_allreduce_sync(

@@ -31,12 +31,17 @@ struct CopyArgs {
 struct SyncCopyArgs {
   CopyArgs copy;
   XSync sync;
+  uint32_t invalidate;  // some bytes are read through the caches: invalidate once per workgroup first
 };
 
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
 // handed out in order.  The body moves as 16-byte vectors aligned on dst (non-temporal both
 // ways for full chunks); a source that is not congruent with dst mod 16 is read with unaligned
 // vector loads.
+// COHERENT: the sources are buffers of other ranks, complete in memory but possibly stale in this
+// kernel's caches: 8-byte aligned sources are read past the caches (the host requests a cache
+// invalidate per workgroup for the others).
+template <bool COHERENT>
 __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
@@ -64,7 +69,10 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
     if (len == (uint32_t)kCopyChunk) {
       u32x4 x[kCopyUnroll];
 #pragma unroll
-      for (int u = 0; u < kCopyUnroll; ++u) x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
+      for (int u = 0; u < kCopyUnroll; ++u) {
+        if (COHERENT && (((uintptr_t)src) & 7u) == 0) x[u] = load_vec_coherent(&((const u32x4*)src)[t + u * kWave]);
+        else x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
+      }
 #pragma unroll
       for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
     } else {
@@ -76,10 +84,14 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
   }
 }
 
-__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) { copy_segments_body(a); }
+__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) { copy_segments_body<false>(a); }
 
 __global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCopyArgs a) {
-  if (xsync_begin(a.sync)) copy_segments_body(a.copy);
+  if (xsync_begin(a.sync)) {
+    // heads, partial chunks and misaligned sources go through the caches
+    if (a.invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    copy_segments_body<true>(a.copy);
+  }
   xsync_end(a.sync, gridDim.x);
 }
 

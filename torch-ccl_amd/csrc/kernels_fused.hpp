@@ -10,9 +10,9 @@
 //      contribution comes from the registers of step 1) and writes the caller's output.
 // A wavefront depends on the wavefronts of the same tile in the peers' launches only, so no grid
 // has to be resident as a whole, and a launch needs no second kernel and no host round trip.
-// Visibility inside the kernel rests on the fences: the release fence writes the tile back before
-// the flag is stored, the acquire fence after the wait invalidates what this wavefront's caches
-// hold of the peers' buffers.
+// Visibility inside the kernel is per access: the staging tile is written through to memory and
+// waited for before its flag is stored, and the peers' tiles are read past the caches, so no
+// cache-wide write-back or invalidate is paid per tile.
 #pragma once
 
 #include "kernels_common.hpp"
@@ -36,16 +36,6 @@ struct FusedArgs {
   int rank;
 };
 
-// 32-bit epochs wrap: compare as a signed distance.
-__device__ __forceinline__ bool wait_flag32(const uint32_t* word, uint32_t epoch, uint64_t limit_ticks) {
-  const uint64_t t0 = wall_clock64();
-  while ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) < 0) {
-    if (wall_clock64() - t0 > limit_ticks) return false;
-    __builtin_amdgcn_s_sleep(1);
-  }
-  return true;
-}
-
 template <int DT, int OP>
 __global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs a) {
   using S = typename Elem<DT>::store_t;
@@ -65,9 +55,9 @@ __global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs 
   } else if (part) {
     for (uint32_t e = 0; e < a.tail; ++e) vec_set<DT>(mine, (int)e, ((const S*)a.in)[v * VE + e]);
   }
-  if (whole || part) ((u32x4*)a.stage[a.rank])[v] = mine.v;
-  // 2. publish: the tile is written back before the flag can be seen
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  if (whole || part) store_vec_coherent(&((u32x4*)a.stage[a.rank])[v], mine.v);  // written through
+  // 2. publish: the tile has reached memory before the flag can be seen
+  wait_own_stores();
   if (lane == 0) __hip_atomic_store(a.flag[a.rank] + tile, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   // 3. wait for the same tile of every peer
   bool ok = true;
@@ -75,7 +65,7 @@ __global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs 
     ok = wait_flag32(a.flag[lane] + tile, a.epoch, a.limit_ticks);
     if (!ok) report_late(a.status, lane, a.epoch);
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the loads below stay below the wait
   // a tile whose peers did not arrive is left alone (the failure is reported through `status`)
   if (__builtin_amdgcn_ballot_w64(!ok) != 0) return;
   if (!(whole || part)) return;
@@ -86,7 +76,7 @@ __global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs 
   for (int k = 0; k < kFusedRanks; ++k) {
     if (k < a.n) {
       if (k == a.rank) x[k].v = mine.v;
-      else x[k].v = __builtin_nontemporal_load(&((const u32x4*)a.stage[k])[v]);
+      else x[k].v = load_vec_coherent(&((const u32x4*)a.stage[k])[v]);  // past the caches: written by another rank just now
     }
   }
   A acc[VE];

@@ -48,13 +48,52 @@ struct LeanBarrierArgs {
 };
 static_assert(sizeof(LeanBarrierArgs) <= 104, "lean barrier arguments must stay below the launch-cost step");
 
+// 16 bytes written through to memory / read past the caches (system scope), as two 64-bit accesses
+// the compiler keeps track of.  For data that a wavefront of another rank (or another workgroup of
+// this kernel) produces or consumes while this kernel runs: coherence per access instead of a
+// cache-wide write-back or invalidate per tile, which with thousands of tiles and several
+// processes on the GPU costs far more than the data movement itself.
+__device__ __forceinline__ void store_vec_coherent(u32x4* p, u32x4 x) {
+  uint64_t* q = (uint64_t*)p;
+  __hip_atomic_store(q, (uint64_t)x.x | ((uint64_t)x.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(q + 1, (uint64_t)x.z | ((uint64_t)x.w << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__device__ __forceinline__ u32x4 load_vec_coherent(const u32x4* p) {
+  const uint64_t* q = (const uint64_t*)p;
+  const uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return (u32x4){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+}
+
+// Everything this wavefront has stored has reached its destination (for written-through stores:
+// memory) -- what has to hold before a flag that announces the data is stored.
+__device__ __forceinline__ void wait_own_stores() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Polls *word until it is at least `epoch` (64-bit, monotonic).  Returns false at the time limit.
+// Between polls the wavefront sleeps about half a microsecond: thousands of workgroups of several
+// processes may be waiting on the same few words.
 __device__ __forceinline__ bool wait_flag64(const uint64_t* word, uint64_t epoch, uint64_t limit_ticks) {
+  if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= epoch) return true;
   const uint64_t t0 = wall_clock64();
-  while (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) < epoch) {
+  do {
     if (wall_clock64() - t0 > limit_ticks) return false;
-    __builtin_amdgcn_s_sleep(1);
-  }
+    __builtin_amdgcn_s_sleep(16);
+  } while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < epoch);
+  return true;
+}
+
+// The same for 32-bit epochs, which wrap: compared as a signed distance.
+__device__ __forceinline__ bool wait_flag32(const uint32_t* word, uint32_t epoch, uint64_t limit_ticks) {
+  if ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) >= 0) return true;
+  const uint64_t t0 = wall_clock64();
+  do {
+    if (wall_clock64() - t0 > limit_ticks) return false;
+    __builtin_amdgcn_s_sleep(8);
+  } while ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) < 0);
   return true;
 }
 
@@ -71,6 +110,10 @@ __device__ __forceinline__ void report_late(uint32_t* status, int late_rank, uin
 //   begin: workgroup 0 publishes `ready_epoch` in this rank's word ("this rank's stream has reached
 //          the collective: its input is complete"); every workgroup waits until all words have
 //          reached it.  Workgroups dispatched later find the words set and pass with one load each.
+//          What the peers wrote before their launch is in memory by then (a finished kernel's
+//          writes are written back), but a stale copy may sit in a cache of this kernel's own: the
+//          callers read the peers' buffers past the caches (load_vec_coherent) instead of
+//          invalidating per workgroup.
 //   end:   every workgroup counts itself out; the last one publishes `done_epoch` ("this rank has
 //          finished reading the peers' buffers") and waits until every rank has done the same, so the
 //          kernel -- and with it the stream -- does not complete before the peers are done with
@@ -91,6 +134,9 @@ struct XSync {
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
 __device__ __forceinline__ bool xsync_begin(const XSync& x) {
   const int lane = threadIdx.x & (kWave - 1);
+#ifdef MCCL_XRANK_TRACE
+  if (blockIdx.x == 0 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[1] = wall_clock64();
+#endif
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
     __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   bool ok = true;
@@ -98,22 +144,33 @@ __device__ __forceinline__ bool xsync_begin(const XSync& x) {
     ok = wait_flag64(x.word[lane], x.ready_epoch, x.limit_ticks);
     if (!ok) report_late(x.status, lane, (uint32_t)x.ready_epoch);
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // nothing below moves above the wait
+#ifdef MCCL_XRANK_TRACE
+  if (blockIdx.x == 0 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[2] = wall_clock64();
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[3] = wall_clock64();
+#endif
   return __builtin_amdgcn_ballot_w64(!ok) == 0;
 }
 
 // Call once per workgroup, by all its lanes, after the workgroup's last access to a peer's buffer.
 __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
   if (x.done_epoch == 0) return;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+  // this workgroup's reads of the peers' buffers have returned (their values were used): no cache
+  // needs writing back for that
+  wait_own_stores();
   __syncthreads();
   if (threadIdx.x >= kWave) return;  // the first wavefront of the workgroup does the rest
   const int lane = threadIdx.x;
   uint32_t last = 0;
   if (lane == 0) {
-    const uint32_t before = __hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    // relaxed: the ordering that matters (this workgroup's accesses are complete) was established
+    // above, and an acquire-release atomic would add a cache write-back and invalidate per workgroup
+    const uint32_t before = __hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last = before + 1 == workgroups ? 1u : 0u;
     if (last) {
+#ifdef MCCL_XRANK_TRACE
+      if (x.status) ((uint64_t*)x.status)[4] = wall_clock64();
+#endif
       __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
       __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -123,6 +180,9 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
   if (lane < x.n && lane != x.rank) {
     if (!wait_flag64(x.word[lane], x.done_epoch, x.limit_ticks)) report_late(x.status, lane, (uint32_t)x.done_epoch);
   }
+#ifdef MCCL_XRANK_TRACE
+  if (lane == 0 && x.status) ((uint64_t*)x.status)[5] = wall_clock64();
+#endif
 }
 
 template <typename ARGS>

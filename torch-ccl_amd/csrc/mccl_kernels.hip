@@ -763,6 +763,13 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsy
     a.copy.chunk_prefix[++m] = (uint32_t)chunks;
   }
   a.copy.nseg = m;  // may be 0: the launch still takes part in the waits
+  // Full chunks of 8-byte aligned sources are read past the caches; whatever else there is (heads,
+  // partial chunks, misaligned sources) is read through them, after an invalidate per workgroup.
+  a.invalidate = 0;
+  for (int k = 0; k < m; ++k) {
+    const CopySeg& cs = a.copy.seg[k];
+    if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
+  }
   const unsigned grid = xrank_grid(chunks, a.sync.n);
   hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
@@ -796,6 +803,10 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
   a.tail1 = (uint32_t)(count % ve);
   a.tiles1 = (uint32_t)((vecs + kWave - 1) / kWave);
   a.stream_out = count * es >= (32u << 20) ? 1u : 0u;
+  a.aligned_in = 1;
+  for (int k = 0; k < a.sync.n; ++k)
+    if (count && ((uintptr_t)in[k] & 7u)) a.aligned_in = 0;
+  if (a.tail1) a.aligned_in = 0;  // the last elements are read one by one, through the caches
   hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n), (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
@@ -840,6 +851,10 @@ int mccl_allreduce_sync(void* const* tensors, void* const* stage, void* const* t
   a.tail1 = (uint32_t)(n_me % ve);
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
   a.tile_epoch = tile_epoch;
+  a.aligned_in = 1;
+  for (int k = 0; k < n; ++k)
+    if (count && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
+  if (a.tail1) a.aligned_in = 0;  // the last elements are read one by one, through the caches
   uint32_t tiles2 = 0;
   for (int q = 0; q < n; ++q) {
     const uint64_t bytes = (uint64_t)shard_len(q) * es;

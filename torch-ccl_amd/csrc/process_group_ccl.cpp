@@ -64,7 +64,12 @@ constexpr size_t kArenaFusedFlagsOff = 4096;                 // two sets of tile
 constexpr size_t kArenaFusedFlagsStride = 8192;
 constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buffers of 1 MiB, each
 constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
-constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
+constexpr size_t kArenaDoneCountOff = 256;  // 32-bit workgroup counter of the one-launch collectives
+// flags of the one-launch large allreduce: two sets of 64 Ki (one per 4 KiB: shards of up to 256 MiB)
+constexpr size_t kXrankFlagTiles = 64u << 10;
+constexpr size_t kArenaXrankFlagsOff = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
+constexpr size_t kArenaXrankFlagsStride = kXrankFlagTiles * 4;
+constexpr size_t kArenaBytes = kArenaXrankFlagsOff + 2 * kArenaXrankFlagsStride;
 static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
 
 #define HIP_CHECK(expr)                                                                     \
@@ -280,8 +285,15 @@ ProcessGroupCCL::WorkCCL::~WorkCCL() {
 }
 
 bool ProcessGroupCCL::WorkCCL::isCompleted() {
-  if (!end_) return true;
-  return hipEventQuery(end_) == hipSuccess;
+  if (end_) return hipEventQuery(end_) == hipSuccess;
+  if (!stream_set_) return true;
+  // No event was recorded for this collective (it ran on the caller's stream; with several
+  // processes on one GPU an event record costs more than the collective's kernel): the stream
+  // having drained is the conservative answer.
+  const hipError_t e = hipStreamQuery(stream_);
+  if (e == hipErrorNotReady) return false;
+  (void)hipGetLastError();
+  return true;  // drained, or the stream no longer exists
 }
 
 bool ProcessGroupCCL::WorkCCL::isSuccess() const {
@@ -295,26 +307,41 @@ std::exception_ptr ProcessGroupCCL::WorkCCL::exception() const {
   return std::make_exception_ptr(std::runtime_error(why));
 }
 
-void ProcessGroupCCL::WorkCCL::waitInternal(std::chrono::milliseconds timeout) {
+// The caller's current stream waits for the collective: through its end event; or, when none was
+// recorded, not at all on the stream the collective ran on, and through an event recorded now (at
+// that stream's current end, which is later than the collective's: conservative) on any other.
+void ProcessGroupCCL::WorkCCL::orderCurrentStreamAfter() {
+  hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
   if (end_) {
-    if (blocking_wait_) {
-      // synchronizeInternal of the reference (src/utils.h:295-319): poll until done or timed out
-      const std::chrono::milliseconds limit = timeout == kNoTimeout ? op_timeout_ : timeout;
-      unsigned spins = 0;
-      while (hipEventQuery(end_) != hipSuccess) {
-        if (limit.count() > 0) {
-          const auto ran = std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now() - start_);
-          TORCH_CHECK(ran < limit, "[Rank ", rank_, "] Caught collective operation timeout:  ran for ", ran.count(),
-                      " milliseconds before timing out.");
-        }
-        if (++spins > 200) std::this_thread::sleep_for(std::chrono::microseconds(50));
+    HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+  } else if (stream_set_ && cur != stream_) {
+    end_ = shared_ ? shared_->getEvent() : nullptr;
+    if (!end_) HIP_CHECK(hipEventCreateWithFlags(&end_, hipEventDisableTiming));
+    HIP_CHECK(hipEventRecord(end_, stream_));
+    HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+  }
+}
+
+void ProcessGroupCCL::WorkCCL::waitInternal(std::chrono::milliseconds timeout) {
+  if (blocking_wait_) {
+    // synchronizeInternal of the reference (src/utils.h:295-319): poll until done or timed out
+    const std::chrono::milliseconds limit = timeout == kNoTimeout ? op_timeout_ : timeout;
+    unsigned spins = 0;
+    while (!isCompleted()) {
+      if (limit.count() > 0) {
+        const auto ran = std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now() - start_);
+        TORCH_CHECK(ran < limit, "[Rank ", rank_, "] Caught collective operation timeout:  ran for ", ran.count(),
+                    " milliseconds before timing out.");
       }
-    } else {
-      // stream-ordered: the caller's current stream waits for the collective (the queue barrier
-      // of src/gpu/dpcpp_ccl.cpp:440-457)
-      hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
-      HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
+      // yield for the first few milliseconds (a sleeping thread wakes up tens of microseconds late,
+      // which would show up as skew between the ranks at their next collective), sleep afterwards
+      if (++spins > 20000) std::this_thread::sleep_for(std::chrono::microseconds(50));
+      else if (spins > 100) sched_yield();
     }
+  } else {
+    // stream-ordered (the queue barrier of src/gpu/dpcpp_ccl.cpp:440-457)
+    c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
+    orderCurrentStreamAfter();
   }
   if (shared_) {
     const std::string why = shared_->failureMessage();
@@ -334,20 +361,17 @@ std::vector<at::Tensor> ProcessGroupCCL::WorkCCL::result() { return outputs_; }
 c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupCCL::WorkCCL::getFuture() {
   if (!future_) {
     std::vector<c10::Device> devs;
-    if (end_) devs.emplace_back(at::kCUDA, (c10::DeviceIndex)device_);
+    if (end_ || stream_set_) devs.emplace_back(at::kCUDA, (c10::DeviceIndex)device_);
     future_ = c10::make_intrusive<at::ivalue::Future>(c10::ListType::create(c10::TensorType::get()), devs);
     if (auto err = exception()) {  // finishAsyncWorkCCLError of the reference: the future carries the error
       future_->setError(err);
       return future_;
     }
-    if (end_) {
+    if (end_ || stream_set_) {
       c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device_));
-      hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device_).stream();
-      HIP_CHECK(hipStreamWaitEvent(cur, end_, 0));
-      future_->markCompleted(at::IValue(outputs_));  // records the current stream: ordered after end_
-    } else {
-      future_->markCompleted(at::IValue(outputs_));
+      orderCurrentStreamAfter();
     }
+    future_->markCompleted(at::IValue(outputs_));  // records the current stream: ordered after the collective
   }
   return future_;
 }
@@ -391,6 +415,8 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   profile_ = envFlag("MCCL_PG_PROFILE", false);
   if (const char* v = std::getenv("MCCL_PG_SYNC")) want_device_sync_ = std::string(v) != "host";
   zero_copy_ = envFlag("MCCL_PG_ZERO_COPY", true);
+  comm_stream_for_large_ = envFlag("MCCL_PG_COMM_STREAM", false);
+  if (const char* v = std::getenv("MCCL_PG_ONE_LAUNCH_MAX_BYTES")) one_launch_max_ = (size_t)std::atoll(v);
   // The staging window can be shrunk (never enlarged) so that tests reach every windowed path
   // with small tensors.
   stage_max_ = kStageMaxDefault;
@@ -432,7 +458,7 @@ ProcessGroupCCL::~ProcessGroupCCL() {
   // finished its kernels, so a timeout here is harmless.
   (void)hipSetDevice(device_);
   if (comm_stream_) (void)hipStreamSynchronize(comm_stream_);
-  if (tail_pending_) (void)hipEventSynchronize(tail_event_);
+  if (tail_pending_) (void)hipStreamSynchronize(tail_stream_);
   // Leaving never advances the barrier epoch (a rank that leaves early must not satisfy its
   // peers' next barrier); it raises a flag instead.
   ctl_->slot[rank_].departed.store(1, std::memory_order_release);
@@ -579,7 +605,9 @@ void ProcessGroupCCL::ensureInit(int device) {
     for (int sl = 0; sl < 2; ++sl) {
       fused_stage_[sl].assign((size_t)size_, nullptr);
       fused_flags_[sl].assign((size_t)size_, nullptr);
+      xrank_flags_[sl].assign((size_t)size_, nullptr);
     }
+    done_counter_ = static_cast<char*>(arena_) + kArenaDoneCountOff;
     for (int r = 0; r < size_; ++r) {
       char* base = nullptr;
       if (r == rank_) {
@@ -597,6 +625,7 @@ void ProcessGroupCCL::ensureInit(int device) {
       for (int sl = 0; sl < 2; ++sl) {
         fused_flags_[sl][(size_t)r] = base + kArenaFusedFlagsOff + (size_t)sl * kArenaFusedFlagsStride;
         fused_stage_[sl][(size_t)r] = base + kArenaFusedStageOff + (size_t)sl * kArenaFusedStageStride + stageOffset(r);
+        xrank_flags_[sl][(size_t)r] = base + kArenaXrankFlagsOff + (size_t)sl * kArenaXrankFlagsStride;
       }
     }
     peer_arena_[(size_t)rank_] = nullptr;
@@ -637,7 +666,8 @@ void ProcessGroupCCL::publishStage(int slot, int pub) {
 }
 
 void ProcessGroupCCL::quiesce() {
-  if (tail_pending_) HIP_CHECK(hipEventSynchronize(tail_event_));
+  if (tail_pending_) HIP_CHECK(hipStreamSynchronize(tail_stream_));
+  tail_pending_ = false;
 }
 
 const void* ProcessGroupCCL::peerStage(int peer, int slot, int pub) {
@@ -864,8 +894,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
 
   auto cur_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_);
   hipStream_t cur = cur_stream.stream();
+  // Which stream: the reference runs collectives on a communication stream that waits for the
+  // caller's (src/gpu/dpcpp_ccl.cpp:186-197) unless CCL_SAME_STREAM=1.  Here all ranks share one
+  // GPU, where the fork and join (two event records, two stream waits: packets of their own that
+  // each wait for the process's turn at the dispatcher) cost several times the collective, and a
+  // second queue per process with a waiting kernel in it makes the scheduler time-slice (measured:
+  // 14 ms per collective with 8 processes).  So device-synchronised groups stay on the caller's
+  // stream unless MCCL_PG_COMM_STREAM=1; host-synchronised ones use the communication stream for
+  // large messages as before.
   const size_t payload = std::max(plan.stage_bytes, plan.share ? plan.share_bytes : (size_t)0);
-  const bool same_stream = same_stream_ || payload <= kInlineStreamMax;
+  const bool same_stream = same_stream_ || payload <= kInlineStreamMax || (device_sync_ && !comm_stream_for_large_);
   hipStream_t s = same_stream ? cur : comm_stream_;
   if (!same_stream) {  // sync_streams of the reference (src/gpu/dpcpp_ccl.cpp:186-197)
     HIP_CHECK(hipEventRecord(fork_event_, cur));
@@ -910,7 +948,7 @@ void ProcessGroupCCL::runHostSynced(Plan& plan, hipStream_t s, int slot) {
     // barrier per collective plus the two alternating buffers give both, provided the
     // synchronisation below covers this rank's earlier kernels.  On one stream it does; a
     // previous collective that ran on another stream is waited for through its tail event.
-    if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipEventSynchronize(tail_event_));
+    if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipStreamSynchronize(tail_stream_));
     HIP_CHECK(hipStreamSynchronize(s));
   } catch (...) {
     // this rank will not arrive: tell the peers now instead of letting them run into the timeout
@@ -970,7 +1008,12 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
   try {
     awaitPeersEntered(seq);
     // a rank's collectives are totally ordered on the device, whichever streams they use
-    if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipStreamWaitEvent(s, tail_event_, 0));
+    // (the event is only recorded when a collective changes streams: a record is a packet of its
+    // own, and with several processes on one GPU every packet waits for the process's turn)
+    if (tail_pending_ && tail_stream_ != s) {
+      HIP_CHECK(hipEventRecord(tail_event_, tail_stream_));
+      HIP_CHECK(hipStreamWaitEvent(s, tail_event_, 0));
+    }
     if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS) {
       const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
       MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
@@ -1022,6 +1065,28 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
     }
     if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
+    if (zero_copy && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS && plan.share_bytes <= one_launch_max_) {
+      // One launch: the kernel itself announces this rank, waits for the others, does the work
+      // and (where a tensor must not be touched before the peers have read it) waits again.  With
+      // several processes on the GPU every launch waits for its turn at the dispatcher, so this
+      // is worth more than any bandwidth.
+      pv.tile_flags = xrank_flags_[slot];
+      pv.tile_flag_count = kXrankFlagTiles;
+      pv.tile_epoch = (uint32_t)(seq + 1);
+      mccl_xsync_t sync;
+      sync.words = bar_flags_.data();
+      sync.n = size_;
+      sync.rank = rank_;
+      sync.ready_epoch = epoch + 1;
+      sync.done_epoch = epoch + 3;
+      sync.done_counter = done_counter_;
+      sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
+      sync.status = status_dev_;
+      if (plan.exec_sync(pv, sync, s)) {
+        if (timed) { phase_us_[2].push_back(0.f); phase_us_[3].push_back((float)us_since(t0)); }
+        return;
+      }
+    }
     if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
     deviceBarrier(epoch + 1, s);  // every rank's input is complete (staged, or ready in place)
     if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
@@ -1043,7 +1108,6 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work) {
   if (device_work) {
-    HIP_CHECK(hipEventRecord(tail_event_, s));
     tail_stream_ = s;
     tail_pending_ = true;
   }
@@ -1051,9 +1115,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_
   work->device_ = device_;
   work->shared_ = shared_;
   work->op_timeout_ = timeout_;
-  work->end_ = shared_->getEvent();
-  HIP_CHECK(hipEventRecord(work->end_, s));
-  if (!same_stream) {  // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
+  work->stream_ = s;
+  work->stream_set_ = true;
+  if (!same_stream) {
+    // the collective ran on the communication stream: its end is an event the caller's streams
+    // can wait for
+    work->end_ = shared_->getEvent();
+    HIP_CHECK(hipEventRecord(work->end_, s));
+    // record_tensor of the reference (src/gpu/dpcpp_ccl.cpp:199-207)
     auto cs = c10::hip::getStreamFromExternalMasqueradingAsCUDA(comm_stream_, (c10::DeviceIndex)device_);
     for (const auto* list : {&plan.inputs, &plan.outputs})
       for (const auto& t : *list)
@@ -1137,6 +1206,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
         mccl_segment_t seg{pv.zero_copy ? pv.user[(size_t)root] : pv.stage[(size_t)root], base, len};
         MCCL_CHECK(mccl_copy_segments(&seg, 1, s));
       };
+    if (len) {
+      const int me = rank_;
+      p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+        mccl_segment_t seg{pv.user[(size_t)root], base, len};
+        MCCL_CHECK(mccl_copy_segments_sync(&seg, me == root ? 0 : 1, &sync, s));  // the root only takes part in the waits
+        return true;
+      };
+    }
     work = run(p);
     off += len;
   } while (off < total);
@@ -1220,6 +1297,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
           void* red = (char*)pv.stage[(size_t)me] + (size_t)me * shard * es;  // pv.stage[me] is this rank's own staging buffer
           MCCL_CHECK(mccl_reduce_n(in.data(), W, red, n_me, dtype, op, MCCL_VARIANT_AUTO, s));
         }
+      };
+      p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+        if ((shard * es + MCCL_SYNC_FLAG_BYTES - 1) / MCCL_SYNC_FLAG_BYTES > pv.tile_flag_count) return false;
+        std::vector<void*> tensors((size_t)W), stages((size_t)W);
+        for (int k = 0; k < W; ++k) {
+          tensors[(size_t)k] = const_cast<void*>(pv.user[(size_t)k]);
+          stages[(size_t)k] = const_cast<void*>(pv.stage[(size_t)k]);
+        }
+        MCCL_CHECK(mccl_allreduce_sync(tensors.data(), stages.data(), pv.tile_flags.data(), len, dtype, op, pv.tile_epoch, &sync, s));
+        return true;
       };
       p.exec2 = [=](const PeerView& pv, hipStream_t s) {
         // the finished shard of rank r: the start of its staging buffer (zero-copy) or shard r of it
@@ -1326,6 +1413,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
         for (int r = 0; r < W; ++r)
           segs[(size_t)r] = {pv.zero_copy ? pv.user[(size_t)r] : pv.stage[(size_t)r], out + (size_t)r * per_rank, len};
         MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
+      };
+      p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+        std::vector<mccl_segment_t> segs((size_t)W);
+        for (int r = 0; r < W; ++r) segs[(size_t)r] = {pv.user[(size_t)r], out + (size_t)r * per_rank, len};
+        MCCL_CHECK(mccl_copy_segments_sync(segs.data(), W, &sync, s));
+        return true;
       };
     }
     work = run(p);
@@ -1495,6 +1588,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
         } else {
           MCCL_CHECK(mccl_reduce_scatter_n(pv.stage.data(), W, &o, len, me, 1, dtype, op, s));
         }
+      };
+      p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+        std::vector<const void*> src((size_t)W);
+        for (int k = 0; k < W; ++k) src[(size_t)k] = (const char*)pv.user[(size_t)k] + ((size_t)me * M + m0) * es;
+        MCCL_CHECK(mccl_reduce_sync(src.data(), out, len, dtype, op, &sync, s));
+        return true;
       };
     }
     work = run(p);
@@ -1704,7 +1803,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
       p.copy_in = [=](void* stage, hipStream_t s) {
         copyAsync(stage, (const char*)input.data_ptr() + w0, wlen, s);
       };
-    p.exec = [=](const PeerView& pv, hipStream_t s) {
+    // the segments this rank pulls in this window (and, from the tables, how many windows there are)
+    auto pulls = [=](const PeerView& pv) {
       size_t largest = 0;
       std::vector<mccl_segment_t> segs;
       for (int r = 0; r < W; ++r) {
@@ -1721,7 +1821,16 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
                           (char*)output.data_ptr() + recv_off[(size_t)r] + (lo - seg0), hi - lo});
       }
       *nwin = std::max<size_t>(1, (largest + window - 1) / window);
+      return segs;
+    };
+    p.exec = [=](const PeerView& pv, hipStream_t s) {
+      const auto segs = pulls(pv);
       if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+    };
+    p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+      const auto segs = pulls(pv);
+      MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), &sync, s));  // empty: still takes part in the waits
+      return true;
     };
     work = run(p);
   }

@@ -27,6 +27,8 @@
 #pragma once
 
 #include <hip/hip_runtime_api.h>
+
+#include "mccl.h"
 #include <torch/csrc/distributed/c10d/Backend.hpp>
 #include <torch/csrc/distributed/c10d/Store.hpp>
 #include <torch/csrc/distributed/c10d/Types.hpp>
@@ -93,7 +95,10 @@ class ProcessGroupCCL : public c10d::Backend {
    private:
     friend class ProcessGroupCCL;
     void waitInternal(std::chrono::milliseconds timeout);
-    hipEvent_t end_ = nullptr;
+    void orderCurrentStreamAfter();
+    hipEvent_t end_ = nullptr;      // recorded after the collective, when it ran on the communication stream
+    hipStream_t stream_ = nullptr;  // the stream the collective ran on
+    bool stream_set_ = false;
     std::shared_ptr<GroupShared> shared_;
     std::chrono::milliseconds op_timeout_{0};
     std::chrono::steady_clock::time_point start_;
@@ -208,8 +213,15 @@ class ProcessGroupCCL : public c10d::Backend {
     std::vector<const int64_t*> tables;     // the scalars rank r published
     bool zero_copy = false;                 // the peers' tensors are read in place: nothing was staged
     std::vector<const void*> user;          // zero_copy: rank r's published tensor range
+    std::vector<void*> tile_flags;          // zero_copy: rank r's tile flags of the one-launch allreduce (this slot)
+    size_t tile_flag_count = 0;             // entries of each
+    uint32_t tile_epoch = 0;
   };
   using ExecFn = std::function<void(const PeerView& pv, hipStream_t s)>;
+  // The whole device side of a zero-copy collective as ONE launch with the rank waits inside the
+  // kernel (mccl_*_sync).  Returns false when the collective does not fit that form; the engine then
+  // runs barrier kernels around exec / exec2.
+  using SyncExecFn = std::function<bool(const PeerView& pv, mccl_xsync_t& sync, hipStream_t s)>;
 
   // What one collective needs from the engine.
   struct Plan {
@@ -227,6 +239,7 @@ class ProcessGroupCCL : public c10d::Backend {
     // used by the two-shot allreduce.  two_phase, when set, says whether this run needs it.
     ExecFn exec2;
     std::function<bool(const PeerView& pv)> two_phase;
+    SyncExecFn exec_sync;
     // Zero-copy offer (device-synchronised groups only): the byte range of the caller's tensor
     // that the peers may read in place of a staged copy.  `share` must come out the same on every
     // rank (it may depend on sizes all ranks agree on, never on this rank's own).  The offer is
@@ -293,6 +306,12 @@ class ProcessGroupCCL : public c10d::Backend {
   bool profile_ = false;        // MCCL_PG_PROFILE: host-side phase timers, printed when the group dies
   bool want_device_sync_ = true;  // MCCL_PG_SYNC != "host"
   bool zero_copy_ = true;         // MCCL_PG_ZERO_COPY != 0
+  // Largest tensor (bytes per rank) whose zero-copy collective is ONE launch with the rank waits
+  // inside the kernel; larger ones run the bandwidth-tuned kernels between barrier kernels (the
+  // persistent one-launch kernels move fewer bytes per second, which outweighs the saved launches
+  // from a few hundred MiB of traffic on).  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides.
+  size_t one_launch_max_ = 32u << 20;
+  bool comm_stream_for_large_ = false;  // MCCL_PG_COMM_STREAM=1: device-synchronised groups fork large collectives too
   // Decided at start-up, the same on every rank: all ranks are processes of their own (and the
   // environment does not ask for the host barrier), so cross-rank waits can live on the device.
   bool device_sync_ = false;
@@ -346,6 +365,8 @@ class ProcessGroupCCL : public c10d::Backend {
   std::vector<void*> final_flags_;          // rank r's departure word
   std::vector<void*> fused_stage_[2];       // rank r's staging buffer of the one-launch allreduce, per slot
   std::vector<void*> fused_flags_[2];
+  std::vector<void*> xrank_flags_[2];       // rank r's tile flags of the one-launch large allreduce, per slot
+  void* done_counter_ = nullptr;            // this rank's workgroup counter of the one-launch collectives
   void* status_dev_ = nullptr;              // device address of shared_->status
   std::shared_ptr<GroupShared> shared_;
 
