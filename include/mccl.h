@@ -119,6 +119,11 @@ size_t mccl_dtype_size(int dtype);
  *   - order: ascending rank; SUM starts from +0 like the reference's "result = 0".
  *   - f16 / bf16 accumulate in fp32 and round once (nearest even) on store; f32, f64 and
  *     the integer types accumulate in their own type (integers wrap).
+ *   - NaN: SUM / AVG / PROD follow IEEE arithmetic.  MIN / MAX propagate NaN whatever the rank
+ *     order (a NaN input replaces the accumulator, nothing replaces a NaN accumulator), like
+ *     torch.min / torch.max; the result is the NaN of the highest rank that holds one.  f16 /
+ *     bf16 results that are NaN are stored as the canonical quiet NaN (0x7E00 / 0x7FC0); f32 /
+ *     f64 NaN payloads of arithmetic results are not part of the contract.
  *   - out may be exactly one of the inputs (in place; on large messages that is 3-5 % faster than
  *     a separate output: the write lands on DRAM pages just read); any other overlap between an output and
  *     a range the same launch reads or writes is refused with MCCL_ERR_INVALID_ARG (this holds

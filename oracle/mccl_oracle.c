@@ -30,11 +30,14 @@
  *               tagged tiny inputs), fp32 N=2 sum (commutative, one value possible),
  *               integer sums (associative), fp32->bf16 / fp32<->fp16 conversions
  *               (checked against numpy / torch CPU conversions).
+ *               AVG (this build's addition): closed forms that a wrong order of divide and
+ *               round fails (tests/test_oracle_pins.py).
  *   parity unpinned : the rounding ORDER of float reductions for N >= 3 inside the
  *               un-vendored oneCCL library, oneCCL's own bf16/fp16 arithmetic, and
- *               NaN payload / MIN,MAX-with-NaN behaviour.  The oracle uses the
+ *               NaN payload / MIN,MAX-with-NaN behaviour of oneCCL.  The oracle uses the
  *               ascending-rank fp32 chain with one final round-to-nearest-even, the
- *               order the in-tree small kernel uses.
+ *               order the in-tree small kernel uses, and propagates NaN through MIN / MAX
+ *               (what torch.min / torch.max do).
  *
  * Build: see oracle/Makefile (gcc -O2 -fopenmp, no fast-math, no FMA contraction).
  */
@@ -49,7 +52,7 @@
 /* dtype and op codes: same numbering as include/mccl.h */
 enum { DT_U8 = 0, DT_I8 = 1, DT_I16 = 2, DT_I32 = 3, DT_I64 = 4,
        DT_F16 = 5, DT_F32 = 6, DT_F64 = 7, DT_BF16 = 8 };
-enum { OP_SUM = 0, OP_PROD = 2, OP_MIN = 3, OP_MAX = 4 };
+enum { OP_SUM = 0, OP_AVG = 1, OP_PROD = 2, OP_MIN = 3, OP_MAX = 4 };
 
 static int g_threads = 1;
 
@@ -125,20 +128,27 @@ uint16_t oracle_f32_to_f16(float f)
 /* ---------- the N-buffer reduction ---------- */
 
 /* One element of the chain.  SUM starts from literal +0 and adds rank 0..N-1
- * (allreduce_small.h:347-352); the other ops start from rank 0's value. */
+ * (allreduce_small.h:347-352); the other ops start from rank 0's value.
+ * AVG (floats only; the reference rejects it on device, dispatch_stub.h:320-335) is the SUM
+ * chain followed by ONE division by n in the accumulation type, then the single rounding to the
+ * storage type.
+ * MIN / MAX propagate NaN whatever the rank order: a NaN input replaces the accumulator
+ * (x != x), and no later value replaces a NaN accumulator (both compares are false), so the
+ * result is the NaN of the highest rank that holds one, bits untouched. */
 #define REDUCE_FLOAT_CHAIN(ACC_T, LOAD, STORE)                         \
   for (size_t i = 0; i < count; ++i) {                                 \
     ACC_T acc;                                                         \
-    if (op == OP_SUM) {                                                \
+    if (op == OP_SUM || op == OP_AVG) {                                \
       acc = (ACC_T)0;                                                  \
       for (int r = 0; r < n; ++r) acc = acc + LOAD(r, i);              \
+      if (op == OP_AVG) acc = acc / (ACC_T)n;                          \
     } else {                                                           \
       acc = LOAD(0, i);                                                \
       for (int r = 1; r < n; ++r) {                                    \
         ACC_T x = LOAD(r, i);                                          \
         if (op == OP_PROD) acc = acc * x;                              \
-        else if (op == OP_MIN) acc = (x < acc) ? x : acc;              \
-        else acc = (x > acc) ? x : acc;                                \
+        else if (op == OP_MIN) acc = (x < acc || x != x) ? x : acc;    \
+        else acc = (x > acc || x != x) ? x : acc;                      \
       }                                                                \
     }                                                                  \
     STORE(i, acc);                                                     \
@@ -230,7 +240,8 @@ int oracle_reduce(const void* const* in, int n, void* out, size_t count, int dty
 {
   size_t es = oracle_dtype_size(dtype);
   if (es == 0 || n < 1) return -1;
-  if (op != OP_SUM && op != OP_PROD && op != OP_MIN && op != OP_MAX) return -1;
+  if (op != OP_SUM && op != OP_AVG && op != OP_PROD && op != OP_MIN && op != OP_MAX) return -1;
+  if (op == OP_AVG && !(dtype == DT_F16 || dtype == DT_F32 || dtype == DT_F64 || dtype == DT_BF16)) return -1;
   int nt = g_threads;
   if (nt <= 1 || count < 4096) return reduce_range(in, n, out, count, dtype, op);
   int rc = 0;

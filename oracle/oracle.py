@@ -15,7 +15,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 # dtype / op codes, identical to include/mccl.h
 U8, I8, I16, I32, I64, F16, F32, F64, BF16 = range(9)
-SUM, PROD, MIN, MAX = 0, 2, 3, 4
+SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
 
 DTYPE_SIZE = {U8: 1, I8: 1, I16: 2, I32: 4, I64: 8, F16: 2, F32: 4, F64: 8, BF16: 2}
 # numpy carrier dtype for each code (bit patterns for the 16-bit floats)

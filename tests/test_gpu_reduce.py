@@ -105,27 +105,33 @@ def test_reduce_in_place(mccl, dtype, which):
 
 
 def _special_values(dtype):
-    """+-0, subnormals, +-inf, max-finite cancellation, rounding ties."""
+    """+-0, subnormals, +-inf, max-finite cancellation, rounding ties, and NaNs: quiet and
+    signalling, both signs, with and without payload."""
     if dtype == torch.bfloat16:
         pats = [0x0000, 0x8000, 0x0001, 0x8001, 0x007f, 0x0080, 0x7f7f, 0xff7f, 0x7f80, 0xff80,
-                0x3f80, 0xbf80, 0x3f81, 0x3c00, 0x3b80, 0x4000, 0x0100, 0x8100]
+                0x3f80, 0xbf80, 0x3f81, 0x3c00, 0x3b80, 0x4000, 0x0100, 0x8100,
+                0x7fc0, 0xffc0, 0x7f81, 0xff81, 0x7fc5]
         return torch.tensor(np.array(pats, dtype=np.uint16).view(np.int16)).view(torch.bfloat16)
     if dtype == torch.float16:
         pats = [0x0000, 0x8000, 0x0001, 0x8001, 0x03ff, 0x0400, 0x7bff, 0xfbff, 0x7c00, 0xfc00,
-                0x3c00, 0xbc00, 0x3c01, 0x1400, 0x1000, 0x4000, 0x0002, 0x8002]
+                0x3c00, 0xbc00, 0x3c01, 0x1400, 0x1000, 0x4000, 0x0002, 0x8002,
+                0x7e00, 0xfe00, 0x7c01, 0xfc01, 0x7e05]
         return torch.tensor(np.array(pats, dtype=np.uint16).view(np.int16)).view(torch.float16)
     pats = [0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x007fffff, 0x00800000, 0x7f7fffff,
             0xff7fffff, 0x7f800000, 0xff800000, 0x3f800000, 0xbf800000, 0x3f800001, 0x33800000,
-            0x33000000, 0x40000000, 0x00000002, 0x80000002]
+            0x33000000, 0x40000000, 0x00000002, 0x80000002,
+            0x7fc00000, 0xffc00000, 0x7f800001, 0xff800001, 0x7fc12345]
     return torch.tensor(np.array(pats, dtype=np.uint32).view(np.int32)).view(torch.float32)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
 @pytest.mark.parametrize("opname", ["sum", "prod", "min", "max"])
 def test_reduce_special_values(mccl, dtype, opname):
-    """Every ordered triple of special values (signed zeros, subnormals, infinities, ties).
-    NaN results are compared as "is NaN" for fp32 (payloads are not part of the contract);
-    f16/bf16 NaNs are canonical in both implementations and compared bit for bit."""
+    """Every ordered triple of special values (signed zeros, subnormals, infinities, ties, NaNs of
+    every kind in every rank position).  MIN / MAX select, so their fp32 results are compared bit
+    for bit, NaN included (the highest rank's NaN, bits untouched); NaN results of fp32 arithmetic
+    (SUM, PROD) are compared as "is NaN" (their payloads are not part of the contract); f16 / bf16
+    NaNs are canonical in both implementations and compared bit for bit."""
     v = _special_values(dtype)
     k = v.numel()
     a = v.repeat_interleave(k * k)
@@ -134,7 +140,7 @@ def test_reduce_special_values(mccl, dtype, opname):
     ins = [a.contiguous(), b.contiguous(), c.contiguous()]
     got = bits(_run(mccl, ins, OPS[opname]))
     want = oracle_reduce_bits(ins, OPS[opname])
-    if dtype == torch.float32:
+    if dtype == torch.float32 and opname in ("sum", "prod"):
         gf, wf = got.view(np.float32), want.view(np.float32)
         nan_g, nan_w = np.isnan(gf), np.isnan(wf)
         assert np.array_equal(nan_g, nan_w)
@@ -165,12 +171,48 @@ def test_reduce_avg(mccl, dtype, n, count):
     (2, 4, 8), the generic path, and a size whose output is written with streaming stores."""
     ins = [rank_buffer(count, dtype, r) for r in range(n)]
     got = _run(mccl, ins, mccl.AVG)
+    assert_bits_equal(bits(got), oracle_reduce_bits(ins, O.AVG), "avg %s n=%d vs the oracle" % (dtype, n))
+    # second witness: the same order of operations in torch on the CPU
     acc_t = torch.float64 if dtype == torch.float64 else torch.float32
     acc = torch.zeros(count, dtype=acc_t)
     for t in ins:
         acc = acc + t.to(acc_t)
     want = (acc / n).to(dtype)
     assert_bits_equal(bits(got), bits(want), "avg %s n=%d" % (dtype, n))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=str)
+def test_reduce_avg_special_values(mccl, dtype):
+    """AVG over every ordered triple of special values, against the oracle (NaN results of fp32
+    arithmetic compared as "is NaN")."""
+    v = _special_values(dtype)
+    k = v.numel()
+    ins = [v.repeat_interleave(k * k).contiguous(), v.repeat_interleave(k).repeat(k).contiguous(), v.repeat(k * k).contiguous()]
+    got = bits(_run(mccl, ins, mccl.AVG))
+    want = oracle_reduce_bits(ins, O.AVG)
+    if dtype == torch.float32:
+        nan_g, nan_w = np.isnan(got.view(np.float32)), np.isnan(want.view(np.float32))
+        assert np.array_equal(nan_g, nan_w)
+        assert_bits_equal(got[~nan_w], want[~nan_w], "avg %s" % dtype)
+    else:
+        assert_bits_equal(got, want, "avg %s" % dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.float64], ids=str)
+@pytest.mark.parametrize("opname", ["min", "max"])
+@pytest.mark.parametrize("n", [2, 3, 8])
+def test_min_max_propagate_nan_from_any_rank(mccl, dtype, opname, n):
+    """A NaN in any one rank (or in several) makes MIN / MAX NaN: specialised and generic rank
+    counts, every launch shape, bit for bit against the oracle."""
+    count = 70_001
+    for pos in range(n):
+        ins = [rank_buffer(count, dtype, r, scale=1.0) for r in range(n)]
+        ins[pos][::7] = float("nan")
+        ins[(pos + 1) % n][3::11] = -float("nan")
+        for variant in (1, 2, 3):  # small, persistent, stream
+            got = _run(mccl, ins, OPS[opname], variant=variant)
+            assert torch.isnan(got[0]) and torch.isnan(got[7]) and torch.isnan(got[3])
+            assert_bits_equal(bits(got), oracle_reduce_bits(ins, OPS[opname]), "%s %s n=%d nan in rank %d" % (dtype, opname, n, pos))
 
 
 def test_reduce_avg_rejects_integers(mccl):

@@ -263,3 +263,136 @@ def test_combine_matches_torch_fp32():
         acc = acc + torch.from_numpy(w[:, k:k + 1]) * rows_k
     want = acc.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16).reshape(-1)
     assert np.array_equal(y, want)
+
+
+# ---------------- AVG: where the division and the roundings sit ----------------
+
+def _rne(x, mant_bits, emin):
+    """Exact rational -> nearest value with `mant_bits` fraction bits (ties to even, gradual
+    underflow below 2**emin); overflow is not needed here.  Pure integer / Fraction arithmetic."""
+    from fractions import Fraction
+    if x == 0:
+        return Fraction(0)
+    sign = -1 if x < 0 else 1
+    x = abs(x)
+    e = 0
+    while Fraction(2) ** (e + 1) <= x:
+        e += 1
+    while Fraction(2) ** e > x:
+        e -= 1
+    e = max(e, emin)
+    ulp = Fraction(2) ** (e - mant_bits)
+    q, r = divmod(x, ulp)
+    if r * 2 > ulp or (r * 2 == ulp and q % 2 == 1):
+        q += 1
+    return sign * q * ulp
+
+
+def _f32(x):
+    return _rne(x, 23, -126)
+
+
+def _bf16(x):
+    return _rne(x, 7, -126)
+
+
+def _bf16_bits(x):
+    """Bit pattern of an exactly representable bf16 value."""
+    return int(np.array([float(x)], dtype=np.float32).view(np.uint32)[0] >> 16)
+
+
+def _avg_orders(xs):
+    """The defined result and three plausible wrong ones, all in exact arithmetic:
+    right  fp32 chain in rank order, ONE division in fp32, one rounding to bf16
+    a      the sum is rounded to bf16 before the division
+    b      every input is divided first, the quotients are summed
+    c      the sum is multiplied by the rounded reciprocal instead of divided"""
+    from fractions import Fraction
+    n = len(xs)
+    s = Fraction(0)
+    for x in xs:
+        s = _f32(s + x)
+    right = _bf16(_f32(s / n))
+    a = _bf16(_f32(_bf16(s) / n))
+    sb = Fraction(0)
+    for x in xs:
+        sb = _f32(sb + _f32(x / n))
+    b = _bf16(sb)
+    c = _bf16(_f32(s * _f32(Fraction(1, n))))
+    return right, a, b, c
+
+
+def test_avg_is_one_division_of_the_fp32_chain_then_one_rounding():
+    """AVG of bf16 inputs against exact rational arithmetic, on vectors picked so that each wrong
+    order of divide and round (sum rounded to bf16 first; inputs divided first; multiplication by
+    the rounded reciprocal) gives different bits than the defined order, plus random vectors."""
+    from fractions import Fraction
+    rng = np.random.default_rng(5)
+    need = {"a": 3, "b": 3, "c": 3}  # discriminating vectors still wanted per wrong order
+    checked = 0
+    for trial in range(4000):
+        n = int(rng.choice([3, 5, 6, 7]))
+        vals = torch.tensor(rng.normal(0, 1, size=n).astype(np.float32) * np.float32(2.0) ** int(rng.integers(-3, 3)))
+        vals = vals.to(torch.bfloat16)
+        xs = [Fraction(float(v)) for v in vals.float()]
+        right, a, b, c = _avg_orders(xs)
+        hits = [k for k, w in (("a", a), ("b", b), ("c", c)) if w != right and need[k] > 0]
+        if not hits and trial >= 300:
+            continue
+        for k in hits:
+            need[k] -= 1
+        carriers = [vals[r:r + 1].view(torch.int16).numpy().view(np.uint16) for r in range(n)]
+        got = int(O.reduce(carriers, O.BF16, O.AVG)[0])
+        assert got == _bf16_bits(right), (n, [hex(int(c_[0])) for c_ in carriers], hex(got), hex(_bf16_bits(right)))
+        checked += 1
+    assert all(v == 0 for v in need.values()), need  # every wrong order was told apart at least three times
+    assert checked >= 300
+
+
+def test_avg_fp32_and_fp64_divide_once_in_their_own_type():
+    """fp32: (1 + 1 + 1e-8...) style: the chain, then one division; checked against numpy scalars
+    of the same type evaluated in the same order, and against the exact-arithmetic model."""
+    from fractions import Fraction
+    rng = np.random.default_rng(6)
+    for n in (2, 3, 7):
+        x = rng.normal(0, 1, size=(n, 257)).astype(np.float32)
+        got = O.reduce([x[r].copy() for r in range(n)], O.F32, O.AVG)
+        for i in range(0, 257, 16):
+            s = Fraction(0)
+            for r in range(n):
+                s = _f32(s + Fraction(float(x[r, i])))
+            assert Fraction(float(got[i])) == _f32(s / n), (n, i)
+        xd = x.astype(np.float64)
+        gd = O.reduce([xd[r].copy() for r in range(n)], O.F64, O.AVG)
+        acc = np.zeros(257)
+        for r in range(n):
+            acc = acc + xd[r]
+        assert np.array_equal(gd, acc / n)
+    # integers have no AVG
+    with pytest.raises(Exception):
+        O.reduce([np.ones(4, np.int32), np.ones(4, np.int32)], O.I32, O.AVG)
+
+
+def test_min_max_propagate_nan_whatever_the_rank_order():
+    """A NaN in any rank makes MIN and MAX NaN (torch.min / torch.max semantics); for fp32 the bits
+    are those of the highest rank's NaN, quiet or signalling, either sign; bf16 / f16 results are
+    the canonical quiet NaN."""
+    nans = np.array([0x7fc00000, 0xffc00000, 0x7f800001, 0xff800001, 0x7fc12345], dtype=np.uint32).view(np.float32)
+    one = np.array([1.0], dtype=np.float32)
+    for op in (O.MIN, O.MAX):
+        for k, nan in enumerate(nans):
+            v = np.array([nan], dtype=np.float32)
+            for order in ([v, one, one], [one, v, one], [one, one, v]):
+                got = O.reduce([a.copy() for a in order], O.F32, op)
+                assert got.view(np.uint32)[0] == v.view(np.uint32)[0], (op, k)
+            other = np.array([nans[(k + 1) % len(nans)]], dtype=np.float32)
+            got = O.reduce([v.copy(), one.copy(), other.copy()], O.F32, op)
+            assert got.view(np.uint32)[0] == other.view(np.uint32)[0]  # the highest rank's NaN
+        for code, qnan, canon, one16 in ((O.BF16, 0x7fc1, 0x7fc0, 0x3f80), (O.F16, 0x7e01, 0x7e00, 0x3c00)):
+            for pos in range(3):
+                ins = [np.array([one16], dtype=np.uint16) for _ in range(3)]
+                ins[pos] = np.array([qnan], dtype=np.uint16)
+                assert int(O.reduce(ins, code, op)[0]) == canon
+    # and without NaN they are still the minimum / maximum, signed zeros compared as equal
+    got = O.reduce([np.array([3.0, -0.0], np.float32), np.array([-2.0, 0.0], np.float32), np.array([5.0, -0.0], np.float32)], O.F32, O.MIN)
+    assert got.tolist()[0] == -2.0 and got.view(np.uint32)[1] == 0x80000000  # first of the equal zeros is kept

@@ -141,8 +141,10 @@ __device__ __forceinline__ typename Elem<DT>::acc_t chain_next(typename Elem<DT>
   if constexpr (Elem<DT>::kIsFloat) {
     if constexpr (OP == MCCL_SUM || OP == MCCL_AVG) return acc + x;
     else if constexpr (OP == MCCL_PROD) return acc * x;
-    else if constexpr (OP == MCCL_MIN) return (x < acc) ? x : acc;
-    else return (x > acc) ? x : acc;
+    // MIN / MAX propagate NaN whatever the rank order: a NaN input replaces the accumulator, and
+    // no later value replaces a NaN accumulator (both compares are false)
+    else if constexpr (OP == MCCL_MIN) return (x < acc || x != x) ? x : acc;
+    else return (x > acc || x != x) ? x : acc;
   } else {
     using U = typename Elem<DT>::uacc_t;
     if constexpr (OP == MCCL_SUM) return (A)(U)((U)acc + (U)x);
