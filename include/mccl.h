@@ -295,6 +295,19 @@ int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, v
  * the storage type on store; bf16 / f16 / f32; rows must be a multiple of 16 bytes.  Entries
  * with rank or row out of range contribute nothing.
  */
+/*
+ * mccl_route_counts: counts[e] = number of i < npairs with expert_ids[i] == e, for e < n_experts
+ * (ids outside [0, n_experts) are ignored).  expert_ids (int32) and counts (int64, n_experts
+ * entries) are DEVICE arrays.  The counts summed per destination rank are the inputSplitSizes of
+ * the dispatch all_to_all_single (src/gpu/dpcpp_ccl.cpp:1436-1445); computing them on the device
+ * keeps the routing decision there until the one copy of n_experts numbers the host needs.
+ * workspace: n_experts 32-bit counters of device memory, 4-byte aligned, used as scratch (cleared by
+ * the call, left zero).  1 <= n_experts <= MCCL_ROUTE_MAX_EXPERTS.
+ */
+#define MCCL_ROUTE_MAX_EXPERTS 4096
+int mccl_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, void* workspace, int64_t* counts,
+                      void* stream);
+
 int mccl_gather_rows(const void* src, size_t src_rows, const int64_t* row_index, size_t nrows,
                      size_t row_bytes, void* dst, void* stream);
 int mccl_moe_dispatch_n(const void* const* hidden, const size_t* hidden_rows,

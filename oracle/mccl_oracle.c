@@ -21,7 +21,7 @@
  *   oracle_alltoallv        src/gpu/dpcpp_ccl.cpp:1428-1455, src/cpu/cpu_ccl.cpp:924-950
  *                           (rank d's segment r comes from rank r's segment d)
  *   oracle_pack/unpack      src/gpu/dpcpp_ccl.cpp:1505-1515, 1528-1538
- *   oracle_gather_rows / oracle_moe_dispatch / oracle_moe_combine
+ *   oracle_gather_rows / oracle_moe_dispatch / oracle_moe_combine / oracle_route_counts
  *                           no reference file: the callers' steps either side of the
  *                           all_to_all_single of src/gpu/dpcpp_ccl.cpp:1428-1455
  *
@@ -422,6 +422,20 @@ int oracle_moe_combine(const void* const* x, const size_t* x_rows, int n, const 
       else if (dtype == DT_F16) ((uint16_t*)y)[o] = oracle_f32_to_f16(acc);
       else ((float*)y)[o] = acc;
     }
+  }
+  return 0;
+}
+
+/* Routing counts of a MoE dispatch: counts[e] = number of pairs routed to expert e; ids outside
+ * [0, n_experts) are ignored.  No reference file: the caller's step before the all_to_all_single
+ * of src/gpu/dpcpp_ccl.cpp:1371-1466 (its inputSplitSizes are these counts summed per rank). */
+int oracle_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, int64_t* counts)
+{
+  if (n_experts < 1 || !counts) return -1;
+  for (int e = 0; e < n_experts; ++e) counts[e] = 0;
+  for (size_t i = 0; i < npairs; ++i) {
+    int32_t e = expert_ids[i];
+    if (e >= 0 && e < n_experts) counts[e] += 1;
   }
   return 0;
 }

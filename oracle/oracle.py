@@ -53,6 +53,7 @@ def lib():
         L.oracle_gather_rows.argtypes = [vp, sz, vp, sz, sz, vp]
         L.oracle_moe_dispatch.argtypes = [vp, vp, vp, vp, i32, vp, sz]
         L.oracle_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp]
+        L.oracle_route_counts.argtypes = [vp, sz, i32, vp]
         L.oracle_set_threads.argtypes = [i32]
         for name in ("f32_to_bf16", "f32_to_f16", "f16_to_f32", "bf16_to_f32"):
             getattr(L, "oracle_%s_array" % name).argtypes = [vp, vp, sz]
@@ -224,3 +225,13 @@ def moe_combine(x, src_rank, src_row, w, tokens, topk, hidden, dtype):
                                   tokens, topk, hidden, dtype, y.ctypes.data)
     assert rc == 0, rc
     return y
+
+
+def route_counts(expert_ids, n_experts):
+    """counts[e] = number of entries of expert_ids equal to e (ids out of range ignored)."""
+    ids = np.ascontiguousarray(expert_ids, dtype=np.int32).reshape(-1)
+    out = np.zeros(n_experts, dtype=np.int64)
+    rc = lib().oracle_route_counts(ids.ctypes.data, ids.size, n_experts, out.ctypes.data)
+    if rc != 0:
+        raise ValueError("oracle_route_counts failed")
+    return out

@@ -185,3 +185,30 @@ def test_gather_small_rows_skip_out_of_range_and_ragged_ends(mccl, row_bytes):
     want = O.moe_dispatch([_u8(h) for h in hid], [t.cpu().numpy() for t in ix], S, row_bytes)
     for d in range(n):
         assert_bits_equal(_u8(fused[d]), want[d], "small-row dispatch dest %d" % d)
+
+
+@pytest.mark.parametrize("n_experts,npairs", [(1, 5), (8, 0), (64, 4096 * 8), (256, 4096 * 8), (4096, 1_000_003), (257, 77)])
+def test_route_counts_match_the_oracle(mccl, n_experts, npairs):
+    """Per-expert pair counts on the device against the oracle; ids out of range are ignored; the
+    workspace comes back zero, so that a second, smaller call through the same workspace is right too."""
+    from oracle import oracle as O
+    g = torch.Generator().manual_seed(11 + n_experts)
+    ids = torch.randint(-2, n_experts + 2, (npairs,), generator=g, dtype=torch.int64).to(torch.int32)
+    ws = torch.full((n_experts,), 12345, dtype=torch.int32, device=DEV)  # dirty on purpose: the call clears it
+    got = mccl.route_counts(ids.to(DEV), n_experts, workspace=ws)
+    assert np.array_equal(got.cpu().numpy(), O.route_counts(ids.numpy(), n_experts))
+    assert int(ws.abs().sum()) == 0
+    half = ids[: npairs // 3].contiguous()
+    got = mccl.route_counts(half.to(DEV), n_experts, workspace=ws)
+    assert np.array_equal(got.cpu().numpy(), O.route_counts(half.numpy(), n_experts))
+
+
+def test_route_counts_of_the_c5_routing_give_the_split_matrix(mccl):
+    """The top-8-of-256 routing of the dispatch workload: counts summed per destination rank equal
+    torch.bincount of the destination ranks, i.e. the row of the all_to_all_single split matrix."""
+    g = torch.Generator().manual_seed(1234 * 1_000_003)
+    experts = torch.topk(torch.randn(4096, 256, generator=g), 8, dim=1).indices.to(torch.int32)
+    counts = mccl.route_counts(experts.reshape(-1).contiguous().to(DEV), 256).cpu()
+    per_rank = counts.view(8, 32).sum(dim=1)
+    assert torch.equal(per_rank, torch.bincount(experts.reshape(-1).long() // 32, minlength=8))
+    assert int(per_rank.sum()) == 4096 * 8

@@ -396,3 +396,13 @@ def test_min_max_propagate_nan_whatever_the_rank_order():
     # and without NaN they are still the minimum / maximum, signed zeros compared as equal
     got = O.reduce([np.array([3.0, -0.0], np.float32), np.array([-2.0, 0.0], np.float32), np.array([5.0, -0.0], np.float32)], O.F32, O.MIN)
     assert got.tolist()[0] == -2.0 and got.view(np.uint32)[1] == 0x80000000  # first of the equal zeros is kept
+
+
+def test_route_counts_vs_numpy_bincount():
+    """oracle_route_counts against numpy's bincount (ids out of range dropped), empty input included."""
+    rng = np.random.default_rng(9)
+    for n_experts, npairs in ((1, 10), (8, 0), (64, 1000), (256, 32768), (4096, 100000)):
+        ids = rng.integers(-3, n_experts + 3, size=npairs).astype(np.int32)
+        keep = ids[(ids >= 0) & (ids < n_experts)]
+        want = np.bincount(keep, minlength=n_experts).astype(np.int64)
+        assert np.array_equal(O.route_counts(ids, n_experts), want)

@@ -283,4 +283,44 @@ __global__ __launch_bounds__(kWave) void moe_combine_kernel(const CombineArgs a)
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Routing counts: how many (token, expert) pairs go to each expert.  The caller's step before the
+// all_to_all_single of src/gpu/dpcpp_ccl.cpp:1371-1466, whose inputSplitSizes are these counts
+// summed per destination rank.  Two kernels: a histogram into 32-bit counters (a workgroup counts
+// its share in LDS first, so the device atomics are one per expert and workgroup, not one per
+// pair), and a finish that widens the counters into the caller's int64 array and leaves them
+// zero for the next call.
+// ------------------------------------------------------------------------------------------
+constexpr int kRouteBlock = 256;
+constexpr int kRouteMaxExperts = 4096;  // LDS histogram: 16 KiB
+
+__global__ __launch_bounds__(kRouteBlock) void route_count_kernel(const int32_t* ids, uint64_t npairs, uint32_t n_experts,
+                                                                  uint32_t* counters) {
+  __shared__ uint32_t hist[kRouteMaxExperts];
+  for (uint32_t e = threadIdx.x; e < n_experts; e += kRouteBlock) hist[e] = 0;
+  __syncthreads();
+  const uint64_t stride = (uint64_t)gridDim.x * kRouteBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kRouteBlock + threadIdx.x; i < npairs; i += stride) {
+    const uint32_t e = (uint32_t)ids[i];  // negative ids become large and are ignored like any id out of range
+    if (e < n_experts) atomicAdd(&hist[e], 1u);
+  }
+  __syncthreads();
+  for (uint32_t e = threadIdx.x; e < n_experts; e += kRouteBlock) {
+    const uint32_t c = hist[e];
+    if (c) atomicAdd(&counters[e], c);
+  }
+}
+
+__global__ __launch_bounds__(kRouteBlock) void route_finish_kernel(uint32_t* counters, uint32_t n_experts, int64_t* counts) {
+  for (uint32_t e = blockIdx.x * kRouteBlock + threadIdx.x; e < n_experts; e += gridDim.x * kRouteBlock) {
+    counts[e] = (int64_t)counters[e];
+    counters[e] = 0;
+  }
+}
+
+// Zeroes a workspace the caller brought (a kernel, not a memset node: callers may capture the call).
+__global__ __launch_bounds__(kRouteBlock) void route_clear_kernel(uint32_t* counters, uint32_t n_experts) {
+  for (uint32_t e = blockIdx.x * kRouteBlock + threadIdx.x; e < n_experts; e += gridDim.x * kRouteBlock) counters[e] = 0;
+}
+
 }  // namespace

@@ -500,7 +500,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 120; }
+int mccl_version(void) { return 130; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -1036,6 +1036,46 @@ int mccl_moe_dispatch_n(const void* const* hidden, const size_t* hidden_rows,
     }
   }
   return MCCL_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+int launch_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, uint32_t* counters, bool clear_first,
+                        int64_t* counts, hipStream_t s) {
+  if (n_experts < 1 || n_experts > kRouteMaxExperts)
+    return fail(MCCL_ERR_INVALID_ARG, "expert count %d outside [1, %d]", n_experts, kRouteMaxExperts);
+  if (!counts) return fail(MCCL_ERR_INVALID_ARG, "counts pointer is null");
+  if (npairs && !expert_ids) return fail(MCCL_ERR_INVALID_ARG, "expert id pointer is null");
+  if ((uintptr_t)expert_ids % 4 || (uintptr_t)counts % 8 || (uintptr_t)counters % 4)
+    return fail(MCCL_ERR_INVALID_ARG, "expert ids, counters or counts not aligned to their element size");
+  int cus = 0;
+  int rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  const unsigned fin = (unsigned)((n_experts + kRouteBlock - 1) / kRouteBlock);
+  if (clear_first) hipLaunchKernelGGL(route_clear_kernel, dim3(fin), dim3(kRouteBlock), 0, s, counters, (uint32_t)n_experts);
+  if (npairs) {
+    uint64_t grid = (npairs + (uint64_t)kRouteBlock * 8 - 1) / ((uint64_t)kRouteBlock * 8);  // about 8 pairs per lane
+    if (grid > (uint64_t)cus * 4) grid = (uint64_t)cus * 4;
+    hipLaunchKernelGGL(route_count_kernel, dim3((unsigned)grid), dim3(kRouteBlock), 0, s, expert_ids, (uint64_t)npairs,
+                       (uint32_t)n_experts, counters);
+  }
+  hipLaunchKernelGGL(route_finish_kernel, dim3(fin), dim3(kRouteBlock), 0, s, counters, (uint32_t)n_experts, counts);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "route count launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, void* workspace, int64_t* counts,
+                      void* stream) {
+  if (!workspace) return fail(MCCL_ERR_INVALID_ARG, "workspace pointer is null");
+  return launch_route_counts(expert_ids, npairs, n_experts, (uint32_t*)workspace, /*clear_first=*/true, counts,
+                             (hipStream_t)stream);
 }
 
 int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const int32_t* src_rank,

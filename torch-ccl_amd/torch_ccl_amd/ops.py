@@ -242,6 +242,24 @@ def moe_combine(x, src_rank, src_row, weights, out=None):
     return out
 
 
+def route_counts(expert_ids, n_experts, workspace=None, out=None):
+    """counts[e] = number of entries of expert_ids (int32, on the GPU) equal to e, as an int64 tensor
+    on the GPU; ids outside [0, n_experts) are ignored.  The per-rank sums of it are the split
+    sizes of the dispatch all_to_all_single."""
+    if expert_ids.dtype != torch.int32 or not expert_ids.is_cuda or not expert_ids.is_contiguous():
+        raise RuntimeError("route_counts: expert_ids must be a contiguous int32 tensor on the GPU")
+    if workspace is None:
+        workspace = torch.empty(n_experts, dtype=torch.int32, device=expert_ids.device)
+    if workspace.dtype != torch.int32 or workspace.numel() < n_experts or not workspace.is_cuda:
+        raise RuntimeError("route_counts: workspace must hold n_experts int32 counters on the GPU")
+    if out is None:
+        out = torch.empty(n_experts, dtype=torch.int64, device=expert_ids.device)
+    with torch.cuda.device(out.device):
+        capi.check(capi.lib().mccl_route_counts(expert_ids.data_ptr(), expert_ids.numel(), n_experts,
+                                                workspace.data_ptr(), out.data_ptr(), _stream()))
+    return out
+
+
 def empty_staggered(n, shape, dtype, device="cuda", stagger_bytes=4096):
     """n uninitialised tensors of one shape carved from a single allocation, buffer k starting
     stagger_bytes past the end of buffer k-1 (rounded up to 256 bytes): rank buffers allocated this
