@@ -308,6 +308,18 @@ int mccl_unpack(const void* src, void* const* dst, const size_t* bytes, int n, v
 int mccl_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, void* workspace, int64_t* counts,
                       void* stream);
 
+/*
+ * mccl_route_counts without a workspace argument and without any allocation.  No counterpart in
+ * the reference: it is for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it.  The counters live in an array the
+ * library holds on every GPU it runs on (MCCL_ROUTE_MAX_EXPERTS x 4 bytes = 16 KiB per GPU, until
+ * the process ends); more experts than that are refused with MCCL_ERR_INVALID_ARG.  All calls on
+ * one GPU share that array: calls that overlap on one GPU (different streams, different threads)
+ * race and must be serialised by the caller.  Same results as mccl_route_counts.
+ */
+int mccl_route_counts_noalloc(const int32_t* expert_ids, size_t npairs, int n_experts, int64_t* counts,
+                              void* stream);
+
 int mccl_gather_rows(const void* src, size_t src_rows, const int64_t* row_index, size_t nrows,
                      size_t row_bytes, void* dst, void* stream);
 int mccl_moe_dispatch_n(const void* const* hidden, const size_t* hidden_rows,

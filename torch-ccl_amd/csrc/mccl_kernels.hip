@@ -1078,6 +1078,51 @@ int mccl_route_counts(const int32_t* expert_ids, size_t npairs, int n_experts, v
                              (hipStream_t)stream);
 }
 
+}  // extern "C"
+
+// The counters of mccl_route_counts_noalloc: one array per GPU the library runs on, held until the
+// process ends.  The name is a host-side handle, not a device address: host code uses the pointer
+// hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) uint32_t scratch[MCCL_ROUTE_MAX_EXPERTS];
+
+namespace {
+
+uint32_t* g_scratch_ptr[64];
+hipError_t g_scratch_err[64];
+std::once_flag g_scratch_once[64];
+
+// Address of `scratch` on the current device (looked up once per device, with that device current).
+int scratch_of_current_device(uint32_t** ptr) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return fail(MCCL_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  std::call_once(g_scratch_once[dev], [dev]() {
+    void* p = nullptr;
+    g_scratch_err[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+  });
+  if (g_scratch_err[dev] != hipSuccess || !g_scratch_ptr[dev])
+    return fail(MCCL_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(g_scratch_err[dev]));
+  *ptr = g_scratch_ptr[dev];
+  return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_route_counts_noalloc(const int32_t* expert_ids, size_t npairs, int n_experts, int64_t* counts,
+                              void* stream) {
+  if (n_experts > MCCL_ROUTE_MAX_EXPERTS)
+    return fail(MCCL_ERR_INVALID_ARG, "%d experts exceed the %d counters the library holds; use mccl_route_counts with a workspace",
+                n_experts, MCCL_ROUTE_MAX_EXPERTS);
+  uint32_t* counters = nullptr;
+  int rc = scratch_of_current_device(&counters);
+  if (rc != MCCL_OK) return rc;
+  // the array keeps whatever the last call left (zero after a complete call): cleared first anyway
+  return launch_route_counts(expert_ids, npairs, n_experts, counters, /*clear_first=*/true, counts, (hipStream_t)stream);
+}
+
 int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const int32_t* src_rank,
                      const int64_t* src_row, const float* weights, size_t tokens, int topk,
                      size_t hidden_elems, int dtype, void* y, void* stream) {
