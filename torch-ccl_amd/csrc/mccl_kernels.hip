@@ -49,7 +49,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "mccl.h"
 
@@ -334,20 +336,42 @@ int launch_jobs(ReduceArgs& a, const JobSpec* specs, int njobs, int dtype, int o
   }
   // An output may be exactly the input range its own job reads from one rank (in place); any
   // other overlap with something this launch reads or writes would race between wavefronts.
-  for (int j = 0; j < nv; ++j) {
-    const uintptr_t o0 = (uintptr_t)a.job[j].out;
-    const uintptr_t o1 = o0 + (a.job[j].head + a.job[j].nvec * ve + a.job[j].tail) * es;
-    for (int i = 0; i < nv; ++i) {
-      const size_t ibytes = (a.job[i].head + a.job[i].nvec * ve + a.job[i].tail) * es;
-      if (i != j) {
-        const uintptr_t q0 = (uintptr_t)a.job[i].out;
-        if (o0 < q0 + ibytes && q0 < o1) return fail(MCCL_ERR_INVALID_ARG, "outputs %d and %d overlap", j, i);
-      }
+  // Checked with a sort and one sweep over the byte ranges (jobs x (ranks + 1) of them), not pair
+  // by pair: a coalesced launch of 64 buckets from 64 ranks has 4160 ranges.
+  {
+    struct Range {
+      uintptr_t lo, hi;
+      int job, rank;  // rank < 0: the job's output
+    };
+    static thread_local std::vector<Range> ranges;
+    ranges.clear();
+    for (int j = 0; j < nv; ++j) {
+      const size_t bytes = (a.job[j].head + a.job[j].nvec * ve + a.job[j].tail) * es;
+      const uintptr_t o0 = (uintptr_t)a.job[j].out;
+      ranges.push_back(Range{o0, o0 + bytes, j, -1});
       for (int k = 0; k < a.n; ++k) {
-        const uintptr_t p0 = (uintptr_t)(a.ptr[a.job_ptr0[i] + k] + a.job[i].in_off);
-        if (o0 < p0 + ibytes && p0 < o1 && !(i == j && p0 == o0))
-          return fail(MCCL_ERR_INVALID_ARG, "output %d partially overlaps input %d of reduction %d", j, k, i);
+        const uintptr_t p0 = (uintptr_t)(a.ptr[a.job_ptr0[j] + k] + a.job[j].in_off);
+        if (p0 != o0) ranges.push_back(Range{p0, p0 + bytes, j, k});  // p0 == o0: in place, allowed
       }
+    }
+    std::sort(ranges.begin(), ranges.end(), [](const Range& x, const Range& y) { return x.lo < y.lo; });
+    const Range* far_any = nullptr;  // the earlier range that reaches farthest
+    const Range* far_out = nullptr;  // the earlier output that reaches farthest
+    for (const Range& r : ranges) {
+      const Range* hit = nullptr;
+      if (r.rank < 0) {
+        if (far_any && far_any->hi > r.lo) hit = far_any;
+      } else if (far_out && far_out->hi > r.lo) {
+        hit = far_out;
+      }
+      if (hit) {
+        const Range& out_r = r.rank < 0 ? r : *hit;
+        const Range& other = r.rank < 0 ? *hit : r;
+        if (other.rank < 0) return fail(MCCL_ERR_INVALID_ARG, "outputs %d and %d overlap", out_r.job, other.job);
+        return fail(MCCL_ERR_INVALID_ARG, "output %d partially overlaps input %d of reduction %d", out_r.job, other.rank, other.job);
+      }
+      if (!far_any || r.hi > far_any->hi) far_any = &r;
+      if (r.rank < 0 && (!far_out || r.hi > far_out->hi)) far_out = &r;
     }
   }
   if (nv) {
