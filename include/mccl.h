@@ -335,6 +335,16 @@ int mccl_moe_combine(const void* const* x, const size_t* x_rows, int n, const in
 int mccl_query_launch(size_t count, int n, int dtype, int op, int variant, int* block_size,
                       int* lds_bytes);
 
+/*
+ * Advisory: 1 when n rank buffers of `bytes` bytes each sit at a spacing measured to cost 6-10 % of
+ * bandwidth on large reductions (equal spacings of 256 MiB or more that are whole multiples of
+ * 2 MiB, which is where a caching allocator puts equal tensors of 1 GiB and more: element i of
+ * every rank then lands in the same DRAM channel and bank), else 0.  Needs no device.  The remedy
+ * is the placement: a further 4 KiB per rank removes the effect.  The kernels run correctly either
+ * way; the traffic is the same (counted), only the DRAM conflicts differ.
+ */
+int mccl_placement_check(const void* const* in, int n, size_t bytes);
+
 /* Sets a knob of mccl_tune_t; value <= 0 restores the default. */
 int mccl_set_tuning(int knob, long long value);
 long long mccl_get_tuning(int knob);

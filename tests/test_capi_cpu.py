@@ -183,3 +183,29 @@ def test_isa_guard_flags_nothing():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     assert mod.main() == 0
+
+
+def test_placement_check_needs_no_device(mccl):
+    """The advisory placement test flags equal spacings of 256 MiB and more that are multiples of
+    2 MiB on large messages (what a caching allocator gives equal tensors of 1 GiB and more), and
+    nothing else: small messages, irregular spacings, the same spacing 4 KiB further apart."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    GiB, MiB = 1 << 30, 1 << 20
+    base = 0x7f0000000000
+
+    def check(spacings, nbytes):
+        ptrs, p = [], base
+        for d in [0] + list(spacings):
+            p += d
+            ptrs.append(p)
+        return L.mccl_placement_check(capi.ptr_table(ptrs), len(ptrs), nbytes)
+
+    assert check([GiB + 2 * MiB] * 7, GiB) == 1
+    assert check([256 * MiB] * 7, 256 * MiB) == 1
+    assert check([-(GiB + 2 * MiB)] * 7, GiB) == 1            # descending addresses too
+    assert check([GiB + 2 * MiB + 4096] * 7, GiB) == 0         # staggered
+    assert check([GiB + 2 * MiB] * 6 + [GiB + 4 * MiB], GiB) == 0  # not regular
+    assert check([66 * MiB] * 7, 64 * MiB) == 0                # small messages have not shown the effect
+    assert check([GiB + 2 * MiB] * 7, 64 * MiB) == 0
+    assert L.mccl_placement_check(None, 8, GiB) == 0

@@ -553,6 +553,22 @@ int mccl_query_launch(size_t count, int n, int dtype, int op, int variant, int* 
   return (int)g.grid_x;
 }
 
+int mccl_placement_check(const void* const* in, int n, size_t bytes) {
+  if (!in || n < 2 || n > MCCL_MAX_RANKS) return 0;
+  if (bytes < (256u << 20)) return 0;  // smaller messages have not shown the effect
+  // Measured on MI355X (8 inputs, bare streaming kernel and the library's): equal spacings of
+  // 256 MiB and more that are whole multiples of 2 MiB -- 256 MiB, 512 MiB, 1 GiB, and the
+  // "size + 2 MiB" a caching allocator gives equal tensors of 1 GiB and more -- run at 76-81 % of
+  // the HBM peak where the same buffers a further 4 KiB apart per rank run at 85-87 %.  Irregular
+  // placements have not collided.
+  const intptr_t d = (intptr_t)((const char*)in[1] - (const char*)in[0]);
+  const uintptr_t ad = (uintptr_t)(d < 0 ? -d : d);
+  if (ad < (256u << 20) || ad % (2u << 20)) return 0;
+  for (int k = 2; k < n; ++k)
+    if ((intptr_t)((const char*)in[k] - (const char*)in[k - 1]) != d) return 0;
+  return 1;
+}
+
 int mccl_reduce_n(const void* const* in, int n, void* out, size_t count, int dtype, int op,
                   int variant, void* stream) {
   int rc = check_reduce_args(in, n, dtype, op);

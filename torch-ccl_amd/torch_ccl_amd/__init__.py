@@ -14,7 +14,7 @@ from . import capi
 from .capi import (AVG, MAX, MIN, PROD, SUM, VARIANT_AUTO, VARIANT_PERSISTENT,  # noqa: F401
                    VARIANT_SMALL, VARIANT_STREAM)
 from .ops import (allgather_n, alltoallv_n, copy_segments, empty_staggered, gather_rows, moe_combine,  # noqa: F401
-                  moe_dispatch_n, pack, reduce_multi, reduce_n, reduce_scatter_n, route_counts, staggered_copies,
+                  moe_dispatch_n, pack, placement_check, reduce_multi, reduce_n, reduce_scatter_n, route_counts, staggered_copies,
                   unpack)
 
 capi.lib()  # fail loudly at import time when the native library is absent

@@ -37,7 +37,7 @@ EXPORTS = (
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
     "mccl_rank_barrier", "mccl_allreduce_fused",
     "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync", "mccl_allreduce_sync_shard",
-    "mccl_route_counts", "mccl_route_counts_noalloc",
+    "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
 
 
@@ -88,6 +88,7 @@ def lib():
     L.mccl_allreduce_sync.argtypes = [vp, vp, vp, sz, i32, i32, ctypes.c_uint32, vp, vp]
     L.mccl_allreduce_sync_shard.argtypes = [sz, i32]
     L.mccl_allreduce_sync_shard.restype = sz
+    L.mccl_placement_check.argtypes = [vp, i32, sz]
     L.mccl_route_counts.argtypes = [vp, sz, i32, vp, vp, vp]
     L.mccl_route_counts_noalloc.argtypes = [vp, sz, i32, vp, vp]
     L.mccl_query_launch.argtypes = [sz, i32, i32, i32, i32, vp, vp]
