@@ -478,6 +478,17 @@ def main():
                                           "pct_of_peak": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS * 100, 1)}
         log("C3 in place:", json.dumps(result["c3_in_place_on_rank0"]))
         del fresh
+        # every op and every rank count up to 8 on 64 MiB messages: % of the HBM peak (AUTO shape)
+        matrix = {}
+        for opname, opcode in (("SUM", capi.SUM), ("AVG", capi.AVG), ("PROD", capi.PROD), ("MIN", capi.MIN), ("MAX", capi.MAX)):
+            row = {}
+            for nr in range(2, N + 1):
+                us = min(benchlib.reduce_throughput([ins[:nr]], [out], op=opcode, warmup=3, iters=20) for _ in range(2))
+                row[str(nr)] = round((nr + 1) * S / us / 1e3 / PEAK_HBM_GBS * 100, 1)
+            matrix[opname] = row
+        result["pct_of_peak_by_op_and_ranks_64MiB"] = matrix
+        log("ops x ranks:", json.dumps(matrix))
+        mccl.reduce_n(ins, out=out, op=mccl.SUM)  # the headline output again, for the checks below
 
     # ---------------- coalesced and list forms: one fused launch against one launch per tensor ----------------
     if "lists" in extras:

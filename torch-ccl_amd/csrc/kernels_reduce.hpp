@@ -90,7 +90,7 @@ __device__ __forceinline__ void store_vec_stream(u32x4* p, u32x4 x) {
 // One tile of BLOCK*U vectors: every lane loads its U vectors from all n inputs, runs the
 // ascending-rank chain in registers and streams the result out.
 // NT > 0: rank count known at compile time, all NT*U loads in flight before the first add.
-// NT == 0: runtime rank count, groups of 4 ranks.
+// NT == 0: runtime rank count, groups of 8 ranks.
 template <int DT, int OP, int NT, int U, int BLOCK, bool GUARD, typename ARGS>
 __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byte_off,
                                             u32x4* ov, size_t v0, size_t nvec, int n, bool stream_out) {
@@ -118,7 +118,9 @@ __device__ __forceinline__ void reduce_tile(const ARGS& a, int p0, size_t in_byt
           acc[u][e] = chain_next<DT, OP>(acc[u][e], Elem<DT>::load(vec_get<DT>(x[k][u], e)));
     }
   } else {
-    constexpr int G = 4;
+    // runtime rank count: groups of up to eight ranks, so that up to eight ranks have all their
+    // loads in flight before the first add, like the compile-time rank counts
+    constexpr int G = 8;
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll

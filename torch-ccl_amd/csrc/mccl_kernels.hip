@@ -219,26 +219,33 @@ uint64_t wait_limit_ticks(uint64_t timeout_us) {
   return timeout_us * kTicksPerUs;
 }
 
-// Loads one wavefront keeps in flight per tile: all ranks when the rank count is a
-// compile-time specialisation (SUM and AVG with 2, 4 or 8 ranks), else one group of four.
-int loads_in_flight(int n, int op, bool own_ptrs) {
-  if (!own_ptrs && (op == MCCL_SUM || op == MCCL_AVG) && (n == 2 || n == 4 || n == 8)) return n;
-  return n < 4 ? n : 4;
-}
+// Loads one wavefront keeps in flight per tile: all ranks up to eight (compile-time rank counts
+// and the generic path alike, which loads in groups of eight).
+int loads_in_flight(int n, int /*op*/, bool /*own_ptrs*/) { return n < 8 ? n : 8; }
 
 // Resident wavefronts per CU of the stream shape.  Enough loads in flight to cover the memory
 // latency at full bandwidth (about 14 MB over the chip), and no more: every further wavefront
 // widens the window of live tiles and costs DRAM page locality.  Measured optima on MI355X
-// (bf16, 64 MiB per rank, one buffer set and rotating through several GiB): 7-8 wavefronts when
-// a wavefront keeps 8 loads in flight (6 falls off a cliff: 75 % of peak against 87 %), 12 with 4
-// (also the generic path, which loads in groups of four), 14 with 3, no cap with 2 or 1.
+// (bf16, 64 MiB per rank; % of the HBM peak at the optimum / two wavefronts off it):
+//   loads in flight   SUM, AVG, PROD          MIN, MAX (compare + select per element: more ALU
+//                                             work per byte wants more wavefronts to hide it)
+//   8                 8   (87 / 84)           12  (83 / 78 at 9, 74 at 8)
+//   7                 10  (86 / 80 at 7)      12
+//   6                 11  (85 / 81 at 8)      14
+//   5                 12  (84 / 79 at 9)      14  (85 / 80 at 12)
+//   4                 14  (85 / 80 at 9)      14  (86 / 77 at 12)
+//   3 or fewer        no cap (85 against 81 at 14 wavefronts for three loads)
 long long stream_waves(int n, int op, bool own_ptrs) {
   if (g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU] > 0) return g_tune[MCCL_TUNE_STREAM_WAVES_PER_CU];
-  switch (loads_in_flight(n, op, own_ptrs)) {
+  const int loads = loads_in_flight(n, op, own_ptrs);
+  if (loads <= 3) return kMaxWavesPerCu;
+  if (op == MCCL_MIN || op == MCCL_MAX) return loads >= 7 ? 12 : 14;
+  switch (loads) {
     case 8: return 8;
-    case 4: return 12;
-    case 3: return 14;
-    default: return kMaxWavesPerCu;
+    case 7: return 10;
+    case 6: return 11;
+    case 5: return 12;
+    default: return 14;
   }
 }
 
