@@ -92,7 +92,15 @@ typedef enum {
                                              stay below what the GPU keeps resident at once
                                              (256 CUs x 32), or ranks could wait for launches
                                              that find no room */
-  MCCL_TUNE_COUNT_ = 8
+  MCCL_TUNE_COPY_VECTORS_PER_LANE = 8,    /* segmented copy: 2 or 4 vectors of 16 bytes per lane per chunk
+                                             (2 KiB or 4 KiB per wavefront); any other value = chosen by
+                                             the total size of the call */
+  MCCL_TUNE_COPY_STREAM_STORES = 9,       /* segmented copy, full chunks: 1 = stores written through past
+                                             the caches, 2 = non-temporal stores; else chosen by size */
+  MCCL_TUNE_COPY_LARGE_MIN_BYTES = 10,    /* total bytes of a copy call from which the large-copy
+                                             geometry applies */
+  MCCL_TUNE_GATHER_WAVES_PER_CU = 11,     /* residency cap of the row gather / fused MoE dispatch */
+  MCCL_TUNE_COUNT_ = 12
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64

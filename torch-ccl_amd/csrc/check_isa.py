@@ -140,8 +140,9 @@ def scan_hints(asm_path):
             if get("store", "plain"):
                 bad.append((fn, "row gather has vector stores without nt: %r" % c))
         elif "copy_segments_kernel" in fn:
-            if get("load", "nt") < 2 or get("store", "nt") < 2:
-                bad.append((fn, "copy kernel lost its nt hints: %r" % c))
+            # full chunks: nt loads; nt stores, or written-through (sc1) ones in the STREAM variants
+            if get("load", "nt") < 2 or max(get("store", "nt"), get("store", "sc1")) < 2:
+                bad.append((fn, "copy kernel lost its cache hints: %r" % c))
     if not seen_reduce:
         bad.append(("reduce_vec_kernel", "no reduction kernel recognised (name mangling changed?)"))
     return bad

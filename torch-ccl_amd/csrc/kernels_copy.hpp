@@ -41,8 +41,12 @@ struct SyncCopyArgs {
 // COHERENT: the sources are buffers of other ranks, complete in memory but possibly stale in this
 // kernel's caches: 8-byte aligned sources are read past the caches (the host requests a cache
 // invalidate per workgroup for the others).
-template <bool COHERENT>
+// UNROLL: 16-byte vectors per lane per chunk (chunk = 64 x 16 x UNROLL bytes; the host computes
+// the segment geometry for the same value).  STREAM: full chunks are written through past the
+// caches (`sc1`) instead of with the non-temporal hint.
+template <bool COHERENT, int UNROLL, bool STREAM>
 __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
+  constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
     // binary search: largest s with chunk_prefix[s] <= chunk
@@ -54,27 +58,30 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
     const uint32_t c = chunk - a.chunk_prefix[lo];
     const uint32_t head = a.seg[lo].head;
     const uint32_t nfull = a.seg[lo].nfull;
-    const uint32_t len = (c < nfull) ? (uint32_t)kCopyChunk : a.seg[lo].last;
+    const uint32_t len = (c < nfull) ? CHUNK : a.seg[lo].last;
     const uint32_t t = threadIdx.x;
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
     if (c == 0)
       for (uint32_t i = t; i < head; i += kWave) dst[i] = src[i];  // head < 128
-    const size_t off = (size_t)head + (size_t)c * kCopyChunk;  // start of this chunk
+    const size_t off = (size_t)head + (size_t)c * CHUNK;  // start of this chunk
     src += off;
     dst += off;
 
     const u32x4_unaligned* sv = (const u32x4_unaligned*)src;
     u32x4* dv = (u32x4*)dst;
-    if (len == (uint32_t)kCopyChunk) {
-      u32x4 x[kCopyUnroll];
+    if (len == CHUNK) {
+      u32x4 x[UNROLL];
 #pragma unroll
-      for (int u = 0; u < kCopyUnroll; ++u) {
+      for (int u = 0; u < UNROLL; ++u) {
         if (COHERENT && (((uintptr_t)src) & 7u) == 0) x[u] = load_vec_coherent(&((const u32x4*)src)[t + u * kWave]);
         else x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
       }
 #pragma unroll
-      for (int u = 0; u < kCopyUnroll; ++u) __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      for (int u = 0; u < UNROLL; ++u) {
+        if constexpr (STREAM) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&dv[t + u * kWave]), "v"(x[u]) : "memory");
+        else __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
+      }
     } else {
       const uint32_t nv = len >> 4;
       for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
@@ -84,13 +91,14 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
   }
 }
 
-__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) { copy_segments_body<false>(a); }
+template <int UNROLL, bool STREAM>
+__global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) { copy_segments_body<false, UNROLL, STREAM>(a); }
 
 __global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCopyArgs a) {
   if (xsync_begin(a.sync)) {
     // heads, partial chunks and misaligned sources go through the caches
     if (a.invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    copy_segments_body<true>(a.copy);
+    copy_segments_body<true, kCopyUnroll, false>(a.copy);
   }
   xsync_end(a.sync, gridDim.x);
 }

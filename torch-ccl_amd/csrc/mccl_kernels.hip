@@ -101,12 +101,18 @@ constexpr long long kTuneDefault[MCCL_TUNE_COUNT_] = {
     /* PERSISTENT_BLOCKS_PER_CU */ 8,
     /* STREAM_WAVES_PER_CU      */ 0,
     /* SMALL_MAX_BYTES          */ 4 << 20,
-    /* COPY_WAVES_PER_CU        */ 28,
+    /* COPY_WAVES_PER_CU        */ 24,
     /* STREAM_MIN_TOTAL_BYTES   */ 112ll << 20,
     /* COMBINE_PIECES_PER_WAVE  */ 2,
     /* COMBINE_WAVES_PER_CU     */ 0,
     /* XRANK_WAVES_ALL_RANKS    */ 4096,
+    /* COPY_VECTORS_PER_LANE    */ 1,  // neither 2 nor 4: chosen by size
+    /* COPY_STREAM_STORES       */ 3,  // neither 1 nor 2: chosen by size
+    /* COPY_LARGE_MIN_BYTES     */ 1ll << 30,
+    /* GATHER_WAVES_PER_CU      */ 28,
 };
+constexpr int kCopyUnrollLarge = 2;   // vectors per lane per chunk of large copies
+constexpr int kCopyStreamLarge = 1;   // store flavour of large copies: 1 = written through (sc1), 2 = non-temporal
 struct TuneTable {
   std::atomic<long long> v[MCCL_TUNE_COUNT_];
   TuneTable() {
@@ -410,11 +416,27 @@ int check_reduce_args_no_ptr(int n, int dtype, int op) {
 }
 
 int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
-  for (int k = 0; k < nseg; ++k)  // refusals first, before anything is enqueued
+  size_t total_bytes = 0;
+  for (int k = 0; k < nseg; ++k) {  // refusals first, before anything is enqueued
     if (segs[k].bytes && (!segs[k].src || !segs[k].dst)) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", k);
+    total_bytes += segs[k].bytes;
+  }
   int cus = 0;
   int rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
+  // Geometry of the call: vectors per lane per chunk and the flavour of the full-chunk stores.
+  // Tunable for sweeps; the defaults follow the total size.  Measured on MI355X (C5: 64 segments,
+  // 3.5 GiB moved; a 512 MiB single-segment copy), % of the HBM peak of 2 x bytes moved:
+  //   2 vectors per lane, nt stores:  C5 81.6 at 24 wavefronts per CU (80.8 at 28, 77.7 at 20), copy 83.5
+  //   2 vectors per lane, sc1 stores: C5 83.7 at 24 (82.8 at 20, 78.6 at 28),                  copy 82.9
+  //   4 vectors per lane (4 KiB per wavefront): 81.5 / 81.6 at 16 wavefronts, lower everywhere else
+  // so chunks stay at 2 KiB, 24 wavefronts are resident per CU, and calls that move 1 GiB or more
+  // write their full chunks through past the caches.
+  long long unroll = g_tune[MCCL_TUNE_COPY_VECTORS_PER_LANE];
+  if (unroll != 2 && unroll != 4) unroll = total_bytes >= (size_t)g_tune[MCCL_TUNE_COPY_LARGE_MIN_BYTES] ? kCopyUnrollLarge : kCopyUnroll;
+  long long stream_store = g_tune[MCCL_TUNE_COPY_STREAM_STORES];
+  if (stream_store != 1 && stream_store != 2) stream_store = total_bytes >= (size_t)g_tune[MCCL_TUNE_COPY_LARGE_MIN_BYTES] ? kCopyStreamLarge : 2;
+  const size_t chunk_bytes = (size_t)kWave * 16 * (size_t)unroll;
   int i = 0;
   while (i < nseg) {
     CopyArgs a;
@@ -432,9 +454,9 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
       size_t head = (128u - (unsigned)(dp & 127u)) & 127u;  // the body starts on a cache line of dst
       if (head > sg.bytes) head = sg.bytes;
       const size_t body = sg.bytes - head;
-      const uint64_t nfull = body / kCopyChunk;
+      const uint64_t nfull = body / chunk_bytes;
       cs.head = (uint32_t)head;
-      cs.last = (uint32_t)(body % kCopyChunk);
+      cs.last = (uint32_t)(body % chunk_bytes);
       uint64_t c = nfull + (cs.last ? 1 : 0);
       if (c == 0) c = 1;  // head only: chunk 0 still has to run
       if (nfull > 0xf0000000ull || chunks + c > kMaxChunks) {
@@ -453,7 +475,14 @@ int launch_copy(const mccl_segment_t* segs, int nseg, hipStream_t s) {
     if (grid > kMaxGridX) grid = kMaxGridX;
     // small copies are latency bound: no residency cap below 4 chunks per CU
     const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_COPY_WAVES_PER_CU]) : 0;
-    hipLaunchKernelGGL(copy_segments_kernel, dim3((unsigned)grid), dim3(kWave), lds, s, a);
+    const dim3 g3((unsigned)grid), b3(kWave);
+    if (unroll == 4) {
+      if (stream_store == 1) hipLaunchKernelGGL((copy_segments_kernel<4, true>), g3, b3, lds, s, a);
+      else hipLaunchKernelGGL((copy_segments_kernel<4, false>), g3, b3, lds, s, a);
+    } else {
+      if (stream_store == 1) hipLaunchKernelGGL((copy_segments_kernel<2, true>), g3, b3, lds, s, a);
+      else hipLaunchKernelGGL((copy_segments_kernel<2, false>), g3, b3, lds, s, a);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   }
@@ -516,7 +545,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
     if (rc != MCCL_OK) return rc;
     uint64_t grid = chunks;
     if (grid > kMaxGridX) grid = kMaxGridX;
-    const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_COPY_WAVES_PER_CU]) : 0;
+    const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_GATHER_WAVES_PER_CU]) : 0;
     hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)grid), dim3(kWave), lds, s, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MCCL_ERR_HIP, "gather kernel launch failed: %s", hipGetErrorString(e));

@@ -20,7 +20,8 @@ SUM, AVG, PROD, MIN, MAX = 0, 1, 2, 3, 4
 VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
 (TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_WAVES_PER_CU, TUNE_SMALL_MAX_BYTES,
  TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
- TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS) = range(8)
+ TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS, TUNE_COPY_VECTORS_PER_LANE, TUNE_COPY_STREAM_STORES,
+ TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU) = range(12)
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
