@@ -134,9 +134,6 @@ struct XSync {
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
 __device__ __forceinline__ bool xsync_begin(const XSync& x) {
   const int lane = threadIdx.x & (kWave - 1);
-#ifdef MCCL_XRANK_TRACE
-  if (blockIdx.x == 0 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[1] = wall_clock64();
-#endif
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
     __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   bool ok = true;
@@ -145,10 +142,6 @@ __device__ __forceinline__ bool xsync_begin(const XSync& x) {
     if (!ok) report_late(x.status, lane, (uint32_t)x.ready_epoch);
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // nothing below moves above the wait
-#ifdef MCCL_XRANK_TRACE
-  if (blockIdx.x == 0 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[2] = wall_clock64();
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0 && x.status) ((uint64_t*)x.status)[3] = wall_clock64();
-#endif
   return __builtin_amdgcn_ballot_w64(!ok) == 0;
 }
 
@@ -168,9 +161,6 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
     const uint32_t before = __hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last = before + 1 == workgroups ? 1u : 0u;
     if (last) {
-#ifdef MCCL_XRANK_TRACE
-      if (x.status) ((uint64_t*)x.status)[4] = wall_clock64();
-#endif
       __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
       __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -180,9 +170,6 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
   if (lane < x.n && lane != x.rank) {
     if (!wait_flag64(x.word[lane], x.done_epoch, x.limit_ticks)) report_late(x.status, lane, (uint32_t)x.done_epoch);
   }
-#ifdef MCCL_XRANK_TRACE
-  if (lane == 0 && x.status) ((uint64_t*)x.status)[5] = wall_clock64();
-#endif
 }
 
 template <typename ARGS>

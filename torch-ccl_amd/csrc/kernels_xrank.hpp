@@ -63,9 +63,6 @@ struct XRankArgs {
 // tensors out of an allocator), else as an ordinary unaligned load after a cache invalidate the
 // host asked for (aligned_in == 0 makes the kernel invalidate once per workgroup).
 __device__ __forceinline__ u32x4 load_in(const char* base, uint32_t v, uint32_t aligned) {
-#ifdef MCCL_XRANK_EXP_NT
-  aligned = 0;
-#endif
   if (aligned) return load_vec_coherent(&((const u32x4*)base)[v]);
   return __builtin_nontemporal_load(&((const u32x4_unaligned*)base)[v]);
 }
