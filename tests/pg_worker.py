@@ -609,6 +609,46 @@ def zero_copy_cases(pg, rank, world):
     pg.alltoall_base(out, host[rank].to(DEV), S[:, rank].tolist(), S[rank].tolist()).wait()
     want = O.alltoallv([to_carrier(h) for h in host], S, hidden * 2)[rank]
     assert np.array_equal(out.cpu().view(torch.uint8).numpy().reshape(-1), want), "alltoallv"
+    # List forms.  A list that is consecutive views of one tensor is read in place; any other list
+    # is packed.  flat_on(r) decides per rank which it is, so that "every rank flat", "no rank
+    # flat" and "some ranks flat" (every rank must then stage) all run.
+    def as_list(host_pieces, flat):
+        if flat:
+            whole = torch.cat([h.reshape(-1) for h in host_pieces]).to(DEV) if host_pieces else None
+            out, at = [], 0
+            for h in host_pieces:
+                out.append(whole[at:at + h.numel()].view(h.shape))
+                at += h.numel()
+            return out
+        return [h.to(DEV) for h in host_pieces]
+
+    for name, flat_on in (("all flat", lambda r: True), ("none flat", lambda r: False), ("mixed", lambda r: r % 2 == 0)):
+        for scale in (1, 64):  # a few KiB per piece, and pieces large enough to be shared
+            # alltoall(list) with uneven pieces (one of them empty)
+            S = np.random.default_rng(777 + scale).integers(1, 40, size=(world, world)) * 129 * scale
+            S[0, world - 1] = 0
+            host = [[rank_buffer(int(S[r, d]), torch.bfloat16, r * world + d, seed=7) for d in range(world)] for r in range(world)]
+            ins = as_list(host[rank], flat_on(rank))
+            outs = as_list([torch.zeros(int(S[r, rank]), dtype=torch.bfloat16) for r in range(world)], flat_on(rank + 1))
+            pg.alltoall(outs, ins).wait()
+            for r in range(world):
+                assert np.array_equal(bits(outs[r]), bits(host[r][rank])), ("alltoall list", name, scale, r)
+            assert all(np.array_equal(bits(ins[d]), bits(host[rank][d])) for d in range(world)), "alltoall list: inputs changed"
+            # reduce_scatter(list): slot d of every rank's list is reduced into rank d's output
+            m = 1031 * scale * 8
+            host = [[rank_buffer(m, torch.float32, r * world + d, seed=8) for d in range(world)] for r in range(world)]
+            ins = as_list(host[rank], flat_on(rank))
+            out = torch.zeros(m, dtype=torch.float32, device=DEV)
+            pg.reduce_scatter([out], [ins]).wait()
+            want = bits_np(O.reduce([to_carrier(host[r][rank]) for r in range(world)], O.F32, O.SUM))
+            assert np.array_equal(bits(out), want), ("reduce_scatter list", name, scale)
+            # allgather(list): every rank contributes a tensor of its own size
+            sizes = [(517 + 3 * r) * scale * 16 for r in range(world)]
+            host = [rank_buffer(sizes[r], torch.bfloat16, r, seed=9) for r in range(world)]
+            outs = as_list([torch.zeros(sizes[r], dtype=torch.bfloat16) for r in range(world)], flat_on(rank))
+            pg.allgather([outs], [host[rank].to(DEV)]).wait()
+            for r in range(world):
+                assert np.array_equal(bits(outs[r]), bits(host[r])), ("allgather list", name, scale, r)
     # rank 1's tensor lives in an allocation too large to be shared between processes: every rank
     # stages, results are the same
     count = (2 << 20) + 5

@@ -1139,6 +1139,27 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_
   return work;
 }
 
+// The list as one range of memory: its non-empty tensors are consecutive views of one storage
+// (computeLengthsAndCheckFlat of the reference, src/utils.cpp:157-193).  A list of empty tensors
+// is flat and empty.
+ProcessGroupCCL::FlatSpan ProcessGroupCCL::flatSpan(const std::vector<at::Tensor>& tensors) {
+  FlatSpan span;
+  span.flat = true;
+  const at::Tensor* first = nullptr;
+  for (const auto& t : tensors) {
+    const size_t b = nbytes(t);
+    if (!b) continue;
+    if (!first) {
+      first = &t;
+      span.ptr = t.data_ptr();
+    } else if (!first->storage().is_alias_of(t.storage()) || (const char*)t.data_ptr() != (const char*)span.ptr + span.bytes) {
+      return FlatSpan{};
+    }
+    span.bytes += b;
+  }
+  return span;
+}
+
 void ProcessGroupCCL::checkDeviceTensors(const std::vector<at::Tensor>& tensors) const {
   // checkSingleTensorHelper / checkSameType of the reference (src/utils.cpp:217-255) with the
   // device test turned around: this backend takes GPU tensors only.
@@ -1474,14 +1495,28 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
     p.copy_in = [=](void* stage, hipStream_t s) {
       copyAsync(stage, input.data_ptr(), mine, s);
     };
-  p.exec = [=](const PeerView& pv, hipStream_t s) {
+  // Large inputs are read in place by the peers.  `largest` is what the longest contribution of
+  // the group measures, which every rank knows from its output list: the offer is the same everywhere.
+  p.share = largest >= kZeroCopyMinBytes;
+  p.share_ptr = mine ? input.data_ptr() : nullptr;
+  p.share_bytes = mine;
+  auto pulls = [=](const PeerView& pv) {
     std::vector<mccl_segment_t> segs;
     for (int r = 0; r < W; ++r) {
       const size_t b = (size_t)pv.tables[(size_t)r][0];  // allgatherv: every rank announces its byte count
       TORCH_CHECK(b == nbytes(outs[(size_t)r]), "allgather: output tensor ", r, " does not match the size rank ", r, " sends");
-      if (b) segs.push_back({pv.stage[(size_t)r], outs[(size_t)r].data_ptr(), b});
+      if (b) segs.push_back({pv.zero_copy ? pv.user[(size_t)r] : pv.stage[(size_t)r], outs[(size_t)r].data_ptr(), b});
     }
+    return segs;
+  };
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
+    const auto segs = pulls(pv);
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+  };
+  p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+    const auto segs = pulls(pv);
+    MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), &sync, s));
+    return true;
   };
   return run(p);
 }
@@ -1627,15 +1662,19 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
   p.inputs = ins;
   p.outputs = {out};
   p.table.resize((size_t)(2 * W));
-  size_t total = 0;
+  const FlatSpan span = flatSpan(ins);
+  size_t total = 0, payload = 0, padded = 0;
   std::vector<size_t> offs((size_t)W);
   for (int d = 0; d < W; ++d) {
     offs[(size_t)d] = total;
     p.table[(size_t)d] = (int64_t)total;
     p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
-    total += roundUp(nbytes(ins[(size_t)d]), 16);
+    payload += nbytes(ins[(size_t)d]);
+    padded += roundUp(nbytes(ins[(size_t)d]), 16);
+    // a flat list is its own image; any other is packed with each slot on a 16-byte boundary
+    total += span.flat ? nbytes(ins[(size_t)d]) : roundUp(nbytes(ins[(size_t)d]), 16);
   }
-  if (total > stage_max_) {
+  if (padded > stage_max_) {  // (the padded size: the same on every rank, flat list or not)
     // more than one staging window: W (windowed) rooted reduces, as the reference does for slots of
     // unequal size.  The root reduces in place in its output, which first takes its own slot.
     c10::intrusive_ptr<c10d::Work> last;
@@ -1665,15 +1704,30 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
         segs.push_back({ins[(size_t)d].data_ptr(), (char*)stage + offs[(size_t)d], nbytes(ins[(size_t)d])});
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
-  p.exec = [=](const PeerView& pv, hipStream_t s) {
+  // A large list that is one range of memory (src/utils.cpp:157-193) is read in place by the
+  // peers.  The offer depends on the unpadded size of the list, which is the same on every rank
+  // of a valid call; a rank whose list is not flat offers nothing, and then every rank stages.
+  p.share = payload >= kZeroCopyMinBytes;
+  p.share_ptr = span.flat ? span.ptr : nullptr;
+  p.share_bytes = span.flat ? span.bytes : payload;
+  auto sources = [=](const PeerView& pv) {
     std::vector<const void*> in((size_t)W);
     for (int k = 0; k < W; ++k) {
       TORCH_CHECK((size_t)pv.tables[(size_t)k][W + me] == nbytes(out),
                   "reduce_scatter: rank ", k, "'s input for rank ", me, " does not match the output size");
-      in[(size_t)k] = (const char*)pv.stage[(size_t)k] + pv.tables[(size_t)k][me];
+      in[(size_t)k] = (const char*)(pv.zero_copy ? pv.user[(size_t)k] : pv.stage[(size_t)k]) + pv.tables[(size_t)k][me];
     }
+    return in;
+  };
+  p.exec = [=](const PeerView& pv, hipStream_t s) {
+    const auto in = sources(pv);
     if (out.numel())
       MCCL_CHECK(mccl_reduce_n(in.data(), W, out.data_ptr(), (size_t)out.numel(), dtype, op, MCCL_VARIANT_AUTO, s));
+  };
+  p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
+    const auto in = sources(pv);
+    MCCL_CHECK(mccl_reduce_sync(in.data(), out.data_ptr(), (size_t)out.numel(), dtype, op, &sync, s));
+    return true;
   };
   return run(p);
 }
@@ -1763,62 +1817,105 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall_base(at::Tensor& output
       recv[(size_t)i] = (out_equal ? out_len : (size_t)outputSplitSizes[(size_t)i] * out_len) * es;
     }
   }
-  const size_t mine = nbytes(input);
-  std::vector<size_t> send_displ((size_t)W), recv_off((size_t)W);
+  std::vector<size_t> send_displ((size_t)W);
+  std::vector<void*> dst((size_t)W);
   size_t displ = 0, roff = 0;
   for (int d = 0; d < W; ++d) {  // displacements = exclusive prefix sums of the counts
     send_displ[(size_t)d] = displ;
-    recv_off[(size_t)d] = roff;
+    dst[(size_t)d] = (char*)output.data_ptr() + roff;
     displ += send[(size_t)d];
     roff += recv[(size_t)d];
   }
-  // Inputs larger than one staging window travel in windows: window w holds bytes
-  // [w * window, (w + 1) * window) of every rank's input, and a rank pulls the part of each
-  // of its segments that lies inside.  How many windows there are depends on the largest input
-  // of the group, which every rank learns from the tables of the first window.
+  ExchangeImage image;
+  image.flat = nbytes(input) ? input.data_ptr() : nullptr;
+  image.offs = std::move(send_displ);
+  image.sizes = std::move(send);
+  image.total = nbytes(input);
+  return exchange(c10d::OpType::ALLTOALL_BASE, "alltoall_base", {input}, {output}, image, dst, recv);
+}
+
+// The all-to-all engine behind alltoall_base and alltoall.  Every rank has an image -- W pieces,
+// piece d for rank d, at image.offs[d] -- that is either a range of the caller's memory
+// (image.flat: the peers read it in place when every rank can share) or packed into the staging
+// buffer from image.pieces by the copy-in (the pack of src/gpu/dpcpp_ccl.cpp:1505-1515).  A rank pulls
+// piece `me` of every image straight to dst[r] (which is the unpack, :1528-1538).
+//
+// Images larger than one staging window travel in windows: window w holds bytes
+// [w * window, (w + 1) * window) of every rank's image, and a rank pulls the part of each of its
+// pieces that lies inside.  How many windows there are depends on the largest image of the
+// group, which every rank learns from the tables of the first window.
+//
+// The images differ in size and kind from rank to rank, so the zero-copy offer cannot depend on
+// either: every exchange offers (a packed image offers nothing, and then every rank stages).
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::exchange(c10d::OpType op, const char* title,
+                                                          const std::vector<at::Tensor>& inputs,
+                                                          const std::vector<at::Tensor>& outputs,
+                                                          const ExchangeImage& image, const std::vector<void*>& dst,
+                                                          const std::vector<size_t>& recv) {
+  const int W = size_;
+  const int me = rank_;
+  const bool is_base = op == c10d::OpType::ALLTOALL_BASE;
+  const size_t total = image.total;
   auto nwin = std::make_shared<size_t>(1);
   const size_t window = stage_max_;
   c10::intrusive_ptr<c10d::Work> work;
   for (size_t w = 0; w < *nwin; ++w) {
-    const size_t w0 = w * window;
-    const size_t wlen = w0 < mine ? std::min(mine - w0, window) : 0;
+    const size_t w0 = w * window, w1 = w0 + window;
+    const size_t wlen = w0 < total ? std::min(total - w0, window) : 0;
     Plan p;
-    p.op = c10d::OpType::ALLTOALL_BASE;
-    p.title = "alltoall_base";
-    p.inputs = {input};
-    p.outputs = {output};
+    p.op = op;
+    p.title = title;
+    p.inputs = inputs;
+    p.outputs = outputs;
     p.stage_bytes = wlen;
     p.table.resize((size_t)(2 * W + 1));
     for (int d = 0; d < W; ++d) {
-      p.table[(size_t)d] = (int64_t)send_displ[(size_t)d];
-      p.table[(size_t)(W + d)] = (int64_t)send[(size_t)d];
+      p.table[(size_t)d] = (int64_t)image.offs[(size_t)d];
+      p.table[(size_t)(W + d)] = (int64_t)image.sizes[(size_t)d];
     }
-    p.table[(size_t)(2 * W)] = (int64_t)mine;
-    // The inputs differ in size from rank to rank, so the offer cannot depend on a size: every
-    // all-to-all offers its input, and the peers pull their segments out of it in place.
+    p.table[(size_t)(2 * W)] = (int64_t)total;
     p.share = true;
-    p.share_ptr = mine ? input.data_ptr() : nullptr;
-    p.share_bytes = mine;
-    if (wlen)
-      p.copy_in = [=](void* stage, hipStream_t s) {
-        copyAsync(stage, (const char*)input.data_ptr() + w0, wlen, s);
-      };
+    p.share_ptr = image.flat;  // null with total > 0: a packed image, which cannot be shared
+    p.share_bytes = total;
+    if (wlen) {
+      if (image.flat) {
+        const char* flat = (const char*)image.flat;
+        p.copy_in = [=](void* stage, hipStream_t s) { copyAsync(stage, flat + w0, wlen, s); };
+      } else {
+        const std::vector<at::Tensor> pieces = image.pieces;
+        const std::vector<size_t> offs = image.offs;
+        p.copy_in = [=](void* stage, hipStream_t s) {
+          std::vector<mccl_segment_t> segs;
+          for (int d = 0; d < W; ++d) {  // the part of piece d that lies inside the window
+            const size_t lo = std::max(offs[(size_t)d], w0), hi = std::min(offs[(size_t)d] + nbytes(pieces[(size_t)d]), w1);
+            if (lo < hi)
+              segs.push_back({(const char*)pieces[(size_t)d].data_ptr() + (lo - offs[(size_t)d]), (char*)stage + (lo - w0), hi - lo});
+          }
+          if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
+        };
+      }
+    }
     // the segments this rank pulls in this window (and, from the tables, how many windows there are)
     auto pulls = [=](const PeerView& pv) {
       size_t largest = 0;
       std::vector<mccl_segment_t> segs;
       for (int r = 0; r < W; ++r) {
         const int64_t* tr = pv.tables[(size_t)r];
-        TORCH_CHECK((size_t)tr[W + me] == recv[(size_t)r],
-                    "alltoall_base: rank ", r, " sends ", tr[W + me], " bytes to rank ", me,
-                    " which expects ", recv[(size_t)r]);
+        if (is_base) {
+          TORCH_CHECK((size_t)tr[W + me] == recv[(size_t)r],
+                      "alltoall_base: rank ", r, " sends ", tr[W + me], " bytes to rank ", me,
+                      " which expects ", recv[(size_t)r]);
+        } else {
+          TORCH_CHECK((size_t)tr[W + me] == recv[(size_t)r], "alltoall: output tensor ", r,
+                      " does not match what rank ", r, " sends");
+        }
         largest = std::max(largest, (size_t)tr[2 * W]);
-        // the segment addressed to this rank inside rank r's input, cut to the window
+        // the piece addressed to this rank inside rank r's image, cut to the window
         const size_t seg0 = (size_t)tr[me], seg1 = seg0 + recv[(size_t)r];
-        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w0 + window);
+        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w1);
         if (lo < hi)
           segs.push_back({pv.zero_copy ? (const char*)pv.user[(size_t)r] + lo : (const char*)pv.stage[(size_t)r] + (lo - w0),
-                          (char*)output.data_ptr() + recv_off[(size_t)r] + (lo - seg0), hi - lo});
+                          (char*)dst[(size_t)r] + (lo - seg0), hi - lo});
       }
       *nwin = std::max<size_t>(1, (largest + window - 1) / window);
       return segs;
@@ -1847,63 +1944,29 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::alltoall(std::vector<at::Tensor>
   all.insert(all.end(), outputs.begin(), outputs.end());
   checkDeviceTensors(all);
   const int W = size_;
-  const int me = rank_;
-  std::vector<at::Tensor> ins = inputs, outs = outputs;
-  // The pack of the reference (src/gpu/dpcpp_ccl.cpp:1505-1515) is the copy-in itself, and the
-  // pull writes straight into the output tensors, which is its unpack (:1528-1538).  The packed
-  // image (the inputs back to back, each on a 16-byte boundary) travels in windows like the input
-  // of alltoall_base: window w holds image bytes [w * window, (w + 1) * window) of every rank.
-  std::vector<size_t> offs((size_t)W);
+  // A list whose tensors are consecutive views of one storage is an image already (the flat check
+  // of src/utils.cpp:157-215, used at src/gpu/dpcpp_ccl.cpp:1499-1504): no pack, and the peers can
+  // read it in place.  Any other list is packed by the copy-in, each piece on a 16-byte boundary.
+  ExchangeImage image;
+  image.sizes.resize((size_t)W);
+  image.offs.resize((size_t)W);
+  const FlatSpan span = flatSpan(inputs);
   size_t total = 0;
   for (int d = 0; d < W; ++d) {
-    offs[(size_t)d] = total;
-    total += roundUp(nbytes(ins[(size_t)d]), 16);
+    image.sizes[(size_t)d] = nbytes(inputs[(size_t)d]);
+    image.offs[(size_t)d] = total;
+    total += span.flat ? image.sizes[(size_t)d] : roundUp(image.sizes[(size_t)d], 16);
   }
-  auto nwin = std::make_shared<size_t>(1);
-  const size_t window = stage_max_;
-  c10::intrusive_ptr<c10d::Work> work;
-  for (size_t w = 0; w < *nwin; ++w) {
-    const size_t w0 = w * window, w1 = w0 + window;
-    Plan p;
-    p.op = c10d::OpType::ALLTOALL;
-    p.title = "alltoall";
-    p.inputs = ins;
-    p.outputs = outs;
-    p.table.resize((size_t)(2 * W + 1));
-    for (int d = 0; d < W; ++d) {
-      p.table[(size_t)d] = (int64_t)offs[(size_t)d];
-      p.table[(size_t)(W + d)] = (int64_t)nbytes(ins[(size_t)d]);
-    }
-    p.table[(size_t)(2 * W)] = (int64_t)total;
-    p.stage_bytes = w0 < total ? std::min(total - w0, window) : 0;
-    p.copy_in = [=](void* stage, hipStream_t s) {
-      std::vector<mccl_segment_t> segs;
-      for (int d = 0; d < W; ++d) {  // the part of input d that lies inside the window
-        const size_t lo = std::max(offs[(size_t)d], w0), hi = std::min(offs[(size_t)d] + nbytes(ins[(size_t)d]), w1);
-        if (lo < hi)
-          segs.push_back({(const char*)ins[(size_t)d].data_ptr() + (lo - offs[(size_t)d]), (char*)stage + (lo - w0), hi - lo});
-      }
-      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
-    };
-    p.exec = [=](const PeerView& pv, hipStream_t s) {
-      size_t largest = 0;
-      std::vector<mccl_segment_t> segs;
-      for (int r = 0; r < W; ++r) {
-        const int64_t* tr = pv.tables[(size_t)r];
-        const size_t b = (size_t)tr[W + me];
-        TORCH_CHECK(b == nbytes(outs[(size_t)r]), "alltoall: output tensor ", r, " does not match what rank ", r, " sends");
-        largest = std::max(largest, (size_t)tr[2 * W]);
-        const size_t seg0 = (size_t)tr[me], seg1 = seg0 + b;
-        const size_t lo = std::max(seg0, w0), hi = std::min(seg1, w1);
-        if (lo < hi)
-          segs.push_back({(const char*)pv.stage[(size_t)r] + (lo - w0), (char*)outs[(size_t)r].data_ptr() + (lo - seg0), hi - lo});
-      }
-      *nwin = std::max<size_t>(1, (largest + window - 1) / window);
-      if (!segs.empty()) MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
-    };
-    work = run(p);
+  image.total = total;
+  if (span.flat) image.flat = span.ptr;
+  else image.pieces = inputs;
+  std::vector<void*> dst((size_t)W);
+  std::vector<size_t> recv((size_t)W);
+  for (int r = 0; r < W; ++r) {
+    dst[(size_t)r] = outputs[(size_t)r].data_ptr();
+    recv[(size_t)r] = nbytes(outputs[(size_t)r]);
   }
-  return work;
+  return exchange(c10d::OpType::ALLTOALL, "alltoall", inputs, outputs, image, dst, recv);
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::barrier(const c10d::BarrierOptions& /*opts*/) {

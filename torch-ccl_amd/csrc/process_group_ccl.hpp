@@ -260,6 +260,24 @@ class ProcessGroupCCL : public c10d::Backend {
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
+  // A tensor list that is one range of memory (its non-empty tensors back to back in one storage)
+  struct FlatSpan {
+    const void* ptr = nullptr;
+    size_t bytes = 0;
+    bool flat = false;
+  };
+  static FlatSpan flatSpan(const std::vector<at::Tensor>& tensors);
+  // What a rank contributes to an all-to-all: W pieces at offs[d] of an image of `total` bytes that
+  // is either caller memory (flat) or packed from `pieces` into the staging buffer
+  struct ExchangeImage {
+    const void* flat = nullptr;
+    std::vector<at::Tensor> pieces;
+    std::vector<size_t> offs, sizes;
+    size_t total = 0;
+  };
+  c10::intrusive_ptr<c10d::Work> exchange(c10d::OpType op, const char* title, const std::vector<at::Tensor>& inputs,
+                                          const std::vector<at::Tensor>& outputs, const ExchangeImage& image,
+                                          const std::vector<void*>& dst, const std::vector<size_t>& recv);
   c10::intrusive_ptr<c10d::Work> run(Plan& plan);
   c10::intrusive_ptr<c10d::Work> finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work);
   void runHostSynced(Plan& plan, hipStream_t s, int slot);
