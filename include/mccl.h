@@ -194,7 +194,6 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
  */
 #define MCCL_FUSED_MAX_RANKS 8
 #define MCCL_FUSED_TILE_BYTES 1024
-#define MCCL_SYNC_FLAG_BYTES 4096 /* bytes of a shard per flag of mccl_allreduce_sync */
 int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
                          void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
                          uint64_t timeout_us, void* status, void* stream);
@@ -237,20 +236,21 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
                      const mccl_xsync_t* sync, void* stream);
 
 /*
- * In-place allreduce of tensors[rank] over all ranks' tensors in one launch: the two-shot
+ * In-place allreduce of tensors[rank] over all ranks' tensors in one launch, for ranks whose
+ * tensors are all writable by all ranks (as IPC-mapped device memory is).  Rank r reduces shard r
+ * (mccl_allreduce_sync_shard(count, n) elements, the last shards may be shorter or empty) of all
+ * tensors and writes the result into shard r of EVERY rank's tensor; nothing is staged and nothing
+ * is copied a second time: n reads and n writes per element of a shard, where the two-shot
  * algorithm of the reference's large path (reduce-scatter through scratch, all-gather:
- * src/gpu/allreduce.h:306-533).  Rank r reduces shard r (mccl_allreduce_sync_shard(count, n)
- * elements, the last shards may be shorter or empty) of all tensors into stage[r] and publishes
- * tile_flags[r][c] = tile_epoch per MCCL_SYNC_FLAG_BYTES of it; all ranks copy the finished shards
- * into their tensors chunk by chunk.  stage[r]: at least one shard, 16-byte aligned; tile_flags[r]:
- * one 32-bit word per MCCL_SYNC_FLAG_BYTES of a shard, zero before the first use; tile epochs grow from call to
- * call; a set may be reused once every peer has started a later collective.  done_epoch of the
- * descriptor is ignored (a rank's kernel ends only after it has seen every owner's every flag,
- * and only shard owners read a tensor).  Same bits as mccl_reduce_n over the n tensors.
+ * src/gpu/allreduce.h:306-533) moves n + 1 reads and 2 writes in two phases with a rank
+ * synchronisation between them (its gather step stores into its peers' buffers likewise,
+ * src/gpu/allreduce.h:470-487).  Only the owner of a shard touches it in any tensor while the
+ * collective runs; done_epoch is required: no rank's kernel ends before every rank has written its
+ * shard everywhere.  Same bits as mccl_reduce_n over the n tensors.
  */
 size_t mccl_allreduce_sync_shard(size_t count, int n);
-int mccl_allreduce_sync(void* const* tensors, void* const* stage, void* const* tile_flags, size_t count,
-                        int dtype, int op, uint32_t tile_epoch, const mccl_xsync_t* sync, void* stream);
+int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                        void* stream);
 
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */

@@ -149,7 +149,7 @@ def fused_case(rank, world, queues, barrier):
 
 def xrank_case(rank, world, queues, barrier):
     """The one-launch collectives that read the peers' buffers in place -- mccl_reduce_sync
-    (reduce_scatter shard), mccl_allreduce_sync (two-shot allreduce) and mccl_copy_segments_sync
+    (reduce_scatter shard), mccl_allreduce_sync (in-place allreduce) and mccl_copy_segments_sync
     (alltoallv pull) -- against the oracle, bit for bit, call after call on the same shared buffers
     with nothing but the kernels' own waits between them."""
     from helpers import TORCH_TO_CODE, assert_bits_equal, bits, oracle_reduce_bits, rank_buffer, to_carrier
@@ -160,10 +160,8 @@ def xrank_case(rank, world, queues, barrier):
     shared_in = torch.zeros(BUF, dtype=torch.uint8, device=DEV)      # what the peers read in place
     word = torch.zeros(8, dtype=torch.int64, device=DEV)             # [0]: the sync word
     counter = torch.zeros(8, dtype=torch.int32, device=DEV)
-    stage = [torch.zeros((4 << 20) + 64, dtype=torch.uint8, device=DEV) for _ in range(2)]
-    tflag = [torch.zeros(4096 + 8, dtype=torch.int32, device=DEV) for _ in range(2)]
     torch.cuda.synchronize()
-    shared = _exchange(rank, world, queues, barrier, [shared_in, word] + stage + tflag)
+    shared = _exchange(rank, world, queues, barrier, [shared_in, word])
     words = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])
     st = _status()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -193,24 +191,20 @@ def xrank_case(rank, world, queues, barrier):
         capi.check(L.mccl_reduce_sync(ins, out.data_ptr(), m, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
         want = oracle_reduce_bits([h[rank * m:(rank + 1) * m] for h in host], ops[name][1])
         checks.append((out, want, ("reduce_sync", str(dtype), m, name)))
-    # allreduce in place on the shared buffer
+    # allreduce in place on the shared buffer: every owner writes its finished shard into every
+    # rank's tensor; the clone behind it reads what the peers wrote
     for i, (dtype, count, name, off) in enumerate([(torch.bfloat16, (2 << 20) + 77, "SUM", 0), (torch.float32, 1025, "SUM", 4), (torch.int8, (3 << 20) + 5, "MAX", 3),
                                                   (torch.float64, 7, "SUM", 8), (torch.bfloat16, 3, "MIN", 2), (torch.float16, 1 << 21, "SUM", 0),
-                                                  (torch.int32, 100003, "PROD", 4), (torch.bfloat16, 4096 * 1024, "SUM", 0)]):
+                                                  (torch.int32, 100003, "PROD", 4), (torch.bfloat16, 4096 * 1024, "SUM", 0), (torch.uint8, 1, "SUM", 5),
+                                                  (torch.bfloat16, 4096 * 1024, "SUM", 6)]):
         es = torch.empty(0, dtype=dtype).element_size()
         off = off // es * es
-        host = [rank_buffer(count, dtype, r, seed=400 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
+        host = [rank_buffer(count, dtype, r, seed=450 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
         t = mine(dtype, count, off)
         t.copy_(host[rank])
-        shard = L.mccl_allreduce_sync_shard(count, world)
-        assert shard * es <= 4 << 20
-        slot = call[0] & 1
-        sy = sync(done=False)
-        capi.check(L.mccl_allreduce_sync(
-            capi.ptr_table([shared[r][0].data_ptr() + off for r in range(world)]),
-            capi.ptr_table([shared[r][2 + slot].data_ptr() for r in range(world)]),
-            capi.ptr_table([shared[r][4 + slot].data_ptr() for r in range(world)]),
-            count, TORCH_TO_CODE[dtype], ops[name][0], call[0], ctypes.byref(sy), stream))
+        sy = sync()
+        capi.check(L.mccl_allreduce_sync(capi.ptr_table([shared[r][0].data_ptr() + off for r in range(world)]),
+                                         count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
         want = oracle_reduce_bits(host, ops[name][1])
         checks.append((t.clone(), want, ("allreduce_sync", str(dtype), count, name)))
     # alltoallv pull: rank d copies its segment out of every rank's buffer

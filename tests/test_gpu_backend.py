@@ -119,6 +119,14 @@ def test_host_synchronised_fallback(monkeypatch, world, mode):
     _spawn(world, mode)
 
 
+def test_zero_copy_with_barrier_kernels_instead_of_one_launch(monkeypatch):
+    """MCCL_PG_ONE_LAUNCH_MAX_BYTES=0: the peers' tensors are still read in place, but between
+    barrier kernels by the bandwidth-tuned kernels (what groups of more than eight ranks and very
+    large tensors use): same bits."""
+    monkeypatch.setenv("MCCL_PG_ONE_LAUNCH_MAX_BYTES", "0")
+    _spawn(4, "zero_copy")
+
+
 def test_staged_when_zero_copy_is_switched_off(monkeypatch):
     monkeypatch.setenv("MCCL_PG_ZERO_COPY", "0")
     _spawn(4, "oracle")

@@ -66,6 +66,12 @@ __device__ __forceinline__ u32x4 load_vec_coherent(const u32x4* p) {
   return (u32x4){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
 }
 
+// 16 bytes written through to memory with one store, at any alignment the element type allows.
+// The wait state after it covers a following write of the data registers.
+__device__ __forceinline__ void store_vec_through(char* p, u32x4 x) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(p), "v"(x) : "memory");
+}
+
 // Everything this wavefront has stored has reached its destination (for written-through stores:
 // memory) -- what has to hold before a flag that announces the data is stored.
 __device__ __forceinline__ void wait_own_stores() {

@@ -560,7 +560,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 130; }
+int mccl_version(void) { return 140; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -894,56 +894,37 @@ size_t mccl_allreduce_sync_shard(size_t count, int n) {
   return (per + 63) / 64 * 64;
 }
 
-int mccl_allreduce_sync(void* const* tensors, void* const* stage, void* const* tile_flags, size_t count,
-                        int dtype, int op, uint32_t tile_epoch, const mccl_xsync_t* sync, void* stream) {
+int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync, void* stream) {
   XRankArgs a;
   memset(&a, 0, sizeof(a));
   int rc = fill_xsync(sync, &a.sync);
   if (rc != MCCL_OK) return rc;
   rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
   if (rc != MCCL_OK) return rc;
-  if (!tensors || !stage || !tile_flags) return fail(MCCL_ERR_INVALID_ARG, "tensor, staging or flag table is null");
+  if (!tensors) return fail(MCCL_ERR_INVALID_ARG, "tensor table is null");
+  if (a.sync.done_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "the pushing allreduce needs a closing wait (done_epoch)");
   const int n = a.sync.n, me = a.sync.rank;
   const size_t es = dtype_size(dtype);
-  const size_t shard = mccl_allreduce_sync_shard(count, n);
   for (int r = 0; r < n; ++r) {
-    if (!stage[r] || !tile_flags[r] || (count && !tensors[r])) return fail(MCCL_ERR_INVALID_ARG, "tensor, staging or flag pointer %d is null", r);
-    if ((uintptr_t)stage[r] % 16) return fail(MCCL_ERR_INVALID_ARG, "staging buffer %d is not 16-byte aligned", r);
-    if ((uintptr_t)tile_flags[r] % 4) return fail(MCCL_ERR_INVALID_ARG, "flag array %d is not 4-byte aligned", r);
+    if (count && !tensors[r]) return fail(MCCL_ERR_INVALID_ARG, "tensor pointer %d is null", r);
     if ((uintptr_t)tensors[r] % es) return fail(MCCL_ERR_INVALID_ARG, "tensor %d not aligned to the element size", r);
   }
-  auto shard_len = [&](int r) {
-    const size_t lo = (size_t)r * shard < count ? (size_t)r * shard : count;
-    const size_t hi = lo + shard < count ? lo + shard : count;
-    return hi - lo;
-  };
-  const size_t n_me = shard_len(me);
+  const size_t shard = mccl_allreduce_sync_shard(count, n);
+  const size_t lo = (size_t)me * shard < count ? (size_t)me * shard : count;
+  const size_t n_me = lo + shard < count ? shard : count - lo;
   const size_t ve = 16 / es;
   if ((uint64_t)shard * es / 16 + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
-  for (int k = 0; k < n; ++k) a.in[k] = (const char*)tensors[k] + (size_t)me * shard * es;
-  a.out1 = (char*)stage[me];
-  a.my_flags = (uint32_t*)tile_flags[me];
+  a.aligned_in = 1;
+  for (int k = 0; k < n; ++k) {
+    a.in[k] = (const char*)tensors[k] + lo * es;
+    if (n_me && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
+  }
+  a.push = 1;
   a.nvec1 = (uint32_t)(n_me / ve);
   a.tail1 = (uint32_t)(n_me % ve);
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
-  a.tile_epoch = tile_epoch;
-  a.aligned_in = 1;
-  for (int k = 0; k < n; ++k)
-    if (count && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
   if (a.tail1) a.aligned_in = 0;  // the last elements are read one by one, through the caches
-  uint32_t tiles2 = 0;
-  for (int q = 0; q < n; ++q) {
-    const uint64_t bytes = (uint64_t)shard_len(q) * es;
-    a.shard_src[q] = (const char*)stage[q];
-    a.shard_flags[q] = (const uint32_t*)tile_flags[q];
-    a.shard_dst[q] = (char*)tensors[me] + (size_t)q * shard * es;
-    a.full2[q] = (uint32_t)(bytes / kXTileBytes);
-    a.last2[q] = (uint32_t)(bytes % kXTileBytes);
-    const uint32_t tq = a.full2[q] + (a.last2[q] ? 1u : 0u);
-    if (tq > tiles2) tiles2 = tq;
-  }
-  a.tiles2 = tiles2;
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(tiles2, n), (hipStream_t)stream);
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n), (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }

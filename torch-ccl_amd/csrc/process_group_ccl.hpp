@@ -213,9 +213,6 @@ class ProcessGroupCCL : public c10d::Backend {
     std::vector<const int64_t*> tables;     // the scalars rank r published
     bool zero_copy = false;                 // the peers' tensors are read in place: nothing was staged
     std::vector<const void*> user;          // zero_copy: rank r's published tensor range
-    std::vector<void*> tile_flags;          // zero_copy: rank r's tile flags of the one-launch allreduce (this slot)
-    size_t tile_flag_count = 0;             // entries of each
-    uint32_t tile_epoch = 0;
   };
   using ExecFn = std::function<void(const PeerView& pv, hipStream_t s)>;
   // The whole device side of a zero-copy collective as ONE launch with the rank waits inside the
@@ -250,6 +247,7 @@ class ProcessGroupCCL : public c10d::Backend {
     const void* share_ptr = nullptr;
     size_t share_bytes = 0;
     size_t zero_copy_stage_bytes = 0;       // staging this rank still needs in zero-copy mode
+    bool one_launch_any_size = false;       // exec_sync wins at every size: the default one-launch limit does not apply
     // Eligible for the one-launch small allreduce (device-synchronised groups of at most 8 ranks):
     // no staging slot, no table, no rendezvous.  The staged plan above stays as the fallback.
     bool fused_ok = false;
@@ -329,6 +327,7 @@ class ProcessGroupCCL : public c10d::Backend {
   // persistent one-launch kernels move fewer bytes per second, which outweighs the saved launches
   // from a few hundred MiB of traffic on).  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides.
   size_t one_launch_max_ = 32u << 20;
+  bool one_launch_max_forced_ = false;
   bool comm_stream_for_large_ = false;  // MCCL_PG_COMM_STREAM=1: device-synchronised groups fork large collectives too
   // Decided at start-up, the same on every rank: all ranks are processes of their own (and the
   // environment does not ask for the host barrier), so cross-rank waits can live on the device.
@@ -383,7 +382,6 @@ class ProcessGroupCCL : public c10d::Backend {
   std::vector<void*> final_flags_;          // rank r's departure word
   std::vector<void*> fused_stage_[2];       // rank r's staging buffer of the one-launch allreduce, per slot
   std::vector<void*> fused_flags_[2];
-  std::vector<void*> xrank_flags_[2];       // rank r's tile flags of the one-launch large allreduce, per slot
   void* done_counter_ = nullptr;            // this rank's workgroup counter of the one-launch collectives
   void* status_dev_ = nullptr;              // device address of shared_->status
   std::shared_ptr<GroupShared> shared_;
