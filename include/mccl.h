@@ -100,7 +100,10 @@ typedef enum {
   MCCL_TUNE_COPY_LARGE_MIN_BYTES = 10,    /* total bytes of a copy call from which the large-copy
                                              geometry applies */
   MCCL_TUNE_GATHER_WAVES_PER_CU = 11,     /* residency cap of the row gather / fused MoE dispatch */
-  MCCL_TUNE_COUNT_ = 12
+  MCCL_TUNE_XRANK_CACHED_LOADS = 12,      /* one-launch reductions: 1 = the peers' tensors are read
+                                             through the caches after one invalidate per workgroup,
+                                             0 = past the caches, access by access */
+  MCCL_TUNE_COUNT_ = 13
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64
@@ -226,8 +229,12 @@ typedef struct {
 
 /* mccl_copy_segments whose sources are peers' buffers: allgather / alltoall(v) / broadcast pulls
  * (ccl::allgatherv, ccl::alltoallv, src/gpu/dpcpp_ccl.cpp:1176-1182, 1428-1455) in one launch.
- * At most 64 segments; zero segments still take part in the waits. */
-int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsync_t* sync, void* stream);
+ * At most 64 segments; zero segments still take part in the waits.  flags: MCCL_COPY_SHARED_SOURCES
+ * when the other ranks read the same source bytes in the same collective (allgather, broadcast):
+ * the sources are then kept in the memory-side cache instead of being streamed past it. */
+#define MCCL_COPY_SHARED_SOURCES 1u
+int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync,
+                            void* stream);
 
 /* mccl_reduce_n whose inputs are peers' buffers (in[r]: rank r's contribution at this rank's
  * slice): the shard reduction of reduce_scatter (ccl::reduce_scatter, src/gpu/dpcpp_ccl.cpp:1002-1008)

@@ -224,7 +224,7 @@ def xrank_case(rank, world, queues, barrier):
             roff += b
         arr = (capi.Segment * max(1, len(segs)))(*segs)
         sy = sync()
-        capi.check(L.mccl_copy_segments_sync(arr, len(segs), ctypes.byref(sy), stream))
+        capi.check(L.mccl_copy_segments_sync(arr, len(segs), i & 1, ctypes.byref(sy), stream))  # both load flavours
         want = O.alltoallv([to_carrier(h) for h in host], S, row)[rank]
         checks.append((out, want, ("copy_segments_sync", row, i)))
     torch.cuda.synchronize()

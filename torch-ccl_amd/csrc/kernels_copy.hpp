@@ -32,6 +32,7 @@ struct SyncCopyArgs {
   CopyArgs copy;
   XSync sync;
   uint32_t invalidate;  // some bytes are read through the caches: invalidate once per workgroup first
+  uint32_t shared;      // other ranks read the same sources: leave them in the memory-side cache
 };
 
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
@@ -45,7 +46,7 @@ struct SyncCopyArgs {
 // the segment geometry for the same value).  STREAM: full chunks are written through past the
 // caches (`sc1`) instead of with the non-temporal hint.
 template <bool COHERENT, int UNROLL, bool STREAM>
-__device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
+__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, bool shared_sources = false) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
@@ -74,7 +75,8 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a) {
       u32x4 x[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if (COHERENT && (((uintptr_t)src) & 7u) == 0) x[u] = load_vec_coherent(&((const u32x4*)src)[t + u * kWave]);
+        if (COHERENT && (((uintptr_t)src) & 7u) == 0)
+          x[u] = shared_sources ? load_tile_coherent_keep(src, (t + u * kWave) * 16u) : load_tile_coherent(src, (t + u * kWave) * 16u);
         else x[u] = __builtin_nontemporal_load(&sv[t + u * kWave]);
       }
 #pragma unroll
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCop
   if (xsync_begin(a.sync)) {
     // heads, partial chunks and misaligned sources go through the caches
     if (a.invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    copy_segments_body<true, kCopyUnroll, false>(a.copy);
+    copy_segments_body<true, kCopyUnroll, false>(a.copy, a.shared != 0);
   }
   xsync_end(a.sync, gridDim.x);
 }

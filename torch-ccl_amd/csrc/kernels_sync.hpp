@@ -66,6 +66,27 @@ __device__ __forceinline__ u32x4 load_vec_coherent(const u32x4* p) {
   return (u32x4){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
 }
 
+// The same for a wavefront that walks a tile: `tile` is the same address in every lane, lane l
+// accesses tile + off (off below 4 GiB).  One 16-byte access per lane through a buffer descriptor,
+// which is how the compiler can be given all three cache bits and still keep count of the access:
+// system scope (read past / written through the caches) and, for the load, non-temporal.  The hint
+// matters: eight read streams run at 6.5 TB/s with it and at 5.3 without, and as pairs of 8-byte
+// accesses at 4.8.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_descriptor(const char* tile) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile), 0, -1, 0x00020000);  // raw bytes, no bound
+}
+constexpr int kAuxSc0 = 1, kAuxNt = 2, kAuxSc1 = 16;
+__device__ __forceinline__ u32x4 load_tile_coherent(const char* tile, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(tile_descriptor(tile), off, 0, kAuxSc0 | kAuxSc1 | kAuxNt);
+}
+// without the non-temporal hint: for bytes that other ranks read as well in the same collective
+__device__ __forceinline__ u32x4 load_tile_coherent_keep(const char* tile, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(tile_descriptor(tile), off, 0, kAuxSc0 | kAuxSc1);
+}
+__device__ __forceinline__ void store_tile_through(char* tile, uint32_t off, u32x4 x) {
+  __builtin_amdgcn_raw_buffer_store_b128(x, tile_descriptor(tile), off, 0, kAuxSc0 | kAuxSc1);
+}
+
 // 16 bytes written through to memory with one store, at any alignment the element type allows.
 // The wait state after it covers a following write of the data registers.
 __device__ __forceinline__ void store_vec_through(char* p, u32x4 x) {

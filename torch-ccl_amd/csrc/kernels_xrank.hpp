@@ -47,44 +47,49 @@ struct XRankArgs {
   XSync sync;
 };
 
-// A vector of a peer's tensor: past the caches when the tensor is 8-byte aligned (always, for whole
-// tensors out of an allocator), else as an ordinary unaligned load after a cache invalidate the
-// host asked for (aligned_in == 0 makes the kernel invalidate once per workgroup).
-__device__ __forceinline__ u32x4 load_in(const char* base, uint32_t v, uint32_t aligned) {
-  if (aligned) return load_vec_coherent(&((const u32x4*)base)[v]);
-  return __builtin_nontemporal_load(&((const u32x4_unaligned*)base)[v]);
+// Lane l's vector of tile `tile` of a peer's tensor.  8-byte aligned tensors (always, for whole
+// tensors out of an allocator) are read past the caches in one streaming access (load_tile_coherent);
+// others as an ordinary unaligned load after a cache invalidate (aligned_in == 0 makes the kernel
+// invalidate once per workgroup).
+__device__ __forceinline__ u32x4 load_in(const char* base, uint32_t tile, uint32_t aligned) {
+  const char* tb = base + (size_t)tile * kXTileBytes;  // uniform
+  if (aligned) return load_tile_coherent(tb, threadIdx.x * 16u);
+  return __builtin_nontemporal_load(&((const u32x4_unaligned*)tb)[threadIdx.x]);
 }
 
-template <int DT, int OP>
-__device__ __forceinline__ void xrank_reduce_tile(const XRankArgs& a, uint32_t tile, int n) {
-  using S = typename Elem<DT>::store_t;
-  using A = typename Elem<DT>::acc_t;
-  constexpr int VE = vec_elems<DT>();
-  const int lane = threadIdx.x;
-  const uint32_t v = tile * kWave + (uint32_t)lane;  // the host keeps tiles1 * 64 below 2^32
-  const bool whole = v < a.nvec1;
-  const bool part = v == a.nvec1 && a.tail1 != 0;
-  if (whole || part) {
-    VecU<DT> x[kXRanks];
+// in[k] for a k known at run time only (a select per rank: no dynamic indexing of the argument block)
+__device__ __forceinline__ const char* pick_in(const XRankArgs& a, int k) {
+  const char* p = a.in[0];
+#pragma unroll
+  for (int q = 1; q < kXRanks; ++q)
+    if (k == q) p = a.in[q];
+  return p;
+}
+
+template <int DT, int NS>
+__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
+  const uint32_t v = tile * kWave + (uint32_t)threadIdx.x;  // the host keeps tiles1 * 64 below 2^32
+  if (v < a.nvec1) {
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) {
-      if (k < n) {
-        x[k].v = (u32x4){0u, 0u, 0u, 0u};
-        if (whole) {
-          x[k].v = load_in(a.in[k], v, a.aligned_in);
-        } else {
-#pragma unroll
-          for (int e = 0; e < VE; ++e)  // static indices: the vectors stay in registers
-            if ((uint32_t)e < a.tail1) vec_set<DT>(x[k], e, ((const S*)a.in[k])[(size_t)v * VE + e]);
-        }
-      }
+      if (NS ? k < NS : k < n) x[k].v = load_in(a.in[k], tile, a.aligned_in);
     }
+  }
+}
+
+// Reduces the loaded vectors of a tile (ascending-rank chain) and stores the result.
+template <int DT, int OP, int NS>
+__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
+  using A = typename Elem<DT>::acc_t;
+  constexpr int VE = vec_elems<DT>();
+  const uint32_t v = tile * kWave + (uint32_t)threadIdx.x;
+  if (v < a.nvec1) {
     A acc[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) acc[e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x[0], e)));
 #pragma unroll
     for (int k = 1; k < kXRanks; ++k) {
-      if (k < n) {
+      if (NS ? k < NS : k < n) {
 #pragma unroll
         for (int e = 0; e < VE; ++e) acc[e] = chain_next<DT, OP>(acc[e], Elem<DT>::load(vec_get<DT>(x[k], e)));
       }
@@ -98,25 +103,63 @@ __device__ __forceinline__ void xrank_reduce_tile(const XRankArgs& a, uint32_t t
       // it with kernels that start after this one has published its closing epoch
 #pragma unroll
       for (int k = 0; k < kXRanks; ++k) {
-        if (k < n) {
-          if (whole) {
-            store_vec_through(const_cast<char*>(a.in[k]) + (size_t)v * 16, r.v);
-          } else {
-#pragma unroll
-            for (int e = 0; e < VE; ++e)
-              if ((uint32_t)e < a.tail1)
-                __hip_atomic_store(&((S*)const_cast<char*>(a.in[k]))[(size_t)v * VE + e], vec_get<DT>(r, e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-          }
+        if (NS ? k < NS : k < n) {
+          char* tb = const_cast<char*>(a.in[k]) + (size_t)tile * kXTileBytes;  // uniform
+          if (a.aligned_in) store_tile_through(tb, threadIdx.x * 16u, r.v);
+          else store_vec_through(tb + threadIdx.x * 16u, r.v);
         }
       }
-    } else if (whole) {
-      u32x4_unaligned* o = &((u32x4_unaligned*)a.out1)[v];
-      if (a.stream_out) __builtin_nontemporal_store(r.v, o);
-      else *o = r.v;
     } else {
-#pragma unroll
-      for (int e = 0; e < VE; ++e)
-        if ((uint32_t)e < a.tail1) ((S*)a.out1)[(size_t)v * VE + e] = vec_get<DT>(r, e);
+      u32x4_unaligned* o = &((u32x4_unaligned*)a.out1)[v];
+      if (a.stream_out) store_vec_stream((u32x4*)o, r.v);
+      else *o = r.v;
+    }
+  }
+}
+
+// The elements after the last whole vector (fewer than a vector holds): lane e takes element e.
+template <int DT, int OP>
+__device__ __forceinline__ void xrank_tail(const XRankArgs& a, int n) {
+  using S = typename Elem<DT>::store_t;
+  using A = typename Elem<DT>::acc_t;
+  constexpr int VE = vec_elems<DT>();
+  if (threadIdx.x < a.tail1) {
+    const size_t i = (size_t)a.nvec1 * VE + threadIdx.x;
+    A acc = chain_first<DT, OP>(Elem<DT>::load(__hip_atomic_load(&((const S*)a.in[0])[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
+    for (int k = 1; k < n; ++k) {
+      const S* src = (const S*)pick_in(a, k);
+      acc = chain_next<DT, OP>(acc, Elem<DT>::load(__hip_atomic_load(&src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
+    }
+    const S r = Elem<DT>::store(chain_last<DT, OP>(acc, n));
+    if (a.push) {
+      for (int k = 0; k < n; ++k) __hip_atomic_store(&((S*)const_cast<char*>(pick_in(a, k)))[i], r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    } else {
+      ((S*)a.out1)[i] = r;
+    }
+  }
+}
+
+// The grid is persistent: a wavefront walks tiles blockIdx.x, + gridDim.x, ...  The loads of its
+// next tile are in flight while it reduces and stores the current one (two register sets, used
+// alternately): without that all wavefronts, released together by the opening wait, alternate
+// between a phase of loads and a phase of stores in step, and the memory pipeline runs dry
+// between the phases.
+template <int DT, int OP, int NS>
+__device__ __forceinline__ void xrank_walk(const XRankArgs& a, int n) {
+  const uint32_t T = a.tiles1, G = gridDim.x;
+  uint32_t t0 = blockIdx.x;
+  if (t0 < T) {
+    VecU<DT> x0[kXRanks], x1[kXRanks];
+    xrank_load_tile<DT, NS>(a, t0, n, x0);
+    for (;;) {
+      const uint32_t t1 = t0 + G;
+      if (t1 < T) xrank_load_tile<DT, NS>(a, t1, n, x1);
+      xrank_finish_tile<DT, OP, NS>(a, t0, n, x0);
+      if (t1 >= T) break;
+      t0 = t1 + G;
+      if (t0 < T) xrank_load_tile<DT, NS>(a, t0, n, x0);
+      xrank_finish_tile<DT, OP, NS>(a, t1, n, x1);
+      if (t0 >= T) break;
     }
   }
 }
@@ -126,7 +169,9 @@ __global__ __launch_bounds__(kWave) void xrank_reduce_kernel(const XRankArgs a) 
   const int n = a.sync.n;
   if (xsync_begin(a.sync)) {
     if (!a.aligned_in) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
-    for (uint32_t tile = blockIdx.x; tile < a.tiles1; tile += gridDim.x) xrank_reduce_tile<DT, OP>(a, tile, n);
+    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, n);
+    else xrank_walk<DT, OP, 0>(a, n);
+    if (a.tail1 && blockIdx.x == gridDim.x - 1) xrank_tail<DT, OP>(a, n);
   }
   xsync_end(a.sync, gridDim.x);
 }

@@ -110,6 +110,7 @@ constexpr long long kTuneDefault[MCCL_TUNE_COUNT_] = {
     /* COPY_STREAM_STORES       */ 3,  // neither 1 nor 2: chosen by size
     /* COPY_LARGE_MIN_BYTES     */ 1ll << 30,
     /* GATHER_WAVES_PER_CU      */ 28,
+    /* XRANK_CACHED_LOADS       */ 0,
 };
 constexpr int kCopyUnrollLarge = 2;   // vectors per lane per chunk of large copies
 constexpr int kCopyStreamLarge = 1;   // store flavour of large copies: 1 = written through (sc1), 2 = non-temporal
@@ -202,17 +203,17 @@ hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned grid
   }
 }
 
-hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned grid_x, hipStream_t s) {
+hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned grid_x, unsigned lds, hipStream_t s) {
   switch (dtype) {
-    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, grid_x, s);
-    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, grid_x, s);
-    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, grid_x, s);
-    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, grid_x, s);
-    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, grid_x, s);
-    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, grid_x, s);
-    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, grid_x, s);
-    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, grid_x, s);
-    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, grid_x, s);
+    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, grid_x, lds, s);
+    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, grid_x, lds, s);
+    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, grid_x, lds, s);
+    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, grid_x, lds, s);
+    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, grid_x, lds, s);
+    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, grid_x, lds, s);
+    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, grid_x, lds, s);
+    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, grid_x, lds, s);
+    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, grid_x, lds, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -806,7 +807,7 @@ int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
 
 extern "C" {
 
-int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsync_t* sync, void* stream) {
+int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync, void* stream) {
   SyncCopyArgs a;
   int rc = fill_xsync(sync, &a.sync);
   if (rc != MCCL_OK) return rc;
@@ -842,6 +843,7 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, const mccl_xsy
   // Full chunks of 8-byte aligned sources are read past the caches; whatever else there is (heads,
   // partial chunks, misaligned sources) is read through them, after an invalidate per workgroup.
   a.invalidate = 0;
+  a.shared = (flags & MCCL_COPY_SHARED_SOURCES) ? 1u : 0u;
   for (int k = 0; k < m; ++k) {
     const CopySeg& cs = a.copy.seg[k];
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
@@ -882,8 +884,8 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
   a.aligned_in = 1;
   for (int k = 0; k < a.sync.n; ++k)
     if (count && ((uintptr_t)in[k] & 7u)) a.aligned_in = 0;
-  if (a.tail1) a.aligned_in = 0;  // the last elements are read one by one, through the caches
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n), (hipStream_t)stream);
+  if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n), 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
@@ -923,8 +925,8 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   a.nvec1 = (uint32_t)(n_me / ve);
   a.tail1 = (uint32_t)(n_me % ve);
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
-  if (a.tail1) a.aligned_in = 0;  // the last elements are read one by one, through the caches
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n), (hipStream_t)stream);
+  if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n), 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }

@@ -28,6 +28,6 @@ extern "C" hipError_t MCCL_PASTE(mccl_launch_fused_dt, MCCL_REDUCE_DT)(MCCL_FUSE
   return launch_fused_dtype<MCCL_REDUCE_DT>(*static_cast<const FusedArgs*>(fused_args), op, grid_x, stream);
 }
 
-extern "C" hipError_t MCCL_PASTE(mccl_launch_xrank_dt, MCCL_REDUCE_DT)(MCCL_FUSED_ENTRY_ARGS) {
-  return launch_xrank_dtype<MCCL_REDUCE_DT>(*static_cast<const XRankArgs*>(fused_args), op, grid_x, stream);
+extern "C" hipError_t MCCL_PASTE(mccl_launch_xrank_dt, MCCL_REDUCE_DT)(MCCL_XRANK_ENTRY_ARGS) {
+  return launch_xrank_dtype<MCCL_REDUCE_DT>(*static_cast<const XRankArgs*>(xrank_args), op, grid_x, lds, stream);
 }

@@ -245,8 +245,11 @@ void GroupShared::putEvent(hipEvent_t e) {
 std::string GroupShared::failureMessage() {
   if (status && status[0] != 0 && !failed.load(std::memory_order_acquire)) {
     std::ostringstream os;
+    // epochs count four per collective: #(epoch / 4), wait (epoch % 4): 1 = inputs ready, 2 = between
+    // the phases of a two-phase collective, 3 = all ranks done with this rank's buffers
     os << "ccl backend: timed out waiting for rank " << (status[0] - 1)
-       << " on the device (cross-rank wait of a collective); the group cannot be used any more";
+       << " on the device (cross-rank wait " << (status[1] & 3u) << " of collective #" << (status[1] >> 2)
+       << ", modulo 2^30); the group cannot be used any more";
     fail(os.str());
   }
   if (!failed.load(std::memory_order_acquire)) return std::string();
@@ -814,7 +817,7 @@ void ProcessGroupCCL::hostBarrier(bool start_up) {
     while (ctl_->slot[r].arrive.load(std::memory_order_acquire) < epoch) {
       if (ctl_->slot[r].failed.load(std::memory_order_acquire)) {
         shared_->fail(c10::str("ccl backend: rank ", r, " reported a failure; aborting the collective"));
-        TORCH_CHECK(false, "ccl backend: rank ", r, " reported a failure; aborting the collective");
+        TORCH_CHECK(false, "ccl backend: rank ", r, " reported a failure; aborting the collective", lastEnqueued());
       }
       if (ctl_->slot[r].departed.load(std::memory_order_acquire)) {
         ctl_->slot[rank_].failed.store(1, std::memory_order_release);
@@ -866,7 +869,18 @@ void ProcessGroupCCL::throwIfFailed() {
   const std::string why = shared_->failureMessage();
   if (why.empty()) return;
   if (ctl_) ctl_->slot[rank_].failed.store(1, std::memory_order_release);
-  TORCH_CHECK(false, why);
+  TORCH_CHECK(false, why, lastEnqueued());
+}
+
+// What this rank enqueued last, for failure reports: a peer that others waited for in vain says
+// here how far it had come.
+std::string ProcessGroupCCL::lastEnqueued() const {
+  if (!last_title_) return std::string();
+  std::ostringstream os;
+  os << " [rank " << rank_ << " had last enqueued collective #" << last_seq_ << " (" << last_title_ << ", " << last_path_ << ")";
+  if (tail_pending_) os << (hipStreamQuery(tail_stream_) == hipSuccess ? ", its stream is idle" : ", its stream is still busy");
+  os << "]";
+  return os.str();
 }
 
 // The device-side cross-rank barrier on `s` (the sync kernels of src/gpu/allreduce.h:731-769).
@@ -1011,6 +1025,9 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       HIP_CHECK(hipEventRecord(tail_event_, tail_stream_));
       HIP_CHECK(hipStreamWaitEvent(s, tail_event_, 0));
     }
+    last_title_ = plan.title;
+    last_seq_ = seq + 1;
+    last_path_ = "one launch, fused";
     if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS) {
       const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
       MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
@@ -1062,8 +1079,17 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
     }
     if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
-    if (zero_copy && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
-        ((plan.one_launch_any_size && !one_launch_max_forced_) || plan.share_bytes <= one_launch_max_)) {
+    const bool one_launch = zero_copy && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
+                            ((plan.one_launch_any_size && !one_launch_max_forced_) || plan.share_bytes <= one_launch_max_);
+    last_path_ = one_launch ? "one launch, peers read in place"
+                            : zero_copy ? "barrier kernels, peers read in place"
+                                        : candidate ? "staged: a rank cannot share its tensor" : "staged";
+    if (verbose_) {
+      std::ostringstream os;
+      os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
+      std::cout << os.str() << std::endl;
+    }
+    if (one_launch) {
       // One launch: the kernel itself announces this rank, waits for the others, does the work
       // and (where a tensor must not be touched before the peers have read it) waits again.  With
       // several processes on the GPU every launch waits for its turn at the dispatcher, so this
@@ -1226,7 +1252,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
       const int me = rank_;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         mccl_segment_t seg{pv.user[(size_t)root], base, len};
-        MCCL_CHECK(mccl_copy_segments_sync(&seg, me == root ? 0 : 1, &sync, s));  // the root only takes part in the waits
+        MCCL_CHECK(mccl_copy_segments_sync(&seg, me == root ? 0 : 1, MCCL_COPY_SHARED_SOURCES, &sync, s));  // the root only takes part in the waits
         return true;
       };
     }
@@ -1434,7 +1460,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<mccl_segment_t> segs((size_t)W);
         for (int r = 0; r < W; ++r) segs[(size_t)r] = {pv.user[(size_t)r], out + (size_t)r * per_rank, len};
-        MCCL_CHECK(mccl_copy_segments_sync(segs.data(), W, &sync, s));
+        MCCL_CHECK(mccl_copy_segments_sync(segs.data(), W, MCCL_COPY_SHARED_SOURCES, &sync, s));
         return true;
       };
     }
@@ -1511,7 +1537,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   };
   p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
     const auto segs = pulls(pv);
-    MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), &sync, s));
+    MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), MCCL_COPY_SHARED_SOURCES, &sync, s));
     return true;
   };
   return run(p);
@@ -1922,7 +1948,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::exchange(c10d::OpType op, const 
     };
     p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
       const auto segs = pulls(pv);
-      MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), &sync, s));  // empty: still takes part in the waits
+      MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), 0u, &sync, s));  // empty: still takes part in the waits
       return true;
     };
     work = run(p);

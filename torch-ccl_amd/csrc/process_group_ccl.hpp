@@ -282,6 +282,7 @@ class ProcessGroupCCL : public c10d::Backend {
   void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void deviceBarrier(uint64_t epoch, hipStream_t s);
   void throwIfFailed();
+  std::string lastEnqueued() const;
   void awaitPeersEntered(uint64_t seq);
   // zero-copy: publish / map caller-owned allocations
   int exportRange(const void* ptr, size_t bytes, uint64_t* offset);
@@ -328,6 +329,9 @@ class ProcessGroupCCL : public c10d::Backend {
   // from a few hundred MiB of traffic on).  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides.
   size_t one_launch_max_ = 32u << 20;
   bool one_launch_max_forced_ = false;
+  const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
+  const char* last_path_ = "";
+  uint64_t last_seq_ = 0;
   bool comm_stream_for_large_ = false;  // MCCL_PG_COMM_STREAM=1: device-synchronised groups fork large collectives too
   // Decided at start-up, the same on every rank: all ranks are processes of their own (and the
   // environment does not ask for the host barrier), so cross-rank waits can live on the device.

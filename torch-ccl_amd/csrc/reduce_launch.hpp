@@ -99,16 +99,16 @@ hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned grid_x, hipSt
 
 // The one-launch cross-rank reduction (reduce_scatter, two-shot allreduce): persistent grid.
 template <int DT>
-hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned grid_x, hipStream_t s) {
+hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned grid_x, unsigned lds, hipStream_t s) {
   const dim3 grid(grid_x, 1, 1), block(kWave);
   switch (op) {
-    case MCCL_SUM: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_SUM>), grid, block, 0, s, a); break;
-    case MCCL_PROD: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_PROD>), grid, block, 0, s, a); break;
-    case MCCL_MIN: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MIN>), grid, block, 0, s, a); break;
-    case MCCL_MAX: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MAX>), grid, block, 0, s, a); break;
+    case MCCL_SUM: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_SUM>), grid, block, lds, s, a); break;
+    case MCCL_PROD: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_PROD>), grid, block, lds, s, a); break;
+    case MCCL_MIN: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MIN>), grid, block, lds, s, a); break;
+    case MCCL_MAX: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MAX>), grid, block, lds, s, a); break;
     case MCCL_AVG:
       if constexpr (Elem<DT>::kIsFloat) {
-        hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_AVG>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_AVG>), grid, block, lds, s, a);
         break;
       } else {
         return hipErrorInvalidValue;
@@ -149,14 +149,15 @@ __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt5(MCCL_FUSE
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt6(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt7(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt8(MCCL_FUSED_ENTRY_ARGS);
-// here `fused_args` points at an XRankArgs
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt0(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt1(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt2(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt3(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt4(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt5(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt6(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt7(MCCL_FUSED_ENTRY_ARGS);
-__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt8(MCCL_FUSED_ENTRY_ARGS);
+// `xrank_args` points at an XRankArgs; lds = dynamic LDS bytes reserved per workgroup (residency cap)
+#define MCCL_XRANK_ENTRY_ARGS const void *xrank_args, int op, unsigned grid_x, unsigned lds, hipStream_t stream
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt0(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt1(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt2(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt3(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt4(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt5(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt6(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt7(MCCL_XRANK_ENTRY_ARGS);
+__attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt8(MCCL_XRANK_ENTRY_ARGS);
 }
