@@ -324,10 +324,12 @@ class ProcessGroupCCL : public c10d::Backend {
   bool want_device_sync_ = true;  // MCCL_PG_SYNC != "host"
   bool zero_copy_ = true;         // MCCL_PG_ZERO_COPY != 0
   // Largest tensor (bytes per rank) whose zero-copy collective is ONE launch with the rank waits
-  // inside the kernel; larger ones run the bandwidth-tuned kernels between barrier kernels (the
-  // persistent one-launch kernels move fewer bytes per second, which outweighs the saved launches
-  // from a few hundred MiB of traffic on).  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides.
-  size_t one_launch_max_ = 32u << 20;
+  // inside the kernel; larger ones run the bandwidth-tuned kernels between barrier kernels.  With 8
+  // rank processes the two forms meet at 128-256 MiB per rank for reduce_scatter_tensor and
+  // all_to_all_single (one launch is 2x faster at 4-16 MiB, 15-20 % slower at 1 GiB: a persistent
+  // grid moves fewer bytes per second than fresh workgroups); the allreduce is one launch at every
+  // size.  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides (and then binds the allreduce, too).
+  size_t one_launch_max_ = 128u << 20;
   bool one_launch_max_forced_ = false;
   const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
   const char* last_path_ = "";
