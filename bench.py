@@ -488,6 +488,16 @@ def main():
             matrix[opname] = row
         result["pct_of_peak_by_op_and_ranks_64MiB"] = matrix
         log("ops x ranks:", json.dumps(matrix))
+        # what a bare kernel (xor, no conversions) sustains for the same read:write mix, best of the
+        # residency caps the library chooses from: a 2:1 mix has a lower ceiling than 8:1
+        sink = torch.empty_like(out)
+        bare = {}
+        for nr in range(2, N + 1):
+            us = min(benchlib.probe_stream(ins[:nr], sink, 1, block=64, workgroups_per_cu=w) for w in (0, 8, 10, 12, 14))
+            bare[str(nr)] = round((nr + 1) * S / us / 1e3 / PEAK_HBM_GBS * 100, 1)
+        result["bare_kernel_pct_of_peak_by_ranks_64MiB"] = bare
+        log("bare kernel by ranks:", json.dumps(bare))
+        del sink
         mccl.reduce_n(ins, out=out, op=mccl.SUM)  # the headline output again, for the checks below
 
     # ---------------- coalesced and list forms: one fused launch against one launch per tensor ----------------

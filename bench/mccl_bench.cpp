@@ -135,7 +135,11 @@ bool probe_dispatch(int n_read, const ProbeArgs& p, unsigned nvec, int block, un
     case 0: if (!WR) return false; probe_launch<0, WR>(p, nvec, block, lds, s); return true;
     case 1: probe_launch<1, WR>(p, nvec, block, lds, s); return true;
     case 2: probe_launch<2, WR>(p, nvec, block, lds, s); return true;
+    case 3: probe_launch<3, WR>(p, nvec, block, lds, s); return true;
     case 4: probe_launch<4, WR>(p, nvec, block, lds, s); return true;
+    case 5: probe_launch<5, WR>(p, nvec, block, lds, s); return true;
+    case 6: probe_launch<6, WR>(p, nvec, block, lds, s); return true;
+    case 7: probe_launch<7, WR>(p, nvec, block, lds, s); return true;
     case 8: probe_launch<8, WR>(p, nvec, block, lds, s); return true;
     default: return false;
   }
