@@ -279,7 +279,7 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--extras", default="all",
-                    help="comma list of c1,c2,c4,c5,moe,variants,ceilings,placement,lists,gloo,backend,copycal or all/none "
+                    help="comma list of c1,c2,c4,c5,moe,variants,ceilings,placement,lists,xrank,gloo,backend,copycal or all/none "
                          "(copycal: a 512 MiB single-segment copy, the known-size kernel that "
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters; not part of 'all')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -290,7 +290,7 @@ def main():
             "--gpus %d is not supported (run with --gpus 1)." % args.gpus)
         sys.exit(2)
 
-    extras = set("c1,c2,c4,c5,moe,variants,ceilings,placement,lists,gloo,backend".split(",")) if args.extras == "all" else \
+    extras = set("c1,c2,c4,c5,moe,variants,ceilings,placement,lists,xrank,gloo,backend".split(",")) if args.extras == "all" else \
         set() if args.extras == "none" else set(args.extras.split(","))
 
     import importlib.util
@@ -499,6 +499,79 @@ def main():
         log("bare kernel by ranks:", json.dumps(bare))
         del sink
         mccl.reduce_n(ins, out=out, op=mccl.SUM)  # the headline output again, for the checks below
+
+    # ---------------- the one-launch cross-rank kernels, all ranks played by this process ----------------
+    # Between rank processes these kernels wait for each other on flag words; here every rank's word is
+    # the same word of this process, so the launches of the 8 "ranks" run one after the other and the
+    # figure is the kernel's own (persistent grid, coherent loads, closing count), without the turn
+    # taking of 8 processes that the backend leg includes.
+    if "xrank" in extras:
+        L = capi.lib()
+        word = torch.zeros(8, dtype=torch.int64, device=dev)
+        counter = torch.zeros(256, dtype=torch.int32, device=dev)  # MCCL_SYNC_COUNTER_BYTES
+        status = torch.zeros(16, dtype=torch.int32).pin_memory()
+        words = capi.ptr_table([word.data_ptr()] * N)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        calls = [0]
+
+        def xsync(rank):
+            calls[0] += 1
+            return capi.XSync(ctypes.cast(words, ctypes.c_void_p), N, rank, 4 * calls[0] + 1, 4 * calls[0] + 3,
+                              counter.data_ptr(), 5_000_000, status.data_ptr())
+
+        def event_us(fn, reps=20):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / reps
+
+        xr = {}
+        # a rank's grid is 1/N of the wavefront budget of all ranks; here no other rank's launch is
+        # resident, so each launch gets the whole budget
+        budget = L.mccl_get_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS)
+        L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget * N)
+        in_tab = capi.ptr_table([t.data_ptr() for t in ins])
+        xout = torch.empty_like(out)
+
+        def reduce_sync():
+            sy = xsync(0)
+            capi.check(L.mccl_reduce_sync(in_tab, xout.data_ptr(), COUNT, capi.BF16, capi.SUM, ctypes.byref(sy), stream))
+        us = event_us(reduce_sync)
+        xr["reduce_sync_8x64MiB_to_64MiB"] = {"us": round(us, 1), "GBps": round(alg_bytes / us / 1e3, 1),
+                                              "pct_of_peak": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                              "bit_identical_to_reduce_n": bool(torch.equal(xout.view(torch.int16), out.view(torch.int16)))}
+        # the in-place allreduce: rank 0's launch alone (its shard of all eight tensors reduced and written
+        # back into all eight), checked against the headline output; the whole collective is timed by the
+        # backend leg, where the eight ranks' launches run side by side
+        tens = [t.clone() for t in ins]
+        ten_tab = capi.ptr_table([t.data_ptr() for t in tens])
+        shard = L.mccl_allreduce_sync_shard(COUNT, N)
+
+        def allreduce_rank0():
+            sy = xsync(0)
+            capi.check(L.mccl_allreduce_sync(ten_tab, COUNT, capi.BF16, capi.SUM, ctypes.byref(sy), stream))
+        allreduce_rank0()
+        torch.cuda.synchronize()
+        same = all(torch.equal(t[:shard].view(torch.int16), out[:shard].view(torch.int16)) for t in tens)
+        us = event_us(allreduce_rank0)  # (the repetitions reduce an already reduced shard: same traffic)
+        moved = 2 * N * shard * 2
+        xr["allreduce_sync_rank0_shard_of_8x64MiB"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
+                                                       "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                                       "first_pass_bit_identical_to_reduce_n": bool(same)}
+        L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget)
+        assert status.tolist()[:2] == [0, 0], status.tolist()
+        xr["wavefronts_per_launch"] = int(budget)
+        xr["note"] = ("single process: every rank's flag word is the same word, so no launch waits, and a launch has "
+                      "the wavefront budget of all ranks")
+        result["cross_rank_kernels_single_process"] = xr
+        log("cross-rank kernels:", json.dumps(xr))
+        del tens, xout
 
     # ---------------- coalesced and list forms: one fused launch against one launch per tensor ----------------
     if "lists" in extras:

@@ -212,10 +212,11 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
  * separate sync kernels of src/gpu/allreduce.h:731-769, 835-877 around the data kernels.
  *   words[r]: rank r's 64-bit word as for mccl_rank_barrier (the same word may serve both; epochs
  * grow: ready_epoch of a call > any epoch used before, done_epoch > ready_epoch).  done_counter:
- * one 32-bit word of this rank's device memory, zero before the first call (the kernel leaves it
- * zero).  Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
+ * MCCL_SYNC_COUNTER_BYTES of this rank's device memory, 64-byte aligned, zero before the first call
+ * (the kernel leaves them zero): the workgroups count themselves out there.  Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
  * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
  */
+#define MCCL_SYNC_COUNTER_BYTES 1024
 typedef struct {
   void* const* words;
   int n;

@@ -151,12 +151,16 @@ struct XSync {
   uint64_t* word[kLeanSyncRanks];  // rank r's 64-bit word
   uint64_t ready_epoch;
   uint64_t done_epoch;
-  uint32_t* done_count;            // this rank's counter: zero between launches
+  uint32_t* done_count;            // this rank's counters (MCCL_SYNC_COUNTER_BYTES): zero between launches
   uint64_t limit_ticks;
   uint32_t* status;
   int n;
   int rank;
 };
+
+constexpr uint32_t kDoneGroups = 8;
+constexpr uint32_t kDoneStride = 16;  // 32-bit words between two counters: one cache line each
+static_assert((1 + kDoneGroups) * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "counters must fit the block the caller provides");
 
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
 __device__ __forceinline__ bool xsync_begin(const XSync& x) {
@@ -183,13 +187,22 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
   const int lane = threadIdx.x;
   uint32_t last = 0;
   if (lane == 0) {
-    // relaxed: the ordering that matters (this workgroup's accesses are complete) was established
-    // above, and an acquire-release atomic would add a cache write-back and invalidate per workgroup
-    const uint32_t before = __hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last = before + 1 == workgroups ? 1u : 0u;
-    if (last) {
-      __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-      __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    // Relaxed: the ordering that matters (this workgroup's accesses are complete) was established
+    // above, and an acquire-release atomic would add a cache write-back and invalidate per workgroup.
+    // Counted in two levels -- eight group counters on cache lines of their own, then one for the
+    // groups -- because atomics on one address are carried out one after the other (about 7 ns
+    // each: 29 us for a grid of 4096 workgroups on a single counter).
+    const uint32_t groups = workgroups < kDoneGroups ? 1u : kDoneGroups;
+    const uint32_t g = blockIdx.x % groups;
+    const uint32_t members = (workgroups - g + groups - 1) / groups;
+    uint32_t* mine = x.done_count + kDoneStride * (1 + g);
+    if (__hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == members) {
+      __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      if (__hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == groups) {
+        last = 1u;
+        __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
     }
   }
   last = __builtin_amdgcn_readfirstlane(last);

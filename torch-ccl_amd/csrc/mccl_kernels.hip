@@ -786,7 +786,8 @@ int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
   if (sy->ready_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "ready_epoch must be positive");
   if (sy->done_epoch != 0 && sy->done_epoch <= sy->ready_epoch) return fail(MCCL_ERR_INVALID_ARG, "done_epoch must be 0 or above ready_epoch");
   if (sy->done_epoch != 0 && !sy->done_counter) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs a done counter");
-  if ((uintptr_t)sy->done_counter % 4 || (uintptr_t)sy->status % 4) return fail(MCCL_ERR_INVALID_ARG, "counter or status word is not 4-byte aligned");
+  if ((uintptr_t)sy->done_counter % 64) return fail(MCCL_ERR_INVALID_ARG, "the done counters are not 64-byte aligned");
+  if ((uintptr_t)sy->status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
   memset(x, 0, sizeof(*x));
   for (int r = 0; r < sy->n; ++r) {
     if (!sy->words[r]) return fail(MCCL_ERR_INVALID_ARG, "sync word %d is null", r);

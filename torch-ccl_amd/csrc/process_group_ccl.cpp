@@ -64,9 +64,10 @@ constexpr size_t kArenaFusedFlagsOff = 4096;                 // two sets of tile
 constexpr size_t kArenaFusedFlagsStride = 8192;
 constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buffers of 1 MiB, each
 constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
-constexpr size_t kArenaDoneCountOff = 256;  // 32-bit workgroup counter of the one-launch collectives
+constexpr size_t kArenaDoneCountOff = 1024;  // MCCL_SYNC_COUNTER_BYTES of workgroup counters of the one-launch collectives
 constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
 static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
+static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedFlagsOff, "the counters end before the flags");
 
 #define HIP_CHECK(expr)                                                                     \
   do {                                                                                      \
