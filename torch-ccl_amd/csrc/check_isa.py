@@ -20,6 +20,13 @@ streaming store (a hand-written `sc1` instruction) beside the cacheable one, and
 followed by the wait state the compiler cannot know it needs; the full-chunk
 path of the copy kernel, the combine kernel and the stores of the row gather must be non-temporal.
 
+A fourth scan covers the kernels that wait for other ranks inside a launch: each must use at most
+128 vector registers, because the wavefront budget of all ranks (4096) is sized for four
+wavefronts per SIMD -- with fewer, the waiting workgroups of seven ranks could fill the GPU and
+keep the eighth rank's first workgroup out for good -- and the reduction among them must read the
+peers' tensors with `buffer_load_dwordx4 ... sc0 sc1 nt` (coherent and streaming) and write
+them back with `buffer_store_dwordx4 ... sc0 sc1`.
+
 Usage: python torch-ccl_amd/csrc/check_isa.py   (exit status 1 if anything is flagged)
 """
 import os
@@ -148,12 +155,42 @@ def scan_hints(asm_path):
     return bad
 
 
+_WAITING_KERNEL = re.compile(r"(xrank_reduce_kernel|copy_segments_sync_kernel|allreduce_fused_kernel|rank_barrier_kernel)")
+_MAX_VGPRS_OF_WAITING_KERNELS = 128
+
+
+def scan_waiting_kernels(asm_path):
+    """Returns a list of (function, problem) for the kernels that wait for other ranks."""
+    bad, seen, fn, acc = [], 0, None, {}
+    with open(asm_path) as f:
+        for line in f:
+            t = line.strip()
+            m = re.match(r"^(_Z[\w.$]*):", t)
+            if m:
+                fn = m.group(1)
+                continue
+            m = re.match(r"^\.set (_Z[\w.$]*)\.num_vgpr, (\d+)", t)
+            if m and _WAITING_KERNEL.search(m.group(1)):
+                seen += 1
+                if int(m.group(2)) > _MAX_VGPRS_OF_WAITING_KERNELS:
+                    bad.append((m.group(1), "%s vector registers: fewer than four wavefronts per SIMD" % m.group(2)))
+            if fn and "xrank_reduce_kernel" in fn and t.startswith(("buffer_load_dwordx4", "buffer_store_dwordx4")):
+                kind = "load" if t.startswith("buffer_load") else "store"
+                acc.setdefault(fn, set()).add((kind, " ".join(sorted(_hint(t).split()))))
+    for fn, kinds in acc.items():
+        if kinds != {("load", "nt sc0 sc1"), ("store", "sc0 sc1")}:
+            bad.append((fn, "coherent accesses of the cross-rank reduction changed flavour: %r" % sorted(kinds)))
+    if not seen or not acc:
+        bad.append(("xrank_reduce_kernel", "no waiting kernel recognised (name mangling changed?)"))
+    return bad
+
+
 def main():
     with tempfile.TemporaryDirectory() as d:
         asm = os.path.join(d, "mccl_kernels.s")
         device_asm(asm)
         flagged = scan(asm)
-        hints = scan_hints(asm)
+        hints = scan_hints(asm) + scan_waiting_kernels(asm)
     for fn, problem in hints:
         print("cache hint in %s: %s" % (fn, problem))
     print("cache hints flagged: %d" % len(hints))
