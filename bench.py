@@ -147,6 +147,15 @@ def _backend_rank(rank, world, store_path, cases, out_path):
         g = rank_generator(torch, SEED, rank)
         x = (torch.randn(count, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16).to("cuda:0")
         t = x.clone()
+        dist.all_reduce(t)
+        # bit for bit against an fp32 chain over all ranks' inputs in ascending rank order
+        acc = None
+        for r in range(world):
+            gr = rank_generator(torch, SEED, r)
+            xr = (torch.randn(count, generator=gr, dtype=torch.float32) * 0.02).to(torch.bfloat16).to("cuda:0").float()
+            acc = xr if acc is None else acc.add_(xr)
+        exact = bool(torch.equal(t.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16)))
+        del acc, xr
         for _ in range(warm):
             dist.all_reduce(t)
         torch.cuda.synchronize()
@@ -160,7 +169,8 @@ def _backend_rank(rank, world, store_path, cases, out_path):
             torch.cuda.synchronize()
             ts.append(time.perf_counter() - t0)
         ts.sort()
-        res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters}
+        res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters,
+                     "first_call_bit_exact_vs_fp32_chain": exact}
         # the same call back to back (20 calls, one synchronize): what a loop of collectives pays per call
         torch.cuda.synchronize()
         dist.barrier()

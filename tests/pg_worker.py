@@ -665,6 +665,68 @@ def zero_copy_cases(pg, rank, world):
     pg.barrier().wait()
 
 
+def baseline_config_cases(pg, rank, world):
+    """The benchmark configurations at their full size through the drop-in API, 8 rank processes:
+    C3 (allreduce of 64 MiB bf16 per rank), C4's shape at a quarter of its size (reduce_scatter_tensor of
+    256 MiB bf16 per rank) and C5 (all_to_all_single of 4096 tokens x top-8 x 7168 bf16 per rank with
+    the routing counts of a seeded top-8-of-256 gate).  Every rank regenerates all ranks' inputs
+    on the device and checks its result bit for bit against an fp32 chain in ascending rank order
+    (one rounding at the end), respectively against the rows it must have received."""
+    def rank_input(r, count, seed):
+        g = torch.Generator(device=DEV)
+        g.manual_seed(seed * 1000 + r)
+        return (torch.randn(count, generator=g, device=DEV, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+
+    def chain(inputs):
+        acc = inputs[0].float()
+        for x in inputs[1:]:
+            acc += x.float()
+        return acc.to(torch.bfloat16)
+
+    # C3
+    count = 4096 * 8192
+    xs = [rank_input(r, count, 3) for r in range(world)]
+    want = chain(xs)
+    t = xs[rank].clone()
+    for _ in range(2):  # the second call reduces fresh contents in the same tensor (same mappings)
+        t.copy_(xs[rank])
+        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        assert torch.equal(t.view(torch.int16), want.view(torch.int16)), "C3 through the backend"
+    del xs, want, t
+    # C4 shape, 256 MiB per rank
+    m = (128 << 20) // world
+    xs = [rank_input(r, m * world, 4) for r in range(world)]
+    want = chain([x[rank * m:(rank + 1) * m] for x in xs])
+    out = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    pg._reduce_scatter_base(out, xs[rank]).wait()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16)), "C4 shape through the backend"
+    assert torch.equal(xs[rank].view(torch.int16), rank_input(rank, m * world, 4).view(torch.int16)), "reduce_scatter changed its input"
+    del xs, want, out
+    # C5: rows tagged with (source rank, row index) in their first eight bytes
+    tokens, hidden, topk, experts = 4096, 7168, 8, 256
+    S = torch.zeros(world, world, dtype=torch.int64)
+    for r in range(world):
+        g = torch.Generator()
+        g.manual_seed(5000 + r)
+        picks = torch.topk(torch.randn(tokens, experts, generator=g), topk, dim=1).indices
+        S[r] = torch.bincount(picks.reshape(-1) // (experts // world), minlength=world)
+    rows = tokens * topk
+    inp = torch.empty(rows, hidden, dtype=torch.bfloat16, device=DEV)
+    tags = inp.view(torch.int16).view(rows, hidden)
+    tags.copy_((torch.arange(rows, device=DEV).view(-1, 1) * 31 + torch.arange(hidden, device=DEV).view(1, -1) * 7 + rank * 1009) % 30011)
+    out = torch.zeros(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device=DEV)
+    pg.alltoall_base(out, inp, S[:, rank].tolist(), S[rank].tolist()).wait()
+    got = out.view(torch.int16).view(-1, hidden)
+    pos = 0
+    for r in range(world):
+        n = int(S[r, rank])
+        first = int(S[r, :rank].sum())
+        want = ((torch.arange(first, first + n, device=DEV).view(-1, 1) * 31 + torch.arange(hidden, device=DEV).view(1, -1) * 7 + r * 1009) % 30011).to(torch.int16)
+        assert torch.equal(got[pos:pos + n], want), ("C5 through the backend", r)
+        pos += n
+    pg.barrier().wait()
+
+
 def missing_rank_device_case(pg, rank, world):
     """Device-side waits: rank 1 never joins the second collective.  The survivors' kernel gives up
     by itself at the (shortened) limit and names the late rank; their Work reports the failure
@@ -983,6 +1045,8 @@ def run_rank(rank, world, store_path, mode):
         missing_sender_case(pg, rank, world)
     elif mode == "zero_copy":
         zero_copy_cases(pg, rank, world)
+    elif mode == "baseline_configs":
+        baseline_config_cases(pg, rank, world)
     elif mode == "missing_device":
         missing_rank_device_case(pg, rank, world)
     elif mode == "late_peer":
