@@ -100,15 +100,29 @@ __device__ __forceinline__ void wait_own_stores() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// Pause between two polls of a flag: half a microsecond at first, then about an eighth of the time
+// waited so far, up to 40 us.  Thousands of wavefronts of several processes may be polling the
+// same few words, past the caches: at a fixed half microsecond the waiting ranks of a collective
+// put tens of billions of uncached requests per second on the memory channels that hold the
+// words, for as long as a late rank needs -- and slow that rank down while it is at it.
+__device__ __forceinline__ void poll_pause(uint64_t waited_ticks) {
+  const uint32_t long_naps = (uint32_t)(waited_ticks >> 12);  // one per 41 us waited (100 MHz ticks)
+  if (long_naps == 0) {
+    __builtin_amdgcn_s_sleep(16);
+  } else {
+    const uint32_t naps = long_naps < 10u ? long_naps : 10u;
+    for (uint32_t i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);  // about 4 us each
+  }
+}
+
 // Polls *word until it is at least `epoch` (64-bit, monotonic).  Returns false at the time limit.
-// Between polls the wavefront sleeps about half a microsecond: thousands of workgroups of several
-// processes may be waiting on the same few words.
 __device__ __forceinline__ bool wait_flag64(const uint64_t* word, uint64_t epoch, uint64_t limit_ticks) {
   if (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) >= epoch) return true;
   const uint64_t t0 = wall_clock64();
   do {
-    if (wall_clock64() - t0 > limit_ticks) return false;
-    __builtin_amdgcn_s_sleep(16);
+    const uint64_t waited = wall_clock64() - t0;
+    if (waited > limit_ticks) return false;
+    poll_pause(waited);
   } while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) < epoch);
   return true;
 }
@@ -118,8 +132,9 @@ __device__ __forceinline__ bool wait_flag32(const uint32_t* word, uint32_t epoch
   if ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) >= 0) return true;
   const uint64_t t0 = wall_clock64();
   do {
-    if (wall_clock64() - t0 > limit_ticks) return false;
-    __builtin_amdgcn_s_sleep(8);
+    const uint64_t waited = wall_clock64() - t0;
+    if (waited > limit_ticks) return false;
+    poll_pause(waited);
   } while ((int32_t)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - epoch) < 0);
   return true;
 }
