@@ -1080,9 +1080,16 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
     }
     if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
-    const bool one_launch = zero_copy && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
-                            ((plan.one_launch_any_size && !one_launch_max_forced_) || plan.share_bytes <= one_launch_max_);
-    last_path_ = one_launch ? "one launch, peers read in place"
+    // One launch: the kernel itself announces this rank, waits for the others, does the work and
+    // (in place: where a tensor must not be touched before the peers have read it) waits again.
+    // With several processes on the GPU every launch waits for its turn at the dispatcher, so this
+    // is worth more than any bandwidth.  Staged collectives get the same kernel behind their
+    // copy-in (two launches instead of three): the launch says "my staging buffer is complete",
+    // and no closing wait is needed, as for every staged collective (see the slot rule above).
+    const size_t moved = zero_copy ? plan.share_bytes : plan.stage_bytes;
+    const bool one_launch = plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS && (zero_copy || !plan.exec_sync_in_place_only) &&
+                            ((zero_copy && plan.one_launch_any_size && !one_launch_max_forced_) || moved <= one_launch_max_);
+    last_path_ = one_launch ? (zero_copy ? "one launch, peers read in place" : "copy-in and one launch")
                             : zero_copy ? "barrier kernels, peers read in place"
                                         : candidate ? "staged: a rank cannot share its tensor" : "staged";
     if (verbose_) {
@@ -1091,16 +1098,13 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       std::cout << os.str() << std::endl;
     }
     if (one_launch) {
-      // One launch: the kernel itself announces this rank, waits for the others, does the work
-      // and (where a tensor must not be touched before the peers have read it) waits again.  With
-      // several processes on the GPU every launch waits for its turn at the dispatcher, so this
-      // is worth more than any bandwidth.
+      if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
       mccl_xsync_t sync;
       sync.words = bar_flags_.data();
       sync.n = size_;
       sync.rank = rank_;
       sync.ready_epoch = epoch + 1;
-      sync.done_epoch = epoch + 3;
+      sync.done_epoch = zero_copy ? epoch + 3 : 0;
       sync.done_counter = done_counter_;
       sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
       sync.status = status_dev_;
@@ -1108,6 +1112,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
         if (timed) { phase_us_[2].push_back(0.f); phase_us_[3].push_back((float)us_since(t0)); }
         return;
       }
+      TORCH_CHECK(zero_copy || !plan.copy_in, "ccl backend: a staged one-launch plan declined after its copy-in");
     }
     if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
     deviceBarrier(epoch + 1, s);  // every rank's input is complete (staged, or ready in place)
@@ -1252,7 +1257,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
     if (len) {
       const int me = rank_;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
-        mccl_segment_t seg{pv.user[(size_t)root], base, len};
+        mccl_segment_t seg{pv.zero_copy ? pv.user[(size_t)root] : pv.stage[(size_t)root], base, len};
         MCCL_CHECK(mccl_copy_segments_sync(&seg, me == root ? 0 : 1, MCCL_COPY_SHARED_SOURCES, &sync, s));  // the root only takes part in the waits
         return true;
       };
@@ -1346,6 +1351,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // written per rank, nothing staged.  Faster than the launches of the form above at every
       // size measured (16 MiB to 512 MiB per rank), so it is not subject to the one-launch limit.
       p.one_launch_any_size = true;
+      p.exec_sync_in_place_only = true;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<void*> tensors((size_t)W);
         for (int k = 0; k < W; ++k) tensors[(size_t)k] = const_cast<void*>(pv.user[(size_t)k]);
@@ -1460,7 +1466,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
       };
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<mccl_segment_t> segs((size_t)W);
-        for (int r = 0; r < W; ++r) segs[(size_t)r] = {pv.user[(size_t)r], out + (size_t)r * per_rank, len};
+        for (int r = 0; r < W; ++r)
+          segs[(size_t)r] = {pv.zero_copy ? pv.user[(size_t)r] : pv.stage[(size_t)r], out + (size_t)r * per_rank, len};
         MCCL_CHECK(mccl_copy_segments_sync(segs.data(), W, MCCL_COPY_SHARED_SOURCES, &sync, s));
         return true;
       };
@@ -1649,7 +1656,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
       };
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<const void*> src((size_t)W);
-        for (int k = 0; k < W; ++k) src[(size_t)k] = (const char*)pv.user[(size_t)k] + ((size_t)me * M + m0) * es;
+        for (int k = 0; k < W; ++k)  // in place: slice `me` of rank k's tensor; staged: slice `me` of the window rank k staged
+          src[(size_t)k] = pv.zero_copy ? (const char*)pv.user[(size_t)k] + ((size_t)me * M + m0) * es
+                                        : (const char*)pv.stage[(size_t)k] + (size_t)me * len * es;
         MCCL_CHECK(mccl_reduce_sync(src.data(), out, len, dtype, op, &sync, s));
         return true;
       };

@@ -247,6 +247,7 @@ class ProcessGroupCCL : public c10d::Backend {
     const void* share_ptr = nullptr;
     size_t share_bytes = 0;
     size_t zero_copy_stage_bytes = 0;       // staging this rank still needs in zero-copy mode
+    bool exec_sync_in_place_only = false;   // exec_sync writes into the peers' tensors: not for staged runs
     bool one_launch_any_size = false;       // exec_sync wins at every size: the default one-launch limit does not apply
     // Eligible for the one-launch small allreduce (device-synchronised groups of at most 8 ranks):
     // no staging slot, no table, no rendezvous.  The staged plan above stays as the fallback.
