@@ -601,6 +601,20 @@ void ProcessGroupCCL::ensureInit(int device) {
     for (int b = a + 1; b < size_; ++b)
       if (ctl_->slot[a].pid == ctl_->slot[b].pid) distinct = false;
   device_sync_ = size_ > 1 && distinct && want_device_sync_;
+  if (device_sync_ && rank_ == 0) {
+    // A kernel that waits for other ranks only makes progress while the hardware queues of all rank
+    // processes are mapped at once.  A process owns up to GPU_MAX_HW_QUEUES of them (4 unless set),
+    // one per group of streams it uses; with 8 rank processes that use three or more streams each
+    // the GPU maps fewer queues than exist and time-slices them, and a collective then takes a
+    // scheduling quantum (measured: 11 ms instead of 0.1 ms).  One or two queues per process are safe.
+    const char* q = std::getenv("GPU_MAX_HW_QUEUES");
+    const long queues = q ? std::atol(q) : 4;
+    if (queues * size_ > 16)
+      TORCH_WARN_ONCE("ccl backend: ", size_, " rank processes share one GPU and wait for each other on the device; if the "
+                      "ranks use more than two streams each, set GPU_MAX_HW_QUEUES=2 (or 1) in their environment, or "
+                      "MCCL_PG_SYNC=host: with more hardware queues than the GPU maps at once a collective costs a "
+                      "scheduling quantum (about 10 ms)");
+  }
   if (size_ > 1) {
     peer_arena_.assign((size_t)size_, nullptr);
     bar_flags_.assign((size_t)size_, nullptr);
