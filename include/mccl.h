@@ -213,7 +213,10 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
  *   words[r]: rank r's 64-bit word as for mccl_rank_barrier (the same word may serve both; epochs
  * grow: ready_epoch of a call > any epoch used before, done_epoch > ready_epoch).  done_counter:
  * MCCL_SYNC_COUNTER_BYTES of this rank's device memory, 64-byte aligned, zero before the first call
- * (the kernel leaves them zero): the workgroups count themselves out there.  Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
+ * (the kernel leaves them zero): the workgroups count themselves out there.  ready_epoch == 0 (then
+ * done_epoch must be 0 as well; words, counters and status are not used): the kernel does not wait
+ * at all, for callers that order the ranks themselves, e.g. with host barriers around the launch.
+ * Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
  * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
  */
 #define MCCL_SYNC_COUNTER_BYTES 1024
@@ -253,8 +256,8 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
  * src/gpu/allreduce.h:306-533) moves n + 1 reads and 2 writes in two phases with a rank
  * synchronisation between them (its gather step stores into its peers' buffers likewise,
  * src/gpu/allreduce.h:470-487).  Only the owner of a shard touches it in any tensor while the
- * collective runs; done_epoch is required: no rank's kernel ends before every rank has written its
- * shard everywhere.  Same bits as mccl_reduce_n over the n tensors.
+ * collective runs; done_epoch is required (unless ready_epoch is 0): no rank's kernel ends before
+ * every rank has written its shard everywhere.  Same bits as mccl_reduce_n over the n tensors.
  */
 size_t mccl_allreduce_sync_shard(size_t count, int n);
 int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync,

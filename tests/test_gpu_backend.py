@@ -115,7 +115,8 @@ def test_baseline_configs_at_full_size_through_the_backend():
     _spawn(8, "baseline_configs")
 
 
-@pytest.mark.parametrize("world,mode", [(2, "reference"), (4, "oracle"), (3, "p2p"), (4, "dist"), (2, "zero_copy")])
+@pytest.mark.parametrize("world,mode", [(2, "reference"), (4, "oracle"), (3, "p2p"), (4, "dist"), (2, "zero_copy"), (8, "zero_copy"),
+                                        (8, "baseline_configs")])
 def test_host_synchronised_fallback(monkeypatch, world, mode):
     """MCCL_PG_SYNC=host: the same cases with hipStreamSynchronize + the host barrier instead of
     device-side waits (what ranks that share a process always use)."""

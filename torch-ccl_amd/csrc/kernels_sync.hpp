@@ -179,6 +179,7 @@ static_assert((1 + kDoneGroups) * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "c
 
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
 __device__ __forceinline__ bool xsync_begin(const XSync& x) {
+  if (x.ready_epoch == 0) return true;  // the caller has ordered the ranks on the host
   const int lane = threadIdx.x & (kWave - 1);
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
     __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);

@@ -780,15 +780,20 @@ unsigned xrank_grid(uint64_t tiles, int n) {
 
 int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
   if (!sy) return fail(MCCL_ERR_INVALID_ARG, "sync descriptor is null");
-  if (!sy->words) return fail(MCCL_ERR_INVALID_ARG, "sync word table is null");
   if (sy->n < 1 || sy->n > kXRanks) return fail(MCCL_ERR_UNSUPPORTED, "one-launch collectives take 1 to %d ranks, got %d", kXRanks, sy->n);
   if (sy->rank < 0 || sy->rank >= sy->n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", sy->rank, sy->n);
-  if (sy->ready_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "ready_epoch must be positive");
+  memset(x, 0, sizeof(*x));
+  x->n = sy->n;
+  x->rank = sy->rank;
+  if (sy->ready_epoch == 0) {  // the caller orders the ranks itself: no wait inside the kernel
+    if (sy->done_epoch != 0) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs an opening one (ready_epoch)");
+    return MCCL_OK;
+  }
+  if (!sy->words) return fail(MCCL_ERR_INVALID_ARG, "sync word table is null");
   if (sy->done_epoch != 0 && sy->done_epoch <= sy->ready_epoch) return fail(MCCL_ERR_INVALID_ARG, "done_epoch must be 0 or above ready_epoch");
   if (sy->done_epoch != 0 && !sy->done_counter) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs a done counter");
   if ((uintptr_t)sy->done_counter % 64) return fail(MCCL_ERR_INVALID_ARG, "the done counters are not 64-byte aligned");
   if ((uintptr_t)sy->status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
-  memset(x, 0, sizeof(*x));
   for (int r = 0; r < sy->n; ++r) {
     if (!sy->words[r]) return fail(MCCL_ERR_INVALID_ARG, "sync word %d is null", r);
     if ((uintptr_t)sy->words[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "sync word %d is not 8-byte aligned", r);
@@ -799,8 +804,6 @@ int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
   x->done_count = (uint32_t*)sy->done_counter;
   x->limit_ticks = wait_limit_ticks(sy->timeout_us);
   x->status = (uint32_t*)sy->status;
-  x->n = sy->n;
-  x->rank = sy->rank;
   return MCCL_OK;
 }
 
@@ -905,7 +908,8 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
   if (rc != MCCL_OK) return rc;
   if (!tensors) return fail(MCCL_ERR_INVALID_ARG, "tensor table is null");
-  if (a.sync.done_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "the pushing allreduce needs a closing wait (done_epoch)");
+  if (a.sync.ready_epoch != 0 && a.sync.done_epoch == 0)
+    return fail(MCCL_ERR_INVALID_ARG, "the in-place allreduce needs a closing wait (done_epoch) when it waits at all");
   const int n = a.sync.n, me = a.sync.rank;
   const size_t es = dtype_size(dtype);
   for (int r = 0; r < n; ++r) {

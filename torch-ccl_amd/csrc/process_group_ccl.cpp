@@ -601,6 +601,7 @@ void ProcessGroupCCL::ensureInit(int device) {
     for (int b = a + 1; b < size_; ++b)
       if (ctl_->slot[a].pid == ctl_->slot[b].pid) distinct = false;
   device_sync_ = size_ > 1 && distinct && want_device_sync_;
+  distinct_pids_ = size_ > 1 && distinct;
   if (device_sync_ && rank_ == 0) {
     // A kernel that waits for other ranks only makes progress while the hardware queues of all rank
     // processes are mapped at once.  A process owns up to GPU_MAX_HW_QUEUES of them (4 unless set),
@@ -963,6 +964,51 @@ void ProcessGroupCCL::runHostSynced(Plan& plan, hipStream_t s, int slot) {
   auto us_since = [](clk::time_point t) { return std::chrono::duration<double, std::micro>(clk::now() - t).count(); };
   const bool timed = profile_ && plan.stage_bytes > 0 && phase_us_[0].size() < (1u << 20);
   auto t0 = clk::now();
+  // In place (rank processes only): an allreduce whose tensors all ranks can share needs no staging
+  // at all -- every rank reduces its shard of all tensors and writes it into all of them -- and the
+  // two host barriers the staged two-shot form needs anyway order it: tensors complete / everybody
+  // done.  The kernel is the one-launch kernel of the device-synchronised mode with its waits off.
+  const bool candidate = distinct_pids_ && zero_copy_ && plan.share && plan.exec_sync && plan.exec_sync_in_place_only &&
+                         size_ <= MCCL_FUSED_MAX_RANKS;
+  if (candidate) {
+    bool in_place = true;
+    try {
+      RankSlot::Published& rec = me.pub[pub];
+      uint64_t off = 0;
+      const int entry = exportRange(plan.share_ptr, plan.share_bytes, &off);
+      rec.share_entry = entry;
+      rec.share_off = off;
+      rec.share_gen = (entry >= 0 && entry < kMaxExports) ? me.exports[entry].gen.load(std::memory_order_acquire) : 0;
+      if (tail_pending_ && tail_stream_ != s) HIP_CHECK(hipStreamSynchronize(tail_stream_));
+      HIP_CHECK(hipStreamSynchronize(s));
+    } catch (...) {
+      me.failed.store(1, std::memory_order_release);
+      throw;
+    }
+    hostBarrier();  // every rank's tensor is complete and its offer published
+    for (int r = 0; r < size_; ++r)
+      if (ctl_->slot[r].pub[pub].share_entry < 0) in_place = false;
+    if (in_place) {
+      try {
+        PeerView pv;
+        pv.zero_copy = true;
+        pv.user.resize((size_t)size_);
+        for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
+        mccl_xsync_t sync{};
+        sync.n = size_;
+        sync.rank = rank_;  // ready_epoch 0: no waits inside the kernel
+        TORCH_CHECK(plan.exec_sync(pv, sync, s), "ccl backend: the in-place plan declined");
+        HIP_CHECK(hipStreamSynchronize(s));
+      } catch (...) {
+        me.failed.store(1, std::memory_order_release);
+        throw;
+      }
+      hostBarrier();  // every rank has written its shard everywhere
+      if (timed) phase_us_[3].push_back((float)us_since(t0));
+      return;
+    }
+    // somebody cannot share: the staged form below (every rank sees the same offers)
+  }
   try {
     void* stage = ensureStage(slot, plan.stage_bytes);
     publishStage(slot, pub);

@@ -332,6 +332,7 @@ class ProcessGroupCCL : public c10d::Backend {
   // size.  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides (and then binds the allreduce, too).
   size_t one_launch_max_ = 128u << 20;
   bool one_launch_max_forced_ = false;
+  bool distinct_pids_ = false;          // every rank is a process of its own
   const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
   const char* last_path_ = "";
   uint64_t last_seq_ = 0;
