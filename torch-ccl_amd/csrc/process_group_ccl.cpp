@@ -285,6 +285,10 @@ ProcessGroupCCL::WorkCCL::~WorkCCL() {
 }
 
 bool ProcessGroupCCL::WorkCCL::isCompleted() {
+  if (pending_polls_ != 0) {
+    if (pending_polls_ > 0) --pending_polls_;
+    return false;
+  }
   if (end_) return hipEventQuery(end_) == hipSuccess;
   if (!stream_set_) return true;
   // No event was recorded for this collective (it ran on the caller's stream; with several
@@ -350,6 +354,14 @@ void ProcessGroupCCL::WorkCCL::waitInternal(std::chrono::milliseconds timeout) {
 }
 
 void ProcessGroupCCL::WorkCCL::synchronize() { waitInternal(kNoTimeout); }
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::pendingWork(int rank, int polls, std::chrono::milliseconds op_timeout) {
+  auto work = c10::make_intrusive<WorkCCL>(rank, c10d::OpType::UNKNOWN, "pending", std::vector<at::Tensor>{},
+                                           std::vector<at::Tensor>{}, /*blocking_wait=*/true);
+  work->pending_polls_ = polls;
+  work->op_timeout_ = op_timeout;
+  return work;
+}
 
 bool ProcessGroupCCL::WorkCCL::wait(std::chrono::milliseconds timeout) {
   waitInternal(timeout);

@@ -104,10 +104,15 @@ class ProcessGroupCCL : public c10d::Backend {
     std::chrono::steady_clock::time_point start_;
     int device_ = 0;
     bool blocking_wait_ = false;
+    int pending_polls_ = 0;  // > 0: isCompleted() says "not yet" this many more times, < 0: for good (pendingWork)
     std::vector<at::Tensor> inputs_;   // held until the Work dies (ownership rule of the reference)
     std::vector<at::Tensor> outputs_;
     c10::intrusive_ptr<c10::ivalue::Future> future_;
   };
+
+  // A Work that is not backed by device work: it completes after `polls` calls of isCompleted()
+  // (never, when polls < 0).  For exercising wait(timeout) without a GPU.
+  static c10::intrusive_ptr<c10d::Work> pendingWork(int rank, int polls, std::chrono::milliseconds op_timeout);
 
   // What a posted receive still has to do; the group keeps these per source in posting order.
   struct RecvState {

@@ -61,6 +61,9 @@ PYBIND11_MODULE(_C, m) {
     register_backend(name, creator, false, std::vector<std::string>{"cuda"});
   });
 
+  // a Work without device work behind it, for tests of wait(timeout) that need no GPU
+  m.def("_pending_work", &ProcessGroupCCL::pendingWork, py::arg("rank"), py::arg("polls"), py::arg("op_timeout"));
+
   py::class_<ProcessGroupCCL, ReleaseGilHolder<ProcessGroupCCL>>(m, "ProcessGroupCCL", backend_base)
       .def(py::init([](const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
                        std::chrono::milliseconds timeout) {
