@@ -126,6 +126,15 @@ def test_host_synchronised_fallback(monkeypatch, world, mode):
     _spawn(world, mode)
 
 
+@pytest.mark.parametrize("world,mode", [(4, "oracle"), (8, "zero_copy"), (8, "baseline_configs"), (2, "reference")])
+def test_waits_in_barrier_kernels_only(monkeypatch, world, mode):
+    """MCCL_PG_SYNC=barrier: the ranks still wait for each other on the device, but only in
+    one-wavefront barrier kernels around the data kernels, never inside one (no kernel keeps
+    hundreds of wavefronts resident while it waits): same bits."""
+    monkeypatch.setenv("MCCL_PG_SYNC", "barrier")
+    _spawn(world, mode)
+
+
 def test_zero_copy_with_barrier_kernels_instead_of_one_launch(monkeypatch):
     """MCCL_PG_ONE_LAUNCH_MAX_BYTES=0: the peers' tensors are still read in place, but between
     barrier kernels by the bandwidth-tuned kernels (what groups of more than eight ranks and very

@@ -777,8 +777,11 @@ namespace {
 
 // Workgroups (single wavefronts) of a launch that waits for its peers inside the kernel: all
 // ranks' launches must be resident at once, so each gets its share of a fixed budget.
-unsigned xrank_grid(uint64_t tiles, int n) {
-  uint64_t cap = (uint64_t)g_tune[MCCL_TUNE_XRANK_WAVES_ALL_RANKS] / (uint64_t)n;
+// A launch that waits for its peers gets its share of the wavefronts all ranks may hold together;
+// one that does not wait (the caller has ordered the ranks) can never keep a peer's launch out and
+// takes the whole budget.
+unsigned xrank_grid(uint64_t tiles, int n, bool waits = true) {
+  uint64_t cap = (uint64_t)g_tune[MCCL_TUNE_XRANK_WAVES_ALL_RANKS] / (uint64_t)(waits ? n : 1);
   if (cap < 1) cap = 1;
   if (tiles < 1) tiles = 1;
   return (unsigned)(tiles < cap ? tiles : cap);
@@ -858,7 +861,7 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
     const CopySeg& cs = a.copy.seg[k];
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
   }
-  const unsigned grid = xrank_grid(chunks, a.sync.n);
+  const unsigned grid = xrank_grid(chunks, a.sync.n, a.sync.ready_epoch != 0);
   hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
@@ -895,7 +898,7 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
   for (int k = 0; k < a.sync.n; ++k)
     if (count && ((uintptr_t)in[k] & 7u)) a.aligned_in = 0;
   if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n), 0u, (hipStream_t)stream);
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n, a.sync.ready_epoch != 0), 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
@@ -937,7 +940,7 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   a.tail1 = (uint32_t)(n_me % ve);
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
   if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n), 0u, (hipStream_t)stream);
+  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n, a.sync.ready_epoch != 0), 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }

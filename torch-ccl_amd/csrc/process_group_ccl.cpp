@@ -425,7 +425,10 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   blocking_wait_ = envFlag("CCL_BLOCKING_WAIT", false);
   verbose_ = envFlag("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", false);
   profile_ = envFlag("MCCL_PG_PROFILE", false);
-  if (const char* v = std::getenv("MCCL_PG_SYNC")) want_device_sync_ = std::string(v) != "host";
+  if (const char* v = std::getenv("MCCL_PG_SYNC")) {
+    want_device_sync_ = std::string(v) != "host";
+    waits_in_data_kernels_ = std::string(v) != "barrier";
+  }
   zero_copy_ = envFlag("MCCL_PG_ZERO_COPY", true);
   comm_stream_for_large_ = envFlag("MCCL_PG_COMM_STREAM", false);
   if (const char* v = std::getenv("MCCL_PG_ONE_LAUNCH_MAX_BYTES")) {
@@ -626,7 +629,8 @@ void ProcessGroupCCL::ensureInit(int device) {
       TORCH_WARN_ONCE("ccl backend: ", size_, " rank processes share one GPU and wait for each other on the device; if the "
                       "ranks use more than two streams each, set GPU_MAX_HW_QUEUES=2 (or 1) in their environment, or "
                       "MCCL_PG_SYNC=host: with more hardware queues than the GPU maps at once a collective costs a "
-                      "scheduling quantum (about 10 ms)");
+                      "scheduling quantum (about 10 ms).  If the ranks run register-heavy kernels of their own between "
+                      "collectives, MCCL_PG_SYNC=barrier keeps the waiting kernels out of their way");
   }
   if (size_ > 1) {
     peer_arena_.assign((size_t)size_, nullptr);
@@ -1101,7 +1105,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     last_title_ = plan.title;
     last_seq_ = seq + 1;
     last_path_ = "one launch, fused";
-    if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS) {
+    if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS && waits_in_data_kernels_) {
       const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
       MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
                                       fused_stage_[slot].data(), fused_flags_[slot].data(), size_, rank_,
@@ -1159,7 +1163,8 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     // copy-in (two launches instead of three): the launch says "my staging buffer is complete",
     // and no closing wait is needed, as for every staged collective (see the slot rule above).
     const size_t moved = zero_copy ? plan.share_bytes : plan.stage_bytes;
-    const bool one_launch = plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS && (zero_copy || !plan.exec_sync_in_place_only) &&
+    const bool one_launch = waits_in_data_kernels_ && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
+                            (zero_copy || !plan.exec_sync_in_place_only) &&
                             ((zero_copy && plan.one_launch_any_size && !one_launch_max_forced_) || moved <= one_launch_max_);
     last_path_ = one_launch ? (zero_copy ? "one launch, peers read in place" : "copy-in and one launch")
                             : zero_copy ? "barrier kernels, peers read in place"
@@ -1189,6 +1194,17 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
     deviceBarrier(epoch + 1, s);  // every rank's input is complete (staged, or ready in place)
     if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
+    if (zero_copy && plan.exec_sync && plan.exec_sync_in_place_only && size_ <= MCCL_FUSED_MAX_RANKS) {
+      // the in-place allreduce between barrier kernels: its own waits are off (ready_epoch 0)
+      mccl_xsync_t sync{};
+      sync.n = size_;
+      sync.rank = rank_;
+      if (plan.exec_sync(pv, sync, s)) {
+        deviceBarrier(epoch + 3, s);  // nobody reads its tensor before every rank has written its shard everywhere
+        if (timed) phase_us_[3].push_back((float)us_since(t0));
+        return;
+      }
+    }
     if (plan.exec) plan.exec(pv, s);
     if (plan.exec2 && (!plan.two_phase || plan.two_phase(pv))) {
       deviceBarrier(epoch + 2, s);
