@@ -213,9 +213,12 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
  *   words[r]: rank r's 64-bit word as for mccl_rank_barrier (the same word may serve both; epochs
  * grow: ready_epoch of a call > any epoch used before, done_epoch > ready_epoch).  done_counter:
  * MCCL_SYNC_COUNTER_BYTES of this rank's device memory, 64-byte aligned, zero before the first call
- * (the kernel leaves them zero): the workgroups count themselves out there.  ready_epoch == 0 (then
- * done_epoch must be 0 as well; words, counters and status are not used): the kernel does not wait
- * at all, for callers that order the ranks themselves, e.g. with host barriers around the launch.
+ * (the kernel leaves them zero): the workgroups count themselves out there.  ready_epoch == 0: no
+ * opening wait, for callers that have ordered the start of the ranks themselves -- with an
+ * mccl_rank_barrier launch in front (then only the kernel's last workgroup ever waits, for the
+ * closing epoch: one wavefront per rank instead of the whole grid, which matters when several
+ * ranks share a GPU with other kernels), or with host barriers around the launch (done_epoch 0 as
+ * well: the kernel does not wait at all; words, counters and status are then not used).
  * Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
  * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
  */

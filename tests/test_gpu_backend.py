@@ -86,24 +86,20 @@ def test_world_size_one_is_a_no_op():
         assert torch.equal(out.cpu(), t.cpu())
 
 
-def test_missing_rank_raises_instead_of_hanging(monkeypatch):
-    """Failure handling forced from the host: a rank skips a collective; the host barrier of the
-    others gives up after the (shortened) limit and raises.  No kernel waits on the GPU."""
+@pytest.mark.parametrize("sync", ["host", "barrier"])
+def test_missing_rank_raises_instead_of_hanging(monkeypatch, sync):
+    """Failure handling forced from the host: a rank skips a collective; the others give up after
+    the (shortened) limit and raise -- at the rendezvous of the host threads, which small collectives
+    have in both modes, before any kernel waits on the GPU."""
     monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
-    monkeypatch.setenv("MCCL_PG_SYNC", "host")
+    monkeypatch.setenv("MCCL_PG_SYNC", sync)
     _spawn(3, "missing")
 
 
-@pytest.mark.parametrize("blocking", ["0", "1"])
-def test_missing_rank_with_device_side_waits(monkeypatch, blocking):
-    """The same failure with the cross-rank wait on the device: the kernel's own bounded wait ends
-    it (a 1.5 s limit forced from the host), the Work reports failure, the group refuses to go on."""
-    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
-    monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
-    _spawn(3, "missing_device")
-
-
 def test_wait_honours_its_timeout(monkeypatch):
+    """(with the waits inside the data kernels: the 1 MiB allreduce of that mode has no rendezvous of
+    the host threads, so the call returns while a peer is still missing and the Work has to wait)"""
+    monkeypatch.setenv("MCCL_PG_SYNC", "kernel")
     monkeypatch.setenv("CCL_BLOCKING_WAIT", "1")
     _spawn(3, "late_peer")
 
@@ -117,8 +113,7 @@ def test_baseline_configs_at_full_size_through_the_backend():
     _spawn(8, "baseline_configs")
 
 
-@pytest.mark.parametrize("world,mode", [(2, "reference"), (4, "oracle"), (3, "p2p"), (4, "dist"), (2, "zero_copy"), (8, "zero_copy"),
-                                        (8, "baseline_configs")])
+@pytest.mark.parametrize("world,mode", [(2, "reference"), (4, "oracle"), (3, "p2p"), (4, "dist"), (2, "zero_copy"), (8, "baseline_configs")])
 def test_host_synchronised_fallback(monkeypatch, world, mode):
     """MCCL_PG_SYNC=host: the same cases with hipStreamSynchronize + the host barrier instead of
     device-side waits (what ranks that share a process always use)."""
@@ -126,13 +121,25 @@ def test_host_synchronised_fallback(monkeypatch, world, mode):
     _spawn(world, mode)
 
 
-@pytest.mark.parametrize("world,mode", [(4, "oracle"), (8, "zero_copy"), (8, "baseline_configs"), (2, "reference")])
-def test_waits_in_barrier_kernels_only(monkeypatch, world, mode):
-    """MCCL_PG_SYNC=barrier: the ranks still wait for each other on the device, but only in
-    one-wavefront barrier kernels around the data kernels, never inside one (no kernel keeps
-    hundreds of wavefronts resident while it waits): same bits."""
-    monkeypatch.setenv("MCCL_PG_SYNC", "barrier")
+@pytest.mark.parametrize("world,mode", [(4, "oracle"), (8, "oracle"), (8, "zero_copy"), (8, "baseline_configs"), (2, "reference"),
+                                        (4, "dist"), (8, "replay")])
+def test_waits_inside_the_data_kernels(monkeypatch, world, mode):
+    """MCCL_PG_SYNC=kernel: one launch per collective, whose workgroups wait for the other ranks
+    themselves (the small fused allreduce, the in-place allreduce, the one-launch pulls and shard
+    reductions) instead of a barrier kernel in front of the data kernel: same bits."""
+    monkeypatch.setenv("MCCL_PG_SYNC", "kernel")
     _spawn(world, mode)
+
+
+@pytest.mark.parametrize("blocking", ["0", "1"])
+def test_missing_rank_with_waits_inside_the_data_kernels(monkeypatch, blocking):
+    """The same failure with the cross-rank wait on the device (the small allreduce of this mode has no
+    rendezvous of the host threads): the kernel's own bounded wait ends it (a 1.5 s limit forced from
+    the host), the Work reports failure, the group refuses to go on."""
+    monkeypatch.setenv("MCCL_PG_SYNC", "kernel")
+    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
+    _spawn(3, "missing_device")
 
 
 def test_zero_copy_with_barrier_kernels_instead_of_one_launch(monkeypatch):

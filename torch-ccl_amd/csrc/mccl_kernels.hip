@@ -794,10 +794,9 @@ int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
   memset(x, 0, sizeof(*x));
   x->n = sy->n;
   x->rank = sy->rank;
-  if (sy->ready_epoch == 0) {  // the caller orders the ranks itself: no wait inside the kernel
-    if (sy->done_epoch != 0) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs an opening one (ready_epoch)");
-    return MCCL_OK;
-  }
+  // ready_epoch 0: the caller has ordered the start of the ranks itself (a barrier kernel in front,
+  // host barriers): no opening wait; done_epoch 0: no closing wait
+  if (sy->ready_epoch == 0 && sy->done_epoch == 0) return MCCL_OK;
   if (!sy->words) return fail(MCCL_ERR_INVALID_ARG, "sync word table is null");
   if (sy->done_epoch != 0 && sy->done_epoch <= sy->ready_epoch) return fail(MCCL_ERR_INVALID_ARG, "done_epoch must be 0 or above ready_epoch");
   if (sy->done_epoch != 0 && !sy->done_counter) return fail(MCCL_ERR_INVALID_ARG, "a closing wait needs a done counter");
@@ -918,7 +917,7 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   if (rc != MCCL_OK) return rc;
   if (!tensors) return fail(MCCL_ERR_INVALID_ARG, "tensor table is null");
   if (a.sync.ready_epoch != 0 && a.sync.done_epoch == 0)
-    return fail(MCCL_ERR_INVALID_ARG, "the in-place allreduce needs a closing wait (done_epoch) when it waits at all");
+    return fail(MCCL_ERR_INVALID_ARG, "the in-place allreduce needs a closing wait (done_epoch) when it has an opening one");
   const int n = a.sync.n, me = a.sync.rank;
   const size_t es = dtype_size(dtype);
   for (int r = 0; r < n; ++r) {

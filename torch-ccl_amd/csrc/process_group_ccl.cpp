@@ -427,7 +427,7 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   profile_ = envFlag("MCCL_PG_PROFILE", false);
   if (const char* v = std::getenv("MCCL_PG_SYNC")) {
     want_device_sync_ = std::string(v) != "host";
-    waits_in_data_kernels_ = std::string(v) != "barrier";
+    waits_in_data_kernels_ = std::string(v) == "kernel";
   }
   zero_copy_ = envFlag("MCCL_PG_ZERO_COPY", true);
   comm_stream_for_large_ = envFlag("MCCL_PG_COMM_STREAM", false);
@@ -1167,7 +1167,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
                             (zero_copy || !plan.exec_sync_in_place_only) &&
                             ((zero_copy && plan.one_launch_any_size && !one_launch_max_forced_) || moved <= one_launch_max_);
     last_path_ = one_launch ? (zero_copy ? "one launch, peers read in place" : "copy-in and one launch")
-                            : zero_copy ? "barrier kernels, peers read in place"
+                            : zero_copy ? "barrier kernel, peers read in place"
                                         : candidate ? "staged: a rank cannot share its tensor" : "staged";
     if (verbose_) {
       std::ostringstream os;
@@ -1194,13 +1194,21 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
     deviceBarrier(epoch + 1, s);  // every rank's input is complete (staged, or ready in place)
     if (timed) { phase_us_[2].push_back((float)us_since(t0)); t0 = clk::now(); }
-    if (zero_copy && plan.exec_sync && plan.exec_sync_in_place_only && size_ <= MCCL_FUSED_MAX_RANKS) {
-      // the in-place allreduce between barrier kernels: its own waits are off (ready_epoch 0)
+    if (zero_copy && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
+        (plan.exec_sync_in_place_only || plan.share_bytes <= one_launch_max_)) {
+      // Peers' tensors in place behind a barrier kernel: the data kernel starts without a wait
+      // (ready_epoch 0) and only its last workgroup waits, for the closing epoch -- nobody may touch
+      // its tensor before every peer has read (allreduce: written) it.  Two launches, and never
+      // more than one waiting wavefront per rank on the GPU.
       mccl_xsync_t sync{};
+      sync.words = bar_flags_.data();
       sync.n = size_;
       sync.rank = rank_;
+      sync.done_epoch = epoch + 3;
+      sync.done_counter = done_counter_;
+      sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
+      sync.status = status_dev_;
       if (plan.exec_sync(pv, sync, s)) {
-        deviceBarrier(epoch + 3, s);  // nobody reads its tensor before every rank has written its shard everywhere
         if (timed) phase_us_[3].push_back((float)us_since(t0));
         return;
       }
@@ -1400,7 +1408,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // reduces shard r of all tensors into its staging buffer (nobody writes a tensor while
       // anybody reads one), then all ranks gather the W finished shards into their tensors:
       // about 3 S bytes per rank and no copy-in, against (4 + 1/W) S for the staged two-shot.
-      p.share = !p.fused_ok && len * es >= kZeroCopyMinBytes;
+      // (without the one-launch small allreduce, in place beats staging from 64 KiB on: two launches against three)
+      p.share = waits_in_data_kernels_ ? (!p.fused_ok && len * es >= kZeroCopyMinBytes) : len * es >= (64u << 10);
       p.share_ptr = base;
       p.share_bytes = len * es;
       p.zero_copy_stage_bytes = shard * es;

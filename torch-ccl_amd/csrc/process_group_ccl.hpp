@@ -328,14 +328,15 @@ class ProcessGroupCCL : public c10d::Backend {
   bool verbose_ = false;        // ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE
   bool profile_ = false;        // MCCL_PG_PROFILE: host-side phase timers, printed when the group dies
   bool want_device_sync_ = true;  // MCCL_PG_SYNC != "host"
-  // MCCL_PG_SYNC=barrier: device-side waits in one-wavefront barrier kernels only, never inside a
-  // data kernel.  The kernels that wait themselves keep up to 512 wavefronts per rank resident
-  // while they wait; with 7 of 8 rank processes waiting on one GPU that is 3 to 4 wavefronts of
-  // 120 registers on every SIMD, and a kernel the late rank still has to run before it can join
-  // (say a GEMM with 128 or more registers per lane) may find no room to start: the waits then
-  // end at their time limit.  Barrier kernels keep one wavefront per rank waiting instead, at
-  // one more launch (two for an allreduce) per collective.  One rank per GPU has no such problem.
-  bool waits_in_data_kernels_ = true;
+  // MCCL_PG_SYNC=kernel: a collective is ONE launch whose workgroups wait for the other ranks
+  // themselves.  Fastest, but such a kernel keeps up to 512 wavefronts per rank resident while it
+  // waits; with 7 of 8 rank processes waiting on one GPU that is 3 to 4 wavefronts of 120 registers
+  // on every SIMD, and a kernel the late rank still has to run before it can join (a GEMM with
+  // 128 or more registers per lane: measured with torch.mm) finds no room to start: the waits
+  // end at their time limit.  One rank per GPU has no such problem.  The default therefore waits
+  // in a one-wavefront barrier kernel in front of the data kernel, whose last workgroup alone
+  // waits for the closing epoch: two launches per collective, one waiting wavefront per rank.
+  bool waits_in_data_kernels_ = false;
   bool zero_copy_ = true;         // MCCL_PG_ZERO_COPY != 0
   // Largest tensor (bytes per rank) whose zero-copy collective is ONE launch with the rank waits
   // inside the kernel; larger ones run the bandwidth-tuned kernels between barrier kernels.  With 8
