@@ -133,7 +133,7 @@ def _gloo_rank(rank, world, store_path, backend, cases, out_path):
     dist.destroy_process_group()
 
 
-def _backend_rank(rank, world, store_path, cases, out_path):
+def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     """One rank process of the drop-in path: dist.all_reduce through backend "ccl" on cuda:0."""
     os.dup2(2, 1)
     sys.path.insert(0, os.path.join(ROOT, "torch-ccl_amd"))
@@ -194,6 +194,13 @@ def _backend_rank(rank, world, store_path, cases, out_path):
     ts.sort()
     res["one_trivial_kernel_plus_synchronize"] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": 200}
 
+    if not large:
+        if rank == 0:
+            with open(out_path, "w") as f:
+                json.dump(res, f)
+        dist.destroy_process_group()
+        return
+
     def timed(fn, iters=8, warm=2):
         for _ in range(warm):
             fn()
@@ -231,22 +238,39 @@ def _backend_rank(rank, world, store_path, cases, out_path):
     dist.destroy_process_group()
 
 
-def backend_path(world=8):
+def backend_path(world=8, sync=None):
     """The drop-in c10d path end to end: `world` rank processes share cuda:0 and call dist.* on GPU
-    tensors, timed on the host around the call plus a synchronize."""
+    tensors, timed on the host around the call plus a synchronize.  sync: value of MCCL_PG_SYNC for
+    the rank processes (None = the backend's default); with a value only C2 and C3 are timed."""
     import tempfile
     import torch.multiprocessing as mp
     cases = [("c2_256KiB_bf16", 16 * 8192, 20, 200), ("c3_64MiB_bf16", 4096 * 8192, 3, 20)]
-    with tempfile.TemporaryDirectory() as d:
-        out_path = os.path.join(d, "res.json")
-        mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path), nprocs=world, join=True)
-        with open(out_path) as f:
-            res = json.load(f)
+    before = os.environ.get("MCCL_PG_SYNC")
+    if sync is not None:
+        os.environ["MCCL_PG_SYNC"] = sync  # the spawned rank processes inherit it
+    try:
+        with tempfile.TemporaryDirectory() as d:
+            out_path = os.path.join(d, "res.json")
+            mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path, sync is None), nprocs=world, join=True)
+            with open(out_path) as f:
+                res = json.load(f)
+    finally:
+        if sync is not None:
+            if before is None:
+                del os.environ["MCCL_PG_SYNC"]
+            else:
+                os.environ["MCCL_PG_SYNC"] = before
+    if sync is not None:
+        return {name: {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()} for name in res}
     out = {"processes": world, "note": "host-timed dist.* call + synchronize per rank process; all ranks share the one "
-                                       "GPU.  Cross-rank waits run on the device (flag kernels, or inside the data "
-                                       "kernel), large tensors are read by the peers in place; every launch of a "
-                                       "process waits for its turn at the dispatcher, which is what "
-                                       "one_trivial_kernel_plus_synchronize measures"}
+                                       "GPU.  The ranks wait for each other on the device: in a one-wavefront barrier "
+                                       "kernel in front of the data kernel, whose last workgroup waits for the closing "
+                                       "epoch (two launches per collective); tensors from 64 KiB on are read by the "
+                                       "peers in place.  Every launch of a process waits for its turn at the dispatcher, "
+                                       "which is what one_trivial_kernel_plus_synchronize measures.  "
+                                       "waits_inside_the_data_kernel: the same with MCCL_PG_SYNC=kernel (one launch per "
+                                       "collective; not the default because the waiting grids of 7 ranks can keep a "
+                                       "register-heavy kernel of the 8th from starting)"}
     for name in res:
         out[name] = {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()}
     return out
@@ -316,6 +340,7 @@ def main():
     if "backend" in extras:
         try:
             backend_result = backend_path(8)
+            backend_result["waits_inside_the_data_kernel"] = backend_path(8, sync="kernel")
             log("c10d backend:", json.dumps(backend_result))
         except Exception as e:  # informational: never fails the benchmark
             backend_result = {"error": repr(e)[:300]}

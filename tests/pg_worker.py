@@ -727,6 +727,38 @@ def baseline_config_cases(pg, rank, world):
     pg.barrier().wait()
 
 
+def heavy_predecessor_case(rank, world):
+    """A late rank with register-heavy kernels of its own (GEMMs) queued in front of its collective,
+    while all other ranks are already waiting on the device: the waiting kernels must leave room
+    for the GEMMs to start, or the group would wait for a rank that cannot get there."""
+    import time
+    a = torch.randn(4096, 4096, dtype=torch.bfloat16, device=DEV)
+    b = torch.randn(4096, 4096, dtype=torch.bfloat16, device=DEV)
+    c = torch.mm(a, b)  # warm the GEMM up
+    t = torch.full((8 << 20,), 1.0, dtype=torch.bfloat16, device=DEV)
+    dist.all_reduce(t)
+    torch.cuda.synchronize()
+    for it in range(3):
+        t.fill_(float(rank + it))
+        dist.barrier()
+        if rank == (it % world):
+            time.sleep(0.003)  # the others have launched and wait on the device
+            for _ in range(20):
+                c = torch.mm(a, b)
+        dist.all_reduce(t)
+        torch.cuda.synchronize()
+        want = float(sum(r + it for r in range(world)))
+        assert float(t[0]) == want and float(t[-1]) == want, (it, float(t[0]), want)
+    out = torch.empty(world * 1024, dtype=torch.float32, device=DEV)
+    if rank == 1:
+        for _ in range(20):
+            c = torch.mm(a, b)
+    dist.all_gather_into_tensor(out, torch.full((1024,), float(rank), device=DEV))
+    torch.cuda.synchronize()
+    assert out.view(world, 1024)[:, 0].tolist() == [float(r) for r in range(world)]
+    del c
+
+
 def missing_rank_device_case(pg, rank, world):
     """Device-side waits: rank 1 never joins the second collective.  The survivors' kernel gives up
     by itself at the (shortened) limit and names the late rank; their Work reports the failure
@@ -1007,12 +1039,12 @@ def run_rank(rank, world, store_path, mode):
         finally:
             dist.destroy_process_group()
         return
-    if mode in ("subgroup", "replay", "reference_p2p", "coalesced_windows"):
+    if mode in ("subgroup", "replay", "reference_p2p", "coalesced_windows", "heavy_predecessor"):
         store = dist.FileStore(store_path, world)
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
             {"subgroup": subgroup_case, "replay": identity_replay_case, "reference_p2p": reference_p2p_cases,
-             "coalesced_windows": coalesced_window_cases}[mode](rank, world)
+             "coalesced_windows": coalesced_window_cases, "heavy_predecessor": heavy_predecessor_case}[mode](rank, world)
         finally:
             dist.destroy_process_group()
         return

@@ -109,6 +109,10 @@ def test_zero_copy_collectives(world):
     _spawn(world, "zero_copy")
 
 
+def test_a_late_rank_with_gemms_of_its_own_still_gets_in():
+    _spawn(8, "heavy_predecessor")
+
+
 def test_baseline_configs_at_full_size_through_the_backend():
     _spawn(8, "baseline_configs")
 

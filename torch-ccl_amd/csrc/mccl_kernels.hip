@@ -860,7 +860,7 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
     const CopySeg& cs = a.copy.seg[k];
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
   }
-  const unsigned grid = xrank_grid(chunks, a.sync.n, a.sync.ready_epoch != 0);
+  const unsigned grid = xrank_grid(chunks, a.sync.n);  // (a copy gains nothing from more wavefronts than its share, waits or not)
   hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
