@@ -629,8 +629,7 @@ void ProcessGroupCCL::ensureInit(int device) {
       TORCH_WARN_ONCE("ccl backend: ", size_, " rank processes share one GPU and wait for each other on the device; if the "
                       "ranks use more than two streams each, set GPU_MAX_HW_QUEUES=2 (or 1) in their environment, or "
                       "MCCL_PG_SYNC=host: with more hardware queues than the GPU maps at once a collective costs a "
-                      "scheduling quantum (about 10 ms).  If the ranks run register-heavy kernels of their own between "
-                      "collectives, MCCL_PG_SYNC=barrier keeps the waiting kernels out of their way");
+                      "scheduling quantum (about 10 ms)");
   }
   if (size_ > 1) {
     peer_arena_.assign((size_t)size_, nullptr);
