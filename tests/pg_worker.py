@@ -1029,6 +1029,9 @@ def subgroup_case(rank, world):
 
 
 def run_rank(rank, world, store_path, mode):
+    # the expected values are computed on the host by every rank: share the cores instead of
+    # letting every rank process start a thread per core
+    torch.set_num_threads(max(1, (os.cpu_count() or 16) // world))
     torch.cuda.set_device(0)
     import torch_ccl_amd  # noqa: F401  registers the backend
     if mode == "dist":

@@ -267,6 +267,7 @@ def timeout_case(rank, world, queues, barrier):
 
 
 def run_rank(rank, world, queues, barrier, mode):
+    torch.set_num_threads(max(1, (os.cpu_count() or 16) // world))  # the ranks share the host's cores
     torch.cuda.set_device(0)
     {"barrier": barrier_case, "fused": fused_case, "timeout": timeout_case, "xrank": xrank_case}[mode](rank, world, queues, barrier)
     torch.cuda.synchronize()

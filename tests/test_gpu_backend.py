@@ -104,7 +104,7 @@ def test_wait_honours_its_timeout(monkeypatch):
     _spawn(3, "late_peer")
 
 
-@pytest.mark.parametrize("world", [2, 8])
+@pytest.mark.parametrize("world", [2, 8, 10])
 def test_zero_copy_collectives(world):
     _spawn(world, "zero_copy")
 
