@@ -193,7 +193,10 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
  * after every peer has started a later collective (two alternating sets do).  Same arithmetic and
  * bits as mccl_reduce_n over the n contributions.  At most MCCL_FUSED_MAX_RANKS ranks.  The wait
  * is bounded and reported like mccl_rank_barrier's; a tile whose peers did not arrive in time is
- * left unwritten.
+ * left unwritten.  The launch is one workgroup per 16 KiB of message, and a workgroup sits on one
+ * compute unit: while it waits for a late rank it holds count * size / 16 KiB of the GPU's 256
+ * compute units, which is how a caller whose ranks share a GPU bounds what the waiting ranks keep
+ * from the late one's other kernels.
  */
 #define MCCL_FUSED_MAX_RANKS 8
 #define MCCL_FUSED_TILE_BYTES 1024
@@ -238,8 +241,15 @@ typedef struct {
  * (ccl::allgatherv, ccl::alltoallv, src/gpu/dpcpp_ccl.cpp:1176-1182, 1428-1455) in one launch.
  * At most 64 segments; zero segments still take part in the waits.  flags: MCCL_COPY_SHARED_SOURCES
  * when the other ranks read the same source bytes in the same collective (allgather, broadcast):
- * the sources are then kept in the memory-side cache instead of being streamed past it. */
+ * the sources are then kept in the memory-side cache instead of being streamed past it.
+ * MCCL_COPY_PUBLISH turns the direction round: the sources are this rank's own memory and the
+ * destinations are buffers that the peers read next (staging buffers; the copy-in of the staged
+ * collectives, src/gpu/allreduce_small.h:165-287, with its announcement in the same launch): every
+ * byte is written through to memory before the closing epoch is published, so a peer that has seen
+ * done_epoch -- its own launch of the same call has then returned -- may read them with its next
+ * kernel.  done_epoch must not be 0; ready_epoch usually is. */
 #define MCCL_COPY_SHARED_SOURCES 1u
+#define MCCL_COPY_PUBLISH 2u
 int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync,
                             void* stream);
 

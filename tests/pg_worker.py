@@ -523,8 +523,10 @@ def large_message_case(pg, rank, world):
 
 
 def missing_rank_case(pg, rank, world):
-    """Rank 1 never joins the second collective: the others must get an error, not hang."""
-    t = torch.ones(16, device=DEV)
+    """Rank 1 never joins the second collective: the others must get an error, not hang.  (2 MiB:
+    a size whose allreduce has the host threads meet first in every mode -- to agree on reading the
+    tensors in place, or around the launches -- so the call itself raises.)"""
+    t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
@@ -749,6 +751,19 @@ def heavy_predecessor_case(rank, world):
         torch.cuda.synchronize()
         want = float(sum(r + it for r in range(world)))
         assert float(t[0]) == want and float(t[-1]) == want, (it, float(t[0]), want)
+    # the same with small messages, whose single launch waits itself (its workgroups are few enough
+    # to leave compute units free); 1 MiB: copy-in whose last workgroup waits, then the reduction
+    for it, elems in enumerate((1 << 17, 1 << 19, 8)):
+        small = torch.full((elems,), float(rank + it), dtype=torch.bfloat16, device=DEV)
+        dist.barrier()
+        if rank == ((it + 3) % world):
+            time.sleep(0.003)
+            for _ in range(20):
+                c = torch.mm(a, b)
+        dist.all_reduce(small)
+        torch.cuda.synchronize()
+        want = float(sum(r + it for r in range(world)))
+        assert float(small[0]) == want and float(small[-1]) == want, (elems, float(small[0]), want)
     out = torch.empty(world * 1024, dtype=torch.float32, device=DEV)
     if rank == 1:
         for _ in range(20):
@@ -762,11 +777,15 @@ def heavy_predecessor_case(rank, world):
 def missing_rank_device_case(pg, rank, world):
     """Device-side waits: rank 1 never joins the second collective.  The survivors' kernel gives up
     by itself at the (shortened) limit and names the late rank; their Work reports the failure
-    instead of success, the tensor is left alone, and the group refuses further collectives."""
-    t = torch.ones(16, device=DEV)
+    instead of success, the group refuses further collectives, and (one-launch form) the tensor is
+    left alone.  MCCL_TEST_ELEMS floats: 16 is one launch in every mode, 2^18 (1 MiB) is an
+    announcing copy-in and a reduction unless MCCL_PG_SYNC=kernel makes it one launch too."""
+    elems = int(os.environ.get("MCCL_TEST_ELEMS", "16"))
+    one_launch = elems * 4 * world <= (2 << 20) or os.environ.get("MCCL_PG_SYNC") == "kernel"
+    t = torch.ones(elems, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     torch.cuda.synchronize()
-    assert t.cpu().tolist() == [float(world)] * 16
+    assert t[:16].cpu().tolist() == [float(world)] * 16
     if rank == 1:
         return
     blocking = os.environ.get("CCL_BLOCKING_WAIT") == "1"
@@ -783,7 +802,8 @@ def missing_rank_device_case(pg, rank, world):
         torch.cuda.synchronize()
     assert w.is_completed()
     assert not w.is_success()
-    assert torch.equal(t, before)
+    if one_launch:
+        assert torch.equal(t, before)  # one kernel: it skips the sum when its wait gives up
     try:
         pg.allreduce([t], c10d.AllreduceOptions())
         raise AssertionError("a failed group accepted another collective")

@@ -227,6 +227,30 @@ def xrank_case(rank, world, queues, barrier):
         capi.check(L.mccl_copy_segments_sync(arr, len(segs), i & 1, ctypes.byref(sy), stream))  # both load flavours
         want = O.alltoallv([to_carrier(h) for h in host], S, row)[rank]
         checks.append((out, want, ("copy_segments_sync", row, i)))
+    # the other direction: every rank copies a buffer of its own into its shared buffer, announces
+    # it with the closing epoch of the same launch, and reads all ranks' shared buffers with the next
+    # kernel on its stream (a plain reduction): the staged small allreduce in two launches
+    for i, (dtype, count, name, off, soff) in enumerate([(torch.bfloat16, 131072, "SUM", 0, 0), (torch.float32, 1025, "SUM", 4, 4), (torch.int8, 70001, "MAX", 3, 1),
+                                                         (torch.float64, 1, "SUM", 8, 0), (torch.bfloat16, 3, "MIN", 2, 6), (torch.float16, 1 << 19, "SUM", 0, 2),
+                                                         (torch.bfloat16, 131072, "SUM", 64, 10)]):
+        es = torch.empty(0, dtype=dtype).element_size()
+        off, soff = off // es * es, soff // es * es
+        host = [rank_buffer(count, dtype, r, seed=600 + i, scale=0.02) for r in range(world)]
+        own = torch.empty(count * es + 64, dtype=torch.uint8, device=DEV)[soff:soff + count * es].view(dtype)
+        own.copy_(host[rank])
+        call[0] += 1
+        sy = capi.XSync(ctypes.cast(words, ctypes.c_void_p), world, rank, 0, 4 * call[0] + 1, counter.data_ptr(), 5_000_000, st.data_ptr())
+        seg = (capi.Segment * 1)(capi.Segment(own.data_ptr(), shared[rank][0].data_ptr() + off, count * es))
+        capi.check(L.mccl_copy_segments_sync(seg, 1, capi.COPY_PUBLISH, ctypes.byref(sy), stream))
+        capi.check(L.mccl_reduce_n(capi.ptr_table([shared[r][0].data_ptr() + off for r in range(world)]), world, own.data_ptr(), count,
+                                   TORCH_TO_CODE[dtype], ops[name][0], capi.VARIANT_AUTO, stream))
+        want = oracle_reduce_bits(host, ops[name][1])
+        checks.append((own, want, ("publishing copy + reduce_n", str(dtype), count, name)))
+        # the next write of the shared buffer must not overtake a slow peer's read of it: the opening
+        # wait of the calls above did that; here an epoch of its own does
+        call[0] += 1
+        flags = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])
+        capi.check(L.mccl_rank_barrier(flags, world, rank, 4 * call[0] + 1, 5_000_000, st.data_ptr(), stream))
     torch.cuda.synchronize()
     assert st.tolist() == [0, 0], st.tolist()
     assert not counter.cpu().any()  # every counter is back at zero

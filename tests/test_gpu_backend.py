@@ -96,10 +96,12 @@ def test_missing_rank_raises_instead_of_hanging(monkeypatch, sync):
     _spawn(3, "missing")
 
 
-def test_wait_honours_its_timeout(monkeypatch):
-    """(with the waits inside the data kernels: the 1 MiB allreduce of that mode has no rendezvous of
-    the host threads, so the call returns while a peer is still missing and the Work has to wait)"""
-    monkeypatch.setenv("MCCL_PG_SYNC", "kernel")
+@pytest.mark.parametrize("sync", ["", "kernel"])
+def test_wait_honours_its_timeout(monkeypatch, sync):
+    """(a 1 MiB allreduce has no rendezvous of the host threads in either device-side mode, so the
+    call returns while a peer is still missing and the Work has to wait)"""
+    if sync:
+        monkeypatch.setenv("MCCL_PG_SYNC", sync)
     monkeypatch.setenv("CCL_BLOCKING_WAIT", "1")
     _spawn(3, "late_peer")
 
@@ -135,12 +137,17 @@ def test_waits_inside_the_data_kernels(monkeypatch, world, mode):
     _spawn(world, mode)
 
 
+@pytest.mark.parametrize("sync,elems", [("", 16), ("", 1 << 18), ("kernel", 1 << 18)])
 @pytest.mark.parametrize("blocking", ["0", "1"])
-def test_missing_rank_with_waits_inside_the_data_kernels(monkeypatch, blocking):
-    """The same failure with the cross-rank wait on the device (the small allreduce of this mode has no
-    rendezvous of the host threads): the kernel's own bounded wait ends it (a 1.5 s limit forced from
-    the host), the Work reports failure, the group refuses to go on."""
-    monkeypatch.setenv("MCCL_PG_SYNC", "kernel")
+def test_missing_rank_found_by_the_wait_on_the_device(monkeypatch, blocking, sync, elems):
+    """The same failure with the cross-rank wait on the device (an allreduce of up to 1 MiB has no
+    rendezvous of the host threads: one kernel does everything when the message is small or with
+    MCCL_PG_SYNC=kernel, otherwise the copy-in announces and waits): the kernel's own bounded wait
+    ends it (a 1.5 s limit forced from the host), the Work reports failure, the group refuses to
+    go on."""
+    if sync:
+        monkeypatch.setenv("MCCL_PG_SYNC", sync)
+    monkeypatch.setenv("MCCL_TEST_ELEMS", str(elems))
     monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
     monkeypatch.setenv("CCL_BLOCKING_WAIT", blocking)
     _spawn(3, "missing_device")

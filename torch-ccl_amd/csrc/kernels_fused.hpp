@@ -10,6 +10,10 @@
 //      contribution comes from the registers of step 1) and writes the caller's output.
 // A wavefront depends on the wavefronts of the same tile in the peers' launches only, so no grid
 // has to be resident as a whole, and a launch needs no second kernel and no host round trip.
+// Sixteen wavefronts (16 KiB of message) share a workgroup, for no other reason than that a
+// workgroup sits on one compute unit: the wavefronts that wait for a late rank then hold
+// bytes / 16 KiB compute units per rank instead of being spread over all of them, and whatever the
+// late rank still has to run in front of its own launch finds whole compute units free.
 // Visibility inside the kernel is per access: the staging tile is written through to memory and
 // waited for before its flag is stored, and the peers' tiles are read past the caches, so no
 // cache-wide write-back or invalidate is paid per tile.
@@ -32,17 +36,21 @@ struct FusedArgs {
   uint32_t* status;
   uint32_t tail;              // elements after the last whole vector (< elements per vector)
   uint32_t epoch;
+  uint32_t tiles;             // 1 KiB tiles of the message: wavefronts with work
   int n;
   int rank;
 };
 
+constexpr int kFusedWavesPerGroup = 16;
+
 template <int DT, int OP>
-__global__ __launch_bounds__(kWave) void allreduce_fused_kernel(const FusedArgs a) {
+__global__ __launch_bounds__(kWave * kFusedWavesPerGroup) void allreduce_fused_kernel(const FusedArgs a) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
-  const uint32_t tile = blockIdx.x;
-  const int lane = threadIdx.x;
+  const uint32_t tile = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (tile >= a.tiles) return;  // (the wavefronts of a workgroup never meet at a barrier)
+  const int lane = threadIdx.x % kWave;
   const uint64_t v = (uint64_t)tile * kWave + lane;
   const bool whole = v < a.nvec;
   const bool part = v == a.nvec && a.tail != 0;  // the one vector that is not whole

@@ -188,17 +188,17 @@ hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g,
   }
 }
 
-hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned grid_x, hipStream_t s) {
+hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned tiles, hipStream_t s) {
   switch (dtype) {
-    case MCCL_U8: return mccl_launch_fused_dt0(&a, op, grid_x, s);
-    case MCCL_I8: return mccl_launch_fused_dt1(&a, op, grid_x, s);
-    case MCCL_I16: return mccl_launch_fused_dt2(&a, op, grid_x, s);
-    case MCCL_I32: return mccl_launch_fused_dt3(&a, op, grid_x, s);
-    case MCCL_I64: return mccl_launch_fused_dt4(&a, op, grid_x, s);
-    case MCCL_F16: return mccl_launch_fused_dt5(&a, op, grid_x, s);
-    case MCCL_F32: return mccl_launch_fused_dt6(&a, op, grid_x, s);
-    case MCCL_F64: return mccl_launch_fused_dt7(&a, op, grid_x, s);
-    case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, grid_x, s);
+    case MCCL_U8: return mccl_launch_fused_dt0(&a, op, tiles, s);
+    case MCCL_I8: return mccl_launch_fused_dt1(&a, op, tiles, s);
+    case MCCL_I16: return mccl_launch_fused_dt2(&a, op, tiles, s);
+    case MCCL_I32: return mccl_launch_fused_dt3(&a, op, tiles, s);
+    case MCCL_I64: return mccl_launch_fused_dt4(&a, op, tiles, s);
+    case MCCL_F16: return mccl_launch_fused_dt5(&a, op, tiles, s);
+    case MCCL_F32: return mccl_launch_fused_dt6(&a, op, tiles, s);
+    case MCCL_F64: return mccl_launch_fused_dt7(&a, op, tiles, s);
+    case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, tiles, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -567,7 +567,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 140; }
+int mccl_version(void) { return 141; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -764,6 +764,7 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
   a.status = (uint32_t*)status;
   a.tail = (uint32_t)(count % ve);
   a.epoch = epoch;
+  a.tiles = (uint32_t)tiles;
   a.n = n;
   a.rank = rank;
   hipError_t e = launch_fused_any(a, dtype, op, (unsigned)tiles, (hipStream_t)stream);
@@ -861,7 +862,13 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
   }
   const unsigned grid = xrank_grid(chunks, a.sync.n);  // (a copy gains nothing from more wavefronts than its share, waits or not)
-  hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  if (flags & ~(MCCL_COPY_SHARED_SOURCES | MCCL_COPY_PUBLISH)) return fail(MCCL_ERR_INVALID_ARG, "unknown copy flags 0x%x", flags);
+  if (flags & MCCL_COPY_PUBLISH) {
+    if (a.sync.done_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "MCCL_COPY_PUBLISH announces the copy with the closing epoch: done_epoch must not be 0");
+    hipLaunchKernelGGL(copy_segments_publish_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  } else {
+    hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;

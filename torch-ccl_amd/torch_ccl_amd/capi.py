@@ -22,6 +22,7 @@ VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
  TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
  TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS, TUNE_COPY_VECTORS_PER_LANE, TUNE_COPY_STREAM_STORES,
  TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU, TUNE_XRANK_CACHED_LOADS) = range(13)
+COPY_SHARED_SOURCES, COPY_PUBLISH = 1, 2  # flags of mccl_copy_segments_sync
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
