@@ -263,11 +263,12 @@ def backend_path(world=8, sync=None):
     if sync is not None:
         return {name: {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()} for name in res}
     out = {"processes": world, "note": "host-timed dist.* call + synchronize per rank process; all ranks share the one "
-                                       "GPU.  The ranks wait for each other on the device: in a one-wavefront barrier "
-                                       "kernel in front of the data kernel, whose last workgroup waits for the closing "
-                                       "epoch (two launches per collective); tensors from 1 MiB on are read by the "
-                                       "peers in place.  C2 (256 KiB) is the one-launch small allreduce in both modes: "
-                                       "its waiting workgroups hold at most half of the compute units.  Every launch of a process waits for its turn at the dispatcher, "
+                                       "GPU.  The ranks wait for each other on the device: large collectives (C3, C4, C5) in "
+                                       "a one-wavefront barrier kernel in front of the data kernel, whose last workgroup "
+                                       "waits for the closing epoch (two launches); small and medium ones (C2) in the "
+                                       "data kernel itself, limited to workgroups that hold at most half of the compute "
+                                       "units over all ranks; tensors from 1 MiB on are read by the peers in place.  "
+                                       "Every launch of a process waits for its turn at the dispatcher, "
                                        "which is what one_trivial_kernel_plus_synchronize measures.  "
                                        "waits_inside_the_data_kernel: the same with MCCL_PG_SYNC=kernel (one launch per "
                                        "collective; not the default because the waiting grids of 7 ranks can keep a "

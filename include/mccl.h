@@ -224,6 +224,12 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
  * well: the kernel does not wait at all; words, counters and status are then not used).
  * Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
  * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
+ * max_compute_units: 0 -- single-wavefront workgroups, spread over the whole GPU, as many as the
+ * budget allows (the fastest shape for large messages); k > 0 -- at most k workgroups of up to 16
+ * wavefronts: a workgroup sits on one compute unit, so the launch holds at most k of the GPU's 256
+ * while it waits for a late rank, and the late rank's other kernels find the rest free.  Ranks
+ * that share a GPU keep the sum over all ranks at half the GPU (8 ranks: 16 each); the message
+ * should then be small enough for 16 k wavefronts (a few MiB).
  */
 #define MCCL_SYNC_COUNTER_BYTES 1024
 typedef struct {
@@ -235,6 +241,8 @@ typedef struct {
   void* done_counter;
   uint64_t timeout_us; /* 0 = 10 s */
   void* status;
+  unsigned max_compute_units; /* 0 = no limit */
+  unsigned reserved;          /* 0 */
 } mccl_xsync_t;
 
 /* mccl_copy_segments whose sources are peers' buffers: allgather / alltoall(v) / broadcast pulls

@@ -753,7 +753,8 @@ def heavy_predecessor_case(rank, world):
         assert float(t[0]) == want and float(t[-1]) == want, (it, float(t[0]), want)
     # the same with small messages, whose single launch waits itself (its workgroups are few enough
     # to leave compute units free); 1 MiB: copy-in whose last workgroup waits, then the reduction
-    for it, elems in enumerate((1 << 17, 1 << 19, 8)):
+    # 4 MiB: one launch again, limited to its share of half of the compute units
+    for it, elems in enumerate((1 << 17, 1 << 19, 8, 1 << 21)):
         small = torch.full((elems,), float(rank + it), dtype=torch.bfloat16, device=DEV)
         dist.barrier()
         if rank == ((it + 3) % world):
@@ -764,6 +765,32 @@ def heavy_predecessor_case(rank, world):
         torch.cuda.synchronize()
         want = float(sum(r + it for r in range(world)))
         assert float(small[0]) == want and float(small[-1]) == want, (elems, float(small[0]), want)
+    # the pulls and the shard reduction at 4 MiB per rank, a late rank each
+    n = (1 << 21) // world * world
+    src = torch.full((n,), float(rank), dtype=torch.bfloat16, device=DEV)
+    for it, what in enumerate(("all_to_all_single", "reduce_scatter_tensor", "all_gather_into_tensor")):
+        dist.barrier()
+        if rank == ((it + 5) % world):
+            time.sleep(0.003)
+            for _ in range(20):
+                c = torch.mm(a, b)
+        if what == "all_to_all_single":
+            got = torch.empty_like(src)
+            dist.all_to_all_single(got, src)
+            want = [float(r) for r in range(world)]
+            have = got.view(world, -1)[:, 0].tolist()
+        elif what == "reduce_scatter_tensor":
+            got = torch.empty(n // world, dtype=torch.bfloat16, device=DEV)
+            dist.reduce_scatter_tensor(got, src)
+            want = [float(sum(range(world)))] * 2
+            have = [float(got[0]), float(got[-1])]
+        else:
+            got = torch.empty(n * world, dtype=torch.bfloat16, device=DEV)
+            dist.all_gather_into_tensor(got, src)
+            want = [float(r) for r in range(world)]
+            have = got.view(world, -1)[:, -1].tolist()
+        torch.cuda.synchronize()
+        assert have == want, (what, have, want)
     out = torch.empty(world * 1024, dtype=torch.float32, device=DEV)
     if rank == 1:
         for _ in range(20):

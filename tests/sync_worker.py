@@ -169,8 +169,10 @@ def xrank_case(rank, world, queues, barrier):
 
     def sync(done=True):
         call[0] += 1
+        # every third call as single wavefronts all over the GPU, the others as at most 16 or 2
+        # workgroups of sixteen wavefronts
         return capi.XSync(ctypes.cast(words, ctypes.c_void_p), world, rank, 4 * call[0] + 1, 4 * call[0] + 3 if done else 0,
-                          counter.data_ptr(), 5_000_000, st.data_ptr())
+                          counter.data_ptr(), 5_000_000, st.data_ptr(), (0, 16, 2)[call[0] % 3], 0)
 
     def mine(dtype, count, off):
         return shared_in[off:off + count * torch.empty(0, dtype=dtype).element_size()].view(dtype)

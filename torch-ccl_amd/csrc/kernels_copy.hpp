@@ -55,10 +55,10 @@ __device__ __forceinline__ void store_byte(char* p, char x, bool publish) {
 }
 
 template <bool COHERENT, int UNROLL, int STORE>
-__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, bool shared_sources = false) {
+__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave& w, bool shared_sources = false) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
-  for (uint32_t chunk = blockIdx.x; chunk < total; chunk += gridDim.x) {
+  for (uint32_t chunk = w.index; chunk < total; chunk += w.count) {
     // binary search: largest s with chunk_prefix[s] <= chunk
     int lo = 0, hi = a.nseg;
     while (hi - lo > 1) {
@@ -69,7 +69,7 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, bool share
     const uint32_t head = a.seg[lo].head;
     const uint32_t nfull = a.seg[lo].nfull;
     const uint32_t len = (c < nfull) ? CHUNK : a.seg[lo].last;
-    const uint32_t t = threadIdx.x;
+    const uint32_t t = w.lane;
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
     if (c == 0)
@@ -108,14 +108,15 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, bool share
 
 template <int UNROLL, bool STREAM>
 __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
-  copy_segments_body<false, UNROLL, STREAM ? kStoreStream : kStoreHint>(a);
+  copy_segments_body<false, UNROLL, STREAM ? kStoreStream : kStoreHint>(a, this_wave<1>());
 }
 
-__global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCopyArgs a) {
+template <int WPG>
+__global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const SyncCopyArgs a) {
   if (xsync_begin(a.sync)) {
     // heads, partial chunks and misaligned sources go through the caches
     if (a.invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    copy_segments_body<true, kCopyUnroll, kStoreHint>(a.copy, a.shared != 0);
+    copy_segments_body<true, kCopyUnroll, kStoreHint>(a.copy, this_wave<WPG>(), a.shared != 0);
   }
   xsync_end(a.sync, gridDim.x);
 }
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(kWave) void copy_segments_sync_kernel(const SyncCop
 // have seen the closing epoch (a staging buffer being filled).  Ordinary loads, every byte written
 // through; xsync_end waits for the stores of each workgroup before it counts it.
 __global__ __launch_bounds__(kWave) void copy_segments_publish_kernel(const SyncCopyArgs a) {
-  if (xsync_begin(a.sync)) copy_segments_body<false, kCopyUnroll, kStorePublish>(a.copy);
+  if (xsync_begin(a.sync)) copy_segments_body<false, kCopyUnroll, kStorePublish>(a.copy, this_wave<1>());
   xsync_end(a.sync, gridDim.x);
 }
 

@@ -173,6 +173,28 @@ struct XSync {
   int rank;
 };
 
+// The unit of work of the cross-rank kernels is the wavefront: which one this is, and of how many.
+// WPG wavefronts share a workgroup.  One, normally.  kPackedWaves for launches whose waiting
+// wavefronts must sit on few compute units (a workgroup lives on one): ranks that share a GPU with
+// each other's other kernels.  The wavefronts of a workgroup never depend on each other; they meet
+// once, in xsync_end.
+struct Wave {
+  uint32_t lane;
+  uint32_t index;  // uniform
+  uint32_t count;  // uniform
+};
+constexpr int kPackedWaves = 16;
+
+template <int WPG>
+__device__ __forceinline__ Wave this_wave() {
+  if constexpr (WPG == 1) {
+    return Wave{threadIdx.x, blockIdx.x, gridDim.x};
+  } else {
+    const uint32_t in_group = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    return Wave{threadIdx.x % kWave, blockIdx.x * WPG + in_group, gridDim.x * WPG};
+  }
+}
+
 constexpr uint32_t kDoneGroups = 8;
 constexpr uint32_t kDoneStride = 16;  // 32-bit words between two counters: one cache line each
 static_assert((1 + kDoneGroups) * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "counters must fit the block the caller provides");

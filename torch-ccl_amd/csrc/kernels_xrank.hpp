@@ -51,10 +51,10 @@ struct XRankArgs {
 // tensors out of an allocator) are read past the caches in one streaming access (load_tile_coherent);
 // others as an ordinary unaligned load after a cache invalidate (aligned_in == 0 makes the kernel
 // invalidate once per workgroup).
-__device__ __forceinline__ u32x4 load_in(const char* base, uint32_t tile, uint32_t aligned) {
+__device__ __forceinline__ u32x4 load_in(const char* base, uint32_t tile, uint32_t aligned, uint32_t lane) {
   const char* tb = base + (size_t)tile * kXTileBytes;  // uniform
-  if (aligned) return load_tile_coherent(tb, threadIdx.x * 16u);
-  return __builtin_nontemporal_load(&((const u32x4_unaligned*)tb)[threadIdx.x]);
+  if (aligned) return load_tile_coherent(tb, lane * 16u);
+  return __builtin_nontemporal_load(&((const u32x4_unaligned*)tb)[lane]);
 }
 
 // in[k] for a k known at run time only (a select per rank: no dynamic indexing of the argument block)
@@ -67,22 +67,22 @@ __device__ __forceinline__ const char* pick_in(const XRankArgs& a, int k) {
 }
 
 template <int DT, int NS>
-__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
-  const uint32_t v = tile * kWave + (uint32_t)threadIdx.x;  // the host keeps tiles1 * 64 below 2^32
+__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, const Wave& w, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
+  const uint32_t v = tile * kWave + w.lane;  // the host keeps tiles1 * 64 below 2^32
   if (v < a.nvec1) {
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) {
-      if (NS ? k < NS : k < n) x[k].v = load_in(a.in[k], tile, a.aligned_in);
+      if (NS ? k < NS : k < n) x[k].v = load_in(a.in[k], tile, a.aligned_in, w.lane);
     }
   }
 }
 
 // Reduces the loaded vectors of a tile (ascending-rank chain) and stores the result.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
+__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const Wave& w, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
-  const uint32_t v = tile * kWave + (uint32_t)threadIdx.x;
+  const uint32_t v = tile * kWave + w.lane;
   if (v < a.nvec1) {
     A acc[VE];
 #pragma unroll
@@ -105,8 +105,8 @@ __device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, uint32_t t
       for (int k = 0; k < kXRanks; ++k) {
         if (NS ? k < NS : k < n) {
           char* tb = const_cast<char*>(a.in[k]) + (size_t)tile * kXTileBytes;  // uniform
-          if (a.aligned_in) store_tile_through(tb, threadIdx.x * 16u, r.v);
-          else store_vec_through(tb + threadIdx.x * 16u, r.v);
+          if (a.aligned_in) store_tile_through(tb, w.lane * 16u, r.v);
+          else store_vec_through(tb + w.lane * 16u, r.v);
         }
       }
     } else {
@@ -119,12 +119,12 @@ __device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, uint32_t t
 
 // The elements after the last whole vector (fewer than a vector holds): lane e takes element e.
 template <int DT, int OP>
-__device__ __forceinline__ void xrank_tail(const XRankArgs& a, int n) {
+__device__ __forceinline__ void xrank_tail(const XRankArgs& a, const Wave& w, int n) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
-  if (threadIdx.x < a.tail1) {
-    const size_t i = (size_t)a.nvec1 * VE + threadIdx.x;
+  if (w.lane < a.tail1) {
+    const size_t i = (size_t)a.nvec1 * VE + w.lane;
     A acc = chain_first<DT, OP>(Elem<DT>::load(__hip_atomic_load(&((const S*)a.in[0])[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
     for (int k = 1; k < n; ++k) {
       const S* src = (const S*)pick_in(a, k);
@@ -139,39 +139,40 @@ __device__ __forceinline__ void xrank_tail(const XRankArgs& a, int n) {
   }
 }
 
-// The grid is persistent: a wavefront walks tiles blockIdx.x, + gridDim.x, ...  The loads of its
+// The grid is persistent: wavefront i of c walks tiles i, i + c, ...  The loads of its
 // next tile are in flight while it reduces and stores the current one (two register sets, used
 // alternately): without that all wavefronts, released together by the opening wait, alternate
 // between a phase of loads and a phase of stores in step, and the memory pipeline runs dry
 // between the phases.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_walk(const XRankArgs& a, int n) {
-  const uint32_t T = a.tiles1, G = gridDim.x;
-  uint32_t t0 = blockIdx.x;
+__device__ __forceinline__ void xrank_walk(const XRankArgs& a, const Wave& w, int n) {
+  const uint32_t T = a.tiles1, G = w.count;
+  uint32_t t0 = w.index;
   if (t0 < T) {
     VecU<DT> x0[kXRanks], x1[kXRanks];
-    xrank_load_tile<DT, NS>(a, t0, n, x0);
+    xrank_load_tile<DT, NS>(a, w, t0, n, x0);
     for (;;) {
       const uint32_t t1 = t0 + G;
-      if (t1 < T) xrank_load_tile<DT, NS>(a, t1, n, x1);
-      xrank_finish_tile<DT, OP, NS>(a, t0, n, x0);
+      if (t1 < T) xrank_load_tile<DT, NS>(a, w, t1, n, x1);
+      xrank_finish_tile<DT, OP, NS>(a, w, t0, n, x0);
       if (t1 >= T) break;
       t0 = t1 + G;
-      if (t0 < T) xrank_load_tile<DT, NS>(a, t0, n, x0);
-      xrank_finish_tile<DT, OP, NS>(a, t1, n, x1);
+      if (t0 < T) xrank_load_tile<DT, NS>(a, w, t0, n, x0);
+      xrank_finish_tile<DT, OP, NS>(a, w, t1, n, x1);
       if (t0 >= T) break;
     }
   }
 }
 
-template <int DT, int OP>
-__global__ __launch_bounds__(kWave) void xrank_reduce_kernel(const XRankArgs a) {
+template <int DT, int OP, int WPG>
+__global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankArgs a) {
   const int n = a.sync.n;
+  const Wave w = this_wave<WPG>();
   if (xsync_begin(a.sync)) {
     if (!a.aligned_in) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
-    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, n);
-    else xrank_walk<DT, OP, 0>(a, n);
-    if (a.tail1 && blockIdx.x == gridDim.x - 1) xrank_tail<DT, OP>(a, n);
+    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, w, n);
+    else xrank_walk<DT, OP, 0>(a, w, n);
+    if (a.tail1 && w.index == w.count - 1) xrank_tail<DT, OP>(a, w, n);
   }
   xsync_end(a.sync, gridDim.x);
 }

@@ -203,17 +203,17 @@ hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned tile
   }
 }
 
-hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned grid_x, unsigned lds, hipStream_t s) {
+hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned groups, int packed, unsigned lds, hipStream_t s) {
   switch (dtype) {
-    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, grid_x, lds, s);
-    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, grid_x, lds, s);
-    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, grid_x, lds, s);
-    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, grid_x, lds, s);
-    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, grid_x, lds, s);
-    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, grid_x, lds, s);
-    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, grid_x, lds, s);
-    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, grid_x, lds, s);
-    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, grid_x, lds, s);
+    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, groups, packed, lds, s);
+    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, groups, packed, lds, s);
+    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, groups, packed, lds, s);
+    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, groups, packed, lds, s);
+    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, groups, packed, lds, s);
+    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, groups, packed, lds, s);
+    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, groups, packed, lds, s);
+    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, groups, packed, lds, s);
+    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, groups, packed, lds, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -567,7 +567,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 141; }
+int mccl_version(void) { return 142; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -788,6 +788,21 @@ unsigned xrank_grid(uint64_t tiles, int n, bool waits = true) {
   return (unsigned)(tiles < cap ? tiles : cap);
 }
 
+// The shape of a cross-rank launch: single wavefronts spread over the GPU, or -- when the caller
+// limits the compute units the launch may hold while it waits -- that many workgroups of
+// kPackedWaves wavefronts at most (and never more wavefronts than the budget above allows).
+struct XShape {
+  unsigned groups;
+  int packed;
+};
+XShape xrank_shape(uint64_t tiles, const mccl_xsync_t* sy, bool waits = true) {
+  if (sy->max_compute_units == 0) return XShape{xrank_grid(tiles, sy->n, waits), 0};
+  const uint64_t waves = xrank_grid(tiles, sy->n, waits);
+  uint64_t groups = (waves + kPackedWaves - 1) / kPackedWaves;
+  if (groups > sy->max_compute_units) groups = sy->max_compute_units;
+  return XShape{(unsigned)groups, 1};
+}
+
 int fill_xsync(const mccl_xsync_t* sy, XSync* x) {
   if (!sy) return fail(MCCL_ERR_INVALID_ARG, "sync descriptor is null");
   if (sy->n < 1 || sy->n > kXRanks) return fail(MCCL_ERR_UNSUPPORTED, "one-launch collectives take 1 to %d ranks, got %d", kXRanks, sy->n);
@@ -861,13 +876,16 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
     const CopySeg& cs = a.copy.seg[k];
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
   }
-  const unsigned grid = xrank_grid(chunks, a.sync.n);  // (a copy gains nothing from more wavefronts than its share, waits or not)
+  const XShape shape = xrank_shape(chunks, sync);  // (a copy gains nothing from more wavefronts than its share, waits or not)
+  const unsigned grid = shape.groups;
   if (flags & ~(MCCL_COPY_SHARED_SOURCES | MCCL_COPY_PUBLISH)) return fail(MCCL_ERR_INVALID_ARG, "unknown copy flags 0x%x", flags);
   if (flags & MCCL_COPY_PUBLISH) {
     if (a.sync.done_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "MCCL_COPY_PUBLISH announces the copy with the closing epoch: done_epoch must not be 0");
+    if (shape.packed) return fail(MCCL_ERR_INVALID_ARG, "MCCL_COPY_PUBLISH waits with one wavefront: max_compute_units does not apply");
     hipLaunchKernelGGL(copy_segments_publish_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   } else {
-    hipLaunchKernelGGL(copy_segments_sync_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+    if (shape.packed) hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
@@ -904,7 +922,8 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
   for (int k = 0; k < a.sync.n; ++k)
     if (count && ((uintptr_t)in[k] & 7u)) a.aligned_in = 0;
   if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, a.sync.n, a.sync.ready_epoch != 0), 0u, (hipStream_t)stream);
+  const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
@@ -946,7 +965,8 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   a.tail1 = (uint32_t)(n_me % ve);
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
   if (g_tune[MCCL_TUNE_XRANK_CACHED_LOADS] == 1) a.aligned_in = 0;
-  hipError_t e = launch_xrank_any(a, dtype, op, xrank_grid(a.tiles1, n, a.sync.ready_epoch != 0), 0u, (hipStream_t)stream);
+  const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }

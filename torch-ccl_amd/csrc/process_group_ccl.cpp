@@ -438,6 +438,8 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
     one_launch_max_ = (size_t)std::atoll(v);
     one_launch_max_forced_ = true;  // binds the collectives that are one launch at every size, too
   }
+  if (const char* v = std::getenv("MCCL_PG_COMPACT_MAX_BYTES")) compact_max_ = (size_t)std::atoll(v);
+  if (const char* v = std::getenv("MCCL_PG_WAITING_COMPUTE_UNITS")) waiting_cus_ = (unsigned)std::max(1, std::atoi(v));
   // The staging window can be shrunk (never enlarged) so that tests reach every windowed path
   // with small tensors.
   stage_max_ = kStageMaxDefault;
@@ -1194,9 +1196,11 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     // copy-in (two launches instead of three): the launch says "my staging buffer is complete",
     // and no closing wait is needed, as for every staged collective (see the slot rule above).
     const size_t moved = zero_copy ? plan.share_bytes : plan.stage_bytes;
-    const bool one_launch = waits_in_data_kernels_ && plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS &&
-                            (zero_copy || !plan.exec_sync_in_place_only) &&
-                            ((zero_copy && plan.one_launch_any_size && !one_launch_max_forced_) || moved <= one_launch_max_);
+    const bool can_wait_inside = plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS && (zero_copy || !plan.exec_sync_in_place_only);
+    // (compact: all ranks' waiting workgroups together on at most half of the compute units)
+    const bool compact = !waits_in_data_kernels_ && can_wait_inside && (double)moved * plan.compact_cost <= (double)compact_max_;
+    const bool one_launch = compact || (waits_in_data_kernels_ && can_wait_inside &&
+                                        ((zero_copy && plan.one_launch_any_size && !one_launch_max_forced_) || moved <= one_launch_max_));
     last_path_ = one_launch ? (zero_copy ? "one launch, peers read in place" : "copy-in and one launch")
                             : zero_copy ? "barrier kernel, peers read in place"
                                         : candidate ? "staged: a rank cannot share its tensor" : "staged";
@@ -1207,12 +1211,13 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     }
     if (one_launch) {
       if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
-      mccl_xsync_t sync;
+      mccl_xsync_t sync{};
       sync.words = bar_flags_.data();
       sync.n = size_;
       sync.rank = rank_;
       sync.ready_epoch = epoch + 1;
       sync.done_epoch = zero_copy ? epoch + 3 : 0;
+      sync.max_compute_units = compact ? std::max(1u, waiting_cus_ / (unsigned)size_) : 0u;
       sync.done_counter = done_counter_;
       sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
       sync.status = status_dev_;
@@ -1479,6 +1484,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // size measured (16 MiB to 512 MiB per rank), so it is not subject to the one-launch limit.
       p.one_launch_any_size = true;
       p.exec_sync_in_place_only = true;
+      p.compact_cost = 1.0;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<void*> tensors((size_t)W);
         for (int k = 0; k < W; ++k) tensors[(size_t)k] = const_cast<void*>(pv.user[(size_t)k]);
@@ -1591,6 +1597,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
           segs[(size_t)r] = {pv.zero_copy ? pv.user[(size_t)r] : pv.stage[(size_t)r], out + (size_t)r * per_rank, len};
         MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
       };
+      p.compact_cost = 2.0 * (double)size_;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<mccl_segment_t> segs((size_t)W);
         for (int r = 0; r < W; ++r)
@@ -1670,6 +1677,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
     const auto segs = pulls(pv);
     MCCL_CHECK(mccl_copy_segments(segs.data(), (int)segs.size(), s));
   };
+  p.compact_cost = 2.0 * (double)size_;
   p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
     const auto segs = pulls(pv);
     MCCL_CHECK(mccl_copy_segments_sync(segs.data(), (int)segs.size(), MCCL_COPY_SHARED_SOURCES, &sync, s));
@@ -1781,6 +1789,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
           MCCL_CHECK(mccl_reduce_scatter_n(pv.stage.data(), W, &o, len, me, 1, dtype, op, s));
         }
       };
+      p.compact_cost = 0.5;
       p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
         std::vector<const void*> src((size_t)W);
         for (int k = 0; k < W; ++k)  // in place: slice `me` of rank k's tensor; staged: slice `me` of the window rank k staged
@@ -1883,6 +1892,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
     if (out.numel())
       MCCL_CHECK(mccl_reduce_n(in.data(), W, out.data_ptr(), (size_t)out.numel(), dtype, op, MCCL_VARIANT_AUTO, s));
   };
+  p.compact_cost = 0.5;
   p.exec_sync = [=](const PeerView& pv, mccl_xsync_t& sync, hipStream_t s) {
     const auto in = sources(pv);
     MCCL_CHECK(mccl_reduce_sync(in.data(), out.data_ptr(), (size_t)out.numel(), dtype, op, &sync, s));

@@ -254,6 +254,11 @@ class ProcessGroupCCL : public c10d::Backend {
     size_t zero_copy_stage_bytes = 0;       // staging this rank still needs in zero-copy mode
     bool exec_sync_in_place_only = false;   // exec_sync writes into the peers' tensors: not for staged runs
     bool one_launch_any_size = false;       // exec_sync wins at every size: the default one-launch limit does not apply
+    // What a byte of share_bytes / stage_bytes costs exec_sync's launch, in bytes of a plain copy's
+    // traffic (read + write): 2 for a pull, 2 W for an allgather (W times the input is read and
+    // written), less for reductions, whose wavefronts keep eight loads in flight each.  Decides up to
+    // which size a launch limited to few compute units beats a barrier kernel and a full grid.
+    double compact_cost = 2.0;
     // Eligible for the one-launch small allreduce (device-synchronised groups of at most 8 ranks):
     // no staging slot, no table, no rendezvous.  The staged plan above stays as the fallback.
     bool fused_ok = false;
@@ -346,6 +351,16 @@ class ProcessGroupCCL : public c10d::Backend {
   // size.  MCCL_PG_ONE_LAUNCH_MAX_BYTES overrides (and then binds the allreduce, too).
   size_t one_launch_max_ = 128u << 20;
   bool one_launch_max_forced_ = false;
+  // Without MCCL_PG_SYNC=kernel a collective is still one launch with the waits inside when its
+  // launch moves at most this much (in bytes of a plain copy's traffic, see Plan::compact_cost): the
+  // launch is then limited to its share of half of the GPU's compute units (workgroups of sixteen
+  // wavefronts), which is enough for a small message and leaves a late rank's other kernels room to
+  // run.  Measured with 8 rank processes, back to back, against barrier kernel + full grid: pulls
+  // win up to 8 MiB per rank (4 MiB: 65-83 against 93-131 us; 16 MiB: 150-160 against 113-147),
+  // all_gather up to 1 MiB per rank (8 MiB written), reduce_scatter and the in-place allreduce up
+  // to 32 MiB (16 MiB: 83-104 against 106-141 us).  MCCL_PG_COMPACT_MAX_BYTES overrides (0: never).
+  size_t compact_max_ = 16u << 20;
+  unsigned waiting_cus_ = 128;  // what all ranks' waiting launches may hold together (MCCL_PG_WAITING_COMPUTE_UNITS)
   bool distinct_pids_ = false;          // every rank is a process of its own
   const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
   const char* last_path_ = "";

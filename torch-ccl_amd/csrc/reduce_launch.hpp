@@ -99,18 +99,19 @@ hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned tiles, hipStr
   return hipGetLastError();
 }
 
-// The one-launch cross-rank reduction (reduce_scatter, two-shot allreduce): persistent grid.
-template <int DT>
-hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned grid_x, unsigned lds, hipStream_t s) {
-  const dim3 grid(grid_x, 1, 1), block(kWave);
+// The one-launch cross-rank reduction (reduce_scatter, in-place allreduce): persistent grid of
+// `groups` workgroups, single wavefronts or (packed) kPackedWaves wavefronts each.
+template <int DT, int WPG>
+hipError_t launch_xrank_packing(const XRankArgs& a, int op, unsigned groups, unsigned lds, hipStream_t s) {
+  const dim3 grid(groups, 1, 1), block(kWave * WPG);
   switch (op) {
-    case MCCL_SUM: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_SUM>), grid, block, lds, s, a); break;
-    case MCCL_PROD: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_PROD>), grid, block, lds, s, a); break;
-    case MCCL_MIN: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MIN>), grid, block, lds, s, a); break;
-    case MCCL_MAX: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MAX>), grid, block, lds, s, a); break;
+    case MCCL_SUM: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_SUM, WPG>), grid, block, lds, s, a); break;
+    case MCCL_PROD: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_PROD, WPG>), grid, block, lds, s, a); break;
+    case MCCL_MIN: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MIN, WPG>), grid, block, lds, s, a); break;
+    case MCCL_MAX: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MAX, WPG>), grid, block, lds, s, a); break;
     case MCCL_AVG:
       if constexpr (Elem<DT>::kIsFloat) {
-        hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_AVG>), grid, block, lds, s, a);
+        hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_AVG, WPG>), grid, block, lds, s, a);
         break;
       } else {
         return hipErrorInvalidValue;
@@ -118,6 +119,11 @@ hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned grid_x, unsig
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
+}
+
+template <int DT>
+hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned groups, int packed, unsigned lds, hipStream_t s) {
+  return packed ? launch_xrank_packing<DT, kPackedWaves>(a, op, groups, lds, s) : launch_xrank_packing<DT, 1>(a, op, groups, lds, s);
 }
 
 }  // namespace
@@ -152,7 +158,7 @@ __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt6(MCCL_FUSE
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt7(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt8(MCCL_FUSED_ENTRY_ARGS);
 // `xrank_args` points at an XRankArgs; lds = dynamic LDS bytes reserved per workgroup (residency cap)
-#define MCCL_XRANK_ENTRY_ARGS const void *xrank_args, int op, unsigned grid_x, unsigned lds, hipStream_t stream
+#define MCCL_XRANK_ENTRY_ARGS const void *xrank_args, int op, unsigned groups, int packed, unsigned lds, hipStream_t stream
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt0(MCCL_XRANK_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt1(MCCL_XRANK_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt2(MCCL_XRANK_ENTRY_ARGS);

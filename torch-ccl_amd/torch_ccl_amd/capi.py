@@ -47,7 +47,8 @@ class XSync(ctypes.Structure):
     """mccl_xsync_t"""
     _fields_ = [("words", ctypes.c_void_p), ("n", ctypes.c_int), ("rank", ctypes.c_int),
                 ("ready_epoch", ctypes.c_uint64), ("done_epoch", ctypes.c_uint64), ("done_counter", ctypes.c_void_p),
-                ("timeout_us", ctypes.c_uint64), ("status", ctypes.c_void_p)]
+                ("timeout_us", ctypes.c_uint64), ("status", ctypes.c_void_p),
+                ("max_compute_units", ctypes.c_uint), ("reserved", ctypes.c_uint)]
 
 
 class Segment(ctypes.Structure):
