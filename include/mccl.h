@@ -195,14 +195,18 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
  * is bounded and reported like mccl_rank_barrier's; a tile whose peers did not arrive in time is
  * left unwritten.  The launch is one workgroup per 16 KiB of message, and a workgroup sits on one
  * compute unit: while it waits for a late rank it holds count * size / 16 KiB of the GPU's 256
- * compute units, which is how a caller whose ranks share a GPU bounds what the waiting ranks keep
- * from the late one's other kernels.
+ * compute units.  max_compute_units (0 = no limit) caps that: the launch is then at most that
+ * many workgroups, whose wavefronts take up to four tiles each, and a message of more than
+ * max_compute_units * 64 KiB is refused.  A wavefront waits for the same tile of every peer, so
+ * the launches of all ranks that share a GPU must be resident together with room to spare (an
+ * MI355X holds 512 such workgroups when nothing else runs): ranks that share a GPU pass a limit
+ * -- at most 256 / n; 128 / n leaves half of the compute units to a late rank's other kernels.
  */
 #define MCCL_FUSED_MAX_RANKS 8
 #define MCCL_FUSED_TILE_BYTES 1024
 int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
                          void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
-                         uint64_t timeout_us, void* status, void* stream);
+                         uint64_t timeout_us, void* status, unsigned max_compute_units, void* stream);
 
 /*
  * One-launch collectives between rank processes that read the peers' buffers in place.  With
@@ -249,15 +253,8 @@ typedef struct {
  * (ccl::allgatherv, ccl::alltoallv, src/gpu/dpcpp_ccl.cpp:1176-1182, 1428-1455) in one launch.
  * At most 64 segments; zero segments still take part in the waits.  flags: MCCL_COPY_SHARED_SOURCES
  * when the other ranks read the same source bytes in the same collective (allgather, broadcast):
- * the sources are then kept in the memory-side cache instead of being streamed past it.
- * MCCL_COPY_PUBLISH turns the direction round: the sources are this rank's own memory and the
- * destinations are buffers that the peers read next (staging buffers; the copy-in of the staged
- * collectives, src/gpu/allreduce_small.h:165-287, with its announcement in the same launch): every
- * byte is written through to memory before the closing epoch is published, so a peer that has seen
- * done_epoch -- its own launch of the same call has then returned -- may read them with its next
- * kernel.  done_epoch must not be 0; ready_epoch usually is. */
+ * the sources are then kept in the memory-side cache instead of being streamed past it. */
 #define MCCL_COPY_SHARED_SOURCES 1u
-#define MCCL_COPY_PUBLISH 2u
 int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync,
                             void* stream);
 

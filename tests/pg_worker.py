@@ -751,9 +751,8 @@ def heavy_predecessor_case(rank, world):
         torch.cuda.synchronize()
         want = float(sum(r + it for r in range(world)))
         assert float(t[0]) == want and float(t[-1]) == want, (it, float(t[0]), want)
-    # the same with small messages, whose single launch waits itself (its workgroups are few enough
-    # to leave compute units free); 1 MiB: copy-in whose last workgroup waits, then the reduction
-    # 4 MiB: one launch again, limited to its share of half of the compute units
+    # the same with small and medium messages, whose single launch waits itself, limited to its
+    # share of half of the compute units
     for it, elems in enumerate((1 << 17, 1 << 19, 8, 1 << 21)):
         small = torch.full((elems,), float(rank + it), dtype=torch.bfloat16, device=DEV)
         dist.barrier()
@@ -805,10 +804,9 @@ def missing_rank_device_case(pg, rank, world):
     """Device-side waits: rank 1 never joins the second collective.  The survivors' kernel gives up
     by itself at the (shortened) limit and names the late rank; their Work reports the failure
     instead of success, the group refuses further collectives, and (one-launch form) the tensor is
-    left alone.  MCCL_TEST_ELEMS floats: 16 is one launch in every mode, 2^18 (1 MiB) is an
-    announcing copy-in and a reduction unless MCCL_PG_SYNC=kernel makes it one launch too."""
+    left alone.  MCCL_TEST_ELEMS floats: 16, or 2^18 (1 MiB: the largest message of this form,
+    four tiles per wavefront when the launch is limited to few compute units)."""
     elems = int(os.environ.get("MCCL_TEST_ELEMS", "16"))
-    one_launch = elems * 4 * world <= (2 << 20) or os.environ.get("MCCL_PG_SYNC") == "kernel"
     t = torch.ones(elems, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     torch.cuda.synchronize()
@@ -829,8 +827,7 @@ def missing_rank_device_case(pg, rank, world):
         torch.cuda.synchronize()
     assert w.is_completed()
     assert not w.is_success()
-    if one_launch:
-        assert torch.equal(t, before)  # one kernel: it skips the sum when its wait gives up
+    assert torch.equal(t, before)  # the kernel skips the sum when its wait gives up
     try:
         pg.allreduce([t], c10d.AllreduceOptions())
         raise AssertionError("a failed group accepted another collective")

@@ -96,6 +96,12 @@ def fused_case(rank, world, queues, barrier):
                 cases.append((dtype, count, name))
     cases.append((torch.bfloat16, 131072, "SUM"))       # the 256 KiB decode message
     cases.append((torch.float32, FUSED_MAX_BYTES // 4, "SUM"))
+    # the same on few compute units: exactly four tiles per wavefront, an uneven split, one workgroup
+    forced = {}
+    for dtype, count, units in ((torch.bfloat16, 131072, 4), (torch.float32, FUSED_MAX_BYTES // 4, 16), (torch.float32, FUSED_MAX_BYTES // 4 - 5, 17),
+                                (torch.bfloat16, 131072 - 9, 5), (torch.int8, 64 << 10, 1), (torch.float64, 3 * 1024 + 1, 1)):
+        forced[len(cases)] = units
+        cases.append((dtype, count, "SUM"))
     pending = []
     epoch = 0
     for i, (dtype, count, name) in enumerate(cases):
@@ -108,9 +114,14 @@ def fused_case(rank, world, queues, barrier):
         out = x if in_place else torch.empty_like(x)
         epoch += 1
         slot = epoch & 1
+        # every third call as many workgroups as the message has 16 KiB pieces, the others limited to
+        # 128 / world of them (the limit bites from 256 KiB on) or to what the message just fits in
+        units = forced.get(i, (0, 128 // world, max(1, -(-count * dtype.itemsize // (64 << 10))))[i % 3])
+        if units == 0 and count * dtype.itemsize * world > (2 << 20):
+            units = 256 // world  # all ranks' launches must be resident together, with room to spare
         capi.check(L.mccl_allreduce_fused(x.data_ptr(), out.data_ptr(), count, TORCH_TO_CODE[dtype], ops[name][0],
                                           tables[slot][0], tables[slot][1], world, rank, epoch, 5_000_000,
-                                          st.data_ptr(), stream))
+                                          st.data_ptr(), units, stream))
         pending.append((out, want, (str(dtype), count, name, in_place)))
         if len(pending) >= 64:
             torch.cuda.synchronize()
@@ -133,7 +144,7 @@ def fused_case(rank, world, queues, barrier):
         out = torch.empty_like(x)
         capi.check(L.mccl_allreduce_fused(x.data_ptr(), out.data_ptr(), count, capi.BF16, capi.SUM,
                                           tables[slot][0], tables[slot][1], world, rank, epoch, 5_000_000,
-                                          st.data_ptr(), stream))
+                                          st.data_ptr(), (0, 4)[it & 1], stream))
         outs.append(out)
         x = out  # the next round reduces the previous result: any stale read changes every later round
     torch.cuda.synchronize()
@@ -229,30 +240,6 @@ def xrank_case(rank, world, queues, barrier):
         capi.check(L.mccl_copy_segments_sync(arr, len(segs), i & 1, ctypes.byref(sy), stream))  # both load flavours
         want = O.alltoallv([to_carrier(h) for h in host], S, row)[rank]
         checks.append((out, want, ("copy_segments_sync", row, i)))
-    # the other direction: every rank copies a buffer of its own into its shared buffer, announces
-    # it with the closing epoch of the same launch, and reads all ranks' shared buffers with the next
-    # kernel on its stream (a plain reduction): the staged small allreduce in two launches
-    for i, (dtype, count, name, off, soff) in enumerate([(torch.bfloat16, 131072, "SUM", 0, 0), (torch.float32, 1025, "SUM", 4, 4), (torch.int8, 70001, "MAX", 3, 1),
-                                                         (torch.float64, 1, "SUM", 8, 0), (torch.bfloat16, 3, "MIN", 2, 6), (torch.float16, 1 << 19, "SUM", 0, 2),
-                                                         (torch.bfloat16, 131072, "SUM", 64, 10)]):
-        es = torch.empty(0, dtype=dtype).element_size()
-        off, soff = off // es * es, soff // es * es
-        host = [rank_buffer(count, dtype, r, seed=600 + i, scale=0.02) for r in range(world)]
-        own = torch.empty(count * es + 64, dtype=torch.uint8, device=DEV)[soff:soff + count * es].view(dtype)
-        own.copy_(host[rank])
-        call[0] += 1
-        sy = capi.XSync(ctypes.cast(words, ctypes.c_void_p), world, rank, 0, 4 * call[0] + 1, counter.data_ptr(), 5_000_000, st.data_ptr())
-        seg = (capi.Segment * 1)(capi.Segment(own.data_ptr(), shared[rank][0].data_ptr() + off, count * es))
-        capi.check(L.mccl_copy_segments_sync(seg, 1, capi.COPY_PUBLISH, ctypes.byref(sy), stream))
-        capi.check(L.mccl_reduce_n(capi.ptr_table([shared[r][0].data_ptr() + off for r in range(world)]), world, own.data_ptr(), count,
-                                   TORCH_TO_CODE[dtype], ops[name][0], capi.VARIANT_AUTO, stream))
-        want = oracle_reduce_bits(host, ops[name][1])
-        checks.append((own, want, ("publishing copy + reduce_n", str(dtype), count, name)))
-        # the next write of the shared buffer must not overtake a slow peer's read of it: the opening
-        # wait of the calls above did that; here an epoch of its own does
-        call[0] += 1
-        flags = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])
-        capi.check(L.mccl_rank_barrier(flags, world, rank, 4 * call[0] + 1, 5_000_000, st.data_ptr(), stream))
     torch.cuda.synchronize()
     assert st.tolist() == [0, 0], st.tolist()
     assert not counter.cpu().any()  # every counter is back at zero
@@ -285,7 +272,7 @@ def timeout_case(rank, world, queues, barrier):
             x.data_ptr(), out.data_ptr(), 256, capi.F32, capi.SUM,
             capi.ptr_table([shared[r][1].data_ptr() for r in range(world)]),
             capi.ptr_table([shared[r][2].data_ptr() for r in range(world)]), world, rank, 9, 200_000,
-            st.data_ptr(), stream))
+            st.data_ptr(), 0, stream))
         torch.cuda.synchronize()
         assert st.tolist() == [2, 9], st.tolist()
         assert out.cpu().tolist() == [-7.0] * 256

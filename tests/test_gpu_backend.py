@@ -140,11 +140,9 @@ def test_waits_inside_the_data_kernels(monkeypatch, world, mode):
 @pytest.mark.parametrize("sync,elems", [("", 16), ("", 1 << 18), ("kernel", 1 << 18)])
 @pytest.mark.parametrize("blocking", ["0", "1"])
 def test_missing_rank_found_by_the_wait_on_the_device(monkeypatch, blocking, sync, elems):
-    """The same failure with the cross-rank wait on the device (an allreduce of up to 1 MiB has no
-    rendezvous of the host threads: one kernel does everything when the message is small or with
-    MCCL_PG_SYNC=kernel, otherwise the copy-in announces and waits): the kernel's own bounded wait
-    ends it (a 1.5 s limit forced from the host), the Work reports failure, the group refuses to
-    go on."""
+    """The same failure with the cross-rank wait on the device (an allreduce of up to 1 MiB is one
+    kernel and has no rendezvous of the host threads): the kernel's own bounded wait ends it (a
+    1.5 s limit forced from the host), the Work reports failure, the group refuses to go on."""
     if sync:
         monkeypatch.setenv("MCCL_PG_SYNC", sync)
     monkeypatch.setenv("MCCL_TEST_ELEMS", str(elems))

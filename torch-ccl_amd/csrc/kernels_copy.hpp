@@ -43,18 +43,9 @@ struct SyncCopyArgs {
 // kernel's caches: 8-byte aligned sources are read past the caches (the host requests a cache
 // invalidate per workgroup for the others).
 // UNROLL: 16-byte vectors per lane per chunk (chunk = 64 x 16 x UNROLL bytes; the host computes
-// the segment geometry for the same value).  STORE: kStoreHint -- non-temporal hint;
-// kStoreStream -- full chunks are written through past the caches at agent scope (`sc1`);
-// kStorePublish -- every byte is written through to memory (`sc0 sc1`), so that a flag stored
-// after wait_own_stores() tells another rank that the destination is complete.
-constexpr int kStoreHint = 0, kStoreStream = 1, kStorePublish = 2;
-
-__device__ __forceinline__ void store_byte(char* p, char x, bool publish) {
-  if (publish) __hip_atomic_store((unsigned char*)p, (unsigned char)x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  else *p = x;
-}
-
-template <bool COHERENT, int UNROLL, int STORE>
+// the segment geometry for the same value).  STREAM: full chunks are written through past the
+// caches (`sc1`) instead of with the non-temporal hint.
+template <bool COHERENT, int UNROLL, bool STREAM>
 __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave& w, bool shared_sources = false) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
@@ -73,7 +64,7 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
     if (c == 0)
-      for (uint32_t i = t; i < head; i += kWave) store_byte(dst + i, src[i], STORE == kStorePublish);  // head < 128
+      for (uint32_t i = t; i < head; i += kWave) dst[i] = src[i];  // head < 128
     const size_t off = (size_t)head + (size_t)c * CHUNK;  // start of this chunk
     src += off;
     dst += off;
@@ -90,25 +81,21 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if constexpr (STORE == kStorePublish) store_vec_through((char*)&dv[t + u * kWave], x[u]);
-        else if constexpr (STORE == kStoreStream) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&dv[t + u * kWave]), "v"(x[u]) : "memory");
+        if constexpr (STREAM) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&dv[t + u * kWave]), "v"(x[u]) : "memory");
         else __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
       }
     } else {
       const uint32_t nv = len >> 4;
-      for (uint32_t v = t; v < nv; v += kWave) {
-        if constexpr (STORE == kStorePublish) store_vec_through((char*)&dv[v], sv[v]);
-        else dv[v] = sv[v];
-      }
+      for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
       const uint32_t rem = len & 15u;
-      if (t < rem) store_byte(dst + (nv << 4) + t, src[(nv << 4) + t], STORE == kStorePublish);
+      if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
     }
   }
 }
 
 template <int UNROLL, bool STREAM>
 __global__ __launch_bounds__(kWave) void copy_segments_kernel(const CopyArgs a) {
-  copy_segments_body<false, UNROLL, STREAM ? kStoreStream : kStoreHint>(a, this_wave<1>());
+  copy_segments_body<false, UNROLL, STREAM>(a, this_wave<1>());
 }
 
 template <int WPG>
@@ -116,16 +103,8 @@ __global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const S
   if (xsync_begin(a.sync)) {
     // heads, partial chunks and misaligned sources go through the caches
     if (a.invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    copy_segments_body<true, kCopyUnroll, kStoreHint>(a.copy, this_wave<WPG>(), a.shared != 0);
+    copy_segments_body<true, kCopyUnroll, false>(a.copy, this_wave<WPG>(), a.shared != 0);
   }
-  xsync_end(a.sync, gridDim.x);
-}
-
-// The other direction: this rank's own memory into a buffer that the peers read as soon as they
-// have seen the closing epoch (a staging buffer being filled).  Ordinary loads, every byte written
-// through; xsync_end waits for the stores of each workgroup before it counts it.
-__global__ __launch_bounds__(kWave) void copy_segments_publish_kernel(const SyncCopyArgs a) {
-  if (xsync_begin(a.sync)) copy_segments_body<false, kCopyUnroll, kStorePublish>(a.copy, this_wave<1>());
   xsync_end(a.sync, gridDim.x);
 }
 

@@ -13,7 +13,9 @@
 // Sixteen wavefronts (16 KiB of message) share a workgroup, for no other reason than that a
 // workgroup sits on one compute unit: the wavefronts that wait for a late rank then hold
 // bytes / 16 KiB compute units per rank instead of being spread over all of them, and whatever the
-// late rank still has to run in front of its own launch finds whole compute units free.
+// late rank still has to run in front of its own launch finds whole compute units free.  A caller
+// that limits the compute units further gets up to four tiles per wavefront: all copied in and
+// published first, then waited for and reduced one after the other.
 // Visibility inside the kernel is per access: the staging tile is written through to memory and
 // waited for before its flag is stored, and the peers' tiles are read past the caches, so no
 // cache-wide write-back or invalidate is paid per tile.
@@ -43,68 +45,92 @@ struct FusedArgs {
 
 constexpr int kFusedWavesPerGroup = 16;
 
+// A launch limited to few workgroups gives a wavefront up to this many tiles.
+constexpr int kFusedMaxTilesPerWave = 4;
+
 template <int DT, int OP>
 __global__ __launch_bounds__(kWave * kFusedWavesPerGroup) void allreduce_fused_kernel(const FusedArgs a) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
-  const uint32_t tile = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (tile >= a.tiles) return;  // (the wavefronts of a workgroup never meet at a barrier)
+  const uint32_t wave = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const uint32_t waves = gridDim.x * (blockDim.x / kWave);
+  if (wave >= a.tiles) return;  // (the wavefronts of a workgroup never meet at a barrier)
   const int lane = threadIdx.x % kWave;
-  const uint64_t v = (uint64_t)tile * kWave + lane;
-  const bool whole = v < a.nvec;
-  const bool part = v == a.nvec && a.tail != 0;  // the one vector that is not whole
+  // this wavefront's tiles: wave, wave + waves, ... (the host launches enough wavefronts for
+  // kFusedMaxTilesPerWave to cover the message)
 
-  // 1. copy-in
-  VecU<DT> mine;
-  mine.v = (u32x4){0u, 0u, 0u, 0u};
-  if (whole) {
-    mine.v = __builtin_nontemporal_load(&((const u32x4_unaligned*)a.in)[v]);
-  } else if (part) {
-    for (uint32_t e = 0; e < a.tail; ++e) vec_set<DT>(mine, (int)e, ((const S*)a.in)[v * VE + e]);
+  // 1. copy-in of all of them
+  VecU<DT> mine[kFusedMaxTilesPerWave];
+#pragma unroll
+  for (int j = 0; j < kFusedMaxTilesPerWave; ++j) {
+    const uint32_t tile = wave + (uint32_t)j * waves;
+    if (tile >= a.tiles) break;
+    const uint64_t v = (uint64_t)tile * kWave + lane;
+    const bool whole = v < a.nvec;
+    const bool part = v == a.nvec && a.tail != 0;  // the one vector that is not whole
+    mine[j].v = (u32x4){0u, 0u, 0u, 0u};
+    if (whole) {
+      mine[j].v = __builtin_nontemporal_load(&((const u32x4_unaligned*)a.in)[v]);
+    } else if (part) {
+      for (uint32_t e = 0; e < a.tail; ++e) vec_set<DT>(mine[j], (int)e, ((const S*)a.in)[v * VE + e]);
+    }
+    if (whole || part) store_vec_coherent(&((u32x4*)a.stage[a.rank])[v], mine[j].v);  // written through
   }
-  if (whole || part) store_vec_coherent(&((u32x4*)a.stage[a.rank])[v], mine.v);  // written through
-  // 2. publish: the tile has reached memory before the flag can be seen
+  // 2. publish: the tiles have reached memory before their flags can be seen
   wait_own_stores();
-  if (lane == 0) __hip_atomic_store(a.flag[a.rank] + tile, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  // 3. wait for the same tile of every peer
-  bool ok = true;
-  if (lane < a.n && lane != a.rank) {
-    ok = wait_flag32(a.flag[lane] + tile, a.epoch, a.limit_ticks);
-    if (!ok) report_late(a.status, lane, a.epoch);
+#pragma unroll
+  for (int j = 0; j < kFusedMaxTilesPerWave; ++j) {
+    const uint32_t tile = wave + (uint32_t)j * waves;
+    if (tile >= a.tiles) break;
+    if (lane == 0) __hip_atomic_store(a.flag[a.rank] + tile, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the loads below stay below the wait
-  // a tile whose peers did not arrive is left alone (the failure is reported through `status`)
-  if (__builtin_amdgcn_ballot_w64(!ok) != 0) return;
-  if (!(whole || part)) return;
+#pragma unroll
+  for (int j = 0; j < kFusedMaxTilesPerWave; ++j) {
+    const uint32_t tile = wave + (uint32_t)j * waves;
+    if (tile >= a.tiles) break;
+    const uint64_t v = (uint64_t)tile * kWave + lane;
+    const bool whole = v < a.nvec;
+    const bool part = v == a.nvec && a.tail != 0;
+    // 3. wait for the same tile of every peer
+    bool ok = true;
+    if (lane < a.n && lane != a.rank) {
+      ok = wait_flag32(a.flag[lane] + tile, a.epoch, a.limit_ticks);
+      if (!ok) report_late(a.status, lane, a.epoch);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the loads below stay below the wait
+    // tiles whose peers did not arrive are left alone (the failure is reported through `status`)
+    if (__builtin_amdgcn_ballot_w64(!ok) != 0) return;
+    if (!(whole || part)) continue;
 
-  // 4. the N-peer reduction, ascending rank order; all peer loads are issued before the first add
-  VecU<DT> x[kFusedRanks];
+    // 4. the N-peer reduction, ascending rank order; all peer loads are issued before the first add
+    VecU<DT> x[kFusedRanks];
 #pragma unroll
-  for (int k = 0; k < kFusedRanks; ++k) {
-    if (k < a.n) {
-      if (k == a.rank) x[k].v = mine.v;
-      else x[k].v = load_vec_coherent(&((const u32x4*)a.stage[k])[v]);  // past the caches: written by another rank just now
+    for (int k = 0; k < kFusedRanks; ++k) {
+      if (k < a.n) {
+        if (k == a.rank) x[k].v = mine[j].v;
+        else x[k].v = load_vec_coherent(&((const u32x4*)a.stage[k])[v]);  // past the caches: written by another rank just now
+      }
     }
-  }
-  A acc[VE];
+    A acc[VE];
 #pragma unroll
-  for (int e = 0; e < VE; ++e) acc[e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x[0], e)));
+    for (int e = 0; e < VE; ++e) acc[e] = chain_first<DT, OP>(Elem<DT>::load(vec_get<DT>(x[0], e)));
 #pragma unroll
-  for (int k = 1; k < kFusedRanks; ++k) {
-    if (k < a.n) {
+    for (int k = 1; k < kFusedRanks; ++k) {
+      if (k < a.n) {
 #pragma unroll
-      for (int e = 0; e < VE; ++e) acc[e] = chain_next<DT, OP>(acc[e], Elem<DT>::load(vec_get<DT>(x[k], e)));
+        for (int e = 0; e < VE; ++e) acc[e] = chain_next<DT, OP>(acc[e], Elem<DT>::load(vec_get<DT>(x[k], e)));
+      }
     }
-  }
-  VecU<DT> r;
-  r.v = (u32x4){0u, 0u, 0u, 0u};
+    VecU<DT> r;
+    r.v = (u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < VE; ++e) vec_set<DT>(r, e, Elem<DT>::store(chain_last<DT, OP>(acc[e], a.n)));
-  if (whole) {
-    ((u32x4_unaligned*)a.out)[v] = r.v;
-  } else {
-    for (uint32_t e = 0; e < a.tail; ++e) ((S*)a.out)[v * VE + e] = vec_get<DT>(r, (int)e);
+    for (int e = 0; e < VE; ++e) vec_set<DT>(r, e, Elem<DT>::store(chain_last<DT, OP>(acc[e], a.n)));
+    if (whole) {
+      ((u32x4_unaligned*)a.out)[v] = r.v;
+    } else {
+      for (uint32_t e = 0; e < a.tail; ++e) ((S*)a.out)[v * VE + e] = vec_get<DT>(r, (int)e);
+    }
   }
 }
 

@@ -188,17 +188,17 @@ hipError_t launch_any(const ReduceArgs& a, int dtype, int op, const Geometry& g,
   }
 }
 
-hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned tiles, hipStream_t s) {
+hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned groups, hipStream_t s) {
   switch (dtype) {
-    case MCCL_U8: return mccl_launch_fused_dt0(&a, op, tiles, s);
-    case MCCL_I8: return mccl_launch_fused_dt1(&a, op, tiles, s);
-    case MCCL_I16: return mccl_launch_fused_dt2(&a, op, tiles, s);
-    case MCCL_I32: return mccl_launch_fused_dt3(&a, op, tiles, s);
-    case MCCL_I64: return mccl_launch_fused_dt4(&a, op, tiles, s);
-    case MCCL_F16: return mccl_launch_fused_dt5(&a, op, tiles, s);
-    case MCCL_F32: return mccl_launch_fused_dt6(&a, op, tiles, s);
-    case MCCL_F64: return mccl_launch_fused_dt7(&a, op, tiles, s);
-    case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, tiles, s);
+    case MCCL_U8: return mccl_launch_fused_dt0(&a, op, groups, s);
+    case MCCL_I8: return mccl_launch_fused_dt1(&a, op, groups, s);
+    case MCCL_I16: return mccl_launch_fused_dt2(&a, op, groups, s);
+    case MCCL_I32: return mccl_launch_fused_dt3(&a, op, groups, s);
+    case MCCL_I64: return mccl_launch_fused_dt4(&a, op, groups, s);
+    case MCCL_F16: return mccl_launch_fused_dt5(&a, op, groups, s);
+    case MCCL_F32: return mccl_launch_fused_dt6(&a, op, groups, s);
+    case MCCL_F64: return mccl_launch_fused_dt7(&a, op, groups, s);
+    case MCCL_BF16: return mccl_launch_fused_dt8(&a, op, groups, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -567,7 +567,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 142; }
+int mccl_version(void) { return 143; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -727,7 +727,7 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
 
 int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
                          void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
-                         uint64_t timeout_us, void* status, void* stream) {
+                         uint64_t timeout_us, void* status, unsigned max_compute_units, void* stream) {
   int rc = check_reduce_args_no_ptr(n, dtype, op);
   if (rc != MCCL_OK) return rc;
   if (n > MCCL_FUSED_MAX_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "the one-launch allreduce takes at most %d ranks, got %d", MCCL_FUSED_MAX_RANKS, n);
@@ -751,6 +751,15 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
   const size_t nvec = count / ve;
   const size_t tiles = (nvec + (count % ve ? 1 : 0) + kWave - 1) / kWave;
   if (tiles > kMaxGridX) return fail(MCCL_ERR_INVALID_ARG, "message too large for the one-launch allreduce");
+  // one wavefront per tile, sixteen to a workgroup; with a limit on the workgroups a wavefront
+  // takes up to kFusedMaxTilesPerWave tiles
+  size_t groups = (tiles + kFusedWavesPerGroup - 1) / kFusedWavesPerGroup;
+  if (max_compute_units && groups > max_compute_units) {
+    groups = max_compute_units;
+    if (tiles > groups * kFusedWavesPerGroup * kFusedMaxTilesPerWave)
+      return fail(MCCL_ERR_INVALID_ARG, "a one-launch allreduce on %u compute units takes at most %zu bytes, got %zu", max_compute_units,
+                  groups * kFusedWavesPerGroup * kFusedMaxTilesPerWave * (size_t)MCCL_FUSED_TILE_BYTES, count * es);
+  }
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   a.in = (const char*)in;
@@ -767,7 +776,7 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
   a.tiles = (uint32_t)tiles;
   a.n = n;
   a.rank = rank;
-  hipError_t e = launch_fused_any(a, dtype, op, (unsigned)tiles, (hipStream_t)stream);
+  hipError_t e = launch_fused_any(a, dtype, op, (unsigned)groups, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "fused allreduce launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
@@ -878,15 +887,9 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   }
   const XShape shape = xrank_shape(chunks, sync);  // (a copy gains nothing from more wavefronts than its share, waits or not)
   const unsigned grid = shape.groups;
-  if (flags & ~(MCCL_COPY_SHARED_SOURCES | MCCL_COPY_PUBLISH)) return fail(MCCL_ERR_INVALID_ARG, "unknown copy flags 0x%x", flags);
-  if (flags & MCCL_COPY_PUBLISH) {
-    if (a.sync.done_epoch == 0) return fail(MCCL_ERR_INVALID_ARG, "MCCL_COPY_PUBLISH announces the copy with the closing epoch: done_epoch must not be 0");
-    if (shape.packed) return fail(MCCL_ERR_INVALID_ARG, "MCCL_COPY_PUBLISH waits with one wavefront: max_compute_units does not apply");
-    hipLaunchKernelGGL(copy_segments_publish_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
-  } else {
-    if (shape.packed) hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
-    else hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
-  }
+  if (flags & ~MCCL_COPY_SHARED_SOURCES) return fail(MCCL_ERR_INVALID_ARG, "unknown copy flags 0x%x", flags);
+  if (shape.packed) hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;

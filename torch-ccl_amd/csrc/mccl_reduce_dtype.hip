@@ -25,7 +25,7 @@ extern "C" hipError_t MCCL_PASTE(mccl_launch_reduce_dt, MCCL_REDUCE_DT)(MCCL_RED
 }
 
 extern "C" hipError_t MCCL_PASTE(mccl_launch_fused_dt, MCCL_REDUCE_DT)(MCCL_FUSED_ENTRY_ARGS) {
-  return launch_fused_dtype<MCCL_REDUCE_DT>(*static_cast<const FusedArgs*>(fused_args), op, tiles, stream);
+  return launch_fused_dtype<MCCL_REDUCE_DT>(*static_cast<const FusedArgs*>(fused_args), op, groups, stream);
 }
 
 extern "C" hipError_t MCCL_PASTE(mccl_launch_xrank_dt, MCCL_REDUCE_DT)(MCCL_XRANK_ENTRY_ARGS) {

@@ -51,9 +51,10 @@ constexpr int kTwoShotMinRanks = 4;
 // Device-synchronised groups: allreduces of at most this many bytes (and at most
 // MCCL_FUSED_MAX_RANKS ranks) are one launch of mccl_allreduce_fused on the caller's stream.
 constexpr size_t kFusedMaxBytes = 1u << 20;
-// One workgroup of the one-launch small allreduce covers 16 KiB and waits on one compute unit:
-// 128 of them over all ranks (8 ranks x 256 KiB) leave half of the 256 compute units free.
-constexpr size_t kFusedCompactMaxBytesAllRanks = 128u * (16u << 10);
+// What a workgroup of the one-launch small allreduce covers at most (sixteen wavefronts, four
+// 1 KiB tiles each) when the launch is limited to a number of compute units.
+constexpr size_t kFusedBytesPerComputeUnit = 16u * 4u * MCCL_FUSED_TILE_BYTES;
+constexpr unsigned kComputeUnits = 256;  // of an MI355X
 // Tensors of at least this many bytes are offered to the peers in place (zero-copy) instead of
 // being staged; an allocation must stay below 2 GiB to be shared between processes.
 constexpr size_t kZeroCopyMinBytes = 1u << 20;
@@ -1109,40 +1110,19 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     last_title_ = plan.title;
     last_seq_ = seq + 1;
     last_path_ = "one launch, fused";
-    // (without MCCL_PG_SYNC=kernel only as long as all ranks' waiting workgroups together hold at
-    // most half of the GPU's compute units: one workgroup per 16 KiB of message and rank)
+    // On this rank's share of the compute units that all ranks' waiting launches may hold together
+    // (a share takes 64 KiB per compute unit).  With MCCL_PG_SYNC=kernel the share is one workgroup
+    // per compute unit and rank, half of what the GPU holds: a wavefront of this kernel waits for
+    // the same tile of every peer, so all of a late rank's workgroups must still find room beside
+    // the waiting ones, and a launch per 16 KiB (8 ranks x 1 MiB: 512 workgroups, exactly what
+    // fits when nothing else runs) leaves none to spare.
+    const unsigned fused_units = std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_);
     if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS &&
-        (waits_in_data_kernels_ || plan.fused_count * mccl_dtype_size(plan.fused_dtype) * (size_t)size_ <= kFusedCompactMaxBytesAllRanks)) {
+        plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= (size_t)fused_units * kFusedBytesPerComputeUnit) {
       const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
       MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
                                       fused_stage_[slot].data(), fused_flags_[slot].data(), size_, rank_,
-                                      (uint32_t)(seq + 1), limit_us, status_dev_, s));
-      if (timed) phase_us_[3].push_back((float)us_since(t0));
-      return;
-    }
-    if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS) {
-      // The same small allreduce with at most one waiting wavefront per rank on the GPU: the
-      // copy-in writes this rank's staging buffer through to memory and its last workgroup
-      // announces it and waits for the peers' announcements; the reduction behind it reads all
-      // staging buffers.  Two launches, no rendezvous of the host threads, nothing exported.
-      last_path_ = "announcing copy-in, reduce";
-      if (verbose_) {
-        std::ostringstream os;
-        os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
-        std::cout << os.str() << std::endl;
-      }
-      mccl_segment_t seg{plan.fused_ptr, fused_stage_[slot][(size_t)rank_], plan.fused_count * mccl_dtype_size(plan.fused_dtype)};
-      mccl_xsync_t sync{};
-      sync.words = bar_flags_.data();
-      sync.n = size_;
-      sync.rank = rank_;
-      sync.done_epoch = epoch + 1;
-      sync.done_counter = done_counter_;
-      sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
-      sync.status = status_dev_;
-      MCCL_CHECK(mccl_copy_segments_sync(&seg, 1, MCCL_COPY_PUBLISH, &sync, s));
-      std::vector<const void*> in(fused_stage_[slot].begin(), fused_stage_[slot].end());
-      MCCL_CHECK(mccl_reduce_n(in.data(), size_, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op, MCCL_VARIANT_AUTO, s));
+                                      (uint32_t)(seq + 1), limit_us, status_dev_, fused_units, s));
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }

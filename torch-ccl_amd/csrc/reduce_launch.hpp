@@ -76,12 +76,12 @@ hipError_t launch_dtype(const ReduceArgs& a, int op, const Geometry& g, int njob
   }
 }
 
-// The one-launch small allreduce: one wavefront per 1 KiB tile, sixteen to a workgroup.
+// The one-launch small allreduce: `groups` workgroups of up to sixteen wavefronts.
 template <int DT>
-hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned tiles, hipStream_t s) {
-  if (tiles < 1) return hipErrorInvalidValue;
-  const unsigned waves = tiles < (unsigned)kFusedWavesPerGroup ? tiles : (unsigned)kFusedWavesPerGroup;
-  const dim3 grid((tiles + waves - 1) / waves, 1, 1), block(kWave * waves);
+hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned groups, hipStream_t s) {
+  if (groups < 1 || a.tiles < 1) return hipErrorInvalidValue;
+  const unsigned waves = a.tiles < (unsigned)kFusedWavesPerGroup ? a.tiles : (unsigned)kFusedWavesPerGroup;
+  const dim3 grid(groups, 1, 1), block(kWave * waves);
   switch (op) {
     case MCCL_SUM: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_SUM>), grid, block, 0, s, a); break;
     case MCCL_PROD: hipLaunchKernelGGL((allreduce_fused_kernel<DT, MCCL_PROD>), grid, block, 0, s, a); break;
@@ -146,7 +146,7 @@ __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt7(MCCL_RED
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_reduce_dt8(MCCL_REDUCE_ENTRY_ARGS);
 }
 // `fused_args` points at a FusedArgs.
-#define MCCL_FUSED_ENTRY_ARGS const void *fused_args, int op, unsigned tiles, hipStream_t stream
+#define MCCL_FUSED_ENTRY_ARGS const void *fused_args, int op, unsigned groups, hipStream_t stream
 extern "C" {
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt0(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt1(MCCL_FUSED_ENTRY_ARGS);

@@ -22,7 +22,7 @@ VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
  TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
  TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS, TUNE_COPY_VECTORS_PER_LANE, TUNE_COPY_STREAM_STORES,
  TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU, TUNE_XRANK_CACHED_LOADS) = range(13)
-COPY_SHARED_SOURCES, COPY_PUBLISH = 1, 2  # flags of mccl_copy_segments_sync
+COPY_SHARED_SOURCES = 1  # flag of mccl_copy_segments_sync
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
@@ -85,7 +85,7 @@ def lib():
     L.mccl_moe_dispatch_n.argtypes = [vp, vp, vp, vp, i32, vp, sz, vp]
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
-    L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, vp]
+    L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
     L.mccl_reduce_sync.argtypes = [vp, vp, sz, i32, i32, vp, vp]
     L.mccl_allreduce_sync.argtypes = [vp, sz, i32, i32, vp, vp]
