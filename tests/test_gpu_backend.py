@@ -219,3 +219,14 @@ def test_env_switches(monkeypatch, same_stream, blocking):
 @pytest.mark.parametrize("world", [2, 4])
 def test_ddp_and_fsdp_style_callers(world):
     _spawn(world, "ddp")
+
+
+def test_verbose_logs_one_line_per_collective(monkeypatch, capfd):
+    """ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE=1: every collective says which way it took, the
+    one-launch small allreduce included."""
+    monkeypatch.setenv("ONECCL_BINDINGS_FOR_PYTORCH_ENV_VERBOSE", "1")
+    _spawn(2, "env")
+    out = capfd.readouterr().out
+    assert "oneccl_bindings_for_pytorch::allreduce [0/2#" in out and "oneccl_bindings_for_pytorch::allreduce [1/2#" in out, out[-2000:]
+    assert "one launch" in out or "peers read in place" in out, out[-2000:]
+

@@ -1110,6 +1110,12 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     last_title_ = plan.title;
     last_seq_ = seq + 1;
     last_path_ = "one launch, fused";
+    auto say_path = [&] {
+      if (!verbose_) return;
+      std::ostringstream os;
+      os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
+      std::cout << os.str() << std::endl;
+    };
     // On this rank's share of the compute units that all ranks' waiting launches may hold together
     // (a share takes 64 KiB per compute unit).  With MCCL_PG_SYNC=kernel the share is one workgroup
     // per compute unit and rank, half of what the GPU holds: a wavefront of this kernel waits for
@@ -1119,6 +1125,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     const unsigned fused_units = std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_);
     if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS &&
         plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= (size_t)fused_units * kFusedBytesPerComputeUnit) {
+      say_path();
       const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
       MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
                                       fused_stage_[slot].data(), fused_flags_[slot].data(), size_, rank_,
@@ -1184,11 +1191,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     last_path_ = one_launch ? (zero_copy ? "one launch, peers read in place" : "copy-in and one launch")
                             : zero_copy ? "barrier kernel, peers read in place"
                                         : candidate ? "staged: a rank cannot share its tensor" : "staged";
-    if (verbose_) {
-      std::ostringstream os;
-      os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
-      std::cout << os.str() << std::endl;
-    }
+    say_path();
     if (one_launch) {
       if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
       mccl_xsync_t sync{};
