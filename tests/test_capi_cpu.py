@@ -209,3 +209,29 @@ def test_placement_check_needs_no_device(mccl):
     assert check([66 * MiB] * 7, 64 * MiB) == 0                # small messages have not shown the effect
     assert check([GiB + 2 * MiB] * 7, 64 * MiB) == 0
     assert L.mccl_placement_check(None, 8, GiB) == 0
+
+
+def test_ctypes_structures_match_the_header(mccl, tmp_path):
+    """The ctypes mirrors of the header's structures have the compiler's size and field offsets
+    (a plain-C program that includes include/mccl.h prints them)."""
+    import subprocess
+    from torch_ccl_amd import capi
+    layouts = {"mccl_xsync_t": (capi.XSync, [f[0] for f in capi.XSync._fields_]),
+               "mccl_segment_t": (capi.Segment, [f[0] for f in capi.Segment._fields_])}
+    lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "mccl.h"', 'int main(void) {']
+    for cname, (_, fields) in layouts.items():
+        lines.append('  printf("%s %%zu", sizeof(%s));' % (cname, cname))
+        for f in fields:
+            lines.append('  printf(" %%zu", offsetof(%s, %s));' % (cname, f))
+        lines.append('  printf("\\n");')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    for line in filter(None, out):
+        cname, size, *offsets = line.split()
+        ctype, fields = layouts[cname]
+        assert ctypes.sizeof(ctype) == int(size), cname
+        assert [getattr(ctype, f).offset for f in fields] == [int(o) for o in offsets], cname
