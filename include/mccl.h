@@ -258,6 +258,15 @@ typedef struct {
 int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync,
                             void* stream);
 
+/* allgather as pushes (ccl::allgatherv, src/gpu/dpcpp_ccl.cpp:1176-1182; stores into the peers'
+ * buffers as in the gather step of src/gpu/allreduce.h:470-487): this rank's `bytes` at src are
+ * written to dst[0..ndst) -- where this rank's contribution belongs in every rank's output, peers'
+ * outputs through writable mappings -- read once and written through, so that a rank that has seen
+ * done_epoch finds all contributions in its output.  1 to 8 destinations, any alignment; src must
+ * not overlap a destination.  With both epochs 0 it is a plain one-to-many copy. */
+int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, const mccl_xsync_t* sync,
+                     void* stream);
+
 /* mccl_reduce_n whose inputs are peers' buffers (in[r]: rank r's contribution at this rank's
  * slice): the shard reduction of reduce_scatter (ccl::reduce_scatter, src/gpu/dpcpp_ccl.cpp:1002-1008)
  * in one launch.  Same arithmetic and bits as mccl_reduce_n; out must not overlap an input. */

@@ -595,6 +595,13 @@ def zero_copy_cases(pg, rank, world):
         out = torch.empty(world * m * 4, dtype=dtype, device=DEV)
         pg._allgather_base(out, view_of(host[rank], pad)).wait()
         assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather", dtype, m)
+        # the output as a view at an odd offset of a larger allocation, which the peers write into:
+        # the bytes either side of it stay as they were
+        big = torch.full((world * m * 4 + 2 * pad + 64,), 7, dtype=dtype, device=DEV)
+        out = big[pad + 3:pad + 3 + world * m * 4]
+        pg._allgather_base(out, view_of(host[rank], pad)).wait()
+        assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather into a view", dtype, m)
+        assert bool((big[:pad + 3] == 7).all()) and bool((big[pad + 3 + world * m * 4:] == 7).all()), ("allgather wrote outside its output", dtype)
         root = m % world
         src = rank_buffer(m * 4 + 3, dtype, root, seed=93)
         t = view_of(src if rank == root else torch.zeros_like(src), pad)

@@ -240,6 +240,19 @@ def xrank_case(rank, world, queues, barrier):
         capi.check(L.mccl_copy_segments_sync(arr, len(segs), i & 1, ctypes.byref(sy), stream))  # both load flavours
         want = O.alltoallv([to_carrier(h) for h in host], S, row)[rank]
         checks.append((out, want, ("copy_segments_sync", row, i)))
+    # allgather as pushes: every rank writes its contribution into slice `rank` of every rank's shared
+    # buffer; the clone behind the call reads what the peers wrote.  Odd lengths and offsets included.
+    for i, (nbytes, src_off, dst_off) in enumerate([(1 << 20, 0, 0), (70001, 3, 5), (15, 1, 0), (16, 0, 16), (1, 0, 7), ((2 << 20) + 48, 16, 32),
+                                                    (1024, 0, 0), (0, 0, 0), (333333, 8, 1)]):
+        host = [rank_buffer(max(nbytes, 1), torch.uint8, r, seed=700 + i)[:nbytes] for r in range(world)]
+        own = torch.empty(nbytes + 64, dtype=torch.uint8, device=DEV)[src_off:src_off + nbytes]
+        own.copy_(host[rank])
+        dst = capi.ptr_table([shared[r][0].data_ptr() + dst_off + rank * nbytes for r in range(world)])
+        sy = sync()
+        capi.check(L.mccl_fanout_sync(own.data_ptr(), dst, world, nbytes, ctypes.byref(sy), stream))
+        got = shared_in[dst_off:dst_off + world * nbytes].clone()
+        want = O.allgather([to_carrier(h) for h in host]) if nbytes else np.zeros(0, np.uint8)
+        checks.append((got, want, ("fanout_sync", nbytes, src_off, dst_off)))
     torch.cuda.synchronize()
     assert st.tolist() == [0, 0], st.tolist()
     assert not counter.cpu().any()  # every counter is back at zero

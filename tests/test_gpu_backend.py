@@ -159,6 +159,13 @@ def test_zero_copy_with_barrier_kernels_instead_of_one_launch(monkeypatch):
     _spawn(4, "zero_copy")
 
 
+def test_all_gather_with_pulls_instead_of_pushes(monkeypatch):
+    """MCCL_PG_ALLGATHER_PUSH=0: all_gather_into_tensor offers the inputs and every rank pulls (what
+    outputs too large to be shared use) instead of writing into the peers' outputs: same bits."""
+    monkeypatch.setenv("MCCL_PG_ALLGATHER_PUSH", "0")
+    _spawn(4, "zero_copy")
+
+
 def test_staged_when_zero_copy_is_switched_off(monkeypatch):
     monkeypatch.setenv("MCCL_PG_ZERO_COPY", "0")
     _spawn(4, "oracle")

@@ -108,4 +108,63 @@ __global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const S
   xsync_end(a.sync, gridDim.x);
 }
 
+// allgather as pushes: this rank's contribution goes into every rank's output in one pass -- read
+// once, written ndst times -- where pulls make every rank read all contributions (W reads of every
+// byte over the group, served by the memory-side cache only while the ranks keep in step).  The
+// peers' outputs are written through, like the shards of the in-place allreduce, so that the closing
+// epoch tells their owners that the data is there.  Any alignment: vectors are 16 bytes of the
+// message, wherever source and destinations start; the bytes after the last vector go one per lane.
+struct FanoutArgs {
+  const char* src;
+  char* dst[kLeanSyncRanks];
+  uint32_t nvec;     // whole 16-byte vectors
+  uint32_t tail;     // bytes after them (< 16)
+  uint32_t tiles;    // 1 KiB tiles that cover the vectors
+  uint32_t aligned;  // every destination is 16-byte aligned
+  int ndst;
+  XSync sync;
+};
+
+__device__ __forceinline__ u32x4 fanout_load(const FanoutArgs& a, uint32_t tile, uint32_t lane) {
+  const uint32_t v = tile * kWave + lane;  // the host keeps tiles * 64 below 2^32
+  if (v >= a.nvec) return (u32x4){0u, 0u, 0u, 0u};
+  return __builtin_nontemporal_load(&((const u32x4_unaligned*)a.src)[v]);
+}
+
+__device__ __forceinline__ void fanout_store(const FanoutArgs& a, uint32_t tile, uint32_t lane, u32x4 x) {
+  if (tile * kWave + lane >= a.nvec) return;
+#pragma unroll
+  for (int k = 0; k < kLeanSyncRanks; ++k) {
+    if (k < a.ndst) {
+      char* tb = a.dst[k] + (size_t)tile * (kWave * 16u);  // uniform
+      if (a.aligned) store_tile_through(tb, lane * 16u, x);
+      else store_vec_through(tb + lane * 16u, x);
+    }
+  }
+}
+
+template <int WPG>
+__global__ __launch_bounds__(kWave * WPG) void fanout_sync_kernel(const FanoutArgs a) {
+  const Wave w = this_wave<WPG>();
+  if (xsync_begin(a.sync)) {
+    const uint32_t T = a.tiles, G = w.count;
+    for (uint32_t t0 = w.index; t0 < T; t0 += 2 * G) {  // two tiles' loads in flight
+      const uint32_t t1 = t0 + G;
+      const u32x4 x0 = fanout_load(a, t0, w.lane);
+      u32x4 x1 = (u32x4){0u, 0u, 0u, 0u};
+      if (t1 < T) x1 = fanout_load(a, t1, w.lane);
+      fanout_store(a, t0, w.lane, x0);
+      if (t1 < T) fanout_store(a, t1, w.lane, x1);
+    }
+    if (a.tail && w.index == w.count - 1 && w.lane < a.tail) {
+      const size_t i = (size_t)a.nvec * 16u + w.lane;
+      const unsigned char b = (unsigned char)a.src[i];
+#pragma unroll
+      for (int k = 0; k < kLeanSyncRanks; ++k)
+        if (k < a.ndst) __hip_atomic_store((unsigned char*)a.dst[k] + i, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+  xsync_end(a.sync, gridDim.x);
+}
+
 }  // namespace

@@ -567,7 +567,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 143; }
+int mccl_version(void) { return 144; }
 
 const char* mccl_last_error(void) { return g_err; }
 
@@ -892,6 +892,39 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   else hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, const mccl_xsync_t* sync, void* stream) {
+  FanoutArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  if (ndst < 1 || ndst > kLeanSyncRanks) return fail(MCCL_ERR_UNSUPPORTED, "a push takes 1 to %d destinations, got %d", kLeanSyncRanks, ndst);
+  if (!dst) return fail(MCCL_ERR_INVALID_ARG, "destination table is null");
+  if (bytes / 16 > 0xf0000000ull) return fail(MCCL_ERR_INVALID_ARG, "message too large for one push");
+  a.ndst = ndst;
+  a.aligned = 1;
+  if (bytes) {
+    if (!src) return fail(MCCL_ERR_INVALID_ARG, "source pointer is null");
+    for (int k = 0; k < ndst; ++k) {
+      if (!dst[k]) return fail(MCCL_ERR_INVALID_ARG, "destination pointer %d is null", k);
+      const uintptr_t s0 = (uintptr_t)src, d0 = (uintptr_t)dst[k];
+      if (s0 < d0 + bytes && d0 < s0 + bytes) return fail(MCCL_ERR_INVALID_ARG, "destination %d overlaps the source", k);
+      if (d0 & 15u) a.aligned = 0;
+      a.dst[k] = (char*)dst[k];
+    }
+    a.src = (const char*)src;
+    a.nvec = (uint32_t)(bytes / 16);
+    a.tail = (uint32_t)(bytes % 16);
+    a.tiles = (uint32_t)((bytes / 16 + kWave - 1) / kWave);
+  }
+  // (the last wavefront takes the tail: a launch of at least one)
+  const XShape shape = xrank_shape(a.tiles, sync, a.sync.ready_epoch != 0);
+  if (shape.packed) hipLaunchKernelGGL(fanout_sync_kernel<kPackedWaves>, dim3(shape.groups), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(fanout_sync_kernel<1>, dim3(shape.groups), dim3(kWave), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "push kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
 

@@ -360,6 +360,7 @@ class ProcessGroupCCL : public c10d::Backend {
   // all_gather up to 1 MiB per rank (8 MiB written), reduce_scatter and the in-place allreduce up
   // to 32 MiB (16 MiB: 83-104 against 106-141 us).  MCCL_PG_COMPACT_MAX_BYTES overrides (0: never).
   size_t compact_max_ = 16u << 20;
+  bool allgather_push_ = true;  // MCCL_PG_ALLGATHER_PUSH != 0: all_gather_into_tensor writes into the peers' outputs
   unsigned waiting_cus_ = 128;  // what all ranks' waiting launches may hold together (MCCL_PG_WAITING_COMPUTE_UNITS)
   bool distinct_pids_ = false;          // every rank is a process of its own
   const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
