@@ -262,8 +262,9 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
  * buffers as in the gather step of src/gpu/allreduce.h:470-487): this rank's `bytes` at src are
  * written to dst[0..ndst) -- where this rank's contribution belongs in every rank's output, peers'
  * outputs through writable mappings -- read once and written through, so that a rank that has seen
- * done_epoch finds all contributions in its output.  1 to 8 destinations, any alignment; src must
- * not overlap a destination.  With both epochs 0 it is a plain one-to-many copy. */
+ * done_epoch finds all contributions in its output.  1 to 8 destinations, any alignment; a
+ * destination may be src itself (an allgather in place: nothing to copy there) but must not overlap
+ * it otherwise.  With both epochs 0 it is a plain one-to-many copy. */
 int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, const mccl_xsync_t* sync,
                      void* stream);
 

@@ -183,6 +183,11 @@ def oracle_cases(pg, rank, world):
         out = torch.empty(world * m, dtype=dtype, device=DEV)
         pg._allgather_base(out, host[rank].to(DEV)).wait()
         assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather", dtype)
+        out.zero_()
+        n_in = host[rank].numel()
+        out[rank * n_in:(rank + 1) * n_in].copy_(host[rank])
+        pg._allgather_base(out, out[rank * n_in:(rank + 1) * n_in]).wait()  # in place
+        assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather in place", dtype)
     # two-shot path (>= 4 MiB, >= 4 ranks): ragged counts, every dtype width, same bits as the oracle
     for dtype, count in ((torch.bfloat16, (4 << 20) + 777), (torch.float32, (2 << 20) + 5), (torch.int8, (8 << 20) + 3),
                          (torch.float64, (1 << 20) + 1)):
@@ -602,6 +607,11 @@ def zero_copy_cases(pg, rank, world):
         pg._allgather_base(out, view_of(host[rank], pad)).wait()
         assert np.array_equal(bits(out), np.concatenate([bits(h) for h in host])), ("allgather into a view", dtype, m)
         assert bool((big[:pad + 3] == 7).all()) and bool((big[pad + 3 + world * m * 4:] == 7).all()), ("allgather wrote outside its output", dtype)
+        # in place, as FSDP calls it: the input is this rank's slice of the output
+        full = torch.zeros(world * m * 4, dtype=dtype, device=DEV)
+        full[rank * m * 4:(rank + 1) * m * 4].copy_(host[rank])
+        pg._allgather_base(full, full[rank * m * 4:(rank + 1) * m * 4]).wait()
+        assert np.array_equal(bits(full), np.concatenate([bits(h) for h in host])), ("allgather in place", dtype, m)
         root = m % world
         src = rank_buffer(m * 4 + 3, dtype, root, seed=93)
         t = view_of(src if rank == root else torch.zeros_like(src), pad)

@@ -907,13 +907,16 @@ int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, 
   a.aligned = 1;
   if (bytes) {
     if (!src) return fail(MCCL_ERR_INVALID_ARG, "source pointer is null");
+    int m = 0;
     for (int k = 0; k < ndst; ++k) {
       if (!dst[k]) return fail(MCCL_ERR_INVALID_ARG, "destination pointer %d is null", k);
       const uintptr_t s0 = (uintptr_t)src, d0 = (uintptr_t)dst[k];
-      if (s0 < d0 + bytes && d0 < s0 + bytes) return fail(MCCL_ERR_INVALID_ARG, "destination %d overlaps the source", k);
+      if (s0 == d0) continue;  // in place: this rank's contribution already sits in its own output
+      if (s0 < d0 + bytes && d0 < s0 + bytes) return fail(MCCL_ERR_INVALID_ARG, "destination %d partially overlaps the source", k);
       if (d0 & 15u) a.aligned = 0;
-      a.dst[k] = (char*)dst[k];
+      a.dst[m++] = (char*)dst[k];
     }
+    a.ndst = m;
     a.src = (const char*)src;
     a.nvec = (uint32_t)(bytes / 16);
     a.tail = (uint32_t)(bytes % 16);
