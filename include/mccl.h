@@ -270,7 +270,9 @@ int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, 
 
 /* mccl_reduce_n whose inputs are peers' buffers (in[r]: rank r's contribution at this rank's
  * slice): the shard reduction of reduce_scatter (ccl::reduce_scatter, src/gpu/dpcpp_ccl.cpp:1002-1008)
- * in one launch.  Same arithmetic and bits as mccl_reduce_n; out must not overlap an input. */
+ * in one launch.  Same arithmetic and bits as mccl_reduce_n; out may be exactly one of the inputs
+ * (a reduce_scatter in place: the output is this rank's slice of its own input, which no other rank
+ * reads), and must not overlap an input otherwise. */
 int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, int op,
                      const mccl_xsync_t* sync, void* stream);
 

@@ -596,6 +596,10 @@ def zero_copy_cases(pg, rank, world):
         pg._reduce_scatter_base(out, view_of(host[rank], pad)).wait()
         want = O.reduce_scatter([to_carrier(h) for h in host], code, O.SUM, shard_first=rank, shard_num=1)[0]
         assert np.array_equal(bits(out), bits_np(want)), ("reduce_scatter", dtype, m)
+        # in place: the output is this rank's slice of its input, which no other rank reads
+        x = view_of(host[rank], pad)
+        pg._reduce_scatter_base(x[rank * m:(rank + 1) * m], x).wait()
+        assert np.array_equal(bits(x[rank * m:(rank + 1) * m]), bits_np(want)), ("reduce_scatter in place", dtype, m)
         host = [rank_buffer(m * 4, dtype, r, seed=92) for r in range(world)]
         out = torch.empty(world * m * 4, dtype=dtype, device=DEV)
         pg._allgather_base(out, view_of(host[rank], pad)).wait()
