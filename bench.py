@@ -232,6 +232,12 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     res["c5_all_to_all_single_448MiB_bf16"] = timed(
         lambda: dist.all_to_all_single(a_out, a_in, S[:, rank].tolist(), S[rank].tolist()), iters=5, warm=1)
     del a_in, a_out
+    # all_gather_into_tensor of 64 MiB per rank (an FSDP parameter gather): every rank writes its shard
+    # into all eight outputs
+    part = torch.empty(33_554_432, dtype=torch.bfloat16, device="cuda:0").normal_()
+    full = torch.empty(33_554_432 * world, dtype=torch.bfloat16, device="cuda:0")
+    res["all_gather_into_tensor_64MiB_bf16"] = timed(lambda: dist.all_gather_into_tensor(full, part), iters=5, warm=1)
+    del part, full
     if rank == 0:
         with open(out_path, "w") as f:
             json.dump(res, f)
@@ -601,6 +607,19 @@ def main():
         xr["allreduce_sync_rank0_shard_of_8x64MiB"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
                                                        "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
                                                        "first_pass_bit_identical_to_reduce_n": bool(same)}
+        # the pushed allgather: rank 0's launch (its 64 MiB written into slice 0 of eight outputs)
+        gathered = [torch.empty(N * COUNT, dtype=torch.bfloat16, device=dev) for _ in range(N)]
+        dst_tab = capi.ptr_table([g.data_ptr() for g in gathered])
+
+        def fanout_rank0():
+            sy = xsync(0)
+            capi.check(L.mccl_fanout_sync(ins[0].data_ptr(), dst_tab, N, COUNT * 2, ctypes.byref(sy), stream))
+        us = event_us(fanout_rank0)
+        moved = (N + 1) * COUNT * 2
+        xr["fanout_sync_64MiB_into_8_outputs"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
+                                                  "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                                  "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
+        del gathered
         L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget)
         assert status.tolist()[:2] == [0, 0], status.tolist()
         xr["wavefronts_per_launch"] = int(budget)
