@@ -209,6 +209,34 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
                          uint64_t timeout_us, void* status, unsigned max_compute_units, void* stream);
 
 /*
+ * mccl_allreduce_fused whose epoch lives on the device, so that the launch can be recorded in a HIP
+ * graph and replayed: the reference advances the index of its triple buffer on the host at every
+ * call (`buffer_index`, src/gpu/allreduce_small.h:118, 139); a replayed launch
+ * has no host call, so the launch reads the epoch from `state` when it starts and its last
+ * wavefront stores the next one.  state: MCCL_FUSED_STATE_BYTES of THIS rank's device memory,
+ * 64-byte aligned, zero before the first use, never written by the caller afterwards.  stage[r] /
+ * tile_flags[r] address the first of rank r's TWO staging buffers / flag arrays; the second lies
+ * stage_stride / flags_stride bytes behind it (multiples of 16 / 4; the message and its flags must
+ * fit in between).  The launch with epoch e uses set (e & 1).  Everything else as
+ * mccl_allreduce_fused, with the same results.  All ranks must issue the same sequence of calls on
+ * the same buffers (as for any collective); eager calls and replays of recorded ones may be mixed
+ * freely, in one stream order per rank.  Records no memset and allocates nothing.
+ *   flags: 0, or one of the bisecting switches of the reference's small allreduce
+ * (TORCH_CCL_WORK_ONLY / TORCH_CCL_SYNC_ONLY, src/gpu/dpcpp_ccl.cpp:56-85; the work_only and
+ * sync_only kernels of src/gpu/allreduce_small.h:414-701, 703-999): MCCL_FUSED_WORK_ONLY runs the
+ * launch without its rank waits (copy-in, flags, and the reduction of whatever the peers' buffers
+ * hold at that moment), MCCL_FUSED_SYNC_ONLY runs nothing but the flags and the waits.  Both are for
+ * timing what each part costs; the output of either is not a result.  All ranks pass the same flags.
+ */
+#define MCCL_FUSED_STATE_BYTES 128
+#define MCCL_FUSED_WORK_ONLY 1u
+#define MCCL_FUSED_SYNC_ONLY 2u
+int mccl_allreduce_fused_replayable(const void* in, void* out, size_t count, int dtype, int op,
+                                    void* const* stage, void* const* tile_flags, size_t stage_stride, size_t flags_stride,
+                                    void* state, int n, int rank, uint64_t timeout_us, void* status,
+                                    unsigned max_compute_units, unsigned flags, void* stream);
+
+/*
  * One-launch collectives between rank processes that read the peers' buffers in place.  With
  * several processes on one GPU every launch of a process waits for its turn at the dispatcher, so
  * the cross-rank waits are folded into the data kernel: the launch itself publishes "this rank's

@@ -1032,6 +1032,110 @@ def identity_replay_case(rank, world):
     dist.barrier()
 
 
+def graph_capture_case(rank, world):
+    """A decode loop from a HIP graph: every rank records K dist.all_reduce of the 256 KiB bf16
+    message with a small kernel of the caller's between them, then replays the graph with fresh
+    inputs, with eager collectives and synchronisations between the replays.  Every result of
+    every replay is compared bit for bit with the oracle's.  What cannot be recorded is refused
+    with a message, and the capture survives the refusal."""
+    from helpers import assert_bits_equal, bits, oracle_reduce_bits, rank_buffer
+    from oracle import oracle as O
+    K, count, replays, windows = 32, 131072, 50, 8
+    pool = [rank_buffer(count + 64 * windows, torch.bfloat16, r, seed=7000) for r in range(world)]
+    want = torch.stack([torch.from_numpy(oracle_reduce_bits([pool[r][64 * w:64 * w + count] for r in range(world)], O.SUM).view(np.int16).copy())
+                        for w in range(windows)]).to(DEV)                       # (windows, count) bit patterns
+    mine = torch.stack([pool[rank][64 * w:64 * w + count] for w in range(windows)]).to(DEV)
+    warm = torch.ones(1, device=DEV)
+    dist.all_reduce(warm)  # the group's buffers are allocated and exchanged at its first collective
+    assert float(warm[0]) == world
+    X = torch.zeros(K, count, dtype=torch.bfloat16, device=DEV)
+    ticks = torch.zeros(8, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # one pass outside the capture, as torch asks for
+        for k in range(K):
+            dist.all_reduce(X[k])
+            ticks.add_(1.0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    big = torch.ones(1 << 20, device=DEV)  # 4 MiB: needs the host rendezvous
+    with torch.cuda.graph(graph):
+        for k in range(K):
+            w = dist.all_reduce(X[k], async_op=True)
+            w.wait()
+            assert w.is_completed()
+            ticks.add_(1.0)
+        if rank == 0:  # (no other rank enters this collective: the refusal comes before anything is exchanged)
+            for refused in (lambda: dist.all_reduce(big), lambda: dist.all_gather_into_tensor(torch.empty(world * 4, device=DEV), torch.ones(4, device=DEV))):
+                try:
+                    refused()
+                    raise AssertionError("recorded a collective that cannot be replayed")
+                except RuntimeError as e:
+                    assert "cannot be recorded into a HIP graph" in str(e), str(e)
+    ticks.zero_()
+    wrong = torch.zeros((), dtype=torch.int64, device=DEV)
+    eager = []
+    gen = torch.Generator().manual_seed(7100)  # the same on every rank
+    for p in range(replays):
+        which = torch.randint(0, windows, (K,), generator=gen).to(DEV)
+        X.copy_(mine[which])
+        graph.replay()
+        wrong += (X.view(torch.int16) != want[which]).sum()
+        if p % 10 == 9:  # eager work of this backend and a synchronisation between two replays
+            e_in = [rank_buffer(5000 + p, torch.float32, r, seed=7200 + p) for r in range(world)]
+            e = e_in[rank].to(DEV)
+            dist.all_reduce(e)
+            eager.append((e, oracle_reduce_bits(e_in, O.SUM), p))
+            big2 = torch.full((1 << 20,), float(rank + 1), device=DEV)
+            dist.all_reduce(big2)
+            torch.cuda.synchronize()
+            assert float(big2[0]) == world * (world + 1) / 2 == float(big2[-1])
+    torch.cuda.synchronize()
+    assert int(wrong) == 0, int(wrong)
+    assert ticks.cpu().tolist() == [float(K * replays)] * 8
+    for e, w, p in eager:
+        assert_bits_equal(bits(e), w, ("eager between replays", p))
+    dist.barrier()
+
+
+def graph_late_rank_case(rank, world):
+    """A rank that does not replay its graph: the bounded waits of the recorded launches on the other
+    ranks run into their (shortened) limit, every kernel ends by itself, and the group reports the
+    late rank at its next call."""
+    warm = torch.ones(1, device=DEV)
+    dist.all_reduce(warm)
+    X = torch.ones(2, 131072, dtype=torch.bfloat16, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for k in range(2):
+            dist.all_reduce(X[k])
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for k in range(2):
+            dist.all_reduce(X[k])
+    X.fill_(1.0)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float(X[0, 0]) == world == float(X[1, -1])
+    if rank == 1:
+        import time
+        time.sleep(6.0)  # stays in the group, replays nothing
+        return
+    X.fill_(1.0)
+    graph.replay()
+    torch.cuda.synchronize()  # both launches have given up by now
+    assert float(X[0, 0]) == 1.0 == float(X[1, -1])  # left alone
+    try:
+        dist.all_reduce(warm)
+        raise AssertionError("a failed group accepted another collective")
+    except RuntimeError as e:
+        assert "timed out waiting for rank 1 on the device (one-launch allreduce #" in str(e), str(e)
+
+
 def coalesced_window_cases(rank, world):
     """Coalesced forms on the default group whose staging image exceeds the (shrunk) window: they
     fall back to one windowed collective per tensor and must give the same results."""
@@ -1107,12 +1211,13 @@ def run_rank(rank, world, store_path, mode):
         finally:
             dist.destroy_process_group()
         return
-    if mode in ("subgroup", "replay", "reference_p2p", "coalesced_windows", "heavy_predecessor"):
+    if mode in ("subgroup", "replay", "reference_p2p", "coalesced_windows", "heavy_predecessor", "graph", "graph_late"):
         store = dist.FileStore(store_path, world)
         dist.init_process_group("ccl", store=store, rank=rank, world_size=world)
         try:
             {"subgroup": subgroup_case, "replay": identity_replay_case, "reference_p2p": reference_p2p_cases,
-             "coalesced_windows": coalesced_window_cases, "heavy_predecessor": heavy_predecessor_case}[mode](rank, world)
+             "coalesced_windows": coalesced_window_cases, "heavy_predecessor": heavy_predecessor_case,
+             "graph": graph_capture_case, "graph_late": graph_late_rank_case}[mode](rank, world)
         finally:
             dist.destroy_process_group()
         return

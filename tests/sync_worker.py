@@ -87,12 +87,15 @@ def fused_case(rank, world, queues, barrier):
                        capi.ptr_table([shared[r][2 + slot].data_ptr() for r in range(world)])))
     st = _status()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    ops = {"SUM": (capi.SUM, O.SUM), "PROD": (capi.PROD, O.PROD), "MIN": (capi.MIN, O.MIN), "MAX": (capi.MAX, O.MAX)}
+    ops = {"SUM": (capi.SUM, O.SUM), "PROD": (capi.PROD, O.PROD), "MIN": (capi.MIN, O.MIN), "MAX": (capi.MAX, O.MAX),
+           "AVG": (capi.AVG, O.AVG)}
     cases = []
     for dtype in ALL_DTYPES:
         es = torch.empty(0, dtype=dtype).element_size()
         for count in (1, 7, 16 // es, 16 // es + 1, 1024 // es, 1024 // es + 3, 5 * 1024 // es - 1, 40_000):
             for name in ops:
+                if name == "AVG" and not dtype.is_floating_point:
+                    continue  # an addition of this library, floats only
                 cases.append((dtype, count, name))
     cases.append((torch.bfloat16, 131072, "SUM"))       # the 256 KiB decode message
     cases.append((torch.float32, FUSED_MAX_BYTES // 4, "SUM"))
@@ -158,6 +161,109 @@ def fused_case(rank, world, queues, barrier):
     barrier.wait(timeout=120)
 
 
+def fused_replay_case(rank, world, queues, barrier):
+    """mccl_allreduce_fused_replayable -- the epoch and the choice of buffer set live on the device and
+    are advanced by the launch itself -- against the oracle, bit for bit: eager calls, then launches
+    recorded in a HIP graph and replayed with fresh inputs, with eager calls between the replays."""
+    from helpers import TORCH_TO_CODE, assert_bits_equal, bits, oracle_reduce_bits, rank_buffer
+    from oracle import oracle as O
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    stage_stride = FUSED_MAX_BYTES + 64
+    flags_stride = (FUSED_MAX_BYTES // TILE + 1) * 4
+    stage = torch.zeros(2 * stage_stride, dtype=torch.uint8, device=DEV)          # both sets, one allocation
+    tflag = torch.zeros(2 * flags_stride // 4, dtype=torch.int32, device=DEV)
+    state = torch.zeros(capi.FUSED_STATE_BYTES // 4, dtype=torch.int32, device=DEV)  # this rank's own
+    torch.cuda.synchronize()
+    shared = _exchange(rank, world, queues, barrier, [stage, tflag])
+    stages = capi.ptr_table([shared[r][0].data_ptr() for r in range(world)])
+    flags = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])
+    st = _status()
+
+    def call(x, out, count, dtype, op, units=0, flags_=0):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        capi.check(L.mccl_allreduce_fused_replayable(x.data_ptr(), out.data_ptr(), count, TORCH_TO_CODE[dtype], op, stages, flags,
+                                                     stage_stride, flags_stride, state.data_ptr(), world, rank, 5_000_000,
+                                                     st.data_ptr(), units, flags_, stream))
+
+    ops = {"SUM": (capi.SUM, O.SUM), "AVG": (capi.AVG, O.AVG), "MAX": (capi.MAX, O.MAX)}
+    launches = 0
+    pending = []
+    for i, (dtype, count, name, units) in enumerate([(torch.bfloat16, 131072, "SUM", 128 // world), (torch.float32, 7, "SUM", 0), (torch.bfloat16, 1025, "AVG", 0),
+                                                    (torch.float32, FUSED_MAX_BYTES // 4, "SUM", 128 // world), (torch.int8, 40_001, "MAX", 1),
+                                                    (torch.float16, 5 * 512 - 1, "AVG", 2), (torch.float64, 3 * 1024 + 1, "SUM", 1),
+                                                    (torch.bfloat16, 131072 - 9, "SUM", 5), (torch.int64, 129, "SUM", 0)]):
+        cpu_in = [rank_buffer(count, dtype, r, seed=6000 + i) for r in range(world)]
+        x = cpu_in[rank].to(DEV)
+        out = x if i % 2 == 0 else torch.empty_like(x)
+        call(x, out, count, dtype, ops[name][0], units)
+        launches += 1
+        pending.append((out, oracle_reduce_bits(cpu_in, ops[name][1]), ("eager", str(dtype), count, name)))
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    for o, w, what in pending:
+        assert_bits_equal(bits(o), w, what)
+    assert state.cpu().tolist()[0] == launches and state.cpu().tolist()[16] == 0, state.cpu().tolist()
+
+    # recorded: K launches of the decode message with a small kernel of the caller's between them
+    K, count, replays = 6, 131072, 12
+    pool = [rank_buffer(count + 4096, torch.bfloat16, r, seed=6100) for r in range(world)]
+    pool_dev = pool[rank].to(DEV)
+    xs = [torch.zeros(count, dtype=torch.bfloat16, device=DEV) for _ in range(K)]
+    ticks = torch.zeros(8, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # (a first pass outside the capture, as torch asks for; every rank does the same)
+        for k in range(K):
+            call(xs[k], xs[k], count, torch.bfloat16, capi.SUM, 128 // world)
+            launches += 1
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for k in range(K):
+            call(xs[k], xs[k], count, torch.bfloat16, capi.SUM, 128 // world)
+            ticks.add_(1.0)
+    results = []
+    for p in range(replays):
+        for k in range(K):
+            off = (p * K + k) * 7 % 4096
+            xs[k].copy_(pool_dev[off:off + count])
+        graph.replay()
+        launches += K
+        results.append(torch.stack(xs).clone())
+        if p % 3 == 2:  # an eager call between two replays: the same counter serves both
+            e_in = [rank_buffer(3000 + p, torch.float32, r, seed=6200 + p) for r in range(world)]
+            e = e_in[rank].to(DEV)
+            call(e, e, 3000 + p, torch.float32, capi.SUM, 0)
+            launches += 1
+            pending.append((e, oracle_reduce_bits(e_in, O.SUM), ("eager between replays", p)))
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    assert ticks.cpu().tolist() == [float(K * replays)] * 8
+    for p in range(replays):
+        got = results[p].cpu()
+        for k in range(K):
+            off = (p * K + k) * 7 % 4096
+            want = oracle_reduce_bits([pool[r][off:off + count] for r in range(world)], O.SUM)
+            assert_bits_equal(bits(got[k]), want, ("replay", p, k))
+    for o, w, what in pending:
+        assert_bits_equal(bits(o), w, what)
+    assert state.cpu().tolist()[0] == launches and state.cpu().tolist()[16] == 0, (state.cpu().tolist(), launches)
+    # the bisecting forms run to their end and keep the counter going; their output is not a result
+    y = torch.ones(4096, device=DEV)
+    call(y, y, 4096, torch.float32, capi.SUM, 0, capi.FUSED_WORK_ONLY)
+    call(y, y, 4096, torch.float32, capi.SUM, 0, capi.FUSED_SYNC_ONLY)
+    z_in = [rank_buffer(4096, torch.float32, r, seed=6300) for r in range(world)]
+    z = z_in[rank].to(DEV)
+    call(z, z, 4096, torch.float32, capi.SUM, 0)
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    assert_bits_equal(bits(z), oracle_reduce_bits(z_in, O.SUM), "after the bisecting forms")
+    assert state.cpu().tolist()[0] == launches + 3
+    barrier.wait(timeout=120)
+
+
 def xrank_case(rank, world, queues, barrier):
     """The one-launch collectives that read the peers' buffers in place -- mccl_reduce_sync
     (reduce_scatter shard), mccl_allreduce_sync (in-place allreduce) and mccl_copy_segments_sync
@@ -188,12 +294,14 @@ def xrank_case(rank, world, queues, barrier):
     def mine(dtype, count, off):
         return shared_in[off:off + count * torch.empty(0, dtype=dtype).element_size()].view(dtype)
 
-    ops = {"SUM": (capi.SUM, O.SUM), "PROD": (capi.PROD, O.PROD), "MIN": (capi.MIN, O.MIN), "MAX": (capi.MAX, O.MAX)}
+    ops = {"SUM": (capi.SUM, O.SUM), "PROD": (capi.PROD, O.PROD), "MIN": (capi.MIN, O.MIN), "MAX": (capi.MAX, O.MAX),
+           "AVG": (capi.AVG, O.AVG)}
     checks = []
     # reduce_scatter shard: rank r reduces slice r of every rank's buffer
     for i, (dtype, m, name, off) in enumerate([(torch.bfloat16, 70001, "SUM", 0), (torch.float32, 4099, "MAX", 4), (torch.int8, 300007, "SUM", 1),
                                               (torch.float64, 1, "PROD", 8), (torch.float16, 1 << 19, "SUM", 16), (torch.int64, 33, "MIN", 0),
-                                              (torch.bfloat16, 1 << 20, "SUM", 2)]):
+                                              (torch.bfloat16, 1 << 20, "SUM", 2), (torch.bfloat16, 70001, "AVG", 2), (torch.float32, 4099, "AVG", 0),
+                                              (torch.float16, 515, "AVG", 6), (torch.float64, 1027, "AVG", 8)]):
         es = torch.empty(0, dtype=dtype).element_size()
         off = off // es * es
         host = [rank_buffer(world * m, dtype, r, seed=300 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
@@ -209,7 +317,8 @@ def xrank_case(rank, world, queues, barrier):
     for i, (dtype, count, name, off) in enumerate([(torch.bfloat16, (2 << 20) + 77, "SUM", 0), (torch.float32, 1025, "SUM", 4), (torch.int8, (3 << 20) + 5, "MAX", 3),
                                                   (torch.float64, 7, "SUM", 8), (torch.bfloat16, 3, "MIN", 2), (torch.float16, 1 << 21, "SUM", 0),
                                                   (torch.int32, 100003, "PROD", 4), (torch.bfloat16, 4096 * 1024, "SUM", 0), (torch.uint8, 1, "SUM", 5),
-                                                  (torch.bfloat16, 4096 * 1024, "SUM", 6)]):
+                                                  (torch.bfloat16, 4096 * 1024, "SUM", 6), (torch.bfloat16, (1 << 20) + 77, "AVG", 0),
+                                                  (torch.float32, 100003, "AVG", 4), (torch.float16, 1025, "AVG", 2), (torch.float64, 4097, "AVG", 8)]):
         es = torch.empty(0, dtype=dtype).element_size()
         off = off // es * es
         host = [rank_buffer(count, dtype, r, seed=450 + i, scale=1.0 if name == "PROD" else 0.02) for r in range(world)]
@@ -295,5 +404,6 @@ def timeout_case(rank, world, queues, barrier):
 def run_rank(rank, world, queues, barrier, mode):
     torch.set_num_threads(max(1, (os.cpu_count() or 16) // world))  # the ranks share the host's cores
     torch.cuda.set_device(0)
-    {"barrier": barrier_case, "fused": fused_case, "timeout": timeout_case, "xrank": xrank_case}[mode](rank, world, queues, barrier)
+    {"barrier": barrier_case, "fused": fused_case, "fused_replay": fused_replay_case, "timeout": timeout_case,
+     "xrank": xrank_case}[mode](rank, world, queues, barrier)
     torch.cuda.synchronize()

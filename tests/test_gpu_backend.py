@@ -45,6 +45,18 @@ def test_identity_replay_interleaved_with_compute(world):
     _spawn(world, "replay")
 
 
+@pytest.mark.parametrize("world", [2, 8])
+def test_all_reduce_recorded_into_a_hip_graph_and_replayed(world):
+    """32 dist.all_reduce of the 256 KiB decode message per graph, 50 replays with fresh inputs,
+    every result against the oracle; larger tensors and other collectives are refused under capture."""
+    _spawn(world, "graph")
+
+
+def test_a_rank_that_does_not_replay_is_found_by_the_recorded_launches(monkeypatch):
+    monkeypatch.setenv("MCCL_BARRIER_TIMEOUT_MS", "1500")
+    _spawn(3, "graph_late")
+
+
 def test_subgroups():
     _spawn(4, "subgroup")
 

@@ -28,6 +28,11 @@ def test_allreduce_fused_matches_the_oracle(world):
     _spawn(world, "fused")
 
 
+@pytest.mark.parametrize("world", [2, 8])
+def test_allreduce_fused_with_its_epoch_on_the_device_eager_and_replayed_from_a_graph(world):
+    _spawn(world, "fused_replay")
+
+
 @pytest.mark.parametrize("world", [2, 5, 8])
 def test_one_launch_collectives_match_the_oracle(world):
     _spawn(world, "xrank")

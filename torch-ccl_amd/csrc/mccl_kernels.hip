@@ -725,10 +725,19 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
   return MCCL_OK;
 }
 
-int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
-                         void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
-                         uint64_t timeout_us, void* status, unsigned max_compute_units, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// Both forms of the one-launch small allreduce: the epoch from the host (state == null), or kept in
+// `state` on the device and advanced by the launch itself.
+int allreduce_fused_impl(const void* in, void* out, size_t count, int dtype, int op, void* const* stage,
+                         void* const* tile_flags, int n, int rank, uint32_t epoch, void* state, size_t stage_stride,
+                         size_t flags_stride, uint64_t timeout_us, void* status, unsigned max_compute_units, unsigned mode,
+                         void* stream) {
   int rc = check_reduce_args_no_ptr(n, dtype, op);
+  if (mode & ~(MCCL_FUSED_WORK_ONLY | MCCL_FUSED_SYNC_ONLY)) return fail(MCCL_ERR_INVALID_ARG, "unknown flags 0x%x", mode);
+  if (mode == (MCCL_FUSED_WORK_ONLY | MCCL_FUSED_SYNC_ONLY)) return fail(MCCL_ERR_INVALID_ARG, "work-only and sync-only exclude each other");
   if (rc != MCCL_OK) return rc;
   if (n > MCCL_FUSED_MAX_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "the one-launch allreduce takes at most %d ranks, got %d", MCCL_FUSED_MAX_RANKS, n);
   if (rank < 0 || rank >= n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", rank, n);
@@ -740,16 +749,22 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
     if ((uintptr_t)stage[r] % 16) return fail(MCCL_ERR_INVALID_ARG, "staging buffer %d is not 16-byte aligned", r);
     if ((uintptr_t)tile_flags[r] % 4) return fail(MCCL_ERR_INVALID_ARG, "flag array %d is not 4-byte aligned", r);
   }
-  if (count == 0) return MCCL_OK;
+  const size_t ve = 16 / es;
+  const size_t nvec = count / ve;
+  const size_t tiles = (nvec + (count % ve ? 1 : 0) + kWave - 1) / kWave;
+  if (state) {
+    if ((uintptr_t)state % 64) return fail(MCCL_ERR_INVALID_ARG, "the epoch state is not 64-byte aligned");
+    if (stage_stride % 16 || stage_stride > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "the staging sets must lie a multiple of 16 bytes (below 4 GiB) apart");
+    if (flags_stride % 4 || flags_stride > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "the flag sets must lie a multiple of 4 bytes (below 4 GiB) apart");
+    if (count * es > stage_stride || tiles * 4 > flags_stride) return fail(MCCL_ERR_INVALID_ARG, "the message does not fit between the two buffer sets");
+  }
+  if (count == 0) return MCCL_OK;  // on every rank alike: no launch, the epoch stays
   if (!in || !out) return fail(MCCL_ERR_INVALID_ARG, "input or output pointer is null");
   if ((uintptr_t)in % es || (uintptr_t)out % es) return fail(MCCL_ERR_INVALID_ARG, "input or output pointer not aligned to the element size");
   if (in != out) {
     const uintptr_t i0 = (uintptr_t)in, o0 = (uintptr_t)out;
     if (i0 < o0 + count * es && o0 < i0 + count * es) return fail(MCCL_ERR_INVALID_ARG, "output partially overlaps the input");
   }
-  const size_t ve = 16 / es;
-  const size_t nvec = count / ve;
-  const size_t tiles = (nvec + (count % ve ? 1 : 0) + kWave - 1) / kWave;
   if (tiles > kMaxGridX) return fail(MCCL_ERR_INVALID_ARG, "message too large for the one-launch allreduce");
   // one wavefront per tile, sixteen to a workgroup; with a limit on the workgroups a wavefront
   // takes up to kFusedMaxTilesPerWave tiles
@@ -776,9 +791,33 @@ int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int
   a.tiles = (uint32_t)tiles;
   a.n = n;
   a.rank = rank;
+  a.state = (uint32_t*)state;
+  a.stage_stride = (uint32_t)stage_stride;
+  a.flag_stride = (uint32_t)(flags_stride / 4);
+  a.mode = mode;
   hipError_t e = launch_fused_any(a, dtype, op, (unsigned)groups, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "fused allreduce launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_allreduce_fused(const void* in, void* out, size_t count, int dtype, int op,
+                         void* const* stage, void* const* tile_flags, int n, int rank, uint32_t epoch,
+                         uint64_t timeout_us, void* status, unsigned max_compute_units, void* stream) {
+  return allreduce_fused_impl(in, out, count, dtype, op, stage, tile_flags, n, rank, epoch, nullptr, 0, 0, timeout_us, status,
+                              max_compute_units, 0u, stream);
+}
+
+int mccl_allreduce_fused_replayable(const void* in, void* out, size_t count, int dtype, int op,
+                                    void* const* stage, void* const* tile_flags, size_t stage_stride, size_t flags_stride,
+                                    void* state, int n, int rank, uint64_t timeout_us, void* status,
+                                    unsigned max_compute_units, unsigned flags, void* stream) {
+  if (!state) return fail(MCCL_ERR_INVALID_ARG, "the epoch state is null");
+  return allreduce_fused_impl(in, out, count, dtype, op, stage, tile_flags, n, rank, 0, state, stage_stride, flags_stride,
+                              timeout_us, status, max_compute_units, flags, stream);
 }
 
 }  // extern "C"

@@ -69,9 +69,11 @@ constexpr size_t kArenaFusedFlagsStride = 8192;
 constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buffers of 1 MiB, each
 constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
 constexpr size_t kArenaDoneCountOff = 1024;  // MCCL_SYNC_COUNTER_BYTES of workgroup counters of the one-launch collectives
+constexpr size_t kArenaFusedStateOff = 2048;  // MCCL_FUSED_STATE_BYTES: the device-resident epoch of the one-launch small allreduce
 constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
 static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
-static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedFlagsOff, "the counters end before the flags");
+static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedStateOff, "the counters end before the epoch state");
+static_assert(kArenaFusedStateOff + MCCL_FUSED_STATE_BYTES <= kArenaFusedFlagsOff, "the epoch state ends before the flags");
 
 #define HIP_CHECK(expr)                                                                     \
   do {                                                                                      \
@@ -248,13 +250,21 @@ void GroupShared::putEvent(hipEvent_t e) {
 }
 
 std::string GroupShared::failureMessage() {
-  if (status && status[0] != 0 && !failed.load(std::memory_order_acquire)) {
+  if (status && (status[0] != 0 || status[2] != 0) && !failed.load(std::memory_order_acquire)) {
     std::ostringstream os;
-    // epochs count four per collective: #(epoch / 4), wait (epoch % 4): 1 = inputs ready, 2 = between
-    // the phases of a two-phase collective, 3 = all ranks done with this rank's buffers
-    os << "ccl backend: timed out waiting for rank " << (status[0] - 1)
-       << " on the device (cross-rank wait " << (status[1] & 3u) << " of collective #" << (status[1] >> 2)
-       << ", modulo 2^30); the group cannot be used any more";
+    if (status[0] != 0) {
+      // epochs count four per collective: #(epoch / 4), wait (epoch % 4): 1 = inputs ready, 2 = between
+      // the phases of a two-phase collective, 3 = all ranks done with this rank's buffers
+      os << "ccl backend: timed out waiting for rank " << (status[0] - 1)
+         << " on the device (cross-rank wait " << (status[1] & 3u) << " of collective #" << (status[1] >> 2)
+         << ", modulo 2^30); the group cannot be used any more";
+    } else {
+      // the one-launch small allreduce counts its own launches, on the device (replays of a recorded
+      // graph included, which the host's collective numbers do not see)
+      os << "ccl backend: timed out waiting for rank " << (status[2] - 1)
+         << " on the device (one-launch allreduce #" << status[3]
+         << " of this group, counting those alone, modulo 2^32); the group cannot be used any more";
+    }
     fail(os.str());
   }
   if (!failed.load(std::memory_order_acquire)) return std::string();
@@ -293,6 +303,7 @@ bool ProcessGroupCCL::WorkCCL::isCompleted() {
     if (pending_polls_ > 0) --pending_polls_;
     return false;
   }
+  if (captured_) return true;  // recorded, not enqueued: nothing of this Work is outstanding
   if (end_) return hipEventQuery(end_) == hipSuccess;
   if (!stream_set_) return true;
   // No event was recorded for this collective (it ran on the caller's stream; with several
@@ -441,6 +452,14 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   }
   if (const char* v = std::getenv("MCCL_PG_COMPACT_MAX_BYTES")) compact_max_ = (size_t)std::atoll(v);
   allgather_push_ = envFlag("MCCL_PG_ALLGATHER_PUSH", true);
+  work_only_ = envFlag("TORCH_CCL_WORK_ONLY", false) || envFlag("MCCL_PG_WORK_ONLY", false);
+  sync_only_ = envFlag("TORCH_CCL_SYNC_ONLY", false) || envFlag("MCCL_PG_SYNC_ONLY", false);
+  disable_allreduce_ = envFlag("TORCH_CCL_DISABLE_ALLREDUCE", false) || envFlag("MCCL_PG_DISABLE_ALLREDUCE", false);
+  TORCH_CHECK(!(work_only_ && sync_only_), "ccl backend: TORCH_CCL_WORK_ONLY and TORCH_CCL_SYNC_ONLY exclude each other");
+  fused_mode_ = work_only_ ? MCCL_FUSED_WORK_ONLY : sync_only_ ? MCCL_FUSED_SYNC_ONLY : 0u;
+  if (work_only_ || sync_only_ || disable_allreduce_)
+    TORCH_WARN_ONCE("ccl backend: a bisecting switch is set (", work_only_ ? "work only: no cross-rank waits" : sync_only_ ? "sync only: no data is moved" : "allreduce disabled",
+                    "); collectives between rank processes do NOT produce results, this is for timing only");
   if (const char* v = std::getenv("MCCL_PG_WAITING_COMPUTE_UNITS")) waiting_cus_ = (unsigned)std::max(1, std::atoi(v));
   // The staging window can be shrunk (never enlarged) so that tests reach every windowed path
   // with small tensors.
@@ -647,6 +666,7 @@ void ProcessGroupCCL::ensureInit(int device) {
       fused_flags_[sl].assign((size_t)size_, nullptr);
     }
     done_counter_ = static_cast<char*>(arena_) + kArenaDoneCountOff;
+    fused_state_ = static_cast<char*>(arena_) + kArenaFusedStateOff;
     for (int r = 0; r < size_; ++r) {
       char* base = nullptr;
       if (r == rank_) {
@@ -670,7 +690,9 @@ void ProcessGroupCCL::ensureInit(int device) {
     // nobody starts a collective before everybody has mapped everything
     hostBarrier(/*start_up=*/true);
   }
-  if (device_sync_ && zero_copy_) {
+  // (also with MCCL_PG_SYNC=host: rank processes offer their tensors for the in-place allreduce there,
+  // and a freed and re-issued segment must retire its export in that mode, too)
+  if (distinct_pids_ && zero_copy_) {
     attachSegmentTracker();
     std::lock_guard<std::mutex> lock(g_registry_mutex);
     g_registry.push_back(this);
@@ -937,12 +959,36 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::run(Plan& plan) {
   if (device < 0) for (const auto& t : plan.outputs) if (t.defined()) { device = t.get_device(); break; }
   if (device < 0) device = initialised_ ? device_ : 0;  // barrier without tensors
   c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device));
+  hipStream_t cur = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device).stream();
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_CHECK(hipStreamIsCapturing(cur, &capture));
+  if (capture != hipStreamCaptureStatusNone) {
+    // The caller is recording a HIP graph.  What can be recorded is the one launch of the small
+    // allreduce in its replayable form: its epoch and buffer choice live on the device, it needs no
+    // rendezvous of the host threads, no memset and no allocation, so every replay is a complete
+    // collective.  Everything else publishes tables or handles from the host at call time, which a
+    // replay would not repeat: refused here rather than recorded wrongly.
+    TORCH_CHECK(capture == hipStreamCaptureStatusActive, "ccl backend: the stream's capture has been invalidated");
+    TORCH_CHECK(initialised_ && device == device_,
+                "ccl backend: run one collective of this group before recording a HIP graph (the group's buffers are "
+                "allocated and exchanged at its first collective, which cannot happen under stream capture)");
+    throwIfFailed();
+    TORCH_CHECK(device_sync_ && fusedFits(plan), "ccl backend: ", plan.title, " cannot be recorded into a HIP graph: under "
+                "stream capture this backend takes all_reduce of at most ",
+                (size_t)std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_) * kFusedBytesPerComputeUnit,
+                " bytes per tensor (and not more than ", kFusedMaxBytes, ") between at most ", MCCL_FUSED_MAX_RANKS,
+                " rank processes; larger tensors and the other collectives exchange tables or memory handles on the host "
+                "at call time");
+    // Not numbered: seq_ counts what the host has enqueued (the staging slots of the other
+    // collectives alternate with it), and a recorded launch runs whenever its graph is replayed.
+    if (verbose_) std::cout << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "] recorded (stream capture)" << std::endl;
+    launchFused(plan, cur);
+    return finishRun(plan, cur, /*same_stream=*/true, /*device_work=*/false, /*capturing=*/true);
+  }
   ensureInit(device);
   TORCH_CHECK((int)plan.table.size() <= kTableMax, "ccl backend: too many tensors in one collective");
   throwIfFailed();
 
-  auto cur_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device_);
-  hipStream_t cur = cur_stream.stream();
   // Which stream: the reference runs collectives on a communication stream that waits for the
   // caller's (src/gpu/dpcpp_ccl.cpp:186-197) unless CCL_SAME_STREAM=1.  Here all ranks share one
   // GPU, where the fork and join (two event records, two stream waits: packets of their own that
@@ -1117,20 +1163,9 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
       std::cout << os.str() << std::endl;
     };
-    // On this rank's share of the compute units that all ranks' waiting launches may hold together
-    // (a share takes 64 KiB per compute unit).  With MCCL_PG_SYNC=kernel the share is one workgroup
-    // per compute unit and rank, half of what the GPU holds: a wavefront of this kernel waits for
-    // the same tile of every peer, so all of a late rank's workgroups must still find room beside
-    // the waiting ones, and a launch per 16 KiB (8 ranks x 1 MiB: 512 workgroups, exactly what
-    // fits when nothing else runs) leaves none to spare.
-    const unsigned fused_units = std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_);
-    if (plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS &&
-        plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= (size_t)fused_units * kFusedBytesPerComputeUnit) {
+    if (fusedFits(plan)) {
       say_path();
-      const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
-      MCCL_CHECK(mccl_allreduce_fused(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
-                                      fused_stage_[slot].data(), fused_flags_[slot].data(), size_, rank_,
-                                      (uint32_t)(seq + 1), limit_us, status_dev_, fused_units, s));
+      launchFused(plan, s);
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }
@@ -1177,6 +1212,27 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       for (int r = 0; r < size_; ++r) pv.user[(size_t)r] = (r == rank_) ? plan.share_ptr : importRange(r, pub);
     }
     if (timed) { phase_us_[1].push_back((float)us_since(t0)); t0 = clk::now(); }
+    if (sync_only_) {
+      // bisecting: the cross-rank waits of the default form and nothing else
+      last_path_ = "sync only";
+      say_path();
+      deviceBarrier(epoch + 1, s);
+      if (zero_copy) deviceBarrier(epoch + 3, s);
+      return;
+    }
+    if (work_only_) {
+      // bisecting: the data movement alone, nobody waits for anybody (results are not valid)
+      last_path_ = "work only";
+      say_path();
+      if (!zero_copy && plan.copy_in) plan.copy_in(stage, s);
+      mccl_xsync_t none{};
+      none.n = size_;
+      none.rank = rank_;
+      if (plan.exec_sync && size_ <= MCCL_FUSED_MAX_RANKS && (zero_copy || !plan.exec_sync_in_place_only) && plan.exec_sync(pv, none, s)) return;
+      if (plan.exec) plan.exec(pv, s);
+      if (plan.exec2 && (!plan.two_phase || plan.two_phase(pv))) plan.exec2(pv, s);
+      return;
+    }
     // One launch: the kernel itself announces this rank, waits for the others, does the work and
     // (in place: where a tensor must not be touched before the peers have read it) waits again.
     // With several processes on the GPU every launch waits for its turn at the dispatcher, so this
@@ -1249,12 +1305,41 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
   }
 }
 
-c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work) {
+// On this rank's share of the compute units that all ranks' waiting launches may hold together (a
+// share takes 64 KiB per compute unit).  With MCCL_PG_SYNC=kernel the share is one workgroup per
+// compute unit and rank, half of what the GPU holds: a wavefront of this kernel waits for the same
+// tile of every peer, so all of a late rank's workgroups must still find room beside the waiting
+// ones, and a launch per 16 KiB (8 ranks x 1 MiB: 512 workgroups, exactly what fits when nothing
+// else runs) leaves none to spare.
+bool ProcessGroupCCL::fusedFits(const Plan& plan) const {
+  const unsigned units = std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_);
+  return plan.fused_ok && size_ <= MCCL_FUSED_MAX_RANKS &&
+         plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= (size_t)units * kFusedBytesPerComputeUnit;
+}
+
+// The epoch of the launch and its choice between the two sets of staging buffers and flags are read
+// from this rank's arena by the launch itself and advanced by it, so the same launch serves eager
+// calls and replays of a recorded graph, in any mixture, and all ranks' counters agree as long as
+// the ranks issue the same collectives (which they must anyway).
+void ProcessGroupCCL::launchFused(const Plan& plan, hipStream_t s) {
+  const unsigned units = std::max(1u, (waits_in_data_kernels_ ? kComputeUnits : waiting_cus_) / (unsigned)size_);
+  last_title_ = plan.title;
+  last_path_ = "one launch, fused";
+  ++enqueue_only_count_;
+  const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+  MCCL_CHECK(mccl_allreduce_fused_replayable(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
+                                             fused_stage_[0].data(), fused_flags_[0].data(), kArenaFusedStageStride,
+                                             kArenaFusedFlagsStride, fused_state_, size_, rank_, limit_us,
+                                             static_cast<char*>(status_dev_) + 8, units, fused_mode_, s));
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work, bool capturing) {
   if (device_work) {
     tail_stream_ = s;
     tail_pending_ = true;
   }
-  auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_);
+  auto work = c10::make_intrusive<WorkCCL>(rank_, plan.op, plan.title, plan.inputs, plan.outputs, blocking_wait_ && !capturing);
+  work->captured_ = capturing;
   work->device_ = device_;
   work->shared_ = shared_;
   work->op_timeout_ = timeout_;
@@ -1406,7 +1491,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
     p.title = "allreduce";
     p.inputs = {t};
     p.outputs = {t};
-    if (size_ > 1 && len) {  // world == 1: nothing to add (src/gpu/dpcpp_ccl.cpp:752-756)
+    if (size_ > 1 && len && !disable_allreduce_) {  // world == 1 or switched off: nothing to add (src/gpu/dpcpp_ccl.cpp:752-756)
       const int W = size_;
       const int me = rank_;
       // elements per shard: a whole number of 64-element groups, so that every shard starts on a

@@ -50,8 +50,10 @@ namespace mccl_pg {
 struct Control;  // shared-memory control block (process_group_ccl.cpp)
 
 // What the Works of a group share with it and may outlive it with: recycled events and the
-// group's health.  `status` is two words of pinned host memory the device-side waits write when
-// they give up (1 + the late rank, the epoch); `failed` is raised by the host side.
+// group's health.  `status` is pinned host memory the device-side waits write when they give up:
+// words 0-1 (1 + the late rank, the epoch) for the barrier and the one-launch collectives, words
+// 2-3 the same for the one-launch small allreduce, whose epochs are counted on the device and in a
+// numbering of their own; `failed` is raised by the host side.
 struct GroupShared {
   std::mutex mutex;
   std::vector<hipEvent_t> free_events;
@@ -105,6 +107,9 @@ class ProcessGroupCCL : public c10d::Backend {
     int device_ = 0;
     bool blocking_wait_ = false;
     int pending_polls_ = 0;  // > 0: isCompleted() says "not yet" this many more times, < 0: for good (pendingWork)
+    // Recorded into a HIP graph under stream capture: nothing has been enqueued, the stream must not
+    // be queried, and when the work runs is up to whoever replays the graph.
+    bool captured_ = false;
     std::vector<at::Tensor> inputs_;   // held until the Work dies (ownership rule of the reference)
     std::vector<at::Tensor> outputs_;
     c10::intrusive_ptr<c10::ivalue::Future> future_;
@@ -288,7 +293,11 @@ class ProcessGroupCCL : public c10d::Backend {
                                           const std::vector<at::Tensor>& outputs, const ExchangeImage& image,
                                           const std::vector<void*>& dst, const std::vector<size_t>& recv);
   c10::intrusive_ptr<c10d::Work> run(Plan& plan);
-  c10::intrusive_ptr<c10d::Work> finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work);
+  c10::intrusive_ptr<c10d::Work> finishRun(Plan& plan, hipStream_t s, bool same_stream, bool device_work, bool capturing = false);
+  // The one-launch small allreduce of `plan` on `s` (also under stream capture: the launch carries
+  // nothing that changes from replay to replay).
+  void launchFused(const Plan& plan, hipStream_t s);
+  bool fusedFits(const Plan& plan) const;
   void runHostSynced(Plan& plan, hipStream_t s, int slot);
   void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void deviceBarrier(uint64_t epoch, hipStream_t s);
@@ -361,6 +370,22 @@ class ProcessGroupCCL : public c10d::Backend {
   // to 32 MiB (16 MiB: 83-104 against 106-141 us).  MCCL_PG_COMPACT_MAX_BYTES overrides (0: never).
   size_t compact_max_ = 16u << 20;
   bool allgather_push_ = true;  // MCCL_PG_ALLGATHER_PUSH != 0: all_gather_into_tensor writes into the peers' outputs
+  // Bisecting switches of the reference (src/gpu/dpcpp_ccl.cpp:56-85), for rank processes: what
+  // does a collective cost without its cross-rank waits, what do the waits cost alone?  Results are
+  // NOT valid with either of the first two; they exist for timing.
+  //   TORCH_CCL_WORK_ONLY / MCCL_PG_WORK_ONLY=1   data kernels only: no barrier kernel, no waits inside
+  //   TORCH_CCL_SYNC_ONLY / MCCL_PG_SYNC_ONLY=1   the cross-rank waits only: no copy-in, no data kernel
+  //   TORCH_CCL_DISABLE_ALLREDUCE=1               allreduce enqueues nothing (src/gpu/dpcpp_ccl.cpp:752-756)
+  bool work_only_ = false;
+  bool sync_only_ = false;
+  bool disable_allreduce_ = false;
+  unsigned fused_mode_ = 0;     // the same two as flags of mccl_allreduce_fused_replayable
+ public:
+  // 0 = none, 1 = work only, 2 = sync only, + 4 when allreduce is disabled (for tests of the parsing)
+  int bisectMode() const { return (work_only_ ? 1 : 0) | (sync_only_ ? 2 : 0) | (disable_allreduce_ ? 4 : 0); }
+  // (collectives that met at the rendezvous of the host threads, collectives that only enqueued)
+  std::pair<uint64_t, uint64_t> rendezvousCounts() const { return {rendezvous_count_, enqueue_only_count_}; }
+ private:
   unsigned waiting_cus_ = 128;  // what all ranks' waiting launches may hold together (MCCL_PG_WAITING_COMPUTE_UNITS)
   bool distinct_pids_ = false;          // every rank is a process of its own
   const char* last_title_ = nullptr;  // the collective this rank enqueued last, for failure reports
@@ -421,6 +446,7 @@ class ProcessGroupCCL : public c10d::Backend {
   std::vector<void*> fused_stage_[2];       // rank r's staging buffer of the one-launch allreduce, per slot
   std::vector<void*> fused_flags_[2];
   void* done_counter_ = nullptr;            // this rank's workgroup counter of the one-launch collectives
+  void* fused_state_ = nullptr;             // this rank's device-resident epoch of the one-launch small allreduce
   void* status_dev_ = nullptr;              // device address of shared_->status
   std::shared_ptr<GroupShared> shared_;
 
@@ -434,6 +460,7 @@ class ProcessGroupCCL : public c10d::Backend {
   int export_clock_ = 0;                    // next table entry to evict
   int recent_export_[2] = {-1, -1};         // entries of the last two offers: not evicted
   uint64_t rendezvous_count_ = 0;           // device-synchronised collectives that met at the host rendezvous
+  uint64_t enqueue_only_count_ = 0;         // device-synchronised collectives that needed none (recorded ones included)
   struct Import {
     void* base = nullptr;
     uint64_t gen = 0;

@@ -71,5 +71,9 @@ PYBIND11_MODULE(_C, m) {
                  c10::make_intrusive<ProcessGroupCCL>(store, rank, size, timeout));
            }),
            py::arg("store"), py::arg("rank"), py::arg("size"),
-           py::arg("timeout") = std::chrono::milliseconds(ProcessGroupCCL::OP_TIMEOUT_MILLIS));
+           py::arg("timeout") = std::chrono::milliseconds(ProcessGroupCCL::OP_TIMEOUT_MILLIS))
+      // what the bisecting switches of the environment parsed to: 1 = work only, 2 = sync only, + 4 = allreduce disabled
+      .def("_bisect_mode", &ProcessGroupCCL::bisectMode)
+      // collectives of this group that met at the host rendezvous / that reused a cached one
+      .def("_rendezvous_counts", &ProcessGroupCCL::rendezvousCounts);
 }

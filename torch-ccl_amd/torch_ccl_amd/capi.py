@@ -23,6 +23,8 @@ VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
  TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS, TUNE_COPY_VECTORS_PER_LANE, TUNE_COPY_STREAM_STORES,
  TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU, TUNE_XRANK_CACHED_LOADS) = range(13)
 COPY_SHARED_SOURCES = 1  # flag of mccl_copy_segments_sync
+FUSED_WORK_ONLY, FUSED_SYNC_ONLY = 1, 2  # flags of mccl_allreduce_fused_replayable
+FUSED_STATE_BYTES = 128
 MAX_RANKS = 64
 
 TORCH_DTYPE = {
@@ -37,7 +39,7 @@ EXPORTS = (
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
-    "mccl_rank_barrier", "mccl_allreduce_fused", "mccl_fanout_sync",
+    "mccl_rank_barrier", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
     "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
     "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
@@ -86,6 +88,7 @@ def lib():
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
     L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, ctypes.c_uint, vp]
+    L.mccl_allreduce_fused_replayable.argtypes = [vp, vp, sz, i32, i32, vp, vp, sz, sz, vp, i32, i32, ctypes.c_uint64, vp, ctypes.c_uint, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
     L.mccl_fanout_sync.argtypes = [vp, vp, i32, sz, vp, vp]
     L.mccl_reduce_sync.argtypes = [vp, vp, sz, i32, i32, vp, vp]
