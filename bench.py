@@ -100,8 +100,20 @@ def cpu_baseline(torch, host_inputs, n, count):
             "ms_per_step": round(dt * 1e3, 3)}, out
 
 
-def _gloo_rank(rank, world, store_path, backend, cases, out_path):
-    """One host process of the N-process CPU baseline: same op, same (seed, rank) data, CPU tensors."""
+def c5_split_matrix(torch, world, tokens=4096, topk=8, experts=256):
+    """S[src][dst]: rows rank src sends to rank dst when each of its tokens goes to its top-k experts
+    (router logits N(0,1) per (seed, rank)) and rank d holds experts [d * experts/world, ...)."""
+    S = torch.zeros(world, world, dtype=torch.int64)
+    for r in range(world):
+        g = rank_generator(torch, SEED, r)
+        chosen = torch.topk(torch.randn(tokens, experts, generator=g), topk, dim=1).indices
+        S[r] = torch.bincount(chosen.reshape(-1) // (experts // world), minlength=world)
+    return S
+
+
+def _gloo_rank(rank, world, store_path, backend, cases, out_path, keep_path):
+    """One host process of the N-process CPU baseline: same op, same (seed, rank) data, CPU tensors.
+    A case that this backend cannot run is reported as such, not dropped."""
     os.dup2(2, 1)  # keep the parent's stdout clean for the one JSON line (gloo prints connection notes)
     import torch
     import torch.distributed as dist
@@ -109,24 +121,60 @@ def _gloo_rank(rank, world, store_path, backend, cases, out_path):
     store = dist.FileStore(store_path, world)
     dist.init_process_group(backend, store=store, rank=rank, world_size=world)
     res = {}
-    for name, count, dtype_name, std, warm, iters in cases:
+    for case in cases:
+        name, op, count, dtype_name, warm, iters = case["name"], case["op"], case["count"], case["dtype"], case["warm"], case["iters"]
         dtype = getattr(torch, dtype_name)
-        g = rank_generator(torch, SEED, rank)
-        x = (torch.randn(count, generator=g, dtype=torch.float32) * std).to(dtype)
-        t = x.clone()
-        for _ in range(warm):
-            t.copy_(x)
-            dist.all_reduce(t)
-        ts = []
-        for _ in range(iters):
-            t.copy_(x)
-            dist.barrier()
-            t0 = time.perf_counter()
-            dist.all_reduce(t)
-            ts.append(time.perf_counter() - t0)
-        ts.sort()
-        res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters,
-                     "checksum": float(t.float().sum())}
+        try:
+            g = rank_generator(torch, SEED, rank)
+            if case.get("dist") == "uniform":
+                x = (torch.rand(count, generator=g, dtype=torch.float32) * 2 - 1).to(dtype)
+            else:  # in pieces: the fp32 samples of a 1 GiB bf16 gradient would take 2 GiB per process
+                x = torch.empty(count, dtype=dtype)
+                for o in range(0, count, 1 << 26):
+                    n = min(1 << 26, count - o)
+                    x[o:o + n] = (torch.randn(n, generator=g, dtype=torch.float32) * case["std"]).to(dtype)
+            if op == "all_reduce":
+                t = x.clone()
+
+                def prepare():
+                    t.copy_(x)
+
+                def run():
+                    dist.all_reduce(t)
+            elif op == "reduce_scatter_tensor":
+                t = torch.empty(count // world, dtype=dtype)
+                prepare = lambda: None  # noqa: E731
+
+                def run():
+                    dist.reduce_scatter_tensor(t, x)
+            elif op == "all_to_all_single":
+                S = c5_split_matrix(torch, world)
+                hidden = case["hidden"]
+                x = x.view(-1, hidden)
+                t = torch.empty(int(S[:, rank].sum()), hidden, dtype=dtype)
+                prepare = lambda: None  # noqa: E731
+
+                def run():
+                    dist.all_to_all_single(t, x, S[:, rank].tolist(), S[rank].tolist())
+            else:
+                raise ValueError(op)
+            for _ in range(warm):
+                prepare()
+                run()
+            ts = []
+            for _ in range(iters):
+                prepare()
+                dist.barrier()
+                t0 = time.perf_counter()
+                run()
+                ts.append(time.perf_counter() - t0)
+            ts.sort()
+            res[name] = {"p50_us": ts[len(ts) // 2] * 1e6, "p99_us": percentile(ts, 0.99) * 1e6, "iters": iters}
+            if case.get("keep") and rank == 0:
+                torch.save(t, keep_path)
+            del x, t
+        except Exception as e:  # e.g. an op this backend does not implement for CPU tensors
+            res[name] = {"error": "%s on the %s backend: %s" % (op, backend, repr(e)[:200])}
     if rank == 0:
         with open(out_path, "w") as f:
             json.dump(res, f)
@@ -180,6 +228,47 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
         torch.cuda.synchronize()
         res[name]["back_to_back_us"] = (time.perf_counter() - t0) / 20 * 1e6
         del x, t
+    # C2 as a decode loop runs it: 32 allreduces recorded into one HIP graph per rank process (one launch
+    # per process for all 32), replayed; once bare and once with a small kernel of the caller's between them
+    try:
+        xs = torch.zeros(32, 16 * 8192, dtype=torch.bfloat16, device="cuda:0")
+        one = torch.zeros(64, device="cuda:0")
+        for between in (False, True):
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for k in range(32):
+                    dist.all_reduce(xs[k])
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for k in range(32):
+                    dist.all_reduce(xs[k])
+                    if between:
+                        one.add_(1.0)
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(30):
+                xs.fill_(2.0 ** -10)
+                torch.cuda.synchronize()
+                dist.barrier()
+                t0 = time.perf_counter()
+                graph.replay()
+                torch.cuda.synchronize()
+                ts.append(time.perf_counter() - t0)
+            ts.sort()
+            ok = bool((xs == 2.0 ** -10 * world).all())
+            key = "c2_per_allreduce_in_replayed_graph_with_a_small_kernel_between_us" if between else "c2_per_allreduce_in_replayed_graph_us"
+            res[key] = {"p50_us": ts[len(ts) // 2] / 32 * 1e6, "p99_us": percentile(ts, 0.99) / 32 * 1e6, "replays": 30,
+                        "allreduces_per_graph": 32, "results_exact": ok}
+            del graph
+        del xs
+    except Exception as e:  # bisecting switches: waits or data are missing, results are not checked
+        res["c2_per_allreduce_in_replayed_graph_us"] = {"error": repr(e)[:200]}
+
     # the floor of this way of timing: one trivial kernel of this process + synchronize, with all rank
     # processes doing the same at the same moment (every launch waits for its process's turn)
     one = torch.zeros(64, device="cuda:0")
@@ -222,11 +311,7 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     del grad, shard
     # C5 through the backend: all_to_all_single with the routing counts of the 256-expert reading
     tokens, hidden, topk = 4096, 7168, 8
-    S = torch.zeros(world, world, dtype=torch.int64)
-    for r in range(world):
-        g = rank_generator(torch, SEED, r)
-        experts = torch.topk(torch.randn(tokens, 256, generator=g), topk, dim=1).indices
-        S[r] = torch.bincount(experts.reshape(-1) // (256 // world), minlength=world)
+    S = c5_split_matrix(torch, world, tokens, topk)
     a_in = torch.empty(tokens * topk, hidden, dtype=torch.bfloat16, device="cuda:0").normal_()
     a_out = torch.empty(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device="cuda:0")
     res["c5_all_to_all_single_448MiB_bf16"] = timed(
@@ -244,30 +329,31 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     dist.destroy_process_group()
 
 
-def backend_path(world=8, sync=None):
+def backend_path(world=8, env=None):
     """The drop-in c10d path end to end: `world` rank processes share cuda:0 and call dist.* on GPU
-    tensors, timed on the host around the call plus a synchronize.  sync: value of MCCL_PG_SYNC for
-    the rank processes (None = the backend's default); with a value only C2 and C3 are timed."""
+    tensors, timed on the host around the call plus a synchronize.  env: environment of the rank
+    processes beyond this process's (None = the backend's defaults); with one only C2 and C3 are timed."""
     import tempfile
     import torch.multiprocessing as mp
     cases = [("c2_256KiB_bf16", 16 * 8192, 20, 200), ("c3_64MiB_bf16", 4096 * 8192, 3, 20)]
-    before = os.environ.get("MCCL_PG_SYNC")
-    if sync is not None:
-        os.environ["MCCL_PG_SYNC"] = sync  # the spawned rank processes inherit it
+    before = {k: os.environ.get(k) for k in (env or {})}
+    os.environ.update(env or {})  # the spawned rank processes inherit it
     try:
         with tempfile.TemporaryDirectory() as d:
             out_path = os.path.join(d, "res.json")
-            mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path, sync is None), nprocs=world, join=True)
+            mp.spawn(_backend_rank, args=(world, os.path.join(d, "store"), cases, out_path, env is None), nprocs=world, join=True)
             with open(out_path) as f:
                 res = json.load(f)
     finally:
-        if sync is not None:
-            if before is None:
-                del os.environ["MCCL_PG_SYNC"]
+        for k, v in before.items():
+            if v is None:
+                del os.environ[k]
             else:
-                os.environ["MCCL_PG_SYNC"] = before
-    if sync is not None:
-        return {name: {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()} for name in res}
+                os.environ[k] = v
+    def rounded(d):
+        return {k: (round(v, 1) if isinstance(v, float) else rounded(v) if isinstance(v, dict) else v) for k, v in d.items()}
+    if env is not None:
+        return rounded(res)
     out = {"processes": world, "note": "host-timed dist.* call + synchronize per rank process; all ranks share the one "
                                        "GPU.  The ranks wait for each other on the device: large collectives (C3, C4, C5) in "
                                        "a one-wavefront barrier kernel in front of the data kernel, whose last workgroup "
@@ -279,15 +365,18 @@ def backend_path(world=8, sync=None):
                                        "waits_inside_the_data_kernel: the same with MCCL_PG_SYNC=kernel (one launch per "
                                        "collective; not the default because the waiting grids of 7 ranks can keep a "
                                        "register-heavy kernel of the 8th from starting)"}
-    for name in res:
-        out[name] = {k: (round(v, 1) if isinstance(v, float) else v) for k, v in res[name].items()}
+    out.update(rounded(res))
     return out
 
 
-def gloo_baseline(world=8):
-    """N host processes running the same allreduce through a CPU c10d backend: the reference's
-    "ccl" backend when its wheel is installed, else gloo (the stand-in the reference's own CPU
-    harness uses, tests/DeepSpeed_test/testccl_cpu.py:20).  Reported baseline only."""
+def gloo_baseline(world=8, c1_gpu_output=None):
+    """N host processes running the same collectives through a CPU c10d backend: the reference's
+    "ccl" backend (src/cpu/cpu_ccl.cpp:306-337 allreduce, 819-868 reduce_scatter, 870-961 alltoall)
+    when its wheel is installed, else gloo (the stand-in the reference's own CPU harness uses,
+    tests/DeepSpeed_test/testccl_cpu.py:20).  C1 runs with 2 processes and its output is compared bit
+    for bit with the GPU's (c1_gpu_output: CPU tensor, or None); C2-C5 with `world`.  Reported
+    baseline only; the iteration counts of the large cases are cut to keep the whole leg near a
+    minute, and say so."""
     import importlib.util
     import tempfile
     import torch
@@ -296,22 +385,51 @@ def gloo_baseline(world=8):
     spec = importlib.util.find_spec("oneccl_bindings_for_pytorch")
     reference_wheel = spec is not None and spec.origin and not os.path.abspath(spec.origin).startswith(ROOT + os.sep)
     backend = "ccl" if reference_wheel else "gloo"
-    cases = [("c2_256KiB_bf16", 16 * 8192, "bfloat16", 0.02, 20, 300),
-             ("c3_64MiB_bf16", 4096 * 8192, "bfloat16", 0.02, 3, 12)]
-    with tempfile.TemporaryDirectory() as d:
-        out_path = os.path.join(d, "res.json")
-        mp.spawn(_gloo_rank, args=(world, os.path.join(d, "store"), backend, cases, out_path),
-                 nprocs=world, join=True)
-        with open(out_path) as f:
-            res = json.load(f)
+    try:
+        import psutil
+        ram_gib = psutil.virtual_memory().available / 2**30
+    except Exception:
+        ram_gib = 0.0
+    c4_factor = 1 if ram_gib >= 24 else 8
+    c4_count = 536_870_912 // c4_factor
+    tokens, hidden, topk = 4096, 7168, 8
+    c1 = [dict(name="c1_16MiB_fp32_2proc", op="all_reduce", count=4_194_304, dtype="float32", dist="uniform", warm=5, iters=20, keep=True)]
+    cases = [dict(name="c2_256KiB_bf16", op="all_reduce", count=16 * 8192, dtype="bfloat16", std=0.02, warm=20, iters=300),
+             dict(name="c3_64MiB_bf16", op="all_reduce", count=4096 * 8192, dtype="bfloat16", std=0.02, warm=3, iters=12),
+             dict(name="c4_reduce_scatter_tensor_bf16", op="reduce_scatter_tensor", count=c4_count, dtype="bfloat16", std=1e-3, warm=1, iters=3),
+             dict(name="c5_all_to_all_single_bf16", op="all_to_all_single", count=tokens * topk * hidden, dtype="bfloat16", std=1.0,
+                  hidden=hidden, warm=1, iters=5)]
     out = {"backend": backend, "processes": world, "host_cores": len(os.sched_getaffinity(0)),
            "os_cpu_count": os.cpu_count(), "torch": torch.__version__,
-           "threads_per_process": max(1, len(os.sched_getaffinity(0)) // world), "pinning": "none"}
-    for name, count, dtype_name, std, warm, iters in cases:
-        r = res[name]
-        nbytes = count * 2
-        out[name] = {"p50_us": round(r["p50_us"], 1), "p99_us": round(r["p99_us"], 1), "iters": r["iters"],
-                     "GBps_effective": round((world + 1) * nbytes / r["p50_us"] / 1e3, 3)}
+           "threads_per_process": max(1, len(os.sched_getaffinity(0)) // world), "pinning": "none",
+           "note": "median of host-timed calls between barriers; effective GB/s = algorithmic bytes of the collective "
+                   "((N+1) x S for the reductions, 2 x rows moved for the alltoall) / p50; C1 with 2 processes, the rest with %d; "
+                   "C4 and C5 with 1 warm-up and 3 / 5 timed calls (a call takes seconds)" % world}
+    with tempfile.TemporaryDirectory() as d:
+        for w, group in ((2, c1), (world, cases)):
+            out_path, keep_path = os.path.join(d, "res%d.json" % w), os.path.join(d, "keep%d.pt" % w)
+            mp.spawn(_gloo_rank, args=(w, os.path.join(d, "store%d" % w), backend, group, out_path, keep_path), nprocs=w, join=True)
+            with open(out_path) as f:
+                res = json.load(f)
+            for case in group:
+                r = res[case["name"]]
+                if "error" in r:
+                    out[case["name"]] = r
+                    continue
+                es = 4 if case["dtype"] == "float32" else 2
+                if case["op"] == "all_reduce":
+                    alg = (w + 1) * case["count"] * es
+                elif case["op"] == "reduce_scatter_tensor":
+                    alg = (w + 1) * case["count"] * es  # all ranks' shards together: N inputs read, one gradient's worth written
+                else:
+                    alg = 2 * w * case["count"] * es
+                out[case["name"]] = {"p50_us": round(r["p50_us"], 1), "p99_us": round(r["p99_us"], 1), "iters": r["iters"],
+                                     "GBps_effective": round(alg / r["p50_us"] / 1e3, 3)}
+            if w == 2 and os.path.exists(keep_path) and c1_gpu_output is not None:
+                cpu_out = torch.load(keep_path, weights_only=True)
+                out["c1_gpu_equals_cpu_bit_exact"] = bool(torch.equal(cpu_out.view(torch.int32), c1_gpu_output.view(torch.int32)))
+    if c4_factor != 1:
+        out["c4_reduce_scatter_tensor_bf16"]["scaled_down_by"] = c4_factor
     return out
 
 
@@ -348,7 +466,11 @@ def main():
     if "backend" in extras:
         try:
             backend_result = backend_path(8)
-            backend_result["waits_inside_the_data_kernel"] = backend_path(8, sync="kernel")
+            backend_result["waits_inside_the_data_kernel"] = backend_path(8, env={"MCCL_PG_SYNC": "kernel"})
+            # the reference's bisecting switches (src/gpu/dpcpp_ccl.cpp:56-85): what the same calls cost
+            # without their cross-rank waits, and what the waits cost alone (neither produces results)
+            backend_result["work_only"] = backend_path(8, env={"MCCL_PG_WORK_ONLY": "1"})
+            backend_result["sync_only"] = backend_path(8, env={"MCCL_PG_SYNC_ONLY": "1"})
             log("c10d backend:", json.dumps(backend_result))
         except Exception as e:  # informational: never fails the benchmark
             backend_result = {"error": repr(e)[:300]}
@@ -429,6 +551,8 @@ def main():
     same = torch.equal(out.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
     result["parity_check"] = "bit-exact vs on-device fp32 chain" if same else "MISMATCH"
     del acc
+
+    c1_gpu_output = None  # kept for the bit-for-bit comparison with the 2-process CPU run
 
     # ---------------- the same workload with all nine buffers carved from one allocation ----------------
     if "placement" in extras:
@@ -683,6 +807,7 @@ def main():
         o = torch.empty(c1, dtype=torch.float32, device=dev)
         us = benchlib.reduce_throughput([a], [o], warmup=20, iters=200)
         ok = torch.equal(o, a[0] + a[1])
+        c1_gpu_output = o.cpu()
         shapes = {name: round(benchlib.reduce_throughput([a], [o], variant=v, warmup=20, iters=200), 2)
                   for name, v in (("small", capi.VARIANT_SMALL), ("persistent", capi.VARIANT_PERSISTENT),
                                   ("stream", capi.VARIANT_STREAM))}
@@ -854,7 +979,11 @@ def main():
     # ---------------- N-process CPU c10d baseline (gloo unless the reference's wheel exists) ----------------
     if "gloo" in extras and not args.no_cpu:
         try:
-            result["cpu_c10d_baseline"] = gloo_baseline(N)
+            if c1_gpu_output is None:  # C1 on the GPU for the cross-check, when its own leg did not run
+                c1_in = [(torch.rand(4_194_304, generator=rank_generator(torch, SEED, r), dtype=torch.float32) * 2 - 1).to(dev) for r in range(2)]
+                c1_gpu_output = mccl.reduce_n(c1_in, op=mccl.SUM).cpu()
+                del c1_in
+            result["cpu_c10d_baseline"] = gloo_baseline(N, c1_gpu_output)
             log("CPU c10d:", json.dumps(result["cpu_c10d_baseline"]))
         except Exception as e:  # reported baseline only: never fails the benchmark
             result["cpu_c10d_baseline"] = {"error": repr(e)[:300]}

@@ -206,6 +206,27 @@ def oracle_cases(pg, rank, world):
         opts.reduceOp = op
         pg.allreduce([t], opts).wait()
         assert np.array_equal(bits(t), bits_np(O.reduce([to_carrier(h) for h in host], O.F32, ocode))), opname
+    # AVG against the oracle's (sum in ascending rank order at the accumulation width, one division,
+    # one rounding): through the one-launch small allreduce, the in-place allreduce of the peers'
+    # tensors (from 1 MiB on), the two-shot form and reduce_scatter_tensor
+    for dtype, count in ((torch.bfloat16, 131072), (torch.float32, 1000), (torch.bfloat16, (1 << 20) + 77), (torch.float32, (1 << 19) + 3),
+                         (torch.float16, (3 << 20) + 1), (torch.float64, (1 << 20) + 5), (torch.bfloat16, (4 << 20) + 777)):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(count, dtype, r, seed=12, scale=1.0) for r in range(world)]
+        t = host[rank].to(DEV)
+        opts = c10d.AllreduceOptions()
+        opts.reduceOp = c10d.ReduceOp.AVG
+        pg.allreduce([t], opts).wait()
+        assert np.array_equal(bits(t), bits_np(O.reduce([to_carrier(h) for h in host], code, O.AVG))), ("avg", dtype, count)
+    for dtype, m in ((torch.bfloat16, 70001), (torch.float32, (1 << 18) + 9)):
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(world * m, dtype, r, seed=13, scale=1.0) for r in range(world)]
+        out = torch.empty(m, dtype=dtype, device=DEV)
+        opts = c10d.ReduceScatterOptions()
+        opts.reduceOp = c10d.ReduceOp.AVG
+        pg._reduce_scatter_base(out, host[rank].to(DEV), opts).wait()
+        want = O.reduce_scatter([to_carrier(h) for h in host], code, O.AVG, shard_first=rank, shard_num=1)[0]
+        assert np.array_equal(bits(out), bits_np(want)), ("reduce_scatter avg", dtype)
     # rooted reduce: only the root's tensor changes, to the oracle's bits
     for dtype, count, op, ocode in ((torch.bfloat16, 300001, c10d.ReduceOp.SUM, O.SUM), (torch.float32, 77, c10d.ReduceOp.MAX, O.MAX),
                                     (torch.int64, 4097, c10d.ReduceOp.PRODUCT, O.PROD)):
@@ -273,7 +294,7 @@ def dist_api_cases(rank, world):
     # AVG
     t = torch.full((100,), float(rank), device=DEV)
     dist.all_reduce(t, op=dist.ReduceOp.AVG)
-    assert torch.allclose(t.cpu(), torch.full((100,), (world - 1) / 2.0))
+    assert torch.equal(t.cpu(), torch.full((100,), (world - 1) / 2.0))  # small integers over W: exact in fp32 for these world sizes
     # coalescing manager (:667-693): two 8-element allreduces equal one 16-element allreduce
     small = [torch.ones(8, device=DEV) for _ in range(2)]
     with c10d._coalescing_manager(device=torch.device(DEV)):

@@ -75,3 +75,23 @@ def test_reference_import_name_registers_the_backend(pkg):
     assert os.path.isdir(torch_ccl.cwd)
     a, b = torch.zeros(4), torch.zeros(4, 4).t()
     assert torch_ccl.is_available([a]) and not torch_ccl.is_available([b]) and not torch_ccl.is_available([a, a])
+
+
+@pytest.mark.parametrize("env,mode", [({}, 0), ({"TORCH_CCL_WORK_ONLY": "1"}, 1), ({"MCCL_PG_WORK_ONLY": "1"}, 1),
+                                      ({"TORCH_CCL_SYNC_ONLY": "1"}, 2), ({"MCCL_PG_SYNC_ONLY": "1"}, 2),
+                                      ({"TORCH_CCL_DISABLE_ALLREDUCE": "1"}, 4),
+                                      ({"TORCH_CCL_WORK_ONLY": "1", "TORCH_CCL_DISABLE_ALLREDUCE": "1"}, 5),
+                                      ({"TORCH_CCL_WORK_ONLY": "0", "MCCL_PG_SYNC_ONLY": "0"}, 0)])
+def test_bisecting_switches_parse(pkg, monkeypatch, env, mode):
+    """TORCH_CCL_WORK_ONLY / TORCH_CCL_SYNC_ONLY / TORCH_CCL_DISABLE_ALLREDUCE of the reference
+    (src/gpu/dpcpp_ccl.cpp:56-85), read when the group is constructed."""
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    assert _pg()._bisect_mode() == mode
+
+
+def test_work_only_and_sync_only_exclude_each_other(pkg, monkeypatch):
+    monkeypatch.setenv("TORCH_CCL_WORK_ONLY", "1")
+    monkeypatch.setenv("MCCL_PG_SYNC_ONLY", "1")
+    with pytest.raises(RuntimeError, match="exclude each other"):
+        _pg()
