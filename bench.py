@@ -233,8 +233,10 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     try:
         xs = torch.zeros(32, 16 * 8192, dtype=torch.bfloat16, device="cuda:0")
         one = torch.zeros(64, device="cuda:0")
+        side = torch.cuda.Stream()  # ONE stream beside the default one for warm-up and capture: every further
+        # stream is another hardware queue of this process, and with more queues than the GPU maps at
+        # once the scheduler time-slices the rank processes, which a collective cannot stand
         for between in (False, True):
-            side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 for k in range(32):
@@ -242,7 +244,7 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with torch.cuda.graph(graph, stream=side):
                 for k in range(32):
                     dist.all_reduce(xs[k])
                     if between:
@@ -336,8 +338,10 @@ def backend_path(world=8, env=None):
     import tempfile
     import torch.multiprocessing as mp
     cases = [("c2_256KiB_bf16", 16 * 8192, 20, 200), ("c3_64MiB_bf16", 4096 * 8192, 3, 20)]
-    before = {k: os.environ.get(k) for k in (env or {})}
-    os.environ.update(env or {})  # the spawned rank processes inherit it
+    env_all = {"GPU_MAX_HW_QUEUES": "2"}  # what rank processes that share a GPU should run with: no more hardware queues than the GPU maps at once
+    env_all.update(env or {})
+    before = {k: os.environ.get(k) for k in env_all}
+    os.environ.update(env_all)  # the spawned rank processes inherit it
     try:
         with tempfile.TemporaryDirectory() as d:
             out_path = os.path.join(d, "res.json")
@@ -355,7 +359,7 @@ def backend_path(world=8, env=None):
     if env is not None:
         return rounded(res)
     out = {"processes": world, "note": "host-timed dist.* call + synchronize per rank process; all ranks share the one "
-                                       "GPU.  The ranks wait for each other on the device: large collectives (C3, C4, C5) in "
+                                       "GPU (GPU_MAX_HW_QUEUES=2 per process).  The ranks wait for each other on the device: large collectives (C3, C4, C5) in "
                                        "a one-wavefront barrier kernel in front of the data kernel, whose last workgroup "
                                        "waits for the closing epoch (two launches); small and medium ones (C2) in the "
                                        "data kernel itself, limited to workgroups that hold at most half of the compute "
@@ -675,15 +679,17 @@ def main():
     if "xrank" in extras:
         L = capi.lib()
         word = torch.zeros(8, dtype=torch.int64, device=dev)
-        counter = torch.zeros(256, dtype=torch.int32, device=dev)  # MCCL_SYNC_COUNTER_BYTES
+        counter = torch.zeros(1024, dtype=torch.int32, device=dev)  # MCCL_SYNC_COUNTER_BYTES
         status = torch.zeros(16, dtype=torch.int32).pin_memory()
         words = capi.ptr_table([word.data_ptr()] * N)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         calls = [0]
 
+        opening = [True]  # False: the form the backend runs behind its barrier kernel (no opening wait, closing wait)
+
         def xsync(rank):
             calls[0] += 1
-            return capi.XSync(ctypes.cast(words, ctypes.c_void_p), N, rank, 4 * calls[0] + 1, 4 * calls[0] + 3,
+            return capi.XSync(ctypes.cast(words, ctypes.c_void_p), N, rank, 4 * calls[0] + 1 if opening[0] else 0, 4 * calls[0] + 3,
                               counter.data_ptr(), 5_000_000, status.data_ptr())
 
         def event_us(fn, reps=20):
@@ -743,8 +749,26 @@ def main():
         xr["fanout_sync_64MiB_into_8_outputs"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
                                                   "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
                                                   "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
-        del gathered
         L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget)
+        # the default between rank processes: a barrier kernel in front, so the data kernel does not wait
+        # at its start (fresh workgroups for the shard reduction and the push) and its last workgroup
+        # does the closing wait
+        opening[0] = False
+        behind = {}
+        xout.zero_()
+        us = event_us(reduce_sync)
+        behind["reduce_sync_8x64MiB_to_64MiB"] = {"us": round(us, 1), "pct_of_peak": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                                  "bit_identical_to_reduce_n": bool(torch.equal(xout.view(torch.int16), out.view(torch.int16)))}
+        us = event_us(allreduce_rank0)
+        behind["allreduce_sync_rank0_shard_of_8x64MiB"] = {"us": round(us, 1), "pct_of_peak": round(2 * N * shard * 2 / us / 1e3 / PEAK_HBM_GBS * 100, 1)}
+        for g in gathered:
+            g[:COUNT].zero_()
+        us = event_us(fanout_rank0)
+        behind["fanout_sync_64MiB_into_8_outputs"] = {"us": round(us, 1), "pct_of_peak": round((N + 1) * COUNT * 2 / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                                      "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
+        xr["behind_a_barrier_kernel"] = behind
+        opening[0] = True
+        del gathered
         assert status.tolist()[:2] == [0, 0], status.tolist()
         xr["wavefronts_per_launch"] = int(budget)
         xr["note"] = ("single process: every rank's flag word is the same word, so no launch waits, and a launch has "

@@ -102,8 +102,19 @@ typedef enum {
   MCCL_TUNE_GATHER_WAVES_PER_CU = 11,     /* residency cap of the row gather / fused MoE dispatch */
   MCCL_TUNE_XRANK_CACHED_LOADS = 12,      /* one-launch reductions: 1 = the peers' tensors are read
                                              through the caches after one invalidate per workgroup,
-                                             0 = past the caches, access by access */
-  MCCL_TUNE_COUNT_ = 13
+                                             0 = past the caches, access by access, 2 (default) =
+                                             through the caches without an invalidate when the
+                                             launch does not wait at its start (whatever the peers
+                                             wrote, they wrote in kernels that had ended before this
+                                             one began: its caches start clean), else as 0 */
+  MCCL_TUNE_XRANK_FRESH_WAVES_PER_CU = 13, /* one-launch reductions and pushes that do not wait at their
+                                             start (ready_epoch 0: the caller has ordered the ranks, e.g.
+                                             with mccl_rank_barrier in front): residency cap of their
+                                             single-wavefront workgroups, 32 and more = none */
+  MCCL_TUNE_XRANK_FRESH_MAX_WAVES = 14,   /* the same launches: at most this many workgroups (a walk
+                                             over several tiles each above it); 0 = one workgroup per
+                                             tile (reductions) or per two tiles (pushes) */
+  MCCL_TUNE_COUNT_ = 15
 } mccl_tune_t;
 
 #define MCCL_MAX_RANKS 64
@@ -248,14 +259,18 @@ int mccl_allreduce_fused_replayable(const void* in, void* out, size_t count, int
  *   words[r]: rank r's 64-bit word as for mccl_rank_barrier (the same word may serve both; epochs
  * grow: ready_epoch of a call > any epoch used before, done_epoch > ready_epoch).  done_counter:
  * MCCL_SYNC_COUNTER_BYTES of this rank's device memory, 64-byte aligned, zero before the first call
- * (the kernel leaves them zero): the workgroups count themselves out there.  ready_epoch == 0: no
+ * (the kernel leaves them zero): the workgroups count themselves out there, and the workgroup with
+ * the highest index watches the counters and does the closing wait.  ready_epoch == 0: no
  * opening wait, for callers that have ordered the start of the ranks themselves -- with an
  * mccl_rank_barrier launch in front (then only the kernel's last workgroup ever waits, for the
  * closing epoch: one wavefront per rank instead of the whole grid, which matters when several
  * ranks share a GPU with other kernels), or with host barriers around the launch (done_epoch 0 as
  * well: the kernel does not wait at all; words, counters and status are then not used).
- * Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids
- * are sized so that all ranks' launches are resident together (MCCL_TUNE_XRANK_WAVES_ALL_RANKS).
+ * Waits are bounded and reported like mccl_rank_barrier's.  At most 8 ranks.  The grids of launches
+ * that wait at their start are sized so that all ranks' launches are resident together
+ * (MCCL_TUNE_XRANK_WAVES_ALL_RANKS); a launch without an opening wait can keep nobody out, and the
+ * shard reduction and the push then run as fresh workgroups of one or two tiles each
+ * (MCCL_TUNE_XRANK_FRESH_MAX_WAVES, MCCL_TUNE_XRANK_FRESH_WAVES_PER_CU).
  * max_compute_units: 0 -- single-wavefront workgroups, spread over the whole GPU, as many as the
  * budget allows (the fastest shape for large messages); k > 0 -- at most k workgroups of up to 16
  * wavefronts: a workgroup sits on one compute unit, so the launch holds at most k of the GPU's 256
@@ -263,7 +278,7 @@ int mccl_allreduce_fused_replayable(const void* in, void* out, size_t count, int
  * that share a GPU keep the sum over all ranks at half the GPU (8 ranks: 16 each); the message
  * should then be small enough for 16 k wavefronts (a few MiB).
  */
-#define MCCL_SYNC_COUNTER_BYTES 1024
+#define MCCL_SYNC_COUNTER_BYTES 4096
 typedef struct {
   void* const* words;
   int n;

@@ -1081,7 +1081,7 @@ def graph_capture_case(rank, world):
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     big = torch.ones(1 << 20, device=DEV)  # 4 MiB: needs the host rendezvous
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=side):  # (every further stream would be another hardware queue of this process)
         for k in range(K):
             w = dist.all_reduce(X[k], async_op=True)
             w.wait()
@@ -1135,7 +1135,7 @@ def graph_late_rank_case(rank, world):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=side):
         for k in range(2):
             dist.all_reduce(X[k])
     X.fill_(1.0)

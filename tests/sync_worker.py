@@ -220,7 +220,7 @@ def fused_replay_case(rank, world, queues, barrier):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=side):
         for k in range(K):
             call(xs[k], xs[k], count, torch.bfloat16, capi.SUM, 128 // world)
             ticks.add_(1.0)
@@ -276,7 +276,7 @@ def xrank_case(rank, world, queues, barrier):
     BUF = 24 << 20
     shared_in = torch.zeros(BUF, dtype=torch.uint8, device=DEV)      # what the peers read in place
     word = torch.zeros(8, dtype=torch.int64, device=DEV)             # [0]: the sync word
-    counter = torch.zeros(256, dtype=torch.int32, device=DEV)  # MCCL_SYNC_COUNTER_BYTES
+    counter = torch.zeros(1024, dtype=torch.int32, device=DEV)  # MCCL_SYNC_COUNTER_BYTES
     torch.cuda.synchronize()
     shared = _exchange(rank, world, queues, barrier, [shared_in, word])
     words = capi.ptr_table([shared[r][1].data_ptr() for r in range(world)])

@@ -195,9 +195,13 @@ __device__ __forceinline__ Wave this_wave() {
   }
 }
 
-constexpr uint32_t kDoneGroups = 8;
-constexpr uint32_t kDoneStride = 16;  // 32-bit words between two counters: one cache line each
-static_assert((1 + kDoneGroups) * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "counters must fit the block the caller provides");
+constexpr uint32_t kDoneGroups = 16;
+// 32-bit words between two counters: 256 bytes.  Counters on neighbouring 64-byte lines still got in
+// each other's way (a shard reduction of 8 x 64 MiB with one workgroup per tile: 104 us with the
+// counters 64 bytes apart, 93 us at 256 bytes and beyond, 90 us without any counting).
+constexpr uint32_t kDoneStride = 64;
+static_assert(kDoneGroups * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "counters must fit the block the caller provides");
+static_assert(kDoneGroups <= kWave, "one lane of the watching wavefront per counter");
 
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
 __device__ __forceinline__ bool xsync_begin(const XSync& x) {
@@ -215,37 +219,51 @@ __device__ __forceinline__ bool xsync_begin(const XSync& x) {
 }
 
 // Call once per workgroup, by all its lanes, after the workgroup's last access to a peer's buffer.
-__device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups) {
+//
+// Every workgroup counts itself out with an atomic add whose result nobody reads: the wavefront
+// does not wait for it and ends.  The counting is spread over sixteen counters on cache lines of
+// their own, 256 bytes apart (atomics on one address are carried out one after the other, about 7 ns
+// each).  The
+// workgroup with the highest index -- dispatched last, so that it holds its slot for the shortest
+// time -- watches the counters, one lane each, until every workgroup of the launch is out, clears
+// them for the next launch, publishes the closing epoch and waits for the peers'.  No workgroup
+// depends on the watching one, so the order in which the hardware starts workgroups only decides
+// how long that one wavefront stays.  (Counting with a returned value, so that the last workgroup
+// out could tell, kept every workgroup for the round trip of its atomic: with one tile per workgroup
+// that doubled the duration of a 64 MiB shard reduction.)
+//
+// wrote_to_peers: the kernel stores into the peers' buffers (written through), and the closing epoch
+// also says that those stores have arrived; a kernel that only reads them (its loads have returned
+// once their values were used) does not wait for the stores into its own output, which the end of
+// the kernel covers -- a wavefront that waits for its stores keeps its slot for their whole way to
+// memory, and a launch of fresh workgroups lives on slots turning over.
+__device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups, bool wrote_to_peers = true) {
   if (x.done_epoch == 0) return;
-  // this workgroup's reads of the peers' buffers have returned (their values were used): no cache
-  // needs writing back for that
-  wait_own_stores();
+  if (wrote_to_peers) wait_own_stores();  // (no cache needs writing back: the stores were written through)
+  else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x >= kWave) return;  // the first wavefront of the workgroup does the rest
-  const int lane = threadIdx.x;
-  uint32_t last = 0;
-  if (lane == 0) {
-    // Relaxed: the ordering that matters (this workgroup's accesses are complete) was established
-    // above, and an acquire-release atomic would add a cache write-back and invalidate per workgroup.
-    // Counted in two levels -- eight group counters on cache lines of their own, then one for the
-    // groups -- because atomics on one address are carried out one after the other (about 7 ns
-    // each: 29 us for a grid of 4096 workgroups on a single counter).
-    const uint32_t groups = workgroups < kDoneGroups ? 1u : kDoneGroups;
-    const uint32_t g = blockIdx.x % groups;
-    const uint32_t members = (workgroups - g + groups - 1) / groups;
-    uint32_t* mine = x.done_count + kDoneStride * (1 + g);
-    if (__hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == members) {
-      __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-      if (__hip_atomic_fetch_add(x.done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == groups) {
-        last = 1u;
-        __hip_atomic_store(x.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-      }
+  const uint32_t lane = threadIdx.x;
+  const uint32_t groups = workgroups < kDoneGroups ? workgroups : kDoneGroups;
+  // Relaxed: the ordering that matters (this workgroup's accesses are complete) was established
+  // above, and an acquire-release atomic would add a cache write-back and invalidate per workgroup.
+  if (lane == 0) (void)__hip_atomic_fetch_add(x.done_count + kDoneStride * (blockIdx.x % groups), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (blockIdx.x != workgroups - 1) return;
+  // lane g watches counter g: workgroups g, g + groups, ... count there
+  const uint32_t members = lane < groups ? (workgroups - lane + groups - 1) / groups : 0u;
+  const uint64_t t0 = wall_clock64();
+  for (;;) {
+    const uint32_t c = lane < groups ? __hip_atomic_load(x.done_count + kDoneStride * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    if (__builtin_amdgcn_ballot_w64(c != members) == 0) break;
+    if (wall_clock64() - t0 > x.limit_ticks) {  // (a workgroup of this launch never ended: reported as this rank itself)
+      if (lane == 0) report_late(x.status, x.rank, (uint32_t)x.done_epoch);
+      return;
     }
+    __builtin_amdgcn_s_sleep(4);
   }
-  last = __builtin_amdgcn_readfirstlane(last);
-  if (!last) return;
-  if (lane < x.n && lane != x.rank) {
+  if (lane < groups) __hip_atomic_store(x.done_count + kDoneStride * lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+  if (lane == 0) __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  if ((int)lane < x.n && (int)lane != x.rank) {
     if (!wait_flag64(x.word[lane], x.done_epoch, x.limit_ticks)) report_late(x.status, lane, (uint32_t)x.done_epoch);
   }
 }

@@ -44,6 +44,7 @@ struct XRankArgs {
   uint32_t stream_out;                // write out1 past the caches (large reduce_scatter outputs)
   uint32_t aligned_in;                // every in[k] is 8-byte aligned: read past the caches
   uint32_t push;                      // allreduce: write the result over in[k] of every rank k instead of out1
+  uint32_t no_invalidate;             // with aligned_in == 0: the caches are clean already (a kernel boundary lies behind the ranks' barrier)
   XSync sync;
 };
 
@@ -169,12 +170,12 @@ __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankAr
   const int n = a.sync.n;
   const Wave w = this_wave<WPG>();
   if (xsync_begin(a.sync)) {
-    if (!a.aligned_in) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
+    if (!a.aligned_in && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
     if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, w, n);
     else xrank_walk<DT, OP, 0>(a, w, n);
     if (a.tail1 && w.index == w.count - 1) xrank_tail<DT, OP>(a, w, n);
   }
-  xsync_end(a.sync, gridDim.x);
+  xsync_end(a.sync, gridDim.x, a.push != 0);
 }
 
 }  // namespace

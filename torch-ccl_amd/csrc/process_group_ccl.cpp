@@ -68,11 +68,12 @@ constexpr size_t kArenaFusedFlagsOff = 4096;                 // two sets of tile
 constexpr size_t kArenaFusedFlagsStride = 8192;
 constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buffers of 1 MiB, each
 constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
-constexpr size_t kArenaDoneCountOff = 1024;  // MCCL_SYNC_COUNTER_BYTES of workgroup counters of the one-launch collectives
+constexpr size_t kArenaDoneCountOff = 24u << 10;  // MCCL_SYNC_COUNTER_BYTES of workgroup counters of the one-launch collectives
 constexpr size_t kArenaFusedStateOff = 2048;  // MCCL_FUSED_STATE_BYTES: the device-resident epoch of the one-launch small allreduce
 constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
 static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
-static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedStateOff, "the counters end before the epoch state");
+static_assert(kArenaFusedFlagsOff + 2 * kArenaFusedFlagsStride <= kArenaDoneCountOff, "the flags end before the counters");
+static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedStageOff, "the counters end before the staging buffers");
 static_assert(kArenaFusedStateOff + MCCL_FUSED_STATE_BYTES <= kArenaFusedFlagsOff, "the epoch state ends before the flags");
 
 #define HIP_CHECK(expr)                                                                     \

@@ -21,7 +21,8 @@ VARIANT_AUTO, VARIANT_SMALL, VARIANT_PERSISTENT, VARIANT_STREAM = 0, 1, 2, 3
 (TUNE_PERSISTENT_BLOCKS_PER_CU, TUNE_STREAM_WAVES_PER_CU, TUNE_SMALL_MAX_BYTES,
  TUNE_COPY_WAVES_PER_CU, TUNE_STREAM_MIN_TOTAL_BYTES, TUNE_COMBINE_PIECES_PER_WAVE,
  TUNE_COMBINE_WAVES_PER_CU, TUNE_XRANK_WAVES_ALL_RANKS, TUNE_COPY_VECTORS_PER_LANE, TUNE_COPY_STREAM_STORES,
- TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU, TUNE_XRANK_CACHED_LOADS) = range(13)
+ TUNE_COPY_LARGE_MIN_BYTES, TUNE_GATHER_WAVES_PER_CU, TUNE_XRANK_CACHED_LOADS, TUNE_XRANK_FRESH_WAVES_PER_CU,
+ TUNE_XRANK_FRESH_MAX_WAVES) = range(15)
 COPY_SHARED_SOURCES = 1  # flag of mccl_copy_segments_sync
 FUSED_WORK_ONLY, FUSED_SYNC_ONLY = 1, 2  # flags of mccl_allreduce_fused_replayable
 FUSED_STATE_BYTES = 128
