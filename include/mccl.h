@@ -88,10 +88,11 @@ typedef enum {
                                              per CU, each walking several chunks (measured slower) */
   MCCL_TUNE_XRANK_WAVES_ALL_RANKS = 7,    /* wavefronts the launches of ALL ranks of a one-launch
                                              collective (mccl_*_sync) may hold together; each
-                                             rank's grid is this divided by the rank count.  Must
-                                             stay below what the GPU keeps resident at once
-                                             (256 CUs x 32), or ranks could wait for launches
-                                             that find no room */
+                                             rank's grid is this divided by the rank count.  A
+                                             launch that waits at its start is cut further, to the
+                                             rank's share of half of what the kernel's registers
+                                             let the GPU hold at once (asked of the runtime per
+                                             kernel), so that waiting ranks never fill the GPU */
   MCCL_TUNE_COPY_VECTORS_PER_LANE = 8,    /* segmented copy: 2 or 4 vectors of 16 bytes per lane per chunk
                                              (2 KiB or 4 KiB per wavefront); any other value = chosen by
                                              the total size of the call */

@@ -637,6 +637,21 @@ def zero_copy_cases(pg, rank, world):
         full[rank * m * 4:(rank + 1) * m * 4].copy_(host[rank])
         pg._allgather_base(full, full[rank * m * 4:(rank + 1) * m * 4]).wait()
         assert np.array_equal(bits(full), np.concatenate([bits(h) for h in host])), ("allgather in place", dtype, m)
+        # aliased, but not the in-place form: the output of reduce_scatter_tensor inside ANOTHER rank's
+        # slice of the input (which that rank reads), the input of all_gather_into_tensor inside another
+        # rank's slice of the output (which that rank writes).  Such calls must be staged, where the
+        # copy-in comes first: the results are those of the calls on separate tensors.
+        other = (rank + 1) % world
+        host = [rank_buffer(world * m, dtype, r, seed=94) for r in range(world)]
+        x = view_of(host[rank], pad)
+        want = O.reduce_scatter([to_carrier(h) for h in host], code, O.SUM, shard_first=rank, shard_num=1)[0]
+        pg._reduce_scatter_base(x[other * m:(other + 1) * m], x).wait()
+        assert np.array_equal(bits(x[other * m:(other + 1) * m]), bits_np(want)), ("reduce_scatter into a foreign slice", dtype, m)
+        host = [rank_buffer(m * 4, dtype, r, seed=95) for r in range(world)]
+        full = torch.zeros(world * m * 4, dtype=dtype, device=DEV)
+        full[other * m * 4:(other + 1) * m * 4].copy_(host[rank])
+        pg._allgather_base(full, full[other * m * 4:(other + 1) * m * 4]).wait()
+        assert np.array_equal(bits(full), np.concatenate([bits(h) for h in host])), ("allgather from a foreign slice", dtype, m)
         root = m % world
         src = rank_buffer(m * 4 + 3, dtype, root, seed=93)
         t = view_of(src if rank == root else torch.zeros_like(src), pad)
@@ -863,7 +878,8 @@ def missing_rank_device_case(pg, rank, world):
             w.wait()
             raise AssertionError("blocking wait on a collective with a missing rank returned")
         except RuntimeError as e:
-            assert "timed out waiting for rank 1 on the device" in str(e), str(e)
+            # (the one-launch allreduce counts its own launches on the device: this is the group's second)
+            assert "timed out waiting for rank 1 on the device (one-launch allreduce #2 of this group" in str(e), str(e)
     else:
         w.wait()  # stream-ordered: returns at once, the failure shows when the device gets there
         torch.cuda.synchronize()
@@ -874,7 +890,7 @@ def missing_rank_device_case(pg, rank, world):
         pg.allreduce([t], c10d.AllreduceOptions())
         raise AssertionError("a failed group accepted another collective")
     except RuntimeError as e:
-        assert "timed out waiting for rank 1" in str(e), str(e)
+        assert "timed out waiting for rank 1 on the device (one-launch allreduce #2 of this group" in str(e), str(e)
 
 
 def late_peer_case(pg, rank, world):
@@ -946,6 +962,14 @@ def env_switch_case(pg, rank, world):
         w.wait()
         if os.environ.get("CCL_BLOCKING_WAIT") == "1":
             assert w.is_completed()
+            # a Work answers for its own collective, not for what the caller enqueues behind it
+            w2 = pg.allreduce([t2.clone()], c10d.AllreduceOptions())
+            w2.wait()
+            a = torch.ones(4096, 4096, device=DEV)
+            for _ in range(40):
+                a = (a @ a) * 1e-4
+            assert w2.is_completed() and w2.is_success()
+            del a
         r = t2 + 1
     side.synchronize()
     assert float(r[0]) == world * (world + 1) + 1 and float(r[-1]) == world * (world + 1) + 1

@@ -99,6 +99,23 @@ def test_overlapping_buffers_are_rejected_before_any_launch(mccl):
     assert b"outputs" in L.mccl_last_error() and b"overlap" in L.mccl_last_error()
 
 
+def test_one_launch_collectives_reject_partial_overlap(mccl):
+    """mccl_reduce_sync: the output may be exactly one of the inputs, nothing else of them;
+    mccl_allreduce_sync: two ranks' tensors may be the same memory, never partly so."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    base = 0x10000000
+    ins = capi.ptr_table([base, base + 0x100000])
+    sy = capi.XSync(None, 2, 0, 0, 0, None, 0, None)  # no waits: words, counters and status are not used
+    assert L.mccl_reduce_sync(ins, ctypes.c_void_p(base + 0x100000 + 64), 4096, capi.F32, capi.SUM, ctypes.byref(sy), None) == -1
+    assert b"partially overlaps input 1" in L.mccl_last_error()
+    assert L.mccl_reduce_sync(ins, ctypes.c_void_p(base - 4096 * 4 + 4), 4096, capi.F32, capi.SUM, ctypes.byref(sy), None) == -1
+    assert b"partially overlaps input 0" in L.mccl_last_error()
+    tens = capi.ptr_table([base, base + 4096 * 4 - 8])
+    assert L.mccl_allreduce_sync(tens, 4096, capi.F32, capi.SUM, ctypes.byref(sy), None) == -1
+    assert b"tensors 0 and 1 partially overlap" in L.mccl_last_error()
+
+
 def test_pack_and_unpack_reject_a_null_flat_buffer(mccl):
     from torch_ccl_amd import capi
     L = capi.lib()

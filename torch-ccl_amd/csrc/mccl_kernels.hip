@@ -205,17 +205,22 @@ hipError_t launch_fused_any(const FusedArgs& a, int dtype, int op, unsigned grou
   }
 }
 
-hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned groups, int packed, unsigned lds, hipStream_t s) {
+// waiting_ranks > 0: the launch waits for that many ranks' launches at its start and is cut to its
+// share of the GPU's residency (reduce_launch.hpp: waiting_share).
+hipError_t launch_xrank_any(const XRankArgs& a, int dtype, int op, unsigned groups, int packed, unsigned lds, unsigned waiting_ranks, hipStream_t s) {
+  int cus_i = 0;
+  if (device_cus(&cus_i) != MCCL_OK) return hipErrorInvalidDevice;
+  const unsigned cus = (unsigned)cus_i;
   switch (dtype) {
-    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, groups, packed, lds, s);
-    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, groups, packed, lds, s);
-    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, groups, packed, lds, s);
-    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, groups, packed, lds, s);
-    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, groups, packed, lds, s);
-    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, groups, packed, lds, s);
-    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, groups, packed, lds, s);
-    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, groups, packed, lds, s);
-    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, groups, packed, lds, s);
+    case MCCL_U8: return mccl_launch_xrank_dt0(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_I8: return mccl_launch_xrank_dt1(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_I16: return mccl_launch_xrank_dt2(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_I32: return mccl_launch_xrank_dt3(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_I64: return mccl_launch_xrank_dt4(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_F16: return mccl_launch_xrank_dt5(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_F32: return mccl_launch_xrank_dt6(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_F64: return mccl_launch_xrank_dt7(&a, op, groups, packed, lds, cus, waiting_ranks, s);
+    case MCCL_BF16: return mccl_launch_xrank_dt8(&a, op, groups, packed, lds, cus, waiting_ranks, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -958,10 +963,20 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
     if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;
   }
   const XShape shape = xrank_shape(chunks, sync);  // (a copy gains nothing from more wavefronts than its share, waits or not)
-  const unsigned grid = shape.groups;
+  unsigned grid = shape.groups;
   if (flags & ~MCCL_COPY_SHARED_SOURCES) return fail(MCCL_ERR_INVALID_ARG, "unknown copy flags 0x%x", flags);
-  if (shape.packed) hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  int cus = 0;
+  rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  if (shape.packed) {
+    static const unsigned per_cu = blocks_per_cu(copy_segments_sync_kernel<kPackedWaves>, kWave * kPackedWaves);
+    if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
+    hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  } else {
+    static const unsigned per_cu = blocks_per_cu(copy_segments_sync_kernel<1>, kWave);
+    if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
+    hipLaunchKernelGGL(copy_segments_sync_kernel<1>, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
@@ -996,8 +1011,19 @@ int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, 
   }
   // (the last wavefront takes the tail: a launch of at least one)
   const XShape shape = xrank_shape(a.tiles, sync, a.sync.ready_epoch != 0, /*fresh_tiles=*/2);
-  if (shape.packed) hipLaunchKernelGGL(fanout_sync_kernel<kPackedWaves>, dim3(shape.groups), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL(fanout_sync_kernel<1>, dim3(shape.groups), dim3(kWave), shape.lds, (hipStream_t)stream, a);
+  unsigned grid = shape.groups;
+  int cus = 0;
+  rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  if (shape.packed) {
+    static const unsigned per_cu = blocks_per_cu(fanout_sync_kernel<kPackedWaves>, kWave * kPackedWaves);
+    if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
+    hipLaunchKernelGGL(fanout_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  } else {
+    static const unsigned per_cu = blocks_per_cu(fanout_sync_kernel<1>, kWave);
+    if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
+    hipLaunchKernelGGL(fanout_sync_kernel<1>, dim3(grid), dim3(kWave), shape.lds, (hipStream_t)stream, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "push kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
@@ -1021,6 +1047,13 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
       a.in[k] = (const char*)in[k];
     }
   }
+  // the output may be exactly one of the inputs (a lane reads element i of every input before it
+  // writes element i); any other overlap would have one workgroup write what another still reads
+  for (int k = 0; k < a.sync.n && count; ++k) {
+    const uintptr_t i0 = (uintptr_t)in[k], o0 = (uintptr_t)out;
+    if (i0 != o0 && i0 < o0 + count * es && o0 < i0 + count * es)
+      return fail(MCCL_ERR_INVALID_ARG, "output partially overlaps input %d", k);
+  }
   const size_t ve = 16 / es;
   const uint64_t vecs = count / ve + (count % ve ? 1 : 0);
   if (vecs + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
@@ -1034,7 +1067,7 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
     if (count && ((uintptr_t)in[k] & 7u)) a.aligned_in = 0;
   apply_cached_loads(&a);
   const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0, /*fresh_tiles=*/1);
-  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, (hipStream_t)stream);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, a.sync.ready_epoch != 0 ? (unsigned)a.sync.n : 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }
@@ -1061,6 +1094,13 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
     if (count && !tensors[r]) return fail(MCCL_ERR_INVALID_ARG, "tensor pointer %d is null", r);
     if ((uintptr_t)tensors[r] % es) return fail(MCCL_ERR_INVALID_ARG, "tensor %d not aligned to the element size", r);
   }
+  // two ranks' tensors may be the same memory (one process playing several ranks), never partly so
+  for (int r = 0; r < n && count; ++r)
+    for (int q = r + 1; q < n; ++q) {
+      const uintptr_t a0 = (uintptr_t)tensors[r], b0 = (uintptr_t)tensors[q];
+      if (a0 != b0 && a0 < b0 + count * es && b0 < a0 + count * es)
+        return fail(MCCL_ERR_INVALID_ARG, "tensors %d and %d partially overlap", r, q);
+    }
   const size_t shard = mccl_allreduce_sync_shard(count, n);
   const size_t lo = (size_t)me * shard < count ? (size_t)me * shard : count;
   const size_t n_me = lo + shard < count ? shard : count - lo;
@@ -1077,7 +1117,7 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
   a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
   apply_cached_loads(&a);
   const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0);
-  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, (hipStream_t)stream);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, a.sync.ready_epoch != 0 ? (unsigned)a.sync.n : 0u, (hipStream_t)stream);
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
 }

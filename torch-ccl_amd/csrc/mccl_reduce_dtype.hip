@@ -29,5 +29,5 @@ extern "C" hipError_t MCCL_PASTE(mccl_launch_fused_dt, MCCL_REDUCE_DT)(MCCL_FUSE
 }
 
 extern "C" hipError_t MCCL_PASTE(mccl_launch_xrank_dt, MCCL_REDUCE_DT)(MCCL_XRANK_ENTRY_ARGS) {
-  return launch_xrank_dtype<MCCL_REDUCE_DT>(*static_cast<const XRankArgs*>(xrank_args), op, groups, packed, lds, stream);
+  return launch_xrank_dtype<MCCL_REDUCE_DT>(*static_cast<const XRankArgs*>(xrank_args), op, groups, packed, lds, cus, waiting_ranks, stream);
 }

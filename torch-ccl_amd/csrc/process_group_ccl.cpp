@@ -148,6 +148,22 @@ void checkRank(int rank, int size) {
 
 size_t nbytes(const at::Tensor& t) { return (size_t)t.numel() * t.element_size(); }
 
+bool rangesOverlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
+  const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+  return a_bytes && b_bytes && a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+// A rank's small tensor (the output of reduce_scatter_tensor, the input of all_gather_into_tensor)
+// against its large one of W slices: does it touch any slice but this rank's own?  In its own slice
+// it is the in-place form; anywhere else the peers would read (or write) the large tensor in place
+// while this rank writes (reads) the small one, so such a call is staged, where the copy-in comes
+// first.
+bool touchesForeignSlice(const void* small, size_t small_bytes, const void* large, size_t slice_bytes, int W, int me) {
+  if (!rangesOverlap(small, small_bytes, large, slice_bytes * (size_t)W)) return false;
+  const uintptr_t s0 = (uintptr_t)small, own = (uintptr_t)large + (size_t)me * slice_bytes;
+  return !(s0 >= own && s0 + small_bytes <= own + slice_bytes);
+}
+
 size_t roundUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Device-to-device copy on the compute queue (the library's own segment copy): no DMA-engine
@@ -869,6 +885,20 @@ std::chrono::milliseconds ProcessGroupCCL::waitLimit(bool start_up) const {
   return limit;
 }
 
+// How long a kernel's own wait for the other ranks may last.  Normally the group's limit.  With
+// MCCL_PG_SYNC=kernel whole grids wait, and a late rank whose other kernels find no room beside them
+// only gets in once those waits have given up: twenty seconds there, not the minutes of the
+// group's timeout (MCCL_PG_DEVICE_WAIT_MS or MCCL_BARRIER_TIMEOUT_MS say otherwise).
+std::chrono::milliseconds ProcessGroupCCL::deviceWaitLimit() const {
+  if (const char* v = std::getenv("MCCL_PG_DEVICE_WAIT_MS")) {
+    const long ms = std::atol(v);
+    if (ms > 0) return std::chrono::milliseconds(ms);
+  }
+  const std::chrono::milliseconds limit = waitLimit(false);
+  if (waits_in_data_kernels_ && !std::getenv("MCCL_BARRIER_TIMEOUT_MS")) return std::min(limit, std::chrono::milliseconds(20000));
+  return limit;
+}
+
 void ProcessGroupCCL::hostBarrier(bool start_up) {
   const uint64_t epoch = ++barrier_epoch_;
   ctl_->slot[rank_].arrive.store(epoch, std::memory_order_release);
@@ -1260,7 +1290,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       sync.done_epoch = zero_copy ? epoch + 3 : 0;
       sync.max_compute_units = compact ? std::max(1u, waiting_cus_ / (unsigned)size_) : 0u;
       sync.done_counter = done_counter_;
-      sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
+      sync.timeout_us = (uint64_t)deviceWaitLimit().count() * 1000ull;
       sync.status = status_dev_;
       if (plan.exec_sync(pv, sync, s)) {
         if (timed) { phase_us_[2].push_back(0.f); phase_us_[3].push_back((float)us_since(t0)); }
@@ -1283,7 +1313,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       sync.rank = rank_;
       sync.done_epoch = epoch + 3;
       sync.done_counter = done_counter_;
-      sync.timeout_us = (uint64_t)waitLimit(false).count() * 1000ull;
+      sync.timeout_us = (uint64_t)deviceWaitLimit().count() * 1000ull;
       sync.status = status_dev_;
       if (plan.exec_sync(pv, sync, s)) {
         if (timed) phase_us_[3].push_back((float)us_since(t0));
@@ -1327,7 +1357,7 @@ void ProcessGroupCCL::launchFused(const Plan& plan, hipStream_t s) {
   last_title_ = plan.title;
   last_path_ = "one launch, fused";
   ++enqueue_only_count_;
-  const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+  const uint64_t limit_us = (uint64_t)deviceWaitLimit().count() * 1000ull;
   MCCL_CHECK(mccl_allreduce_fused_replayable(plan.fused_ptr, plan.fused_ptr, plan.fused_count, plan.fused_dtype, plan.fused_op,
                                              fused_stage_[0].data(), fused_flags_[0].data(), kArenaFusedStageStride,
                                              kArenaFusedFlagsStride, fused_state_, size_, rank_, limit_us,
@@ -1357,6 +1387,13 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::finishRun(Plan& plan, hipStream_
       for (const auto& t : *list)
         if (t.defined() && t.has_storage() && t.numel() > 0)
           c10::hip::HIPCachingAllocatorMasqueradingAsCUDA::recordStreamMasqueradingAsCUDA(t.storage().data_ptr(), cs);
+  }
+  if (same_stream && blocking_wait_ && !capturing) {
+    // CCL_BLOCKING_WAIT: wait() polls until THIS collective is done or its time is up, so its end is
+    // marked -- the state of the whole stream would count kernels the caller enqueues behind the
+    // collective against its timeout.  The record is a packet of its own, paid in this mode only.
+    work->end_ = shared_->getEvent();
+    HIP_CHECK(hipEventRecord(work->end_, s));
   }
   if (plan.host_complete) {
     // a barrier returns once every rank has arrived: the host waits for the flag kernel
@@ -1674,7 +1711,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
       const bool push = allgather_push_ && (uint64_t)per_rank * (uint64_t)W < kShareMaxAllocation;
       if (push) {
         p.share = len * (size_t)W >= kZeroCopyMinBytes;
-        p.share_ptr = output.data_ptr();
+        // (an input inside another rank's slice of the output: nothing is offered, and then every rank stages)
+        p.share_ptr = touchesForeignSlice(input.data_ptr(), per_rank, output.data_ptr(), per_rank, W, me) ? nullptr : output.data_ptr();
         p.share_bytes = per_rank * (size_t)W;
         auto destinations = [=](const PeerView& pv, int k0, int k1) {
           std::vector<void*> dst;
@@ -1706,7 +1744,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
         };
       } else {
         p.share = len >= kZeroCopyMinBytes;  // the inputs are read in place by the peers
-        p.share_ptr = in;
+        p.share_ptr = touchesForeignSlice(input.data_ptr(), per_rank, output.data_ptr(), per_rank, W, me) ? nullptr : in;
         p.share_bytes = len;
         p.exec = [=](const PeerView& pv, hipStream_t s) {
           const auto segs = pulls(pv);
@@ -1777,6 +1815,11 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   // the group measures, which every rank knows from its output list: the offer is the same everywhere.
   p.share = largest >= kZeroCopyMinBytes;
   p.share_ptr = mine ? input.data_ptr() : nullptr;
+  // (an input that one of this rank's outputs overlaps, other than as the very tensor it is gathered
+  // into: not offered, the peers would read it while this rank's copies write over it)
+  for (size_t r = 0; r < outs.size() && p.share_ptr; ++r)
+    if (rangesOverlap(input.data_ptr(), mine, outs[r].data_ptr(), nbytes(outs[r])) && !((int)r == rank_ && outs[r].data_ptr() == input.data_ptr()))
+      p.share_ptr = nullptr;
   p.share_bytes = mine;
   auto pulls = [=](const PeerView& pv) {
     std::vector<mccl_segment_t> segs;
@@ -1891,7 +1934,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
       };
       // large inputs are read in place by the peers: rank r reduces slice r of every rank's tensor
       p.share = len * es * (size_t)W >= kZeroCopyMinBytes;
-      p.share_ptr = in;
+      // (an output inside another rank's slice of the input: nothing is offered, and then every rank stages)
+      p.share_ptr = touchesForeignSlice(output.data_ptr(), M * es, in, M * es, W, me) ? nullptr : in;
       p.share_bytes = M * es * (size_t)W;
       p.exec = [=](const PeerView& pv, hipStream_t s) {
         void* o = out;
@@ -2159,6 +2203,10 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::exchange(c10d::OpType op, const 
     p.table[(size_t)(2 * W)] = (int64_t)total;
     p.share = true;
     p.share_ptr = image.flat;  // null with total > 0: a packed image, which cannot be shared
+    // (nor can an image that a destination of this rank overlaps: the peers would read it while this
+    // rank's copies write over it; staged, the copy-in comes first)
+    for (size_t d = 0; d < dst.size() && p.share_ptr; ++d)
+      if (rangesOverlap(image.flat, total, dst[d], recv[d])) p.share_ptr = nullptr;
     p.share_bytes = total;
     if (wlen) {
       if (image.flat) {

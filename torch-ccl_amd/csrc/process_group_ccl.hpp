@@ -301,6 +301,7 @@ class ProcessGroupCCL : public c10d::Backend {
   void runHostSynced(Plan& plan, hipStream_t s, int slot);
   void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void deviceBarrier(uint64_t epoch, hipStream_t s);
+  std::chrono::milliseconds deviceWaitLimit() const;
   void throwIfFailed();
   std::string lastEnqueued() const;
   void awaitPeersEntered(uint64_t seq);

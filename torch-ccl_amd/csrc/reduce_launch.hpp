@@ -99,31 +99,58 @@ hipError_t launch_fused_dtype(const FusedArgs& a, int op, unsigned groups, hipSt
   return hipGetLastError();
 }
 
-// The one-launch cross-rank reduction (reduce_scatter, in-place allreduce): persistent grid of
-// `groups` workgroups, single wavefronts or (packed) kPackedWaves wavefronts each.
-template <int DT, int WPG>
-hipError_t launch_xrank_packing(const XRankArgs& a, int op, unsigned groups, unsigned lds, hipStream_t s) {
-  const dim3 grid(groups, 1, 1), block(kWave * WPG);
-  switch (op) {
-    case MCCL_SUM: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_SUM, WPG>), grid, block, lds, s, a); break;
-    case MCCL_PROD: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_PROD, WPG>), grid, block, lds, s, a); break;
-    case MCCL_MIN: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MIN, WPG>), grid, block, lds, s, a); break;
-    case MCCL_MAX: hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_MAX, WPG>), grid, block, lds, s, a); break;
-    case MCCL_AVG:
-      if constexpr (Elem<DT>::kIsFloat) {
-        hipLaunchKernelGGL((xrank_reduce_kernel<DT, MCCL_AVG, WPG>), grid, block, lds, s, a);
-        break;
-      } else {
-        return hipErrorInvalidValue;
-      }
-    default: return hipErrorInvalidValue;
+// Workgroups of `kernel` (of `block` work-items) a launch that waits for `ranks` launches at its
+// start may have: this rank's share of HALF of what the kernel's register use lets the GPU hold at
+// once.  The other half is room for whatever a late rank still has to run before it can join -- a
+// budget equal to the whole residency (which a fixed 4096 wavefronts once was, for a kernel of 114
+// registers) lets seven waiting ranks fill every slot.
+template <typename K>
+unsigned blocks_per_cu(K kernel, int block) {
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, 0) != hipSuccess || per_cu < 1) {
+    (void)hipGetLastError();
+    per_cu = 1;
   }
+  return (unsigned)per_cu;
+}
+inline unsigned waiting_share(unsigned per_cu, unsigned cus, unsigned ranks) {
+  const uint64_t share = (uint64_t)per_cu * cus / 2u / (ranks ? ranks : 1u);
+  return share ? (unsigned)share : 1u;
+}
+
+// The one-launch cross-rank reduction (reduce_scatter, in-place allreduce): grid of `groups`
+// workgroups, single wavefronts or (packed) kPackedWaves wavefronts each.  waiting_ranks > 0: the
+// launch waits for its peers at its start, so its grid is cut to this rank's share of the GPU
+// (the kernel walks its tiles with whatever grid it gets).
+template <int DT, int OP, int WPG>
+hipError_t launch_xrank_kernel(const XRankArgs& a, unsigned groups, unsigned lds, unsigned cus, unsigned waiting_ranks, hipStream_t s) {
+  if (waiting_ranks) {
+    static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, WPG>, kWave * WPG);  // asked once per kernel
+    const unsigned cap = waiting_share(per_cu, cus, waiting_ranks);
+    if (groups > cap) groups = cap;
+  }
+  hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, WPG>), dim3(groups, 1, 1), dim3(kWave * WPG), lds, s, a);
   return hipGetLastError();
 }
 
+template <int DT, int WPG>
+hipError_t launch_xrank_packing(const XRankArgs& a, int op, unsigned groups, unsigned lds, unsigned cus, unsigned waiting_ranks, hipStream_t s) {
+  switch (op) {
+    case MCCL_SUM: return launch_xrank_kernel<DT, MCCL_SUM, WPG>(a, groups, lds, cus, waiting_ranks, s);
+    case MCCL_PROD: return launch_xrank_kernel<DT, MCCL_PROD, WPG>(a, groups, lds, cus, waiting_ranks, s);
+    case MCCL_MIN: return launch_xrank_kernel<DT, MCCL_MIN, WPG>(a, groups, lds, cus, waiting_ranks, s);
+    case MCCL_MAX: return launch_xrank_kernel<DT, MCCL_MAX, WPG>(a, groups, lds, cus, waiting_ranks, s);
+    case MCCL_AVG:
+      if constexpr (Elem<DT>::kIsFloat) return launch_xrank_kernel<DT, MCCL_AVG, WPG>(a, groups, lds, cus, waiting_ranks, s);
+      else return hipErrorInvalidValue;
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int DT>
-hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned groups, int packed, unsigned lds, hipStream_t s) {
-  return packed ? launch_xrank_packing<DT, kPackedWaves>(a, op, groups, lds, s) : launch_xrank_packing<DT, 1>(a, op, groups, lds, s);
+hipError_t launch_xrank_dtype(const XRankArgs& a, int op, unsigned groups, int packed, unsigned lds, unsigned cus, unsigned waiting_ranks, hipStream_t s) {
+  return packed ? launch_xrank_packing<DT, kPackedWaves>(a, op, groups, lds, cus, waiting_ranks, s)
+                : launch_xrank_packing<DT, 1>(a, op, groups, lds, cus, waiting_ranks, s);
 }
 
 }  // namespace
@@ -157,8 +184,10 @@ __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt5(MCCL_FUSE
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt6(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt7(MCCL_FUSED_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_fused_dt8(MCCL_FUSED_ENTRY_ARGS);
-// `xrank_args` points at an XRankArgs; lds = dynamic LDS bytes reserved per workgroup (residency cap)
-#define MCCL_XRANK_ENTRY_ARGS const void *xrank_args, int op, unsigned groups, int packed, unsigned lds, hipStream_t stream
+// `xrank_args` points at an XRankArgs; lds = dynamic LDS bytes reserved per workgroup (residency cap);
+// waiting_ranks > 0: the launch waits for that many ranks' launches and is cut to its share of `cus` compute units
+#define MCCL_XRANK_ENTRY_ARGS \
+  const void *xrank_args, int op, unsigned groups, int packed, unsigned lds, unsigned cus, unsigned waiting_ranks, hipStream_t stream
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt0(MCCL_XRANK_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt1(MCCL_XRANK_ENTRY_ARGS);
 __attribute__((visibility("hidden"))) hipError_t mccl_launch_xrank_dt2(MCCL_XRANK_ENTRY_ARGS);
