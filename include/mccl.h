@@ -194,6 +194,66 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
                       void* status, void* stream);
 
 /*
+ * mccl_rank_barrier that also tells every rank WHERE the other ranks' buffers of the coming
+ * collective are, so that no host thread has to: the reference exchanges the handles of its buffers
+ * once (src/gpu/dpcpp_ccl.cpp:105-121 -> src/gpu/allreduce.h:546-594, 1208-1248) and afterwards a
+ * collective is a pure enqueue; here the buffers are the callers' own tensors, which change from
+ * call to call, so what is exchanged once is the ALLOCATION (mapped by every peer, on the host,
+ * whenever the owner announces a new one) and what travels per collective, on the device, is which
+ * allocation and where in it.
+ *   Before it stores `epoch` into flags[rank], the wavefront stores *mine into offers[rank] (this
+ * rank's offer slot: 32 bytes of device memory the peers can reach, 8-byte aligned; a slot may be
+ * written again once every peer has started a later barrier -- two alternating slots do).  After
+ * rank r's flag has arrived, lane r reads offers[r] and looks the offer up in *imports, this rank's
+ * table of the peers' allocations as it has mapped them (device memory of this rank, filled by the
+ * host in stream order before the launch): entry e of rank r at generation g is at
+ * imports->base[r][e] when imports->generation[r][e] == g; entry MCCL_OFFER_STAGED means rank r's
+ * staging buffer `slot`, imports->staging[r][slot].  The address of every rank's buffer in this
+ * rank's address space -- base + offset; my_buffer for this rank itself -- goes to resolved[0..n),
+ * n 64-bit words of this rank's device memory, for the kernels that follow on the stream
+ * (mccl_allreduce_sync_resolved).  An offer that this rank has not mapped leaves a null pointer
+ * there and is reported: status[0] = 1 + the rank, status[1] = MCCL_STATUS_UNMAPPED.  At most
+ * MCCL_OFFER_RANKS ranks.  Everything else as mccl_rank_barrier.
+ */
+#define MCCL_OFFER_RANKS 8
+#define MCCL_OFFER_ENTRIES 32
+#define MCCL_OFFER_STAGED 0xffffffffu
+#define MCCL_STATUS_UNMAPPED 0xfffffffeu
+typedef struct mccl_offer {
+  uint32_t entry;      /* index in the owner's table of announced allocations, or MCCL_OFFER_STAGED */
+  uint32_t slot;       /* with MCCL_OFFER_STAGED: which of the owner's two staging buffers */
+  uint64_t generation; /* of the entry: changes when the owner reuses it for another allocation */
+  uint64_t offset;     /* bytes from the start of the allocation (or of the staging buffer) */
+  uint64_t reserved;
+} mccl_offer_t;
+typedef struct mccl_import_table {
+  uint64_t base[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES];
+  uint64_t generation[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES];
+  uint64_t staging[MCCL_OFFER_RANKS][2];
+} mccl_import_table_t;
+int mccl_rank_barrier_offers(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us, void* status,
+                             const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                             const mccl_import_table_t* imports, void* resolved, void* stream);
+
+/*
+ * Stream-ordered update of an import table in device memory: entry `entry` of rank `rank` is now
+ * mapped at `base` at generation `generation` (base 0: not mapped any more), or staging buffer
+ * `slot` of rank `rank` is at `base` (entry MCCL_OFFER_STAGED).  The values travel inside the launch, so
+ * the caller's memory may change as soon as the call returns, and a barrier enqueued earlier on the
+ * stream still resolves against the table as it was.  At most MCCL_IMPORT_UPDATES per call.
+ */
+#define MCCL_IMPORT_UPDATES 8
+typedef struct mccl_import_update {
+  uint32_t rank;
+  uint32_t entry;       /* < MCCL_OFFER_ENTRIES: an allocation; MCCL_OFFER_STAGED: a staging buffer, `slot` says which */
+  uint32_t slot;
+  uint32_t reserved;
+  uint64_t base;
+  uint64_t generation;
+} mccl_import_update_t;
+int mccl_import_table_update(mccl_import_table_t* table, const mccl_import_update_t* updates, int n, void* stream);
+
+/*
  * One-launch small allreduce across rank processes: copy-in, rank synchronisation and the
  * N-peer reduction in a single kernel, the structure of allreducer_small<T>::allreduce
  * (src/gpu/allreduce_small.h:166-361).  Rank `rank` contributes in[0..count) and receives the
@@ -336,6 +396,14 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
 size_t mccl_allreduce_sync_shard(size_t count, int n);
 int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync,
                         void* stream);
+
+/* mccl_allreduce_sync whose tensor addresses come from device memory: resolved[0..n) as
+ * mccl_rank_barrier_offers of the same stream has just left them (the kernel reads them when it
+ * starts).  The barrier in front has ordered the ranks: sync->ready_epoch must be 0 and
+ * sync->done_epoch set.  A null address among them (an offer that could not be resolved, already
+ * reported by the barrier) makes the launch skip its work and still take part in the closing wait. */
+int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                                 void* stream);
 
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */

@@ -549,15 +549,16 @@ def large_message_case(pg, rank, world):
 
 
 def missing_rank_case(pg, rank, world):
-    """Rank 1 never joins the second collective: the others must get an error, not hang.  (2 MiB:
-    a size whose allreduce has the host threads meet first in every mode -- to agree on reading the
-    tensors in place, or around the launches -- so the call itself raises.)"""
+    """Rank 1 never joins the second collective: the others must get an error, not hang.  (A
+    reduce_scatter_tensor of 2 MiB per rank: a collective whose host threads meet first in every
+    mode -- to agree on reading the tensors in place, or around the launches -- so the call itself
+    raises.)"""
     t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
     try:
-        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        pg._reduce_scatter_base(t, torch.ones(world << 19, device=DEV)).wait()
         raise AssertionError("collective with a missing rank returned")
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
@@ -1077,6 +1078,125 @@ def identity_replay_case(rank, world):
     dist.barrier()
 
 
+def standing_offer_cases(pg, rank, world):
+    """all_reduce above the one-launch size between rank processes: the ranks' host threads never
+    wait for each other.  Where each rank's tensor is travels on the device; a rank whose allocation
+    the peers have not mapped yet copies through its staging buffer meanwhile.  Every result is the
+    oracle's, bit for bit."""
+    import time
+    from helpers import TORCH_TO_CODE, bits, rank_buffer, to_carrier
+    from oracle import oracle as O
+
+    def bits_np(arr):
+        return arr.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[arr.dtype.itemsize])
+
+    def check(t, host, what, op=O.SUM):
+        want = bits_np(O.reduce([to_carrier(h) for h in host], TORCH_TO_CODE[t.dtype], op))
+        assert np.array_equal(bits(t), want), what
+
+    # the same tensor again and again: after the first calls nobody rendezvous, everybody reads in place
+    count = (2 << 20) + 5
+    t = torch.empty(count, dtype=torch.bfloat16, device=DEV)
+    paths = []
+    for i in range(12):
+        host = [rank_buffer(count, torch.bfloat16, r, seed=500 + i) for r in range(world)]
+        t.copy_(host[rank])
+        if i == 4:
+            torch.cuda.synchronize()
+            before = pg._rendezvous_counts()
+        pg.allreduce([t], c10d.AllreduceOptions()).wait()
+        paths.append(pg._last_path())
+        check(t, host, ("same tensor", i, paths[-1]))
+    after = pg._rendezvous_counts()
+    assert after[0] == before[0] and after[1] == before[1] + 8, (before, after)  # no rendezvous, eight that only enqueued
+    assert all(p.startswith("standing offers") for p in paths), paths
+    assert paths[-1] == "standing offers, peers read in place", paths  # (the first calls are staged until every peer has mapped the allocation)
+    # a new allocation per call (each tensor fills a segment of its own), all alive at once, more of
+    # them than the table of announced allocations holds: entries are reused, results stay right
+    keep = []
+    for i in range(40):
+        n = (12 << 20) // 4 + i
+        x = torch.full((n,), float(rank + 1 + i), device=DEV)
+        keep.append(x)
+        pg.allreduce([x], c10d.AllreduceOptions()).wait()
+    for again in range(2):
+        for i, x in enumerate(keep):
+            if again:
+                x.fill_(float(rank + 1 + i))
+                pg.allreduce([x], c10d.AllreduceOptions()).wait()
+            want = float(sum(r + 1 + i for r in range(world)))
+            assert float(x.min()) == want == float(x.max()), ("many allocations", again, i, float(x.min()), want)
+    del keep
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    # odd counts, offsets into an allocation, every element width, AVG and MAX
+    for dtype, n, pad, op, oop in ((torch.float32, (1 << 20) + 1, 1, c10d.ReduceOp.SUM, O.SUM), (torch.int8, (5 << 20) + 13, 5, c10d.ReduceOp.MAX, O.MAX),
+                                   (torch.float64, (1 << 19) + 3, 0, c10d.ReduceOp.SUM, O.SUM), (torch.bfloat16, (3 << 20) + 7, 3, c10d.ReduceOp.AVG, O.AVG),
+                                   (torch.float16, (1 << 20) + 9, 2, c10d.ReduceOp.SUM, O.SUM)):
+        host = [rank_buffer(n, dtype, r, seed=540) for r in range(world)]
+        whole = torch.zeros(n + 2 * pad + 8, dtype=dtype, device=DEV)
+        view = whole[pad:pad + n]
+        for rep in range(3):  # staged at first, in place once the peers have mapped the allocation
+            view.copy_(host[rank])
+            opts = c10d.AllreduceOptions()
+            opts.reduceOp = op
+            pg.allreduce([view], opts).wait()
+            check(view, host, ("view", dtype, n, rep, pg._last_path()), oop)
+            assert bool((whole[:pad] == 0).all()) and bool((whole[pad + n:] == 0).all()), ("wrote outside the tensor", dtype)
+    # rank 1's tensor lives in an allocation too large to be shared: that rank stages every time,
+    # the others read and write its staging buffer, everybody else is read in place
+    n = (2 << 20) + 5
+    host = [rank_buffer(n, torch.bfloat16, r, seed=560) for r in range(world)]
+    if rank == 1:
+        huge = torch.empty((2 << 30) + 64, dtype=torch.uint8, device=DEV)
+        x = huge[64:64 + 2 * n].view(torch.bfloat16)
+    else:
+        x = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    for rep in range(4):
+        x.copy_(host[rank])
+        pg.allreduce([x], c10d.AllreduceOptions()).wait()
+        check(x, host, ("unshareable on rank 1", rep))
+    assert pg._last_path() == ("standing offers, this rank staged" if rank == 1 else "standing offers, peers read in place"), pg._last_path()
+    del x
+    if rank == 1:
+        del huge
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    # freed and allocated again between the calls (usually the same address, new contents)
+    for i in range(4):
+        host = [rank_buffer((3 << 20) + 11, torch.float32, r, seed=580 + i) for r in range(world)]
+        y = host[rank].to(DEV)
+        pg.allreduce([y], c10d.AllreduceOptions()).wait()
+        check(y, host, ("freed and allocated again", i))
+        del y
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+    # a rank that comes 50 ms late: the others' calls return at once (nobody's host thread waits
+    # for anybody), their Works complete when the late rank's kernels have run
+    z = torch.full((1 << 20,), float(rank + 1), device=DEV)  # 4 MiB
+    pg.allreduce([z], c10d.AllreduceOptions()).wait()
+    pg.allreduce([z], c10d.AllreduceOptions()).wait()  # (mapped by every peer now)
+    torch.cuda.synchronize()
+    pg.barrier().wait()
+    z.fill_(float(rank + 1))
+    torch.cuda.synchronize()
+    if rank == 1:
+        time.sleep(0.05)
+    t0 = time.perf_counter()
+    w = pg.allreduce([z], c10d.AllreduceOptions())
+    call_ms = (time.perf_counter() - t0) * 1e3
+    w.wait()
+    torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - t0) * 1e3
+    assert float(z[0]) == world * (world + 1) / 2 == float(z[-1])
+    print("standing offers: rank %d of %d, all_reduce(4 MiB) with rank 1 50 ms late: call %.3f ms, call + synchronize %.3f ms" % (
+        rank, world, call_ms, total_ms), flush=True)
+    assert call_ms < 5.0, call_ms  # (measured: below 0.1 ms; the late rank itself included)
+    if rank != 1:
+        assert total_ms > 30.0, total_ms  # the result did wait for the late rank
+    pg.barrier().wait()
+
+
 def graph_capture_case(rank, world):
     """A decode loop from a HIP graph: every rank records K dist.all_reduce of the 256 KiB bf16
     message with a small kernel of the caller's between them, then replays the graph with fresh
@@ -1301,6 +1421,8 @@ def run_rank(rank, world, store_path, mode):
         missing_rank_device_case(pg, rank, world)
     elif mode == "late_peer":
         late_peer_case(pg, rank, world)
+    elif mode == "standing":
+        standing_offer_cases(pg, rank, world)
     else:
         raise ValueError(mode)
     torch.cuda.synchronize()

@@ -123,6 +123,19 @@ def test_zero_copy_collectives(world):
     _spawn(world, "zero_copy")
 
 
+@pytest.mark.parametrize("world", [2, 5, 8])
+def test_allreduce_with_offers_exchanged_on_the_device(world):
+    """No rendezvous of the host threads in steady state; a late rank does not hold up the others' calls."""
+    _spawn(world, "standing")
+
+
+def test_allreduce_with_the_host_rendezvous_instead(monkeypatch):
+    """MCCL_PG_STANDING_OFFERS=0: the allreduce above the one-launch size meets at the host rendezvous as
+    the other collectives do (tables and offers published per call): same bits."""
+    monkeypatch.setenv("MCCL_PG_STANDING_OFFERS", "0")
+    _spawn(4, "zero_copy")
+
+
 def test_a_late_rank_with_gemms_of_its_own_still_gets_in():
     _spawn(8, "heavy_predecessor")
 
@@ -247,5 +260,5 @@ def test_verbose_logs_one_line_per_collective(monkeypatch, capfd):
     _spawn(2, "env")
     out = capfd.readouterr().out
     assert "oneccl_bindings_for_pytorch::allreduce [0/2#" in out and "oneccl_bindings_for_pytorch::allreduce [1/2#" in out, out[-2000:]
-    assert "one launch" in out or "peers read in place" in out, out[-2000:]
+    assert "standing offers" in out, out[-2000:]  # (the 4 MiB allreduce of the case: offers exchanged on the device)
 

@@ -268,6 +268,75 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups, b
   }
 }
 
+// The barrier that also carries every rank's offer for the coming collective and resolves the
+// peers' offers against this rank's table of mapped allocations.
+struct OfferBarrierArgs {
+  uint64_t* flag[MCCL_OFFER_RANKS];
+  uint64_t* offer[MCCL_OFFER_RANKS];  // rank r's offer slot (four 64-bit words)
+  uint64_t epoch;
+  uint64_t limit_ticks;
+  uint32_t* status;
+  uint64_t mine[4];                   // this rank's offer, as the words of an mccl_offer_t
+  uint64_t my_buffer;
+  const mccl_import_table_t* imports;
+  uint64_t* resolved;
+  int n;
+  int rank;
+};
+
+__global__ __launch_bounds__(kWave) void rank_barrier_offers_kernel(const OfferBarrierArgs a) {
+  const int lane = threadIdx.x;
+  if (lane == 0) {
+    // the offer first, then the flag that says it is there
+#pragma unroll
+    for (int i = 0; i < 4; ++i) __hip_atomic_store(a.offer[a.rank] + i, a.mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  if (lane >= a.n) return;
+  uint64_t where = a.my_buffer;
+  if (lane != a.rank) {
+    where = 0;
+    if (!wait_flag64(a.flag[lane], a.epoch, a.limit_ticks)) {
+      report_late(a.status, lane, (uint32_t)a.epoch);
+    } else {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the offer is read after the flag
+      const uint64_t w0 = __hip_atomic_load(a.offer[lane] + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      const uint64_t gen = __hip_atomic_load(a.offer[lane] + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      const uint64_t off = __hip_atomic_load(a.offer[lane] + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      const uint32_t entry = (uint32_t)w0, slot = (uint32_t)(w0 >> 32);
+      if (entry == MCCL_OFFER_STAGED) {
+        const uint64_t b = a.imports->staging[lane][slot & 1u];
+        if (b) where = b + off;
+      } else if (entry < MCCL_OFFER_ENTRIES) {
+        const uint64_t b = a.imports->base[lane][entry];
+        if (b && a.imports->generation[lane][entry] == gen) where = b + off;
+      }
+      if (!where) report_late(a.status, lane, MCCL_STATUS_UNMAPPED);
+    }
+  }
+  a.resolved[lane] = where;
+}
+
+// Stream-ordered update of the table that rank_barrier_offers_kernel resolves against: one lane
+// per update, the values are kernel arguments.
+struct ImportUpdateArgs {
+  mccl_import_table_t* table;
+  mccl_import_update_t update[MCCL_IMPORT_UPDATES];
+  int n;
+};
+
+__global__ __launch_bounds__(kWave) void import_table_update_kernel(const ImportUpdateArgs a) {
+  const int lane = threadIdx.x;
+  if (lane >= a.n) return;
+  const mccl_import_update_t u = a.update[lane];
+  if (u.entry == MCCL_OFFER_STAGED) {
+    a.table->staging[u.rank][u.slot & 1u] = u.base;
+  } else {
+    a.table->generation[u.rank][u.entry] = u.generation;
+    a.table->base[u.rank][u.entry] = u.base;
+  }
+}
+
 template <typename ARGS>
 __global__ __launch_bounds__(kWave) void rank_barrier_kernel(const ARGS a) {
   const int lane = threadIdx.x;

@@ -45,6 +45,11 @@ struct XRankArgs {
   uint32_t aligned_in;                // every in[k] is 8-byte aligned: read past the caches
   uint32_t push;                      // allreduce: write the result over in[k] of every rank k instead of out1
   uint32_t no_invalidate;             // with aligned_in == 0: the caches are clean already (a kernel boundary lies behind the ranks' barrier)
+  // The addresses of the ranks' tensors from device memory instead (null: in[] above holds them):
+  // in_table[k] + in_off, as the barrier kernel in front of this launch has resolved them from the
+  // ranks' offers.  A null entry: the launch does nothing but take part in the closing wait.
+  const uint64_t* in_table;
+  uint64_t in_off;
   XSync sync;
 };
 
@@ -58,29 +63,35 @@ __device__ __forceinline__ u32x4 load_in(const char* base, uint32_t tile, uint32
   return __builtin_nontemporal_load(&((const u32x4_unaligned*)tb)[lane]);
 }
 
-// in[k] for a k known at run time only (a select per rank: no dynamic indexing of the argument block)
-__device__ __forceinline__ const char* pick_in(const XRankArgs& a, int k) {
-  const char* p = a.in[0];
+// Where the ranks' tensors are: from the argument block, or from device memory (in_table).  Only
+// ever indexed with constants, so that it lives in scalar registers.
+struct XIns {
+  const char* p[kXRanks];
+};
+
+// in[k] for a k known at run time only (a select per rank: no dynamic indexing)
+__device__ __forceinline__ const char* pick_in(const XIns& in, int k) {
+  const char* p = in.p[0];
 #pragma unroll
   for (int q = 1; q < kXRanks; ++q)
-    if (k == q) p = a.in[q];
+    if (k == q) p = in.p[q];
   return p;
 }
 
 template <int DT, int NS>
-__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, const Wave& w, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
+__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
   const uint32_t v = tile * kWave + w.lane;  // the host keeps tiles1 * 64 below 2^32
   if (v < a.nvec1) {
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) {
-      if (NS ? k < NS : k < n) x[k].v = load_in(a.in[k], tile, a.aligned_in, w.lane);
+      if (NS ? k < NS : k < n) x[k].v = load_in(in.p[k], tile, a.aligned_in, w.lane);
     }
   }
 }
 
 // Reduces the loaded vectors of a tile (ascending-rank chain) and stores the result.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const Wave& w, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
+__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
   const uint32_t v = tile * kWave + w.lane;
@@ -105,7 +116,7 @@ __device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const Wave
 #pragma unroll
       for (int k = 0; k < kXRanks; ++k) {
         if (NS ? k < NS : k < n) {
-          char* tb = const_cast<char*>(a.in[k]) + (size_t)tile * kXTileBytes;  // uniform
+          char* tb = const_cast<char*>(in.p[k]) + (size_t)tile * kXTileBytes;  // uniform
           if (a.aligned_in) store_tile_through(tb, w.lane * 16u, r.v);
           else store_vec_through(tb + w.lane * 16u, r.v);
         }
@@ -120,20 +131,20 @@ __device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const Wave
 
 // The elements after the last whole vector (fewer than a vector holds): lane e takes element e.
 template <int DT, int OP>
-__device__ __forceinline__ void xrank_tail(const XRankArgs& a, const Wave& w, int n) {
+__device__ __forceinline__ void xrank_tail(const XRankArgs& a, const XIns& in, const Wave& w, int n) {
   using S = typename Elem<DT>::store_t;
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
   if (w.lane < a.tail1) {
     const size_t i = (size_t)a.nvec1 * VE + w.lane;
-    A acc = chain_first<DT, OP>(Elem<DT>::load(__hip_atomic_load(&((const S*)a.in[0])[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
+    A acc = chain_first<DT, OP>(Elem<DT>::load(__hip_atomic_load(&((const S*)in.p[0])[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
     for (int k = 1; k < n; ++k) {
-      const S* src = (const S*)pick_in(a, k);
+      const S* src = (const S*)pick_in(in, k);
       acc = chain_next<DT, OP>(acc, Elem<DT>::load(__hip_atomic_load(&src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)));
     }
     const S r = Elem<DT>::store(chain_last<DT, OP>(acc, n));
     if (a.push) {
-      for (int k = 0; k < n; ++k) __hip_atomic_store(&((S*)const_cast<char*>(pick_in(a, k)))[i], r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      for (int k = 0; k < n; ++k) __hip_atomic_store(&((S*)const_cast<char*>(pick_in(in, k)))[i], r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     } else {
       ((S*)a.out1)[i] = r;
     }
@@ -146,20 +157,20 @@ __device__ __forceinline__ void xrank_tail(const XRankArgs& a, const Wave& w, in
 // between a phase of loads and a phase of stores in step, and the memory pipeline runs dry
 // between the phases.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_walk(const XRankArgs& a, const Wave& w, int n) {
+__device__ __forceinline__ void xrank_walk(const XRankArgs& a, const XIns& in, const Wave& w, int n) {
   const uint32_t T = a.tiles1, G = w.count;
   uint32_t t0 = w.index;
   if (t0 < T) {
     VecU<DT> x0[kXRanks], x1[kXRanks];
-    xrank_load_tile<DT, NS>(a, w, t0, n, x0);
+    xrank_load_tile<DT, NS>(a, in, w, t0, n, x0);
     for (;;) {
       const uint32_t t1 = t0 + G;
-      if (t1 < T) xrank_load_tile<DT, NS>(a, w, t1, n, x1);
-      xrank_finish_tile<DT, OP, NS>(a, w, t0, n, x0);
+      if (t1 < T) xrank_load_tile<DT, NS>(a, in, w, t1, n, x1);
+      xrank_finish_tile<DT, OP, NS>(a, in, w, t0, n, x0);
       if (t1 >= T) break;
       t0 = t1 + G;
-      if (t0 < T) xrank_load_tile<DT, NS>(a, w, t0, n, x0);
-      xrank_finish_tile<DT, OP, NS>(a, w, t1, n, x1);
+      if (t0 < T) xrank_load_tile<DT, NS>(a, in, w, t0, n, x0);
+      xrank_finish_tile<DT, OP, NS>(a, in, w, t1, n, x1);
       if (t0 >= T) break;
     }
   }
@@ -169,11 +180,22 @@ template <int DT, int OP, int WPG>
 __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankArgs a) {
   const int n = a.sync.n;
   const Wave w = this_wave<WPG>();
-  if (xsync_begin(a.sync)) {
+  XIns in;
+  bool resolved = true;
+#pragma unroll
+  for (int k = 0; k < kXRanks; ++k) {
+    in.p[k] = a.in[k];
+    if (a.in_table && k < n) {
+      const uint64_t p = a.in_table[k];  // uniform: written by the kernel in front of this one
+      resolved = resolved && p != 0;
+      in.p[k] = (const char*)(p + a.in_off);
+    }
+  }
+  if (resolved && xsync_begin(a.sync)) {
     if (!a.aligned_in && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
-    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, w, n);
-    else xrank_walk<DT, OP, 0>(a, w, n);
-    if (a.tail1 && w.index == w.count - 1) xrank_tail<DT, OP>(a, w, n);
+    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, in, w, n);
+    else xrank_walk<DT, OP, 0>(a, in, w, n);
+    if (a.tail1 && w.index == w.count - 1) xrank_tail<DT, OP>(a, in, w, n);
   }
   xsync_end(a.sync, gridDim.x, a.push != 0);
 }

@@ -732,6 +732,66 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
   return MCCL_OK;
 }
 
+int mccl_rank_barrier_offers(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us, void* status,
+                             const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                             const mccl_import_table_t* imports, void* resolved, void* stream) {
+  if (!flags || !offers) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer table is null");
+  if (n < 1 || n > MCCL_OFFER_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "a barrier with offers takes 1 to %d ranks, got %d", MCCL_OFFER_RANKS, n);
+  if (rank < 0 || rank >= n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", rank, n);
+  if ((uintptr_t)status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
+  if (!mine || !imports || !resolved) return fail(MCCL_ERR_INVALID_ARG, "offer, import table or output table is null");
+  if ((uintptr_t)imports % 8 || (uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "import table or output table is not 8-byte aligned");
+  if (mine->entry != MCCL_OFFER_STAGED && mine->entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "offer names entry %u of %d", mine->entry, MCCL_OFFER_ENTRIES);
+  OfferBarrierArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int r = 0; r < n; ++r) {
+    if (!flags[r] || !offers[r]) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer %d is null", r);
+    if ((uintptr_t)flags[r] % 8 || (uintptr_t)offers[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer %d is not 8-byte aligned", r);
+    a.flag[r] = (uint64_t*)flags[r];
+    a.offer[r] = (uint64_t*)offers[r];
+  }
+  a.epoch = epoch;
+  a.limit_ticks = wait_limit_ticks(timeout_us);
+  a.status = (uint32_t*)status;
+  a.mine[0] = (uint64_t)mine->entry | ((uint64_t)mine->slot << 32);
+  a.mine[1] = mine->generation;
+  a.mine[2] = mine->offset;
+  a.mine[3] = mine->reserved;
+  a.my_buffer = (uint64_t)(uintptr_t)my_buffer;
+  a.imports = imports;
+  a.resolved = (uint64_t*)resolved;
+  a.n = n;
+  a.rank = rank;
+  hipLaunchKernelGGL(rank_barrier_offers_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "barrier kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int mccl_import_table_update(mccl_import_table_t* table, const mccl_import_update_t* updates, int n, void* stream) {
+  if (n == 0) return MCCL_OK;
+  if (!table || !updates) return fail(MCCL_ERR_INVALID_ARG, "table or update list is null");
+  if ((uintptr_t)table % 8) return fail(MCCL_ERR_INVALID_ARG, "import table is not 8-byte aligned");
+  if (n < 0 || n > MCCL_IMPORT_UPDATES) return fail(MCCL_ERR_INVALID_ARG, "%d updates in one call, at most %d", n, MCCL_IMPORT_UPDATES);
+  ImportUpdateArgs a;
+  memset(&a, 0, sizeof(a));
+  a.table = table;
+  a.n = n;
+  for (int i = 0; i < n; ++i) {
+    const mccl_import_update_t& u = updates[i];
+    if (u.rank >= MCCL_OFFER_RANKS) return fail(MCCL_ERR_INVALID_ARG, "update %d names rank %u of %d", i, u.rank, MCCL_OFFER_RANKS);
+    if (u.entry != MCCL_OFFER_STAGED && u.entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "update %d names entry %u of %d", i, u.entry, MCCL_OFFER_ENTRIES);
+    for (int j = 0; j < i; ++j)
+      if (updates[j].rank == u.rank && updates[j].entry == u.entry && (u.entry != MCCL_OFFER_STAGED || (updates[j].slot & 1u) == (u.slot & 1u)))
+        return fail(MCCL_ERR_INVALID_ARG, "updates %d and %d name the same entry", j, i);
+    a.update[i] = u;
+  }
+  hipLaunchKernelGGL(import_table_update_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "table update launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
 }  // extern "C"
 
 namespace {
@@ -917,6 +977,63 @@ void apply_cached_loads(XRankArgs* a) {
   }
 }
 
+// The in-place allreduce with its tensors' addresses from the host (tensors) or from device memory
+// (resolved: read by the kernel when it starts).
+int allreduce_sync_impl(void* const* tensors, const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                        void* stream) {
+  XRankArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  if (a.sync.ready_epoch != 0 && a.sync.done_epoch == 0)
+    return fail(MCCL_ERR_INVALID_ARG, "the in-place allreduce needs a closing wait (done_epoch) when it has an opening one");
+  const int n = a.sync.n, me = a.sync.rank;
+  const size_t es = dtype_size(dtype);
+  if (tensors) {
+    for (int r = 0; r < n; ++r) {
+      if (count && !tensors[r]) return fail(MCCL_ERR_INVALID_ARG, "tensor pointer %d is null", r);
+      if ((uintptr_t)tensors[r] % es) return fail(MCCL_ERR_INVALID_ARG, "tensor %d not aligned to the element size", r);
+    }
+    // two ranks' tensors may be the same memory (one process playing several ranks), never partly so
+    for (int r = 0; r < n && count; ++r)
+      for (int q = r + 1; q < n; ++q) {
+        const uintptr_t a0 = (uintptr_t)tensors[r], b0 = (uintptr_t)tensors[q];
+        if (a0 != b0 && a0 < b0 + count * es && b0 < a0 + count * es)
+          return fail(MCCL_ERR_INVALID_ARG, "tensors %d and %d partially overlap", r, q);
+      }
+  }
+  const size_t shard = mccl_allreduce_sync_shard(count, n);
+  const size_t lo = (size_t)me * shard < count ? (size_t)me * shard : count;
+  const size_t n_me = lo + shard < count ? shard : count - lo;
+  const size_t ve = 16 / es;
+  if ((uint64_t)shard * es / 16 + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  a.aligned_in = 1;
+  if (tensors) {
+    for (int k = 0; k < n; ++k) {
+      a.in[k] = (const char*)tensors[k] + lo * es;
+      if (n_me && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
+    }
+  } else {
+    // where the tensors lie is not known here: any alignment, read through the caches (the barrier
+    // in front has ordered the ranks, so the caches start clean)
+    a.in_table = (const uint64_t*)resolved;
+    a.in_off = lo * es;
+    a.aligned_in = 0;
+    a.no_invalidate = 1;
+  }
+  a.push = 1;
+  a.nvec1 = (uint32_t)(n_me / ve);
+  a.tail1 = (uint32_t)(n_me % ve);
+  a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
+  apply_cached_loads(&a);
+  const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, a.sync.ready_epoch != 0 ? (unsigned)a.sync.n : 0u, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1079,47 +1196,17 @@ size_t mccl_allreduce_sync_shard(size_t count, int n) {
 }
 
 int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync, void* stream) {
-  XRankArgs a;
-  memset(&a, 0, sizeof(a));
-  int rc = fill_xsync(sync, &a.sync);
-  if (rc != MCCL_OK) return rc;
-  rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
-  if (rc != MCCL_OK) return rc;
   if (!tensors) return fail(MCCL_ERR_INVALID_ARG, "tensor table is null");
-  if (a.sync.ready_epoch != 0 && a.sync.done_epoch == 0)
-    return fail(MCCL_ERR_INVALID_ARG, "the in-place allreduce needs a closing wait (done_epoch) when it has an opening one");
-  const int n = a.sync.n, me = a.sync.rank;
-  const size_t es = dtype_size(dtype);
-  for (int r = 0; r < n; ++r) {
-    if (count && !tensors[r]) return fail(MCCL_ERR_INVALID_ARG, "tensor pointer %d is null", r);
-    if ((uintptr_t)tensors[r] % es) return fail(MCCL_ERR_INVALID_ARG, "tensor %d not aligned to the element size", r);
-  }
-  // two ranks' tensors may be the same memory (one process playing several ranks), never partly so
-  for (int r = 0; r < n && count; ++r)
-    for (int q = r + 1; q < n; ++q) {
-      const uintptr_t a0 = (uintptr_t)tensors[r], b0 = (uintptr_t)tensors[q];
-      if (a0 != b0 && a0 < b0 + count * es && b0 < a0 + count * es)
-        return fail(MCCL_ERR_INVALID_ARG, "tensors %d and %d partially overlap", r, q);
-    }
-  const size_t shard = mccl_allreduce_sync_shard(count, n);
-  const size_t lo = (size_t)me * shard < count ? (size_t)me * shard : count;
-  const size_t n_me = lo + shard < count ? shard : count - lo;
-  const size_t ve = 16 / es;
-  if ((uint64_t)shard * es / 16 + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
-  a.aligned_in = 1;
-  for (int k = 0; k < n; ++k) {
-    a.in[k] = (const char*)tensors[k] + lo * es;
-    if (n_me && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
-  }
-  a.push = 1;
-  a.nvec1 = (uint32_t)(n_me / ve);
-  a.tail1 = (uint32_t)(n_me % ve);
-  a.tiles1 = (uint32_t)((n_me / ve + (n_me % ve ? 1 : 0) + kWave - 1) / kWave);
-  apply_cached_loads(&a);
-  const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0);
-  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, a.sync.ready_epoch != 0 ? (unsigned)a.sync.n : 0u, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "allreduce kernel launch failed: %s", hipGetErrorString(e));
-  return MCCL_OK;
+  return allreduce_sync_impl(tensors, nullptr, count, dtype, op, sync, stream);
+}
+
+int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                                 void* stream) {
+  if (!resolved) return fail(MCCL_ERR_INVALID_ARG, "address table is null");
+  if ((uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "address table is not 8-byte aligned");
+  if (sync && (sync->ready_epoch != 0 || sync->done_epoch == 0))
+    return fail(MCCL_ERR_INVALID_ARG, "the allreduce over resolved addresses runs behind a barrier: ready_epoch 0, done_epoch set");
+  return allreduce_sync_impl(nullptr, resolved, count, dtype, op, sync, stream);
 }
 
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream) {

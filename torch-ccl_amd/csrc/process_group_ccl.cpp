@@ -70,10 +70,19 @@ constexpr size_t kArenaFusedStageOff = 64u << 10;            // two staging buff
 constexpr size_t kArenaFusedStageStride = kFusedMaxBytes + (64u << 10);  // followed by room for the rank stagger
 constexpr size_t kArenaDoneCountOff = 24u << 10;  // MCCL_SYNC_COUNTER_BYTES of workgroup counters of the one-launch collectives
 constexpr size_t kArenaFusedStateOff = 2048;  // MCCL_FUSED_STATE_BYTES: the device-resident epoch of the one-launch small allreduce
+constexpr size_t kArenaOfferOff = 3072;       // two mccl_offer_t, 64 bytes apart: what this rank's tensor of a collective is
+constexpr size_t kArenaOfferStride = 64;
+constexpr size_t kArenaImportTableOff = 32u << 10;  // mccl_import_table_t: the peers' allocations as this rank has mapped them
+constexpr size_t kArenaResolvedOff = 40u << 10;     // MCCL_OFFER_RANKS addresses: the ranks' tensors of the collective under way
 constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
+static_assert(kArenaFusedStateOff + MCCL_FUSED_STATE_BYTES <= kArenaOfferOff && kArenaOfferOff + 2 * kArenaOfferStride <= kArenaFusedFlagsOff, "the offers lie between the epoch state and the flags");
+static_assert(sizeof(mccl_offer_t) <= kArenaOfferStride, "an offer fits its slot");
+static_assert(kArenaImportTableOff + sizeof(mccl_import_table_t) <= kArenaResolvedOff, "the import table ends before the resolved addresses");
+static_assert(kArenaResolvedOff + MCCL_OFFER_RANKS * 8 <= kArenaFusedStageOff, "the resolved addresses end before the staging buffers");
+static_assert(kMaxExports == MCCL_OFFER_ENTRIES, "an offer names an entry of the export table");
 static_assert(kFusedMaxBytes / MCCL_FUSED_TILE_BYTES * 4 <= kArenaFusedFlagsStride, "tile flags must fit their slot");
 static_assert(kArenaFusedFlagsOff + 2 * kArenaFusedFlagsStride <= kArenaDoneCountOff, "the flags end before the counters");
-static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaFusedStageOff, "the counters end before the staging buffers");
+static_assert(kArenaDoneCountOff + MCCL_SYNC_COUNTER_BYTES <= kArenaImportTableOff, "the counters end before the import table");
 static_assert(kArenaFusedStateOff + MCCL_FUSED_STATE_BYTES <= kArenaFusedFlagsOff, "the epoch state ends before the flags");
 
 #define HIP_CHECK(expr)                                                                     \
@@ -229,10 +238,21 @@ struct alignas(128) RankSlot {
   // zero-copy: allocations of this rank the peers may map
   struct ExportEntry {
     std::atomic<uint64_t> gen;  // bumped whenever the entry changes or its allocation is freed
+    // `gen` while the fields below describe a live allocation, 0 while they are being rewritten or
+    // the allocation is gone: what a peer that reads the table on its own (no rendezvous) goes by
+    std::atomic<uint64_t> live;
     uint64_t base;
     uint64_t size;
     hipIpcMemHandle_t handle;
   } exports[kMaxExports];
+  // Standing offers: acked[o][e] = the generation of rank o's export entry e that THIS rank has
+  // mapped, and the first collective of this rank whose kernels see that mapping.  Rank o offers
+  // the entry to its peers' kernels only when every peer's ack says "mapped, from a collective not
+  // later than this one".
+  struct Ack {
+    std::atomic<uint64_t> gen;
+    std::atomic<uint64_t> from_seq;
+  } acked[MCCL_OFFER_RANKS][kMaxExports];
   P2PBox p2p[kMaxWorld];
 };
 
@@ -269,7 +289,10 @@ void GroupShared::putEvent(hipEvent_t e) {
 std::string GroupShared::failureMessage() {
   if (status && (status[0] != 0 || status[2] != 0) && !failed.load(std::memory_order_acquire)) {
     std::ostringstream os;
-    if (status[0] != 0) {
+    if (status[0] != 0 && status[1] == MCCL_STATUS_UNMAPPED) {
+      os << "ccl backend: rank " << (status[0] - 1) << " offered a tensor in an allocation that this rank has not mapped "
+            "(standing offers out of step); the group cannot be used any more";
+    } else if (status[0] != 0) {
       // epochs count four per collective: #(epoch / 4), wait (epoch % 4): 1 = inputs ready, 2 = between
       // the phases of a two-phase collective, 3 = all ranks done with this rank's buffers
       os << "ccl backend: timed out waiting for rank " << (status[0] - 1)
@@ -469,6 +492,7 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   }
   if (const char* v = std::getenv("MCCL_PG_COMPACT_MAX_BYTES")) compact_max_ = (size_t)std::atoll(v);
   allgather_push_ = envFlag("MCCL_PG_ALLGATHER_PUSH", true);
+  standing_offers_ = envFlag("MCCL_PG_STANDING_OFFERS", true);
   work_only_ = envFlag("TORCH_CCL_WORK_ONLY", false) || envFlag("MCCL_PG_WORK_ONLY", false);
   sync_only_ = envFlag("TORCH_CCL_SYNC_ONLY", false) || envFlag("MCCL_PG_SYNC_ONLY", false);
   disable_allreduce_ = envFlag("TORCH_CCL_DISABLE_ALLREDUCE", false) || envFlag("MCCL_PG_DISABLE_ALLREDUCE", false);
@@ -684,6 +708,9 @@ void ProcessGroupCCL::ensureInit(int device) {
     }
     done_counter_ = static_cast<char*>(arena_) + kArenaDoneCountOff;
     fused_state_ = static_cast<char*>(arena_) + kArenaFusedStateOff;
+    import_table_ = reinterpret_cast<mccl_import_table_t*>(static_cast<char*>(arena_) + kArenaImportTableOff);
+    resolved_ = static_cast<char*>(arena_) + kArenaResolvedOff;
+    for (int sl = 0; sl < 2; ++sl) offer_slots_[sl].assign((size_t)size_, nullptr);
     for (int r = 0; r < size_; ++r) {
       char* base = nullptr;
       if (r == rank_) {
@@ -699,6 +726,7 @@ void ProcessGroupCCL::ensureInit(int device) {
       bar_flags_[(size_t)r] = base + kArenaBarOff;
       final_flags_[(size_t)r] = base + kArenaFinalOff;
       for (int sl = 0; sl < 2; ++sl) {
+        offer_slots_[sl][(size_t)r] = base + kArenaOfferOff + (size_t)sl * kArenaOfferStride;
         fused_flags_[sl][(size_t)r] = base + kArenaFusedFlagsOff + (size_t)sl * kArenaFusedFlagsStride;
         fused_stage_[sl][(size_t)r] = base + kArenaFusedStageOff + (size_t)sl * kArenaFusedStageStride + stageOffset(r);
       }
@@ -770,6 +798,7 @@ const void* ProcessGroupCCL::peerStage(int peer, int slot, int pub) {
       pm.ipc[slot] = true;
     }
     pm.gen[slot] = rec.stage_gen;
+    if (peer < MCCL_OFFER_RANKS) noteImport((uint32_t)peer, MCCL_OFFER_STAGED, (uint32_t)slot, (uint64_t)(uintptr_t)pm.ptr[slot], 0);
   }
   return pm.ptr[slot];
 }
@@ -784,6 +813,7 @@ void ProcessGroupCCL::segmentFreed(uint64_t base) {
   for (int i = 0; i < kMaxExports; ++i) {
     if (exports_[(size_t)i].valid && exports_[(size_t)i].base == base) {
       exports_[(size_t)i].valid = false;
+      ctl_->slot[rank_].exports[i].live.store(0, std::memory_order_release);
       ctl_->slot[rank_].exports[i].gen.fetch_add(1, std::memory_order_release);
     }
   }
@@ -819,19 +849,30 @@ int ProcessGroupCCL::exportRange(const void* ptr, size_t bytes, uint64_t* offset
       (void)hipGetLastError();  // e.g. memory of an expandable segment: not shareable
       return -1;
     }
+    // An entry that a standing offer has named may only change once every peer has entered a later
+    // collective than the offer's: a peer reads this table when it enters a collective, and the
+    // kernels of that collective resolve the offer against what it read.
+    uint64_t entered = ~0ull;
+    for (int r = 0; r < size_; ++r)
+      if (r != rank_) entered = std::min(entered, ctl_->slot[r].entered.load(std::memory_order_acquire));
+    auto settled = [&](int i) { return last_offer_seq_[i] == 0 || entered >= last_offer_seq_[i] + 1; };
     for (int i = 0; i < kMaxExports && idx < 0; ++i)
-      if (!exports_[(size_t)i].valid) idx = i;  // a never-used entry, or one whose allocation is gone
-    while (idx < 0) {
+      if (!exports_[(size_t)i].valid && settled(i)) idx = i;  // a never-used entry, or one whose allocation is gone
+    for (int tries = 0; idx < 0 && tries < kMaxExports; ++tries) {
       // evict round robin, but never an entry of the last two offers: a slow peer may still be
       // opening it
       const int victim = export_clock_;
       export_clock_ = (export_clock_ + 1) % kMaxExports;
-      if (victim != recent_export_[0] && victim != recent_export_[1]) idx = victim;
+      if (victim != recent_export_[0] && victim != recent_export_[1] && settled(victim)) idx = victim;
     }
-    me.exports[idx].gen.fetch_add(1, std::memory_order_release);
+    if (idx < 0) return -1;  // every entry is still spoken for: this tensor is staged
+    me.exports[idx].live.store(0, std::memory_order_release);
+    const uint64_t gen = me.exports[idx].gen.fetch_add(1, std::memory_order_acq_rel) + 1;
     me.exports[idx].base = (uint64_t)(uintptr_t)base;
     me.exports[idx].size = size;
     me.exports[idx].handle = h;
+    me.exports[idx].live.store(gen, std::memory_order_release);
+    last_offer_seq_[idx] = 0;
     exports_[(size_t)idx] = Export{(uint64_t)(uintptr_t)base, size, true};
   }
   *offset = off;
@@ -860,8 +901,182 @@ const void* ProcessGroupCCL::importRange(int peer, int pub) {
     HIP_CHECK(hipIpcOpenMemHandle(&p, rs.exports[idx].handle, hipIpcMemLazyEnablePeerAccess));
     im.base = p;
     im.gen = gen;
+    if (peer < MCCL_OFFER_RANKS && size_ <= MCCL_OFFER_RANKS) {  // the standing offers go by the same mappings
+      noteImport((uint32_t)peer, (uint32_t)idx, 0, (uint64_t)(uintptr_t)p, gen);
+      seen_live_[peer][idx] = gen;
+      acknowledge(peer, idx, gen, seq_ - 1);  // (run() has counted this collective already)
+    }
   }
   return static_cast<const char*>(im.base) + rec.share_off;
+}
+
+// ---------------------------------------------------------------------------------------------
+// standing offers: collectives between rank processes that only enqueue
+// ---------------------------------------------------------------------------------------------
+// The reference exchanges the handles of its buffers once (src/gpu/dpcpp_ccl.cpp:105-121); after
+// that an allreduce is a pure enqueue.  Here the buffers are the callers' tensors, so what is
+// exchanged once is the ALLOCATION a tensor lives in -- a rank announces it in its export table,
+// every peer maps it when it next enters a collective and says so (acked) -- and what changes from
+// call to call, which allocation and where in it, travels on the device: the barrier kernel of the
+// collective publishes this rank's offer and resolves the peers' against this rank's table of
+// mappings (mccl_rank_barrier_offers).  No host thread waits for another: a rank whose allocation
+// the peers have not all mapped yet (or that cannot be shared at all) copies its tensor into its
+// staging buffer, which every peer has mapped since the group last grew it, and offers that.
+
+// A mapping of this rank changed: the device table learns of it in stream order, before the next
+// barrier that resolves offers (the values travel in the launch).
+void ProcessGroupCCL::noteImport(uint32_t rank, uint32_t entry, uint32_t slot, uint64_t base, uint64_t gen) {
+  for (auto& u : table_updates_)
+    if (u.rank == rank && u.entry == entry && (entry != MCCL_OFFER_STAGED || u.slot == slot)) {
+      u.base = base;
+      u.generation = gen;
+      return;
+    }
+  mccl_import_update_t u{};
+  u.rank = rank;
+  u.entry = entry;
+  u.slot = slot;
+  u.base = base;
+  u.generation = gen;
+  table_updates_.push_back(u);
+}
+
+void ProcessGroupCCL::flushImportTable(hipStream_t s) {
+  for (size_t at = 0; at < table_updates_.size(); at += MCCL_IMPORT_UPDATES) {
+    const int n = (int)std::min<size_t>(MCCL_IMPORT_UPDATES, table_updates_.size() - at);
+    MCCL_CHECK(mccl_import_table_update(import_table_, table_updates_.data() + at, n, s));
+  }
+  table_updates_.clear();
+}
+
+void ProcessGroupCCL::acknowledge(int owner, int entry, uint64_t gen, uint64_t from_seq) {
+  RankSlot::Ack& a = ctl_->slot[rank_].acked[owner][entry];
+  a.gen.store(0, std::memory_order_release);
+  a.from_seq.store(from_seq, std::memory_order_release);
+  a.gen.store(gen, std::memory_order_release);
+}
+
+// Maps what the peers have announced since this rank last looked, drops what they have retired,
+// and acknowledges: the kernels of collective `seq` and later see these mappings.  Nobody is waited
+// for; an entry that changes while it is read is left for the next look.
+void ProcessGroupCCL::scanPeerExports(uint64_t seq) {
+  for (int r = 0; r < size_; ++r) {
+    if (r == rank_) continue;
+    RankSlot& rs = ctl_->slot[r];
+    for (int e = 0; e < kMaxExports; ++e) {
+      const uint64_t live = rs.exports[e].live.load(std::memory_order_acquire);
+      if (live == seen_live_[r][e]) continue;
+      Import& im = imports_[(size_t)r][(size_t)e];
+      if (im.base && im.gen != live) {
+        quiesce();  // earlier kernels of this rank may still read through the old mapping
+        (void)hipIpcCloseMemHandle(im.base);
+        im = Import{};
+        noteImport((uint32_t)r, (uint32_t)e, 0, 0, 0);
+      }
+      if (live == 0) {
+        seen_live_[r][e] = 0;
+        acknowledge(r, e, 0, seq);
+        continue;
+      }
+      const hipIpcMemHandle_t handle = rs.exports[e].handle;
+      if (rs.exports[e].live.load(std::memory_order_acquire) != live) continue;  // being rewritten: next time
+      if (!im.base) {
+        void* p = nullptr;
+        if (hipIpcOpenMemHandle(&p, handle, hipIpcMemLazyEnablePeerAccess) != hipSuccess) {
+          (void)hipGetLastError();
+          seen_live_[r][e] = live;  // cannot be mapped here: never acknowledged, its owner keeps staging
+          continue;
+        }
+        im.base = p;
+        im.gen = live;
+        noteImport((uint32_t)r, (uint32_t)e, 0, (uint64_t)(uintptr_t)p, live);
+      }
+      seen_live_[r][e] = live;
+      acknowledge(r, e, live, seq);
+    }
+  }
+}
+
+// Have all peers mapped this rank's export entry at this generation, for collectives from `seq` on?
+bool ProcessGroupCCL::allAcknowledged(int entry, uint64_t gen, uint64_t seq) const {
+  for (int r = 0; r < size_; ++r) {
+    if (r == rank_) continue;
+    const RankSlot::Ack& a = ctl_->slot[r].acked[rank_][entry];
+    if (a.gen.load(std::memory_order_acquire) != gen) return false;
+    const uint64_t from = a.from_seq.load(std::memory_order_acquire);
+    if (a.gen.load(std::memory_order_acquire) != gen || from > seq) return false;
+  }
+  return true;
+}
+
+// Staging buffers of both slots that hold `bytes` on every rank and that every peer has mapped:
+// what a rank falls back to without asking anybody.  Grown when a message exceeds it, which every
+// rank finds at the same collective (the sizes of an allreduce agree), in two rendezvous of the host
+// threads -- the only ones this path ever has.
+void ProcessGroupCCL::growStandingCapacity(size_t bytes) {
+  size_t cap = kStageMin;
+  while (cap < bytes) cap <<= 1;
+  cap = std::min(cap, stage_max_);
+  for (int sl = 0; sl < 2; ++sl) {
+    ensureStage(sl, cap);
+    const int pub = (int)(rendezvous_count_++ & 1);
+    ctl_->slot[rank_].pub[pub].share_entry = -1;
+    publishStage(sl, pub);
+    hostBarrier();
+    for (int r = 0; r < size_; ++r) (void)peerStage(r, sl, pub);
+  }
+  standing_capacity_ = cap;
+}
+
+bool ProcessGroupCCL::standingFits(const Plan& plan) const {
+  return standing_offers_ && plan.standing_ok && device_sync_ && distinct_pids_ && zero_copy_ && !waits_in_data_kernels_ &&
+         !work_only_ && !sync_only_ && size_ <= MCCL_OFFER_RANKS &&
+         plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= stage_max_;
+}
+
+void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
+  const size_t bytes = plan.fused_count * mccl_dtype_size(plan.fused_dtype);
+  const uint64_t epoch = 4 * seq;
+  if (bytes > standing_capacity_) growStandingCapacity(bytes);
+  scanPeerExports(seq);
+  uint64_t off = 0;
+  const int entry = exportRange(plan.fused_ptr, bytes, &off);
+  const uint64_t gen = entry >= 0 ? ctl_->slot[rank_].exports[entry].gen.load(std::memory_order_acquire) : 0;
+  const bool in_place = entry >= 0 && allAcknowledged(entry, gen, seq);
+  mccl_offer_t mine{};
+  void* buffer = plan.fused_ptr;
+  if (in_place) {
+    mine.entry = (uint32_t)entry;
+    mine.generation = gen;
+    mine.offset = off;
+    last_offer_seq_[entry] = seq + 1;  // in the units of `entered`: collective `seq` is under way at seq + 1
+  } else {
+    buffer = stage_[slot].ptr;
+    copyAsync(buffer, plan.fused_ptr, bytes, s);
+    mine.entry = MCCL_OFFER_STAGED;
+    mine.slot = (uint32_t)slot;
+  }
+  last_path_ = in_place ? "standing offers, peers read in place" : "standing offers, this rank staged";
+  if (verbose_) {
+    std::ostringstream os;
+    os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
+    std::cout << os.str() << std::endl;
+  }
+  ++enqueue_only_count_;
+  flushImportTable(s);
+  const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+  MCCL_CHECK(mccl_rank_barrier_offers(bar_flags_.data(), size_, rank_, epoch + 1, limit_us, status_dev_, &mine, buffer,
+                                      offer_slots_[slot].data(), import_table_, resolved_, s));
+  mccl_xsync_t sync{};
+  sync.words = bar_flags_.data();
+  sync.n = size_;
+  sync.rank = rank_;
+  sync.done_epoch = epoch + 3;  // nobody's stream goes on before every rank has written its shard everywhere
+  sync.done_counter = done_counter_;
+  sync.timeout_us = limit_us;
+  sync.status = status_dev_;
+  MCCL_CHECK(mccl_allreduce_sync_resolved(resolved_, plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, s));
+  if (!in_place) copyAsync(plan.fused_ptr, buffer, bytes, s);
 }
 
 void ProcessGroupCCL::closeImports() {
@@ -1197,6 +1412,11 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     if (fusedFits(plan)) {
       say_path();
       launchFused(plan, s);
+      if (timed) phase_us_[3].push_back((float)us_since(t0));
+      return;
+    }
+    if (standingFits(plan)) {
+      runStanding(plan, s, slot, seq);
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }
@@ -1543,6 +1763,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // Small messages between rank processes: one launch does copy-in, rank synchronisation and
       // the N-peer sum (the reference's small allreduce, src/gpu/allreduce_small.h:166-361).
       p.fused_ok = len * es <= kFusedMaxBytes;
+      p.standing_ok = true;  // whatever is too large for that launch: offers resolved on the device, no rendezvous
       p.fused_ptr = base;
       p.fused_count = len;
       p.fused_dtype = dtype;

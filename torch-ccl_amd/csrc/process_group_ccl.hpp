@@ -271,6 +271,9 @@ class ProcessGroupCCL : public c10d::Backend {
     size_t fused_count = 0;
     int fused_dtype = 0;
     int fused_op = 0;
+    // An allreduce too large for that launch: fused_ptr / fused_count / fused_dtype / fused_op describe
+    // it for the path that exchanges offers on the device (runStanding).
+    bool standing_ok = false;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
@@ -301,6 +304,15 @@ class ProcessGroupCCL : public c10d::Backend {
   void runHostSynced(Plan& plan, hipStream_t s, int slot);
   void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void deviceBarrier(uint64_t epoch, hipStream_t s);
+  // standing offers (process_group_ccl.cpp: "standing offers")
+  bool standingFits(const Plan& plan) const;
+  void runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq);
+  void growStandingCapacity(size_t bytes);
+  void scanPeerExports(uint64_t seq);
+  bool allAcknowledged(int entry, uint64_t gen, uint64_t seq) const;
+  void acknowledge(int owner, int entry, uint64_t gen, uint64_t from_seq);
+  void noteImport(uint32_t rank, uint32_t entry, uint32_t slot, uint64_t base, uint64_t gen);
+  void flushImportTable(hipStream_t s);
   std::chrono::milliseconds deviceWaitLimit() const;
   void throwIfFailed();
   std::string lastEnqueued() const;
@@ -386,6 +398,7 @@ class ProcessGroupCCL : public c10d::Backend {
   int bisectMode() const { return (work_only_ ? 1 : 0) | (sync_only_ ? 2 : 0) | (disable_allreduce_ ? 4 : 0); }
   // (collectives that met at the rendezvous of the host threads, collectives that only enqueued)
   std::pair<uint64_t, uint64_t> rendezvousCounts() const { return {rendezvous_count_, enqueue_only_count_}; }
+  std::string lastPath() const { return last_path_ ? last_path_ : ""; }
  private:
   unsigned waiting_cus_ = 128;  // what all ranks' waiting launches may hold together (MCCL_PG_WAITING_COMPUTE_UNITS)
   bool distinct_pids_ = false;          // every rank is a process of its own
@@ -449,6 +462,16 @@ class ProcessGroupCCL : public c10d::Backend {
   void* done_counter_ = nullptr;            // this rank's workgroup counter of the one-launch collectives
   void* fused_state_ = nullptr;             // this rank's device-resident epoch of the one-launch small allreduce
   void* status_dev_ = nullptr;              // device address of shared_->status
+  // standing offers: MCCL_PG_STANDING_OFFERS != 0 -- allreduces above the one-launch size exchange
+  // where their tensors are on the device and never meet on the host
+  bool standing_offers_ = true;
+  size_t standing_capacity_ = 0;            // staging of both slots that holds this much on every rank, mapped by every peer
+  mccl_import_table_t* import_table_ = nullptr;  // device: the peers' allocations as this rank has mapped them
+  void* resolved_ = nullptr;                // device: where the ranks' tensors of the collective under way are
+  std::vector<void*> offer_slots_[2];       // rank r's offer slot, per parity of the collective
+  std::vector<mccl_import_update_t> table_updates_;  // mappings that changed since the device table last heard
+  uint64_t seen_live_[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES] = {};  // peers' export entries as this rank last read them
+  uint64_t last_offer_seq_[MCCL_OFFER_ENTRIES] = {};               // 1 + the last collective that offered the entry (0: none)
   std::shared_ptr<GroupShared> shared_;
 
   // zero-copy exports (this rank's allocations the peers may map) and imports

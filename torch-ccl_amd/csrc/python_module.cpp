@@ -75,5 +75,7 @@ PYBIND11_MODULE(_C, m) {
       // what the bisecting switches of the environment parsed to: 1 = work only, 2 = sync only, + 4 = allreduce disabled
       .def("_bisect_mode", &ProcessGroupCCL::bisectMode)
       // collectives of this group that met at the host rendezvous / that reused a cached one
-      .def("_rendezvous_counts", &ProcessGroupCCL::rendezvousCounts);
+      .def("_rendezvous_counts", &ProcessGroupCCL::rendezvousCounts)
+      // which way the collective this rank enqueued last took (what the verbose log prints)
+      .def("_last_path", &ProcessGroupCCL::lastPath);
 }

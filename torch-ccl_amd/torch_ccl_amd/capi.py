@@ -40,7 +40,7 @@ EXPORTS = (
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
-    "mccl_rank_barrier", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
+    "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
     "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
     "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
@@ -52,6 +52,28 @@ class XSync(ctypes.Structure):
                 ("ready_epoch", ctypes.c_uint64), ("done_epoch", ctypes.c_uint64), ("done_counter", ctypes.c_void_p),
                 ("timeout_us", ctypes.c_uint64), ("status", ctypes.c_void_p),
                 ("max_compute_units", ctypes.c_uint), ("reserved", ctypes.c_uint)]
+
+
+OFFER_RANKS, OFFER_ENTRIES, OFFER_STAGED, STATUS_UNMAPPED = 8, 32, 0xffffffff, 0xfffffffe
+
+
+class Offer(ctypes.Structure):
+    """mccl_offer_t"""
+    _fields_ = [("entry", ctypes.c_uint32), ("slot", ctypes.c_uint32), ("generation", ctypes.c_uint64),
+                ("offset", ctypes.c_uint64), ("reserved", ctypes.c_uint64)]
+
+
+class ImportTable(ctypes.Structure):
+    """mccl_import_table_t"""
+    _fields_ = [("base", ctypes.c_uint64 * OFFER_ENTRIES * OFFER_RANKS),
+                ("generation", ctypes.c_uint64 * OFFER_ENTRIES * OFFER_RANKS),
+                ("staging", ctypes.c_uint64 * 2 * OFFER_RANKS)]
+
+
+class ImportUpdate(ctypes.Structure):
+    """mccl_import_update_t"""
+    _fields_ = [("rank", ctypes.c_uint32), ("entry", ctypes.c_uint32), ("slot", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+                ("base", ctypes.c_uint64), ("generation", ctypes.c_uint64)]
 
 
 class Segment(ctypes.Structure):
@@ -88,6 +110,9 @@ def lib():
     L.mccl_moe_dispatch_n.argtypes = [vp, vp, vp, vp, i32, vp, sz, vp]
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
+    L.mccl_rank_barrier_offers.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp, vp, vp, vp, vp, vp]
+    L.mccl_allreduce_sync_resolved.argtypes = [vp, sz, i32, i32, vp, vp]
+    L.mccl_import_table_update.argtypes = [vp, vp, i32, vp]
     L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, ctypes.c_uint, vp]
     L.mccl_allreduce_fused_replayable.argtypes = [vp, vp, sz, i32, i32, vp, vp, sz, sz, vp, i32, i32, ctypes.c_uint64, vp, ctypes.c_uint, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
