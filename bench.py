@@ -228,6 +228,47 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
         torch.cuda.synchronize()
         res[name]["back_to_back_us"] = (time.perf_counter() - t0) / 20 * 1e6
         del x, t
+    # What the call itself costs the host, and whether anybody's host thread waits for anybody: 20 calls of
+    # the 64 MiB allreduce (enqueue time per call, rendezvous of the host threads among them), then one
+    # 4 MiB allreduce that rank 1 enters 50 ms late (how long the OTHER ranks' calls take)
+    try:
+        be = dist.distributed_c10d._get_default_group()._get_backend(torch.device("cuda"))
+        t = torch.ones(4096 * 8192, dtype=torch.bfloat16, device="cuda:0")
+        for _ in range(3):
+            dist.all_reduce(t)
+            torch.cuda.synchronize()
+        dist.barrier()
+        before = be._rendezvous_counts()
+        enq = []
+        for _ in range(20):
+            t0 = time.perf_counter()
+            dist.all_reduce(t)
+            enq.append(time.perf_counter() - t0)
+        torch.cuda.synchronize()
+        after = be._rendezvous_counts()
+        enq.sort()
+        z = torch.ones(1 << 21, dtype=torch.bfloat16, device="cuda:0")
+        for _ in range(3):
+            dist.all_reduce(z)
+            torch.cuda.synchronize()
+        dist.barrier()
+        if rank == 1:
+            time.sleep(0.05)
+        t0 = time.perf_counter()
+        w = dist.all_reduce(z, async_op=True)
+        call_us = (time.perf_counter() - t0) * 1e6
+        w.wait()
+        torch.cuda.synchronize()
+        done_us = (time.perf_counter() - t0) * 1e6
+        res["host_side_of_all_reduce"] = {"c3_enqueue_us_p50": enq[10] * 1e6, "c3_calls": 20,
+                                          "host_rendezvous_among_them": int(after[0] - before[0]),
+                                          "path": be._last_path(),
+                                          "4MiB_call_us_on_rank_0_while_rank_1_is_50_ms_late": call_us,
+                                          "4MiB_call_plus_synchronize_us_on_rank_0": done_us}
+        del t, z
+    except Exception as e:
+        res["host_side_of_all_reduce"] = {"error": repr(e)[:200]}
+
     # C2 as a decode loop runs it: 32 allreduces recorded into one HIP graph per rank process (one launch
     # per process for all 32), replayed; once bare and once with a small kernel of the caller's between them
     try:

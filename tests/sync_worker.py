@@ -264,6 +264,101 @@ def fused_replay_case(rank, world, queues, barrier):
     barrier.wait(timeout=120)
 
 
+def offers_case(rank, world, queues, barrier):
+    """mccl_rank_barrier_offers + mccl_allreduce_sync_resolved: where each rank's tensor is travels on
+    the device.  Every rank has two "allocations" the peers have mapped (entries 3 and 17 of its
+    table, with generations of their own) and two staging buffers; from call to call a rank offers
+    a range at another offset of one of them, or its staging buffer.  Bit for bit against the
+    oracle, call after call with nothing but the kernels' own waits between them; then an offer at
+    a generation the peers have not mapped: reported, nothing written."""
+    from helpers import assert_bits_equal, bits, oracle_reduce_bits, rank_buffer
+    from oracle import oracle as O
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    BUF = 10 << 20
+    allocs = [torch.zeros(BUF, dtype=torch.uint8, device=DEV) for _ in range(2)]   # entries 3 and 17
+    stages = [torch.zeros(BUF, dtype=torch.uint8, device=DEV) for _ in range(2)]
+    ctl = torch.zeros(64, dtype=torch.int64, device=DEV)  # [0]: the flag word, [8..12) and [16..20): the two offer slots
+    counter = torch.zeros(1024, dtype=torch.int32, device=DEV)
+    table = torch.zeros(ctypes.sizeof(capi.ImportTable) // 8, dtype=torch.int64, device=DEV)
+    resolved = torch.zeros(8, dtype=torch.int64, device=DEV)
+    torch.cuda.synchronize()
+    shared = _exchange(rank, world, queues, barrier, allocs + stages + [ctl])
+    flags = capi.ptr_table([shared[r][4].data_ptr() for r in range(world)])
+    slots = [capi.ptr_table([shared[r][4].data_ptr() + 8 * (8 + 8 * sl) for r in range(world)]) for sl in range(2)]
+    st = _status()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    entries = (3, 17)
+
+    def gen_of(r, which):
+        return 100 * (r + 1) + which
+
+    # this rank's table of the peers' mappings, in stream order, at most eight entries per call
+    ups = []
+    for r in range(world):
+        if r == rank:
+            continue
+        for which in range(2):
+            ups.append(capi.ImportUpdate(r, entries[which], 0, 0, shared[r][which].data_ptr(), gen_of(r, which)))
+            ups.append(capi.ImportUpdate(r, capi.OFFER_STAGED, which, 0, shared[r][2 + which].data_ptr(), 0))
+    for at in range(0, len(ups), 8):
+        chunk = (capi.ImportUpdate * len(ups[at:at + 8]))(*ups[at:at + 8])
+        capi.check(L.mccl_import_table_update(table.data_ptr(), chunk, len(ups[at:at + 8]), stream))
+
+    ops = {"SUM": (capi.SUM, O.SUM), "AVG": (capi.AVG, O.AVG), "MAX": (capi.MAX, O.MAX)}
+    from helpers import TORCH_TO_CODE
+    pending = []
+    call = 0
+    for i, (dtype, count, name) in enumerate([(torch.bfloat16, (1 << 20) + 77, "SUM"), (torch.float32, 100003, "SUM"), (torch.int8, (3 << 20) + 5, "MAX"),
+                                              (torch.float64, 7, "SUM"), (torch.bfloat16, 3, "SUM"), (torch.float16, 1 << 21, "AVG"),
+                                              (torch.bfloat16, 4096 * 1024, "SUM"), (torch.float32, 1025, "AVG"), (torch.bfloat16, (2 << 20) + 9, "SUM")]):
+        es = torch.empty(0, dtype=dtype).element_size()
+        host = [rank_buffer(count, dtype, r, seed=900 + i, scale=0.02) for r in range(world)]
+        call += 1
+        # what this rank offers this time: by call and rank, so that every mixture occurs
+        kind = (call + rank) % 3            # 0, 1: one of its allocations, 2: its staging buffer
+        off = ((call * 37 + rank * 11) % 64) * es
+        if kind < 2:
+            where = allocs[kind][off:off + count * es].view(dtype)
+            offer = capi.Offer(entries[kind], 0, gen_of(rank, kind), off, 0)
+        else:
+            where = stages[call & 1][off:off + count * es].view(dtype)
+            offer = capi.Offer(capi.OFFER_STAGED, call & 1, 0, off, 0)
+        where.copy_(host[rank])
+        capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
+                                              where.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+        sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+        capi.check(L.mccl_allreduce_sync_resolved(resolved.data_ptr(), count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
+        pending.append((where.clone(), oracle_reduce_bits(host, ops[name][1]), (str(dtype), count, name, kind)))
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    for got, want, what in pending:
+        assert_bits_equal(bits(got), want, what)
+    assert int(counter.abs().sum()) == 0
+    # rank 0 offers an allocation at a generation nobody has mapped: every other rank reports it
+    # and leaves all tensors alone, and every launch still ends
+    barrier.wait(timeout=120)
+    call += 1
+    count = 70001
+    where = allocs[0][:count * 4].view(torch.float32)
+    where.fill_(float(rank + 1))
+    offer = capi.Offer(entries[0], 0, gen_of(rank, 0) + (7 if rank == 0 else 0), 0, 0)
+    capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
+                                          where.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+    sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+    capi.check(L.mccl_allreduce_sync_resolved(resolved.data_ptr(), count, capi.F32, capi.SUM, ctypes.byref(sy), stream))
+    torch.cuda.synchronize()
+    if rank == 0:
+        assert st.tolist() == [0, 0], st.tolist()
+    else:
+        assert st.tolist()[0] == 1 and (st.tolist()[1] & 0xffffffff) == capi.STATUS_UNMAPPED, st.tolist()
+    barrier.wait(timeout=120)
+    # (rank 0 itself resolved everybody and reduced its shard: only that shard of the tensors has changed)
+    shard = L.mccl_allreduce_sync_shard(count, world)
+    assert bool((where[shard:] == float(rank + 1)).all())
+    barrier.wait(timeout=120)
+
+
 def xrank_case(rank, world, queues, barrier):
     """The one-launch collectives that read the peers' buffers in place -- mccl_reduce_sync
     (reduce_scatter shard), mccl_allreduce_sync (in-place allreduce) and mccl_copy_segments_sync
@@ -405,5 +500,5 @@ def run_rank(rank, world, queues, barrier, mode):
     torch.set_num_threads(max(1, (os.cpu_count() or 16) // world))  # the ranks share the host's cores
     torch.cuda.set_device(0)
     {"barrier": barrier_case, "fused": fused_case, "fused_replay": fused_replay_case, "timeout": timeout_case,
-     "xrank": xrank_case}[mode](rank, world, queues, barrier)
+     "xrank": xrank_case, "offers": offers_case}[mode](rank, world, queues, barrier)
     torch.cuda.synchronize()

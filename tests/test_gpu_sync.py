@@ -34,6 +34,11 @@ def test_allreduce_fused_with_its_epoch_on_the_device_eager_and_replayed_from_a_
 
 
 @pytest.mark.parametrize("world", [2, 5, 8])
+def test_allreduce_over_offers_resolved_on_the_device(world):
+    _spawn(world, "offers")
+
+
+@pytest.mark.parametrize("world", [2, 5, 8])
 def test_one_launch_collectives_match_the_oracle(world):
     _spawn(world, "xrank")
 
