@@ -712,11 +712,14 @@ def main():
         del sink
         mccl.reduce_n(ins, out=out, op=mccl.SUM)  # the headline output again, for the checks below
 
-    # ---------------- the one-launch cross-rank kernels, all ranks played by this process ----------------
-    # Between rank processes these kernels wait for each other on flag words; here every rank's word is
-    # the same word of this process, so the launches of the 8 "ranks" run one after the other and the
-    # figure is the kernel's own (persistent grid, coherent loads, closing count), without the turn
-    # taking of 8 processes that the backend leg includes.
+    # ---------------- the cross-rank kernels, all ranks played by this process ----------------
+    # Between rank processes these kernels run behind a barrier kernel (the default): no wait at
+    # their start, fresh workgroups for the shard reduction and the push, and the last-dispatched
+    # workgroup does the closing wait on the ranks' flag words.  Here every rank's word is the same
+    # word of this process, so the closing wait passes at once and the figure is the kernel's own
+    # (closing count included), without the turn taking of 8 processes that the backend leg includes.
+    # (The form that waits at its start, MCCL_PG_SYNC=kernel, is cut to a rank's share of half the
+    # GPU's residency and only means something with eight ranks' launches side by side: backend leg.)
     if "xrank" in extras:
         L = capi.lib()
         word = torch.zeros(8, dtype=torch.int64, device=dev)
@@ -726,11 +729,9 @@ def main():
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         calls = [0]
 
-        opening = [True]  # False: the form the backend runs behind its barrier kernel (no opening wait, closing wait)
-
         def xsync(rank):
             calls[0] += 1
-            return capi.XSync(ctypes.cast(words, ctypes.c_void_p), N, rank, 4 * calls[0] + 1 if opening[0] else 0, 4 * calls[0] + 3,
+            return capi.XSync(ctypes.cast(words, ctypes.c_void_p), N, rank, 0, 4 * calls[0] + 3,
                               counter.data_ptr(), 5_000_000, status.data_ptr())
 
         def event_us(fn, reps=20):
@@ -746,12 +747,8 @@ def main():
             return e0.elapsed_time(e1) * 1e3 / reps
 
         xr = {}
-        # a rank's grid is 1/N of the wavefront budget of all ranks; here no other rank's launch is
-        # resident, so each launch gets the whole budget
-        budget = L.mccl_get_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS)
-        L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget * N)
         in_tab = capi.ptr_table([t.data_ptr() for t in ins])
-        xout = torch.empty_like(out)
+        xout = torch.zeros_like(out)
 
         def reduce_sync():
             sy = xsync(0)
@@ -779,7 +776,7 @@ def main():
                                                        "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
                                                        "first_pass_bit_identical_to_reduce_n": bool(same)}
         # the pushed allgather: rank 0's launch (its 64 MiB written into slice 0 of eight outputs)
-        gathered = [torch.empty(N * COUNT, dtype=torch.bfloat16, device=dev) for _ in range(N)]
+        gathered = [torch.zeros(N * COUNT, dtype=torch.bfloat16, device=dev) for _ in range(N)]
         dst_tab = capi.ptr_table([g.data_ptr() for g in gathered])
 
         def fanout_rank0():
@@ -790,30 +787,10 @@ def main():
         xr["fanout_sync_64MiB_into_8_outputs"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
                                                   "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
                                                   "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
-        L.mccl_set_tuning(capi.TUNE_XRANK_WAVES_ALL_RANKS, budget)
-        # the default between rank processes: a barrier kernel in front, so the data kernel does not wait
-        # at its start (fresh workgroups for the shard reduction and the push) and its last workgroup
-        # does the closing wait
-        opening[0] = False
-        behind = {}
-        xout.zero_()
-        us = event_us(reduce_sync)
-        behind["reduce_sync_8x64MiB_to_64MiB"] = {"us": round(us, 1), "pct_of_peak": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS * 100, 1),
-                                                  "bit_identical_to_reduce_n": bool(torch.equal(xout.view(torch.int16), out.view(torch.int16)))}
-        us = event_us(allreduce_rank0)
-        behind["allreduce_sync_rank0_shard_of_8x64MiB"] = {"us": round(us, 1), "pct_of_peak": round(2 * N * shard * 2 / us / 1e3 / PEAK_HBM_GBS * 100, 1)}
-        for g in gathered:
-            g[:COUNT].zero_()
-        us = event_us(fanout_rank0)
-        behind["fanout_sync_64MiB_into_8_outputs"] = {"us": round(us, 1), "pct_of_peak": round((N + 1) * COUNT * 2 / us / 1e3 / PEAK_HBM_GBS * 100, 1),
-                                                      "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
-        xr["behind_a_barrier_kernel"] = behind
-        opening[0] = True
         del gathered
         assert status.tolist()[:2] == [0, 0], status.tolist()
-        xr["wavefronts_per_launch"] = int(budget)
-        xr["note"] = ("single process: every rank's flag word is the same word, so no launch waits, and a launch has "
-                      "the wavefront budget of all ranks")
+        xr["note"] = ("single process, the form that runs behind a barrier kernel (no opening wait, closing count and "
+                      "closing wait): every rank's flag word is the same word, so no launch waits")
         result["cross_rank_kernels_single_process"] = xr
         log("cross-rank kernels:", json.dumps(xr))
         del tens, xout

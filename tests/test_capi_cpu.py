@@ -234,7 +234,10 @@ def test_ctypes_structures_match_the_header(mccl, tmp_path):
     import subprocess
     from torch_ccl_amd import capi
     layouts = {"mccl_xsync_t": (capi.XSync, [f[0] for f in capi.XSync._fields_]),
-               "mccl_segment_t": (capi.Segment, [f[0] for f in capi.Segment._fields_])}
+               "mccl_segment_t": (capi.Segment, [f[0] for f in capi.Segment._fields_]),
+               "mccl_offer_t": (capi.Offer, [f[0] for f in capi.Offer._fields_]),
+               "mccl_import_table_t": (capi.ImportTable, [f[0] for f in capi.ImportTable._fields_]),
+               "mccl_import_update_t": (capi.ImportUpdate, [f[0] for f in capi.ImportUpdate._fields_])}
     lines = ['#include <stddef.h>', '#include <stdio.h>', '#include "mccl.h"', 'int main(void) {']
     for cname, (_, fields) in layouts.items():
         lines.append('  printf("%s %%zu", sizeof(%s));' % (cname, cname))

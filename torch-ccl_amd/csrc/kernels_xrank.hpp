@@ -176,20 +176,28 @@ __device__ __forceinline__ void xrank_walk(const XRankArgs& a, const XIns& in, c
   }
 }
 
-template <int DT, int OP, int WPG>
+// INDIRECT: the tensors' addresses come from the table in device memory that the kernel in front of
+// this one has written (a kernel of its own, so that the common form starts exactly as before: a
+// wavefront of one tile lives for a few microseconds, and a chain of selects in front of its loads
+// showed as 15 % of the shard reduction's time).  Read with scalar loads, like the arguments; a table
+// entry of a rank that takes part must not be null.
+template <int DT, int OP, int WPG, bool INDIRECT>
 __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankArgs a) {
   const int n = a.sync.n;
   const Wave w = this_wave<WPG>();
   XIns in;
   bool resolved = true;
+  if constexpr (INDIRECT) {
+    const auto* table = (const __attribute__((address_space(4))) uint64_t*)a.in_table;
 #pragma unroll
-  for (int k = 0; k < kXRanks; ++k) {
-    in.p[k] = a.in[k];
-    if (a.in_table && k < n) {
-      const uint64_t p = a.in_table[k];  // uniform: written by the kernel in front of this one
-      resolved = resolved && p != 0;
+    for (int k = 0; k < kXRanks; ++k) {
+      const uint64_t p = table[k];
+      if (k < n) resolved = resolved && p != 0;
       in.p[k] = (const char*)(p + a.in_off);
     }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kXRanks; ++k) in.p[k] = a.in[k];
   }
   if (resolved && xsync_begin(a.sync)) {
     if (!a.aligned_in && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches

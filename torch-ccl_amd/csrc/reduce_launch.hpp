@@ -124,12 +124,22 @@ inline unsigned waiting_share(unsigned per_cu, unsigned cus, unsigned ranks) {
 // (the kernel walks its tiles with whatever grid it gets).
 template <int DT, int OP, int WPG>
 hipError_t launch_xrank_kernel(const XRankArgs& a, unsigned groups, unsigned lds, unsigned cus, unsigned waiting_ranks, hipStream_t s) {
+  if (a.in_table) {
+    // addresses from device memory: behind a barrier kernel only (no opening wait, single wavefronts)
+    if constexpr (WPG == 1) {
+      if (waiting_ranks) return hipErrorInvalidValue;
+      hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, 1, true>), dim3(groups, 1, 1), dim3(kWave), lds, s, a);
+      return hipGetLastError();
+    } else {
+      return hipErrorInvalidValue;
+    }
+  }
   if (waiting_ranks) {
-    static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, WPG>, kWave * WPG);  // asked once per kernel
+    static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, WPG, false>, kWave * WPG);  // asked once per kernel
     const unsigned cap = waiting_share(per_cu, cus, waiting_ranks);
     if (groups > cap) groups = cap;
   }
-  hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, WPG>), dim3(groups, 1, 1), dim3(kWave * WPG), lds, s, a);
+  hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, WPG, false>), dim3(groups, 1, 1), dim3(kWave * WPG), lds, s, a);
   return hipGetLastError();
 }
 
