@@ -405,6 +405,15 @@ int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, c
 int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
                                  void* stream);
 
+/* The two in one launch, for messages small enough for a launch on few compute units: the launch
+ * itself stores *mine into offers[rank] before its ready epoch, and after the opening wait every
+ * wavefront resolves the peers' offers against *imports as mccl_rank_barrier_offers does (an offer
+ * that does not resolve: reported, the launch only takes part in the closing wait).  sync->ready_epoch,
+ * sync->done_epoch and sync->max_compute_units must be set (the packed shape: workgroups of sixteen
+ * wavefronts on at most that many compute units). */
+int mccl_allreduce_sync_offers(size_t count, int dtype, int op, const mccl_xsync_t* sync, const mccl_offer_t* mine,
+                               const void* my_buffer, void* const* offers, const mccl_import_table_t* imports, void* stream);
+
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream);

@@ -284,12 +284,35 @@ struct OfferBarrierArgs {
   int rank;
 };
 
+// This rank's offer into its slot (by the one thread that stores the rank's flag afterwards).
+__device__ __forceinline__ void publish_offer(uint64_t* slot, const uint64_t (&mine)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) __hip_atomic_store(slot + i, mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Where rank `r`'s buffer is in this rank's address space, from the offer in its slot (read after
+// its flag has arrived) and this rank's table of mappings; 0 when this rank has not mapped it.
+__device__ __forceinline__ uint64_t resolve_offer(const uint64_t* slot, const mccl_import_table_t* imports, int r) {
+  const uint64_t w0 = __hip_atomic_load(slot + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const uint64_t gen = __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const uint64_t off = __hip_atomic_load(slot + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const uint32_t entry = (uint32_t)w0, which = (uint32_t)(w0 >> 32);
+  if (entry == MCCL_OFFER_STAGED) {
+    const uint64_t b = imports->staging[r][which & 1u];
+    return b ? b + off : 0;
+  }
+  if (entry < MCCL_OFFER_ENTRIES) {
+    const uint64_t b = imports->base[r][entry];
+    if (b && imports->generation[r][entry] == gen) return b + off;
+  }
+  return 0;
+}
+
 __global__ __launch_bounds__(kWave) void rank_barrier_offers_kernel(const OfferBarrierArgs a) {
   const int lane = threadIdx.x;
   if (lane == 0) {
     // the offer first, then the flag that says it is there
-#pragma unroll
-    for (int i = 0; i < 4; ++i) __hip_atomic_store(a.offer[a.rank] + i, a.mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    publish_offer(a.offer[a.rank], a.mine);
     __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
   if (lane >= a.n) return;
@@ -300,17 +323,7 @@ __global__ __launch_bounds__(kWave) void rank_barrier_offers_kernel(const OfferB
       report_late(a.status, lane, (uint32_t)a.epoch);
     } else {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the offer is read after the flag
-      const uint64_t w0 = __hip_atomic_load(a.offer[lane] + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      const uint64_t gen = __hip_atomic_load(a.offer[lane] + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      const uint64_t off = __hip_atomic_load(a.offer[lane] + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      const uint32_t entry = (uint32_t)w0, slot = (uint32_t)(w0 >> 32);
-      if (entry == MCCL_OFFER_STAGED) {
-        const uint64_t b = a.imports->staging[lane][slot & 1u];
-        if (b) where = b + off;
-      } else if (entry < MCCL_OFFER_ENTRIES) {
-        const uint64_t b = a.imports->base[lane][entry];
-        if (b && a.imports->generation[lane][entry] == gen) where = b + off;
-      }
+      where = resolve_offer(a.offer[lane], a.imports, lane);
       if (!where) report_late(a.status, lane, MCCL_STATUS_UNMAPPED);
     }
   }

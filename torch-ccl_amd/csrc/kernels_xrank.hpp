@@ -50,6 +50,13 @@ struct XRankArgs {
   // ranks' offers.  A null entry: the launch does nothing but take part in the closing wait.
   const uint64_t* in_table;
   uint64_t in_off;
+  // Or exchanged by this launch itself (the one-launch form with offers): this rank's offer goes into
+  // offer[rank] before its ready flag, and every wavefront resolves the peers' offers against
+  // `imports` after the opening wait (in_off applies as above).
+  uint64_t* offer[kXRanks];
+  uint64_t mine[4];
+  const mccl_import_table_t* imports;
+  uint64_t my_buffer;
   XSync sync;
 };
 
@@ -176,18 +183,21 @@ __device__ __forceinline__ void xrank_walk(const XRankArgs& a, const XIns& in, c
   }
 }
 
-// INDIRECT: the tensors' addresses come from the table in device memory that the kernel in front of
+// INDIRECT 1: the tensors' addresses come from the table in device memory that the kernel in front of
 // this one has written (a kernel of its own, so that the common form starts exactly as before: a
 // wavefront of one tile lives for a few microseconds, and a chain of selects in front of its loads
 // showed as 15 % of the shard reduction's time).  Read with scalar loads, like the arguments; a table
 // entry of a rank that takes part must not be null.
-template <int DT, int OP, int WPG, bool INDIRECT>
+// INDIRECT 2: the launch exchanges the offers itself -- the one-launch form, whose opening wait is
+// the barrier: lane r of every wavefront resolves rank r's offer once the wait has passed and the
+// addresses are broadcast into scalar registers.
+template <int DT, int OP, int WPG, int INDIRECT>
 __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankArgs a) {
   const int n = a.sync.n;
   const Wave w = this_wave<WPG>();
   XIns in;
   bool resolved = true;
-  if constexpr (INDIRECT) {
+  if constexpr (INDIRECT == 1) {
     const auto* table = (const __attribute__((address_space(4))) uint64_t*)a.in_table;
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) {
@@ -195,11 +205,35 @@ __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankAr
       if (k < n) resolved = resolved && p != 0;
       in.p[k] = (const char*)(p + a.in_off);
     }
+  } else if constexpr (INDIRECT == 2) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) publish_offer(a.offer[a.sync.rank], a.mine);  // before xsync_begin stores this rank's flag
   } else {
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) in.p[k] = a.in[k];
   }
-  if (resolved && xsync_begin(a.sync)) {
+  bool begun = resolved && xsync_begin(a.sync);
+  if constexpr (INDIRECT == 2) {
+    if (begun) {
+      uint64_t where = a.my_buffer;
+      const int r = (int)w.lane;
+      if (r < n && r != a.sync.rank) {
+        where = resolve_offer(a.offer[r], a.imports, r);
+        if (!where) report_late(a.sync.status, r, MCCL_STATUS_UNMAPPED);
+      }
+      begun = __builtin_amdgcn_ballot_w64(r < n && where == 0) == 0;
+      where += a.in_off;
+#pragma unroll
+      for (int k = 0; k < kXRanks; ++k) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)where, k);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(where >> 32), k);
+        in.p[k] = (const char*)(((uint64_t)hi << 32) | lo);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kXRanks; ++k) in.p[k] = nullptr;
+    }
+  }
+  if (begun) {
     if (!a.aligned_in && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
     if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, in, w, n);
     else xrank_walk<DT, OP, 0>(a, in, w, n);

@@ -979,8 +979,15 @@ void apply_cached_loads(XRankArgs* a) {
 
 // The in-place allreduce with its tensors' addresses from the host (tensors) or from device memory
 // (resolved: read by the kernel when it starts).
-int allreduce_sync_impl(void* const* tensors, const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
-                        void* stream) {
+struct OfferExchange {  // the launch exchanges the ranks' offers itself
+  const mccl_offer_t* mine;
+  const void* my_buffer;
+  void* const* offers;
+  const mccl_import_table_t* imports;
+};
+
+int allreduce_sync_impl(void* const* tensors, const void* resolved, const OfferExchange* ox, size_t count, int dtype, int op,
+                        const mccl_xsync_t* sync, void* stream) {
   XRankArgs a;
   memset(&a, 0, sizeof(a));
   int rc = fill_xsync(sync, &a.sync);
@@ -1015,13 +1022,30 @@ int allreduce_sync_impl(void* const* tensors, const void* resolved, size_t count
       a.in[k] = (const char*)tensors[k] + lo * es;
       if (n_me && ((uintptr_t)a.in[k] & 7u)) a.aligned_in = 0;
     }
-  } else {
+  } else if (resolved) {
     // where the tensors lie is not known here: any alignment, read through the caches (the barrier
     // in front has ordered the ranks, so the caches start clean)
     a.in_table = (const uint64_t*)resolved;
     a.in_off = lo * es;
     a.aligned_in = 0;
     a.no_invalidate = 1;
+  } else {
+    // the same, the offers exchanged by this launch: the peers' data was complete before their
+    // launches began, but lines of it may sit in this launch's caches from before: one invalidate
+    // per workgroup after the opening wait (aligned_in 0 without no_invalidate)
+    for (int r = 0; r < n; ++r) {
+      if (!ox->offers[r]) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is null", r);
+      if ((uintptr_t)ox->offers[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is not 8-byte aligned", r);
+      a.offer[r] = (uint64_t*)ox->offers[r];
+    }
+    a.mine[0] = (uint64_t)ox->mine->entry | ((uint64_t)ox->mine->slot << 32);
+    a.mine[1] = ox->mine->generation;
+    a.mine[2] = ox->mine->offset;
+    a.mine[3] = ox->mine->reserved;
+    a.imports = ox->imports;
+    a.my_buffer = (uint64_t)(uintptr_t)ox->my_buffer;
+    a.in_off = lo * es;
+    a.aligned_in = 0;
   }
   a.push = 1;
   a.nvec1 = (uint32_t)(n_me / ve);
@@ -1197,7 +1221,7 @@ size_t mccl_allreduce_sync_shard(size_t count, int n) {
 
 int mccl_allreduce_sync(void* const* tensors, size_t count, int dtype, int op, const mccl_xsync_t* sync, void* stream) {
   if (!tensors) return fail(MCCL_ERR_INVALID_ARG, "tensor table is null");
-  return allreduce_sync_impl(tensors, nullptr, count, dtype, op, sync, stream);
+  return allreduce_sync_impl(tensors, nullptr, nullptr, count, dtype, op, sync, stream);
 }
 
 int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, int op, const mccl_xsync_t* sync,
@@ -1206,7 +1230,18 @@ int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, 
   if ((uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "address table is not 8-byte aligned");
   if (sync && (sync->ready_epoch != 0 || sync->done_epoch == 0))
     return fail(MCCL_ERR_INVALID_ARG, "the allreduce over resolved addresses runs behind a barrier: ready_epoch 0, done_epoch set");
-  return allreduce_sync_impl(nullptr, resolved, count, dtype, op, sync, stream);
+  return allreduce_sync_impl(nullptr, resolved, nullptr, count, dtype, op, sync, stream);
+}
+
+int mccl_allreduce_sync_offers(size_t count, int dtype, int op, const mccl_xsync_t* sync, const mccl_offer_t* mine,
+                               const void* my_buffer, void* const* offers, const mccl_import_table_t* imports, void* stream) {
+  if (!mine || !offers || !imports) return fail(MCCL_ERR_INVALID_ARG, "offer, offer table or import table is null");
+  if ((uintptr_t)imports % 8) return fail(MCCL_ERR_INVALID_ARG, "import table is not 8-byte aligned");
+  if (mine->entry != MCCL_OFFER_STAGED && mine->entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "offer names entry %u of %d", mine->entry, MCCL_OFFER_ENTRIES);
+  if (sync && (sync->ready_epoch == 0 || sync->done_epoch == 0 || sync->max_compute_units == 0))
+    return fail(MCCL_ERR_INVALID_ARG, "the one-launch allreduce with offers needs ready_epoch, done_epoch and max_compute_units");
+  const OfferExchange ox{mine, my_buffer, offers, imports};
+  return allreduce_sync_impl(nullptr, nullptr, &ox, count, dtype, op, sync, stream);
 }
 
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream) {

@@ -1065,8 +1065,6 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
   ++enqueue_only_count_;
   flushImportTable(s);
   const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
-  MCCL_CHECK(mccl_rank_barrier_offers(bar_flags_.data(), size_, rank_, epoch + 1, limit_us, status_dev_, &mine, buffer,
-                                      offer_slots_[slot].data(), import_table_, resolved_, s));
   mccl_xsync_t sync{};
   sync.words = bar_flags_.data();
   sync.n = size_;
@@ -1075,7 +1073,19 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
   sync.done_counter = done_counter_;
   sync.timeout_us = limit_us;
   sync.status = status_dev_;
-  MCCL_CHECK(mccl_allreduce_sync_resolved(resolved_, plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, s));
+  if ((double)bytes * plan.compact_cost <= (double)compact_max_) {
+    // little to move: ONE launch on this rank's share of half of the compute units, which carries the
+    // offers itself (its opening wait is the barrier) -- with several processes on the GPU every
+    // launch waits for its turn at the dispatcher, which costs more than the data at these sizes
+    sync.ready_epoch = epoch + 1;
+    sync.max_compute_units = std::max(1u, waiting_cus_ / (unsigned)size_);
+    MCCL_CHECK(mccl_allreduce_sync_offers(plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, &mine, buffer,
+                                          offer_slots_[slot].data(), import_table_, s));
+  } else {
+    MCCL_CHECK(mccl_rank_barrier_offers(bar_flags_.data(), size_, rank_, epoch + 1, limit_us, status_dev_, &mine, buffer,
+                                        offer_slots_[slot].data(), import_table_, resolved_, s));
+    MCCL_CHECK(mccl_allreduce_sync_resolved(resolved_, plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, s));
+  }
   if (!in_place) copyAsync(plan.fused_ptr, buffer, bytes, s);
 }
 

@@ -128,18 +128,31 @@ hipError_t launch_xrank_kernel(const XRankArgs& a, unsigned groups, unsigned lds
     // addresses from device memory: behind a barrier kernel only (no opening wait, single wavefronts)
     if constexpr (WPG == 1) {
       if (waiting_ranks) return hipErrorInvalidValue;
-      hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, 1, true>), dim3(groups, 1, 1), dim3(kWave), lds, s, a);
+      hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, 1, 1>), dim3(groups, 1, 1), dim3(kWave), lds, s, a);
+      return hipGetLastError();
+    } else {
+      return hipErrorInvalidValue;
+    }
+  }
+  if (a.imports) {
+    // the launch exchanges the offers itself: the one-launch form on few compute units (packed)
+    if constexpr (WPG == kPackedWaves) {
+      if (!waiting_ranks) return hipErrorInvalidValue;
+      static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, kPackedWaves, 2>, kWave * kPackedWaves);
+      const unsigned cap = waiting_share(per_cu, cus, waiting_ranks);
+      if (groups > cap) groups = cap;
+      hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, kPackedWaves, 2>), dim3(groups, 1, 1), dim3(kWave * kPackedWaves), lds, s, a);
       return hipGetLastError();
     } else {
       return hipErrorInvalidValue;
     }
   }
   if (waiting_ranks) {
-    static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, WPG, false>, kWave * WPG);  // asked once per kernel
+    static const unsigned per_cu = blocks_per_cu(xrank_reduce_kernel<DT, OP, WPG, 0>, kWave * WPG);  // asked once per kernel
     const unsigned cap = waiting_share(per_cu, cus, waiting_ranks);
     if (groups > cap) groups = cap;
   }
-  hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, WPG, false>), dim3(groups, 1, 1), dim3(kWave * WPG), lds, s, a);
+  hipLaunchKernelGGL((xrank_reduce_kernel<DT, OP, WPG, 0>), dim3(groups, 1, 1), dim3(kWave * WPG), lds, s, a);
   return hipGetLastError();
 }
 
