@@ -325,11 +325,17 @@ def offers_case(rank, world, queues, barrier):
             where = stages[call & 1][off:off + count * es].view(dtype)
             offer = capi.Offer(capi.OFFER_STAGED, call & 1, 0, off, 0)
         where.copy_(host[rank])
-        capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
-                                              where.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
-        sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
-        capi.check(L.mccl_allreduce_sync_resolved(resolved.data_ptr(), count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
-        pending.append((where.clone(), oracle_reduce_bits(host, ops[name][1]), (str(dtype), count, name, kind)))
+        if i % 2 == 0:  # a barrier kernel that carries the offers, then the allreduce over the resolved addresses
+            capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
+                                                  where.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+            capi.check(L.mccl_allreduce_sync_resolved(resolved.data_ptr(), count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), stream))
+        else:           # one launch that does both, on few compute units
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 4 * call + 1, 4 * call + 3, counter.data_ptr(), 5_000_000,
+                            st.data_ptr(), (16, 3)[i % 4 == 1], 0)
+            capi.check(L.mccl_allreduce_sync_offers(count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), ctypes.byref(offer),
+                                                    where.data_ptr(), slots[call & 1], table.data_ptr(), stream))
+        pending.append((where.clone(), oracle_reduce_bits(host, ops[name][1]), (str(dtype), count, name, kind, i % 2)))
     torch.cuda.synchronize()
     assert st.tolist() == [0, 0], st.tolist()
     for got, want, what in pending:
