@@ -414,6 +414,25 @@ int mccl_allreduce_sync_resolved(const void* resolved, size_t count, int dtype, 
 int mccl_allreduce_sync_offers(size_t count, int dtype, int op, const mccl_xsync_t* sync, const mccl_offer_t* mine,
                                const void* my_buffer, void* const* offers, const mccl_import_table_t* imports, void* stream);
 
+/* mccl_reduce_sync and mccl_fanout_sync over addresses from the ranks' offers, in the same two
+ * forms: `_resolved` behind mccl_rank_barrier_offers (sync->ready_epoch 0, done_epoch set), `_offers`
+ * as one launch on few compute units that exchanges the offers itself (ready_epoch, done_epoch and
+ * max_compute_units set).  What a rank offers is the buffer its peers address: for the shard
+ * reduction (reduce_scatter) its whole input, of which rank r reads the `count` elements at byte
+ * in_offset (its slice) of every rank's; for the push (allgather) its whole output, into which rank r
+ * writes its `bytes` at byte dst_offset (its slice) of every rank's -- of its own as well, unless
+ * skip_own is set (in place: the contribution already sits there). */
+int mccl_reduce_sync_resolved(const void* resolved, size_t in_offset, void* out, size_t count, int dtype, int op,
+                              const mccl_xsync_t* sync, void* stream);
+int mccl_reduce_sync_offers(size_t in_offset, void* out, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                            const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                            const mccl_import_table_t* imports, void* stream);
+int mccl_fanout_sync_resolved(const void* src, const void* resolved, size_t dst_offset, size_t bytes, int skip_own,
+                              const mccl_xsync_t* sync, void* stream);
+int mccl_fanout_sync_offers(const void* src, size_t dst_offset, size_t bytes, int skip_own, const mccl_xsync_t* sync,
+                            const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                            const mccl_import_table_t* imports, void* stream);
+
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream);

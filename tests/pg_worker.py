@@ -549,16 +549,15 @@ def large_message_case(pg, rank, world):
 
 
 def missing_rank_case(pg, rank, world):
-    """Rank 1 never joins the second collective: the others must get an error, not hang.  (A
-    reduce_scatter_tensor of 2 MiB per rank: a collective whose host threads meet first in every
-    mode -- to agree on reading the tensors in place, or around the launches -- so the call itself
-    raises.)"""
+    """Rank 1 never joins the second collective: the others must get an error, not hang.  (An
+    all_to_all_single of 2 MiB per rank: a collective whose host threads meet first in every mode
+    -- its split tables are published per call -- so the call itself raises.)"""
     t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
     try:
-        pg._reduce_scatter_base(t, torch.ones(world << 19, device=DEV)).wait()
+        pg.alltoall_base(torch.empty(world << 17, device=DEV), torch.ones(world << 17, device=DEV), [], []).wait()
         raise AssertionError("collective with a missing rank returned")
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)

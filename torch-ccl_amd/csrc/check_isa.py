@@ -155,7 +155,8 @@ def scan_hints(asm_path):
     return bad
 
 
-_WAITING_KERNEL = re.compile(r"(xrank_reduce_kernel|copy_segments_sync_kernel|fanout_sync_kernel|allreduce_fused_kernel|rank_barrier_kernel)")
+_WAITING_KERNEL = re.compile(r"(xrank_reduce_kernel|copy_segments_sync_kernel|fanout_sync_kernel|fanout_indirect_kernel|allreduce_fused_kernel|"
+                             r"rank_barrier_kernel|rank_barrier_offers_kernel)")
 _MAX_VGPRS_OF_WAITING_KERNELS = 128
 
 

@@ -122,7 +122,21 @@ struct FanoutArgs {
   uint32_t tiles;    // 1 KiB tiles that cover the vectors
   uint32_t aligned;  // every destination is 16-byte aligned
   int ndst;
+  // The destinations from device memory instead (INDIRECT kernels): rank k's buffer + dst_off, for
+  // every rank k < sync.n whose bit is set in dst_mask -- resolved by the barrier kernel in front
+  // (dst_table), or from the ranks' offers by this launch itself (offer / mine / imports / my_buffer).
+  const uint64_t* dst_table;
+  uint64_t dst_off;
+  uint32_t dst_mask;
+  uint64_t* offer[kLeanSyncRanks];
+  uint64_t mine[4];
+  const mccl_import_table_t* imports;
+  uint64_t my_buffer;
   XSync sync;
+};
+
+struct FanoutDst {  // only ever indexed with constants: scalar registers
+  char* p[kLeanSyncRanks];
 };
 
 __device__ __forceinline__ u32x4 fanout_load(const FanoutArgs& a, uint32_t tile, uint32_t lane) {
@@ -141,6 +155,76 @@ __device__ __forceinline__ void fanout_store(const FanoutArgs& a, uint32_t tile,
       else store_vec_through(tb + lane * 16u, x);
     }
   }
+}
+
+// The same with the destinations in `d` (any alignment), those whose bit is set in the mask.
+__device__ __forceinline__ void fanout_store_to(const FanoutArgs& a, const FanoutDst& d, uint32_t tile, uint32_t lane, u32x4 x) {
+  if (tile * kWave + lane >= a.nvec) return;
+#pragma unroll
+  for (int k = 0; k < kLeanSyncRanks; ++k)
+    if (a.dst_mask & (1u << k)) store_vec_through(d.p[k] + (size_t)tile * (kWave * 16u) + lane * 16u, x);
+}
+
+// INDIRECT 1: behind a barrier kernel that has resolved the ranks' offers; INDIRECT 2: the launch
+// exchanges the offers itself (see xrank_reduce_kernel).
+template <int WPG, int INDIRECT>
+__global__ __launch_bounds__(kWave * WPG) void fanout_indirect_kernel(const FanoutArgs a) {
+  const Wave w = this_wave<WPG>();
+  const int n = a.sync.n;
+  FanoutDst d;
+  bool resolved = true;
+  if constexpr (INDIRECT == 1) {
+    const auto* table = (const __attribute__((address_space(4))) uint64_t*)a.dst_table;
+#pragma unroll
+    for (int k = 0; k < kLeanSyncRanks; ++k) {
+      const uint64_t p = table[k];
+      if (k < n) resolved = resolved && p != 0;
+      d.p[k] = (char*)(p + a.dst_off);
+    }
+  } else {
+    if (blockIdx.x == 0 && threadIdx.x == 0) publish_offer(a.offer[a.sync.rank], a.mine);  // before xsync_begin stores this rank's flag
+  }
+  bool begun = resolved && xsync_begin(a.sync);
+  if constexpr (INDIRECT == 2) {
+    if (begun) {
+      uint64_t where = a.my_buffer;
+      const int r = (int)w.lane;
+      if (r < n && r != a.sync.rank) {
+        where = resolve_offer(a.offer[r], a.imports, r);
+        if (!where) report_late(a.sync.status, r, MCCL_STATUS_UNMAPPED);
+      }
+      begun = __builtin_amdgcn_ballot_w64(r < n && where == 0) == 0;
+      where += a.dst_off;
+#pragma unroll
+      for (int k = 0; k < kLeanSyncRanks; ++k) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)where, k);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(where >> 32), k);
+        d.p[k] = (char*)(((uint64_t)hi << 32) | lo);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kLeanSyncRanks; ++k) d.p[k] = nullptr;
+    }
+  }
+  if (begun) {
+    const uint32_t T = a.tiles, G = w.count;
+    for (uint32_t t0 = w.index; t0 < T; t0 += 2 * G) {  // two tiles' loads in flight
+      const uint32_t t1 = t0 + G;
+      const u32x4 x0 = fanout_load(a, t0, w.lane);
+      u32x4 x1 = (u32x4){0u, 0u, 0u, 0u};
+      if (t1 < T) x1 = fanout_load(a, t1, w.lane);
+      fanout_store_to(a, d, t0, w.lane, x0);
+      if (t1 < T) fanout_store_to(a, d, t1, w.lane, x1);
+    }
+    if (a.tail && w.index == w.count - 1 && w.lane < a.tail) {
+      const size_t i = (size_t)a.nvec * 16u + w.lane;
+      const unsigned char b = (unsigned char)a.src[i];
+#pragma unroll
+      for (int k = 0; k < kLeanSyncRanks; ++k)
+        if (a.dst_mask & (1u << k)) __hip_atomic_store((unsigned char*)d.p[k] + i, b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+  xsync_end(a.sync, gridDim.x);
 }
 
 template <int WPG>

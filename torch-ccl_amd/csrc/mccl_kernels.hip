@@ -1213,6 +1213,162 @@ int mccl_reduce_sync(const void* const* in, void* out, size_t count, int dtype, 
   return MCCL_OK;
 }
 
+}  // extern "C"
+
+namespace {
+
+int check_offer_exchange(const OfferExchange& ox, int n) {
+  if (!ox.mine || !ox.offers || !ox.imports) return fail(MCCL_ERR_INVALID_ARG, "offer, offer table or import table is null");
+  if ((uintptr_t)ox.imports % 8) return fail(MCCL_ERR_INVALID_ARG, "import table is not 8-byte aligned");
+  if (ox.mine->entry != MCCL_OFFER_STAGED && ox.mine->entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "offer names entry %u of %d", ox.mine->entry, MCCL_OFFER_ENTRIES);
+  for (int r = 0; r < n; ++r) {
+    if (!ox.offers[r]) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is null", r);
+    if ((uintptr_t)ox.offers[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is not 8-byte aligned", r);
+  }
+  return MCCL_OK;
+}
+
+void offer_words(const mccl_offer_t& mine, uint64_t (&w)[4]) {
+  w[0] = (uint64_t)mine.entry | ((uint64_t)mine.slot << 32);
+  w[1] = mine.generation;
+  w[2] = mine.offset;
+  w[3] = mine.reserved;
+}
+
+int check_indirect_sync(const mccl_xsync_t* sync, bool one_launch) {
+  if (!sync) return MCCL_OK;  // fill_xsync reports it
+  if (one_launch) {
+    if (sync->ready_epoch == 0 || sync->done_epoch == 0 || sync->max_compute_units == 0)
+      return fail(MCCL_ERR_INVALID_ARG, "the one-launch form with offers needs ready_epoch, done_epoch and max_compute_units");
+  } else if (sync->ready_epoch != 0 || sync->done_epoch == 0) {
+    return fail(MCCL_ERR_INVALID_ARG, "a launch over resolved addresses runs behind a barrier: ready_epoch 0, done_epoch set");
+  }
+  return MCCL_OK;
+}
+
+// The shard reduction over addresses from the ranks' offers: `resolved` (behind the barrier that
+// resolved them) or `ox` (the launch exchanges them itself).
+int reduce_sync_indirect(const void* resolved, const OfferExchange* ox, size_t in_offset, void* out, size_t count, int dtype,
+                         int op, const mccl_xsync_t* sync, void* stream) {
+  XRankArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_reduce_args_no_ptr(a.sync.n, dtype, op);
+  if (rc != MCCL_OK) return rc;
+  rc = check_indirect_sync(sync, ox != nullptr);
+  if (rc != MCCL_OK) return rc;
+  const size_t es = dtype_size(dtype);
+  if (in_offset % es) return fail(MCCL_ERR_INVALID_ARG, "input offset not aligned to the element size");
+  if (count) {
+    if (!out) return fail(MCCL_ERR_INVALID_ARG, "output pointer is null");
+    if ((uintptr_t)out % es) return fail(MCCL_ERR_INVALID_ARG, "output pointer not aligned to the element size");
+  }
+  const size_t ve = 16 / es;
+  const uint64_t vecs = count / ve + (count % ve ? 1 : 0);
+  if (vecs + kWave > 0xffffffffull) return fail(MCCL_ERR_INVALID_ARG, "message too large");
+  a.out1 = (char*)out;
+  a.nvec1 = (uint32_t)(count / ve);
+  a.tail1 = (uint32_t)(count % ve);
+  a.tiles1 = (uint32_t)((vecs + kWave - 1) / kWave);
+  a.stream_out = count * es >= (32u << 20) ? 1u : 0u;
+  a.in_off = in_offset;
+  a.aligned_in = 0;  // where the inputs lie is not known here: any alignment, through the caches
+  if (resolved) {
+    a.in_table = (const uint64_t*)resolved;
+    a.no_invalidate = 1;  // behind a kernel boundary: the caches start clean
+  } else {
+    rc = check_offer_exchange(*ox, a.sync.n);
+    if (rc != MCCL_OK) return rc;
+    for (int r = 0; r < a.sync.n; ++r) a.offer[r] = (uint64_t*)ox->offers[r];
+    offer_words(*ox->mine, a.mine);
+    a.imports = ox->imports;
+    a.my_buffer = (uint64_t)(uintptr_t)ox->my_buffer;
+  }
+  const XShape shape = xrank_shape(a.tiles1, sync, a.sync.ready_epoch != 0, /*fresh_tiles=*/1);
+  hipError_t e = launch_xrank_any(a, dtype, op, shape.groups, shape.packed, shape.lds, a.sync.ready_epoch != 0 ? (unsigned)a.sync.n : 0u, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "reduce kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int fanout_sync_indirect(const void* src, const void* resolved, const OfferExchange* ox, size_t dst_offset, size_t bytes,
+                         int skip_own, const mccl_xsync_t* sync, void* stream) {
+  FanoutArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_indirect_sync(sync, ox != nullptr);
+  if (rc != MCCL_OK) return rc;
+  if (bytes / 16 > 0xf0000000ull) return fail(MCCL_ERR_INVALID_ARG, "message too large for one push");
+  if (bytes && !src) return fail(MCCL_ERR_INVALID_ARG, "source pointer is null");
+  a.src = (const char*)src;
+  a.nvec = (uint32_t)(bytes / 16);
+  a.tail = (uint32_t)(bytes % 16);
+  a.tiles = (uint32_t)((bytes / 16 + kWave - 1) / kWave);
+  a.dst_off = dst_offset;
+  a.dst_mask = (1u << a.sync.n) - 1u;
+  if (skip_own) a.dst_mask &= ~(1u << a.sync.rank);
+  if (resolved) {
+    a.dst_table = (const uint64_t*)resolved;
+  } else {
+    rc = check_offer_exchange(*ox, a.sync.n);
+    if (rc != MCCL_OK) return rc;
+    for (int r = 0; r < a.sync.n; ++r) a.offer[r] = (uint64_t*)ox->offers[r];
+    offer_words(*ox->mine, a.mine);
+    a.imports = ox->imports;
+    a.my_buffer = (uint64_t)(uintptr_t)ox->my_buffer;
+  }
+  const XShape shape = xrank_shape(a.tiles, sync, a.sync.ready_epoch != 0, /*fresh_tiles=*/2);
+  unsigned grid = shape.groups;
+  int cus = 0;
+  rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  if (ox) {
+    if (!shape.packed) return fail(MCCL_ERR_INVALID_ARG, "the one-launch push with offers runs packed (max_compute_units)");
+    static const unsigned per_cu = blocks_per_cu(fanout_indirect_kernel<kPackedWaves, 2>, kWave * kPackedWaves);
+    grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
+    hipLaunchKernelGGL((fanout_indirect_kernel<kPackedWaves, 2>), dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  } else {
+    if (shape.packed) return fail(MCCL_ERR_INVALID_ARG, "a push over resolved addresses runs as single wavefronts (max_compute_units 0)");
+    hipLaunchKernelGGL((fanout_indirect_kernel<1, 1>), dim3(grid), dim3(kWave), shape.lds, (hipStream_t)stream, a);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "push kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_reduce_sync_resolved(const void* resolved, size_t in_offset, void* out, size_t count, int dtype, int op,
+                              const mccl_xsync_t* sync, void* stream) {
+  if (!resolved) return fail(MCCL_ERR_INVALID_ARG, "address table is null");
+  if ((uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "address table is not 8-byte aligned");
+  return reduce_sync_indirect(resolved, nullptr, in_offset, out, count, dtype, op, sync, stream);
+}
+
+int mccl_reduce_sync_offers(size_t in_offset, void* out, size_t count, int dtype, int op, const mccl_xsync_t* sync,
+                            const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                            const mccl_import_table_t* imports, void* stream) {
+  const OfferExchange ox{mine, my_buffer, offers, imports};
+  return reduce_sync_indirect(nullptr, &ox, in_offset, out, count, dtype, op, sync, stream);
+}
+
+int mccl_fanout_sync_resolved(const void* src, const void* resolved, size_t dst_offset, size_t bytes, int skip_own,
+                              const mccl_xsync_t* sync, void* stream) {
+  if (!resolved) return fail(MCCL_ERR_INVALID_ARG, "address table is null");
+  if ((uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "address table is not 8-byte aligned");
+  return fanout_sync_indirect(src, resolved, nullptr, dst_offset, bytes, skip_own, sync, stream);
+}
+
+int mccl_fanout_sync_offers(const void* src, size_t dst_offset, size_t bytes, int skip_own, const mccl_xsync_t* sync,
+                            const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
+                            const mccl_import_table_t* imports, void* stream) {
+  const OfferExchange ox{mine, my_buffer, offers, imports};
+  return fanout_sync_indirect(src, nullptr, &ox, dst_offset, bytes, skip_own, sync, stream);
+}
+
 size_t mccl_allreduce_sync_shard(size_t count, int n) {
   if (n < 1) return 0;
   const size_t per = (count + (size_t)n - 1) / (size_t)n;

@@ -493,6 +493,7 @@ ProcessGroupCCL::ProcessGroupCCL(const c10::intrusive_ptr<c10d::Store>& store, i
   if (const char* v = std::getenv("MCCL_PG_COMPACT_MAX_BYTES")) compact_max_ = (size_t)std::atoll(v);
   allgather_push_ = envFlag("MCCL_PG_ALLGATHER_PUSH", true);
   standing_offers_ = envFlag("MCCL_PG_STANDING_OFFERS", true);
+  if (const char* v = std::getenv("MCCL_PG_STANDING_MAX_BYTES")) standing_max_ = (size_t)std::atoll(v);
   work_only_ = envFlag("TORCH_CCL_WORK_ONLY", false) || envFlag("MCCL_PG_WORK_ONLY", false);
   sync_only_ = envFlag("TORCH_CCL_SYNC_ONLY", false) || envFlag("MCCL_PG_SYNC_ONLY", false);
   disable_allreduce_ = envFlag("TORCH_CCL_DISABLE_ALLREDUCE", false) || envFlag("MCCL_PG_DISABLE_ALLREDUCE", false);
@@ -1029,22 +1030,25 @@ void ProcessGroupCCL::growStandingCapacity(size_t bytes) {
 }
 
 bool ProcessGroupCCL::standingFits(const Plan& plan) const {
-  return standing_offers_ && plan.standing_ok && device_sync_ && distinct_pids_ && zero_copy_ && !waits_in_data_kernels_ &&
-         !work_only_ && !sync_only_ && size_ <= MCCL_OFFER_RANKS &&
-         plan.fused_count * mccl_dtype_size(plan.fused_dtype) <= stage_max_;
+  return standing_offers_ && plan.standing.ok && device_sync_ && distinct_pids_ && zero_copy_ && !waits_in_data_kernels_ &&
+         !work_only_ && !sync_only_ && size_ <= MCCL_OFFER_RANKS && plan.standing.bytes > 0 &&
+         plan.standing.bytes <= std::min(stage_max_, standing_max_);
 }
 
 void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
-  const size_t bytes = plan.fused_count * mccl_dtype_size(plan.fused_dtype);
+  const Plan::Standing& st = plan.standing;
+  const size_t bytes = st.bytes;
   const uint64_t epoch = 4 * seq;
   if (bytes > standing_capacity_) growStandingCapacity(bytes);
   scanPeerExports(seq);
   uint64_t off = 0;
-  const int entry = exportRange(plan.fused_ptr, bytes, &off);
+  // (small buffers live in the allocator's 2 MiB segments, many of them: announcing those would turn
+  // the table of allocations over all the time, and copying them costs next to nothing)
+  const int entry = (st.force_staged || bytes < kZeroCopyMinBytes) ? -1 : exportRange(st.buffer, bytes, &off);
   const uint64_t gen = entry >= 0 ? ctl_->slot[rank_].exports[entry].gen.load(std::memory_order_acquire) : 0;
   const bool in_place = entry >= 0 && allAcknowledged(entry, gen, seq);
   mccl_offer_t mine{};
-  void* buffer = plan.fused_ptr;
+  void* buffer = st.buffer;
   if (in_place) {
     mine.entry = (uint32_t)entry;
     mine.generation = gen;
@@ -1052,7 +1056,7 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
     last_offer_seq_[entry] = seq + 1;  // in the units of `entered`: collective `seq` is under way at seq + 1
   } else {
     buffer = stage_[slot].ptr;
-    copyAsync(buffer, plan.fused_ptr, bytes, s);
+    if (st.copy_in) copyAsync(buffer, st.buffer, bytes, s);
     mine.entry = MCCL_OFFER_STAGED;
     mine.slot = (uint32_t)slot;
   }
@@ -1069,24 +1073,23 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
   sync.words = bar_flags_.data();
   sync.n = size_;
   sync.rank = rank_;
-  sync.done_epoch = epoch + 3;  // nobody's stream goes on before every rank has written its shard everywhere
+  sync.done_epoch = epoch + 3;  // nobody's stream goes on before every rank is done with every rank's buffer
   sync.done_counter = done_counter_;
   sync.timeout_us = limit_us;
   sync.status = status_dev_;
-  if ((double)bytes * plan.compact_cost <= (double)compact_max_) {
+  if ((double)bytes * st.compact_cost <= (double)compact_max_) {
     // little to move: ONE launch on this rank's share of half of the compute units, which carries the
     // offers itself (its opening wait is the barrier) -- with several processes on the GPU every
     // launch waits for its turn at the dispatcher, which costs more than the data at these sizes
     sync.ready_epoch = epoch + 1;
     sync.max_compute_units = std::max(1u, waiting_cus_ / (unsigned)size_);
-    MCCL_CHECK(mccl_allreduce_sync_offers(plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, &mine, buffer,
-                                          offer_slots_[slot].data(), import_table_, s));
+    st.one_launch(!in_place, sync, mine, buffer, offer_slots_[slot].data(), import_table_, s);
   } else {
     MCCL_CHECK(mccl_rank_barrier_offers(bar_flags_.data(), size_, rank_, epoch + 1, limit_us, status_dev_, &mine, buffer,
                                         offer_slots_[slot].data(), import_table_, resolved_, s));
-    MCCL_CHECK(mccl_allreduce_sync_resolved(resolved_, plan.fused_count, plan.fused_dtype, plan.fused_op, &sync, s));
+    st.behind_barrier(resolved_, !in_place, sync, s);
   }
-  if (!in_place) copyAsync(plan.fused_ptr, buffer, bytes, s);
+  if (!in_place && st.copy_out) copyAsync(st.buffer, buffer, bytes, s);
 }
 
 void ProcessGroupCCL::closeImports() {
@@ -1773,7 +1776,19 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       // Small messages between rank processes: one launch does copy-in, rank synchronisation and
       // the N-peer sum (the reference's small allreduce, src/gpu/allreduce_small.h:166-361).
       p.fused_ok = len * es <= kFusedMaxBytes;
-      p.standing_ok = true;  // whatever is too large for that launch: offers resolved on the device, no rendezvous
+      // whatever is too large for that launch: where the tensors are is exchanged on the device, no rendezvous
+      p.standing.ok = true;
+      p.standing.buffer = base;
+      p.standing.bytes = len * es;
+      p.standing.copy_in = p.standing.copy_out = true;
+      p.standing.compact_cost = 1.0;
+      p.standing.behind_barrier = [=](const void* resolved, bool, const mccl_xsync_t& sync, hipStream_t s) {
+        MCCL_CHECK(mccl_allreduce_sync_resolved(resolved, len, dtype, op, &sync, s));
+      };
+      p.standing.one_launch = [=](bool, const mccl_xsync_t& sync, const mccl_offer_t& mine, const void* buffer, void* const* offers,
+                                  const mccl_import_table_t* imports, hipStream_t s) {
+        MCCL_CHECK(mccl_allreduce_sync_offers(len, dtype, op, &sync, &mine, buffer, offers, imports, s));
+      };
       p.fused_ptr = base;
       p.fused_count = len;
       p.fused_dtype = dtype;
@@ -1940,6 +1955,27 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
       // too large to be shared leaves the pulls: the inputs are offered instead.  Which of the two
       // depends on sizes only, which agree across the ranks.
       const bool push = allgather_push_ && (uint64_t)per_rank * (uint64_t)W < kShareMaxAllocation;
+      if (push && len == per_rank && W <= MCCL_OFFER_RANKS) {
+        // One window, at most eight ranks: no rendezvous.  What the peers address is this rank's whole
+        // OUTPUT, into which rank r writes slice r; a rank that stages receives in its staging buffer
+        // and copies it out afterwards (also when its input lies inside another rank's slice of its
+        // output).  In place -- the input is this rank's slice of its output -- nothing is written there.
+        const bool input_is_own_slice = (const char*)input.data_ptr() == (const char*)output.data_ptr() + (size_t)me * per_rank;
+        p.standing.ok = true;
+        p.standing.buffer = output.data_ptr();
+        p.standing.bytes = per_rank * (size_t)W;
+        p.standing.copy_out = true;
+        p.standing.force_staged = touchesForeignSlice(input.data_ptr(), per_rank, output.data_ptr(), per_rank, W, me);
+        p.standing.compact_cost = 1.0;
+        p.standing.behind_barrier = [=](const void* resolved, bool staged, const mccl_xsync_t& sync, hipStream_t s) {
+          MCCL_CHECK(mccl_fanout_sync_resolved(in, resolved, (size_t)me * per_rank, per_rank, !staged && input_is_own_slice, &sync, s));
+        };
+        p.standing.one_launch = [=](bool staged, const mccl_xsync_t& sync, const mccl_offer_t& mine, const void* buffer, void* const* offers,
+                                    const mccl_import_table_t* imports, hipStream_t s) {
+          MCCL_CHECK(mccl_fanout_sync_offers(in, (size_t)me * per_rank, per_rank, !staged && input_is_own_slice, &sync, &mine, buffer,
+                                             offers, imports, s));
+        };
+      }
       if (push) {
         p.share = len * (size_t)W >= kZeroCopyMinBytes;
         // (an input inside another rank's slice of the output: nothing is offered, and then every rank stages)
@@ -2163,6 +2199,24 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
           MCCL_CHECK(mccl_copy_segments(segs.data(), W, s));
         }
       };
+      // One window, at most eight ranks: no rendezvous.  What the peers address is this rank's whole
+      // input (rank r reads slice r of everybody's); a rank that stages copies its input first,
+      // which is also how an output inside another rank's slice of the input is handled.
+      if (len == M) {
+        p.standing.ok = true;
+        p.standing.buffer = in;
+        p.standing.bytes = M * es * (size_t)W;
+        p.standing.copy_in = true;
+        p.standing.force_staged = touchesForeignSlice(output.data_ptr(), M * es, in, M * es, W, me);
+        p.standing.compact_cost = 0.5;
+        p.standing.behind_barrier = [=](const void* resolved, bool, const mccl_xsync_t& sync, hipStream_t s) {
+          MCCL_CHECK(mccl_reduce_sync_resolved(resolved, (size_t)me * M * es, out, M, dtype, op, &sync, s));
+        };
+        p.standing.one_launch = [=](bool, const mccl_xsync_t& sync, const mccl_offer_t& mine, const void* buffer, void* const* offers,
+                                    const mccl_import_table_t* imports, hipStream_t s) {
+          MCCL_CHECK(mccl_reduce_sync_offers((size_t)me * M * es, out, M, dtype, op, &sync, &mine, buffer, offers, imports, s));
+        };
+      }
       // large inputs are read in place by the peers: rank r reduces slice r of every rank's tensor
       p.share = len * es * (size_t)W >= kZeroCopyMinBytes;
       // (an output inside another rank's slice of the input: nothing is offered, and then every rank stages)

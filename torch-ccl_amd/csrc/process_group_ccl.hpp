@@ -271,9 +271,23 @@ class ProcessGroupCCL : public c10d::Backend {
     size_t fused_count = 0;
     int fused_dtype = 0;
     int fused_op = 0;
-    // An allreduce too large for that launch: fused_ptr / fused_count / fused_dtype / fused_op describe
-    // it for the path that exchanges offers on the device (runStanding).
-    bool standing_ok = false;
+    // Eligible for the path that exchanges where the ranks' buffers are on the device and never meets
+    // on the host (runStanding): what this rank's peers address, and the kernels over the resolved
+    // addresses.  `ok` and `bytes` must come out the same on every rank (sizes all ranks agree on).
+    struct Standing {
+      bool ok = false;
+      void* buffer = nullptr;      // the tensor the peers read (allreduce, reduce_scatter: the input) or write (all_gather: the output)
+      size_t bytes = 0;
+      bool copy_in = false;        // a rank that stages copies its tensor into the staging buffer first ...
+      bool copy_out = false;       // ... and / or the staging buffer back into it afterwards
+      bool force_staged = false;   // this rank's tensors overlap in a way only a staged run handles (its own matter: the peers do not care)
+      double compact_cost = 1.0;   // as Plan::compact_cost: up to which size ONE launch on few compute units wins
+      // the data kernel behind the barrier kernel that resolved the offers into `resolved`
+      std::function<void(const void* resolved, bool staged, const mccl_xsync_t& sync, hipStream_t s)> behind_barrier;
+      // one launch that exchanges the offers itself
+      std::function<void(bool staged, const mccl_xsync_t& sync, const mccl_offer_t& mine, const void* buffer,
+                         void* const* offers, const mccl_import_table_t* imports, hipStream_t s)> one_launch;
+    } standing;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
@@ -466,6 +480,7 @@ class ProcessGroupCCL : public c10d::Backend {
   // where their tensors are on the device and never meet on the host
   bool standing_offers_ = true;
   size_t standing_capacity_ = 0;            // staging of both slots that holds this much on every rank, mapped by every peer
+  size_t standing_max_ = 256u << 20;        // larger buffers meet at the rendezvous (MCCL_PG_STANDING_MAX_BYTES): the fallback needs staging of that size
   mccl_import_table_t* import_table_ = nullptr;  // device: the peers' allocations as this rank has mapped them
   void* resolved_ = nullptr;                // device: where the ranks' tensors of the collective under way are
   std::vector<void*> offer_slots_[2];       // rank r's offer slot, per parity of the collective

@@ -40,7 +40,8 @@ EXPORTS = (
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
-    "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_sync_offers", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
+    "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_sync_offers",
+    "mccl_reduce_sync_resolved", "mccl_reduce_sync_offers", "mccl_fanout_sync_resolved", "mccl_fanout_sync_offers", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
     "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
     "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
@@ -114,6 +115,10 @@ def lib():
     L.mccl_allreduce_sync_resolved.argtypes = [vp, sz, i32, i32, vp, vp]
     L.mccl_import_table_update.argtypes = [vp, vp, i32, vp]
     L.mccl_allreduce_sync_offers.argtypes = [sz, i32, i32, vp, vp, vp, vp, vp, vp]
+    L.mccl_reduce_sync_resolved.argtypes = [vp, sz, vp, sz, i32, i32, vp, vp]
+    L.mccl_reduce_sync_offers.argtypes = [sz, vp, sz, i32, i32, vp, vp, vp, vp, vp, vp]
+    L.mccl_fanout_sync_resolved.argtypes = [vp, vp, sz, sz, i32, vp, vp]
+    L.mccl_fanout_sync_offers.argtypes = [vp, sz, sz, i32, vp, vp, vp, vp, vp, vp]
     L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, ctypes.c_uint, vp]
     L.mccl_allreduce_fused_replayable.argtypes = [vp, vp, sz, i32, i32, vp, vp, sz, sz, vp, i32, i32, ctypes.c_uint64, vp, ctypes.c_uint, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
