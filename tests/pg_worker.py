@@ -1170,6 +1170,58 @@ def standing_offer_cases(pg, rank, world):
         del y
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
+    # reduce_scatter_tensor and all_gather_into_tensor the same way: no rendezvous in steady state, small
+    # and large, in place and not, rank 1 staging for good (its tensors sit in an allocation too large
+    # to share), and the forms whose tensors overlap outside the rank's own slice
+    for dtype, m in ((torch.bfloat16, 300007), (torch.float32, 1 << 20), (torch.float32, 33)):
+        code = TORCH_TO_CODE[dtype]
+        es = torch.empty(0, dtype=dtype).element_size()
+        if rank == 1:
+            huge = torch.empty((2 << 30) + 64, dtype=torch.uint8, device=DEV)
+            x = huge[64:64 + world * m * es].view(dtype)
+            full = huge[(1 << 30):(1 << 30) + world * m * es].view(dtype)
+        else:
+            x = torch.empty(world * m, dtype=dtype, device=DEV)
+            full = torch.empty(world * m, dtype=dtype, device=DEV)
+        out = torch.empty(m, dtype=dtype, device=DEV)
+        for rep in range(4):
+            host = [rank_buffer(world * m, dtype, r, seed=600 + rep) for r in range(world)]
+            want = bits_np(O.reduce_scatter([to_carrier(h) for h in host], code, O.SUM, shard_first=rank, shard_num=1)[0])
+            x.copy_(host[rank])
+            if rep == 2:
+                before = pg._rendezvous_counts()
+            pg._reduce_scatter_base(out, x).wait()
+            assert np.array_equal(bits(out), want), ("reduce_scatter", dtype, m, rep, pg._last_path())
+            x.copy_(host[rank])
+            pg._reduce_scatter_base(x[rank * m:(rank + 1) * m], x).wait()  # in place
+            assert np.array_equal(bits(x[rank * m:(rank + 1) * m]), want), ("reduce_scatter in place", dtype, m, rep)
+            other = (rank + 1) % world
+            x.copy_(host[rank])
+            pg._reduce_scatter_base(x[other * m:(other + 1) * m], x).wait()  # output in a foreign slice: this rank stages
+            assert np.array_equal(bits(x[other * m:(other + 1) * m]), want), ("reduce_scatter into a foreign slice", dtype, m, rep)
+            assert pg._last_path() == "standing offers, this rank staged", pg._last_path()
+            parts = [rank_buffer(m, dtype, r, seed=650 + rep) for r in range(world)]
+            whole = np.concatenate([bits(h) for h in parts])
+            full.zero_()
+            pg._allgather_base(full, parts[rank].to(DEV)).wait()
+            assert np.array_equal(bits(full), whole), ("allgather", dtype, m, rep, pg._last_path())
+            full.zero_()
+            full[rank * m:(rank + 1) * m].copy_(parts[rank])
+            pg._allgather_base(full, full[rank * m:(rank + 1) * m]).wait()  # in place
+            assert np.array_equal(bits(full), whole), ("allgather in place", dtype, m, rep)
+            full.zero_()
+            full[other * m:(other + 1) * m].copy_(parts[rank])
+            pg._allgather_base(full, full[other * m:(other + 1) * m]).wait()  # input in a foreign slice: this rank stages
+            assert np.array_equal(bits(full), whole), ("allgather from a foreign slice", dtype, m, rep)
+        after = pg._rendezvous_counts()
+        assert after[0] == before[0] and after[1] == before[1] + 12, (before, after)
+        large = world * m * es >= (1 << 20)
+        assert pg._last_path() == "standing offers, this rank staged"  # (the foreign-slice form was last)
+        del x, full, out
+        if rank == 1:
+            del huge
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
     # a rank that comes 50 ms late: the others' calls return at once (nobody's host thread waits
     # for anybody), their Works complete when the late rank's kernels have run
     z = torch.full((1 << 20,), float(rank + 1), device=DEV)  # 4 MiB
@@ -1193,6 +1245,29 @@ def standing_offer_cases(pg, rank, world):
     assert call_ms < 5.0, call_ms  # (measured: below 0.1 ms; the late rank itself included)
     if rank != 1:
         assert total_ms > 30.0, total_ms  # the result did wait for the late rank
+    pg.barrier().wait()
+    # the same for reduce_scatter_tensor and all_gather_into_tensor of 8 MiB per rank's buffer
+    inp = torch.full((world << 18,), float(rank + 1), device=DEV)
+    shard = torch.empty(1 << 18, device=DEV)
+    gathered = torch.empty(world << 18, device=DEV)
+    for _ in range(2):
+        pg._reduce_scatter_base(shard, inp).wait()
+        pg._allgather_base(gathered, shard).wait()
+    torch.cuda.synchronize()
+    pg.barrier().wait()
+    if rank == 1:
+        time.sleep(0.05)
+    t0 = time.perf_counter()
+    w1 = pg._reduce_scatter_base(shard, inp)
+    w2 = pg._allgather_base(gathered, shard)
+    call_ms = (time.perf_counter() - t0) * 1e3
+    w1.wait()
+    w2.wait()
+    torch.cuda.synchronize()
+    assert float(gathered.min()) == world * (world + 1) / 2 == float(gathered.max())
+    print("standing offers: rank %d of %d, reduce_scatter_tensor + all_gather_into_tensor with rank 1 50 ms late: both calls %.3f ms" % (
+        rank, world, call_ms), flush=True)
+    assert call_ms < 5.0, call_ms
     pg.barrier().wait()
 
 

@@ -336,6 +336,68 @@ def offers_case(rank, world, queues, barrier):
             capi.check(L.mccl_allreduce_sync_offers(count, TORCH_TO_CODE[dtype], ops[name][0], ctypes.byref(sy), ctypes.byref(offer),
                                                     where.data_ptr(), slots[call & 1], table.data_ptr(), stream))
         pending.append((where.clone(), oracle_reduce_bits(host, ops[name][1]), (str(dtype), count, name, kind, i % 2)))
+    # the shard reduction (reduce_scatter: rank r reduces slice r of every rank's offered input) and the
+    # push (allgather: rank r writes its contribution into slice r of every rank's offered output)
+    # over the same offers, in both forms
+    from helpers import to_carrier
+    for i, (dtype, m, name) in enumerate([(torch.bfloat16, 70001, "SUM"), (torch.float32, 4099, "MAX"), (torch.float16, 1 << 17, "AVG"),
+                                          (torch.int8, 300007, "SUM"), (torch.float64, 1027, "SUM"), (torch.bfloat16, 1 << 19, "SUM")]):
+        es = torch.empty(0, dtype=dtype).element_size()
+        code = TORCH_TO_CODE[dtype]
+        host = [rank_buffer(world * m, dtype, r, seed=950 + i, scale=0.02) for r in range(world)]
+        call += 1
+        kind = (call + rank) % 3
+        off = ((call * 37 + rank * 11) % 64) * es
+        nbytes = world * m * es
+        if kind < 2:
+            where = allocs[kind][off:off + nbytes].view(dtype)
+            offer = capi.Offer(entries[kind], 0, gen_of(rank, kind), off, 0)
+        else:
+            where = stages[call & 1][off:off + nbytes].view(dtype)
+            offer = capi.Offer(capi.OFFER_STAGED, call & 1, 0, off, 0)
+        where.copy_(host[rank])
+        out = torch.zeros(m, dtype=dtype, device=DEV)
+        if i % 2 == 0:
+            capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
+                                                  where.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+            capi.check(L.mccl_reduce_sync_resolved(resolved.data_ptr(), rank * m * es, out.data_ptr(), m, code, ops[name][0], ctypes.byref(sy), stream))
+        else:
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 4 * call + 1, 4 * call + 3, counter.data_ptr(), 5_000_000,
+                            st.data_ptr(), 16, 0)
+            capi.check(L.mccl_reduce_sync_offers(rank * m * es, out.data_ptr(), m, code, ops[name][0], ctypes.byref(sy), ctypes.byref(offer),
+                                                 where.data_ptr(), slots[call & 1], table.data_ptr(), stream))
+        want = O.reduce_scatter([to_carrier(h) for h in host], code, ops[name][1], shard_first=rank, shard_num=1)[0]
+        pending.append((out, want.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[want.dtype.itemsize]), ("reduce_scatter", str(dtype), m, name, kind, i % 2)))
+        # the push: what is offered is the OUTPUT (world * nb bytes), rank r's contribution is nb bytes
+        nb = m * es + (i % 3)  # not always a whole number of vectors or elements: bytes
+        parts = [rank_buffer(nb, torch.uint8, r, seed=970 + i) for r in range(world)]
+        call += 1
+        kind = (call + rank) % 3
+        off = (call * 5 + rank) % 32
+        if kind < 2:
+            dest = allocs[kind][off:off + world * nb]
+            offer = capi.Offer(entries[kind], 0, gen_of(rank, kind), off, 0)
+        else:
+            dest = stages[call & 1][off:off + world * nb]
+            offer = capi.Offer(capi.OFFER_STAGED, call & 1, 0, off, 0)
+        dest.zero_()
+        in_place = i % 3 == 1  # the contribution already sits in this rank's slice of its own output
+        src = parts[rank].to(DEV)
+        if in_place:
+            dest[rank * nb:(rank + 1) * nb].copy_(src)
+            src = dest[rank * nb:(rank + 1) * nb]
+        if i % 2 == 1:
+            capi.check(L.mccl_rank_barrier_offers(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), ctypes.byref(offer),
+                                                  dest.data_ptr(), slots[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+            capi.check(L.mccl_fanout_sync_resolved(src.data_ptr(), resolved.data_ptr(), rank * nb, nb, int(in_place), ctypes.byref(sy), stream))
+        else:
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 4 * call + 1, 4 * call + 3, counter.data_ptr(), 5_000_000,
+                            st.data_ptr(), 16, 0)
+            capi.check(L.mccl_fanout_sync_offers(src.data_ptr(), rank * nb, nb, int(in_place), ctypes.byref(sy), ctypes.byref(offer),
+                                                 dest.data_ptr(), slots[call & 1], table.data_ptr(), stream))
+        pending.append((dest.clone(), np.concatenate([bits(p) for p in parts]), ("allgather", nb, kind, in_place, i % 2)))
     torch.cuda.synchronize()
     assert st.tolist() == [0, 0], st.tolist()
     for got, want, what in pending:
