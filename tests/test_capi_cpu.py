@@ -116,6 +116,70 @@ def test_one_launch_collectives_reject_partial_overlap(mccl):
     assert b"tensors 0 and 1 partially overlap" in L.mccl_last_error()
 
 
+def test_offer_entry_points_reject_bad_arguments_without_a_device(mccl):
+    """mccl_rank_barrier_offers, mccl_import_table_update, the `_resolved` and `_offers` forms and
+    mccl_allreduce_fused_replayable: every refusal that depends on arguments only."""
+    from torch_ccl_amd import capi
+    L = capi.lib()
+    err = lambda: L.mccl_last_error().decode()
+    vp = ctypes.c_void_p
+    two = capi.ptr_table([0x10000, 0x20000])
+    nine = capi.ptr_table([0x10000 + 64 * i for i in range(9)])
+    offer = capi.Offer(3, 0, 7, 0, 0)
+    tab, res = vp(0x40000), vp(0x50000)
+    assert L.mccl_rank_barrier_offers(nine, 9, 0, 1, 0, None, ctypes.byref(offer), vp(0x1000), nine, tab, res, None) == -3 and "1 to 8 ranks" in err()
+    assert L.mccl_rank_barrier_offers(two, 2, 2, 1, 0, None, ctypes.byref(offer), vp(0x1000), two, tab, res, None) == -1 and "rank 2" in err()
+    assert L.mccl_rank_barrier_offers(two, 2, 0, 1, 0, None, None, vp(0x1000), two, tab, res, None) == -1 and "null" in err()
+    assert L.mccl_rank_barrier_offers(two, 2, 0, 1, 0, None, ctypes.byref(offer), vp(0x1000), two, vp(0x40004), res, None) == -1 and "8-byte" in err()
+    assert L.mccl_rank_barrier_offers(two, 2, 0, 1, 0, None, ctypes.byref(offer), vp(0x1000), capi.ptr_table([0x10000, 0x20004]), tab, res, None) == -1
+    assert "offer pointer 1" in err()
+    bad = capi.Offer(32, 0, 7, 0, 0)
+    assert L.mccl_rank_barrier_offers(two, 2, 0, 1, 0, None, ctypes.byref(bad), vp(0x1000), two, tab, res, None) == -1 and "entry 32" in err()
+    # table updates
+    ups = (capi.ImportUpdate * 9)()
+    assert L.mccl_import_table_update(tab, ups, 0, None) == 0
+    assert L.mccl_import_table_update(tab, ups, 9, None) == -1 and "at most 8" in err()
+    ups[0] = capi.ImportUpdate(8, 0, 0, 0, 0x1000, 1)
+    assert L.mccl_import_table_update(tab, ups, 1, None) == -1 and "rank 8" in err()
+    ups[0] = capi.ImportUpdate(1, 40, 0, 0, 0x1000, 1)
+    assert L.mccl_import_table_update(tab, ups, 1, None) == -1 and "entry 40" in err()
+    ups[0] = capi.ImportUpdate(1, 5, 0, 0, 0x1000, 1)
+    ups[1] = capi.ImportUpdate(1, 5, 0, 0, 0x2000, 2)
+    assert L.mccl_import_table_update(tab, ups, 2, None) == -1 and "same entry" in err()
+    ups[0] = capi.ImportUpdate(1, capi.OFFER_STAGED, 0, 0, 0x1000, 0)
+    ups[1] = capi.ImportUpdate(1, capi.OFFER_STAGED, 1, 0, 0x2000, 0)  # the two staging slots of one rank: different entries
+    assert L.mccl_import_table_update(None, ups, 2, None) == -1 and "null" in err()
+    # the forms behind a barrier want no opening epoch and a closing one; the one-launch forms want all three
+    words = capi.ptr_table([0x60000, 0x60040])
+    behind = capi.XSync(ctypes.cast(words, vp), 2, 0, 0, 7, vp(0x70000), 0, None, 0, 0)
+    opening = capi.XSync(ctypes.cast(words, vp), 2, 0, 5, 7, vp(0x70000), 0, None, 0, 0)
+    one = capi.XSync(ctypes.cast(words, vp), 2, 0, 5, 7, vp(0x70000), 0, None, 16, 0)
+    assert L.mccl_allreduce_sync_resolved(res, 64, capi.F32, capi.SUM, ctypes.byref(opening), None) == -1 and "behind a barrier" in err()
+    assert L.mccl_allreduce_sync_resolved(None, 64, capi.F32, capi.SUM, ctypes.byref(behind), None) == -1 and "null" in err()
+    assert L.mccl_reduce_sync_resolved(res, 0, vp(0x80000), 64, capi.F32, capi.SUM, ctypes.byref(opening), None) == -1 and "behind a barrier" in err()
+    assert L.mccl_reduce_sync_resolved(res, 2, vp(0x80000), 64, capi.F32, capi.SUM, ctypes.byref(behind), None) == -1 and "offset" in err()
+    assert L.mccl_fanout_sync_resolved(vp(0x90000), res, 0, 64, 0, ctypes.byref(opening), None) == -1 and "behind a barrier" in err()
+    assert L.mccl_allreduce_sync_offers(64, capi.F32, capi.SUM, ctypes.byref(opening), ctypes.byref(offer), vp(0x1000), two, tab, None) == -1
+    assert "max_compute_units" in err()
+    assert L.mccl_reduce_sync_offers(0, vp(0x80000), 64, capi.F32, capi.SUM, ctypes.byref(behind), ctypes.byref(offer), vp(0x1000), two, tab, None) == -1
+    assert "max_compute_units" in err()
+    assert L.mccl_fanout_sync_offers(vp(0x90000), 0, 64, 0, ctypes.byref(one), ctypes.byref(bad), vp(0x1000), two, tab, None) == -1 and "entry 32" in err()
+    assert L.mccl_reduce_sync_offers(0, vp(0x80000), 64, capi.I32, capi.AVG, ctypes.byref(one), ctypes.byref(offer), vp(0x1000), two, tab, None) == -3
+    # the small allreduce with its epoch on the device
+    stage = capi.ptr_table([0x100000, 0x300000])
+    tf = capi.ptr_table([0x500000, 0x510000])
+    call = lambda state, ss, fs, flags, count=1024: L.mccl_allreduce_fused_replayable(
+        vp(0x600000), vp(0x600000), count, capi.F32, capi.SUM, stage, tf, ss, fs, state, 2, 0, 0, None, 0, flags, None)
+    assert call(None, 1 << 20, 8192, 0) == -1 and "state is null" in err()
+    assert call(vp(0x700020), 1 << 20, 8192, 0) == -1 and "64-byte" in err()
+    assert call(vp(0x700000), (1 << 20) + 8, 8192, 0) == -1 and "multiple of 16" in err()
+    assert call(vp(0x700000), 1 << 20, 8190, 0) == -1 and "multiple of 4" in err()
+    assert call(vp(0x700000), 2048, 8192, 0) == -1 and "does not fit" in err()
+    assert call(vp(0x700000), 1 << 20, 8192, 4) == -1 and "unknown flags" in err()
+    assert call(vp(0x700000), 1 << 20, 8192, capi.FUSED_WORK_ONLY | capi.FUSED_SYNC_ONLY) == -1 and "exclude each other" in err()
+    assert call(vp(0x700000), 1 << 20, 8192, 0, count=0) == 0  # empty message: no launch
+
+
 def test_pack_and_unpack_reject_a_null_flat_buffer(mccl):
     from torch_ccl_amd import capi
     L = capi.lib()
