@@ -1110,6 +1110,19 @@ def standing_offer_cases(pg, rank, world):
     assert after[0] == before[0] and after[1] == before[1] + 8, (before, after)  # no rendezvous, eight that only enqueued
     assert all(p.startswith("standing offers") for p in paths), paths
     assert paths[-1] == "standing offers, peers read in place", paths  # (the first calls are staged until every peer has mapped the allocation)
+    # a message larger than any before: the ranks meet once to enlarge their staging buffers, and since
+    # they meet they map each other's new tensors there and then -- in place from the first call on
+    count = (10 << 20) + 3  # 40 MiB of int32
+    big = torch.empty(count, dtype=torch.int32, device=DEV)
+    for i in range(2):
+        host = [rank_buffer(count, torch.int32, r, seed=520 + i) for r in range(world)]
+        big.copy_(host[rank])
+        pg.allreduce([big], c10d.AllreduceOptions()).wait()
+        assert pg._last_path() == "standing offers, peers read in place", (i, pg._last_path())
+        check(big, host, ("larger than any before", i))
+    del big
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
     # a new allocation per call (each tensor fills a segment of its own), all alive at once, more of
     # them than the table of announced allocations holds: entries are reused, results stay right
     keep = []

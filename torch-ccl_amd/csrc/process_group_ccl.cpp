@@ -1039,12 +1039,17 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
   const Plan::Standing& st = plan.standing;
   const size_t bytes = st.bytes;
   const uint64_t epoch = 4 * seq;
-  if (bytes > standing_capacity_) growStandingCapacity(bytes);
-  scanPeerExports(seq);
   uint64_t off = 0;
   // (small buffers live in the allocator's 2 MiB segments, many of them: announcing those would turn
   // the table of allocations over all the time, and copying them costs next to nothing)
   const int entry = (st.force_staged || bytes < kZeroCopyMinBytes) ? -1 : exportRange(st.buffer, bytes, &off);
+  // A message larger than the staging every rank keeps mapped: the host threads meet (all at this
+  // collective: the sizes agree) -- and since they do, they also look at what everybody has just
+  // announced before anybody decides, so that the first collective of a new size already runs in place.
+  const bool grow = bytes > standing_capacity_;
+  if (grow) growStandingCapacity(bytes);
+  scanPeerExports(seq);
+  if (grow) hostBarrier();
   const uint64_t gen = entry >= 0 ? ctl_->slot[rank_].exports[entry].gen.load(std::memory_order_acquire) : 0;
   const bool in_place = entry >= 0 && allAcknowledged(entry, gen, seq);
   mccl_offer_t mine{};
