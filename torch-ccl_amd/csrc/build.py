@@ -2,8 +2,10 @@
 
   libmi355ccl.so   HIP kernels + C ABI (include/mccl.h); depends on the HIP runtime only.
   libmcclbench.so  HIP-event timing loops around that ABI (bench/mccl_bench.h; lands in bench/).
-  _C.*.so          the c10d backend (process_group_ccl.cpp) and its Python module; host code
-                   only, links torch's c10d and libmi355ccl.so.
+  _C.*.so          the c10d backend (process_group_ccl.cpp: the group and how a collective runs;
+                   pg_sharing.cpp: staging, shared allocations, standing offers; pg_collectives.cpp;
+                   pg_p2p.cpp) and its Python module; host code only, links torch's c10d and
+                   libmi355ccl.so.
 
 Usage: python torch-ccl_amd/csrc/build.py [--force]
 Outputs land in torch-ccl_amd/torch_ccl_amd/lib/.
@@ -100,8 +102,8 @@ def build_bench(force=False):
     return BENCH_LIB
 
 
-BACKEND_SRCS = [os.path.join(HERE, "process_group_ccl.cpp"), os.path.join(HERE, "python_module.cpp")]
-BACKEND_HDRS = [os.path.join(HERE, "process_group_ccl.hpp"), os.path.join(INCLUDE, "mccl.h")]
+BACKEND_SRCS = [os.path.join(HERE, f) for f in ("process_group_ccl.cpp", "pg_sharing.cpp", "pg_collectives.cpp", "pg_p2p.cpp", "python_module.cpp")]
+BACKEND_HDRS = [os.path.join(HERE, "process_group_ccl.hpp"), os.path.join(HERE, "pg_internal.hpp"), os.path.join(INCLUDE, "mccl.h")]
 
 
 def backend_lib_path():

@@ -47,7 +47,7 @@
 
 namespace mccl_pg {
 
-struct Control;  // shared-memory control block (process_group_ccl.cpp)
+struct Control;  // shared-memory control block (pg_internal.hpp)
 
 // What the Works of a group share with it and may outlive it with: recycled events and the
 // group's health.  `status` is pinned host memory the device-side waits write when they give up:
@@ -318,7 +318,7 @@ class ProcessGroupCCL : public c10d::Backend {
   void runHostSynced(Plan& plan, hipStream_t s, int slot);
   void runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void deviceBarrier(uint64_t epoch, hipStream_t s);
-  // standing offers (process_group_ccl.cpp: "standing offers")
+  // standing offers (pg_sharing.cpp)
   bool standingFits(const Plan& plan) const;
   void runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void growStandingCapacity(size_t bytes);
