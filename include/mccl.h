@@ -208,7 +208,9 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
  * table of the peers' allocations as it has mapped them (device memory of this rank, filled by the
  * host in stream order before the launch): entry e of rank r at generation g is at
  * imports->base[r][e] when imports->generation[r][e] == g; entry MCCL_OFFER_STAGED means rank r's
- * staging buffer `slot`, imports->staging[r][slot].  The address of every rank's buffer in this
+ * staging buffer `slot`, imports->staging[r][slot] (slots 0 and 1: the rank's two staging buffers,
+ * the same for every reader; MCCL_OFFER_SLOT_OUTBOX: the buffer rank r keeps for THIS reader
+ * alone, see mccl_rank_barrier_offers_each).  The address of every rank's buffer in this
  * rank's address space -- base + offset; my_buffer for this rank itself -- goes to resolved[0..n),
  * n 64-bit words of this rank's device memory, for the kernels that follow on the stream
  * (mccl_allreduce_sync_resolved).  An offer that this rank has not mapped leaves a null pointer
@@ -218,22 +220,45 @@ int mccl_rank_barrier(void* const* flags, int n, int rank, uint64_t epoch, uint6
 #define MCCL_OFFER_RANKS 8
 #define MCCL_OFFER_ENTRIES 32
 #define MCCL_OFFER_STAGED 0xffffffffu
+#define MCCL_OFFER_SLOTS 4
+#define MCCL_OFFER_SLOT_OUTBOX 2u
 #define MCCL_STATUS_UNMAPPED 0xfffffffeu
+#define MCCL_STATUS_MISMATCH 0xfffffffdu
 typedef struct mccl_offer {
   uint32_t entry;      /* index in the owner's table of announced allocations, or MCCL_OFFER_STAGED */
-  uint32_t slot;       /* with MCCL_OFFER_STAGED: which of the owner's two staging buffers */
+  uint32_t slot;       /* with MCCL_OFFER_STAGED: which of the owner's staging buffers (< MCCL_OFFER_SLOTS) */
   uint64_t generation; /* of the entry: changes when the owner reuses it for another allocation */
   uint64_t offset;     /* bytes from the start of the allocation (or of the staging buffer) */
-  uint64_t reserved;
+  uint64_t bytes;      /* mccl_rank_barrier_offers_each: length of the piece, which the reader checks; else 0 */
 } mccl_offer_t;
 typedef struct mccl_import_table {
   uint64_t base[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES];
   uint64_t generation[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES];
-  uint64_t staging[MCCL_OFFER_RANKS][2];
+  uint64_t staging[MCCL_OFFER_RANKS][MCCL_OFFER_SLOTS];
 } mccl_import_table_t;
 int mccl_rank_barrier_offers(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us, void* status,
                              const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
                              const mccl_import_table_t* imports, void* resolved, void* stream);
+
+/*
+ * The same for collectives in which a rank hands every peer a DIFFERENT piece (alltoall(v):
+ * src/gpu/dpcpp_ccl.cpp:1371-1466): a rank publishes a row of n offers, mine[k] = where the piece
+ * for rank k is and how long it is (mine[k].bytes), and reads the column addressed to it:
+ * offers[r] is rank r's row (n x 32 bytes of device memory the peers can reach), of which this rank
+ * reads entry `rank`.  expect_bytes[r] is what this rank expects from rank r: a piece of another
+ * length is reported (status[0] = 1 + r, status[1] = MCCL_STATUS_MISMATCH) and resolves to null -- the
+ * counts of an alltoallv are the callers' to keep consistent (outSplit_d[r] == inSplit_r[d]), and
+ * nobody else can check them without a rendezvous.  A piece of length 0 resolves to null without
+ * being looked up.  resolved[r] = where rank r's piece for this rank starts, for
+ * mccl_copy_segments_sync_resolved behind it on the stream; resolved[rank] = my_source, this rank's
+ * own piece.  Pieces a rank cannot offer in place it copies into a buffer it keeps for that one
+ * reader (MCCL_OFFER_STAGED, slot MCCL_OFFER_SLOT_OUTBOX: imports->staging[r][2] is rank r's outbox
+ * for this rank): only the two of them know the length of the piece, so only they can agree, without
+ * anybody else, on when that buffer has to grow.
+ */
+int mccl_rank_barrier_offers_each(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us, void* status,
+                                  const mccl_offer_t* mine, const uint64_t* expect_bytes, const void* my_source,
+                                  void* const* offers, const mccl_import_table_t* imports, void* resolved, void* stream);
 
 /*
  * Stream-ordered update of an import table in device memory: entry `entry` of rank `rank` is now
@@ -245,7 +270,7 @@ int mccl_rank_barrier_offers(void* const* flags, int n, int rank, uint64_t epoch
 #define MCCL_IMPORT_UPDATES 8
 typedef struct mccl_import_update {
   uint32_t rank;
-  uint32_t entry;       /* < MCCL_OFFER_ENTRIES: an allocation; MCCL_OFFER_STAGED: a staging buffer, `slot` says which */
+  uint32_t entry;       /* < MCCL_OFFER_ENTRIES: an allocation; MCCL_OFFER_STAGED: a staging buffer, `slot` (< MCCL_OFFER_SLOTS) says which */
   uint32_t slot;
   uint32_t reserved;
   uint64_t base;
@@ -432,6 +457,18 @@ int mccl_fanout_sync_resolved(const void* src, const void* resolved, size_t dst_
 int mccl_fanout_sync_offers(const void* src, size_t dst_offset, size_t bytes, int skip_own, const mccl_xsync_t* sync,
                             const mccl_offer_t* mine, const void* my_buffer, void* const* offers,
                             const mccl_import_table_t* imports, void* stream);
+
+/*
+ * mccl_copy_segments_sync whose sources come from the table a barrier with offers has resolved
+ * (behind it on the stream: ready_epoch 0, done_epoch set): segment i is read from
+ * resolved[src_rank[i]] + (size_t)segs[i].src -- segs[i].src is a byte offset there -- or, with
+ * src_rank[i] < 0, from the address segs[i].src as it stands.  A segment whose table entry is null
+ * (the barrier has reported why) is skipped.  This rank's share of an alltoall(v) as pulls
+ * (ccl::alltoallv at src/gpu/dpcpp_ccl.cpp:1447-1455), with nothing about the peers' buffers known
+ * on the host.
+ */
+int mccl_copy_segments_sync_resolved(const mccl_segment_t* segs, const int* src_rank, int nseg, const void* resolved,
+                                     unsigned flags, const mccl_xsync_t* sync, void* stream);
 
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */

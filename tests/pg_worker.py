@@ -550,14 +550,14 @@ def large_message_case(pg, rank, world):
 
 def missing_rank_case(pg, rank, world):
     """Rank 1 never joins the second collective: the others must get an error, not hang.  (An
-    all_to_all_single of 2 MiB per rank: a collective whose host threads meet first in every mode
-    -- its split tables are published per call -- so the call itself raises.)"""
+    all_gather into a list of tensors, 2 MiB per rank: a collective whose host threads meet first in
+    every mode -- where its output tensors are is published per call -- so the call itself raises.)"""
     t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
     try:
-        pg.alltoall_base(torch.empty(world << 17, device=DEV), torch.ones(world << 17, device=DEV), [], []).wait()
+        pg.allgather([[torch.empty(1 << 19, device=DEV) for _ in range(world)]], [t]).wait()
         raise AssertionError("collective with a missing rank returned")
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
@@ -1284,6 +1284,121 @@ def standing_offer_cases(pg, rank, world):
     pg.barrier().wait()
 
 
+def standing_alltoall_cases(pg, rank, world):
+    """all_to_all_single / all_to_all between rank processes without a rendezvous of the host threads: the
+    ranks' pieces are offered on the device, pair by pair in place or through the outbox a rank keeps
+    for that one peer.  Every result is the index map's (oracle), byte for byte."""
+    import time
+    from helpers import bits, rank_buffer, to_carrier
+    from oracle import oracle as O
+
+    def a2a(S, hidden, seed, dtype=torch.bfloat16, inp=None, out=None, overlapping=False):
+        es = torch.empty(0, dtype=dtype).element_size()
+        host = [rank_buffer(int(S[r].sum()) * hidden, dtype, r, seed=seed).view(int(S[r].sum()), hidden) for r in range(world)]
+        if inp is None:
+            inp = torch.empty(int(S[rank].sum()), hidden, dtype=dtype, device=DEV)
+        if out is None:
+            out = torch.empty(int(S[:, rank].sum()), hidden, dtype=dtype, device=DEV)
+        if not overlapping:
+            out.zero_()
+        inp.copy_(host[rank])
+        pg.alltoall_base(out, inp, S[:, rank].tolist(), S[rank].tolist()).wait()
+        want = O.alltoallv([to_carrier(h) for h in host], S, hidden * es)[rank]
+        assert np.array_equal(out.cpu().view(torch.uint8).numpy().reshape(-1), want), ("alltoallv", seed, pg._last_path())
+        if not overlapping:
+            assert np.array_equal(bits(inp.view(-1)), bits(host[rank].view(-1))), ("alltoallv changed its input", seed)
+        return inp, out
+
+    rng = np.random.default_rng(4321)
+    hidden = 512
+    # the same tensors again and again (1 KiB rows, up to 600 per piece): after the first calls every piece is
+    # read in place and nobody waits for anybody
+    S = rng.integers(0, 600, size=(world, world))
+    S[0, world - 1] = 0
+    S[world - 1, 0] = 0
+    inp = out = None
+    for i in range(8):
+        if i == 3:
+            torch.cuda.synchronize()
+            before = pg._rendezvous_counts()
+        inp, out = a2a(S, hidden, 700 + i, inp=inp, out=out)
+    after = pg._rendezvous_counts()
+    assert after[0] == before[0] and after[2] == before[2] and after[1] == before[1] + 5, (before, after)
+    if int(S[rank].sum()) * hidden * 2 >= (1 << 20):
+        sent = sum(1 for d in range(world) if d != rank and S[rank][d])
+        assert pg._last_path() == "standing offers, %d pieces read in place, 0 through outboxes" % sent, pg._last_path()
+    # new tensors per call, pieces that grow from call to call (each growth: the pair meets, nobody else)
+    for i, top in enumerate((40, 700, 3000, 3000, 300, 9000)):
+        S = rng.integers(0, top, size=(world, world))
+        S[i % world, (i + 1) % world] = top  # (one pair grows for sure)
+        a2a(S, hidden, 720 + i)
+    # rows of odd widths and element sizes, empty pieces, a rank that sends nothing, one that gets nothing
+    for i, (dtype, hid) in enumerate(((torch.uint8, 333), (torch.float64, 17), (torch.float32, 1), (torch.int16, 4099))):
+        S = rng.integers(0, 400, size=(world, world))
+        S[rng.integers(0, world)] = 0
+        S[:, rng.integers(0, world)] = 0
+        a2a(S, hid, 740 + i, dtype=dtype)
+    # input and output in one tensor, overlapping: every piece is copied out of the way first
+    S = np.full((world, world), 200)
+    whole = torch.empty(world * 200 + 100, hidden, dtype=torch.bfloat16, device=DEV)
+    for i in range(2):
+        a2a(S, hidden, 760 + i, inp=whole[:world * 200], out=whole[100:100 + world * 200], overlapping=True)
+        assert pg._last_path().endswith("0 pieces read in place, %d through outboxes" % (world - 1)), pg._last_path()
+    # the list form: pieces in tensors of their own (small ones through outboxes, large ones in place once mapped)
+    for i in range(3):
+        sizes = [[(37 + 11 * r + 5 * d) * (1 if (r + d) % 3 else 9000) for d in range(world)] for r in range(world)]
+        sizes[0][world - 1] = 0
+        host = [[rank_buffer(sizes[r][d], torch.float32, r * world + d, seed=780 + i) for d in range(world)] for r in range(world)]
+        ins = [h.to(DEV) for h in host[rank]]
+        outs = [torch.zeros(sizes[r][rank], device=DEV) for r in range(world)]
+        pg.alltoall(outs, ins).wait()
+        for r in range(world):
+            assert np.array_equal(bits(outs[r]), bits(host[r][rank])), ("alltoall list", i, r, pg._last_path())
+    # a rank that comes 50 ms late: the others' calls return at once
+    S = rng.integers(100, 600, size=(world, world))
+    inp = out = None
+    for i in range(3):
+        inp, out = a2a(S, hidden, 800 + i, inp=inp, out=out)
+    torch.cuda.synchronize()
+    pg.barrier().wait()
+    if rank == 1:
+        time.sleep(0.05)
+    t0 = time.perf_counter()
+    w = pg.alltoall_base(out, inp, S[:, rank].tolist(), S[rank].tolist())
+    call_ms = (time.perf_counter() - t0) * 1e3
+    w.wait()
+    torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - t0) * 1e3
+    print("standing offers: rank %d of %d, all_to_all_single with rank 1 50 ms late: call %.3f ms, call + synchronize %.3f ms" % (
+        rank, world, call_ms, total_ms), flush=True)
+    assert call_ms < 5.0, call_ms
+    if rank != 1:
+        assert total_ms > 30.0, total_ms
+    pg.barrier().wait()
+
+
+def standing_alltoall_big_case(pg, rank, world):
+    """Pieces larger than any outbox (the limit shrunk by MCCL_PG_STANDING_MAX_BYTES) are read in place
+    always: the receiver waits for the sender to enter the collective, and for nobody else."""
+    from helpers import rank_buffer, to_carrier
+    from oracle import oracle as O
+    rng = np.random.default_rng(99)
+    hidden = 1024
+    for i in range(4):
+        S = rng.integers(0, 200, size=(world, world))
+        S[0, 1] = 3000 + i  # 3 MiB and more at one byte per element: above the 2 MiB limit of this run
+        S[1, 0] = 0 if i % 2 else 2500
+        host = [rank_buffer(int(S[r].sum()) * hidden, torch.uint8, r, seed=900 + i).view(-1, hidden) for r in range(world)]
+        out = torch.zeros(int(S[:, rank].sum()), hidden, dtype=torch.uint8, device=DEV)
+        before = pg._rendezvous_counts()
+        pg.alltoall_base(out, host[rank].to(DEV), S[:, rank].tolist(), S[rank].tolist()).wait()
+        after = pg._rendezvous_counts()
+        assert after[0] == before[0], (before, after)
+        want = O.alltoallv([to_carrier(h) for h in host], S, hidden)[rank]
+        assert np.array_equal(out.cpu().numpy().reshape(-1), want), ("alltoallv with an oversized piece", i, pg._last_path())
+    pg.barrier().wait()
+
+
 def graph_capture_case(rank, world):
     """A decode loop from a HIP graph: every rank records K dist.all_reduce of the 256 KiB bf16
     message with a small kernel of the caller's between them, then replays the graph with fresh
@@ -1510,6 +1625,10 @@ def run_rank(rank, world, store_path, mode):
         late_peer_case(pg, rank, world)
     elif mode == "standing":
         standing_offer_cases(pg, rank, world)
+    elif mode == "standing_alltoall":
+        standing_alltoall_cases(pg, rank, world)
+    elif mode == "standing_big":
+        standing_alltoall_big_case(pg, rank, world)
     else:
         raise ValueError(mode)
     torch.cuda.synchronize()

@@ -278,14 +278,18 @@ def offers_case(rank, world, queues, barrier):
     BUF = 10 << 20
     allocs = [torch.zeros(BUF, dtype=torch.uint8, device=DEV) for _ in range(2)]   # entries 3 and 17
     stages = [torch.zeros(BUF, dtype=torch.uint8, device=DEV) for _ in range(2)]
-    ctl = torch.zeros(64, dtype=torch.int64, device=DEV)  # [0]: the flag word, [8..12) and [16..20): the two offer slots
+    # [0]: the flag word, [8..12) and [16..20): the two offer slots, [64..96) and [96..128): the two rows of offers (alltoall)
+    ctl = torch.zeros(128, dtype=torch.int64, device=DEV)
+    OUTBOX = 1 << 20
+    outbox = torch.zeros(world * OUTBOX, dtype=torch.uint8, device=DEV)  # piece d of this rank's, when it is not offered in place
     counter = torch.zeros(1024, dtype=torch.int32, device=DEV)
     table = torch.zeros(ctypes.sizeof(capi.ImportTable) // 8, dtype=torch.int64, device=DEV)
     resolved = torch.zeros(8, dtype=torch.int64, device=DEV)
     torch.cuda.synchronize()
-    shared = _exchange(rank, world, queues, barrier, allocs + stages + [ctl])
+    shared = _exchange(rank, world, queues, barrier, allocs + stages + [ctl, outbox])
     flags = capi.ptr_table([shared[r][4].data_ptr() for r in range(world)])
     slots = [capi.ptr_table([shared[r][4].data_ptr() + 8 * (8 + 8 * sl) for r in range(world)]) for sl in range(2)]
+    rows = [capi.ptr_table([shared[r][4].data_ptr() + 8 * (64 + 32 * sl) for r in range(world)]) for sl in range(2)]
     st = _status()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     entries = (3, 17)
@@ -301,6 +305,7 @@ def offers_case(rank, world, queues, barrier):
         for which in range(2):
             ups.append(capi.ImportUpdate(r, entries[which], 0, 0, shared[r][which].data_ptr(), gen_of(r, which)))
             ups.append(capi.ImportUpdate(r, capi.OFFER_STAGED, which, 0, shared[r][2 + which].data_ptr(), 0))
+        ups.append(capi.ImportUpdate(r, capi.OFFER_STAGED, capi.OFFER_SLOT_OUTBOX, 0, shared[r][5].data_ptr() + rank * OUTBOX, 0))  # rank r's outbox for this rank
     for at in range(0, len(ups), 8):
         chunk = (capi.ImportUpdate * len(ups[at:at + 8]))(*ups[at:at + 8])
         capi.check(L.mccl_import_table_update(table.data_ptr(), chunk, len(ups[at:at + 8]), stream))
@@ -403,6 +408,66 @@ def offers_case(rank, world, queues, barrier):
     for got, want, what in pending:
         assert_bits_equal(bits(got), want, what)
     assert int(counter.abs().sum()) == 0
+    # alltoall(v): every rank publishes a row of offers -- piece d in place (somewhere in one of its
+    # allocations) or in its outbox for rank d -- and pulls the column addressed to it
+    def alltoall_round(call, seed, break_length=False):
+        rng = np.random.default_rng(seed)
+        S = rng.integers(0, 3, size=(world, world)) * rng.integers(1, 200000, size=(world, world)) + rng.integers(0, 2, size=(world, world)) * 13
+        S[rng.integers(0, world)][rng.integers(0, world)] = 0
+        pieces = [[rng.integers(0, 256, size=int(S[r][d]), dtype=np.uint8) for d in range(world)] for r in range(world)]
+        displ = np.concatenate([[0], np.cumsum(S[rank])[:-1]])
+        total = int(S[rank].sum())
+        kind = (call + rank) % 2
+        off = (call * 7 + rank * 3) % 61
+        image = allocs[kind][off:off + total]
+        if total:
+            image.copy_(torch.from_numpy(np.concatenate(pieces[rank])).to(DEV))
+        mine = (capi.Offer * world)()
+        for d in range(world):
+            nb = int(S[rank][d])
+            told = nb + 16 if (break_length and rank == 0 and d == 1) else nb
+            if (call + rank + d) % 3 == 0:  # through the outbox for rank d
+                outbox[d * OUTBOX:d * OUTBOX + nb].copy_(image[int(displ[d]):int(displ[d]) + nb])
+                mine[d] = capi.Offer(capi.OFFER_STAGED, capi.OFFER_SLOT_OUTBOX, 0, 0, told)
+            else:
+                mine[d] = capi.Offer(entries[kind], 0, gen_of(rank, kind), off + int(displ[d]), told)
+        expect = (ctypes.c_uint64 * world)(*[int(S[r][rank]) for r in range(world)])
+        odispl = np.concatenate([[0], np.cumsum(S[:, rank])[:-1]])
+        out = torch.full((int(S[:, rank].sum()) + 64,), 0xee, dtype=torch.uint8, device=DEV)
+        capi.check(L.mccl_rank_barrier_offers_each(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), mine, expect,
+                                                    image.data_ptr() + int(displ[rank]), rows[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+        segs = (capi.Segment * world)(*[capi.Segment(0, out.data_ptr() + int(odispl[r]), int(S[r][rank])) for r in range(world)])
+        src_rank = (ctypes.c_int * world)(*range(world))
+        sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+        capi.check(L.mccl_copy_segments_sync_resolved(segs, src_rank, world, resolved.data_ptr(), 0, ctypes.byref(sy), stream))
+        want = np.concatenate([pieces[r][rank] for r in range(world)] + [np.full(64, 0xee, dtype=np.uint8)])
+        return out, want, S
+
+    pending = []
+    for i in range(6):
+        call += 1
+        out, want, S = alltoall_round(call, seed=1000 + i)
+        pending.append((out, want, ("alltoall", i, S.tolist())))
+    torch.cuda.synchronize()
+    assert st.tolist() == [0, 0], st.tolist()
+    for got, want, what in pending:
+        assert_bits_equal(bits(got), want, what)
+    assert int(counter.abs().sum()) == 0
+    if world > 1:
+        # rank 0 tells rank 1 a length that rank 1 does not expect: rank 1 reports it and leaves that piece alone
+        barrier.wait(timeout=120)
+        call += 1
+        out, want, S = alltoall_round(call, seed=1100, break_length=True)
+        torch.cuda.synchronize()
+        if rank == 1 and S[0][1] + 16 != S[0][1]:
+            assert st.tolist()[0] == 1 and (st.tolist()[1] & 0xffffffff) == capi.STATUS_MISMATCH, st.tolist()
+            lo = int(S[:0, 1].sum())
+            want[lo:lo + int(S[0][1])] = 0xee
+            st.zero_()
+        else:
+            assert st.tolist() == [0, 0], st.tolist()
+        assert_bits_equal(bits(out), want, ("alltoall with a wrong length", rank))
+        barrier.wait(timeout=120)
     # rank 0 offers an allocation at a generation nobody has mapped: every other rank reports it
     # and leaves all tensors alone, and every launch still ends
     barrier.wait(timeout=120)

@@ -117,7 +117,7 @@ def test_one_launch_collectives_reject_partial_overlap(mccl):
 
 
 def test_offer_entry_points_reject_bad_arguments_without_a_device(mccl):
-    """mccl_rank_barrier_offers, mccl_import_table_update, the `_resolved` and `_offers` forms and
+    """mccl_rank_barrier_offers(_each), mccl_import_table_update, the `_resolved` and `_offers` forms and
     mccl_allreduce_fused_replayable: every refusal that depends on arguments only."""
     from torch_ccl_amd import capi
     L = capi.lib()
@@ -165,6 +165,36 @@ def test_offer_entry_points_reject_bad_arguments_without_a_device(mccl):
     assert "max_compute_units" in err()
     assert L.mccl_fanout_sync_offers(vp(0x90000), 0, 64, 0, ctypes.byref(one), ctypes.byref(bad), vp(0x1000), two, tab, None) == -1 and "entry 32" in err()
     assert L.mccl_reduce_sync_offers(0, vp(0x80000), 64, capi.I32, capi.AVG, ctypes.byref(one), ctypes.byref(offer), vp(0x1000), two, tab, None) == -3
+    # a row of offers per rank (alltoall): the same refusals, per offer
+    rows = (capi.Offer * 2)(capi.Offer(3, 0, 7, 0, 64), capi.Offer(capi.OFFER_STAGED, capi.OFFER_SLOT_OUTBOX, 0, 0, 64))
+    expect = (ctypes.c_uint64 * 2)(64, 64)
+    each = lambda n, rank, mine, exp, offers, imports=tab, flags=two: L.mccl_rank_barrier_offers_each(
+        flags, n, rank, 1, 0, None, mine, exp, vp(0x1000), offers, imports, res, None)
+    assert each(9, 0, rows, expect, nine, flags=nine) == -3 and "1 to 8 ranks" in err()
+    assert each(2, 2, rows, expect, two) == -1 and "rank 2" in err()
+    assert each(2, 0, None, expect, two) == -1 and "null" in err()
+    assert each(2, 0, rows, None, two) == -1 and "null" in err()
+    assert each(2, 0, rows, expect, two, imports=vp(0x40004)) == -1 and "8-byte" in err()
+    assert each(2, 0, rows, expect, capi.ptr_table([0x10000, 0x20004])) == -1 and "offer pointer 1" in err()
+    rows[1] = capi.Offer(40, 0, 7, 0, 64)
+    assert each(2, 0, rows, expect, two) == -1 and "offer 1 names entry 40" in err()
+    rows[1] = capi.Offer(capi.OFFER_STAGED, 4, 0, 0, 64)
+    assert each(2, 0, rows, expect, two) == -1 and "staging buffer 4" in err()
+    ups[0] = capi.ImportUpdate(1, capi.OFFER_STAGED, 4, 0, 0x1000, 0)
+    assert L.mccl_import_table_update(tab, ups, 1, None) == -1 and "staging buffer 4" in err()
+    # the pulls behind it
+    segs = (capi.Segment * 2)(capi.Segment(0, 0xa0000, 4096), capi.Segment(0x100, 0xb0000, 4096))
+    from_ = (ctypes.c_int * 2)(0, 1)
+    pull = lambda sy, table=res, ranks=from_, n=2: L.mccl_copy_segments_sync_resolved(segs, ranks, n, table, 0, ctypes.byref(sy), None)
+    assert pull(opening) == -1 and "behind a barrier" in err()
+    assert pull(behind, table=None) == -1 and "null" in err()
+    assert pull(behind, table=vp(0x50004)) == -1 and "8-byte" in err()
+    assert pull(behind, ranks=None) == -1 and "source rank table" in err()
+    assert pull(behind, ranks=(ctypes.c_int * 2)(0, 2)) == -1 and "rank 2 of 2" in err()
+    segs[1] = capi.Segment(0x100, 0, 4096)
+    assert pull(behind) == -1 and "null pointer" in err()
+    segs[1] = capi.Segment(0, 0xb0000, 4096)
+    assert pull(behind, ranks=(ctypes.c_int * 2)(0, -1)) == -1 and "null pointer" in err()  # a plain address must not be null
     # the small allreduce with its epoch on the device
     stage = capi.ptr_table([0x100000, 0x300000])
     tf = capi.ptr_table([0x500000, 0x510000])

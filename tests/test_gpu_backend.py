@@ -65,22 +65,28 @@ def test_reference_send_recv_cases():
     _spawn(6, "reference_p2p")
 
 
-@pytest.mark.parametrize("window,world,mode", [("65536", 2, "oracle"), ("65536", 4, "oracle"), ("4096", 3, "p2p"),
-                                               ("65536", 2, "reference"), ("65536", 4, "dist"),
-                                               ("65536", 4, "coalesced_windows"), ("6291456", 8, "oracle"),
-                                               ("8192", 2, "ddp"), ("4096", 6, "reference_p2p"), ("65536", 4, "subgroup"),
-                                               ("65536", 2, "replay"), ("4096", 8, "p2p"),
-                                               ("4096", 3, "list_windows"), ("4096", 8, "list_windows"),
-                                               ("1073741824", 4, "list_windows")])
-def test_every_windowed_path_with_a_shrunk_window(monkeypatch, window, world, mode):
+@pytest.mark.parametrize("window,world,mode,standing", [("65536", 2, "oracle", "0"), ("65536", 4, "oracle", "1"), ("4096", 3, "p2p", "1"),
+                                                        ("65536", 2, "reference", "0"), ("65536", 4, "dist", "0"),
+                                                        ("65536", 4, "coalesced_windows", "1"), ("6291456", 8, "oracle", "1"),
+                                                        ("8192", 2, "ddp", "1"), ("4096", 6, "reference_p2p", "1"), ("65536", 4, "subgroup", "1"),
+                                                        ("65536", 2, "replay", "1"), ("4096", 8, "p2p", "1"),
+                                                        ("4096", 3, "list_windows", "0"), ("4096", 8, "list_windows", "0"),
+                                                        ("1073741824", 4, "list_windows", "1")])
+def test_every_windowed_path_with_a_shrunk_window(monkeypatch, window, world, mode, standing):
     """MCCL_STAGE_WINDOW_BYTES shrinks the staging window, so that messages of a few hundred KiB travel
     in many windows: the same case sets as above must give the same bits.  The 6 MiB window with 8
-    ranks puts the two-shot allreduce and a second, shorter window into one message."""
+    ranks puts the two-shot allreduce and a second, shorter window into one message.  (The all-to-alls
+    have windows only where the ranks meet on the host: MCCL_PG_STANDING_OFFERS=0 in those runs.)"""
     monkeypatch.setenv("MCCL_STAGE_WINDOW_BYTES", window)
+    monkeypatch.setenv("MCCL_PG_STANDING_OFFERS", standing)
     _spawn(world, mode)
 
 
-def test_message_larger_than_one_staging_window():
+@pytest.mark.parametrize("standing", ["1", "0"])
+def test_message_larger_than_one_staging_window(monkeypatch, standing):
+    """(with standing offers the all-to-all's pieces of 900 and 1100 MiB are read in place, whatever the
+    peers have mapped before; without, the images travel in windows)"""
+    monkeypatch.setenv("MCCL_PG_STANDING_OFFERS", standing)
     _spawn(2, "large")
 
 
@@ -127,6 +133,18 @@ def test_zero_copy_collectives(world):
 def test_allreduce_with_offers_exchanged_on_the_device(world):
     """No rendezvous of the host threads in steady state; a late rank does not hold up the others' calls."""
     _spawn(world, "standing")
+
+
+@pytest.mark.parametrize("world", [2, 5, 8])
+def test_all_to_all_with_offers_exchanged_on_the_device(world):
+    """all_to_all_single and all_to_all: no rendezvous of the host threads; two ranks meet (nobody else)
+    when a piece between them outgrows the buffer kept for it."""
+    _spawn(world, "standing_alltoall")
+
+
+def test_all_to_all_pieces_larger_than_any_outbox_are_read_in_place(monkeypatch):
+    monkeypatch.setenv("MCCL_PG_STANDING_MAX_BYTES", str(2 << 20))
+    _spawn(4, "standing_big")
 
 
 def test_allreduce_with_the_host_rendezvous_instead(monkeypatch):

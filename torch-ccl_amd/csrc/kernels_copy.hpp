@@ -33,6 +33,16 @@ struct SyncCopyArgs {
   XSync sync;
   uint32_t invalidate;  // some bytes are read through the caches: invalidate once per workgroup first
   uint32_t shared;      // other ranks read the same sources: leave them in the memory-side cache
+  // INDIRECT kernel: segment s is read from src_table[src_rank[s]] + (its src taken as a byte offset)
+  // when src_rank[s] >= 0 -- the table a barrier kernel in front has resolved the ranks' offers into
+  const uint64_t* src_table;
+  int8_t src_rank[kMaxSegs];
+};
+
+// Where the sources of the segments are when the host does not know.
+struct CopySources {
+  const uint64_t* table;
+  const int8_t* rank;
 };
 
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
@@ -45,8 +55,9 @@ struct SyncCopyArgs {
 // UNROLL: 16-byte vectors per lane per chunk (chunk = 64 x 16 x UNROLL bytes; the host computes
 // the segment geometry for the same value).  STREAM: full chunks are written through past the
 // caches (`sc1`) instead of with the non-temporal hint.
-template <bool COHERENT, int UNROLL, bool STREAM>
-__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave& w, bool shared_sources = false) {
+template <bool COHERENT, int UNROLL, bool STREAM, bool INDIRECT = false>
+__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave& w, bool shared_sources = false,
+                                                   const CopySources from = CopySources{nullptr, nullptr}) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = w.index; chunk < total; chunk += w.count) {
@@ -63,6 +74,15 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave
     const uint32_t t = w.lane;
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
+    if constexpr (INDIRECT) {
+      const int r = from.rank[lo];  // uniform
+      if (r >= 0) {
+        // written by the kernel in front on the stream, constant while this one runs: a scalar load
+        const uint64_t base = ((const __attribute__((address_space(4))) uint64_t*)from.table)[r];
+        if (base == 0) continue;  // not resolved: the barrier in front has reported it
+        src = (const char*)(base + (uint64_t)(uintptr_t)src);
+      }
+    }
     if (c == 0)
       for (uint32_t i = t; i < head; i += kWave) dst[i] = src[i];  // head < 128
     const size_t off = (size_t)head + (size_t)c * CHUNK;  // start of this chunk
@@ -106,6 +126,13 @@ __global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const S
     copy_segments_body<true, kCopyUnroll, false>(a.copy, this_wave<WPG>(), a.shared != 0);
   }
   xsync_end(a.sync, gridDim.x);
+}
+
+// The same behind a barrier kernel that has resolved where the sources are (no opening wait).
+__global__ __launch_bounds__(kWave) void copy_segments_resolved_kernel(const SyncCopyArgs a) {
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // alignment of the sources unknown: anything may go through the caches
+  copy_segments_body<true, kCopyUnroll, false, true>(a.copy, this_wave<1>(), a.shared != 0, CopySources{a.src_table, a.src_rank});
+  xsync_end(a.sync, gridDim.x, /*wrote_to_peers=*/false);
 }
 
 // allgather as pushes: this rank's contribution goes into every rank's output in one pass -- read

@@ -298,7 +298,7 @@ __device__ __forceinline__ uint64_t resolve_offer(const uint64_t* slot, const mc
   const uint64_t off = __hip_atomic_load(slot + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   const uint32_t entry = (uint32_t)w0, which = (uint32_t)(w0 >> 32);
   if (entry == MCCL_OFFER_STAGED) {
-    const uint64_t b = imports->staging[r][which & 1u];
+    const uint64_t b = imports->staging[r][which & (MCCL_OFFER_SLOTS - 1u)];
     return b ? b + off : 0;
   }
   if (entry < MCCL_OFFER_ENTRIES) {
@@ -330,6 +330,59 @@ __global__ __launch_bounds__(kWave) void rank_barrier_offers_kernel(const OfferB
   a.resolved[lane] = where;
 }
 
+// The barrier of a collective in which every rank hands every peer a different piece: a rank
+// publishes a row of offers (entry k: the piece for rank k, and its length) and resolves the column
+// addressed to it.
+struct OfferEachArgs {
+  uint64_t* flag[MCCL_OFFER_RANKS];
+  uint64_t* row[MCCL_OFFER_RANKS];    // rank r's row of n offers, four 64-bit words each
+  uint64_t epoch;
+  uint64_t limit_ticks;
+  uint32_t* status;
+  uint64_t mine[MCCL_OFFER_RANKS][4];  // this rank's row
+  uint64_t expect[MCCL_OFFER_RANKS];   // bytes this rank expects from rank r
+  uint64_t my_source;
+  const mccl_import_table_t* imports;
+  uint64_t* resolved;
+  int n;
+  int rank;
+};
+
+__global__ __launch_bounds__(kWave) void rank_barrier_offers_each_kernel(const OfferEachArgs a) {
+  const int lane = threadIdx.x;
+  if (lane == 0) {
+    // the whole row by the thread that stores the flag after it (its release covers them)
+    uint64_t* row = a.row[a.rank];
+#pragma unroll
+    for (int k = 0; k < MCCL_OFFER_RANKS; ++k) {
+      if (k < a.n) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) __hip_atomic_store(row + 4 * k + i, a.mine[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+    __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  if (lane >= a.n) return;
+  uint64_t where = a.my_source;
+  if (lane != a.rank) {
+    where = 0;
+    if (!wait_flag64(a.flag[lane], a.epoch, a.limit_ticks)) {
+      report_late(a.status, lane, (uint32_t)a.epoch);
+    } else {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the offer is read after the flag
+      const uint64_t* slot = a.row[lane] + 4 * a.rank;
+      const uint64_t bytes = __hip_atomic_load(slot + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      if (bytes != a.expect[lane]) {
+        report_late(a.status, lane, MCCL_STATUS_MISMATCH);
+      } else if (bytes != 0) {
+        where = resolve_offer(slot, a.imports, lane);
+        if (!where) report_late(a.status, lane, MCCL_STATUS_UNMAPPED);
+      }
+    }
+  }
+  a.resolved[lane] = where;
+}
+
 // Stream-ordered update of the table that rank_barrier_offers_kernel resolves against: one lane
 // per update, the values are kernel arguments.
 struct ImportUpdateArgs {
@@ -343,7 +396,7 @@ __global__ __launch_bounds__(kWave) void import_table_update_kernel(const Import
   if (lane >= a.n) return;
   const mccl_import_update_t u = a.update[lane];
   if (u.entry == MCCL_OFFER_STAGED) {
-    a.table->staging[u.rank][u.slot & 1u] = u.base;
+    a.table->staging[u.rank][u.slot & (MCCL_OFFER_SLOTS - 1u)] = u.base;
   } else {
     a.table->generation[u.rank][u.entry] = u.generation;
     a.table->base[u.rank][u.entry] = u.base;

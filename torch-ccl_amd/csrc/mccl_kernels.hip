@@ -756,13 +756,52 @@ int mccl_rank_barrier_offers(void* const* flags, int n, int rank, uint64_t epoch
   a.mine[0] = (uint64_t)mine->entry | ((uint64_t)mine->slot << 32);
   a.mine[1] = mine->generation;
   a.mine[2] = mine->offset;
-  a.mine[3] = mine->reserved;
+  a.mine[3] = mine->bytes;
   a.my_buffer = (uint64_t)(uintptr_t)my_buffer;
   a.imports = imports;
   a.resolved = (uint64_t*)resolved;
   a.n = n;
   a.rank = rank;
   hipLaunchKernelGGL(rank_barrier_offers_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "barrier kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
+}
+
+int mccl_rank_barrier_offers_each(void* const* flags, int n, int rank, uint64_t epoch, uint64_t timeout_us, void* status,
+                                  const mccl_offer_t* mine, const uint64_t* expect_bytes, const void* my_source,
+                                  void* const* offers, const mccl_import_table_t* imports, void* resolved, void* stream) {
+  if (!flags || !offers) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer table is null");
+  if (n < 1 || n > MCCL_OFFER_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "a barrier with offers takes 1 to %d ranks, got %d", MCCL_OFFER_RANKS, n);
+  if (rank < 0 || rank >= n) return fail(MCCL_ERR_INVALID_ARG, "rank %d outside [0, %d)", rank, n);
+  if ((uintptr_t)status % 4) return fail(MCCL_ERR_INVALID_ARG, "status word is not 4-byte aligned");
+  if (!mine || !expect_bytes || !imports || !resolved) return fail(MCCL_ERR_INVALID_ARG, "offers, expected lengths, import table or output table is null");
+  if ((uintptr_t)imports % 8 || (uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "import table or output table is not 8-byte aligned");
+  OfferEachArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int r = 0; r < n; ++r) {
+    if (!flags[r] || !offers[r]) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer %d is null", r);
+    if ((uintptr_t)flags[r] % 8 || (uintptr_t)offers[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "flag or offer pointer %d is not 8-byte aligned", r);
+    const mccl_offer_t& o = mine[r];
+    if (o.entry != MCCL_OFFER_STAGED && o.entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "offer %d names entry %u of %d", r, o.entry, MCCL_OFFER_ENTRIES);
+    if (o.entry == MCCL_OFFER_STAGED && o.slot >= MCCL_OFFER_SLOTS) return fail(MCCL_ERR_INVALID_ARG, "offer %d names staging buffer %u of %d", r, o.slot, MCCL_OFFER_SLOTS);
+    a.flag[r] = (uint64_t*)flags[r];
+    a.row[r] = (uint64_t*)offers[r];
+    a.mine[r][0] = (uint64_t)o.entry | ((uint64_t)o.slot << 32);
+    a.mine[r][1] = o.generation;
+    a.mine[r][2] = o.offset;
+    a.mine[r][3] = o.bytes;
+    a.expect[r] = expect_bytes[r];
+  }
+  a.epoch = epoch;
+  a.limit_ticks = wait_limit_ticks(timeout_us);
+  a.status = (uint32_t*)status;
+  a.my_source = (uint64_t)(uintptr_t)my_source;
+  a.imports = imports;
+  a.resolved = (uint64_t*)resolved;
+  a.n = n;
+  a.rank = rank;
+  hipLaunchKernelGGL(rank_barrier_offers_each_kernel, dim3(1), dim3(kWave), 0, (hipStream_t)stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "barrier kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
@@ -781,8 +820,9 @@ int mccl_import_table_update(mccl_import_table_t* table, const mccl_import_updat
     const mccl_import_update_t& u = updates[i];
     if (u.rank >= MCCL_OFFER_RANKS) return fail(MCCL_ERR_INVALID_ARG, "update %d names rank %u of %d", i, u.rank, MCCL_OFFER_RANKS);
     if (u.entry != MCCL_OFFER_STAGED && u.entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "update %d names entry %u of %d", i, u.entry, MCCL_OFFER_ENTRIES);
+    if (u.entry == MCCL_OFFER_STAGED && u.slot >= MCCL_OFFER_SLOTS) return fail(MCCL_ERR_INVALID_ARG, "update %d names staging buffer %u of %d", i, u.slot, MCCL_OFFER_SLOTS);
     for (int j = 0; j < i; ++j)
-      if (updates[j].rank == u.rank && updates[j].entry == u.entry && (u.entry != MCCL_OFFER_STAGED || (updates[j].slot & 1u) == (u.slot & 1u)))
+      if (updates[j].rank == u.rank && updates[j].entry == u.entry && (u.entry != MCCL_OFFER_STAGED || updates[j].slot == u.slot))
         return fail(MCCL_ERR_INVALID_ARG, "updates %d and %d name the same entry", j, i);
     a.update[i] = u;
   }
@@ -1041,7 +1081,7 @@ int allreduce_sync_impl(void* const* tensors, const void* resolved, const OfferE
     a.mine[0] = (uint64_t)ox->mine->entry | ((uint64_t)ox->mine->slot << 32);
     a.mine[1] = ox->mine->generation;
     a.mine[2] = ox->mine->offset;
-    a.mine[3] = ox->mine->reserved;
+    a.mine[3] = ox->mine->bytes;
     a.imports = ox->imports;
     a.my_buffer = (uint64_t)(uintptr_t)ox->my_buffer;
     a.in_off = lo * es;
@@ -1058,14 +1098,14 @@ int allreduce_sync_impl(void* const* tensors, const void* resolved, const OfferE
   return MCCL_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync, void* stream) {
+// src_rank / resolved: the sources come from a table in device memory (mccl_copy_segments_sync_resolved).
+int copy_segments_sync_impl(const mccl_segment_t* segs, const int* src_rank, const void* resolved, int nseg, unsigned flags,
+                            const mccl_xsync_t* sync, void* stream) {
   SyncCopyArgs a;
   int rc = fill_xsync(sync, &a.sync);
   if (rc != MCCL_OK) return rc;
+  a.src_table = (const uint64_t*)resolved;
+  memset(a.src_rank, 0xff, sizeof(a.src_rank));
   if (nseg < 0 || nseg > kMaxSegs) return fail(MCCL_ERR_INVALID_ARG, "a one-launch copy takes 0 to %d segments, got %d", kMaxSegs, nseg);
   if (nseg && !segs) return fail(MCCL_ERR_INVALID_ARG, "segment table is null");
   int m = 0;
@@ -1074,7 +1114,10 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   for (int i = 0; i < nseg; ++i) {
     const mccl_segment_t& sg = segs[i];
     if (sg.bytes == 0) continue;
-    if (!sg.src || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
+    const int from = src_rank ? src_rank[i] : -1;
+    if (from >= a.sync.n) return fail(MCCL_ERR_INVALID_ARG, "segment %d reads from rank %d of %d", i, from, a.sync.n);
+    if ((from < 0 && !sg.src) || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "segment %d has a null pointer", i);
+    a.src_rank[m] = (int8_t)(from < 0 ? -1 : from);
     const uintptr_t dp = (uintptr_t)sg.dst;
     CopySeg cs;
     cs.src = (const char*)sg.src;
@@ -1109,7 +1152,10 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   int cus = 0;
   rc = device_cus(&cus);
   if (rc != MCCL_OK) return rc;
-  if (shape.packed) {
+  if (resolved) {
+    if (shape.packed) return fail(MCCL_ERR_INVALID_ARG, "a copy over resolved addresses runs as single wavefronts (max_compute_units 0)");
+    hipLaunchKernelGGL(copy_segments_resolved_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+  } else if (shape.packed) {
     static const unsigned per_cu = blocks_per_cu(copy_segments_sync_kernel<kPackedWaves>, kWave * kPackedWaves);
     if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
     hipLaunchKernelGGL(copy_segments_sync_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
@@ -1121,6 +1167,24 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MCCL_ERR_HIP, "copy kernel launch failed: %s", hipGetErrorString(e));
   return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags, const mccl_xsync_t* sync, void* stream) {
+  return copy_segments_sync_impl(segs, nullptr, nullptr, nseg, flags, sync, stream);
+}
+
+int mccl_copy_segments_sync_resolved(const mccl_segment_t* segs, const int* src_rank, int nseg, const void* resolved,
+                                     unsigned flags, const mccl_xsync_t* sync, void* stream) {
+  if (!resolved) return fail(MCCL_ERR_INVALID_ARG, "address table is null");
+  if ((uintptr_t)resolved % 8) return fail(MCCL_ERR_INVALID_ARG, "address table is not 8-byte aligned");
+  if (nseg > 0 && !src_rank) return fail(MCCL_ERR_INVALID_ARG, "source rank table is null");
+  if (sync && (sync->ready_epoch != 0 || sync->done_epoch == 0))
+    return fail(MCCL_ERR_INVALID_ARG, "a launch over resolved addresses runs behind a barrier: ready_epoch 0, done_epoch set");
+  return copy_segments_sync_impl(segs, src_rank, resolved, nseg, flags, sync, stream);
 }
 
 int mccl_fanout_sync(const void* src, void* const* dst, int ndst, size_t bytes, const mccl_xsync_t* sync, void* stream) {
@@ -1232,7 +1296,7 @@ void offer_words(const mccl_offer_t& mine, uint64_t (&w)[4]) {
   w[0] = (uint64_t)mine.entry | ((uint64_t)mine.slot << 32);
   w[1] = mine.generation;
   w[2] = mine.offset;
-  w[3] = mine.reserved;
+  w[3] = mine.bytes;
 }
 
 int check_indirect_sync(const mccl_xsync_t* sync, bool one_launch) {

@@ -109,6 +109,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce(std::vector<at::Tensor
       p.standing.ok = true;
       p.standing.buffer = base;
       p.standing.bytes = len * es;
+      p.standing.block = t.storage().data();
+      p.standing.block_bytes = t.storage().nbytes();
       p.standing.copy_in = p.standing.copy_out = true;
       p.standing.compact_cost = 1.0;
       p.standing.behind_barrier = [=](const void* resolved, bool, const mccl_xsync_t& sync, hipStream_t s) {
@@ -293,6 +295,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_allgather_base(at::Tensor& outp
         p.standing.ok = true;
         p.standing.buffer = output.data_ptr();
         p.standing.bytes = per_rank * (size_t)W;
+        p.standing.block = output.storage().data();
+        p.standing.block_bytes = output.storage().nbytes();
         p.standing.copy_out = true;
         p.standing.force_staged = touchesForeignSlice(input.data_ptr(), per_rank, output.data_ptr(), per_rank, W, me);
         p.standing.compact_cost = 1.0;
@@ -535,6 +539,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::_reduce_scatter_base(at::Tensor&
         p.standing.ok = true;
         p.standing.buffer = in;
         p.standing.bytes = M * es * (size_t)W;
+        p.standing.block = input.storage().data();
+        p.standing.block_bytes = input.storage().nbytes();
         p.standing.copy_in = true;
         p.standing.force_staged = touchesForeignSlice(output.data_ptr(), M * es, in, M * es, W, me);
         p.standing.compact_cost = 0.5;
@@ -797,6 +803,34 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::exchange(c10d::OpType op, const 
   const int me = rank_;
   const bool is_base = op == c10d::OpType::ALLTOALL_BASE;
   const size_t total = image.total;
+  if (standingExchangeNow(inputs, outputs)) {
+    // rank processes that exchange where their pieces are on the device: nothing is published on the
+    // host, nobody meets (runStandingExchange)
+    Plan p;
+    p.op = op;
+    p.title = title;
+    p.inputs = inputs;
+    p.outputs = outputs;
+    Plan::StandingExchange& x = p.standing_exchange;
+    x.ok = true;
+    x.send = image.sizes;
+    x.recv = recv;
+    x.dst = dst;
+    x.piece.assign((size_t)W, nullptr);
+    x.block.assign((size_t)W, nullptr);
+    x.block_bytes.assign((size_t)W, 0);
+    for (int d = 0; d < W; ++d) {
+      if (!image.sizes[(size_t)d]) continue;
+      x.piece[(size_t)d] = image.flat ? (const void*)((const char*)image.flat + image.offs[(size_t)d]) : image.pieces[(size_t)d].data_ptr();
+      // (a flat image is one tensor, or consecutive views of one storage)
+      const at::Tensor& holder = image.flat ? (is_base ? inputs[0] : inputs[(size_t)d]) : image.pieces[(size_t)d];
+      x.block[(size_t)d] = holder.storage().data();
+      x.block_bytes[(size_t)d] = holder.storage().nbytes();
+      for (int r = 0; r < W; ++r)
+        if (rangesOverlap(x.piece[(size_t)d], image.sizes[(size_t)d], dst[(size_t)r], recv[(size_t)r])) x.force_staged = true;
+    }
+    return run(p);
+  }
   auto nwin = std::make_shared<size_t>(1);
   const size_t window = stage_max_;
   c10::intrusive_ptr<c10d::Work> work;

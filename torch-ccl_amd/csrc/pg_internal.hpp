@@ -73,11 +73,22 @@ constexpr size_t kArenaDoneCountOff = 24u << 10;  // MCCL_SYNC_COUNTER_BYTES of 
 constexpr size_t kArenaFusedStateOff = 2048;  // MCCL_FUSED_STATE_BYTES: the device-resident epoch of the one-launch small allreduce
 constexpr size_t kArenaOfferOff = 3072;       // two mccl_offer_t, 64 bytes apart: what this rank's tensor of a collective is
 constexpr size_t kArenaOfferStride = 64;
+constexpr size_t kArenaOfferRowOff = 3584;    // two rows of MCCL_OFFER_RANKS offers (all-to-all: one offer per reader), 256 bytes each
+constexpr size_t kArenaOfferRowStride = MCCL_OFFER_RANKS * sizeof(mccl_offer_t);
 constexpr size_t kArenaImportTableOff = 32u << 10;  // mccl_import_table_t: the peers' allocations as this rank has mapped them
 constexpr size_t kArenaResolvedOff = 40u << 10;     // MCCL_OFFER_RANKS addresses: the ranks' tensors of the collective under way
 constexpr size_t kArenaBytes = kArenaFusedStageOff + 2 * kArenaFusedStageStride;
 static_assert(kArenaFusedStateOff + MCCL_FUSED_STATE_BYTES <= kArenaOfferOff && kArenaOfferOff + 2 * kArenaOfferStride <= kArenaFusedFlagsOff, "the offers lie between the epoch state and the flags");
 static_assert(sizeof(mccl_offer_t) <= kArenaOfferStride, "an offer fits its slot");
+static_assert(kArenaOfferOff + 2 * kArenaOfferStride <= kArenaOfferRowOff && kArenaOfferRowOff + 2 * kArenaOfferRowStride <= kArenaFusedFlagsOff, "the rows of offers lie between the offers and the flags");
+// Outboxes of the all-to-all with standing offers: buffers of 2 MiB << level, level < kOutboxLevels.
+constexpr size_t kOutboxMin = 2u << 20;
+constexpr int kOutboxLevels = 10;  // up to 1 GiB: an allocation must stay below 2 GiB to be shared
+inline int outboxLevel(size_t bytes) {
+  int level = 0;
+  while ((kOutboxMin << level) < bytes) ++level;
+  return level;
+}
 static_assert(kArenaImportTableOff + sizeof(mccl_import_table_t) <= kArenaResolvedOff, "the import table ends before the resolved addresses");
 static_assert(kArenaResolvedOff + MCCL_OFFER_RANKS * 8 <= kArenaFusedStageOff, "the resolved addresses end before the staging buffers");
 static_assert(kMaxExports == MCCL_OFFER_ENTRIES, "an offer names an entry of the export table");
@@ -253,6 +264,27 @@ struct alignas(128) RankSlot {
     std::atomic<uint64_t> gen;
     std::atomic<uint64_t> from_seq;
   } acked[MCCL_OFFER_RANKS][kMaxExports];
+  // All-to-all with standing offers.  outbox[d] is what this rank keeps for the pieces it sends rank d
+  // when it cannot offer them in place: one buffer per size class (level), created when a piece first
+  // needs it -- which rank d knows as well as this rank, because the length of the piece is the one
+  // thing both of them know.  `ready` is written last.
+  struct OutboxLevel {
+    std::atomic<uint64_t> ready;
+    uint64_t ptr;
+    hipIpcMemHandle_t handle;
+  };
+  struct Outbox {
+    OutboxLevel level[kOutboxLevels];
+  } outbox[MCCL_OFFER_RANKS];
+  // A piece too large for any outbox is always read in place: big[d] says where the piece of this
+  // rank's collective #seq for rank d is, and rank d maps it before it enqueues (big_seen[r]: the last
+  // record of rank r's that this rank has read; the owner does not overwrite an unread one).
+  struct BigPiece {
+    std::atomic<uint64_t> seq;
+    int64_t entry;   // of this rank's export table; < 0: cannot be shared
+    uint64_t gen;
+  } big[MCCL_OFFER_RANKS];
+  std::atomic<uint64_t> big_seen[MCCL_OFFER_RANKS];
   P2PBox p2p[kMaxWorld];
 };
 

@@ -322,7 +322,13 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
   uint64_t off = 0;
   // (small buffers live in the allocator's 2 MiB segments, many of them: announcing those would turn
   // the table of allocations over all the time, and copying them costs next to nothing)
-  const int entry = (st.force_staged || bytes < kZeroCopyMinBytes) ? -1 : exportRange(st.buffer, bytes, &off);
+  int entry = -1;
+  if (!st.force_staged && bytes >= kZeroCopyMinBytes) {
+    const bool inside = st.block && (const char*)st.buffer >= (const char*)st.block &&
+                        (const char*)st.buffer + bytes <= (const char*)st.block + st.block_bytes;
+    entry = inside ? exportRange(st.block, st.block_bytes, &off) : exportRange(st.buffer, bytes, &off);
+    if (inside && entry >= 0) off += (uint64_t)((const char*)st.buffer - (const char*)st.block);
+  }
   // A message larger than the staging every rank keeps mapped: the host threads meet (all at this
   // collective: the sizes agree) -- and since they do, they also look at what everybody has just
   // announced before anybody decides, so that the first collective of a new size already runs in place.
@@ -375,6 +381,255 @@ void ProcessGroupCCL::runStanding(Plan& plan, hipStream_t s, int slot, uint64_t 
     st.behind_barrier(resolved_, !in_place, sync, s);
   }
   if (!in_place && st.copy_out) copyAsync(st.buffer, buffer, bytes, s);
+}
+
+// ---------------------------------------------------------------------------------------------
+// all-to-all with standing offers
+// ---------------------------------------------------------------------------------------------
+// In an all-to-all every rank hands every peer a different piece, and the sizes differ from rank to
+// rank: there is no number that all ranks know, so nothing the whole group could agree on without
+// meeting -- not "everybody stages", not "the staging buffers grow now".  What two ranks do know in
+// common is the length of the piece that goes from one to the other.  So everything is decided pair
+// by pair: rank r offers rank d its piece in place when d has mapped the allocation it lives in, and
+// through a buffer it keeps for d alone (its outbox for d) otherwise; the outbox has the size class
+// of the largest piece that ever went from r to d, so both know when a larger one is due -- r
+// creates it on entering that collective, d waits for it there (the only wait of this path, and only
+// for that one peer).  Pieces beyond the largest outbox are read in place always: the receiver waits
+// until the sender has entered the collective and said where the piece is, and maps it then.
+// The offers travel on the device as a row per rank (mccl_rank_barrier_offers_each); each rank pulls
+// the column addressed to it (mccl_copy_segments_sync_resolved).
+bool ProcessGroupCCL::standingExchangeFits() const {
+  return standing_offers_ && device_sync_ && distinct_pids_ && zero_copy_ && !waits_in_data_kernels_ && !work_only_ &&
+         !sync_only_ && size_ > 1 && size_ <= MCCL_OFFER_RANKS;
+}
+
+// For the all-to-all engine, which has to know before it plans (the fallback moves images larger than
+// a staging window in several rounds, this path never does): initialises the group if this is its
+// first collective, like run() would a moment later.
+bool ProcessGroupCCL::standingExchangeNow(const std::vector<at::Tensor>& inputs, const std::vector<at::Tensor>& outputs) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  int device = -1;
+  for (const auto& t : inputs) if (t.defined()) { device = t.get_device(); break; }
+  if (device < 0) for (const auto& t : outputs) if (t.defined()) { device = t.get_device(); break; }
+  if (device < 0) return false;
+  c10::DeviceGuard guard(c10::Device(at::kCUDA, (c10::DeviceIndex)device));
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_CHECK(hipStreamIsCapturing(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA((c10::DeviceIndex)device).stream(), &capture));
+  if (capture != hipStreamCaptureStatusNone) return false;  // run() refuses it with the reason
+  ensureInit(device);
+  return standingExchangeFits();
+}
+
+bool ProcessGroupCCL::acknowledgedBy(int peer, int entry, uint64_t gen, uint64_t seq) const {
+  const RankSlot::Ack& a = ctl_->slot[peer].acked[rank_][entry];
+  if (a.gen.load(std::memory_order_acquire) != gen) return false;
+  const uint64_t from = a.from_seq.load(std::memory_order_acquire);
+  return a.gen.load(std::memory_order_acquire) == gen && from <= seq;
+}
+
+// A larger outbox for rank `peer` (for this rank itself: scratch).  The old one stays until the group
+// goes: the peer's kernels of earlier collectives may still read it.
+void ProcessGroupCCL::growOutbox(int peer, int level) {
+  TORCH_CHECK(level < kOutboxLevels, "ccl backend: outbox level ", level);
+  void* base = nullptr;
+  HIP_CHECK(hipMalloc(&base, kOutboxMin << level));
+  OutboxOut& out = outbox_out_[peer];
+  if (out.base) retired_.push_back(out.base);
+  out.base = base;
+  out.level = level;
+  if (peer == rank_) return;
+  RankSlot::OutboxLevel& lv = ctl_->slot[rank_].outbox[peer].level[level];
+  HIP_CHECK(hipIpcGetMemHandle(&lv.handle, base));
+  lv.ptr = (uint64_t)(uintptr_t)base;
+  lv.ready.store(1, std::memory_order_release);
+}
+
+// Rank `peer`'s outbox of size class `level` for this rank: the peer creates it when it enters the
+// collective whose piece needs it, which is the collective this rank is entering.
+void ProcessGroupCCL::mapOutbox(int peer, int level) {
+  RankSlot::OutboxLevel& lv = ctl_->slot[peer].outbox[rank_].level[level];
+  if (!lv.ready.load(std::memory_order_acquire)) {
+    ++pairwise_waits_now_;
+    spinUntil([&] { return lv.ready.load(std::memory_order_acquire) != 0; }, peer,
+              "the buffer a rank keeps for the pieces of its all-to-alls to this rank (if that rank has entered the same all-to-all, "
+              "its inputSplitSizes do not match this rank's outputSplitSizes)",
+              [] { return true; });
+  }
+  OutboxIn& in = outbox_in_[peer];
+  if (in.base) {
+    quiesce();  // earlier kernels of this rank may still read through the old mapping
+    (void)hipIpcCloseMemHandle(in.base);
+    in.base = nullptr;
+  }
+  void* p = nullptr;
+  HIP_CHECK(hipIpcOpenMemHandle(&p, lv.handle, hipIpcMemLazyEnablePeerAccess));
+  in.base = p;
+  in.level = level;
+  noteImport((uint32_t)peer, MCCL_OFFER_STAGED, MCCL_OFFER_SLOT_OUTBOX, (uint64_t)(uintptr_t)p, 0);
+}
+
+void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t seq) {
+  const Plan::StandingExchange& x = plan.standing_exchange;
+  const int W = size_, me = rank_;
+  const uint64_t epoch = 4 * seq;
+  RankSlot& mine_slot = ctl_->slot[me];
+  const size_t outbox_max = std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1));
+  pairwise_waits_now_ = 0;
+  // 1. Everything this rank has to say, before it waits for anything of anybody's: the allocations
+  // its pieces live in, larger outboxes where a piece has outgrown the old one, where its oversized
+  // pieces are.
+  struct Where {
+    int entry = -1;
+    uint64_t gen = 0, off = 0;
+  } where[MCCL_OFFER_RANKS];
+  bool unshareable_big = false;
+  for (int d = 0; d < W; ++d) {
+    const size_t b = x.send[(size_t)d];
+    if (d == me || !b || x.force_staged) continue;
+    const bool big = b > outbox_max;
+    // (small tensors live in the allocator's 2 MiB segments, many of them: announcing those would turn
+    // the table of allocations over all the time, and copying them costs next to nothing)
+    if (!big && x.block_bytes[(size_t)d] < kZeroCopyMinBytes) continue;
+    Where& w = where[d];
+    w.entry = exportRange(x.block[(size_t)d], x.block_bytes[(size_t)d], &w.off);
+    if (w.entry >= 0 && w.entry < kMaxExports) {
+      w.gen = mine_slot.exports[w.entry].gen.load(std::memory_order_acquire);
+      w.off += (uint64_t)((const char*)x.piece[(size_t)d] - (const char*)x.block[(size_t)d]);
+    } else {
+      w.entry = -1;
+    }
+  }
+  // (pieces in more allocations than the table has free entries: a later one may have taken the entry
+  // of an earlier one)
+  for (int d = 0; d < W; ++d)
+    if (where[d].entry >= 0 && mine_slot.exports[where[d].entry].gen.load(std::memory_order_acquire) != where[d].gen) where[d].entry = -1;
+  for (int d = 0; d < W; ++d) {
+    const size_t b = x.send[(size_t)d];
+    if (!b) continue;
+    if (b <= outbox_max) {
+      const int level = outboxLevel(b);
+      const bool needed = d != me || x.force_staged;  // (this rank's piece for itself is copied where it lies, unless that overlaps)
+      if (needed && level > outbox_out_[d].level) growOutbox(d, level);
+    } else if (d != me) {
+      TORCH_CHECK(!x.force_staged, "ccl backend: ", plan.title, ": input and output overlap and the piece for rank ", d, " (", b,
+                  " bytes) is larger than the buffers kept for such pieces (", outbox_max, " bytes); set MCCL_PG_STANDING_OFFERS=0");
+      RankSlot::BigPiece& rec = mine_slot.big[d];
+      if (big_published_[d]) {  // rank d has not read the last such record yet: not overwritten before it has
+        const uint64_t last = big_published_[d];
+        if (ctl_->slot[d].big_seen[me].load(std::memory_order_acquire) < last) {
+          ++pairwise_waits_now_;
+          spinUntil([&] { return ctl_->slot[d].big_seen[me].load(std::memory_order_acquire) >= last; }, d,
+                    "a rank to take note of an earlier oversized all-to-all piece", [] { return true; });
+        }
+      }
+      rec.entry = where[d].entry;
+      rec.gen = where[d].gen;
+      rec.seq.store(seq + 1, std::memory_order_release);
+      big_published_[d] = seq + 1;
+      if (where[d].entry < 0) unshareable_big = true;
+    }
+  }
+  TORCH_CHECK(!unshareable_big, "ccl backend: ", plan.title, ": a piece larger than ", outbox_max,
+              " bytes lives in memory that cannot be shared between processes (not from torch's caching allocator, or an allocation of 2 GiB "
+              "or more); set MCCL_PG_STANDING_OFFERS=0");
+  // 2. What the peers must have said by now, pair by pair.
+  for (int r = 0; r < W; ++r) {
+    const size_t b = x.recv[(size_t)r];
+    if (r == me || !b) continue;
+    if (b <= outbox_max) {
+      const int level = outboxLevel(b);
+      if (level > outbox_in_[r].level) mapOutbox(r, level);
+    } else {
+      RankSlot::BigPiece& rec = ctl_->slot[r].big[me];
+      if (rec.seq.load(std::memory_order_acquire) != seq + 1) {
+        ++pairwise_waits_now_;
+        spinUntil([&] { return rec.seq.load(std::memory_order_acquire) >= seq + 1; }, r,
+                  "a rank to enter the all-to-all in which it sends this rank an oversized piece", [] { return true; });
+      }
+      TORCH_CHECK(rec.seq.load(std::memory_order_acquire) == seq + 1, "ccl backend: ", plan.title, ": rank ", r,
+                  " is at another oversized all-to-all piece for this rank (the ranks' split sizes do not match)");
+    }
+  }
+  scanPeerExports(seq);
+  for (int r = 0; r < W; ++r) {
+    const size_t b = x.recv[(size_t)r];
+    if (r == me || b <= outbox_max) continue;
+    RankSlot::BigPiece& rec = ctl_->slot[r].big[me];
+    const int64_t entry = rec.entry;
+    const uint64_t gen = rec.gen;
+    ctl_->slot[me].big_seen[r].store(seq + 1, std::memory_order_release);
+    TORCH_CHECK(entry >= 0 && entry < kMaxExports, "ccl backend: ", plan.title, ": rank ", r, " cannot share the memory that holds its piece of ", b,
+                " bytes for this rank, which is larger than the buffers kept for such pieces; set MCCL_PG_STANDING_OFFERS=0");
+    const Import& im = imports_[(size_t)r][(size_t)entry];
+    TORCH_CHECK(im.base && im.gen == gen, "ccl backend: ", plan.title, ": could not map the allocation that holds rank ", r, "'s piece for this rank");
+  }
+  // 3. This rank's row of offers.
+  mccl_offer_t row[MCCL_OFFER_RANKS] = {};
+  uint64_t expect[MCCL_OFFER_RANKS] = {};
+  std::vector<mccl_segment_t> copy_in;
+  int in_place = 0, staged = 0;
+  for (int d = 0; d < W; ++d) {
+    const size_t b = x.send[(size_t)d];
+    mccl_offer_t& o = row[d];
+    o.bytes = b;
+    o.entry = MCCL_OFFER_STAGED;
+    o.slot = MCCL_OFFER_SLOT_OUTBOX;
+    expect[d] = x.recv[(size_t)d];
+    if (!b || d == me) continue;
+    const Where& w = where[d];
+    if (w.entry >= 0 && (b > outbox_max || acknowledgedBy(d, w.entry, w.gen, seq))) {
+      o.entry = (uint32_t)w.entry;
+      o.slot = 0;
+      o.generation = w.gen;
+      o.offset = w.off;
+      last_offer_seq_[w.entry] = seq + 1;  // in the units of `entered`: collective `seq` is under way at seq + 1
+      ++in_place;
+    } else {
+      copy_in.push_back({x.piece[(size_t)d], outbox_out_[d].base, b});
+      ++staged;
+    }
+  }
+  const void* my_source = x.piece[(size_t)me];
+  if (x.force_staged && x.send[(size_t)me]) {
+    copy_in.push_back({x.piece[(size_t)me], outbox_out_[me].base, x.send[(size_t)me]});
+    my_source = outbox_out_[me].base;
+  }
+  if (!copy_in.empty()) MCCL_CHECK(mccl_copy_segments(copy_in.data(), (int)copy_in.size(), s));
+  {
+    std::ostringstream os;
+    os << "standing offers, " << in_place << " pieces read in place, " << staged << " through outboxes";
+    last_path_storage_ = os.str();
+    last_path_ = last_path_storage_.c_str();
+  }
+  if (verbose_) {
+    std::ostringstream os;
+    os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
+    std::cout << os.str() << std::endl;
+  }
+  if (pairwise_waits_now_) ++pairwise_wait_count_;
+  else ++enqueue_only_count_;
+  // 4. On the device: the rows, then the pulls.
+  flushImportTable(s);
+  const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
+  const int par = (int)(seq & 1);
+  MCCL_CHECK(mccl_rank_barrier_offers_each(bar_flags_.data(), W, me, epoch + 1, limit_us, status_dev_, row, expect, my_source,
+                                           offer_rows_[par].data(), import_table_, resolved_, s));
+  mccl_xsync_t sync{};
+  sync.words = bar_flags_.data();
+  sync.n = W;
+  sync.rank = me;
+  sync.done_epoch = epoch + 3;  // nobody's stream goes on before every rank has pulled what it gets from it
+  sync.done_counter = done_counter_;
+  sync.timeout_us = limit_us;
+  sync.status = status_dev_;
+  std::vector<mccl_segment_t> pulls;
+  std::vector<int> from;
+  for (int r = 0; r < W; ++r) {
+    if (!x.recv[(size_t)r]) continue;
+    pulls.push_back({nullptr, x.dst[(size_t)r], x.recv[(size_t)r]});
+    from.push_back(r);
+  }
+  MCCL_CHECK(mccl_copy_segments_sync_resolved(pulls.data(), from.data(), (int)pulls.size(), resolved_, 0u, &sync, s));
 }
 
 void ProcessGroupCCL::closeImports() {

@@ -28,7 +28,11 @@ void GroupShared::putEvent(hipEvent_t e) {
 std::string GroupShared::failureMessage() {
   if (status && (status[0] != 0 || status[2] != 0) && !failed.load(std::memory_order_acquire)) {
     std::ostringstream os;
-    if (status[0] != 0 && status[1] == MCCL_STATUS_UNMAPPED) {
+    if (status[0] != 0 && status[1] == MCCL_STATUS_MISMATCH) {
+      os << "ccl backend: alltoall: the piece rank " << (status[0] - 1) << " sends to this rank does not have the length this rank "
+            "expects (the split sizes of the ranks do not match: outputSplitSizes[r] here must equal rank r's inputSplitSizes "
+            "for this rank); the group cannot be used any more";
+    } else if (status[0] != 0 && status[1] == MCCL_STATUS_UNMAPPED) {
       os << "ccl backend: rank " << (status[0] - 1) << " offered a tensor in an allocation that this rank has not mapped "
             "(standing offers out of step); the group cannot be used any more";
     } else if (status[0] != 0) {
@@ -313,6 +317,10 @@ ProcessGroupCCL::~ProcessGroupCCL() {
     if (r != rank_ && peer_arena_[(size_t)r]) (void)hipIpcCloseMemHandle(peer_arena_[(size_t)r]);
   for (int s = 0; s < 2; ++s)
     if (stage_[s].base) (void)hipFree(stage_[s].base);
+  for (auto& in : outbox_in_)
+    if (in.base) (void)hipIpcCloseMemHandle(in.base);
+  for (auto& out : outbox_out_)
+    if (out.base) (void)hipFree(out.base);
   for (void* p : retired_) (void)hipFree(p);
   if (arena_) (void)hipFree(arena_);
   if (fork_event_) (void)hipEventDestroy(fork_event_);
@@ -426,7 +434,10 @@ void ProcessGroupCCL::ensureInit(int device) {
     fused_state_ = static_cast<char*>(arena_) + kArenaFusedStateOff;
     import_table_ = reinterpret_cast<mccl_import_table_t*>(static_cast<char*>(arena_) + kArenaImportTableOff);
     resolved_ = static_cast<char*>(arena_) + kArenaResolvedOff;
-    for (int sl = 0; sl < 2; ++sl) offer_slots_[sl].assign((size_t)size_, nullptr);
+    for (int sl = 0; sl < 2; ++sl) {
+      offer_slots_[sl].assign((size_t)size_, nullptr);
+      offer_rows_[sl].assign((size_t)size_, nullptr);
+    }
     for (int r = 0; r < size_; ++r) {
       char* base = nullptr;
       if (r == rank_) {
@@ -443,6 +454,7 @@ void ProcessGroupCCL::ensureInit(int device) {
       final_flags_[(size_t)r] = base + kArenaFinalOff;
       for (int sl = 0; sl < 2; ++sl) {
         offer_slots_[sl][(size_t)r] = base + kArenaOfferOff + (size_t)sl * kArenaOfferStride;
+        offer_rows_[sl][(size_t)r] = base + kArenaOfferRowOff + (size_t)sl * kArenaOfferRowStride;
         fused_flags_[sl][(size_t)r] = base + kArenaFusedFlagsOff + (size_t)sl * kArenaFusedFlagsStride;
         fused_stage_[sl][(size_t)r] = base + kArenaFusedStageOff + (size_t)sl * kArenaFusedStageStride + stageOffset(r);
       }
@@ -784,6 +796,11 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
     if (fusedFits(plan)) {
       say_path();
       launchFused(plan, s);
+      if (timed) phase_us_[3].push_back((float)us_since(t0));
+      return;
+    }
+    if (plan.standing_exchange.ok) {
+      runStandingExchange(plan, s, seq);
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }

@@ -43,6 +43,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <tuple>
 #include <vector>
 
 namespace mccl_pg {
@@ -278,6 +279,10 @@ class ProcessGroupCCL : public c10d::Backend {
       bool ok = false;
       void* buffer = nullptr;      // the tensor the peers read (allreduce, reduce_scatter: the input) or write (all_gather: the output)
       size_t bytes = 0;
+      // the storage (one block of the allocator) the buffer is part of: what is announced to the peers, so
+      // that a view somewhere inside a larger tensor is read in place like any other
+      const void* block = nullptr;
+      size_t block_bytes = 0;
       bool copy_in = false;        // a rank that stages copies its tensor into the staging buffer first ...
       bool copy_out = false;       // ... and / or the staging buffer back into it afterwards
       bool force_staged = false;   // this rank's tensors overlap in a way only a staged run handles (its own matter: the peers do not care)
@@ -288,6 +293,21 @@ class ProcessGroupCCL : public c10d::Backend {
       std::function<void(bool staged, const mccl_xsync_t& sync, const mccl_offer_t& mine, const void* buffer,
                          void* const* offers, const mccl_import_table_t* imports, hipStream_t s)> one_launch;
     } standing;
+    // An all-to-all on the same footing (runStandingExchange): a rank offers every reader its own piece.
+    // `ok` depends on the group alone; the sizes differ from rank to rank and decide nothing that more
+    // than the two ranks of a pair have to agree on.
+    struct StandingExchange {
+      bool ok = false;
+      std::vector<const void*> piece;  // where this rank's piece for rank d is
+      std::vector<size_t> send;        // its length
+      // the storage (one block of the allocator) the piece is part of: what can be announced to the peers
+      // (small ones are not worth it)
+      std::vector<const void*> block;
+      std::vector<size_t> block_bytes;
+      std::vector<void*> dst;          // where rank r's piece for this rank goes
+      std::vector<size_t> recv;        // its length
+      bool force_staged = false;       // input and output overlap: every piece is copied out of the way first
+    } standing_exchange;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
@@ -322,6 +342,12 @@ class ProcessGroupCCL : public c10d::Backend {
   bool standingFits(const Plan& plan) const;
   void runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void growStandingCapacity(size_t bytes);
+  bool standingExchangeFits() const;
+  bool standingExchangeNow(const std::vector<at::Tensor>& inputs, const std::vector<at::Tensor>& outputs);
+  void runStandingExchange(Plan& plan, hipStream_t s, uint64_t seq);
+  void growOutbox(int peer, int level);
+  void mapOutbox(int peer, int level);
+  bool acknowledgedBy(int peer, int entry, uint64_t gen, uint64_t seq) const;
   void scanPeerExports(uint64_t seq);
   bool allAcknowledged(int entry, uint64_t gen, uint64_t seq) const;
   void acknowledge(int owner, int entry, uint64_t gen, uint64_t from_seq);
@@ -411,7 +437,9 @@ class ProcessGroupCCL : public c10d::Backend {
   // 0 = none, 1 = work only, 2 = sync only, + 4 when allreduce is disabled (for tests of the parsing)
   int bisectMode() const { return (work_only_ ? 1 : 0) | (sync_only_ ? 2 : 0) | (disable_allreduce_ ? 4 : 0); }
   // (collectives that met at the rendezvous of the host threads, collectives that only enqueued)
-  std::pair<uint64_t, uint64_t> rendezvousCounts() const { return {rendezvous_count_, enqueue_only_count_}; }
+  // collectives that met at the host rendezvous; that only enqueued; that only enqueued after waiting for
+  // single peers (an all-to-all whose piece for or from that peer outgrew the buffer kept for it)
+  std::tuple<uint64_t, uint64_t, uint64_t> rendezvousCounts() const { return {rendezvous_count_, enqueue_only_count_, pairwise_wait_count_}; }
   std::string lastPath() const { return last_path_ ? last_path_ : ""; }
  private:
   unsigned waiting_cus_ = 128;  // what all ranks' waiting launches may hold together (MCCL_PG_WAITING_COMPUTE_UNITS)
@@ -484,6 +512,19 @@ class ProcessGroupCCL : public c10d::Backend {
   mccl_import_table_t* import_table_ = nullptr;  // device: the peers' allocations as this rank has mapped them
   void* resolved_ = nullptr;                // device: where the ranks' tensors of the collective under way are
   std::vector<void*> offer_slots_[2];       // rank r's offer slot, per parity of the collective
+  std::vector<void*> offer_rows_[2];        // rank r's row of offers (all-to-all), per parity of the collective
+  struct OutboxOut {                        // this rank's outbox for rank d (for itself: scratch nobody else maps)
+    void* base = nullptr;
+    int level = -1;
+  } outbox_out_[MCCL_OFFER_RANKS];
+  struct OutboxIn {                         // rank r's outbox for this rank, as mapped here
+    void* base = nullptr;
+    int level = -1;
+  } outbox_in_[MCCL_OFFER_RANKS];
+  uint64_t big_published_[MCCL_OFFER_RANKS] = {};  // the last BigPiece record written for rank d (its seq)
+  uint64_t pairwise_wait_count_ = 0;
+  unsigned pairwise_waits_now_ = 0;         // waits for single peers in the all-to-all under way
+  std::string last_path_storage_;
   std::vector<mccl_import_update_t> table_updates_;  // mappings that changed since the device table last heard
   uint64_t seen_live_[MCCL_OFFER_RANKS][MCCL_OFFER_ENTRIES] = {};  // peers' export entries as this rank last read them
   uint64_t last_offer_seq_[MCCL_OFFER_ENTRIES] = {};               // 1 + the last collective that offered the entry (0: none)

@@ -40,9 +40,9 @@ EXPORTS = (
     "mccl_alltoallv_n", "mccl_alltoallv_pull", "mccl_pack", "mccl_unpack",
     "mccl_query_launch", "mccl_set_tuning", "mccl_get_tuning",
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
-    "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_sync_offers",
+    "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_rank_barrier_offers_each", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_sync_offers",
     "mccl_reduce_sync_resolved", "mccl_reduce_sync_offers", "mccl_fanout_sync_resolved", "mccl_fanout_sync_offers", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
-    "mccl_copy_segments_sync", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
+    "mccl_copy_segments_sync", "mccl_copy_segments_sync_resolved", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
     "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
 
@@ -56,19 +56,20 @@ class XSync(ctypes.Structure):
 
 
 OFFER_RANKS, OFFER_ENTRIES, OFFER_STAGED, STATUS_UNMAPPED = 8, 32, 0xffffffff, 0xfffffffe
+OFFER_SLOTS, OFFER_SLOT_OUTBOX, STATUS_MISMATCH = 4, 2, 0xfffffffd
 
 
 class Offer(ctypes.Structure):
     """mccl_offer_t"""
     _fields_ = [("entry", ctypes.c_uint32), ("slot", ctypes.c_uint32), ("generation", ctypes.c_uint64),
-                ("offset", ctypes.c_uint64), ("reserved", ctypes.c_uint64)]
+                ("offset", ctypes.c_uint64), ("bytes", ctypes.c_uint64)]
 
 
 class ImportTable(ctypes.Structure):
     """mccl_import_table_t"""
     _fields_ = [("base", ctypes.c_uint64 * OFFER_ENTRIES * OFFER_RANKS),
                 ("generation", ctypes.c_uint64 * OFFER_ENTRIES * OFFER_RANKS),
-                ("staging", ctypes.c_uint64 * 2 * OFFER_RANKS)]
+                ("staging", ctypes.c_uint64 * OFFER_SLOTS * OFFER_RANKS)]
 
 
 class ImportUpdate(ctypes.Structure):
@@ -112,6 +113,7 @@ def lib():
     L.mccl_moe_combine.argtypes = [vp, vp, i32, vp, vp, vp, sz, i32, sz, i32, vp, vp]
     L.mccl_rank_barrier.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp]
     L.mccl_rank_barrier_offers.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp, vp, vp, vp, vp, vp]
+    L.mccl_rank_barrier_offers_each.argtypes = [vp, i32, i32, ctypes.c_uint64, ctypes.c_uint64, vp, vp, vp, vp, vp, vp, vp, vp]
     L.mccl_allreduce_sync_resolved.argtypes = [vp, sz, i32, i32, vp, vp]
     L.mccl_import_table_update.argtypes = [vp, vp, i32, vp]
     L.mccl_allreduce_sync_offers.argtypes = [sz, i32, i32, vp, vp, vp, vp, vp, vp]
@@ -122,6 +124,7 @@ def lib():
     L.mccl_allreduce_fused.argtypes = [vp, vp, sz, i32, i32, vp, vp, i32, i32, ctypes.c_uint32, ctypes.c_uint64, vp, ctypes.c_uint, vp]
     L.mccl_allreduce_fused_replayable.argtypes = [vp, vp, sz, i32, i32, vp, vp, sz, sz, vp, i32, i32, ctypes.c_uint64, vp, ctypes.c_uint, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
+    L.mccl_copy_segments_sync_resolved.argtypes = [vp, vp, i32, vp, ctypes.c_uint, vp, vp]
     L.mccl_fanout_sync.argtypes = [vp, vp, i32, sz, vp, vp]
     L.mccl_reduce_sync.argtypes = [vp, vp, sz, i32, i32, vp, vp]
     L.mccl_allreduce_sync.argtypes = [vp, sz, i32, i32, vp, vp]
