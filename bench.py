@@ -357,8 +357,40 @@ def _backend_rank(rank, world, store_path, cases, out_path, large=True):
     S = c5_split_matrix(torch, world, tokens, topk)
     a_in = torch.empty(tokens * topk, hidden, dtype=torch.bfloat16, device="cuda:0").normal_()
     a_out = torch.empty(int(S[:, rank].sum()), hidden, dtype=torch.bfloat16, device="cuda:0")
+    in_split, out_split = S[rank].tolist(), S[:, rank].tolist()
     res["c5_all_to_all_single_448MiB_bf16"] = timed(
-        lambda: dist.all_to_all_single(a_out, a_in, S[:, rank].tolist(), S[rank].tolist()), iters=5, warm=1)
+        lambda: dist.all_to_all_single(a_out, a_in, out_split, in_split), iters=5, warm=2)
+    # ... back to back, what the call costs the host, whether anybody's host thread waits for anybody, and
+    # how long the other ranks' calls take when rank 1 enters 50 ms late
+    try:
+        be = dist.distributed_c10d._get_default_group()._get_backend(torch.device("cuda"))
+        dist.barrier()
+        before = be._rendezvous_counts()
+        enq = []
+        t00 = time.perf_counter()
+        for _ in range(10):
+            t0 = time.perf_counter()
+            dist.all_to_all_single(a_out, a_in, out_split, in_split)
+            enq.append(time.perf_counter() - t0)
+        torch.cuda.synchronize()
+        b2b_us = (time.perf_counter() - t00) / 10 * 1e6
+        after = be._rendezvous_counts()
+        enq.sort()
+        dist.barrier()
+        if rank == 1:
+            time.sleep(0.05)
+        t0 = time.perf_counter()
+        w = dist.all_to_all_single(a_out, a_in, out_split, in_split, async_op=True)
+        call_us = (time.perf_counter() - t0) * 1e6
+        w.wait()
+        torch.cuda.synchronize()
+        res["host_side_of_all_to_all_single"] = {"c5_back_to_back_us": b2b_us, "c5_enqueue_us_p50": enq[5] * 1e6, "c5_calls": 10,
+                                                 "host_rendezvous_among_them": int(after[0] - before[0]),
+                                                 "waits_for_single_peers_among_them": int(after[2] - before[2]),
+                                                 "path": be._last_path(),
+                                                 "c5_call_us_on_rank_0_while_rank_1_is_50_ms_late": call_us}
+    except Exception as e:
+        res["host_side_of_all_to_all_single"] = {"error": repr(e)[:200]}
     del a_in, a_out
     # all_gather_into_tensor of 64 MiB per rank (an FSDP parameter gather): every rank writes its shard
     # into all eight outputs

@@ -128,10 +128,13 @@ __global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const S
   xsync_end(a.sync, gridDim.x);
 }
 
-// The same behind a barrier kernel that has resolved where the sources are (no opening wait).
+// The same behind a barrier kernel that has resolved where the sources are: no opening wait, and the
+// peers' data were complete before this kernel started, so the loads go through the caches like any
+// copy's (they start clean at a kernel boundary) and the launch has the plain copy's geometry --
+// one chunk per workgroup -- plus the closing count.
+template <bool STREAM>
 __global__ __launch_bounds__(kWave) void copy_segments_resolved_kernel(const SyncCopyArgs a) {
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // alignment of the sources unknown: anything may go through the caches
-  copy_segments_body<true, kCopyUnroll, false, true>(a.copy, this_wave<1>(), a.shared != 0, CopySources{a.src_table, a.src_rank});
+  copy_segments_body<false, kCopyUnroll, STREAM, true>(a.copy, this_wave<1>(), false, CopySources{a.src_table, a.src_rank});
   xsync_end(a.sync, gridDim.x, /*wrote_to_peers=*/false);
 }
 

@@ -1154,7 +1154,13 @@ int copy_segments_sync_impl(const mccl_segment_t* segs, const int* src_rank, con
   if (rc != MCCL_OK) return rc;
   if (resolved) {
     if (shape.packed) return fail(MCCL_ERR_INVALID_ARG, "a copy over resolved addresses runs as single wavefronts (max_compute_units 0)");
-    hipLaunchKernelGGL(copy_segments_resolved_kernel, dim3(grid), dim3(kWave), 0, (hipStream_t)stream, a);
+    // the plain copy's launch (launch_copy): a workgroup per chunk, its residency cap, its choice of stores
+    grid = (unsigned)std::min<uint64_t>(std::max<uint64_t>(chunks, 1), kMaxGridX);
+    const unsigned lds = (chunks > (uint64_t)cus * 4) ? lds_for_waves(g_tune[MCCL_TUNE_COPY_WAVES_PER_CU]) : 0;
+    long long stream_store = g_tune[MCCL_TUNE_COPY_STREAM_STORES];
+    if (stream_store != 1 && stream_store != 2) stream_store = chunks * kCopyChunk >= (uint64_t)g_tune[MCCL_TUNE_COPY_LARGE_MIN_BYTES] ? kCopyStreamLarge : 2;
+    if (stream_store == 1) hipLaunchKernelGGL(copy_segments_resolved_kernel<true>, dim3(grid), dim3(kWave), lds, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL(copy_segments_resolved_kernel<false>, dim3(grid), dim3(kWave), lds, (hipStream_t)stream, a);
   } else if (shape.packed) {
     static const unsigned per_cu = blocks_per_cu(copy_segments_sync_kernel<kPackedWaves>, kWave * kPackedWaves);
     if (a.sync.ready_epoch != 0) grid = std::min(grid, waiting_share(per_cu, (unsigned)cus, (unsigned)a.sync.n));
