@@ -470,6 +470,24 @@ int mccl_fanout_sync_offers(const void* src, size_t dst_offset, size_t bytes, in
 int mccl_copy_segments_sync_resolved(const mccl_segment_t* segs, const int* src_rank, int nseg, const void* resolved,
                                      unsigned flags, const mccl_xsync_t* sync, void* stream);
 
+/*
+ * The all-to-all of one rank as ONE launch (ccl::alltoallv at src/gpu/dpcpp_ccl.cpp:1447-1455): what
+ * mccl_rank_barrier_offers_each and mccl_copy_segments_sync_resolved do in two, plus the copies in
+ * front of them, on sync->max_compute_units compute units (ready_epoch, done_epoch and
+ * max_compute_units all set).  `stage` (at most MCCL_OFFER_RANKS segments) are the copies of this
+ * rank's pieces into its outboxes, for the pieces it does not offer in place; when they are in memory
+ * the launch publishes the row `mine` and the rank's ready epoch, waits for the peers', resolves the
+ * column addressed to this rank and carries out `pulls` (at most MCCL_OFFER_RANKS; sources as in
+ * mccl_copy_segments_sync_resolved, from what the launch has resolved).  Uses the word 128 bytes into
+ * sync->done_counter besides the counters of the closing wait.  For messages small enough that a
+ * launch costs more than the data; between rank processes that share a GPU every launch waits for
+ * its process's turn.  The two-launch form and this one may be mixed among the ranks of one
+ * collective.
+ */
+int mccl_alltoall_sync_offers(const mccl_segment_t* stage, int nstage, const mccl_segment_t* pulls, const int* src_rank, int npull,
+                              const mccl_xsync_t* sync, const mccl_offer_t* mine, const uint64_t* expect_bytes, const void* my_source,
+                              void* const* offers, const mccl_import_table_t* imports, void* stream);
+
 /* Generic segmented copy: every segment is copied byte-exactly; segments must not overlap
  * each other's destinations.  The building block of the copy collectives below. */
 int mccl_copy_segments(const mccl_segment_t* segs, int nseg, void* stream);

@@ -422,29 +422,42 @@ def offers_case(rank, world, queues, barrier):
         image = allocs[kind][off:off + total]
         if total:
             image.copy_(torch.from_numpy(np.concatenate(pieces[rank])).to(DEV))
+        one_launch = (call + rank) % 3 != 0  # the two forms mix among the ranks of one collective
         mine = (capi.Offer * world)()
+        stage = []
         for d in range(world):
             nb = int(S[rank][d])
             told = nb + 16 if (break_length and rank == 0 and d == 1) else nb
             if (call + rank + d) % 3 == 0:  # through the outbox for rank d
-                outbox[d * OUTBOX:d * OUTBOX + nb].copy_(image[int(displ[d]):int(displ[d]) + nb])
+                if one_launch:
+                    stage.append(capi.Segment(image.data_ptr() + int(displ[d]), outbox.data_ptr() + d * OUTBOX, nb))
+                else:
+                    outbox[d * OUTBOX:d * OUTBOX + nb].copy_(image[int(displ[d]):int(displ[d]) + nb])
                 mine[d] = capi.Offer(capi.OFFER_STAGED, capi.OFFER_SLOT_OUTBOX, 0, 0, told)
             else:
                 mine[d] = capi.Offer(entries[kind], 0, gen_of(rank, kind), off + int(displ[d]), told)
         expect = (ctypes.c_uint64 * world)(*[int(S[r][rank]) for r in range(world)])
         odispl = np.concatenate([[0], np.cumsum(S[:, rank])[:-1]])
         out = torch.full((int(S[:, rank].sum()) + 64,), 0xee, dtype=torch.uint8, device=DEV)
-        capi.check(L.mccl_rank_barrier_offers_each(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), mine, expect,
-                                                    image.data_ptr() + int(displ[rank]), rows[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
         segs = (capi.Segment * world)(*[capi.Segment(0, out.data_ptr() + int(odispl[r]), int(S[r][rank])) for r in range(world)])
         src_rank = (ctypes.c_int * world)(*range(world))
-        sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
-        capi.check(L.mccl_copy_segments_sync_resolved(segs, src_rank, world, resolved.data_ptr(), 0, ctypes.byref(sy), stream))
+        my_source = image.data_ptr() + int(displ[rank])
+        if one_launch:
+            stage_segs = (capi.Segment * max(1, len(stage)))(*stage)
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 4 * call + 1, 4 * call + 3, counter.data_ptr(), 5_000_000,
+                            st.data_ptr(), (16, 2)[call % 2], 0)
+            capi.check(L.mccl_alltoall_sync_offers(stage_segs, len(stage), segs, src_rank, world, ctypes.byref(sy), mine, expect, my_source,
+                                                   rows[call & 1], table.data_ptr(), stream))
+        else:
+            capi.check(L.mccl_rank_barrier_offers_each(flags, world, rank, 4 * call + 1, 5_000_000, st.data_ptr(), mine, expect,
+                                                        my_source, rows[call & 1], table.data_ptr(), resolved.data_ptr(), stream))
+            sy = capi.XSync(ctypes.cast(flags, ctypes.c_void_p), world, rank, 0, 4 * call + 3, counter.data_ptr(), 5_000_000, st.data_ptr(), 0, 0)
+            capi.check(L.mccl_copy_segments_sync_resolved(segs, src_rank, world, resolved.data_ptr(), 0, ctypes.byref(sy), stream))
         want = np.concatenate([pieces[r][rank] for r in range(world)] + [np.full(64, 0xee, dtype=np.uint8)])
         return out, want, S
 
     pending = []
-    for i in range(6):
+    for i in range(9):
         call += 1
         out, want, S = alltoall_round(call, seed=1000 + i)
         pending.append((out, want, ("alltoall", i, S.tolist())))

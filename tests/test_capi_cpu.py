@@ -195,6 +195,22 @@ def test_offer_entry_points_reject_bad_arguments_without_a_device(mccl):
     assert pull(behind) == -1 and "null pointer" in err()
     segs[1] = capi.Segment(0, 0xb0000, 4096)
     assert pull(behind, ranks=(ctypes.c_int * 2)(0, -1)) == -1 and "null pointer" in err()  # a plain address must not be null
+    # the same as one launch
+    copies = (capi.Segment * 1)(capi.Segment(0xc0000, 0xd0000, 4096))
+    segs[1] = capi.Segment(0x100, 0xb0000, 4096)
+    rows[1] = capi.Offer(capi.OFFER_STAGED, capi.OFFER_SLOT_OUTBOX, 0, 0, 64)
+    a2a = lambda sy, stage=copies, ns=1, mine=rows, exp=expect, offers=two, imports=tab: L.mccl_alltoall_sync_offers(
+        stage, ns, segs, from_, 2, ctypes.byref(sy), mine, exp, vp(0x1000), offers, imports, None)
+    assert a2a(behind) == -1 and "max_compute_units" in err()
+    assert a2a(opening) == -1 and "max_compute_units" in err()
+    assert a2a(one, mine=None) == -1 and "null" in err()
+    assert a2a(one, exp=None) == -1 and "null" in err()
+    assert a2a(one, imports=vp(0x40004)) == -1 and "8-byte" in err()
+    assert a2a(one, ns=9) == -1 and "0 to 8 segments" in err()
+    assert a2a(one, stage=(capi.Segment * 1)(capi.Segment(0, 0xd0000, 4096))) == -1 and "outboxes: segment 0 has a null pointer" in err()
+    assert a2a(one, offers=capi.ptr_table([0x10000, 0x20004])) == -1 and "offer pointer 1" in err()
+    rows[0] = capi.Offer(40, 0, 7, 0, 64)
+    assert a2a(one) == -1 and "offer 0 names entry 40" in err()
     # the small allreduce with its epoch on the device
     stage = capi.ptr_table([0x100000, 0x300000])
     tf = capi.ptr_table([0x500000, 0x510000])

@@ -156,7 +156,7 @@ def scan_hints(asm_path):
 
 
 _WAITING_KERNEL = re.compile(r"(xrank_reduce_kernel|copy_segments_sync_kernel|fanout_sync_kernel|fanout_indirect_kernel|allreduce_fused_kernel|"
-                             r"rank_barrier_kernel|rank_barrier_offers_kernel|rank_barrier_offers_each_kernel|copy_segments_resolved_kernel)")
+                             r"rank_barrier_kernel|rank_barrier_offers_kernel|rank_barrier_offers_each_kernel|copy_segments_resolved_kernel|exchange_offers_kernel)")
 _MAX_VGPRS_OF_WAITING_KERNELS = 128
 
 

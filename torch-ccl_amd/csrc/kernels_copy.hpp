@@ -39,10 +39,19 @@ struct SyncCopyArgs {
   int8_t src_rank[kMaxSegs];
 };
 
-// Where the sources of the segments are when the host does not know.
+// Where the sources of the segments are when the host does not know: a table in memory (INDIRECT 1),
+// or lane r of the wavefront holds rank r's address (INDIRECT 2).
 struct CopySources {
   const uint64_t* table;
   const int8_t* rank;
+  uint64_t held;
+};
+
+// A copy of at most MCCL_OFFER_RANKS segments: the same as CopyArgs to the kernels, an eighth of it to the launch.
+struct LeanCopyArgs {
+  CopySeg seg[MCCL_OFFER_RANKS];
+  uint32_t chunk_prefix[MCCL_OFFER_RANKS + 1];
+  int nseg;
 };
 
 // Segmented copy.  One wavefront per workgroup, one 2 KiB chunk per wavefront, chunks
@@ -55,9 +64,9 @@ struct CopySources {
 // UNROLL: 16-byte vectors per lane per chunk (chunk = 64 x 16 x UNROLL bytes; the host computes
 // the segment geometry for the same value).  STREAM: full chunks are written through past the
 // caches (`sc1`) instead of with the non-temporal hint.
-template <bool COHERENT, int UNROLL, bool STREAM, bool INDIRECT = false>
-__device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave& w, bool shared_sources = false,
-                                                   const CopySources from = CopySources{nullptr, nullptr}) {
+template <bool COHERENT, int UNROLL, bool STREAM, int INDIRECT = 0, typename ARGS = CopyArgs>
+__device__ __forceinline__ void copy_segments_body(const ARGS& a, const Wave& w, bool shared_sources = false,
+                                                   const CopySources from = CopySources{nullptr, nullptr, 0}) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
   const uint32_t total = a.chunk_prefix[a.nseg];
   for (uint32_t chunk = w.index; chunk < total; chunk += w.count) {
@@ -74,12 +83,19 @@ __device__ __forceinline__ void copy_segments_body(const CopyArgs& a, const Wave
     const uint32_t t = w.lane;
     const char* src = a.seg[lo].src;
     char* dst = a.seg[lo].dst;
-    if constexpr (INDIRECT) {
+    if constexpr (INDIRECT != 0) {
       const int r = from.rank[lo];  // uniform
       if (r >= 0) {
-        // written by the kernel in front on the stream, constant while this one runs: a scalar load
-        const uint64_t base = ((const __attribute__((address_space(4))) uint64_t*)from.table)[r];
-        if (base == 0) continue;  // not resolved: the barrier in front has reported it
+        uint64_t base;
+        if constexpr (INDIRECT == 1) {
+          // written by the kernel in front on the stream, constant while this one runs: a scalar load
+          base = ((const __attribute__((address_space(4))) uint64_t*)from.table)[r];
+        } else {
+          const uint32_t lo32 = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)from.held, r);
+          const uint32_t hi32 = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(from.held >> 32), r);
+          base = ((uint64_t)hi32 << 32) | lo32;
+        }
+        if (base == 0) continue;  // not resolved: whoever resolved it has reported why
         src = (const char*)(base + (uint64_t)(uintptr_t)src);
       }
     }
@@ -134,7 +150,75 @@ __global__ __launch_bounds__(kWave * WPG) void copy_segments_sync_kernel(const S
 // one chunk per workgroup -- plus the closing count.
 template <bool STREAM>
 __global__ __launch_bounds__(kWave) void copy_segments_resolved_kernel(const SyncCopyArgs a) {
-  copy_segments_body<false, kCopyUnroll, STREAM, true>(a.copy, this_wave<1>(), false, CopySources{a.src_table, a.src_rank});
+  copy_segments_body<false, kCopyUnroll, STREAM, 1>(a.copy, this_wave<1>(), false, CopySources{a.src_table, a.src_rank, 0});
+  xsync_end(a.sync, gridDim.x, /*wrote_to_peers=*/false);
+}
+
+// An all-to-all between rank processes as ONE launch, on few compute units (every launch of a process
+// waits for its turn at the dispatcher, which at small sizes costs more than the data).  The pieces
+// this rank does not offer in place go into its outboxes first, by all workgroups; when the last
+// of them is there -- counted in a word of the rank's counter block, which only this launch touches
+// then -- the first workgroup publishes the rank's row of offers and its flag.  Every workgroup waits
+// for all flags, this rank's own included (the pulls may write where the copies read: an output that
+// overlaps the input), every wavefront resolves the column addressed to this rank (lane r: rank r's
+// piece) and they pull.  The outboxes are written and read past the caches of the two kernels, which
+// run at the same time.
+struct ExchangeArgs {
+  LeanCopyArgs stage;                  // this rank's pieces -> its outboxes
+  LeanCopyArgs pull;                   // the peers' pieces -> this rank's output; src = offset from the resolved address
+  int8_t src_rank[MCCL_OFFER_RANKS];   // of the pull segments (< 0: src is an address as it stands)
+  uint64_t* row[MCCL_OFFER_RANKS];
+  uint64_t mine[MCCL_OFFER_RANKS][4];
+  uint64_t expect[MCCL_OFFER_RANKS];
+  uint64_t my_source;
+  const mccl_import_table_t* imports;
+  uint32_t* staged_count;              // zero between launches
+  XSync sync;
+};
+
+template <int WPG>
+__global__ __launch_bounds__(kWave * WPG) void exchange_offers_kernel(const ExchangeArgs a) {
+  const Wave w = this_wave<WPG>();
+  const int n = a.sync.n, me = a.sync.rank;
+  const bool staging = a.stage.nseg != 0;  // (nothing to copy: the row and the flag go out at once, as in every other one-launch form)
+  if (staging) {
+    copy_segments_body<false, kCopyUnroll, false, 0, LeanCopyArgs>(a.stage, w);
+    // what this workgroup has put into the outboxes is in memory before it counts itself in
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    __syncthreads();
+    if (threadIdx.x == 0) (void)__hip_atomic_fetch_add(a.staged_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (staging) {
+      const uint64_t t0 = wall_clock64();
+      while (__hip_atomic_load(a.staged_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != gridDim.x) {
+        if (wall_clock64() - t0 > a.sync.limit_ticks) {  // (a workgroup of this launch never got there: reported as this rank itself)
+          report_late(a.sync.status, me, (uint32_t)a.sync.ready_epoch);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the flag below follows what the counted workgroups did
+      __hip_atomic_store(a.staged_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    }
+    uint64_t* row = a.row[me];
+#pragma unroll
+    for (int k = 0; k < MCCL_OFFER_RANKS; ++k) {
+      if (k < n) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) __hip_atomic_store(row + 4 * k + i, a.mine[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+    __hip_atomic_store(a.sync.word[me], a.sync.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  if (xsync_begin(a.sync, /*publish=*/false)) {  // (publish = false also makes it wait for this rank's own flag)
+    uint64_t where = a.my_source;
+    const int r = (int)w.lane;
+    if (r >= n) where = 0;
+    else if (r != me) where = resolve_piece(a.row[r] + 4 * me, a.expect[r], a.imports, r, a.sync.status);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // outboxes, heads and partial chunks go through the caches
+    copy_segments_body<true, kCopyUnroll, false, 2, LeanCopyArgs>(a.pull, w, false, CopySources{nullptr, a.src_rank, where});
+  }
   xsync_end(a.sync, gridDim.x, /*wrote_to_peers=*/false);
 }
 

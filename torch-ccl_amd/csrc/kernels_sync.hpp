@@ -202,15 +202,21 @@ constexpr uint32_t kDoneGroups = 16;
 constexpr uint32_t kDoneStride = 64;
 static_assert(kDoneGroups * kDoneStride * 4 <= MCCL_SYNC_COUNTER_BYTES, "counters must fit the block the caller provides");
 static_assert(kDoneGroups <= kWave, "one lane of the watching wavefront per counter");
+// A word of the same block that the closing count leaves alone (128 bytes into the first counter's
+// 256): counts the workgroups of a one-launch all-to-all whose share of the copy-in is done.
+constexpr uint32_t kStagedCountWord = 32;
 
 // Returns false (for the whole wavefront) when a peer did not arrive in time.
-__device__ __forceinline__ bool xsync_begin(const XSync& x) {
+// publish = false: the kernel stores this rank's word itself, once something else has happened first.
+__device__ __forceinline__ bool xsync_begin(const XSync& x, bool publish = true) {
   if (x.ready_epoch == 0) return true;  // the caller has ordered the ranks on the host
   const int lane = threadIdx.x & (kWave - 1);
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
+  if (publish && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
     __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   bool ok = true;
-  if (lane < x.n && lane != x.rank) {
+  // (publish = false: this rank's own word says that all its workgroups are through with what comes
+  // before -- waited for like the peers')
+  if (lane < x.n && (lane != x.rank || !publish)) {
     ok = wait_flag64(x.word[lane], x.ready_epoch, x.limit_ticks);
     if (!ok) report_late(x.status, lane, (uint32_t)x.ready_epoch);
   }
@@ -348,6 +354,22 @@ struct OfferEachArgs {
   int rank;
 };
 
+// Where rank r's piece for this rank is, from r's offer for this rank (read after r's flag has
+// arrived): null when it is empty, not of the expected length, or in memory this rank has not mapped
+// (the latter two reported).
+__device__ __forceinline__ uint64_t resolve_piece(const uint64_t* slot, uint64_t expect, const mccl_import_table_t* imports, int r,
+                                                  uint32_t* status) {
+  const uint64_t bytes = __hip_atomic_load(slot + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (bytes != expect) {
+    report_late(status, r, MCCL_STATUS_MISMATCH);
+    return 0;
+  }
+  if (bytes == 0) return 0;
+  const uint64_t where = resolve_offer(slot, imports, r);
+  if (!where) report_late(status, r, MCCL_STATUS_UNMAPPED);
+  return where;
+}
+
 __global__ __launch_bounds__(kWave) void rank_barrier_offers_each_kernel(const OfferEachArgs a) {
   const int lane = threadIdx.x;
   if (lane == 0) {
@@ -370,14 +392,7 @@ __global__ __launch_bounds__(kWave) void rank_barrier_offers_each_kernel(const O
       report_late(a.status, lane, (uint32_t)a.epoch);
     } else {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the offer is read after the flag
-      const uint64_t* slot = a.row[lane] + 4 * a.rank;
-      const uint64_t bytes = __hip_atomic_load(slot + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      if (bytes != a.expect[lane]) {
-        report_late(a.status, lane, MCCL_STATUS_MISMATCH);
-      } else if (bytes != 0) {
-        where = resolve_offer(slot, a.imports, lane);
-        if (!where) report_late(a.status, lane, MCCL_STATUS_UNMAPPED);
-      }
+      where = resolve_piece(a.row[lane] + 4 * a.rank, a.expect[lane], a.imports, lane, a.status);
     }
   }
   a.resolved[lane] = where;

@@ -1183,6 +1183,7 @@ int mccl_copy_segments_sync(const mccl_segment_t* segs, int nseg, unsigned flags
   return copy_segments_sync_impl(segs, nullptr, nullptr, nseg, flags, sync, stream);
 }
 
+
 int mccl_copy_segments_sync_resolved(const mccl_segment_t* segs, const int* src_rank, int nseg, const void* resolved,
                                      unsigned flags, const mccl_xsync_t* sync, void* stream) {
   if (!resolved) return fail(MCCL_ERR_INVALID_ARG, "address table is null");
@@ -1437,6 +1438,98 @@ int mccl_fanout_sync_offers(const void* src, size_t dst_offset, size_t bytes, in
                             const mccl_import_table_t* imports, void* stream) {
   const OfferExchange ox{mine, my_buffer, offers, imports};
   return fanout_sync_indirect(src, nullptr, &ox, dst_offset, bytes, skip_own, sync, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+// The kernels' view of at most MCCL_OFFER_RANKS segments; src_is_offset[i]: segs[i].src is no address.
+int fill_lean_copy(const mccl_segment_t* segs, const int* src_rank, int nseg, const char* what, LeanCopyArgs* out, int8_t* ranks, int n,
+                   uint64_t* total_chunks) {
+  if (nseg < 0 || nseg > MCCL_OFFER_RANKS) return fail(MCCL_ERR_INVALID_ARG, "%s: 0 to %d segments, got %d", what, MCCL_OFFER_RANKS, nseg);
+  if (nseg && !segs) return fail(MCCL_ERR_INVALID_ARG, "%s: segment table is null", what);
+  int m = 0;
+  uint64_t chunks = 0;
+  out->chunk_prefix[0] = 0;
+  for (int i = 0; i < nseg; ++i) {
+    const mccl_segment_t& sg = segs[i];
+    if (sg.bytes == 0) continue;
+    const int from = src_rank ? src_rank[i] : -1;
+    if (from >= n) return fail(MCCL_ERR_INVALID_ARG, "%s: segment %d reads from rank %d of %d", what, i, from, n);
+    if ((from < 0 && !sg.src) || !sg.dst) return fail(MCCL_ERR_INVALID_ARG, "%s: segment %d has a null pointer", what, i);
+    CopySeg cs;
+    cs.src = (const char*)sg.src;
+    cs.dst = (char*)sg.dst;
+    cs.pad_ = 0;
+    size_t head = (128u - (unsigned)((uintptr_t)sg.dst & 127u)) & 127u;
+    if (head > sg.bytes) head = sg.bytes;
+    const size_t body = sg.bytes - head;
+    const uint64_t nfull = body / kCopyChunk;
+    cs.head = (uint32_t)head;
+    cs.last = (uint32_t)(body % kCopyChunk);
+    uint64_t c = nfull + (cs.last ? 1 : 0);
+    if (c == 0) c = 1;
+    if (nfull > 0xf0000000ull || chunks + c > kMaxChunks) return fail(MCCL_ERR_INVALID_ARG, "%s: segment %d too large for one launch", what, i);
+    cs.nfull = (uint32_t)nfull;
+    if (ranks) ranks[m] = (int8_t)(from < 0 ? -1 : from);
+    out->seg[m] = cs;
+    chunks += c;
+    out->chunk_prefix[++m] = (uint32_t)chunks;
+  }
+  out->nseg = m;
+  *total_chunks += chunks;
+  return MCCL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mccl_alltoall_sync_offers(const mccl_segment_t* stage, int nstage, const mccl_segment_t* pulls, const int* src_rank, int npull,
+                              const mccl_xsync_t* sync, const mccl_offer_t* mine, const uint64_t* expect_bytes, const void* my_source,
+                              void* const* offers, const mccl_import_table_t* imports, void* stream) {
+  ExchangeArgs a;
+  memset(&a, 0, sizeof(a));
+  int rc = fill_xsync(sync, &a.sync);
+  if (rc != MCCL_OK) return rc;
+  rc = check_indirect_sync(sync, /*one_launch=*/true);
+  if (rc != MCCL_OK) return rc;
+  const int n = a.sync.n;
+  if (n > MCCL_OFFER_RANKS) return fail(MCCL_ERR_UNSUPPORTED, "an all-to-all with offers takes 1 to %d ranks, got %d", MCCL_OFFER_RANKS, n);
+  if (!mine || !expect_bytes || !offers || !imports) return fail(MCCL_ERR_INVALID_ARG, "offers, expected lengths, offer table or import table is null");
+  if ((uintptr_t)imports % 8) return fail(MCCL_ERR_INVALID_ARG, "import table is not 8-byte aligned");
+  if (npull > 0 && !src_rank) return fail(MCCL_ERR_INVALID_ARG, "source rank table is null");
+  uint64_t chunks = 0;
+  rc = fill_lean_copy(stage, nullptr, nstage, "copies into the outboxes", &a.stage, nullptr, n, &chunks);
+  if (rc != MCCL_OK) return rc;
+  memset(a.src_rank, 0xff, sizeof(a.src_rank));
+  rc = fill_lean_copy(pulls, src_rank, npull, "pulls", &a.pull, a.src_rank, n, &chunks);
+  if (rc != MCCL_OK) return rc;
+  for (int r = 0; r < n; ++r) {
+    if (!offers[r]) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is null", r);
+    if ((uintptr_t)offers[r] % 8) return fail(MCCL_ERR_INVALID_ARG, "offer pointer %d is not 8-byte aligned", r);
+    const mccl_offer_t& o = mine[r];
+    if (o.entry != MCCL_OFFER_STAGED && o.entry >= MCCL_OFFER_ENTRIES) return fail(MCCL_ERR_INVALID_ARG, "offer %d names entry %u of %d", r, o.entry, MCCL_OFFER_ENTRIES);
+    if (o.entry == MCCL_OFFER_STAGED && o.slot >= MCCL_OFFER_SLOTS) return fail(MCCL_ERR_INVALID_ARG, "offer %d names staging buffer %u of %d", r, o.slot, MCCL_OFFER_SLOTS);
+    a.row[r] = (uint64_t*)offers[r];
+    offer_words(o, a.mine[r]);
+    a.expect[r] = expect_bytes[r];
+  }
+  a.my_source = (uint64_t)(uintptr_t)my_source;
+  a.imports = imports;
+  a.staged_count = a.sync.done_count + kStagedCountWord;
+  const XShape shape = xrank_shape(chunks, sync);
+  if (!shape.packed) return fail(MCCL_ERR_INVALID_ARG, "the one-launch all-to-all with offers runs packed (max_compute_units)");
+  int cus = 0;
+  rc = device_cus(&cus);
+  if (rc != MCCL_OK) return rc;
+  static const unsigned per_cu = blocks_per_cu(exchange_offers_kernel<kPackedWaves>, kWave * kPackedWaves);
+  const unsigned grid = std::min(shape.groups, waiting_share(per_cu, (unsigned)cus, (unsigned)n));
+  hipLaunchKernelGGL(exchange_offers_kernel<kPackedWaves>, dim3(grid), dim3(kWave * kPackedWaves), 0, (hipStream_t)stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MCCL_ERR_HIP, "all-to-all kernel launch failed: %s", hipGetErrorString(e));
+  return MCCL_OK;
 }
 
 size_t mccl_allreduce_sync_shard(size_t count, int n) {

@@ -594,7 +594,15 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
     copy_in.push_back({x.piece[(size_t)me], outbox_out_[me].base, x.send[(size_t)me]});
     my_source = outbox_out_[me].base;
   }
-  if (!copy_in.empty()) MCCL_CHECK(mccl_copy_segments(copy_in.data(), (int)copy_in.size(), s));
+  // Little to move: ONE launch on this rank's share of half of the compute units, which copies into the
+  // outboxes, carries the row and pulls -- with several processes on the GPU every launch waits for
+  // its turn at the dispatcher, which costs more than the data at these sizes.  (A matter of this
+  // rank alone: the two forms look the same to the peers.)
+  size_t moved = 0;
+  for (const auto& sg : copy_in) moved += sg.bytes;
+  for (int r = 0; r < W; ++r) moved += x.recv[(size_t)r];
+  const bool one_launch = 2.0 * (double)moved <= (double)compact_max_;
+  if (!one_launch && !copy_in.empty()) MCCL_CHECK(mccl_copy_segments(copy_in.data(), (int)copy_in.size(), s));
   {
     std::ostringstream os;
     os << "standing offers, " << in_place << " pieces read in place, " << staged << " through outboxes";
@@ -612,8 +620,9 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
   flushImportTable(s);
   const uint64_t limit_us = (uint64_t)waitLimit(false).count() * 1000ull;
   const int par = (int)(seq & 1);
-  MCCL_CHECK(mccl_rank_barrier_offers_each(bar_flags_.data(), W, me, epoch + 1, limit_us, status_dev_, row, expect, my_source,
-                                           offer_rows_[par].data(), import_table_, resolved_, s));
+  if (!one_launch)
+    MCCL_CHECK(mccl_rank_barrier_offers_each(bar_flags_.data(), W, me, epoch + 1, limit_us, status_dev_, row, expect, my_source,
+                                             offer_rows_[par].data(), import_table_, resolved_, s));
   mccl_xsync_t sync{};
   sync.words = bar_flags_.data();
   sync.n = W;
@@ -629,7 +638,14 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
     pulls.push_back({nullptr, x.dst[(size_t)r], x.recv[(size_t)r]});
     from.push_back(r);
   }
-  MCCL_CHECK(mccl_copy_segments_sync_resolved(pulls.data(), from.data(), (int)pulls.size(), resolved_, 0u, &sync, s));
+  if (one_launch) {
+    sync.ready_epoch = epoch + 1;
+    sync.max_compute_units = std::max(1u, waiting_cus_ / (unsigned)W);
+    MCCL_CHECK(mccl_alltoall_sync_offers(copy_in.data(), (int)copy_in.size(), pulls.data(), from.data(), (int)pulls.size(), &sync, row, expect,
+                                         my_source, offer_rows_[par].data(), import_table_, s));
+  } else {
+    MCCL_CHECK(mccl_copy_segments_sync_resolved(pulls.data(), from.data(), (int)pulls.size(), resolved_, 0u, &sync, s));
+  }
 }
 
 void ProcessGroupCCL::closeImports() {

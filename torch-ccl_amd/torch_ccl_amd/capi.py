@@ -42,7 +42,7 @@ EXPORTS = (
     "mccl_gather_rows", "mccl_moe_dispatch_n", "mccl_moe_combine",
     "mccl_rank_barrier", "mccl_rank_barrier_offers", "mccl_rank_barrier_offers_each", "mccl_import_table_update", "mccl_allreduce_sync_resolved", "mccl_allreduce_sync_offers",
     "mccl_reduce_sync_resolved", "mccl_reduce_sync_offers", "mccl_fanout_sync_resolved", "mccl_fanout_sync_offers", "mccl_allreduce_fused", "mccl_allreduce_fused_replayable", "mccl_fanout_sync",
-    "mccl_copy_segments_sync", "mccl_copy_segments_sync_resolved", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
+    "mccl_copy_segments_sync", "mccl_copy_segments_sync_resolved", "mccl_alltoall_sync_offers", "mccl_reduce_sync", "mccl_allreduce_sync_shard", "mccl_allreduce_sync",
     "mccl_route_counts", "mccl_route_counts_noalloc", "mccl_placement_check",
 )
 
@@ -125,6 +125,7 @@ def lib():
     L.mccl_allreduce_fused_replayable.argtypes = [vp, vp, sz, i32, i32, vp, vp, sz, sz, vp, i32, i32, ctypes.c_uint64, vp, ctypes.c_uint, ctypes.c_uint, vp]
     L.mccl_copy_segments_sync.argtypes = [vp, i32, ctypes.c_uint, vp, vp]
     L.mccl_copy_segments_sync_resolved.argtypes = [vp, vp, i32, vp, ctypes.c_uint, vp, vp]
+    L.mccl_alltoall_sync_offers.argtypes = [vp, i32, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp]
     L.mccl_fanout_sync.argtypes = [vp, vp, i32, sz, vp, vp]
     L.mccl_reduce_sync.argtypes = [vp, vp, sz, i32, i32, vp, vp]
     L.mccl_allreduce_sync.argtypes = [vp, sz, i32, i32, vp, vp]
