@@ -1399,6 +1399,32 @@ def standing_alltoall_big_case(pg, rank, world):
     pg.barrier().wait()
 
 
+def alltoall_mismatch_case(pg, rank, world):
+    """Split sizes that do not match between two ranks (rank 1 expects less from rank 0 than rank 0
+    sends): with the offers on the device nobody's host thread can notice, so the reader's kernel does --
+    it leaves that piece alone, reports, and rank 1's next call raises with the reason."""
+    rows, hidden = 64, 256
+    S = np.full((world, world), rows)
+    out_splits = S[:, rank].tolist()
+    if rank == 1:
+        out_splits[0] = rows - 8
+    inp = torch.full((rows * world, hidden), float(rank + 1), device=DEV)
+    out = torch.zeros(sum(out_splits), hidden, device=DEV)
+    pg.alltoall_base(out, inp, out_splits, S[rank].tolist()).wait()
+    torch.cuda.synchronize()
+    if rank == 1:
+        assert float(out[:rows - 8].abs().max()) == 0.0  # the piece of the wrong length was not copied
+        assert float(out[rows - 8:rows - 8 + rows].min()) == 2.0  # its own piece was
+        try:
+            pg.allreduce([inp], c10d.AllreduceOptions()).wait()
+            raise AssertionError("the call after a mismatch returned")
+        except RuntimeError as e:
+            assert "does not have the length this rank expects" in str(e) and "rank 0" in str(e), str(e)
+    else:
+        for r in range(world):
+            assert float(out[r * rows:(r + 1) * rows].min()) == float(r + 1) == float(out[r * rows:(r + 1) * rows].max()), r
+
+
 def graph_capture_case(rank, world):
     """A decode loop from a HIP graph: every rank records K dist.all_reduce of the 256 KiB bf16
     message with a small kernel of the caller's between them, then replays the graph with fresh
@@ -1627,6 +1653,8 @@ def run_rank(rank, world, store_path, mode):
         standing_offer_cases(pg, rank, world)
     elif mode == "standing_alltoall":
         standing_alltoall_cases(pg, rank, world)
+    elif mode == "alltoall_mismatch":
+        alltoall_mismatch_case(pg, rank, world)
     elif mode == "standing_big":
         standing_alltoall_big_case(pg, rank, world)
     else:

@@ -142,6 +142,10 @@ def test_all_to_all_with_offers_exchanged_on_the_device(world):
     _spawn(world, "standing_alltoall")
 
 
+def test_all_to_all_with_split_sizes_that_do_not_match_is_reported():
+    _spawn(3, "alltoall_mismatch")
+
+
 def test_all_to_all_pieces_larger_than_any_outbox_are_read_in_place(monkeypatch):
     monkeypatch.setenv("MCCL_PG_STANDING_MAX_BYTES", str(2 << 20))
     _spawn(4, "standing_big")
