@@ -549,15 +549,16 @@ def large_message_case(pg, rank, world):
 
 
 def missing_rank_case(pg, rank, world):
-    """Rank 1 never joins the second collective: the others must get an error, not hang.  (An
-    all_gather into a list of tensors, 2 MiB per rank: a collective whose host threads meet first in
-    every mode -- where its output tensors are is published per call -- so the call itself raises.)"""
+    """Rank 1 never joins the second collective: the others must get an error, not hang.  (A
+    reduce_scatter from a list of tensors, 2 MiB each: a collective whose host threads meet first in
+    every mode -- the list is packed into the staging buffer, whose handle is published per call --
+    so the call itself raises.)"""
     t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
     try:
-        pg.allgather([[torch.empty(1 << 19, device=DEV) for _ in range(world)]], [t]).wait()
+        pg.reduce_scatter([t], [[torch.ones(1 << 19, device=DEV) for _ in range(world)]], c10d.ReduceScatterOptions()).wait()
         raise AssertionError("collective with a missing rank returned")
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
@@ -1354,6 +1355,42 @@ def standing_alltoall_cases(pg, rank, world):
         pg.alltoall(outs, ins).wait()
         for r in range(world):
             assert np.array_equal(bits(outs[r]), bits(host[r][rank])), ("alltoall list", i, r, pg._last_path())
+    # all_gather into a list (every rank's size is known to all from the output list: sizes may differ) and
+    # broadcast: the same piece for every reader, staged through the rank's staging buffer when it is
+    # not offered in place
+    for i in range(4):
+        sizes = [((3 << 18) + 1000 * r + 7) * (1 if i % 2 else 3) for r in range(world)]  # floats: 3 and 9 MiB and a bit
+        sizes[world - 1] = 0 if i == 2 else sizes[world - 1]
+        host = [rank_buffer(sizes[r], torch.float32, r, seed=820 + i) for r in range(world)]
+        mine_t = host[rank].to(DEV)
+        outs = [torch.zeros(sizes[r], device=DEV) for r in range(world)]
+        if i == 3:
+            outs[rank] = mine_t  # gathered into the very tensor it comes from
+        before = pg._rendezvous_counts()
+        pg.allgather([outs], [mine_t]).wait()
+        after = pg._rendezvous_counts()
+        assert after[0] == before[0] or i == 0, (i, before, after)  # (the first one enlarges the staging buffers: the ranks meet)
+        for r in range(world):
+            assert np.array_equal(bits(outs[r]), bits(host[r])), ("allgather list", i, r, pg._last_path())
+    small = [torch.zeros(100 + r, dtype=torch.int16, device=DEV) for r in range(world)]
+    pg.allgather([small], [torch.full((100 + rank,), rank + 1, dtype=torch.int16, device=DEV)]).wait()
+    for r in range(world):
+        assert int(small[r].min()) == r + 1 == int(small[r].max()), ("allgather list, small", r)
+    keep = torch.empty((5 << 20) + 3, dtype=torch.uint8, device=DEV)
+    for i in range(6):
+        root = i % world
+        n = ((5 << 20) + 3) if i < 4 else 4099
+        want = rank_buffer(n, torch.uint8, root, seed=840 + i)
+        t = keep[:n] if i % 2 else torch.empty(n, dtype=torch.uint8, device=DEV)
+        t.copy_(want if rank == root else torch.zeros(n, dtype=torch.uint8))
+        opts = c10d.BroadcastOptions()
+        opts.rootRank = root
+        opts.rootTensor = 0
+        before = pg._rendezvous_counts()
+        pg.broadcast([t], opts).wait()
+        after = pg._rendezvous_counts()
+        assert after[0] == before[0], (i, before, after)
+        assert np.array_equal(bits(t), bits(want)), ("broadcast", i, root, pg._last_path())
     # a rank that comes 50 ms late: the others' calls return at once
     S = rng.integers(100, 600, size=(world, world))
     inp = out = None

@@ -30,6 +30,31 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::broadcast(std::vector<at::Tensor
   at::Tensor t = tensors[0];
   const int root = (int)opts.rootRank;
   const size_t total = nbytes(t);
+  if (total && total <= std::min(stage_max_, standing_max_) && standingExchangeNow({t}, {t})) {
+    // rank processes: where the root's tensor is travels on the device, nobody meets (runStandingExchange)
+    const int W = size_, me = rank_;
+    Plan p;
+    p.op = c10d::OpType::BROADCAST;
+    p.title = "broadcast";
+    p.inputs = {t};
+    p.outputs = {t};
+    Plan::StandingExchange& x = p.standing_exchange;
+    x.ok = true;
+    x.same_piece = true;
+    x.unanimous_bytes = total;
+    x.piece.assign((size_t)W, me == root ? t.data_ptr() : nullptr);
+    x.send.assign((size_t)W, me == root ? total : 0);
+    x.send[(size_t)me] = 0;  // the root keeps what it has
+    x.block.assign((size_t)W, t.storage().data());
+    x.block_bytes.assign((size_t)W, t.storage().nbytes());
+    x.dst.assign((size_t)W, nullptr);
+    x.recv.assign((size_t)W, 0);
+    if (me != root) {
+      x.dst[(size_t)root] = t.data_ptr();
+      x.recv[(size_t)root] = total;
+    }
+    return run(p);
+  }
   c10::intrusive_ptr<c10d::Work> work;
   size_t off = 0;
   do {
@@ -399,6 +424,36 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
     }
     return last;
   }
+  const int W = size_;
+  if (largest && largest <= standing_max_ && standingExchangeNow({input}, outs)) {
+    // rank processes: where the inputs are travels on the device, nobody meets (runStandingExchange:
+    // every reader gets the same piece, and every rank knows every rank's size from its output list)
+    const int me = rank_;
+    TORCH_CHECK(mine == nbytes(outs[(size_t)me]), "allgather: output tensor ", me, " does not match the size rank ", me, " sends");
+    Plan p;
+    p.op = c10d::OpType::ALLGATHER;
+    p.title = "allgather";
+    p.inputs = {input};
+    p.outputs = outs;
+    Plan::StandingExchange& x = p.standing_exchange;
+    x.ok = true;
+    x.same_piece = true;
+    x.unanimous_bytes = largest;
+    x.piece.assign((size_t)W, mine ? input.data_ptr() : nullptr);
+    x.send.assign((size_t)W, mine);
+    x.block.assign((size_t)W, input.storage().data());
+    x.block_bytes.assign((size_t)W, input.storage().nbytes());
+    x.dst.resize((size_t)W);
+    x.recv.resize((size_t)W);
+    for (int r = 0; r < W; ++r) {
+      x.dst[(size_t)r] = outs[(size_t)r].data_ptr();
+      x.recv[(size_t)r] = nbytes(outs[(size_t)r]);
+      const bool itself = r == me && outs[(size_t)r].data_ptr() == input.data_ptr();  // gathered into the very tensor it comes from
+      if (itself) x.recv[(size_t)r] = 0;
+      else if (rangesOverlap(input.data_ptr(), mine, x.dst[(size_t)r], x.recv[(size_t)r])) x.force_staged = true;
+    }
+    return run(p);
+  }
   Plan p;
   p.op = c10d::OpType::ALLGATHER;
   p.title = "allgather";
@@ -406,7 +461,6 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather(std::vector<std::vecto
   p.outputs = outs;
   p.stage_bytes = mine;
   p.table = {(int64_t)mine};
-  const int W = size_;
   if (mine)
     p.copy_in = [=](void* stage, hipStream_t s) {
       copyAsync(stage, input.data_ptr(), mine, s);

@@ -468,12 +468,13 @@ void ProcessGroupCCL::mapOutbox(int peer, int level) {
   noteImport((uint32_t)peer, MCCL_OFFER_STAGED, MCCL_OFFER_SLOT_OUTBOX, (uint64_t)(uintptr_t)p, 0);
 }
 
-void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t seq) {
+void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
   const Plan::StandingExchange& x = plan.standing_exchange;
   const int W = size_, me = rank_;
   const uint64_t epoch = 4 * seq;
   RankSlot& mine_slot = ctl_->slot[me];
-  const size_t outbox_max = std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1));
+  const bool same = x.same_piece;  // one piece for all readers, sizes known to all: staged through the staging buffer, nothing pairwise
+  const size_t outbox_max = same ? ~(size_t)0 : std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1));
   pairwise_waits_now_ = 0;
   // 1. Everything this rank has to say, before it waits for anything of anybody's: the allocations
   // its pieces live in, larger outboxes where a piece has outgrown the old one, where its oversized
@@ -503,7 +504,12 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
   // of an earlier one)
   for (int d = 0; d < W; ++d)
     if (where[d].entry >= 0 && mine_slot.exports[where[d].entry].gen.load(std::memory_order_acquire) != where[d].gen) where[d].entry = -1;
-  for (int d = 0; d < W; ++d) {
+  // (the staging buffers of a group grow when a message exceeds them, which all ranks find at the same
+  // collective where all ranks know the sizes; and since they meet there, they also look at what
+  // everybody has just announced before anybody decides: see runStanding)
+  const bool grow = same && x.unanimous_bytes > standing_capacity_;
+  if (grow) growStandingCapacity(x.unanimous_bytes);
+  for (int d = 0; d < W && !same; ++d) {
     const size_t b = x.send[(size_t)d];
     if (!b) continue;
     if (b <= outbox_max) {
@@ -533,7 +539,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
               " bytes lives in memory that cannot be shared between processes (not from torch's caching allocator, or an allocation of 2 GiB "
               "or more); set MCCL_PG_STANDING_OFFERS=0");
   // 2. What the peers must have said by now, pair by pair.
-  for (int r = 0; r < W; ++r) {
+  for (int r = 0; r < W && !same; ++r) {
     const size_t b = x.recv[(size_t)r];
     if (r == me || !b) continue;
     if (b <= outbox_max) {
@@ -551,6 +557,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
     }
   }
   scanPeerExports(seq);
+  if (grow) hostBarrier();
   for (int r = 0; r < W; ++r) {
     const size_t b = x.recv[(size_t)r];
     if (r == me || b <= outbox_max) continue;
@@ -573,7 +580,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
     mccl_offer_t& o = row[d];
     o.bytes = b;
     o.entry = MCCL_OFFER_STAGED;
-    o.slot = MCCL_OFFER_SLOT_OUTBOX;
+    o.slot = same ? (uint32_t)slot : MCCL_OFFER_SLOT_OUTBOX;
     expect[d] = x.recv[(size_t)d];
     if (!b || d == me) continue;
     const Where& w = where[d];
@@ -585,14 +592,16 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
       last_offer_seq_[w.entry] = seq + 1;  // in the units of `entered`: collective `seq` is under way at seq + 1
       ++in_place;
     } else {
-      copy_in.push_back({x.piece[(size_t)d], outbox_out_[d].base, b});
+      if (!same) copy_in.push_back({x.piece[(size_t)d], outbox_out_[d].base, b});
+      else if (copy_in.empty()) copy_in.push_back({x.piece[(size_t)d], stage_[slot].ptr, b});  // once, for all readers that need it
       ++staged;
     }
   }
   const void* my_source = x.piece[(size_t)me];
   if (x.force_staged && x.send[(size_t)me]) {
-    copy_in.push_back({x.piece[(size_t)me], outbox_out_[me].base, x.send[(size_t)me]});
-    my_source = outbox_out_[me].base;
+    void* scratch = same ? stage_[slot].ptr : outbox_out_[me].base;
+    if (!same || copy_in.empty()) copy_in.push_back({x.piece[(size_t)me], scratch, x.send[(size_t)me]});
+    my_source = scratch;
   }
   // Little to move: ONE launch on this rank's share of half of the compute units, which copies into the
   // outboxes, carries the row and pulls -- with several processes on the GPU every launch waits for
@@ -605,7 +614,8 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, uint64_t se
   if (!one_launch && !copy_in.empty()) MCCL_CHECK(mccl_copy_segments(copy_in.data(), (int)copy_in.size(), s));
   {
     std::ostringstream os;
-    os << "standing offers, " << in_place << " pieces read in place, " << staged << " through outboxes";
+    if (same) os << "standing offers, " << (staged ? "this rank staged" : "peers read in place");
+    else os << "standing offers, " << in_place << " pieces read in place, " << staged << " through outboxes";
     last_path_storage_ = os.str();
     last_path_ = last_path_storage_.c_str();
   }

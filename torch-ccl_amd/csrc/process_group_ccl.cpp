@@ -800,7 +800,7 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       return;
     }
     if (plan.standing_exchange.ok) {
-      runStandingExchange(plan, s, seq);
+      runStandingExchange(plan, s, slot, seq);
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }

@@ -307,6 +307,11 @@ class ProcessGroupCCL : public c10d::Backend {
       std::vector<void*> dst;          // where rank r's piece for this rank goes
       std::vector<size_t> recv;        // its length
       bool force_staged = false;       // input and output overlap: every piece is copied out of the way first
+      // all_gather into a list, broadcast: every reader gets the SAME piece, and every rank knows how long
+      // every rank's piece is (`unanimous_bytes`: the longest).  A rank that cannot offer it in place copies
+      // it into its staging buffer once, as in runStanding, instead of into an outbox per reader.
+      bool same_piece = false;
+      size_t unanimous_bytes = 0;
     } standing_exchange;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
@@ -344,7 +349,7 @@ class ProcessGroupCCL : public c10d::Backend {
   void growStandingCapacity(size_t bytes);
   bool standingExchangeFits() const;
   bool standingExchangeNow(const std::vector<at::Tensor>& inputs, const std::vector<at::Tensor>& outputs);
-  void runStandingExchange(Plan& plan, hipStream_t s, uint64_t seq);
+  void runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void growOutbox(int peer, int level);
   void mapOutbox(int peer, int level);
   bool acknowledgedBy(int peer, int entry, uint64_t gen, uint64_t seq) const;
