@@ -549,16 +549,17 @@ def large_message_case(pg, rank, world):
 
 
 def missing_rank_case(pg, rank, world):
-    """Rank 1 never joins the second collective: the others must get an error, not hang.  (A
-    reduce_scatter from a list of tensors, 2 MiB each: a collective whose host threads meet first in
-    every mode -- the list is packed into the staging buffer, whose handle is published per call --
-    so the call itself raises.)"""
+    """Rank 1 never joins the second collective: the others must get an error, not hang.  (A gather
+    to rank 0, 2 MiB per rank: a collective whose host threads meet first in every mode -- the staging
+    buffers' handles are published per call -- so the call itself raises.)"""
     t = torch.ones(1 << 19, device=DEV)
     pg.allreduce([t], c10d.AllreduceOptions()).wait()
     if rank == 1:
         return
     try:
-        pg.reduce_scatter([t], [[torch.ones(1 << 19, device=DEV) for _ in range(world)]], c10d.ReduceScatterOptions()).wait()
+        opts = c10d.GatherOptions()
+        opts.rootRank = 0
+        pg.gather([[torch.empty(1 << 19, device=DEV) for _ in range(world)]] if rank == 0 else [], [t], opts).wait()
         raise AssertionError("collective with a missing rank returned")
     except RuntimeError as e:
         assert ("timed out waiting for rank 1" in str(e) or "reported a failure" in str(e)
@@ -1372,6 +1373,32 @@ def standing_alltoall_cases(pg, rank, world):
         assert after[0] == before[0] or i == 0, (i, before, after)  # (the first one enlarges the staging buffers: the ranks meet)
         for r in range(world):
             assert np.array_equal(bits(outs[r]), bits(host[r])), ("allgather list", i, r, pg._last_path())
+    # reduce_scatter from a list: slot d of every rank's list is reduced into rank d's output; slots of
+    # different sizes, in tensors of their own or views of one, the output one of the slots
+    from helpers import TORCH_TO_CODE
+    for i, (dtype, base_n, op, oop) in enumerate(((torch.bfloat16, 300007, c10d.ReduceOp.SUM, O.SUM), (torch.float32, 1 << 19, c10d.ReduceOp.MAX, O.MAX),
+                                                    (torch.float32, 33, c10d.ReduceOp.SUM, O.SUM), (torch.float16, (1 << 20) + 5, c10d.ReduceOp.AVG, O.AVG))):
+        sizes = [base_n + 17 * d for d in range(world)]
+        host = [[rank_buffer(sizes[d], dtype, r * world + d, seed=860 + i) for d in range(world)] for r in range(world)]
+        for rep in range(3):
+            if rep == 2:  # one storage, slots back to back
+                flat = torch.cat([h.view(-1) for h in host[rank]]).to(DEV)
+                ins = list(flat.split(sizes))
+            else:
+                ins = [h.to(DEV) for h in host[rank]]
+            out = ins[rank] if rep == 1 else torch.zeros(sizes[rank], dtype=dtype, device=DEV)
+            opts = c10d.ReduceScatterOptions()
+            opts.reduceOp = op
+            before = pg._rendezvous_counts()
+            pg.reduce_scatter([out], [ins], opts).wait()
+            after = pg._rendezvous_counts()
+            assert after[0] == before[0], (i, rep, before, after)
+            want = O.reduce([to_carrier(host[r][rank]) for r in range(world)], TORCH_TO_CODE[dtype], oop)
+            want = want.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[want.dtype.itemsize])
+            assert np.array_equal(bits(out), want), ("reduce_scatter list", dtype, i, rep, pg._last_path())
+            for d in range(world):
+                if d != rank or rep != 1:
+                    assert np.array_equal(bits(ins[d]), bits(host[rank][d])), ("reduce_scatter list changed slot", d)
     small = [torch.zeros(100 + r, dtype=torch.int16, device=DEV) for r in range(world)]
     pg.allgather([small], [torch.full((100 + rank,), rank + 1, dtype=torch.int16, device=DEV)]).wait()
     for r in range(world):

@@ -674,6 +674,43 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter(std::vector<at::T
     // a flat list is its own image; any other is packed with each slot on a 16-byte boundary
     total += span.flat ? nbytes(ins[(size_t)d]) : roundUp(nbytes(ins[(size_t)d]), 16);
   }
+  size_t largest_slot = 0;
+  for (const auto& slot : ins) largest_slot = std::max(largest_slot, nbytes(slot));  // the same on every rank of a valid call
+  if (largest_slot <= std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1)) && standingExchangeNow(ins, {out})) {
+    // rank processes: where the slots are travels on the device, nobody meets (runStandingExchange: slot d
+    // of this rank's list is its piece for rank d, in place or through the outbox kept for rank d)
+    TORCH_CHECK(nbytes(out) == nbytes(ins[(size_t)me]), "reduce_scatter: output tensor does not match slot ", me);
+    Plan q;
+    q.op = c10d::OpType::REDUCE_SCATTER;
+    q.title = "reduce_scatter";
+    q.inputs = ins;
+    q.outputs = {out};
+    Plan::StandingExchange& x = q.standing_exchange;
+    x.ok = true;
+    x.piece.resize((size_t)W);
+    x.send.resize((size_t)W);
+    x.block.resize((size_t)W);
+    x.block_bytes.resize((size_t)W);
+    x.dst.assign((size_t)W, out.data_ptr());
+    x.recv.assign((size_t)W, nbytes(out));  // every rank's slot for this rank has the size of this rank's output
+    for (int d = 0; d < W; ++d) {
+      const at::Tensor& slot = ins[(size_t)d];
+      x.send[(size_t)d] = nbytes(slot);
+      x.piece[(size_t)d] = x.send[(size_t)d] ? slot.data_ptr() : nullptr;
+      x.block[(size_t)d] = slot.storage().data();
+      x.block_bytes[(size_t)d] = slot.storage().nbytes();
+      // (the output may be this rank's own slot for itself, exactly: the reduction reads element i of
+      // every input before it writes element i)
+      const bool itself = d == me && slot.data_ptr() == out.data_ptr();
+      if (!itself && rangesOverlap(slot.data_ptr(), x.send[(size_t)d], out.data_ptr(), nbytes(out))) x.force_staged = true;
+    }
+    const size_t count = (size_t)out.numel();
+    void* const out_ptr = out.data_ptr();
+    x.reduce = [=](const void* resolved, const mccl_xsync_t& sync, hipStream_t s) {
+      MCCL_CHECK(mccl_reduce_sync_resolved(resolved, 0, out_ptr, count, dtype, op, &sync, s));
+    };
+    return run(q);
+  }
   if (padded > stage_max_) {  // (the padded size: the same on every rank, flat list or not)
     // more than one staging window: W (windowed) rooted reduces, as the reference does for slots of
     // unequal size.  The root reduces in place in its output, which first takes its own slot.

@@ -610,7 +610,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
   size_t moved = 0;
   for (const auto& sg : copy_in) moved += sg.bytes;
   for (int r = 0; r < W; ++r) moved += x.recv[(size_t)r];
-  const bool one_launch = 2.0 * (double)moved <= (double)compact_max_;
+  const bool one_launch = !x.reduce && 2.0 * (double)moved <= (double)compact_max_;
   if (!one_launch && !copy_in.empty()) MCCL_CHECK(mccl_copy_segments(copy_in.data(), (int)copy_in.size(), s));
   {
     std::ostringstream os;
@@ -648,7 +648,9 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     pulls.push_back({nullptr, x.dst[(size_t)r], x.recv[(size_t)r]});
     from.push_back(r);
   }
-  if (one_launch) {
+  if (x.reduce) {
+    x.reduce(resolved_, sync, s);
+  } else if (one_launch) {
     sync.ready_epoch = epoch + 1;
     sync.max_compute_units = std::max(1u, waiting_cus_ / (unsigned)W);
     MCCL_CHECK(mccl_alltoall_sync_offers(copy_in.data(), (int)copy_in.size(), pulls.data(), from.data(), (int)pulls.size(), &sync, row, expect,

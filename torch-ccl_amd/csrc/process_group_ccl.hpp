@@ -312,6 +312,9 @@ class ProcessGroupCCL : public c10d::Backend {
       // it into its staging buffer once, as in runStanding, instead of into an outbox per reader.
       bool same_piece = false;
       size_t unanimous_bytes = 0;
+      // reduce_scatter from a list: what arrives is not copied to dst but reduced, by this kernel over the
+      // resolved addresses (rank r's piece for this rank, this rank's own included)
+      std::function<void(const void* resolved, const mccl_xsync_t& sync, hipStream_t s)> reduce;
     } standing_exchange;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
