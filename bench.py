@@ -820,6 +820,26 @@ def main():
                                                   "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
                                                   "byte_identical": all(bool(torch.equal(g[:COUNT].view(torch.int16), ins[0].view(torch.int16))) for g in gathered)}
         del gathered
+        # the pulls of an all-to-all over resolved addresses: one rank's share of C5's shape (eight pieces of
+        # 56 MiB from eight buffers into 448 MiB), beside the plain segment copy of the same segments
+        piece = 56 << 20
+        a2a_out = torch.zeros(N * piece, dtype=torch.uint8, device=dev)
+        table = torch.tensor([t.data_ptr() for t in ins], dtype=torch.int64, device=dev)
+        pull_segs = (capi.Segment * N)(*[capi.Segment(0, a2a_out.data_ptr() + r * piece, piece) for r in range(N)])
+        plain_segs = (capi.Segment * N)(*[capi.Segment(ins[r].data_ptr(), a2a_out.data_ptr() + r * piece, piece) for r in range(N)])
+        from_rank = (ctypes.c_int * N)(*range(N))
+
+        def pulls_resolved():
+            sy = xsync(0)
+            capi.check(L.mccl_copy_segments_sync_resolved(pull_segs, from_rank, N, table.data_ptr(), 0, ctypes.byref(sy), stream))
+        us = event_us(pulls_resolved)
+        same = all(bool(torch.equal(a2a_out[r * piece:(r + 1) * piece], ins[r].view(torch.uint8)[:piece])) for r in range(N))
+        us_plain = event_us(lambda: capi.check(L.mccl_copy_segments(plain_segs, N, stream)))
+        moved = 2 * N * piece
+        xr["alltoall_pulls_resolved_8x56MiB"] = {"us": round(us, 1), "bytes_moved": moved, "GBps": round(moved / us / 1e3, 1),
+                                                 "pct_of_peak": round(moved / us / 1e3 / PEAK_HBM_GBS * 100, 1),
+                                                 "plain_copy_of_the_same_segments_us": round(us_plain, 1), "byte_identical": same}
+        del a2a_out
         assert status.tolist()[:2] == [0, 0], status.tolist()
         xr["note"] = ("single process, the form that runs behind a barrier kernel (no opening wait, closing count and "
                       "closing wait): every rank's flag word is the same word, so no launch waits")

@@ -516,9 +516,10 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
       const int level = outboxLevel(b);
       const bool needed = d != me || x.force_staged;  // (this rank's piece for itself is copied where it lies, unless that overlaps)
       if (needed && level > outbox_out_[d].level) growOutbox(d, level);
-    } else if (d != me) {
+    } else {
       TORCH_CHECK(!x.force_staged, "ccl backend: ", plan.title, ": input and output overlap and the piece for rank ", d, " (", b,
                   " bytes) is larger than the buffers kept for such pieces (", outbox_max, " bytes); set MCCL_PG_STANDING_OFFERS=0");
+      if (d == me) continue;  // (copied where it lies)
       RankSlot::BigPiece& rec = mine_slot.big[d];
       if (big_published_[d]) {  // rank d has not read the last such record yet: not overwritten before it has
         const uint64_t last = big_published_[d];
