@@ -1237,6 +1237,22 @@ def standing_offer_cases(pg, rank, world):
             del huge
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
+    # the coalesced forms pack their tensors into the staging buffer, which every peer has mapped since
+    # it last grew: after the first call of a size nobody meets
+    for rep in range(3):
+        ts = [torch.full((5000 + 300 * i,), float(rank + 1 + i), device=DEV) for i in range(6)] + [torch.full((1 << 20,), float(rank + 1), device=DEV)]
+        o = c10d.AllreduceCoalescedOptions()
+        o.reduceOp = c10d.ReduceOp.SUM
+        before = pg._rendezvous_counts()
+        pg.allreduce_coalesced(ts, o).wait()
+        mid = pg._rendezvous_counts()
+        for i, t in enumerate(ts[:6]):
+            want = float(sum(r + 1 + i for r in range(world)))
+            assert float(t.min()) == want == float(t.max()), ("allreduce_coalesced", rep, i)
+        assert float(ts[6].min()) == world * (world + 1) / 2 == float(ts[6].max())
+        assert pg._last_path() == "staged, staging buffers mapped for good", pg._last_path()
+        if rep:
+            assert mid[0] == before[0], (rep, before, mid)
     # a rank that comes 50 ms late: the others' calls return at once (nobody's host thread waits
     # for anybody), their Works complete when the late rank's kernels have run
     z = torch.full((1 << 20,), float(rank + 1), device=DEV)  # 4 MiB

@@ -82,6 +82,11 @@ def test_every_windowed_path_with_a_shrunk_window(monkeypatch, window, world, mo
     _spawn(world, mode)
 
 
+def test_coalesced_forms_between_rank_processes_in_one_window():
+    """(the same cases without the shrunk window: packed into the staging buffers, which the peers keep mapped)"""
+    _spawn(4, "coalesced_windows")
+
+
 @pytest.mark.parametrize("standing", ["1", "0"])
 def test_message_larger_than_one_staging_window(monkeypatch, standing):
     """(with standing offers the all-to-all's pieces of 900 and 1100 MiB are read in place, whatever the

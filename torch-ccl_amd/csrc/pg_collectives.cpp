@@ -245,6 +245,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allreduce_coalesced(
   Plan p;
   p.op = c10d::OpType::ALLREDUCE_COALESCED;
   p.title = "allreduce_coalesced";
+  p.static_staged = true;
   p.inputs = tensors;
   p.outputs = tensors;
   if (size_ > 1 && total) {
@@ -525,6 +526,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::allgather_into_tensor_coalesced(
   Plan p;
   p.op = c10d::OpType::ALLGATHER_COALESCED;
   p.title = "allgather_into_tensor_coalesced";
+  p.static_staged = true;
   p.inputs = inputs;
   p.outputs = outputs;
   p.stage_bytes = total;
@@ -797,6 +799,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupCCL::reduce_scatter_tensor_coalesced(
   Plan p;
   p.op = c10d::OpType::COALESCED;
   p.title = "reduce_scatter_tensor_coalesced";
+  p.static_staged = true;
   p.inputs = inputs;
   p.outputs = outputs;
   p.stage_bytes = total;

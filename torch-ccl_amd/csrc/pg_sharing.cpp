@@ -661,6 +661,43 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// coalesced forms: packed into the staging buffer, which the peers have mapped for good
+// ---------------------------------------------------------------------------------------------
+// What the rendezvous of a staged collective publishes is the handle of the staging buffer, which
+// only changes when the buffer grows.  The coalesced forms pack their tensors into it at offsets
+// every rank computes for itself, so once the buffers of both slots are large enough on every rank
+// (the sizes of a coalesced call agree, so all ranks find out together: growStandingCapacity) such
+// a collective is copy-in, barrier kernel, kernel over the peers' staging buffers -- and no
+// meeting of the host threads.  The two slots alternate by collective as ever: every collective
+// waits on the device for every peer's start of it, so a slot is free again two collectives on.
+bool ProcessGroupCCL::staticStagedFits(const Plan& plan) const {
+  return plan.static_staged && standing_offers_ && device_sync_ && distinct_pids_ && !waits_in_data_kernels_ && !work_only_ &&
+         !sync_only_ && size_ > 1 && plan.stage_bytes > 0 && plan.stage_bytes <= std::min(stage_max_, standing_max_) && plan.exec &&
+         !plan.exec2;
+}
+
+void ProcessGroupCCL::runStaticStaged(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
+  const uint64_t epoch = 4 * seq;
+  if (plan.stage_bytes > standing_capacity_) growStandingCapacity(plan.stage_bytes);
+  void* stage = stage_[slot].ptr;
+  if (plan.copy_in) plan.copy_in(stage, s);
+  last_path_ = "staged, staging buffers mapped for good";
+  if (verbose_) {
+    std::ostringstream os;
+    os << "oneccl_bindings_for_pytorch::" << plan.title << " [" << rank_ << "/" << size_ << "#" << (seq + 1) << "] " << last_path_;
+    std::cout << os.str() << std::endl;
+  }
+  ++enqueue_only_count_;
+  deviceBarrier(epoch + 1, s);
+  PeerView pv;
+  pv.zero_copy = false;
+  pv.stage.resize((size_t)size_);
+  pv.tables.assign((size_t)size_, nullptr);
+  for (int r = 0; r < size_; ++r) pv.stage[(size_t)r] = (r == rank_) ? stage : peers_[(size_t)r].ptr[slot];
+  plan.exec(pv, s);
+}
+
 void ProcessGroupCCL::closeImports() {
   for (auto& per_peer : imports_)
     for (auto& im : per_peer)

@@ -804,6 +804,11 @@ void ProcessGroupCCL::runDeviceSynced(Plan& plan, hipStream_t s, int slot, uint6
       if (timed) phase_us_[3].push_back((float)us_since(t0));
       return;
     }
+    if (staticStagedFits(plan)) {
+      runStaticStaged(plan, s, slot, seq);
+      if (timed) phase_us_[3].push_back((float)us_since(t0));
+      return;
+    }
     if (standingFits(plan)) {
       runStanding(plan, s, slot, seq);
       if (timed) phase_us_[3].push_back((float)us_since(t0));

@@ -316,6 +316,11 @@ class ProcessGroupCCL : public c10d::Backend {
       // resolved addresses (rank r's piece for this rank, this rank's own included)
       std::function<void(const void* resolved, const mccl_xsync_t& sync, hipStream_t s)> reduce;
     } standing_exchange;
+    // Everything this collective needs of its peers is in their staging buffers, at places every rank
+    // computes for itself (the shapes of a coalesced call agree across ranks): exec reads pv.stage and
+    // nothing else of pv.  Between rank processes such a collective needs no rendezvous once the
+    // staging buffers are large enough and mapped (runStaticStaged).
+    bool static_staged = false;
     bool host_complete = false;             // the call returns only when the device work is done (barrier)
   };
 
@@ -351,6 +356,8 @@ class ProcessGroupCCL : public c10d::Backend {
   void runStanding(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void growStandingCapacity(size_t bytes);
   bool standingExchangeFits() const;
+  bool staticStagedFits(const Plan& plan) const;
+  void runStaticStaged(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   bool standingExchangeNow(const std::vector<at::Tensor>& inputs, const std::vector<at::Tensor>& outputs);
   void runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   void growOutbox(int peer, int level);
