@@ -574,7 +574,7 @@ int launch_gather(const GatherSpec* specs, int nspec, size_t row_bytes, hipStrea
 // ------------------------------------------------------------------------------------------
 extern "C" {
 
-int mccl_version(void) { return 144; }
+int mccl_version(void) { return 150; }
 
 const char* mccl_last_error(void) { return g_err; }
 
