@@ -1505,6 +1505,89 @@ def alltoall_mismatch_case(pg, rank, world):
             assert float(out[r * rows:(r + 1) * rows].min()) == float(r + 1) == float(out[r * rows:(r + 1) * rows].max()), r
 
 
+def standing_mix_case(pg, rank, world):
+    """A seeded mixture of the collectives that only enqueue -- all-to-alls with pieces of every size class
+    (and beyond the largest, when the limit is shrunk), all_reduce, reduce_scatter / all_gather in both
+    forms, broadcast -- on new and on reused tensors, with every rank late at random: the offers, the
+    acknowledgements, the outboxes and their growth have to keep in step whatever the order in which
+    the host threads get there.  Values are chosen so that every result has a closed form."""
+    import random
+    import time
+    ops = random.Random(2024)       # the same sequence on every rank
+    lag = random.Random(77 + rank)  # this rank's own delays
+    kept = {}
+    for it in range(250):
+        op = ops.choice(("a2a", "a2a", "a2a", "allreduce", "rs", "ag", "ag_list", "rs_list", "bcast"))
+        scale = ops.choice((1, 1, 40, 700, 3000))  # KiB: pieces from a few bytes to several MiB
+        reuse = ops.random() < 0.5
+        root = ops.randrange(world)
+        S = [[ops.randrange(0, scale * 256 + 2) for _ in range(world)] for _ in range(world)]  # floats
+        n = ops.randrange(1, scale * 256 + 2)
+        if lag.random() < 0.3:
+            time.sleep(lag.random() * 0.002)
+        def tensor(key, numel, value):
+            if reuse and key in kept and kept[key].numel() >= numel:
+                t = kept[key][:numel]
+            else:
+                t = torch.empty(numel, device=DEV)
+                kept[key] = t
+            t.fill_(value)
+            return t
+        if op == "a2a":
+            inp = tensor("a2a_in", sum(S[rank]), 0.0)
+            pos = 0
+            for d in range(world):
+                inp[pos:pos + S[rank][d]] = float(rank * 16 + d + it)
+                pos += S[rank][d]
+            out = tensor("a2a_out", sum(S[r][rank] for r in range(world)), -1.0)
+            pg.alltoall_base(out, inp, [S[r][rank] for r in range(world)], S[rank]).wait()
+            pos = 0
+            for r in range(world):
+                piece = out[pos:pos + S[r][rank]]
+                if S[r][rank]:
+                    assert float(piece.min()) == float(r * 16 + rank + it) == float(piece.max()), ("a2a", it, r, pg._last_path())
+                pos += S[r][rank]
+        elif op == "allreduce":
+            t = tensor("ar", n + (1 << 18), float(rank + it))
+            pg.allreduce([t], c10d.AllreduceOptions()).wait()
+            want = float(sum(r + it for r in range(world)))
+            assert float(t.min()) == want == float(t.max()), ("allreduce", it, pg._last_path())
+        elif op == "rs":
+            t = tensor("rs_in", n * world, float(rank + 1))
+            out = tensor("rs_out", n, 0.0)
+            pg._reduce_scatter_base(out, t).wait()
+            assert float(out.min()) == world * (world + 1) / 2 == float(out.max()), ("rs", it, pg._last_path())
+        elif op == "ag":
+            t = tensor("ag_in", n, float(rank + it))
+            out = tensor("ag_out", n * world, -1.0)
+            pg._allgather_base(out, t).wait()
+            for r in range(world):
+                assert float(out[r * n:(r + 1) * n].min()) == float(r + it) == float(out[r * n:(r + 1) * n].max()), ("ag", it, r)
+        elif op == "ag_list":
+            sizes = [S[0][r] + 1 for r in range(world)]
+            t = tensor("agl_in", sizes[rank], float(rank + it))
+            outs = [torch.full((sizes[r],), -1.0, device=DEV) for r in range(world)]
+            pg.allgather([outs], [t]).wait()
+            for r in range(world):
+                assert float(outs[r].min()) == float(r + it) == float(outs[r].max()), ("ag_list", it, r, pg._last_path())
+        elif op == "rs_list":
+            sizes = [S[0][d] + 1 for d in range(world)]
+            ins = [torch.full((sizes[d],), float(rank + d), device=DEV) for d in range(world)]
+            out = torch.zeros(sizes[rank], device=DEV)
+            pg.reduce_scatter([out], [ins], c10d.ReduceScatterOptions()).wait()
+            want = float(sum(r + rank for r in range(world)))
+            assert float(out.min()) == want == float(out.max()), ("rs_list", it, pg._last_path())
+        else:
+            t = tensor("bc", n, float(it) if rank == root else -1.0)
+            o = c10d.BroadcastOptions()
+            o.rootRank = root
+            o.rootTensor = 0
+            pg.broadcast([t], o).wait()
+            assert float(t.min()) == float(it) == float(t.max()), ("bcast", it, root, pg._last_path())
+    torch.cuda.synchronize()
+    pg.barrier().wait()
+
+
 def graph_capture_case(rank, world):
     """A decode loop from a HIP graph: every rank records K dist.all_reduce of the 256 KiB bf16
     message with a small kernel of the caller's between them, then replays the graph with fresh
@@ -1733,6 +1816,8 @@ def run_rank(rank, world, store_path, mode):
         standing_offer_cases(pg, rank, world)
     elif mode == "standing_alltoall":
         standing_alltoall_cases(pg, rank, world)
+    elif mode == "standing_mix":
+        standing_mix_case(pg, rank, world)
     elif mode == "alltoall_mismatch":
         alltoall_mismatch_case(pg, rank, world)
     elif mode == "standing_big":

@@ -147,6 +147,15 @@ def test_all_to_all_with_offers_exchanged_on_the_device(world):
     _spawn(world, "standing_alltoall")
 
 
+@pytest.mark.parametrize("world,limit", [(8, ""), (5, ""), (4, str(1 << 20))])
+def test_a_mixture_of_the_collectives_that_only_enqueue(monkeypatch, world, limit):
+    """(limit: MCCL_PG_STANDING_MAX_BYTES shrunk to 1 MiB, so that the all-to-alls' pieces also go the
+    way of those larger than any outbox and the other collectives fall back to the rendezvous in between)"""
+    if limit:
+        monkeypatch.setenv("MCCL_PG_STANDING_MAX_BYTES", limit)
+    _spawn(world, "standing_mix")
+
+
 def test_all_to_all_with_split_sizes_that_do_not_match_is_reported():
     _spawn(3, "alltoall_mismatch")
 
