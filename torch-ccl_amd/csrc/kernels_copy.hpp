@@ -64,7 +64,9 @@ struct LeanCopyArgs {
 // UNROLL: 16-byte vectors per lane per chunk (chunk = 64 x 16 x UNROLL bytes; the host computes
 // the segment geometry for the same value).  STREAM: full chunks are written through past the
 // caches (`sc1`) instead of with the non-temporal hint.
-template <bool COHERENT, int UNROLL, bool STREAM, int INDIRECT = 0, typename ARGS = CopyArgs>
+// THROUGH: every store is written through to memory (for readers in other processes that are running at
+// the same time and are told by a flag), not only the full chunks.
+template <bool COHERENT, int UNROLL, bool STREAM, int INDIRECT = 0, typename ARGS = CopyArgs, bool THROUGH = false>
 __device__ __forceinline__ void copy_segments_body(const ARGS& a, const Wave& w, bool shared_sources = false,
                                                    const CopySources from = CopySources{nullptr, nullptr, 0}) {
   constexpr uint32_t CHUNK = (uint32_t)kWave * 16u * UNROLL;
@@ -99,8 +101,12 @@ __device__ __forceinline__ void copy_segments_body(const ARGS& a, const Wave& w,
         src = (const char*)(base + (uint64_t)(uintptr_t)src);
       }
     }
-    if (c == 0)
-      for (uint32_t i = t; i < head; i += kWave) dst[i] = src[i];  // head < 128
+    if (c == 0) {
+      for (uint32_t i = t; i < head; i += kWave) {  // head < 128
+        if constexpr (THROUGH) __hip_atomic_store((unsigned char*)dst + i, (unsigned char)src[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        else dst[i] = src[i];
+      }
+    }
     const size_t off = (size_t)head + (size_t)c * CHUNK;  // start of this chunk
     src += off;
     dst += off;
@@ -117,14 +123,21 @@ __device__ __forceinline__ void copy_segments_body(const ARGS& a, const Wave& w,
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        if constexpr (STREAM) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&dv[t + u * kWave]), "v"(x[u]) : "memory");
+        if constexpr (THROUGH) store_vec_through((char*)&dv[t + u * kWave], x[u]);
+        else if constexpr (STREAM) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(&dv[t + u * kWave]), "v"(x[u]) : "memory");
         else __builtin_nontemporal_store(x[u], &dv[t + u * kWave]);
       }
     } else {
       const uint32_t nv = len >> 4;
-      for (uint32_t v = t; v < nv; v += kWave) dv[v] = sv[v];
+      for (uint32_t v = t; v < nv; v += kWave) {
+        if constexpr (THROUGH) store_vec_through((char*)&dv[v], (u32x4)sv[v]);
+        else dv[v] = sv[v];
+      }
       const uint32_t rem = len & 15u;
-      if (t < rem) dst[(nv << 4) + t] = src[(nv << 4) + t];
+      if (t < rem) {
+        if constexpr (THROUGH) __hip_atomic_store((unsigned char*)dst + (nv << 4) + t, (unsigned char)src[(nv << 4) + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        else dst[(nv << 4) + t] = src[(nv << 4) + t];
+      }
     }
   }
 }
@@ -182,9 +195,11 @@ __global__ __launch_bounds__(kWave * WPG) void exchange_offers_kernel(const Exch
   const int n = a.sync.n, me = a.sync.rank;
   const bool staging = a.stage.nseg != 0;  // (nothing to copy: the row and the flag go out at once, as in every other one-launch form)
   if (staging) {
-    copy_segments_body<false, kCopyUnroll, false, 0, LeanCopyArgs>(a.stage, w);
-    // what this workgroup has put into the outboxes is in memory before it counts itself in
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
+    copy_segments_body<false, kCopyUnroll, false, 0, LeanCopyArgs, /*THROUGH=*/true>(a.stage, w);
+    // what this workgroup has put into the outboxes -- written through -- is in memory before it counts
+    // itself in (a release fence of system scope instead would write back all of the L2 this workgroup
+    // runs on, other processes' lines included)
+    wait_own_stores();
     __syncthreads();
     if (threadIdx.x == 0) (void)__hip_atomic_fetch_add(a.staged_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
