@@ -484,6 +484,8 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     uint64_t gen = 0, off = 0;
   } where[MCCL_OFFER_RANKS];
   bool unshareable_big = false;
+  const void* announced_block = nullptr;
+  Where announced;
   for (int d = 0; d < W; ++d) {
     const size_t b = x.send[(size_t)d];
     if (d == me || !b || x.force_staged) continue;
@@ -492,13 +494,16 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     // the table of allocations over all the time, and copying them costs next to nothing)
     if (!big && x.block_bytes[(size_t)d] < kZeroCopyMinBytes) continue;
     Where& w = where[d];
-    w.entry = exportRange(x.block[(size_t)d], x.block_bytes[(size_t)d], &w.off);
-    if (w.entry >= 0 && w.entry < kMaxExports) {
-      w.gen = mine_slot.exports[w.entry].gen.load(std::memory_order_acquire);
-      w.off += (uint64_t)((const char*)x.piece[(size_t)d] - (const char*)x.block[(size_t)d]);
+    if (announced_block == x.block[(size_t)d]) {  // (one tensor, or a flat list: the pieces share a storage)
+      w = announced;
     } else {
-      w.entry = -1;
+      w.entry = exportRange(x.block[(size_t)d], x.block_bytes[(size_t)d], &w.off);
+      if (w.entry >= 0 && w.entry < kMaxExports) w.gen = mine_slot.exports[w.entry].gen.load(std::memory_order_acquire);
+      else w.entry = -1;
+      announced_block = x.block[(size_t)d];
+      announced = w;
     }
+    if (w.entry >= 0) w.off += (uint64_t)((const char*)x.piece[(size_t)d] - (const char*)x.block[(size_t)d]);
   }
   // (pieces in more allocations than the table has free entries: a later one may have taken the entry
   // of an earlier one)
