@@ -468,24 +468,18 @@ void ProcessGroupCCL::mapOutbox(int peer, int level) {
   noteImport((uint32_t)peer, MCCL_OFFER_STAGED, MCCL_OFFER_SLOT_OUTBOX, (uint64_t)(uintptr_t)p, 0);
 }
 
-void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
+// Step 1 of an exchange: everything this rank has to say, before it waits for anything of anybody's --
+// the allocations its pieces live in (where[d]: what rank d can be offered in place), larger
+// outboxes where a piece has outgrown the old one, where its oversized pieces are.  Returns whether
+// the group's staging buffers had to grow (one piece for all readers only).
+bool ProcessGroupCCL::announcePieces(const Plan& plan, uint64_t seq, size_t outbox_max, PieceWhere* where) {
   const Plan::StandingExchange& x = plan.standing_exchange;
   const int W = size_, me = rank_;
-  const uint64_t epoch = 4 * seq;
   RankSlot& mine_slot = ctl_->slot[me];
-  const bool same = x.same_piece;  // one piece for all readers, sizes known to all: staged through the staging buffer, nothing pairwise
-  const size_t outbox_max = same ? ~(size_t)0 : std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1));
-  pairwise_waits_now_ = 0;
-  // 1. Everything this rank has to say, before it waits for anything of anybody's: the allocations
-  // its pieces live in, larger outboxes where a piece has outgrown the old one, where its oversized
-  // pieces are.
-  struct Where {
-    int entry = -1;
-    uint64_t gen = 0, off = 0;
-  } where[MCCL_OFFER_RANKS];
+  const bool same = x.same_piece;
   bool unshareable_big = false;
   const void* announced_block = nullptr;
-  Where announced;
+  PieceWhere announced;
   for (int d = 0; d < W; ++d) {
     const size_t b = x.send[(size_t)d];
     if (d == me || !b || x.force_staged) continue;
@@ -493,7 +487,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     // (small tensors live in the allocator's 2 MiB segments, many of them: announcing those would turn
     // the table of allocations over all the time, and copying them costs next to nothing)
     if (!big && x.block_bytes[(size_t)d] < kZeroCopyMinBytes) continue;
-    Where& w = where[d];
+    PieceWhere& w = where[d];
     if (announced_block == x.block[(size_t)d]) {  // (one tensor, or a flat list: the pieces share a storage)
       w = announced;
     } else {
@@ -544,8 +538,15 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
   TORCH_CHECK(!unshareable_big, "ccl backend: ", plan.title, ": a piece larger than ", outbox_max,
               " bytes lives in memory that cannot be shared between processes (not from torch's caching allocator, or an allocation of 2 GiB "
               "or more); set MCCL_PG_STANDING_OFFERS=0");
-  // 2. What the peers must have said by now, pair by pair.
-  for (int r = 0; r < W && !same; ++r) {
+  return grow;
+}
+
+// Step 2: what the peers must have said by now, pair by pair -- the outbox of a size class this rank
+// has not mapped yet, where an oversized piece is -- and a look at what they have announced.
+void ProcessGroupCCL::awaitPeerPieces(const Plan& plan, uint64_t seq, size_t outbox_max, bool grew) {
+  const Plan::StandingExchange& x = plan.standing_exchange;
+  const int W = size_, me = rank_;
+  for (int r = 0; r < W && !x.same_piece; ++r) {
     const size_t b = x.recv[(size_t)r];
     if (r == me || !b) continue;
     if (b <= outbox_max) {
@@ -563,7 +564,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     }
   }
   scanPeerExports(seq);
-  if (grow) hostBarrier();
+  if (grew) hostBarrier();
   for (int r = 0; r < W; ++r) {
     const size_t b = x.recv[(size_t)r];
     if (r == me || b <= outbox_max) continue;
@@ -576,6 +577,18 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     const Import& im = imports_[(size_t)r][(size_t)entry];
     TORCH_CHECK(im.base && im.gen == gen, "ccl backend: ", plan.title, ": could not map the allocation that holds rank ", r, "'s piece for this rank");
   }
+}
+
+void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq) {
+  const Plan::StandingExchange& x = plan.standing_exchange;
+  const int W = size_, me = rank_;
+  const uint64_t epoch = 4 * seq;
+  const bool same = x.same_piece;  // one piece for all readers, sizes known to all: staged through the staging buffer, nothing pairwise
+  const size_t outbox_max = same ? ~(size_t)0 : std::min(standing_max_, kOutboxMin << (kOutboxLevels - 1));
+  pairwise_waits_now_ = 0;
+  PieceWhere where[MCCL_OFFER_RANKS];
+  const bool grew = announcePieces(plan, seq, outbox_max, where);
+  awaitPeerPieces(plan, seq, outbox_max, grew);
   // 3. This rank's row of offers.
   mccl_offer_t row[MCCL_OFFER_RANKS] = {};
   uint64_t expect[MCCL_OFFER_RANKS] = {};
@@ -589,7 +602,7 @@ void ProcessGroupCCL::runStandingExchange(Plan& plan, hipStream_t s, int slot, u
     o.slot = same ? (uint32_t)slot : MCCL_OFFER_SLOT_OUTBOX;
     expect[d] = x.recv[(size_t)d];
     if (!b || d == me) continue;
-    const Where& w = where[d];
+    const PieceWhere& w = where[d];
     if (w.entry >= 0 && (b > outbox_max || acknowledgedBy(d, w.entry, w.gen, seq))) {
       o.entry = (uint32_t)w.entry;
       o.slot = 0;

@@ -360,6 +360,12 @@ class ProcessGroupCCL : public c10d::Backend {
   void runStaticStaged(Plan& plan, hipStream_t s, int slot, uint64_t seq);
   bool standingExchangeNow(const std::vector<at::Tensor>& inputs, const std::vector<at::Tensor>& outputs);
   void runStandingExchange(Plan& plan, hipStream_t s, int slot, uint64_t seq);
+  struct PieceWhere {  // what a reader can be offered in place: entry of this rank's export table, its generation, where in it
+    int entry = -1;
+    uint64_t gen = 0, off = 0;
+  };
+  bool announcePieces(const Plan& plan, uint64_t seq, size_t outbox_max, PieceWhere* where);
+  void awaitPeerPieces(const Plan& plan, uint64_t seq, size_t outbox_max, bool grew);
   void growOutbox(int peer, int level);
   void mapOutbox(int peer, int level);
   bool acknowledgedBy(int peer, int entry, uint64_t gen, uint64_t seq) const;
