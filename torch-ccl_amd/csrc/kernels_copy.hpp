@@ -186,6 +186,7 @@ struct ExchangeArgs {
   uint64_t my_source;
   const mccl_import_table_t* imports;
   uint32_t* staged_count;              // zero between launches
+  uint32_t invalidate;                 // a pull has a head or a partial chunk, or an odd offset: those bytes go through the caches
   XSync sync;
 };
 
@@ -231,7 +232,10 @@ __global__ __launch_bounds__(kWave * WPG) void exchange_offers_kernel(const Exch
     const int r = (int)w.lane;
     if (r >= n) where = 0;
     else if (r != me) where = resolve_piece(a.row[r] + 4 * me, a.expect[r], a.imports, r, a.sync.status);
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // outboxes, heads and partial chunks go through the caches
+    // Full chunks of 8-byte aligned sources are read past the caches; whatever else there is (heads,
+    // partial chunks, sources at odd addresses) is read through them, after an invalidate -- only then:
+    // with several processes on the GPU an invalidate is everybody's loss.
+    if (a.invalidate || __builtin_amdgcn_ballot_w64((where & 7u) != 0) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
     copy_segments_body<true, kCopyUnroll, false, 2, LeanCopyArgs>(a.pull, w, false, CopySources{nullptr, a.src_rank, where});
   }
   xsync_end(a.sync, gridDim.x, /*wrote_to_peers=*/false);

@@ -1522,6 +1522,10 @@ int mccl_alltoall_sync_offers(const mccl_segment_t* stage, int nstage, const mcc
   }
   a.my_source = (uint64_t)(uintptr_t)my_source;
   a.imports = imports;
+  for (int k = 0; k < a.pull.nseg; ++k) {
+    const CopySeg& cs = a.pull.seg[k];
+    if (cs.head || cs.last || (((uintptr_t)cs.src + cs.head) & 7u)) a.invalidate = 1;  // (src: an offset from an address the launch resolves)
+  }
   a.staged_count = a.sync.done_count + kStagedCountWord;
   const XShape shape = xrank_shape(chunks, sync);
   if (!shape.packed) return fail(MCCL_ERR_INVALID_ARG, "the one-launch all-to-all with offers runs packed (max_compute_units)");
