@@ -86,19 +86,19 @@ __device__ __forceinline__ const char* pick_in(const XIns& in, int k) {
 }
 
 template <int DT, int NS>
-__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, VecU<DT> (&x)[kXRanks]) {
+__device__ __forceinline__ void xrank_load_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, uint32_t aligned, VecU<DT> (&x)[kXRanks]) {
   const uint32_t v = tile * kWave + w.lane;  // the host keeps tiles1 * 64 below 2^32
   if (v < a.nvec1) {
 #pragma unroll
     for (int k = 0; k < kXRanks; ++k) {
-      if (NS ? k < NS : k < n) x[k].v = load_in(in.p[k], tile, a.aligned_in, w.lane);
+      if (NS ? k < NS : k < n) x[k].v = load_in(in.p[k], tile, aligned, w.lane);
     }
   }
 }
 
 // Reduces the loaded vectors of a tile (ascending-rank chain) and stores the result.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, const VecU<DT> (&x)[kXRanks]) {
+__device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const XIns& in, const Wave& w, uint32_t tile, int n, uint32_t aligned, const VecU<DT> (&x)[kXRanks]) {
   using A = typename Elem<DT>::acc_t;
   constexpr int VE = vec_elems<DT>();
   const uint32_t v = tile * kWave + w.lane;
@@ -124,7 +124,7 @@ __device__ __forceinline__ void xrank_finish_tile(const XRankArgs& a, const XIns
       for (int k = 0; k < kXRanks; ++k) {
         if (NS ? k < NS : k < n) {
           char* tb = const_cast<char*>(in.p[k]) + (size_t)tile * kXTileBytes;  // uniform
-          if (a.aligned_in) store_tile_through(tb, w.lane * 16u, r.v);
+          if (aligned) store_tile_through(tb, w.lane * 16u, r.v);
           else store_vec_through(tb + w.lane * 16u, r.v);
         }
       }
@@ -164,20 +164,20 @@ __device__ __forceinline__ void xrank_tail(const XRankArgs& a, const XIns& in, c
 // between a phase of loads and a phase of stores in step, and the memory pipeline runs dry
 // between the phases.
 template <int DT, int OP, int NS>
-__device__ __forceinline__ void xrank_walk(const XRankArgs& a, const XIns& in, const Wave& w, int n) {
+__device__ __forceinline__ void xrank_walk(const XRankArgs& a, const XIns& in, const Wave& w, int n, uint32_t aligned) {
   const uint32_t T = a.tiles1, G = w.count;
   uint32_t t0 = w.index;
   if (t0 < T) {
     VecU<DT> x0[kXRanks], x1[kXRanks];
-    xrank_load_tile<DT, NS>(a, in, w, t0, n, x0);
+    xrank_load_tile<DT, NS>(a, in, w, t0, n, aligned, x0);
     for (;;) {
       const uint32_t t1 = t0 + G;
-      if (t1 < T) xrank_load_tile<DT, NS>(a, in, w, t1, n, x1);
-      xrank_finish_tile<DT, OP, NS>(a, in, w, t0, n, x0);
+      if (t1 < T) xrank_load_tile<DT, NS>(a, in, w, t1, n, aligned, x1);
+      xrank_finish_tile<DT, OP, NS>(a, in, w, t0, n, aligned, x0);
       if (t1 >= T) break;
       t0 = t1 + G;
-      if (t0 < T) xrank_load_tile<DT, NS>(a, in, w, t0, n, x0);
-      xrank_finish_tile<DT, OP, NS>(a, in, w, t1, n, x1);
+      if (t0 < T) xrank_load_tile<DT, NS>(a, in, w, t0, n, aligned, x0);
+      xrank_finish_tile<DT, OP, NS>(a, in, w, t1, n, aligned, x1);
       if (t0 >= T) break;
     }
   }
@@ -212,6 +212,7 @@ __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankAr
     for (int k = 0; k < kXRanks; ++k) in.p[k] = a.in[k];
   }
   bool begun = resolved && xsync_begin(a.sync);
+  uint32_t aligned = a.aligned_in;
   if constexpr (INDIRECT == 2) {
     if (begun) {
       uint64_t where = a.my_buffer;
@@ -222,6 +223,10 @@ __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankAr
       }
       begun = __builtin_amdgcn_ballot_w64(r < n && where == 0) == 0;
       where += a.in_off;
+      // (only now is it known where the tensors lie: 8-byte aligned ones -- whole tensors out of an
+      // allocator always are -- are read past the caches in one streaming access each and need no
+      // invalidate, which with several processes on the GPU is everybody's loss)
+      aligned = __builtin_amdgcn_ballot_w64(r < n && (where & 7u) != 0) == 0 ? 1u : 0u;
 #pragma unroll
       for (int k = 0; k < kXRanks; ++k) {
         const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)where, k);
@@ -234,9 +239,9 @@ __global__ __launch_bounds__(kWave * WPG) void xrank_reduce_kernel(const XRankAr
     }
   }
   if (begun) {
-    if (!a.aligned_in && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
-    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, in, w, n);
-    else xrank_walk<DT, OP, 0>(a, in, w, n);
+    if (!aligned && !a.no_invalidate) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");  // misaligned inputs go through the caches
+    if (n == kXRanks) xrank_walk<DT, OP, kXRanks>(a, in, w, n, aligned);
+    else xrank_walk<DT, OP, 0>(a, in, w, n, aligned);
     if (a.tail1 && w.index == w.count - 1) xrank_tail<DT, OP>(a, in, w, n);
   }
   xsync_end(a.sync, gridDim.x, a.push != 0);
