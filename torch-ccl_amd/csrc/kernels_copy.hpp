@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kWave * WPG) void exchange_offers_kernel(const Exch
         }
         __builtin_amdgcn_s_sleep(2);
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the flag below follows what the counted workgroups did
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the flag below stays below the count (the copies were written through: no cache to invalidate)
       __hip_atomic_store(a.staged_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     }
     uint64_t* row = a.row[me];
