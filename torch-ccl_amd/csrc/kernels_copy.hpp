@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kWave * WPG) void exchange_offers_kernel(const Exch
         for (int i = 0; i < 4; ++i) __hip_atomic_store(row + 4 * k + i, a.mine[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       }
     }
-    __hip_atomic_store(a.sync.word[me], a.sync.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    publish_flag64(a.sync.word[me], a.sync.ready_epoch);
   }
   if (xsync_begin(a.sync, /*publish=*/false)) {  // (publish = false also makes it wait for this rank's own flag)
     uint64_t where = a.my_source;

@@ -100,6 +100,16 @@ __device__ __forceinline__ void wait_own_stores() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// Stores a flag that announces what this wavefront has stored before it.  Those stores are written
+// through and have been acknowledged (wait_own_stores); what earlier kernels of the stream wrote is in
+// memory since they ended.  A release of system scope on the store itself would add a write-back of
+// the whole L2 the wavefront happens to run on -- other processes' lines included -- and make the
+// peers wait for it.
+__device__ __forceinline__ void publish_flag64(uint64_t* word, uint64_t value) {
+  wait_own_stores();
+  __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Pause between two polls of a flag: half a microsecond at first, then about an eighth of the time
 // waited so far, up to 40 us.  Thousands of wavefronts of several processes may be polling the
 // same few words, past the caches: at a fixed half microsecond the waiting ranks of a collective
@@ -212,7 +222,7 @@ __device__ __forceinline__ bool xsync_begin(const XSync& x, bool publish = true)
   if (x.ready_epoch == 0) return true;  // the caller has ordered the ranks on the host
   const int lane = threadIdx.x & (kWave - 1);
   if (publish && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
-    __hip_atomic_store(x.word[x.rank], x.ready_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    publish_flag64(x.word[x.rank], x.ready_epoch);
   bool ok = true;
   // (publish = false: this rank's own word says that all its workgroups are through with what comes
   // before -- waited for like the peers')
@@ -268,7 +278,7 @@ __device__ __forceinline__ void xsync_end(const XSync& x, uint32_t workgroups, b
     __builtin_amdgcn_s_sleep(4);
   }
   if (lane < groups) __hip_atomic_store(x.done_count + kDoneStride * lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-  if (lane == 0) __hip_atomic_store(x.word[x.rank], x.done_epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (lane == 0) publish_flag64(x.word[x.rank], x.done_epoch);
   if ((int)lane < x.n && (int)lane != x.rank) {
     if (!wait_flag64(x.word[lane], x.done_epoch, x.limit_ticks)) report_late(x.status, lane, (uint32_t)x.done_epoch);
   }
@@ -319,7 +329,7 @@ __global__ __launch_bounds__(kWave) void rank_barrier_offers_kernel(const OfferB
   if (lane == 0) {
     // the offer first, then the flag that says it is there
     publish_offer(a.offer[a.rank], a.mine);
-    __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    publish_flag64(a.flag[a.rank], a.epoch);
   }
   if (lane >= a.n) return;
   uint64_t where = a.my_buffer;
@@ -382,7 +392,7 @@ __global__ __launch_bounds__(kWave) void rank_barrier_offers_each_kernel(const O
         for (int i = 0; i < 4; ++i) __hip_atomic_store(row + 4 * k + i, a.mine[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       }
     }
-    __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    publish_flag64(a.flag[a.rank], a.epoch);
   }
   if (lane >= a.n) return;
   uint64_t where = a.my_source;
@@ -421,7 +431,7 @@ __global__ __launch_bounds__(kWave) void import_table_update_kernel(const Import
 template <typename ARGS>
 __global__ __launch_bounds__(kWave) void rank_barrier_kernel(const ARGS a) {
   const int lane = threadIdx.x;
-  if (lane == 0) __hip_atomic_store(a.flag[a.rank], a.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (lane == 0) publish_flag64(a.flag[a.rank], a.epoch);
   if (lane < a.n && lane != a.rank) {
     if (!wait_flag64(a.flag[lane], a.epoch, a.limit_ticks)) report_late(a.status, lane, (uint32_t)a.epoch);
   }
